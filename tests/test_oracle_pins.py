@@ -1,0 +1,277 @@
+"""Pins the CPU oracle against library routines, closed forms and brute force.
+
+Nothing here repeats the oracle's own formulas: compression is checked against
+F.conv1d / unfold().mean() / a flatten-and-matmul loop, pooling against
+F.avg_pool1d, the attention branches against F.scaled_dot_product_attention with
+explicit boolean masks and against a per-token loop, the packed layout against
+per-sequence runs and the decode step against the last prefill row.
+"""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import nsa_oracle as O
+
+D64 = torch.float64
+
+
+def _rand(*shape, seed=0, scale=1.0, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype)
+
+
+# ---------------------------------------------------------------- counts
+@pytest.mark.parametrize("T,l,d", [(1024, 32, 16), (1000, 32, 16), (31, 32, 16), (32, 32, 16),
+                                   (1024, 64, 16), (77, 8, 4)])
+def test_counts_match_conv1d(T, l, d):
+    if T >= l:
+        n = F.conv1d(torch.zeros(1, 1, T), torch.zeros(1, 1, l), stride=d).shape[-1]
+    else:
+        n = 0
+    assert O.compressed_len_conv(T, l, d) == n
+    assert O.compressed_len_functional(T, l, d) == max(n - 1, 0)
+
+
+# ---------------------------------------------------------------- compression
+@pytest.mark.parametrize("T,H,D,l,d", [(200, 2, 16, 32, 16), (133, 1, 8, 8, 4), (96, 3, 32, 64, 16)])
+def test_compress_weighted_is_conv1d(T, H, D, l, d):
+    x = _rand(T, H, D, seed=1)
+    conv = torch.nn.Conv1d(D, D, l, d)
+    w_lin = conv.weight.detach().permute(2, 1, 0).reshape(l * D, D)      # [j*D+i, o] = W[o,i,j]
+    n = O.compressed_len_conv(T, l, d)
+    got = O.compress_weighted(x, w_lin, conv.bias.detach(), l, d, n, math_dtype=D64, out_dtype=D64)
+    ref = conv.double()(x.double().permute(1, 2, 0)).permute(2, 0, 1)    # [H,D,T]->[H,D,n]->[n,H,D]
+    torch.testing.assert_close(got, ref.detach(), rtol=1e-10, atol=1e-10)
+    brute = O.compress_loop(x, w_lin, conv.bias.detach(), l, d, n)
+    torch.testing.assert_close(got, brute, rtol=1e-10, atol=1e-10)
+
+
+@pytest.mark.parametrize("T,l,d", [(256, 32, 16), (250, 32, 16), (100, 64, 16)])
+def test_compress_meanpool_is_unfold_mean(T, l, d):
+    x = _rand(T, 2, 16, seed=2)
+    n = O.compressed_len_conv(T, l, d)
+    got = O.compress_meanpool(x, l, d, n, math_dtype=D64, out_dtype=D64)
+    ref = x.double().unfold(0, l, d).mean(-1)
+    torch.testing.assert_close(got, ref, rtol=1e-12, atol=1e-12)
+    eye = (torch.eye(16) / l).repeat(l, 1)                               # W[j*D+i,o] = delta_io / l
+    via_w = O.compress_weighted(x, eye, None, l, d, n, math_dtype=D64, out_dtype=D64)
+    torch.testing.assert_close(got, via_w, rtol=1e-12, atol=1e-12)
+
+
+def test_functional_count_drops_last_block():
+    x = _rand(128, 1, 8, seed=3)
+    w = _rand(32 * 8, 8, seed=4)
+    n_conv = O.compressed_len_conv(128, 32, 16)
+    n_fun = O.compressed_len_functional(128, 32, 16)
+    assert n_fun == n_conv - 1
+    a = O.compress_weighted(x, w, None, 32, 16, n_conv, D64, D64)
+    b = O.compress_weighted(x, w, None, 32, 16, n_fun, D64, D64)
+    torch.testing.assert_close(a[:n_fun], b)
+
+
+# ---------------------------------------------------------------- pooling
+@pytest.mark.parametrize("Nc", [5, 6, 7, 8, 9, 15, 16, 17, 61, 62, 63, 64, 65, 511, 2047])
+@pytest.mark.parametrize("k,s,p", [(5, 4, 0), (5, 4, 2), (3, 2, 0), (9, 8, 0)])
+def test_pool_matches_avg_pool1d(Nc, k, s, p):
+    if Nc + 2 * p < k:
+        pytest.skip("window larger than input")
+    x = _rand(3, Nc, seed=Nc, dtype=D64).abs()
+    ref = F.avg_pool1d(x[None], k, s, p, True)[0]
+    Ns, _ = O.pool_geometry(Nc, k, s, p)
+    assert Ns == ref.shape[-1]
+    torch.testing.assert_close(O.pool_scores_direct(x, k, s, p), ref, rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(O.pool_scores(x, k, s, p), ref, rtol=1e-9, atol=1e-12)
+
+
+def test_ns_equals_T_over_64_when_divisible():
+    for T in (1024, 8192, 32768):
+        Nc = O.compressed_len_conv(T, 32, 16)
+        assert O.pool_geometry(Nc, 5, 4, 0)[0] == T // 64
+    assert O.pool_geometry(O.compressed_len_conv(1000, 32, 16), 5, 4, 0)[0] == 15
+    assert O.pool_geometry(O.compressed_len_conv(1055, 32, 16), 5, 4, 0)[0] == 16
+
+
+# ---------------------------------------------------------------- importance + top-n
+def test_importance_matches_library_pipeline():
+    T, Hq, Hkv, Dk = 192, 8, 2, 16
+    q = _rand(T, Hq, Dk, seed=5)
+    ck = _rand(11, Hkv, Dk, seed=6)
+    got = O.importance_scores(q, ck, 5, 4, 0, math_dtype=D64)
+    # library route: einsum over repeated heads -> softmax -> reshape/sum -> avg_pool1d
+    ckr = ck.double().repeat_interleave(Hq // Hkv, dim=1)
+    p = torch.softmax(torch.einsum("thd,shd->hts", q.double(), ckr), -1)      # [Hq,T,Nc]
+    p = p.reshape(Hkv, Hq // Hkv, T, -1).sum(1)
+    ref = F.avg_pool1d(p, 5, 4, 0, True).transpose(0, 1)                      # [T,Hkv,Ns]
+    torch.testing.assert_close(got, ref, rtol=1e-10, atol=1e-12)
+    # invariant: un-pooled importance sums to G per (t, h); the pooled sum brackets it
+    assert torch.allclose(p.sum(-1), torch.full((Hkv, T), float(Hq // Hkv), dtype=D64))
+    idx = O.select_blocks(got, 2)
+    ref_idx = torch.topk(ref, 2, dim=-1).indices
+    assert torch.equal(idx.sort(-1).values, ref_idx.sort(-1).values)
+
+
+def test_select_blocks_pads_when_few_bins():
+    pooled = torch.tensor([[[0.1, 0.7, 0.2]]])
+    idx = O.select_blocks(pooled, 5)
+    assert idx[0, 0].tolist() == [1, 2, 0, -1, -1]
+
+
+# ---------------------------------------------------------------- compressed attention
+def test_compressed_attention_is_masked_sdpa():
+    T, Hq, Hkv, Dk, Dv, l, d = 160, 4, 2, 16, 8, 32, 16
+    q, k, v = _rand(T, Hq, Dk, seed=7), _rand(T, Hkv, Dk, seed=8), _rand(T, Hkv, Dv, seed=9)
+    Nc = O.compressed_len_conv(T, l, d)
+    ck = O.compress_meanpool(k, l, d, Nc, D64, D64)
+    cv = O.compress_meanpool(v, l, d, Nc, D64, D64)
+    got = O.compressed_attention(q, ck, cv, l, d, None, D64)
+    vis = (torch.arange(Nc)[None] * d + l) <= torch.arange(T)[:, None]        # [T,Nc]
+    G = Hq // Hkv
+    qq = q.double().transpose(0, 1)[None]                                     # [1,Hq,T,Dk]
+    kk = ck.repeat_interleave(G, 1).transpose(0, 1)[None]
+    vv = cv.repeat_interleave(G, 1).transpose(0, 1)[None]
+    rows = vis.any(-1)
+    ref = F.scaled_dot_product_attention(qq[:, :, rows], kk, vv, attn_mask=vis[rows][None, None])
+    torch.testing.assert_close(got[rows], ref[0].transpose(0, 1), rtol=1e-9, atol=1e-10)
+    assert rows[:l].sum() == 0 and rows[l:].all()
+    assert torch.count_nonzero(got[:l]) == 0
+    # row t depends only on the first n_c(t) compressed rows
+    t = 100
+    n_vis = (t - l) // d + 1
+    ck2, cv2 = ck.clone(), cv.clone()
+    ck2[n_vis:] += 3.0
+    cv2[n_vis:] -= 5.0
+    got2 = O.compressed_attention(q, ck2, cv2, l, d, None, D64)
+    torch.testing.assert_close(got2[t], got[t])
+
+
+# ---------------------------------------------------------------- selected / sliding
+def _sdpa_causal(q, k, v, mask=None):
+    G = q.shape[1] // k.shape[1]
+    qq = q.double().transpose(0, 1)[None]
+    kk = k.double().repeat_interleave(G, 1).transpose(0, 1)[None]
+    vv = v.double().repeat_interleave(G, 1).transpose(0, 1)[None]
+    if mask is None:
+        out = F.scaled_dot_product_attention(qq, kk, vv, is_causal=True)
+    else:
+        out = F.scaled_dot_product_attention(qq, kk, vv, attn_mask=mask[None, None])
+    return out[0].transpose(0, 1)
+
+
+def test_all_blocks_selected_is_causal_attention():
+    T, Hq, Hkv, Dk, Dv, bs = 96, 4, 2, 16, 8, 16
+    q, k, v = _rand(T, Hq, Dk, seed=10), _rand(T, Hkv, Dk, seed=11), _rand(T, Hkv, Dv, seed=12)
+    nb = T // bs
+    idx = torch.arange(nb).flip(0).expand(T, Hkv, nb).contiguous()
+    got = O.selected_attention(q, k, v, idx, None, bs, None, D64)
+    torch.testing.assert_close(got, _sdpa_causal(q, k, v), rtol=1e-9, atol=1e-10)
+
+
+@pytest.mark.parametrize("W", [1, 7, 32, 96, 500])
+def test_sliding_is_banded_sdpa(W):
+    T, Hq, Hkv, Dk, Dv = 96, 4, 2, 16, 8
+    q, k, v = _rand(T, Hq, Dk, seed=13), _rand(T, Hkv, Dk, seed=14), _rand(T, Hkv, Dv, seed=15)
+    got = O.sliding_attention(q, k, v, W, None, D64, row_chunk=40)
+    r, c = torch.arange(T)[:, None], torch.arange(T)[None]
+    band = (c <= r) & (c >= r - W + 1)
+    torch.testing.assert_close(got, _sdpa_causal(q, k, v, band), rtol=1e-9, atol=1e-10)
+    if W >= T:
+        torch.testing.assert_close(got, _sdpa_causal(q, k, v), rtol=1e-9, atol=1e-10)
+
+
+def test_selected_matches_token_loop_with_counts_and_poison():
+    # shaped like the reference's own test: B=1,T=64,H=1,HQ=16,D=32,S=2,bs=32, random counts,
+    # future/out-of-range ids as padding, two rows forced to an empty selection.
+    T, Hq, Hkv, D, S, bs, W = 64, 16, 1, 32, 2, 32, 128
+    q, k, v = _rand(T, Hq, D, seed=16), _rand(T, Hkv, D, seed=17), _rand(T, Hkv, D, seed=18)
+    g = torch.Generator().manual_seed(19)
+    idx = torch.full((T, Hkv, S), T, dtype=torch.int64)
+    for t in range(T):
+        perm = torch.randperm(max(1, t // bs), generator=g)[:S]
+        idx[t, 0, :len(perm)] = perm
+    idx = idx.sort(-1).values
+    idx[0, 0, 0] = 4
+    idx[63, 0, 0] = 7
+    idx[63, 0, 1] = -3
+    counts = torch.randint(1, S + 1, (T, Hkv), generator=g)
+    got_slc = O.selected_attention(q, k, v, idx, counts, bs, None, D64, row_chunk=24)
+    got_swa = O.sliding_attention(q, k, v, W, None, D64, row_chunk=24)
+    ref_slc, ref_swa = O.selected_sliding_loop(q, k, v, idx, counts, bs, W)
+    torch.testing.assert_close(got_slc, ref_slc, rtol=1e-9, atol=1e-10)
+    torch.testing.assert_close(got_swa, ref_swa, rtol=1e-9, atol=1e-10)
+    assert torch.count_nonzero(got_slc[0]) == 0 and torch.count_nonzero(got_slc[63]) == 0
+
+
+def test_token_loop_is_itself_sdpa_on_a_dense_case():
+    # guards the loop used above: with every past block listed it must be causal attention
+    T, Hq, Hkv, D, bs = 48, 2, 1, 8, 16
+    q, k, v = _rand(T, Hq, D, seed=20), _rand(T, Hkv, D, seed=21), _rand(T, Hkv, D, seed=22)
+    idx = torch.arange(T // bs).expand(T, Hkv, -1).contiguous()
+    slc, swa = O.selected_sliding_loop(q, k, v, idx, None, bs, T)
+    ref = _sdpa_causal(q, k, v)
+    torch.testing.assert_close(slc, ref, rtol=1e-9, atol=1e-10)
+    torch.testing.assert_close(swa, ref, rtol=1e-9, atol=1e-10)
+
+
+# ---------------------------------------------------------------- combine / full forward
+def test_gated_combine_closed_form():
+    a, b, c = _rand(5, 3, 4, seed=23), _rand(5, 3, 4, seed=24), _rand(5, 3, 4, seed=25)
+    g = torch.sigmoid(_rand(5, 3, 3, seed=26))
+    got = O.gated_combine(g[..., 0], a, g[..., 1], b, g[..., 2], c)
+    ref = torch.stack([a, b, c], -1) @ g.unsqueeze(-1)
+    torch.testing.assert_close(got, ref.squeeze(-1))
+
+
+def _cfg(T, Hq, Hkv, Dk, Dv, seed, dtype=torch.float32, scale=1.0):
+    q = _rand(T, Hq, Dk, seed=seed, scale=scale, dtype=dtype)
+    k = _rand(T, Hkv, Dk, seed=seed + 1, scale=scale, dtype=dtype)
+    v = _rand(T, Hkv, Dv, seed=seed + 2, scale=scale, dtype=dtype)
+    gates = torch.sigmoid(_rand(T, Hq, 3, seed=seed + 3)).to(dtype)
+    return q, k, v, gates
+
+
+def test_forward_is_sum_of_pinned_parts_and_finite():
+    p = O.NSAParams(32, 16, 64, 4, 128)
+    q, k, v, gates = _cfg(512, 4, 1, 64, 64, 30)
+    out, parts = O.nsa_forward_single(q, k, v, gates, p, return_parts=True)
+    assert torch.isfinite(out).all()
+    assert parts["idx"].shape == (512, 1, 4) and parts["pooled"].shape[-1] == 8
+    ref = (torch.stack([parts["o_slc"], parts["o_swa"], parts["o_cmp"]], -1)
+           @ gates.unsqueeze(-1)).squeeze(-1)
+    torch.testing.assert_close(out, ref, rtol=1e-5, atol=1e-6)
+    # a row whose picks are all future blocks has an exactly-zero selected branch
+    valid = (parts["idx"] * 64 <= torch.arange(512)[:, None, None]) & (parts["idx"] >= 0)
+    empty = ~valid.any(-1)[:, 0]
+    assert empty.any()
+    assert torch.count_nonzero(parts["o_slc"][empty]) == 0
+
+
+def test_varlen_is_concatenation():
+    p = O.NSAParams(32, 16, 64, 2, 64)
+    lens = [130, 64, 257]
+    cu = [0, 130, 194, 451]
+    q, k, v, gates = _cfg(sum(lens), 4, 2, 16, 16, 40)
+    packed = O.nsa_forward_varlen(q, k, v, gates, cu, p)
+    for b in range(3):
+        s, e = cu[b], cu[b + 1]
+        alone = O.nsa_forward_single(q[s:e].clone(), k[s:e].clone(), v[s:e].clone(), gates[s:e].clone(), p)
+        assert torch.equal(packed[s:e], alone)
+
+
+@pytest.mark.parametrize("ctx", [256, 250, 70, 33, 20])
+def test_decode_is_last_prefill_row(ctx):
+    p = O.NSAParams(32, 16, 64, 2, 48)
+    q, k, v, gates = _cfg(ctx, 4, 2, 16, 16, 50)
+    full, parts = O.nsa_forward_single(q, k, v, gates, p, math_dtype=D64, return_parts=True)
+    step, sp = O.nsa_decode_step(q[-1], k, v, gates[-1], p, math_dtype=D64, return_parts=True)
+    torch.testing.assert_close(step, full[-1], rtol=1e-5, atol=1e-6)
+    assert torch.equal(sp["idx"].sort(-1).values, parts["idx"][-1].sort(-1).values)
+
+
+def test_compare_selection_rule():
+    pooled = torch.tensor([[[0.5, 0.3, 0.2995, 0.1]]])
+    ref = torch.tensor([[[0, 1]]])
+    assert O.compare_selection(torch.tensor([[[1, 0]]]), ref, pooled) == (1, 1, 0, 0)
+    assert O.compare_selection(torch.tensor([[[0, 2]]]), ref, pooled) == (1, 0, 1, 0)
+    assert O.compare_selection(torch.tensor([[[0, 3]]]), ref, pooled) == (1, 0, 0, 1)
