@@ -1,0 +1,106 @@
+/* C ABI of libnsa_hip.so: the gfx950 kernels behind the NSA forward path.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless stated otherwise; the library never allocates, frees
+ *     or synchronises; work is enqueued on `stream` and outputs are fully overwritten
+ *   - tensors are packed ("varlen"): rows of all sequences back to back, `cu_seqlens` int32[batch+1]
+ *     with cu_seqlens[0] == 0 holds the row offsets; a batch of equal lengths is the special case
+ *     cu_seqlens[b] = b*T
+ *   - dtype: NSA_BF16 or NSA_F32 for every floating tensor of a call (accumulation is always fp32)
+ *   - return value: 0 on success, negative on error (NSA_ERR_*); nsa_last_error_string() describes
+ *     the last error of the calling thread.  No exception crosses this boundary.
+ *   - "transposed" buffers hold one key-contiguous plane per head: element (h, d, col) lives at
+ *     (h*dim + d)*cols + col, sequence b starts at column nsa_transposed_offset(cu[b], b) and
+ *     `cols` = nsa_transposed_cols(total_rows, batch).  They are produced by nsa_transpose_fwd.
+ *
+ * The reference (yukavio/nsa) has no FFI layer; each entry point names the Python/Triton interface
+ * of the reference it stands behind (file:line inside the reference tree).
+ */
+#ifndef NSA_HIP_H
+#define NSA_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ihipStream_t* nsa_stream_t; /* hipStream_t */
+
+enum { NSA_BF16 = 0, NSA_F32 = 1 };
+enum {
+  NSA_OK = 0,
+  NSA_ERR_INVALID = -1,     /* bad argument (null pointer, non-positive size, misalignment) */
+  NSA_ERR_UNSUPPORTED = -2, /* shape outside what the kernels are built for */
+  NSA_ERR_RESOURCE = -3,    /* needs more LDS than a gfx950 CU has */
+  NSA_ERR_LAUNCH = -4       /* HIP reported a launch failure */
+};
+enum { NSA_GATE_IDENTITY = 0, NSA_GATE_SIGMOID = 1 };
+
+int nsa_version(void);
+const char* nsa_last_error_string(void);
+
+/* Column bookkeeping of transposed buffers (host helpers, pure arithmetic). */
+int nsa_transposed_offset(int cu_b, int b);
+int nsa_transposed_cols(int total_rows, int batch);
+
+/* KV block compression.  Replaces nsa/compression_kv.py:21-57 (_compress_fwd), :178-217
+ * (_compress_kv.forward) and the two nn.Conv1d calls of KVCompressor.forward (:301-307).
+ *   x      [total, heads, dim]        out [out_rows, heads, dim]
+ *   wt     NULL -> mean over the window (eye/block weights, no bias); otherwise the weight as
+ *          [dim_out = dim][block*dim] with wt[o][j*dim + i] = W_conv[o][i][j] = W_lin[j*dim+i][o]
+ *   bias   [dim] or NULL
+ *   cu_out int32[batch+1] offsets of every sequence's rows in `out`; row n of a sequence covers
+ *          its tokens [n*stride, n*stride + block).  out_rows_bound >= cu_out[batch] sizes the grid. */
+int nsa_compress_fwd(const void* x, const void* wt, const void* bias, void* out,
+                     const int32_t* cu_seqlens, const int32_t* cu_out, int batch, int out_rows_bound,
+                     int heads, int dim, int block, int stride, int dtype, nsa_stream_t stream);
+
+/* Key-contiguous copy of a packed [rows, heads, dim] tensor (row_stride / head_stride in elements).
+ * Layout preparation for the MFMA PV product; no counterpart in the reference. */
+int nsa_transpose_fwd(const void* x, void* out, const int32_t* cu, int batch, int heads, int dim,
+                      int64_t row_stride, int64_t head_stride, int out_cols, int dtype,
+                      nsa_stream_t stream);
+
+/* Compressed attention fused with block-importance scoring and top-n selection.  Replaces
+ * nsa/triton_attention.py:419-476 (_attention.forward: _attn_fwd, softmax_kernel, sum / avg_pool1d /
+ * topk) with the semantics of nsa/torch_attention.py:66-163 (attention_ref, get_indices).
+ *   q [total, hq, dk]; ck rows at ck + (cu_cmp[b] + c)*ck_row_stride + h*ck_head_stride (dk elements);
+ *   cvt transposed [hkv][dv][cvt_cols] over cu_cmp; o [total, hq, dv];
+ *   indices [total, hkv, top_n] int32 or int64 (idx64), descending score, -1 where fewer bins exist;
+ *   NULL skips the selection;  pooled (optional, float) [total, hkv, pooled_stride] block scores.
+ *   Compressed row c of a sequence is visible to token t iff c*stride + block <= t (causal != 0;
+ *   causal == 0 makes every row visible).
+ *   max_ns >= pooled bins of the longest sequence (sizes LDS). */
+int nsa_cmp_attn_select_fwd(const void* q, const void* ck, const void* cvt, void* o, void* indices,
+                            float* pooled, const int32_t* cu_seqlens, const int32_t* cu_cmp, int batch,
+                            int total, int hq, int hkv, int dk, int dv, int64_t ck_row_stride,
+                            int64_t ck_head_stride, int cvt_cols, int block, int stride, int pool_kernel,
+                            int pool_stride, int pool_pad, int top_n, int max_ns, int pooled_stride,
+                            float scale, int causal, int idx64, int dtype, nsa_stream_t stream);
+
+/* Sliding window attention: token t attends keys [max(0, t-window+1), t] of its sequence.  Replaces
+ * the window loop of nsa/selection_attn.py:483-517.  q [total,hq,dk], k [total,hkv,dk],
+ * vt transposed [hkv][dv][vt_cols] over cu_seqlens, o [total,hq,dv]. */
+int nsa_swa_fwd(const void* q, const void* k, const void* vt, void* o, const int32_t* cu_seqlens,
+                int batch, int total, int hq, int hkv, int dk, int dv, int vt_cols, int window,
+                float scale, int dtype, nsa_stream_t stream);
+
+/* Selected-block attention with the gated combine of the branches in the epilogue.  Replaces
+ * nsa/selection_attn.py:401-481 (parallel_nsa_fwd_kernel, selected part), :808-811 and nsa/nsa.py:133.
+ *   indices [total, hkv, top_n] block numbers local to the sequence (int32 / int64); entry i of
+ *   token t is used iff i < counts[t,h] (counts NULL -> top_n), 0 <= idx and idx*block_size <= t.
+ *   out = act(g_slc)*o_slc + act(g_swa)*o_swa + act(g_cmp)*o_cmp, where o_swa / o_cmp
+ *   [total,hq,dv] may be NULL (term dropped), a NULL gate means 1, and gate (t,hq) is read at
+ *   g[(t*hq + hq_idx)*gate_stride].  A token with no usable block has o_slc = 0. */
+int nsa_slc_combine_fwd(const void* q, const void* k, const void* vt, const void* indices,
+                        const int32_t* counts, const void* g_slc, const void* g_swa, const void* g_cmp,
+                        int64_t gate_stride, const void* o_swa, const void* o_cmp, void* out,
+                        const int32_t* cu_seqlens, int batch, int total, int hq, int hkv, int dk, int dv,
+                        int vt_cols, int top_n, int block_size, float scale, int idx64, int gate_act,
+                        int dtype, nsa_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NSA_HIP_H */

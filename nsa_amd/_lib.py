@@ -1,0 +1,67 @@
+"""ctypes binding of libnsa_hip.so (the C ABI declared in include/nsa_hip.h).
+
+There is no fallback: if the library is missing every op raises.  Build it with
+`python -m nsa_amd.build` (hipcc, gfx950).
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libnsa_hip.so")
+
+NSA_BF16, NSA_F32 = 0, 1
+GATE_IDENTITY, GATE_SIGMOID = 0, 1
+
+_P, _I, _L, _F = C.c_void_p, C.c_int, C.c_int64, C.c_float
+
+# name -> (restype, argtypes); mirrors include/nsa_hip.h one to one
+SIGNATURES = {
+    "nsa_version": (_I, []),
+    "nsa_last_error_string": (C.c_char_p, []),
+    "nsa_transposed_offset": (_I, [_I, _I]),
+    "nsa_transposed_cols": (_I, [_I, _I]),
+    "nsa_compress_fwd": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
+    "nsa_transpose_fwd": (_I, [_P, _P, _P, _I, _I, _I, _L, _L, _I, _I, _P]),
+    "nsa_cmp_attn_select_fwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _L, _I,
+                                     _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P]),
+    "nsa_swa_fwd": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P]),
+    "nsa_slc_combine_fwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _L, _P, _P, _P, _P, _I, _I, _I, _I, _I,
+                                 _I, _I, _I, _I, _F, _I, _I, _I, _P]),
+}
+
+_lib = None
+
+
+class NSALibraryError(RuntimeError):
+    pass
+
+
+def load():
+    """Loads the shared library once; raises NSALibraryError when it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise NSALibraryError(
+            "libnsa_hip.so not found at %s - run `python -m nsa_amd.build` (needs hipcc). "
+            "There is no CPU or PyTorch fallback for the NSA kernels." % LIB_PATH)
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(rc: int, what: str):
+    if rc == 0:
+        return
+    msg = load().nsa_last_error_string().decode("utf-8", "replace")
+    if rc in (-1,):
+        raise ValueError("%s: %s" % (what, msg))
+    if rc == -2:
+        raise NotImplementedError("%s: %s" % (what, msg))
+    raise RuntimeError("%s failed (%d): %s" % (what, rc, msg))

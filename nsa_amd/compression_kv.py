@@ -1,0 +1,119 @@
+"""KV block compression with the interface of the reference's nsa/compression_kv.py.
+
+calc_compressed_len (compression_kv.py:9-10), compress_kv (:178-217, :269), KVCompressorVarlen
+(:272-289) and KVCompressor (:292-312) keep their names, argument order, parameter names/shapes and
+return arity.  The arithmetic runs in the HIP kernels of libnsa_hip.so; forward only.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+import torch.nn as nn
+from torch.nn import init
+
+from . import ops
+
+
+def calc_compressed_len(x, stride, size):
+    """Rows the functional compressor emits for a sequence of x tokens (one fewer than a Conv1d)."""
+    return (x - size) // stride
+
+
+def conv_compressed_len(x, stride, size):
+    """Rows nn.Conv1d(kernel=size, stride=stride) emits for x tokens."""
+    return 0 if x < size else (x - size) // stride + 1
+
+
+@torch.no_grad()
+def compress_kv(k, v, w_k, w_v, cu_seq_len, block_stride, block_size):
+    """k, v [total, H, D]; w_* [block_size*D, D] (row j*D+i); cu_seq_len int32 [B+1].
+    Returns (ck, cv, cu_out_len): bf16 [sum Nc', H, D] with Nc' = (T - block_size)//block_stride."""
+    cu = cu_seq_len.to(torch.int32)
+    cu_out = ops.compressed_offsets(cu, block_size, block_stride, extra=0)
+    out_rows = int(cu_out[-1].item())      # the reference syncs here as well (cu_seq_len.tolist())
+    wk_t = w_k.detach().t().contiguous()
+    wv_t = w_v.detach().t().contiguous()
+    kk = k if k.dtype in (torch.bfloat16, torch.float32) else k.to(torch.bfloat16)
+    vv = v if v.dtype in (torch.bfloat16, torch.float32) else v.to(torch.bfloat16)
+    ck = ops.compress(kk, cu, cu_out, out_rows, block_size, block_stride, wk_t)
+    cv = ops.compress(vv, cu, cu_out, out_rows, block_size, block_stride, wv_t)
+    return ck.to(torch.bfloat16), cv.to(torch.bfloat16), cu_out
+
+
+class KVCompressorVarlen(nn.Module):
+    def __init__(self, block_stride, block_size, head_dim, device, dtype):
+        factory_kwargs = {"device": device, "dtype": dtype}
+        super().__init__()
+        self.block_stride = block_stride
+        self.block_size = block_size
+        self.k_weight = nn.Parameter(torch.empty(block_size * head_dim, head_dim, **factory_kwargs))
+        self.v_weight = nn.Parameter(torch.empty(block_size * head_dim, head_dim, **factory_kwargs))
+        self.reset_parameters()
+
+    def forward(self, k, v, cu_seq_len, group=None):
+        return compress_kv(k, v, self.k_weight, self.v_weight, cu_seq_len, self.block_stride, self.block_size)
+
+    def reset_parameters(self) -> None:
+        init.kaiming_uniform_(self.k_weight, a=math.sqrt(5))
+        init.kaiming_uniform_(self.v_weight, a=math.sqrt(5))
+
+
+class KVCompressor(nn.Module):
+    """Conv1d-parameterised compressor (weight [D, D, block], bias [D], shared over heads).
+
+    mode="conv" is the reference; mode="mean" ignores the parameters and averages each window
+    (the conv with eye/block weights and zero bias)."""
+
+    def __init__(self, block_stride, block_size, head_dim, device=None, dtype=None, mode: str = "conv"):
+        super().__init__()
+        factory_kwargs = {"device": device, "dtype": dtype}
+        self.block_stride = block_stride
+        self.block_size = block_size
+        self.mode = mode
+        self.compressor_k = nn.Conv1d(head_dim, head_dim, block_size, block_stride, **factory_kwargs)
+        self.compressor_v = nn.Conv1d(head_dim, head_dim, block_size, block_stride, **factory_kwargs)
+
+    def _wt(self, conv: nn.Conv1d) -> torch.Tensor:
+        # [o, i, j] -> [o, j*D + i]
+        w = conv.weight.detach()
+        return w.permute(0, 2, 1).reshape(w.shape[0], -1).contiguous()
+
+    @torch.no_grad()
+    def compress_packed(self, k, v, cu_seq_len, seq_len: Optional[int] = None):
+        """Un-repeated result: (ck, cv [sum Nc, H, D], cu_cmp int32 [B+1], max Nc or None)."""
+        cu = cu_seq_len.to(torch.int32)
+        batch = cu.numel() - 1
+        if seq_len is not None:
+            nc = conv_compressed_len(seq_len, self.block_stride, self.block_size)
+            cu_out = ops.uniform_cu(batch, nc, k.device)
+            rows = nc * batch
+        else:
+            cu_out = ops.compressed_offsets(cu, self.block_size, self.block_stride, extra=1)
+            rows = k.shape[0] // self.block_stride + batch
+            nc = None
+        if self.mode == "mean":
+            ck = ops.compress(k, cu, cu_out, rows, self.block_size, self.block_stride)
+            cv = ops.compress(v, cu, cu_out, rows, self.block_size, self.block_stride)
+        else:
+            ck = ops.compress(k, cu, cu_out, rows, self.block_size, self.block_stride,
+                              self._wt(self.compressor_k), self.compressor_k.bias)
+            cv = ops.compress(v, cu, cu_out, rows, self.block_size, self.block_stride,
+                              self._wt(self.compressor_v), self.compressor_v.bias)
+        return ck, cv, cu_out, nc
+
+    def forward(self, k, v, cu_seq_len, group=None):
+        """k, v [B*T, H, D] with B = len(cu_seq_len)-1 equal-length sequences.
+        Returns (ck, cv [B, Nc, H*group, D], cu_seq_len) like the reference."""
+        BT, H, D = k.shape
+        B = cu_seq_len.shape[0] - 1
+        T = BT // B
+        cu = ops.uniform_cu(B, T, k.device)
+        ck, cv, _, nc = self.compress_packed(k, v, cu, seq_len=T)
+        ck = ck.view(B, nc, H, D)
+        cv = cv.view(B, nc, H, v.shape[-1])
+        if group is not None:
+            ck = ck.repeat_interleave(group, dim=2)
+            cv = cv.repeat_interleave(group, dim=2)
+        return ck, cv, cu_seq_len

@@ -1,0 +1,142 @@
+// extern "C" boundary of libnsa_hip.so: argument checks, error strings, dispatch to the launchers.
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/nsa_hip.h"
+#include "common.h"
+#include "kernels.h"
+
+namespace {
+
+thread_local char g_err[256] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int finish(int rc, const char* what) {
+  if (rc == -2) return fail(NSA_ERR_UNSUPPORTED, "%s: head dims not built (dk,dv in (32,32),(64,64),(128,128),(192,128))", what);
+  if (rc == -3) return fail(NSA_ERR_RESOURCE, "%s: needs more than 160 KB of LDS (sequence too long)", what);
+  if (rc != 0) return fail(NSA_ERR_LAUNCH, "%s: could not configure the kernel", what);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(NSA_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+  return NSA_OK;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+int check_heads(const char* what, int hq, int hkv, int dk, int dv) {
+  if (hq <= 0 || hkv <= 0 || hq % hkv != 0) return fail(NSA_ERR_INVALID, "%s: hq must be a positive multiple of hkv", what);
+  if (hq / hkv > 16) return fail(NSA_ERR_UNSUPPORTED, "%s: GQA group size %d > 16 is not built", what, hq / hkv);
+  if (dk % 32 != 0 || dv % 16 != 0) return fail(NSA_ERR_UNSUPPORTED, "%s: dk must be a multiple of 32 and dv of 16", what);
+  return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int nsa_version(void) { return 100; }
+const char* nsa_last_error_string(void) { return g_err; }
+
+int nsa_transposed_offset(int cu_b, int b) { return nsa::transposed_offset(cu_b, b); }
+int nsa_transposed_cols(int total_rows, int batch) {
+  const int need = nsa::transposed_offset(total_rows, batch) + 64;
+  return (need + 63) / 64 * 64;
+}
+
+int nsa_compress_fwd(const void* x, const void* wt, const void* bias, void* out, const int32_t* cu_seqlens,
+                     const int32_t* cu_out, int batch, int out_rows_bound, int heads, int dim, int block,
+                     int stride, int dtype, nsa_stream_t stream) {
+  if (!x || !out || !cu_seqlens || !cu_out) return fail(NSA_ERR_INVALID, "compress: null pointer");
+  if (batch <= 0 || heads <= 0 || block <= 0 || stride <= 0 || out_rows_bound < 0)
+    return fail(NSA_ERR_INVALID, "compress: sizes must be positive");
+  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "compress: bad dtype");
+  if (dim % 8 != 0) return fail(NSA_ERR_UNSUPPORTED, "compress: dim must be a multiple of 8");
+  if (!aligned16(x) || !aligned16(out) || (wt && !aligned16(wt))) return fail(NSA_ERR_INVALID, "compress: pointers must be 16-byte aligned");
+  if (wt && dim % 32 != 0) return fail(NSA_ERR_UNSUPPORTED, "compress: weighted path needs dim %% 32 == 0");
+  nsa::CompressArgs a{x, wt, bias, out, cu_seqlens, cu_out, batch, out_rows_bound, heads, dim, block, stride, dtype};
+  const int rc = nsa::launch_compress(a, stream);
+  if (rc == -2) return fail(NSA_ERR_UNSUPPORTED, "compress: weighted path is built for dim 32/64/128/192");
+  return finish(rc, "compress");
+}
+
+int nsa_transpose_fwd(const void* x, void* out, const int32_t* cu, int batch, int heads, int dim,
+                      int64_t row_stride, int64_t head_stride, int out_cols, int dtype, nsa_stream_t stream) {
+  if (!x || !out || !cu) return fail(NSA_ERR_INVALID, "transpose: null pointer");
+  if (batch <= 0 || heads <= 0 || dim <= 0 || dim % 8 != 0 || out_cols <= 0 || out_cols % 64 != 0)
+    return fail(NSA_ERR_INVALID, "transpose: dim must be a multiple of 8 and out_cols of 64");
+  if (row_stride % 8 != 0 || head_stride % 8 != 0 || !aligned16(x) || !aligned16(out))
+    return fail(NSA_ERR_INVALID, "transpose: strides must be multiples of 8 elements, pointers 16-byte aligned");
+  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "transpose: bad dtype");
+  nsa::TransposeArgs a{x, out, cu, batch, heads, dim, (long)row_stride, (long)head_stride, out_cols, dtype};
+  return finish(nsa::launch_transpose(a, stream), "transpose");
+}
+
+int nsa_cmp_attn_select_fwd(const void* q, const void* ck, const void* cvt, void* o, void* indices,
+                            float* pooled, const int32_t* cu_seqlens, const int32_t* cu_cmp, int batch,
+                            int total, int hq, int hkv, int dk, int dv, int64_t ck_row_stride,
+                            int64_t ck_head_stride, int cvt_cols, int block, int stride, int pool_kernel,
+                            int pool_stride, int pool_pad, int top_n, int max_ns, int pooled_stride,
+                            float scale, int causal, int idx64, int dtype, nsa_stream_t stream) {
+  if (!q || !ck || !cvt || !o || !cu_seqlens || !cu_cmp) return fail(NSA_ERR_INVALID, "cmp_attn_select: null pointer");
+  if (batch <= 0 || total <= 0 || block <= 0 || stride <= 0) return fail(NSA_ERR_INVALID, "cmp_attn_select: sizes must be positive");
+  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "cmp_attn_select: bad dtype");
+  if (int rc = check_heads("cmp_attn_select", hq, hkv, dk, dv)) return rc;
+  if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "cmp_attn_select: scale must be positive");
+  if (ck_row_stride % 8 != 0 || ck_head_stride % 8 != 0 || cvt_cols % 64 != 0)
+    return fail(NSA_ERR_INVALID, "cmp_attn_select: ck strides must be multiples of 8, cvt_cols of 64");
+  if (!aligned16(q) || !aligned16(ck) || !aligned16(cvt) || !aligned16(o))
+    return fail(NSA_ERR_INVALID, "cmp_attn_select: pointers must be 16-byte aligned");
+  if (indices) {
+    if (pool_kernel <= 0 || pool_stride <= 0 || pool_pad < 0 || pool_pad >= pool_kernel || top_n <= 0 || max_ns < 0)
+      return fail(NSA_ERR_INVALID, "cmp_attn_select: bad pooling / top-n parameters");
+    if (pooled && pooled_stride < max_ns) return fail(NSA_ERR_INVALID, "cmp_attn_select: pooled_stride < max_ns");
+  } else {
+    max_ns = 0;
+  }
+  nsa::CmpArgs a{q, ck, cvt, o, indices, pooled, cu_seqlens, cu_cmp, batch, total, hq, hkv, dk, dv,
+                 (long)ck_row_stride, (long)ck_head_stride, cvt_cols, block, stride, pool_kernel, pool_stride,
+                 pool_pad, top_n, max_ns, pooled_stride, scale, idx64, dtype, causal};
+  return finish(nsa::launch_cmp_select(a, stream), "cmp_attn_select");
+}
+
+int nsa_swa_fwd(const void* q, const void* k, const void* vt, void* o, const int32_t* cu_seqlens, int batch,
+                int total, int hq, int hkv, int dk, int dv, int vt_cols, int window, float scale, int dtype,
+                nsa_stream_t stream) {
+  if (!q || !k || !vt || !o || !cu_seqlens) return fail(NSA_ERR_INVALID, "swa: null pointer");
+  if (batch <= 0 || total <= 0 || window <= 0) return fail(NSA_ERR_INVALID, "swa: sizes must be positive");
+  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "swa: bad dtype");
+  if (int rc = check_heads("swa", hq, hkv, dk, dv)) return rc;
+  if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "swa: scale must be positive");
+  if (vt_cols % 64 != 0 || vt_cols < nsa_transposed_cols(total, batch)) return fail(NSA_ERR_INVALID, "swa: vt_cols too small or not a multiple of 64");
+  if (!aligned16(q) || !aligned16(k) || !aligned16(vt) || !aligned16(o)) return fail(NSA_ERR_INVALID, "swa: pointers must be 16-byte aligned");
+  nsa::SwaArgs a{q, k, vt, o, cu_seqlens, batch, total, hq, hkv, dk, dv, vt_cols, window, scale, dtype};
+  return finish(nsa::launch_swa(a, stream), "swa");
+}
+
+int nsa_slc_combine_fwd(const void* q, const void* k, const void* vt, const void* indices, const int32_t* counts,
+                        const void* g_slc, const void* g_swa, const void* g_cmp, int64_t gate_stride,
+                        const void* o_swa, const void* o_cmp, void* out, const int32_t* cu_seqlens, int batch,
+                        int total, int hq, int hkv, int dk, int dv, int vt_cols, int top_n, int block_size,
+                        float scale, int idx64, int gate_act, int dtype, nsa_stream_t stream) {
+  if (!q || !k || !vt || !indices || !out || !cu_seqlens) return fail(NSA_ERR_INVALID, "slc_combine: null pointer");
+  if (batch <= 0 || total <= 0) return fail(NSA_ERR_INVALID, "slc_combine: sizes must be positive");
+  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "slc_combine: bad dtype");
+  if (int rc = check_heads("slc_combine", hq, hkv, dk, dv)) return rc;
+  if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "slc_combine: scale must be positive");
+  if (top_n <= 0 || top_n > 64) return fail(NSA_ERR_UNSUPPORTED, "slc_combine: 1 <= top_n <= 64");
+  if (block_size <= 0 || block_size % 8 != 0) return fail(NSA_ERR_UNSUPPORTED, "slc_combine: block_size must be a multiple of 8");
+  if (vt_cols % 64 != 0 || vt_cols < nsa_transposed_cols(total, batch)) return fail(NSA_ERR_INVALID, "slc_combine: vt_cols too small or not a multiple of 64");
+  if (gate_act != NSA_GATE_IDENTITY && gate_act != NSA_GATE_SIGMOID) return fail(NSA_ERR_INVALID, "slc_combine: bad gate activation");
+  if (!aligned16(q) || !aligned16(k) || !aligned16(vt)) return fail(NSA_ERR_INVALID, "slc_combine: pointers must be 16-byte aligned");
+  nsa::SlcArgs a{q, k, vt, indices, counts, g_slc, g_swa, g_cmp, (long)gate_stride, o_swa, o_cmp, out, cu_seqlens,
+                 batch, total, hq, hkv, dk, dv, vt_cols, top_n, block_size, scale, idx64, gate_act, dtype};
+  return finish(nsa::launch_slc_combine(a, stream), "slc_combine");
+}
+
+}  // extern "C"

@@ -1,0 +1,173 @@
+// Shared device helpers for the gfx950 NSA kernels: 16x16 MFMA tiles on 64-wide wavefronts.
+//
+// Fragment convention used by every attention kernel here ("transposed scores"):
+//   S^T[key][row] = sum_d K[key][d] * Q[row][d]
+//     A operand = K rows   : lane (m = lane%16, g = lane/16) holds K[key(m)][32*kk + 8g .. +7]
+//     B operand = Q rows   : lane (n = lane%16, g)           holds Q[row n][32*kk + 8g .. +7]
+//     C tile               : lane (n, g) holds S^T[key 4g+i][row n], i = 0..3
+//   A 32-key chunk is two such tiles whose A rows are permuted (tile0 row m -> key 8*(m/4)+m%4,
+//   tile1 -> +4) so that lane (n, g) ends up with the 8 *contiguous* keys 8g..8g+7 of the chunk.
+//   Those 8 probabilities are then directly the B operand of
+//   O^T[dv][row] = sum_key V^T[dv][key] * P^T[key][row]
+//     A operand = V^T rows : lane (m = dv%16, g) holds V^T[dv][chunk + 8g .. +7]  (16 B contiguous)
+//   so P never leaves registers and V is consumed from a key-contiguous (transposed) layout.
+// fp32 inputs use the same fragments with eight v_mfma_f32_16x16x4_f32 per step.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace nsa {
+
+typedef __bf16 bf16_t;
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x8_t __attribute__((ext_vector_type(8)));
+
+constexpr int kWave = 64;
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kNegInf = -__builtin_huge_valf();
+
+template <typename T> struct Vec8;
+template <> struct Vec8<bf16_t> { using type = bf16x8_t; };
+template <> struct Vec8<float> { using type = f32x8_t; };
+template <typename T> using vec8_t = typename Vec8<T>::type;
+
+__device__ __forceinline__ f32x4_t mma16(bf16x8_t a, bf16x8_t b, f32x4_t c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4_t mma16(f32x8_t a, f32x8_t b, f32x4_t c) {
+#pragma unroll
+  for (int j = 0; j < 8; ++j) c = __builtin_amdgcn_mfma_f32_16x16x4f32(a[j], b[j], c, 0, 0, 0);
+  return c;
+}
+
+// 8 consecutive elements; p must be 16-byte aligned.
+__device__ __forceinline__ bf16x8_t load8(const bf16_t* p) {
+  return *reinterpret_cast<const bf16x8_t*>(p);
+}
+__device__ __forceinline__ f32x8_t load8(const float* p) {
+  const f32x4_t a = *reinterpret_cast<const f32x4_t*>(p);
+  const f32x4_t b = *reinterpret_cast<const f32x4_t*>(p + 4);
+  f32x8_t r;
+  r[0] = a[0]; r[1] = a[1]; r[2] = a[2]; r[3] = a[3];
+  r[4] = b[0]; r[5] = b[1]; r[6] = b[2]; r[7] = b[3];
+  return r;
+}
+__device__ __forceinline__ void store8(bf16_t* p, bf16x8_t v) {
+  *reinterpret_cast<bf16x8_t*>(p) = v;
+}
+__device__ __forceinline__ void store8(float* p, f32x8_t v) {
+  f32x4_t a, b;
+  a[0] = v[0]; a[1] = v[1]; a[2] = v[2]; a[3] = v[3];
+  b[0] = v[4]; b[1] = v[5]; b[2] = v[6]; b[3] = v[7];
+  *reinterpret_cast<f32x4_t*>(p) = a;
+  *reinterpret_cast<f32x4_t*>(p + 4) = b;
+}
+
+template <typename T> __device__ __forceinline__ vec8_t<T> zero8() {
+  vec8_t<T> r;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) r[i] = (T)0.0f;
+  return r;
+}
+template <typename T> __device__ __forceinline__ vec8_t<T> pack8(const float (&p)[8]) {
+  vec8_t<T> r;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) r[i] = (T)p[i];
+  return r;
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// A-operand row m of tile `tile` (0/1) of a 32-key chunk -> key offset inside the chunk.
+__device__ __forceinline__ int chunk_key_of_row(int tile, int m) {
+  return 8 * (m >> 2) + (m & 3) + 4 * tile;
+}
+
+// Butterfly over the four lanes that share one tile column (lane%16).
+__device__ __forceinline__ float colgroup_max(float x) {
+  x = fmaxf(x, __shfl_xor(x, 16));
+  x = fmaxf(x, __shfl_xor(x, 32));
+  return x;
+}
+__device__ __forceinline__ float colgroup_sum(float x) {
+  x += __shfl_xor(x, 16);
+  x += __shfl_xor(x, 32);
+  return x;
+}
+
+// Column offset of sequence b inside a key-contiguous ("transposed") buffer: every sequence starts
+// on a multiple of 8 elements so that 8-key fragments are 16-byte aligned.
+__host__ __device__ __forceinline__ int transposed_offset(int cu_b, int b) {
+  return ((cu_b + 7) & ~7) + 8 * b;
+}
+
+// Sequence / tile lookup for packed (varlen) inputs.  Tiles of `tq` tokens are numbered sequence
+// after sequence; a tile index past the last one yields valid = false.
+struct SeqTile {
+  int b, t0, start, len;
+  bool valid;
+};
+__device__ __forceinline__ SeqTile find_tile(const int32_t* __restrict__ cu, int batch, int tq, int tile) {
+  SeqTile r;
+  r.valid = false;
+  r.b = 0; r.t0 = 0; r.start = 0; r.len = 0;
+  int prev = cu[0];
+  for (int b = 0; b < batch; ++b) {
+    const int next = cu[b + 1];
+    const int len = next - prev;
+    const int nt = (len + tq - 1) / tq;
+    if (tile < nt) {
+      r.b = b; r.t0 = tile * tq; r.start = prev; r.len = len; r.valid = true;
+      return r;
+    }
+    tile -= nt;
+    prev = next;
+  }
+  return r;
+}
+
+// Per-row-group state of the online softmax.  One group = 16 rows = the 16 columns of a tile.
+template <typename T, int DK, int DV>
+struct RowGroup {
+  vec8_t<T> q[DK / 32];
+  f32x4_t o[DV / 16];
+  float m;  // running maximum of the raw (unscaled) visible scores of column lane%16
+  float l;  // this lane's share of the running denominator
+};
+
+template <typename T, int DK, int DV>
+__device__ __forceinline__ void group_reset(RowGroup<T, DK, DV>& g) {
+#pragma unroll
+  for (int i = 0; i < DV / 16; ++i) g.o[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  g.m = kNegInf;
+  g.l = 0.f;
+}
+
+// Online-softmax update for the 8 scores a lane holds of one 32-key chunk (masked entries are
+// -inf).  Returns the probabilities in p (unnormalised) and rescales the accumulator.
+template <typename T, int DK, int DV>
+__device__ __forceinline__ void softmax_update(RowGroup<T, DK, DV>& g, const float (&s)[8], float c,
+                                               float (&p)[8]) {
+  float mx = s[0];
+#pragma unroll
+  for (int i = 1; i < 8; ++i) mx = fmaxf(mx, s[i]);
+  mx = colgroup_max(mx);
+  const float m_new = fmaxf(g.m, mx);
+  const float mref = (m_new == kNegInf) ? 0.f : m_new;
+  const float alpha = fast_exp2((g.m - mref) * c);
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    p[i] = fast_exp2((s[i] - mref) * c);
+    sum += p[i];
+  }
+  g.l = g.l * alpha + sum;
+  g.m = m_new;
+#pragma unroll
+  for (int i = 0; i < DV / 16; ++i) {
+    g.o[i][0] *= alpha; g.o[i][1] *= alpha; g.o[i][2] *= alpha; g.o[i][3] *= alpha;
+  }
+}
+
+}  // namespace nsa

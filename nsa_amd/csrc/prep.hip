@@ -1,0 +1,188 @@
+// KV block compression and the key-contiguous ("transposed") copy the attention kernels read V from.
+//
+// compress (mean-pool): pure HBM streaming. One thread owns 8 contiguous channels of one output
+//   row; consecutive threads cover one full [heads*dim] token row, so every load instruction of a
+//   wavefront reads whole contiguous token rows. Each input row is needed by block/stride output
+//   rows; the second use hits L2. Algorithmic bytes: rows_in*heads*dim*sizeof(T) read +
+//   rows_out*heads*dim*sizeof(T) written.
+// compress (weighted): out[n][o] = b[o] + sum_{j,i} x[n*stride+j][i] * Wt[o][j*dim+i] as an MFMA
+//   GEMM with the [dim_out x block*dim] weight (L2 resident) as the A operand.
+// transpose: out[h][d][col] = x[row(col)][h][d], 64-column tiles through LDS.
+#include "common.h"
+#include "kernels.h"
+
+namespace nsa {
+
+__device__ __forceinline__ int upper_seq(const int32_t* __restrict__ cu, int batch, int r) {
+  // largest b in [0,batch) with cu[b] <= r   (cu non-decreasing, cu[0] <= r assumed)
+  int lo = 0, hi = batch;  // invariant: cu[lo] <= r, answer in [lo, hi)
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (cu[mid] <= r) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+compress_mean_kernel(const T* __restrict__ x, T* __restrict__ out, const int32_t* __restrict__ cu_seq,
+                     const int32_t* __restrict__ cu_out, int batch, int heads, int dim, int block,
+                     int stride) {
+  const int ppr = heads * dim / 8;  // 8-element pieces per token row
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  const int r = (int)(idx / ppr);
+  const int piece = (int)(idx % ppr);
+  if (r >= cu_out[batch]) return;
+  const int b = upper_seq(cu_out, batch, r);
+  const int n = r - cu_out[b];
+  const T* src = x + ((long)cu_seq[b] + (long)n * stride) * (heads * dim) + piece * 8;
+  float acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+#pragma unroll 4
+  for (int j = 0; j < block; ++j) {
+    const vec8_t<T> v = load8(src + (long)j * heads * dim);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] += (float)v[i];
+  }
+  const float inv = 1.0f / (float)block;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc[i] *= inv;
+  store8(out + (long)r * heads * dim + piece * 8, pack8<T>(acc));
+}
+
+template <typename T, int DIM>
+__global__ void __launch_bounds__(256)
+compress_weighted_kernel(const T* __restrict__ x, const T* __restrict__ wt, const T* __restrict__ bias,
+                         T* __restrict__ out, const int32_t* __restrict__ cu_seq,
+                         const int32_t* __restrict__ cu_out, int batch, int heads, int block, int stride) {
+  const int lane = threadIdx.x & 63;
+  const int n = lane & 15, g = lane >> 4;
+  const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int total_out = cu_out[batch];
+  const int ntile = (total_out + 15) / 16;
+  const int tile = wave / heads, h = wave % heads;
+  if (tile >= ntile) return;
+  const int r = tile * 16 + n;
+  const bool live = r < total_out;
+  const int rc = live ? r : total_out - 1;
+  const int b = upper_seq(cu_out, batch, rc);
+  const T* xrow = x + (((long)cu_seq[b] + (long)(rc - cu_out[b]) * stride) * heads + h) * DIM;
+  f32x4_t acc[DIM / 16];
+#pragma unroll
+  for (int i = 0; i < DIM / 16; ++i) acc[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const int K = block * DIM;
+  for (int j = 0; j < block; ++j) {
+#pragma unroll
+    for (int i0 = 0; i0 < DIM; i0 += 32) {
+      const vec8_t<T> xb = load8(xrow + (long)j * heads * DIM + i0 + 8 * g);
+      const int k0 = j * DIM + i0 + 8 * g;
+#pragma unroll
+      for (int t = 0; t < DIM / 16; ++t) {
+        const vec8_t<T> wa = load8(wt + (long)(t * 16 + n) * K + k0);
+        acc[t] = mma16(wa, xb, acc[t]);
+      }
+    }
+  }
+  if (!live) return;
+  T* orow = out + ((long)r * heads + h) * DIM;
+#pragma unroll
+  for (int t = 0; t < DIM / 16; ++t) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int o = t * 16 + 4 * g + i;
+      float v = acc[t][i];
+      if (bias != nullptr) v += (float)bias[o];
+      orow[o] = (T)v;
+    }
+  }
+}
+
+// out[(h*dim + d) * out_cols + col], col = transposed_offset(cu[b], b) + row; every other column is 0.
+template <typename T>
+__global__ void __launch_bounds__(256)
+transpose_kernel(const T* __restrict__ x, T* __restrict__ out, const int32_t* __restrict__ cu, int batch,
+                 int dim, long row_stride, long head_stride, int out_cols) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  int* src_row = reinterpret_cast<int*>(smem_raw);           // [64]
+  T* tile = reinterpret_cast<T*>(smem_raw + 64 * sizeof(int));  // [64][dim + 8]
+  const int ld = dim + 8;
+  const int col0 = blockIdx.x * 64;
+  const int h = blockIdx.y;
+  if (threadIdx.x < 64) {
+    const int col = col0 + threadIdx.x;
+    int row = -1;
+    // largest b with transposed_offset(cu[b], b) <= col
+    int lo = 0, hi = batch;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (transposed_offset(cu[mid], mid) <= col) lo = mid; else hi = mid;
+    }
+    const int rel = col - transposed_offset(cu[lo], lo);
+    if (rel >= 0 && rel < cu[lo + 1] - cu[lo]) row = cu[lo] + rel;
+    src_row[threadIdx.x] = row;
+  }
+  __syncthreads();
+  const int pieces = dim / 8;
+  for (int p = threadIdx.x; p < 64 * pieces; p += 256) {
+    const int c = p / pieces, pc = p % pieces;
+    const int row = src_row[c];
+    vec8_t<T> v = zero8<T>();
+    if (row >= 0) v = load8(x + (long)row * row_stride + (long)h * head_stride + pc * 8);
+    store8(tile + c * ld + pc * 8, v);
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < dim * 8; p += 256) {
+    const int d = p >> 3, pc = p & 7;
+    vec8_t<T> v;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = tile[(pc * 8 + j) * ld + d];
+    store8(out + ((long)h * dim + d) * out_cols + col0 + pc * 8, v);
+  }
+}
+
+template <typename T>
+static int launch_compress_t(const CompressArgs& a, hipStream_t st) {
+  if (a.out_rows_bound <= 0) return 0;
+  if (a.wt == nullptr) {
+    const long threads = (long)a.out_rows_bound * (a.heads * a.dim / 8);
+    const int grid = (int)((threads + 255) / 256);
+    hipLaunchKernelGGL(compress_mean_kernel<T>, dim3(grid), dim3(256), 0, st, (const T*)a.x, (T*)a.out,
+                       a.cu_seq, a.cu_out, a.batch, a.heads, a.dim, a.block, a.stride);
+    return 0;
+  }
+  const int waves = ((a.out_rows_bound + 15) / 16) * a.heads;
+  const int grid = (waves + 3) / 4;
+#define NSA_WEIGHTED(D)                                                                              \
+  hipLaunchKernelGGL((compress_weighted_kernel<T, D>), dim3(grid), dim3(256), 0, st, (const T*)a.x, \
+                     (const T*)a.wt, (const T*)a.bias, (T*)a.out, a.cu_seq, a.cu_out, a.batch,      \
+                     a.heads, a.block, a.stride)
+  switch (a.dim) {
+    case 32: NSA_WEIGHTED(32); break;
+    case 64: NSA_WEIGHTED(64); break;
+    case 128: NSA_WEIGHTED(128); break;
+    case 192: NSA_WEIGHTED(192); break;
+    default: return -2;
+  }
+#undef NSA_WEIGHTED
+  return 0;
+}
+
+int launch_compress(const CompressArgs& a, hipStream_t st) {
+  return a.dtype == 0 ? launch_compress_t<bf16_t>(a, st) : launch_compress_t<float>(a, st);
+}
+
+template <typename T>
+static int launch_transpose_t(const TransposeArgs& a, hipStream_t st) {
+  const size_t smem = 64 * sizeof(int) + (size_t)64 * (a.dim + 8) * sizeof(T);
+  hipLaunchKernelGGL(transpose_kernel<T>, dim3(a.out_cols / 64, a.heads), dim3(256), smem, st,
+                     (const T*)a.x, (T*)a.out, a.cu, a.batch, a.dim, a.row_stride, a.head_stride,
+                     a.out_cols);
+  return 0;
+}
+
+int launch_transpose(const TransposeArgs& a, hipStream_t st) {
+  return a.dtype == 0 ? launch_transpose_t<bf16_t>(a, st) : launch_transpose_t<float>(a, st);
+}
+
+}  // namespace nsa

@@ -1,0 +1,108 @@
+"""NSAAttention with the constructor and forward signature of the reference's nsa/nsa.py:15-135."""
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+from torch import nn
+
+from . import _lib, ops
+from .compression_kv import KVCompressor, conv_compressed_len
+
+
+class NSAAttention(nn.Module):
+    """Native Sparse Attention forward: compress -> compressed attention + block selection ->
+    selected + sliding-window attention -> gated sum, all on hand-written gfx950 kernels.
+
+    Parameters follow the reference (`compressor.compressor_k/v.{weight,bias}`,
+    `gating.{weight,bias}`), so its state_dict loads.  Two build-owned switches:
+      compressor_mode  "conv" (reference: learned Conv1d) | "mean" (average each window)
+      gate_activation  None (reference: raw Linear output) | "sigmoid"
+    Unlike the reference, ragged `cu_seqlens` are honoured (each sequence is attended on its own)."""
+
+    def __init__(
+        self,
+        head_dim: int,
+        causal=False,
+        softmax_scale=None,
+        attention_dropout=0.0,
+        deterministic=False,
+        compression_stride=16,
+        compression_block=32,
+        selection_block=64,
+        selected_block_count=16,
+        sliding_window=512,
+        device=None,
+        dtype=None,
+        compressor_mode: str = "conv",
+        gate_activation: Optional[str] = None,
+    ):
+        super().__init__()
+        if attention_dropout not in (0, 0.0, None):
+            raise NotImplementedError("attention dropout is not part of the forward kernels")
+        if compressor_mode not in ("conv", "mean") or gate_activation not in (None, "sigmoid"):
+            raise ValueError("compressor_mode in {'conv','mean'}, gate_activation in {None,'sigmoid'}")
+        self.causal = causal
+        self.softmax_scale = softmax_scale
+        self.drop_p = attention_dropout
+        self.deterministic = deterministic
+        self.sliding_window = sliding_window
+        self.selected_block_count = selected_block_count
+        self.selection_block_size = selection_block
+        self.compression_stride = compression_stride
+        self.compression_block = compression_block
+        self.compressor = KVCompressor(compression_stride, compression_block, head_dim, device, dtype,
+                                       mode=compressor_mode)
+        self.pool_kernel_size = selection_block // compression_stride + 1
+        self.pool_padding = compression_block // compression_stride - 2
+        self.pool_stride = selection_block // compression_stride
+        self.gating = nn.Linear(head_dim, 3, device=device, dtype=dtype)
+        self.gate_activation = gate_activation
+
+    @torch.no_grad()
+    def forward(
+        self,
+        q: torch.Tensor,
+        k: torch.Tensor,
+        v: torch.Tensor,
+        cu_seqlens: torch.Tensor,
+        max_seqlen=None,
+        cu_seqlens_k: torch.Tensor = None,
+        max_seqlen_k=None,
+        causal: bool = None,
+        gates: Optional[torch.Tensor] = None,
+    ) -> torch.Tensor:
+        """q [total,Hq,Dk], k [total,Hkv,Dk], v [total,Hkv,Dv], cu_seqlens int32 [B+1] -> [total,Hq,Dv].
+
+        max_seqlen: longest sequence (int); 0/None means "all sequences have total/B tokens" as in
+        the reference.  gates [total,Hq,3] (selected, sliding, compressed) overrides the gating
+        Linear (pre-activation values)."""
+        causal = self.causal if causal is None else causal
+        cu = (cu_seqlens if cu_seqlens_k is None else cu_seqlens_k).to(torch.int32)
+        batch = cu.numel() - 1
+        total, hq, dk = q.shape
+        hkv, dv = v.shape[1], v.shape[2]
+        scale = self.softmax_scale
+        if scale is None or scale is True:
+            scale = 1.0 / math.sqrt(dk)
+        uniform = not max_seqlen
+        seq_len = total // batch if uniform else int(max_seqlen)
+
+        ck, cv, cu_cmp, nc = self.compressor.compress_packed(k, v, cu, seq_len=seq_len if uniform else None)
+        max_nc = nc if nc is not None else conv_compressed_len(seq_len, self.compression_stride,
+                                                               self.compression_block)
+        cvt = ops.transpose(cv, cu_cmp, batch)
+        vt = ops.transpose(v, cu, batch)
+        o_cmp, idx, _ = ops.cmp_attn_select(
+            q, ck, cvt, cu, cu_cmp, batch, hkv, dv, ck.stride(0), ck.stride(1), self.compression_block,
+            self.compression_stride, self.pool_kernel_size, self.pool_stride, self.pool_padding,
+            self.selected_block_count, max_nc, scale, causal=bool(causal), select=True, idx64=False)
+        if gates is None:
+            gates = self.gating(q)                       # [total, Hq, 3]
+        g = gates.reshape(total * hq, 3)
+        g_slc, g_swa, g_cmp = (g[:, i].view(total, hq) for i in range(3))
+        o_swa = ops.swa(q, k, vt, cu, batch, self.sliding_window, scale) if self.sliding_window > 0 else None
+        act = _lib.GATE_SIGMOID if self.gate_activation == "sigmoid" else _lib.GATE_IDENTITY
+        return ops.slc_combine(q, k, vt, idx, None, g_slc, g_swa if o_swa is not None else None, g_cmp,
+                               o_swa, o_cmp, cu, batch, self.selection_block_size, scale, gate_act=act)

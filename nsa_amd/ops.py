@@ -1,0 +1,188 @@
+"""Thin tensor-level wrappers over the C ABI: they check layouts, allocate outputs with torch and
+enqueue the kernels on the current stream.  No arithmetic happens in Python."""
+from __future__ import annotations
+
+import ctypes as C
+import math
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.bfloat16:
+        return _lib.NSA_BF16
+    if t.dtype == torch.float32:
+        return _lib.NSA_F32
+    raise TypeError("NSA kernels take bfloat16 or float32 tensors, got %s" % t.dtype)
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _need_cuda(*ts):
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("NSA kernels run on the GPU only; got a %s tensor" % t.device)
+
+
+def _dense(t: torch.Tensor) -> torch.Tensor:
+    """Contiguous and 16-byte aligned."""
+    if not t.is_contiguous() or t.data_ptr() % 16:
+        t = t.contiguous()
+        if t.data_ptr() % 16:
+            t = t.clone()
+    return t
+
+
+def pool_bins(nc: int, kernel: int, stride: int, pad: int) -> int:
+    """Bins of a ceil-mode average pool (kernel, stride, pad) over nc columns."""
+    if nc <= 0 or nc + 2 * pad < kernel:
+        return 0
+    ns = -(-(nc + 2 * pad - kernel) // stride) + 1
+    if (ns - 1) * stride >= nc + pad:
+        ns -= 1
+    return ns
+
+
+def transposed_cols(total_rows: int, batch: int) -> int:
+    return _lib.load().nsa_transposed_cols(total_rows, batch)
+
+
+def uniform_cu(batch: int, length: int, device) -> torch.Tensor:
+    return torch.arange(0, (batch + 1) * length, length, dtype=torch.int32, device=device)
+
+
+def compressed_offsets(cu_seqlens: torch.Tensor, block: int, stride: int, extra: int = 1) -> torch.Tensor:
+    """Row offsets of every sequence in the packed compressed tensor, computed on the device.
+    extra = 1: Conv1d count (len-block)//stride + 1;  extra = 0: the functional count."""
+    lens = (cu_seqlens[1:] - cu_seqlens[:-1]).to(torch.int64)
+    nc = torch.where(lens >= block, (lens - block) // stride + extra, torch.zeros_like(lens)).clamp_(min=0)
+    out = torch.zeros(cu_seqlens.numel(), dtype=torch.int32, device=cu_seqlens.device)
+    out[1:] = torch.cumsum(nc, 0).to(torch.int32)
+    return out
+
+
+def transpose(x: torch.Tensor, cu: torch.Tensor, batch: int, heads: Optional[int] = None,
+              head_stride: Optional[int] = None) -> torch.Tensor:
+    """x [rows, H, dim] (last dim contiguous) -> key-contiguous [heads, dim, cols].
+    heads/head_stride let a caller read every (H/heads)-th head of a head-repeated tensor."""
+    _need_cuda(x, cu)
+    rows, H, dim = x.shape
+    if x.stride(2) != 1 or x.data_ptr() % 16:
+        x = _dense(x)
+    heads = H if heads is None else heads
+    head_stride = x.stride(1) if head_stride is None else head_stride
+    cols = transposed_cols(rows, batch)
+    out = torch.empty(heads, dim, cols, dtype=x.dtype, device=x.device)
+    lib = _lib.load()
+    rc = lib.nsa_transpose_fwd(_ptr(x), _ptr(out), _ptr(cu), batch, heads, dim, x.stride(0), head_stride,
+                               cols, _dtype_code(x), _stream())
+    _lib.check(rc, "nsa_transpose_fwd")
+    return out
+
+
+def compress(x: torch.Tensor, cu_seqlens: torch.Tensor, cu_out: torch.Tensor, out_rows: int, block: int,
+             stride: int, wt: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x [total, H, D] -> [out_rows, H, D]; wt None = mean over each window, else [D, block*D]."""
+    _need_cuda(x, cu_seqlens, cu_out)
+    x = _dense(x)
+    total, H, D = x.shape
+    out = torch.empty(out_rows, H, D, dtype=x.dtype, device=x.device)
+    if wt is not None:
+        wt = _dense(wt.to(x.dtype))
+        if tuple(wt.shape) != (D, block * D):
+            raise ValueError("weight must be [dim, block*dim], got %s" % (tuple(wt.shape),))
+    if bias is not None:
+        bias = _dense(bias.to(x.dtype))
+    if out_rows == 0:
+        return out
+    lib = _lib.load()
+    rc = lib.nsa_compress_fwd(_ptr(x), _ptr(wt), _ptr(bias), _ptr(out), _ptr(cu_seqlens), _ptr(cu_out),
+                              cu_seqlens.numel() - 1, out_rows, H, D, block, stride, _dtype_code(x), _stream())
+    _lib.check(rc, "nsa_compress_fwd")
+    return out
+
+
+def cmp_attn_select(q, ck, cvt, cu_seqlens, cu_cmp, batch, hkv, dv, ck_row_stride, ck_head_stride, block,
+                    stride, pool_kernel, pool_stride, pool_pad, top_n, max_nc, scale, causal=True,
+                    select=True, idx64=True, want_pooled=False):
+    """q [total,Hq,Dk] packed; ck any tensor whose rows are reachable with the two strides;
+    cvt [hkv, dv, cols].  Returns (o [total,Hq,dv], indices [total,hkv,top_n] or None, pooled or None)."""
+    _need_cuda(q, ck, cvt, cu_seqlens, cu_cmp)
+    q = _dense(q)
+    total, hq, dk = q.shape
+    o = torch.empty(total, hq, dv, dtype=q.dtype, device=q.device)
+    max_ns = pool_bins(max_nc, pool_kernel, pool_stride, pool_pad) if select else 0
+    idx = pooled = None
+    if select:
+        idx = torch.empty(total, hkv, top_n, dtype=torch.int64 if idx64 else torch.int32, device=q.device)
+        if want_pooled:
+            pooled = torch.zeros(total, hkv, max(max_ns, 1), dtype=torch.float32, device=q.device)
+    lib = _lib.load()
+    rc = lib.nsa_cmp_attn_select_fwd(
+        _ptr(q), _ptr(ck), _ptr(cvt), _ptr(o), _ptr(idx), _ptr(pooled), _ptr(cu_seqlens), _ptr(cu_cmp), batch,
+        total, hq, hkv, dk, dv, ck_row_stride, ck_head_stride, cvt.shape[-1], block, stride, pool_kernel,
+        pool_stride, pool_pad, max(top_n, 1), max_ns, max(max_ns, 1), float(scale), int(bool(causal)),
+        int(idx64), _dtype_code(q), _stream())
+    _lib.check(rc, "nsa_cmp_attn_select_fwd")
+    return o, idx, pooled
+
+
+def swa(q, k, vt, cu_seqlens, batch, window, scale):
+    _need_cuda(q, k, vt, cu_seqlens)
+    q, k = _dense(q), _dense(k)
+    total, hq, dk = q.shape
+    hkv, dv = vt.shape[0], vt.shape[1]
+    o = torch.empty(total, hq, dv, dtype=q.dtype, device=q.device)
+    lib = _lib.load()
+    rc = lib.nsa_swa_fwd(_ptr(q), _ptr(k), _ptr(vt), _ptr(o), _ptr(cu_seqlens), batch, total, hq, hkv, dk, dv,
+                         vt.shape[-1], window, float(scale), _dtype_code(q), _stream())
+    _lib.check(rc, "nsa_swa_fwd")
+    return o
+
+
+def _gate_views(gates, q):
+    """gates: list of [total, Hq] tensors or None.  Returns (tensors, common element stride)."""
+    live = [g for g in gates if g is not None]
+    if not live:
+        return gates, 1
+    hq = q.shape[1]
+    s = live[0].stride(-1) if live[0].dim() == 2 else 0
+    ok = all(g.dim() == 2 and g.dtype == q.dtype and g.stride(1) == s and g.stride(0) == hq * s and s > 0
+             and g.data_ptr() % g.element_size() == 0 for g in live)
+    if ok:
+        return gates, s
+    return [None if g is None else g.to(q.dtype).contiguous() for g in gates], 1
+
+
+def slc_combine(q, k, vt, indices, counts, g_slc, g_swa, g_cmp, o_swa, o_cmp, cu_seqlens, batch, block_size,
+                scale, gate_act=0):
+    _need_cuda(q, k, vt, indices, cu_seqlens)
+    q, k = _dense(q), _dense(k)
+    total, hq, dk = q.shape
+    hkv, dv = vt.shape[0], vt.shape[1]
+    if indices.dtype not in (torch.int32, torch.int64):
+        raise TypeError("block indices must be int32 or int64")
+    indices = indices.contiguous()
+    top_n = indices.shape[-1]
+    if counts is not None:
+        counts = counts.to(torch.int32).contiguous()
+    (g_slc, g_swa, g_cmp), gs = _gate_views([g_slc, g_swa, g_cmp], q)
+    o_swa = None if o_swa is None else _dense(o_swa)
+    o_cmp = None if o_cmp is None else _dense(o_cmp)
+    out = torch.empty(total, hq, dv, dtype=q.dtype, device=q.device)
+    lib = _lib.load()
+    rc = lib.nsa_slc_combine_fwd(
+        _ptr(q), _ptr(k), _ptr(vt), _ptr(indices), _ptr(counts), _ptr(g_slc), _ptr(g_swa), _ptr(g_cmp), gs,
+        _ptr(o_swa), _ptr(o_cmp), _ptr(out), _ptr(cu_seqlens), batch, total, hq, hkv, dk, dv, vt.shape[-1],
+        top_n, block_size, float(scale), int(indices.dtype == torch.int64), gate_act, _dtype_code(q), _stream())
+    _lib.check(rc, "nsa_slc_combine_fwd")
+    return out

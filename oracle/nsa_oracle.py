@@ -356,10 +356,11 @@ class NSAParams:
 
 
 def nsa_forward_single(q, k, v, gates, p: NSAParams, compressor=None,
-                       math_dtype=torch.float32, return_parts=False):
+                       math_dtype=torch.float32, return_parts=False, force_idx=None):
     """One sequence.  q [T,Hq,Dk], k [T,Hkv,Dk], v [T,Hkv,Dv], gates [T,Hq,3] already activated,
     ordered (selected, sliding, compressed).  compressor: None -> mean-pool, else a dict with
     'wk','wv' ([block*D, D] row j*D+i) and optional 'bk','bv'.  Returns [T,Hq,Dv] in q.dtype.
+    force_idx replaces the selected block ids (the returned 'idx_own' keeps the oracle's own).
     """
     T = q.shape[0]
     Nc = compressed_len_conv(T, p.block, p.stride)
@@ -379,12 +380,16 @@ def nsa_forward_single(q, k, v, gates, p: NSAParams, compressor=None,
         pooled = torch.zeros(T, Hkv, 0, dtype=math_dtype)
         idx = torch.full((T, Hkv, p.top_n), -1, dtype=torch.int64)
         o_cmp = torch.zeros(T, q.shape[1], v.shape[2], dtype=math_dtype)
+    if force_idx is not None:          # branch parity independent of how score ties were broken
+        idx = force_idx.to(torch.int64)
     o_slc = selected_attention(q, k, v, idx, None, p.sel_block, p.scale, math_dtype)
     o_swa = sliding_attention(q, k, v, p.window, p.scale, math_dtype) if p.window > 0 else None
     gm = gates.to(math_dtype)
     out = gated_combine(gm[..., 0], o_slc, gm[..., 1], o_swa, gm[..., 2], o_cmp).to(q.dtype)
     if return_parts:
-        return out, dict(ck=ck, cv=cv, pooled=pooled, idx=idx, o_cmp=o_cmp, o_slc=o_slc, o_swa=o_swa)
+        own = select_blocks(pooled, p.top_n) if pooled.shape[-1] > 0 else idx
+        return out, dict(ck=ck, cv=cv, pooled=pooled, idx=idx, idx_own=own, o_cmp=o_cmp, o_slc=o_slc,
+                         o_swa=o_swa)
     return out
 
 

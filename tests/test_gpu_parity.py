@@ -1,0 +1,384 @@
+"""GPU parity: every kernel is called through the C ABI (via the thin ctypes wrappers) and compared
+with the CPU oracle on the same seeded inputs.  Bars: bf16 max-abs <= 2e-2, fp32 <= 1e-4, selected
+block sets identical except where the oracle's scores tie within 1e-3."""
+import math
+
+import pytest
+import torch
+
+from oracle import nsa_oracle as O
+from tests.util import TOL, make_qkv, max_abs, ragged_cu, randn
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _ops():
+    from nsa_amd import ops
+    return ops
+
+
+def _cu(lens):
+    return torch.tensor(ragged_cu(lens), dtype=torch.int32, device=DEV)
+
+
+# ------------------------------------------------------------------------------ compression
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("lens,H,D,l,d", [([1024], 1, 64, 32, 16), ([300, 31, 64, 1000], 4, 128, 32, 16),
+                                          ([200, 77], 2, 192, 64, 16)])
+def test_compress_mean(dtype, lens, H, D, l, d):
+    ops = _ops()
+    x = randn(sum(lens), H, D, seed=1, dtype=dtype)
+    cu = _cu(lens)
+    cu_out = ops.compressed_offsets(cu, l, d, extra=1)
+    ncs = [O.compressed_len_conv(t, l, d) for t in lens]
+    assert cu_out.cpu().tolist() == ragged_cu(ncs)
+    out = ops.compress(x.to(DEV), cu, cu_out, sum(ncs), l, d)
+    ref = torch.cat([O.compress_meanpool(x[s:e], l, d, n) for s, e, n in
+                     zip(ragged_cu(lens)[:-1], ragged_cu(lens)[1:], ncs)])
+    err = max_abs(out, ref)
+    print("compress_mean", dtype, lens, "max_abs", err)
+    assert err <= (1e-6 if dtype == torch.float32 else 4e-3)
+    # closed form on the first sequence
+    if ncs[0] > 0:
+        cf = x[:lens[0]].float().unfold(0, l, d).mean(-1).to(dtype)
+        assert max_abs(out[:ncs[0]], cf) <= (1e-6 if dtype == torch.float32 else 4e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("lens,H,D,l,d,extra", [([256, 100], 2, 64, 32, 16, 1), ([1024] * 2, 2, 128, 64, 16, 0),
+                                                ([90], 1, 32, 8, 4, 1)])
+def test_compress_weighted(dtype, lens, H, D, l, d, extra):
+    ops = _ops()
+    x = randn(sum(lens), H, D, seed=2, dtype=dtype)
+    w_lin = randn(l * D, D, seed=3, scale=1.0 / math.sqrt(l * D), dtype=dtype)
+    bias = randn(D, seed=4, dtype=dtype) if extra else None
+    cu = _cu(lens)
+    cu_out = ops.compressed_offsets(cu, l, d, extra=extra)
+    ncs = [O.compressed_len_conv(t, l, d) if extra else O.compressed_len_functional(t, l, d) for t in lens]
+    assert cu_out.cpu().tolist() == ragged_cu(ncs)
+    out = ops.compress(x.to(DEV), cu, cu_out, sum(ncs), l, d, w_lin.t().contiguous().to(DEV),
+                       None if bias is None else bias.to(DEV))
+    ref = torch.cat([O.compress_weighted(x[s:e], w_lin, bias, l, d, n) for s, e, n in
+                     zip(ragged_cu(lens)[:-1], ragged_cu(lens)[1:], ncs)])
+    err = max_abs(out, ref)
+    print("compress_weighted", dtype, lens, "max_abs", err)
+    assert err <= TOL[dtype]
+
+
+def test_transpose_layout():
+    ops = _ops()
+    lens = [70, 5, 129]
+    x = randn(sum(lens), 3, 64, seed=5, dtype=torch.bfloat16)
+    cu = _cu(lens)
+    out = ops.transpose(x.to(DEV), cu, len(lens)).cpu()
+    from nsa_amd import _lib
+    lib = _lib.load()
+    cuh = ragged_cu(lens)
+    seen = torch.zeros(out.shape[-1], dtype=torch.bool)
+    for b, (s, e) in enumerate(zip(cuh[:-1], cuh[1:])):
+        off = lib.nsa_transposed_offset(s, b)
+        assert off % 8 == 0
+        assert torch.equal(out[:, :, off:off + e - s], x[s:e].permute(1, 2, 0))
+        seen[off:off + e - s] = True
+    assert torch.count_nonzero(out[:, :, ~seen]) == 0
+
+
+# ------------------------------------------------------------------------------ compressed attention + selection
+def _cmp_case(dtype, lens, Hq, Hkv, Dk, Dv, l, d, lsel, S, seed, scale_in=1.0):
+    ops = _ops()
+    p = O.NSAParams(l, d, lsel, S, 0)
+    T = sum(lens)
+    q, k, v, _ = make_qkv(T, Hq, Hkv, Dk, Dv, seed, dtype, scale_in)
+    cu = _cu(lens)
+    cu_cmp = ops.compressed_offsets(cu, l, d, extra=1)
+    ncs = [O.compressed_len_conv(t, l, d) for t in lens]
+    ck = ops.compress(k.to(DEV), cu, cu_cmp, sum(ncs), l, d)
+    cv = ops.compress(v.to(DEV), cu, cu_cmp, sum(ncs), l, d)
+    cvt = ops.transpose(cv, cu_cmp, len(lens))
+    scale = 1.0 / math.sqrt(Dk)
+    o, idx, pooled = ops.cmp_attn_select(q.to(DEV), ck, cvt, cu, cu_cmp, len(lens), Hkv, Dv, ck.stride(0),
+                                         ck.stride(1), l, d, p.pool_kernel, p.pool_stride, p.pool_pad, S,
+                                         max(ncs), scale, want_pooled=True)
+    torch.cuda.synchronize()
+    o, idx, pooled = o.cpu(), idx.cpu(), pooled.cpu()
+    cuh, cuc = ragged_cu(lens), ragged_cu(ncs)
+    worst = dict(o=0.0, pooled=0.0, rows=0, exact=0, excused=0, fail=0)
+    for b in range(len(lens)):
+        s, e = cuh[b], cuh[b + 1]
+        ckb, cvb = ck[cuc[b]:cuc[b + 1]].cpu(), cv[cuc[b]:cuc[b + 1]].cpu()
+        if ncs[b] == 0:
+            assert torch.count_nonzero(o[s:e]) == 0
+            assert (idx[s:e] == -1).all()
+            continue
+        ref_o = O.compressed_attention(q[s:e], ckb, cvb, l, d, scale)
+        worst["o"] = max(worst["o"], max_abs(o[s:e], ref_o))
+        assert torch.count_nonzero(o[s:s + min(l, e - s)]) == 0          # rows that see nothing
+        ref_p = O.importance_scores(q[s:e], ckb, p.pool_kernel, p.pool_stride, p.pool_pad)
+        Ns = ref_p.shape[-1]
+        if Ns == 0:
+            assert (idx[s:e] == -1).all()
+            continue
+        worst["pooled"] = max(worst["pooled"], max_abs(pooled[s:e, :, :Ns], ref_p))
+        ref_idx = O.select_blocks(ref_p, S)
+        n, ex, exc, fail = O.compare_selection(idx[s:e], ref_idx, ref_p, 1e-3)
+        worst["rows"] += n; worst["exact"] += ex; worst["excused"] += exc; worst["fail"] += fail
+        # descending order of the kernel's own scores
+        got = torch.gather(pooled[s:e, :, :Ns], 2, idx[s:e].clamp(min=0))
+        got = torch.where(idx[s:e] >= 0, got, torch.full_like(got, -1.0))
+        assert (got[..., :-1] >= got[..., 1:]).all()
+    print("cmp", dtype, lens, (Hq, Hkv, Dk, Dv), worst)
+    assert worst["o"] <= TOL[dtype]
+    assert worst["pooled"] <= 1e-3
+    assert worst["fail"] == 0
+    return worst
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_cmp_select_cfg1_shape(dtype):
+    _cmp_case(dtype, [1024], 4, 1, 64, 64, 32, 16, 64, 4, seed=0)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_cmp_select_g16(dtype):
+    _cmp_case(dtype, [2048], 32, 2, 128, 128, 32, 16, 64, 16, seed=10, scale_in=0.5)
+
+
+def test_cmp_select_dqk192_ragged():
+    _cmp_case(torch.bfloat16, [700, 31, 1055, 64, 1000], 32, 2, 192, 128, 32, 16, 64, 4, seed=20, scale_in=0.5)
+
+
+def test_cmp_select_block64_padded_pool():
+    # l=64,d=16 -> pool kernel 5 stride 4 pad 2 (padding counted in the divisor)
+    _cmp_case(torch.bfloat16, [1024, 333], 16, 1, 64, 64, 64, 16, 64, 4, seed=30)
+
+
+def test_cmp_select_odd_groups():
+    _cmp_case(torch.float32, [500], 6, 2, 64, 64, 32, 16, 64, 2, seed=40)      # G=3 -> padded to 4
+    _cmp_case(torch.float32, [500], 8, 1, 32, 32, 32, 16, 64, 2, seed=41)      # G=8
+    _cmp_case(torch.float32, [300], 2, 2, 32, 32, 32, 16, 64, 2, seed=42)      # G=1
+
+
+# ------------------------------------------------------------------------------ sliding window
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("lens,Hq,Hkv,Dk,Dv,W", [([1024], 4, 1, 64, 64, 128), ([777, 40, 513], 32, 2, 128, 128, 512),
+                                                 ([600], 16, 1, 192, 128, 100), ([130], 8, 2, 32, 32, 1),
+                                                 ([300], 6, 2, 64, 64, 1000)])
+def test_swa(dtype, lens, Hq, Hkv, Dk, Dv, W):
+    ops = _ops()
+    T = sum(lens)
+    q, k, v, _ = make_qkv(T, Hq, Hkv, Dk, Dv, 50, dtype, 0.7)
+    cu = _cu(lens)
+    vt = ops.transpose(v.to(DEV), cu, len(lens))
+    scale = 1.0 / math.sqrt(Dk)
+    o = ops.swa(q.to(DEV), k.to(DEV), vt, cu, len(lens), W, scale).cpu()
+    cuh = ragged_cu(lens)
+    err = 0.0
+    for s, e in zip(cuh[:-1], cuh[1:]):
+        err = max(err, max_abs(o[s:e], O.sliding_attention(q[s:e], k[s:e], v[s:e], W, scale)))
+    print("swa", dtype, lens, (Hq, Hkv, Dk, Dv, W), "max_abs", err)
+    assert err <= TOL[dtype]
+
+
+# ------------------------------------------------------------------------------ selected blocks + combine
+def _random_indices(T, Hkv, S, bs, seed, poison=True):
+    g = torch.Generator().manual_seed(seed)
+    nblk = (T + bs - 1) // bs
+    idx = torch.full((T, Hkv, S), nblk + 3, dtype=torch.int64)       # out-of-range padding
+    for t in range(T):
+        for h in range(Hkv):
+            perm = torch.randperm(nblk, generator=g)[:S]             # past and future blocks, no duplicates
+            idx[t, h, :len(perm)] = perm
+    if poison:
+        idx[0] = nblk + 1
+        idx[T // 2, :, 0] = -5
+    return idx
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("lens,Hq,Hkv,Dk,Dv,S,bs", [([256], 16, 1, 32, 32, 2, 32), ([512, 100], 32, 2, 128, 128, 8, 64),
+                                                   ([384], 4, 1, 64, 64, 4, 64), ([200], 16, 1, 192, 128, 3, 64),
+                                                   ([160], 6, 2, 64, 64, 3, 16)])
+def test_slc_only(dtype, lens, Hq, Hkv, Dk, Dv, S, bs):
+    ops = _ops()
+    T = sum(lens)
+    q, k, v, gl = make_qkv(T, Hq, Hkv, Dk, Dv, 60, dtype, 0.7)
+    cu = _cu(lens)
+    cuh = ragged_cu(lens)
+    idx = torch.cat([_random_indices(e - s, Hkv, S, bs, 61 + s) for s, e in zip(cuh[:-1], cuh[1:])])
+    g = torch.Generator().manual_seed(62)
+    counts = torch.randint(0, S + 1, (T, Hkv), generator=g)
+    vt = ops.transpose(v.to(DEV), cu, len(lens))
+    scale = 1.0 / math.sqrt(Dk)
+    for use_counts, dt_idx in ((False, torch.int64), (True, torch.int32)):
+        o = ops.slc_combine(q.to(DEV), k.to(DEV), vt, idx.to(dt_idx).to(DEV),
+                            counts.to(DEV) if use_counts else None, None, None, None, None, None, cu,
+                            len(lens), bs, scale).cpu()
+        err = 0.0
+        for s, e in zip(cuh[:-1], cuh[1:]):
+            ref = O.selected_attention(q[s:e], k[s:e], v[s:e], idx[s:e], counts[s:e] if use_counts else None,
+                                       bs, scale)
+            err = max(err, max_abs(o[s:e], ref))
+            assert torch.count_nonzero(o[s]) == 0                     # poisoned row: empty selection -> 0
+        print("slc", dtype, lens, (Hq, Hkv, Dk, Dv, S, bs), "counts", use_counts, "max_abs", err)
+        assert err <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_parallel_nsa_api_like_reference_test(dtype):
+    """Shape of the reference's own test (B=2,T=64,H=1,HQ=16,D=32,S=2,bs=32,W=128, ones gates,
+    random counts, two rows forced to an empty selection), fp16 replaced by bf16/fp32."""
+    import nsa_amd
+    B, T, H, HQ, D, S, bs, W = 2, 64, 1, 16, 32, 2, 32, 128
+    q = randn(B, T, HQ, D, seed=70, dtype=dtype)
+    k = randn(B, T, H, D, seed=71, dtype=dtype)
+    v = randn(B, T, H, D, seed=72, dtype=dtype)
+    g_slc = torch.ones(B, T, HQ, dtype=dtype)
+    g_swa = torch.ones(B, T, HQ, dtype=dtype)
+    gen = torch.Generator().manual_seed(73)
+    idx = torch.full((B, T, H, S), T, dtype=torch.long)
+    for b in range(B):
+        for t in range(T):
+            perm = torch.randperm(max(1, t // bs), generator=gen)[:S]
+            idx[b, t, 0, :len(perm)] = perm
+    idx = idx.sort(-1)[0]
+    idx[0, 0, 0, 0] = 4
+    idx[1, 63, 0, 0] = 7
+    idx[1, 63, 0, 1] = 9
+    counts = torch.randint(1, S + 1, (B, T, H), generator=gen)
+    out = nsa_amd.selection_attention(q.to(DEV), k.to(DEV), v.to(DEV), g_slc.to(DEV), g_swa.to(DEV), idx.to(DEV),
+                                      counts.to(DEV), bs, W).cpu()
+    for b in range(B):
+        slc, swa = O.selected_sliding_loop(q[b], k[b], v[b], idx[b], counts[b], bs, W)
+        ref = slc + swa
+        err = max_abs(out[b], ref)
+        print("parallel_nsa", dtype, "batch", b, "max_abs", err)
+        assert err <= TOL[dtype]
+    # head_first and int block_counts
+    out_hf = nsa_amd.parallel_nsa(q.transpose(1, 2).to(DEV), k.transpose(1, 2).to(DEV), v.transpose(1, 2).to(DEV),
+                                  g_slc.transpose(1, 2).to(DEV), g_swa.transpose(1, 2).to(DEV),
+                                  idx.transpose(1, 2).to(DEV), 1, bs, W, head_first=True).cpu()
+    slc, swa = O.selected_sliding_loop(q[0], k[0], v[0], idx[0], 1, bs, W)
+    assert max_abs(out_hf[0].transpose(0, 1), slc + swa) <= TOL[dtype]
+
+
+# ------------------------------------------------------------------------------ whole forward
+def _module_case(dtype, lens, Hq, Hkv, Dk, Dv, S, W, seed, scale_in, mode="mean", act="sigmoid", l=32, d=16, lsel=64):
+    from nsa_amd.nsa import NSAAttention
+    T = sum(lens)
+    q, k, v, gl = make_qkv(T, Hq, Hkv, Dk, Dv, seed, dtype, scale_in)
+    torch.manual_seed(seed)
+    m = NSAAttention(Dk, causal=True, compression_stride=d, compression_block=l, selection_block=lsel,
+                     selected_block_count=S, sliding_window=W, dtype=dtype, compressor_mode=mode,
+                     gate_activation=act)
+    comp = None
+    if mode == "conv":
+        assert Dk == Dv
+        comp = dict(wk=m.compressor.compressor_k.weight.detach().permute(2, 1, 0).reshape(l * Dk, Dk).clone(),
+                    wv=m.compressor.compressor_v.weight.detach().permute(2, 1, 0).reshape(l * Dk, Dk).clone(),
+                    bk=m.compressor.compressor_k.bias.detach().clone(),
+                    bv=m.compressor.compressor_v.bias.detach().clone())
+    m = m.to(DEV)
+    uniform = len(set(lens)) == 1
+    cu = _cu(lens)
+    out = m(q.to(DEV), k.to(DEV), v.to(DEV), cu, 0 if uniform else max(lens), gates=gl.to(DEV)).cpu()
+    # second pass only to read the kernel's own picks (for the forced-index comparison)
+    from nsa_amd import ops
+    gates = torch.sigmoid(gl.float()).to(dtype) if act == "sigmoid" else gl
+    p = O.NSAParams(l, d, lsel, S, W)
+    cuh = ragged_cu(lens)
+    ck, cv, cu_cmp, nc = m.compressor.compress_packed(k.to(DEV), v.to(DEV), cu, seq_len=lens[0] if uniform else None)
+    cvt = ops.transpose(cv, cu_cmp, len(lens))
+    max_nc = max(O.compressed_len_conv(t, l, d) for t in lens)
+    _, idx, _ = ops.cmp_attn_select(q.to(DEV), ck, cvt, cu, cu_cmp, len(lens), Hkv, Dv, ck.stride(0), ck.stride(1),
+                                    l, d, p.pool_kernel, p.pool_stride, p.pool_pad, S, max_nc, 1 / math.sqrt(Dk))
+    idx = idx.cpu()
+    err = 0.0
+    stats = [0, 0, 0, 0]
+    for s, e in zip(cuh[:-1], cuh[1:]):
+        ref, parts = O.nsa_forward_single(q[s:e], k[s:e], v[s:e], gates[s:e], p, comp, return_parts=True,
+                                          force_idx=idx[s:e])
+        err = max(err, max_abs(out[s:e], ref))
+        if parts["pooled"].shape[-1] > 0:
+            r = O.compare_selection(idx[s:e], parts["idx_own"], parts["pooled"], 1e-3)
+            stats = [a + b for a, b in zip(stats, r)]
+    print("module", dtype, lens, (Hq, Hkv, Dk, Dv, S, W), mode, act, "max_abs", err, "rows/exact/excused/fail", stats)
+    assert torch.isfinite(out).all()
+    assert err <= TOL[dtype]
+    assert stats[3] == 0
+    return err
+
+
+def test_module_cfg1_fp32():
+    """BASELINE config 1: B1, T1024, Hq4, Hkv1, D64, fp32, mean-pool 32/16, blocks of 64, top-4, window 128."""
+    _module_case(torch.float32, [1024], 4, 1, 64, 64, 4, 128, seed=0, scale_in=1.0)
+
+
+def test_module_cfg2_shape_reduced_bf16():
+    """BASELINE config 2 at T=2048 (the full T=8192 case is test_module_cfg2_full)."""
+    _module_case(torch.bfloat16, [2048], 64, 4, 128, 128, 16, 512, seed=1, scale_in=0.5)
+
+
+def test_module_cfg4_shape_reduced_dqk192():
+    _module_case(torch.bfloat16, [2048], 64, 4, 192, 128, 16, 512, seed=3, scale_in=0.5)
+
+
+def test_module_varlen_ragged():
+    _module_case(torch.bfloat16, [1100, 64, 1000, 33, 1536], 32, 2, 128, 128, 16, 512, seed=2, scale_in=0.5)
+
+
+def test_module_reference_defaults_conv_raw_gates():
+    """Reference configuration: learned Conv1d compressor with bias, raw (un-activated) gates."""
+    _module_case(torch.bfloat16, [1024, 1024], 16, 1, 128, 128, 16, 512, seed=5, scale_in=1.0, mode="conv", act=None)
+    _module_case(torch.float32, [512], 16, 1, 64, 64, 4, 128, seed=6, scale_in=1.0, mode="conv", act=None)
+
+
+def test_flash_attn_func_api():
+    import nsa_amd
+    from nsa_amd.compression_kv import KVCompressor
+    B, T, Hq, Hkv, D, l, d, S = 2, 1024, 16, 1, 128, 32, 16, 16
+    dtype = torch.bfloat16
+    q = randn(B * T, Hq, D, seed=80, dtype=dtype)
+    k = randn(B * T, Hkv, D, seed=81, dtype=dtype)
+    v = randn(B * T, Hkv, D, seed=82, dtype=dtype)
+    torch.manual_seed(83)
+    comp = KVCompressor(d, l, D, None, dtype)
+    wk = comp.compressor_k.weight.detach().permute(2, 1, 0).reshape(l * D, D).clone()
+    wv = comp.compressor_v.weight.detach().permute(2, 1, 0).reshape(l * D, D).clone()
+    bk, bv = comp.compressor_k.bias.detach().clone(), comp.compressor_v.bias.detach().clone()
+    comp = comp.to(DEV)
+    cu = torch.arange(0, (B + 1) * T, T, dtype=torch.int32, device=DEV)
+    ck, cv, _ = comp(k.to(DEV), v.to(DEV), cu, Hq // Hkv)
+    Nc = O.compressed_len_conv(T, l, d)
+    assert ck.shape == (B, Nc, Hq, D)
+    o, idx = nsa_amd.flash_attn_func(q.view(B, T, Hq, D).to(DEV), ck, cv, d, l, True, None, Hkv, 5, 4, 0, S)
+    assert o.shape == (B, T, Hq, D) and idx.shape == (B, T, Hkv, S) and idx.dtype == torch.int64
+    o, idx = o.cpu(), idx.cpu()
+    for b in range(B):
+        sl = slice(b * T, (b + 1) * T)
+        ckr = O.compress_weighted(k[sl], wk, bk, l, d, Nc)
+        cvr = O.compress_weighted(v[sl], wv, bv, l, d, Nc)
+        assert max_abs(ck[b, :, ::Hq // Hkv], ckr) <= 2e-2
+        ref = O.compressed_attention(q[sl], ck[b, :, ::Hq // Hkv].cpu(), cv[b, :, ::Hq // Hkv].cpu(), l, d)
+        assert max_abs(o[b], ref) <= 2e-2
+        pooled = O.importance_scores(q[sl], ck[b, :, ::Hq // Hkv].cpu(), 5, 4, 0)
+        r = O.compare_selection(idx[b], O.select_blocks(pooled, S), pooled, 1e-3)
+        print("flash_attn_func batch", b, r)
+        assert r[3] == 0
+
+
+def test_error_paths():
+    import nsa_amd
+    from nsa_amd import ops
+    q = torch.zeros(64, 40, 64, dtype=torch.bfloat16, device=DEV)      # G = 40 > 16
+    k = torch.zeros(64, 1, 64, dtype=torch.bfloat16, device=DEV)
+    cu = _cu([64])
+    vt = ops.transpose(k, cu, 1)
+    with pytest.raises(NotImplementedError):
+        ops.swa(q, k, vt, cu, 1, 16, 0.1)
+    with pytest.raises(TypeError):
+        ops.swa(q.half(), k.half(), vt, cu, 1, 16, 0.1)
+    with pytest.raises(ValueError):
+        ops.swa(q[:, :4].contiguous(), k, vt, cu, 1, 16, -1.0)
+    with pytest.raises(RuntimeError):
+        ops.swa(q.cpu(), k, vt, cu, 1, 16, 0.1)

@@ -1,0 +1,119 @@
+"""CPU-side checks of the boundary: the shared library loads, exports every symbol the header
+declares, and the host-only helpers and error paths behave (no kernel is launched here)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _header_symbols():
+    src = open(os.path.join(ROOT, "include", "nsa_hip.h")).read()
+    src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+    return sorted(set(re.findall(r"\b(nsa_[a-z0-9_]+)\s*\(", src)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from nsa_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        from nsa_amd import build
+        build.build()
+    return _lib.load()
+
+
+def test_every_declared_symbol_is_exported_and_bound(lib):
+    from nsa_amd import _lib
+    names = _header_symbols()
+    assert "nsa_compress_fwd" in names and "nsa_slc_combine_fwd" in names
+    raw = ctypes.CDLL(_lib.LIB_PATH)
+    for n in names:
+        assert hasattr(raw, n), "header declares %s but the library does not export it" % n
+        assert n in _lib.SIGNATURES, "%s has no ctypes signature" % n
+    for n in _lib.SIGNATURES:
+        assert n in names, "%s is bound but not declared in include/nsa_hip.h" % n
+
+
+def test_signature_arity_matches_header(lib):
+    from nsa_amd import _lib
+    src = open(os.path.join(ROOT, "include", "nsa_hip.h")).read()
+    src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+    for name, (_, args) in _lib.SIGNATURES.items():
+        m = re.search(r"\b%s\s*\(([^)]*)\)" % name, src)
+        params = m.group(1).strip()
+        n = 0 if params in ("", "void") else params.count(",") + 1
+        assert n == len(args), "%s: header has %d parameters, binding has %d" % (name, n, len(args))
+
+
+def test_host_helpers(lib):
+    assert lib.nsa_version() >= 100
+    for cu_b, b in [(0, 0), (1, 1), (8, 1), (1000, 3), (32768, 1)]:
+        off = lib.nsa_transposed_offset(cu_b, b)
+        assert off % 8 == 0 and off >= cu_b
+    # offsets never overlap: next sequence starts after the previous one ends
+    cu = [0, 5, 5, 77, 1024, 1031]
+    offs = [lib.nsa_transposed_offset(c, b) for b, c in enumerate(cu)]
+    for b in range(len(cu) - 1):
+        assert offs[b] + (cu[b + 1] - cu[b]) <= offs[b + 1]
+    cols = lib.nsa_transposed_cols(cu[-1], len(cu) - 1)
+    assert cols % 64 == 0 and cols >= offs[-1] + 64
+
+
+def test_argument_errors_do_not_launch(lib):
+    # null pointers / bad sizes are rejected before any HIP call, so this runs without a GPU
+    rc = lib.nsa_swa_fwd(None, None, None, None, None, 1, 64, 4, 1, 64, 64, 128, 16, 0.1, 0, None)
+    assert rc == -1 and b"null" in lib.nsa_last_error_string()
+    buf = ctypes.create_string_buffer(4096)
+    p = ctypes.c_void_p((ctypes.addressof(buf) + 15) & ~15)
+    rc = lib.nsa_swa_fwd(p, p, p, p, p, 1, 64, 64, 2, 64, 64, 128, 16, 0.1, 0, None)
+    assert rc == -2 and b"group size" in lib.nsa_last_error_string()
+    rc = lib.nsa_swa_fwd(p, p, p, p, p, 1, 64, 4, 1, 48, 64, 128, 16, 0.1, 0, None)
+    assert rc == -2
+    rc = lib.nsa_swa_fwd(p, p, p, p, p, 1, 64, 4, 1, 64, 64, 128, 16, 0.1, 7, None)
+    assert rc == -1
+    rc = lib.nsa_slc_combine_fwd(p, p, p, p, None, None, None, None, 1, None, None, p, p, 1, 64, 4, 1, 64, 64, 128,
+                                 4, 60, 0.1, 1, 0, 0, None)
+    assert rc == -2 and b"block_size" in lib.nsa_last_error_string()
+    rc = lib.nsa_compress_fwd(p, None, None, p, p, p, 1, 10, 2, 60, 32, 16, 0, None)
+    assert rc == -2
+
+
+def test_python_wrappers_refuse_cpu_tensors_and_missing_library(monkeypatch):
+    from nsa_amd import _lib, ops
+    x = torch.zeros(64, 1, 64, dtype=torch.bfloat16)
+    cu = torch.tensor([0, 64], dtype=torch.int32)
+    with pytest.raises(RuntimeError):
+        ops.transpose(x, cu, 1)
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libnsa_hip.so")
+    with pytest.raises(_lib.NSALibraryError):
+        _lib.load()
+
+
+def test_host_side_shapes_and_counts():
+    from nsa_amd import ops
+    from nsa_amd.compression_kv import calc_compressed_len, conv_compressed_len
+    from oracle import nsa_oracle as O
+    for T in (31, 32, 64, 1000, 1024, 32768):
+        assert conv_compressed_len(T, 16, 32) == O.compressed_len_conv(T, 32, 16)
+    assert calc_compressed_len(1024, 16, 64) == (1024 - 64) // 16
+    for nc in (0, 3, 5, 63, 511, 2047):
+        for k, s, p in ((5, 4, 0), (5, 4, 2)):
+            assert ops.pool_bins(nc, k, s, p) == (O.pool_geometry(nc, k, s, p)[0] if nc > 0 else 0)
+    cu = torch.tensor([0, 100, 131, 1131], dtype=torch.int32)
+    assert ops.compressed_offsets(cu, 32, 16, 1).tolist() == [0, 5, 5, 66]
+    assert ops.compressed_offsets(cu, 32, 16, 0).tolist() == [0, 4, 4, 64]
+
+
+def test_module_keeps_reference_parameter_names():
+    from nsa_amd.nsa import NSAAttention
+    m = NSAAttention(64, True)
+    names = set(dict(m.named_parameters()))
+    assert names == {"compressor.compressor_k.weight", "compressor.compressor_k.bias",
+                     "compressor.compressor_v.weight", "compressor.compressor_v.bias",
+                     "gating.weight", "gating.bias"}
+    assert m.compressor.compressor_k.weight.shape == (64, 64, 32) and m.gating.weight.shape == (3, 64)
+    assert (m.pool_kernel_size, m.pool_stride, m.pool_padding) == (5, 4, 0)

@@ -1,0 +1,30 @@
+"""Seeded inputs shared by the GPU parity tests (generated on the CPU so oracle and kernels see the same bits)."""
+import torch
+
+from oracle import nsa_oracle as O
+
+TOL = {torch.bfloat16: 2e-2, torch.float32: 1e-4}   # max-abs bound per dtype
+
+
+def randn(*shape, seed, scale=1.0, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype)
+
+
+def make_qkv(T, Hq, Hkv, Dk, Dv, seed, dtype, scale=1.0):
+    q = randn(T, Hq, Dk, seed=seed, scale=scale, dtype=dtype)
+    k = randn(T, Hkv, Dk, seed=seed + 1, scale=scale, dtype=dtype)
+    v = randn(T, Hkv, Dv, seed=seed + 2, scale=scale, dtype=dtype)
+    gl = randn(T, Hq, 3, seed=seed + 3, dtype=dtype)          # gate logits
+    return q, k, v, gl
+
+
+def max_abs(a, b):
+    return float((a.double().cpu() - b.double().cpu()).abs().max()) if a.numel() else 0.0
+
+
+def ragged_cu(lens):
+    cu = [0]
+    for x in lens:
+        cu.append(cu[-1] + x)
+    return cu
