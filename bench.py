@@ -1,0 +1,182 @@
+#!/usr/bin/env python3
+"""NSA forward benchmark on one MI355X.
+
+One "step" is one pass of the NSA forward path (compress -> compressed attention + block selection
+-> sliding window -> selected blocks + gated combine) over one batch of synthetic input that is
+already resident in HBM.  Prints ONE JSON line.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload prefill_cfg4|prefill_cfg2|prefill_32k_d128]
+                  [--no-cpu-baseline]
+
+roofline: taken for the kernel stage with the largest share of the step; its algorithmic flops
+(causal compressed rows, whole valid selected blocks, exact window; nothing for exp / pooling /
+top-n or for the non-causal part of the importance scores) divided by its mean duration measured
+with events on the launch stream.  cpu_baseline: the CPU oracle (a port of the reference's naive
+torch path) on a bounded sample of query rows of the same workload, on this host's cores.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (lens, Hq, Hkv, Dqk, Dv, top_n, window, seed)
+    "prefill_cfg4": ([32768], 64, 4, 192, 128, 16, 512, 3),
+    "prefill_32k_d128": ([32768], 64, 4, 128, 128, 16, 512, 3),
+    "prefill_cfg2": ([8192], 64, 4, 128, 128, 16, 512, 1),
+}
+BLOCK, STRIDE, SEL_BLOCK = 32, 16, 64
+
+
+def flops_model(lens, hq, hkv, dqk, dv, window, valid_blocks_total):
+    """Effective sparse flops of one forward, split per branch."""
+    per = 2.0 * (dqk + dv)
+    cmp_f = swa_f = 0.0
+    for T in lens:
+        nc = (T - BLOCK) // STRIDE + 1 if T >= BLOCK else 0
+        # n_c(t) = clamp((t-32)//16 + 1, 0, Nc)
+        n_vis = 0
+        for t0 in range(0, T, STRIDE):          # n_c is constant over runs of STRIDE tokens
+            t = t0
+            cnt = min(max((t - BLOCK) // STRIDE + 1, 0), nc) if t >= BLOCK else 0
+            n_vis += cnt * min(STRIDE, T - t0)
+        cmp_f += hq * per * n_vis
+        w = sum(min(t + 1, window) for t in range(min(T, window))) + max(T - window, 0) * window
+        swa_f += hq * per * w
+    g = hq // hkv
+    slc_f = g * per * SEL_BLOCK * valid_blocks_total
+    return dict(cmp=cmp_f, slc=slc_f, swa=swa_f)
+
+
+def cpu_baseline(q, k, v, gl, top_n, window, budget_s=20.0):
+    """Oracle on a sample of query rows of the same workload; compression cost added pro rata."""
+    import torch
+    from oracle import nsa_oracle as O
+    T = q.shape[0]
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    p = O.NSAParams(BLOCK, STRIDE, SEL_BLOCK, top_n, window)
+    gates = torch.sigmoid(gl.float()).to(q.dtype)
+    nc = O.compressed_len_conv(T, BLOCK, STRIDE)
+    t0 = time.perf_counter()
+    ckcv = (O.compress_meanpool(k, BLOCK, STRIDE, nc), O.compress_meanpool(v, BLOCK, STRIDE, nc))
+    t_comp = time.perf_counter() - t0
+    g = torch.Generator().manual_seed(123)
+    n = 8
+    done_rows, spent = 0, 0.0
+    while True:
+        rows = torch.sort(torch.randint(0, T, (n,), generator=g)).values.unique()
+        t0 = time.perf_counter()
+        O.nsa_forward_single(q, k, v, gates, p, rows=rows, compressed=ckcv)
+        dt = time.perf_counter() - t0
+        done_rows += len(rows)
+        spent += dt
+        if spent > budget_s or n >= 512:
+            break
+        n *= 2
+    per_row = spent / done_rows + t_comp / T
+    return dict(value=1.0 / per_row, unit="tokens/s", cores=cores, kind="port",
+                sample="CPU oracle (torch fp32 port of the reference's naive path) on %d sampled query rows "
+                       "of the same workload in %.1f s; compression of the whole K/V (%.2f s) charged pro rata"
+                       % (done_rows, spent, t_comp))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="prefill_cfg4", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-budget", type=float, default=20.0)
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures the one-GPU NSA forward path; --gpus %d is not supported (this build has no "
+              "multi-GPU path)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from nsa_amd.nsa import NSAAttention
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = "cuda:0"
+    lens, hq, hkv, dqk, dv, top_n, window, seed = WORKLOADS[args.workload]
+    total = sum(lens)
+    g = torch.Generator().manual_seed(seed)
+    q = (torch.randn(total, hq, dqk, generator=g) * 0.5).bfloat16()
+    k = (torch.randn(total, hkv, dqk, generator=g) * 0.5).bfloat16()
+    v = (torch.randn(total, hkv, dv, generator=g) * 0.5).bfloat16()
+    gl = torch.randn(total, hq, 3, generator=g).bfloat16()
+    cu_list = [0]
+    for x in lens:
+        cu_list.append(cu_list[-1] + x)
+    cu = torch.tensor(cu_list, dtype=torch.int32, device=dev)
+    qd, kd, vd, gd = q.to(dev), k.to(dev), v.to(dev), gl.to(dev)
+    m = NSAAttention(dqk, True, compression_stride=STRIDE, compression_block=BLOCK, selection_block=SEL_BLOCK,
+                     selected_block_count=top_n, sliding_window=window, dtype=torch.bfloat16,
+                     compressor_mode="mean", gate_activation="sigmoid").to(dev)
+    max_len = 0 if len(set(lens)) == 1 else max(lens)
+
+    def step():
+        return m(qd, kd, vd, cu, max_len, gates=gd)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out = step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms = dt / args.steps * 1e3
+
+    # per-stage durations (events on the launch stream), separate from the timed region
+    acc = {}
+    reps = max(3, min(args.steps, 10))
+    idx = None
+    for _ in range(reps):
+        st = []
+        out, idx = m(qd, kd, vd, cu, max_len, gates=gd, stage_times=st, return_indices=True)
+        torch.cuda.synchronize()
+        for name, beg, end in st:
+            acc[name] = acc.get(name, 0.0) + beg.elapsed_time(end)
+    stage_ms = {n: t / reps for n, t in acc.items()}
+    assert torch.isfinite(out).all()
+
+    tok = torch.cat([torch.arange(x) for x in lens]).to(dev)
+    valid = ((idx >= 0) & (idx.long() * SEL_BLOCK <= tok[:, None, None])).sum().item()
+    fl = flops_model(lens, hq, hkv, dqk, dv, window, valid)
+    f_eff = fl["cmp"] + fl["slc"] + fl["swa"]
+    stage_flops = {"cmp_select": fl["cmp"], "swa": fl["swa"], "slc_combine": fl["slc"]}
+    dom = max(stage_flops, key=lambda n: stage_ms.get(n, 0.0))
+    dom_tflops = stage_flops[dom] / (stage_ms[dom] * 1e-3) / 1e12
+
+    res = {
+        "metric": "nsa_prefill_fwd_tokens_per_s", "value": total / (ms * 1e-3), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": args.workload, "seq_lens": lens if len(lens) > 1 else lens[0], "hq": hq, "hkv": hkv,
+                   "dqk": dqk, "dv": dv, "compress": "mean %d/%d" % (BLOCK, STRIDE), "sel_block": SEL_BLOCK,
+                   "top_n": top_n, "window": window, "gates": "sigmoid"},
+        "effective_tflops": f_eff / (ms * 1e-3) / 1e12,
+        "effective_flops": {"total": f_eff, **fl, "valid_selected_blocks": valid},
+        "mfma_peak_frac_whole_step": f_eff / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+        "stage_ms": stage_ms,
+        "roofline": {"bound": "mfma", "kernel": dom, "achieved": dom_tflops, "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": dom_tflops / PEAK_BF16_TFLOPS, "traffic": None},
+    }
+    if not args.no_cpu_baseline:
+        res["cpu_baseline"] = cpu_baseline(q, k, v, gl, top_n, window, args.cpu_budget)
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

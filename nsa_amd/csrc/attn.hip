@@ -143,6 +143,7 @@ cmp_select_kernel(const CmpArgs a) {
     Ns = (Nc + 2 * a.pool_p - a.pool_k + a.pool_s - 1) / a.pool_s + 1;
     if ((Ns - 1) * a.pool_s >= Nc + a.pool_p) --Ns;
   }
+  Ns = min(Ns, a.max_ns);   // LDS was sized for max_ns bins per token
   const int t_last = min(st.t0 + TQ, st.len) - 1;
   const T* qb = reinterpret_cast<const T*>(a.q);
   const T* ckb = reinterpret_cast<const T*>(a.ck) + (long)coff * a.ck_row_stride + (long)h * a.ck_head_stride;

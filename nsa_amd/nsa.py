@@ -72,12 +72,15 @@ class NSAAttention(nn.Module):
         max_seqlen_k=None,
         causal: bool = None,
         gates: Optional[torch.Tensor] = None,
+        stage_times: Optional[list] = None,
+        return_indices: bool = False,
     ) -> torch.Tensor:
         """q [total,Hq,Dk], k [total,Hkv,Dk], v [total,Hkv,Dv], cu_seqlens int32 [B+1] -> [total,Hq,Dv].
 
         max_seqlen: longest sequence (int); 0/None means "all sequences have total/B tokens" as in
         the reference.  gates [total,Hq,3] (selected, sliding, compressed) overrides the gating
-        Linear (pre-activation values)."""
+        Linear (pre-activation values).  stage_times: a list that receives (name, start_event,
+        end_event) per kernel stage; return_indices also returns the int32 block ids [total,Hkv,S]."""
         causal = self.causal if causal is None else causal
         cu = (cu_seqlens if cu_seqlens_k is None else cu_seqlens_k).to(torch.int32)
         batch = cu.numel() - 1
@@ -89,20 +92,35 @@ class NSAAttention(nn.Module):
         uniform = not max_seqlen
         seq_len = total // batch if uniform else int(max_seqlen)
 
-        ck, cv, cu_cmp, nc = self.compressor.compress_packed(k, v, cu, seq_len=seq_len if uniform else None)
+        def stage(name, fn):
+            if stage_times is None:
+                return fn()
+            beg, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            beg.record()
+            out = fn()
+            end.record()
+            stage_times.append((name, beg, end))
+            return out
+
+        ck, cv, cu_cmp, nc = stage("compress", lambda: self.compressor.compress_packed(
+            k, v, cu, seq_len=seq_len if uniform else None))
         max_nc = nc if nc is not None else conv_compressed_len(seq_len, self.compression_stride,
                                                                self.compression_block)
-        cvt = ops.transpose(cv, cu_cmp, batch)
-        vt = ops.transpose(v, cu, batch)
-        o_cmp, idx, _ = ops.cmp_attn_select(
+        cvt, vt = stage("transpose", lambda: (ops.transpose(cv, cu_cmp, batch), ops.transpose(v, cu, batch)))
+        o_cmp, idx, _ = stage("cmp_select", lambda: ops.cmp_attn_select(
             q, ck, cvt, cu, cu_cmp, batch, hkv, dv, ck.stride(0), ck.stride(1), self.compression_block,
             self.compression_stride, self.pool_kernel_size, self.pool_stride, self.pool_padding,
-            self.selected_block_count, max_nc, scale, causal=bool(causal), select=True, idx64=False)
+            self.selected_block_count, max_nc, scale, causal=bool(causal), select=True, idx64=False))
         if gates is None:
             gates = self.gating(q)                       # [total, Hq, 3]
         g = gates.reshape(total * hq, 3)
         g_slc, g_swa, g_cmp = (g[:, i].view(total, hq) for i in range(3))
-        o_swa = ops.swa(q, k, vt, cu, batch, self.sliding_window, scale) if self.sliding_window > 0 else None
+        o_swa = stage("swa", lambda: ops.swa(q, k, vt, cu, batch, self.sliding_window, scale)) \
+            if self.sliding_window > 0 else None
         act = _lib.GATE_SIGMOID if self.gate_activation == "sigmoid" else _lib.GATE_IDENTITY
-        return ops.slc_combine(q, k, vt, idx, None, g_slc, g_swa if o_swa is not None else None, g_cmp,
-                               o_swa, o_cmp, cu, batch, self.selection_block_size, scale, gate_act=act)
+        out = stage("slc_combine", lambda: ops.slc_combine(
+            q, k, vt, idx, None, g_slc, g_swa if o_swa is not None else None, g_cmp, o_swa, o_cmp, cu, batch,
+            self.selection_block_size, scale, gate_act=act))
+        if return_indices:
+            return out, idx
+        return out

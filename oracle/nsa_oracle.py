@@ -148,9 +148,16 @@ def _group(hq: int, hkv: int) -> int:
     return hq // hkv
 
 
+def _row_chunks(T: int, rows: Optional[torch.Tensor], chunk: int):
+    """Yields (positions in the output, token indices) for all rows or for the subset `rows`."""
+    ids = torch.arange(T) if rows is None else rows.to(torch.int64)
+    for i in range(0, ids.numel(), chunk):
+        yield slice(i, min(i + chunk, ids.numel())), ids[i:i + chunk]
+
+
 def importance_scores(q: torch.Tensor, ck: torch.Tensor, kernel: int, stride: int, pad: int,
-                      math_dtype=torch.float32, row_chunk: int = 1024) -> torch.Tensor:
-    """q [T,Hq,D], ck [Nc,Hkv,D] -> pooled block scores [T,Hkv,Ns].
+                      math_dtype=torch.float32, row_chunk: int = 1024, rows=None) -> torch.Tensor:
+    """q [T,Hq,D], ck [Nc,Hkv,D] -> pooled block scores [T,Hkv,Ns] (or [len(rows),Hkv,Ns]).
 
     p = softmax over ALL Nc columns of the raw q.ck (no scale, no causal mask), summed
     over the G query heads of each kv head, then average-pooled.
@@ -160,12 +167,13 @@ def importance_scores(q: torch.Tensor, ck: torch.Tensor, kernel: int, stride: in
     G = _group(Hq, Hkv)
     Ns, _ = pool_geometry(Nc, kernel, stride, pad)
     ckm = ck.to(math_dtype)
-    out = torch.zeros(T, Hkv, Ns, dtype=math_dtype)
-    for r0 in range(0, T, row_chunk):
-        qm = q[r0:r0 + row_chunk].to(math_dtype).reshape(-1, Hkv, G, D)
+    n_out = T if rows is None else len(rows)
+    out = torch.zeros(n_out, Hkv, Ns, dtype=math_dtype)
+    for pos, ids in _row_chunks(T, rows, row_chunk):
+        qm = q[ids].to(math_dtype).reshape(-1, Hkv, G, D)
         s = torch.einsum("thgd,chd->thgc", qm, ckm)
         p = torch.softmax(s, dim=-1).sum(2)                       # [t,Hkv,Nc]
-        out[r0:r0 + row_chunk] = pool_scores_direct(p, kernel, stride, pad)
+        out[pos] = pool_scores_direct(p, kernel, stride, pad)
     return out
 
 
@@ -181,7 +189,7 @@ def select_blocks(pooled: torch.Tensor, top_n: int) -> torch.Tensor:
 
 def compressed_attention(q: torch.Tensor, ck: torch.Tensor, cv: torch.Tensor, block: int,
                          stride: int, scale: Optional[float] = None,
-                         math_dtype=torch.float32, row_chunk: int = 1024) -> torch.Tensor:
+                         math_dtype=torch.float32, row_chunk: int = 1024, rows=None) -> torch.Tensor:
     """q [T,Hq,Dk], ck [Nc,Hkv,Dk], cv [Nc,Hkv,Dv] -> [T,Hq,Dv] in math_dtype.
 
     Column c is visible to row t iff c*stride + block <= t.  Rows that see nothing give 0.
@@ -191,12 +199,11 @@ def compressed_attention(q: torch.Tensor, ck: torch.Tensor, cv: torch.Tensor, bl
     G = _group(Hq, Hkv)
     scale = 1.0 / math.sqrt(Dk) if scale is None else scale
     ckm, cvm = ck.to(math_dtype), cv.to(math_dtype)
-    out = torch.zeros(T, Hq, Dv, dtype=math_dtype)
+    out = torch.zeros(T if rows is None else len(rows), Hq, Dv, dtype=math_dtype)
     col_end = torch.arange(Nc) * stride + block                   # first row that may see c
-    for r0 in range(0, T, row_chunk):
-        qm = q[r0:r0 + row_chunk].to(math_dtype).reshape(-1, Hkv, G, Dk)
-        rows = torch.arange(r0, r0 + qm.shape[0])
-        vis = col_end[None, :] <= rows[:, None]                   # [t,Nc]
+    for pos, ids in _row_chunks(T, rows, row_chunk):
+        qm = q[ids].to(math_dtype).reshape(-1, Hkv, G, Dk)
+        vis = col_end[None, :] <= ids[:, None]                    # [t,Nc]
         s = torch.einsum("thgd,chd->thgc", qm, ckm) * scale
         s = s.masked_fill(~vis[:, None, None, :], float("-inf"))
         m = s.amax(-1, keepdim=True)
@@ -205,7 +212,7 @@ def compressed_attention(q: torch.Tensor, ck: torch.Tensor, cv: torch.Tensor, bl
         z = e.sum(-1, keepdim=True)
         p = torch.where(z > 0, e / z.clamp_min(1e-300), torch.zeros_like(e))
         o = torch.einsum("thgc,chv->thgv", p, cvm)
-        out[r0:r0 + row_chunk] = o.reshape(-1, Hq, Dv)
+        out[pos] = o.reshape(-1, Hq, Dv)
     return out
 
 
@@ -226,7 +233,7 @@ def _masked_attention(qm, km, vm, allowed, scale):
 def selected_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                        block_indices: torch.Tensor, block_counts, block_size: int,
                        scale: Optional[float] = None, math_dtype=torch.float32,
-                       row_chunk: int = 512) -> torch.Tensor:
+                       row_chunk: int = 512, rows=None) -> torch.Tensor:
     """One sequence.  q [T,Hq,Dk], k [T,Hkv,Dk], v [T,Hkv,Dv], block_indices [T,Hkv,S] (block
     numbers local to the sequence).  Entry i of row t is used iff i < count, idx >= 0 and
     idx*block_size <= t; it contributes keys [idx*bs, min(idx*bs+bs-1, t)].  No usable entry -> 0.
@@ -237,7 +244,7 @@ def selected_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     S = block_indices.shape[-1]
     scale = 1.0 / math.sqrt(Dk) if scale is None else scale
     km, vm = k.to(math_dtype), v.to(math_dtype)
-    out = torch.zeros(T, Hq, Dv, dtype=math_dtype)
+    out = torch.zeros(T if rows is None else len(rows), Hq, Dv, dtype=math_dtype)
     if isinstance(block_counts, int):
         counts = torch.full((T, Hkv), block_counts, dtype=torch.int64)
     elif block_counts is None:
@@ -245,43 +252,40 @@ def selected_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     else:
         counts = block_counts.to(torch.int64)
     nblk = (T + block_size - 1) // block_size
-    for r0 in range(0, T, row_chunk):
-        r1 = min(r0 + row_chunk, T)
-        n = r1 - r0
-        rows = torch.arange(r0, r1)
-        idx = block_indices[r0:r1].to(torch.int64)                         # [n,Hkv,S]
-        use = (torch.arange(S)[None, None, :] < counts[r0:r1, :, None]) & (idx >= 0) \
-            & (idx * block_size <= rows[:, None, None])
+    for pos, ids in _row_chunks(T, rows, row_chunk):
+        n = ids.numel()
+        idx = block_indices[ids].to(torch.int64)                           # [n,Hkv,S]
+        use = (torch.arange(S)[None, None, :] < counts[ids][:, :, None]) & (idx >= 0) \
+            & (idx * block_size <= ids[:, None, None])
         blk = torch.zeros(n, Hkv, nblk + 1, dtype=torch.bool)
         tgt = torch.where(use, idx, torch.full_like(idx, nblk)).clamp(max=nblk)
         blk.scatter_(2, tgt, torch.ones_like(tgt, dtype=torch.bool))
         blk = blk[..., :nblk]
         allowed = blk.repeat_interleave(block_size, dim=2)[..., :T]        # [n,Hkv,T]
-        allowed = allowed & (torch.arange(T)[None, None, :] <= rows[:, None, None])
-        qm = q[r0:r1].to(math_dtype).reshape(n, Hkv, G, Dk)
-        out[r0:r1] = _masked_attention(qm, km, vm, allowed, scale).reshape(n, Hq, Dv)
+        allowed = allowed & (torch.arange(T)[None, None, :] <= ids[:, None, None])
+        qm = q[ids].to(math_dtype).reshape(n, Hkv, G, Dk)
+        out[pos] = _masked_attention(qm, km, vm, allowed, scale).reshape(n, Hq, Dv)
     return out
 
 
 def sliding_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, window: int,
                       scale: Optional[float] = None, math_dtype=torch.float32,
-                      row_chunk: int = 512) -> torch.Tensor:
+                      row_chunk: int = 512, rows=None) -> torch.Tensor:
     """One sequence.  Row t attends keys [max(0, t-window+1), t]."""
     T, Hq, Dk = q.shape
     _, Hkv, Dv = v.shape
     G = _group(Hq, Hkv)
     scale = 1.0 / math.sqrt(Dk) if scale is None else scale
     km, vm = k.to(math_dtype), v.to(math_dtype)
-    out = torch.zeros(T, Hq, Dv, dtype=math_dtype)
+    out = torch.zeros(T if rows is None else len(rows), Hq, Dv, dtype=math_dtype)
     cols = torch.arange(T)
-    for r0 in range(0, T, row_chunk):
-        r1 = min(r0 + row_chunk, T)
-        rows = torch.arange(r0, r1)
-        lo = max(0, r0 - window + 1)
-        allowed = (cols[None, lo:r1] <= rows[:, None]) & (cols[None, lo:r1] > rows[:, None] - window)
+    for pos, ids in _row_chunks(T, rows, row_chunk):
+        lo = max(0, int(ids.min()) - window + 1)
+        hi = int(ids.max()) + 1
+        allowed = (cols[None, lo:hi] <= ids[:, None]) & (cols[None, lo:hi] > ids[:, None] - window)
         allowed = allowed[:, None, :].expand(-1, Hkv, -1)
-        qm = q[r0:r1].to(math_dtype).reshape(r1 - r0, Hkv, G, Dk)
-        out[r0:r1] = _masked_attention(qm, km[lo:r1], vm[lo:r1], allowed, scale).reshape(-1, Hq, Dv)
+        qm = q[ids].to(math_dtype).reshape(ids.numel(), Hkv, G, Dk)
+        out[pos] = _masked_attention(qm, km[lo:hi], vm[lo:hi], allowed, scale).reshape(-1, Hq, Dv)
     return out
 
 
@@ -356,39 +360,55 @@ class NSAParams:
 
 
 def nsa_forward_single(q, k, v, gates, p: NSAParams, compressor=None,
-                       math_dtype=torch.float32, return_parts=False, force_idx=None):
+                       math_dtype=torch.float32, return_parts=False, force_idx=None, rows=None,
+                       compressed=None):
     """One sequence.  q [T,Hq,Dk], k [T,Hkv,Dk], v [T,Hkv,Dv], gates [T,Hq,3] already activated,
     ordered (selected, sliding, compressed).  compressor: None -> mean-pool, else a dict with
     'wk','wv' ([block*D, D] row j*D+i) and optional 'bk','bv'.  Returns [T,Hq,Dv] in q.dtype.
-    force_idx replaces the selected block ids (the returned 'idx_own' keeps the oracle's own).
+    force_idx [T,Hkv,S] replaces the selected block ids (the returned 'idx_own' keeps the oracle's own).
+    rows (sorted token ids) restricts the computation to those query rows: every result then has
+    len(rows) rows.  A sequence too short for one pooled bin selects nothing (the reference's
+    avg_pool1d would raise there); its compressed and sliding branches are still computed.
     """
     T = q.shape[0]
+    Hkv = k.shape[1]
     Nc = compressed_len_conv(T, p.block, p.stride)
-    if compressor is None:
+    if compressed is not None:         # (ck, cv) computed earlier by one of the compress_* functions
+        ck, cv = compressed
+    elif compressor is None:
         ck = compress_meanpool(k, p.block, p.stride, Nc, math_dtype)
         cv = compress_meanpool(v, p.block, p.stride, Nc, math_dtype)
     else:
         ck = compress_weighted(k, compressor["wk"], compressor.get("bk"), p.block, p.stride, Nc, math_dtype)
         cv = compress_weighted(v, compressor["wv"], compressor.get("bv"), p.block, p.stride, Nc, math_dtype)
-    Hkv = k.shape[1]
-    Ns, _ = pool_geometry(Nc, p.pool_kernel, p.pool_stride, p.pool_pad) if Nc > 0 else (0, None)
-    if Nc > 0 and Ns > 0:
-        pooled = importance_scores(q, ck, p.pool_kernel, p.pool_stride, p.pool_pad, math_dtype)
-        idx = select_blocks(pooled, p.top_n)
-        o_cmp = compressed_attention(q, ck, cv, p.block, p.stride, p.scale, math_dtype)
+    n_rows = T if rows is None else len(rows)
+    Ns = pool_geometry(Nc, p.pool_kernel, p.pool_stride, p.pool_pad)[0] if Nc > 0 else 0
+    if Ns > 0:
+        pooled = importance_scores(q, ck, p.pool_kernel, p.pool_stride, p.pool_pad, math_dtype, rows=rows)
+        idx_own = select_blocks(pooled, p.top_n)
     else:
-        pooled = torch.zeros(T, Hkv, 0, dtype=math_dtype)
-        idx = torch.full((T, Hkv, p.top_n), -1, dtype=torch.int64)
-        o_cmp = torch.zeros(T, q.shape[1], v.shape[2], dtype=math_dtype)
+        pooled = torch.zeros(n_rows, Hkv, 0, dtype=math_dtype)
+        idx_own = torch.full((n_rows, Hkv, p.top_n), -1, dtype=torch.int64)
+    if Nc > 0:
+        o_cmp = compressed_attention(q, ck, cv, p.block, p.stride, p.scale, math_dtype, rows=rows)
+    else:
+        o_cmp = torch.zeros(n_rows, q.shape[1], v.shape[2], dtype=math_dtype)
     if force_idx is not None:          # branch parity independent of how score ties were broken
-        idx = force_idx.to(torch.int64)
-    o_slc = selected_attention(q, k, v, idx, None, p.sel_block, p.scale, math_dtype)
-    o_swa = sliding_attention(q, k, v, p.window, p.scale, math_dtype) if p.window > 0 else None
-    gm = gates.to(math_dtype)
+        idx_full = force_idx.to(torch.int64)
+        idx = idx_full if rows is None else idx_full[rows]
+    else:
+        idx = idx_own
+        if rows is None:
+            idx_full = idx
+        else:
+            idx_full = torch.full((T, Hkv, p.top_n), -1, dtype=torch.int64)
+            idx_full[rows] = idx
+    o_slc = selected_attention(q, k, v, idx_full, None, p.sel_block, p.scale, math_dtype, rows=rows)
+    o_swa = sliding_attention(q, k, v, p.window, p.scale, math_dtype, rows=rows) if p.window > 0 else None
+    gm = gates.to(math_dtype) if rows is None else gates[rows].to(math_dtype)
     out = gated_combine(gm[..., 0], o_slc, gm[..., 1], o_swa, gm[..., 2], o_cmp).to(q.dtype)
     if return_parts:
-        own = select_blocks(pooled, p.top_n) if pooled.shape[-1] > 0 else idx
-        return out, dict(ck=ck, cv=cv, pooled=pooled, idx=idx, idx_own=own, o_cmp=o_cmp, o_slc=o_slc,
+        return out, dict(ck=ck, cv=cv, pooled=pooled, idx=idx, idx_own=idx_own, o_cmp=o_cmp, o_slc=o_slc,
                          o_swa=o_swa)
     return out
 
@@ -418,21 +438,20 @@ def nsa_decode_step(q_last, k_cache, v_cache, gates_last, p: NSAParams, math_dty
     ck = compress_meanpool(k_cache, p.block, p.stride, Nc, math_dtype)
     cv = compress_meanpool(v_cache, p.block, p.stride, Nc, math_dtype)
     parts = {}
+    scale = 1.0 / math.sqrt(Dk) if p.scale is None else p.scale
     if Nc > 0 and pool_geometry(Nc, p.pool_kernel, p.pool_stride, p.pool_pad)[0] > 0:
         pooled = importance_scores(q1, ck, p.pool_kernel, p.pool_stride, p.pool_pad, math_dtype)
         idx = select_blocks(pooled, p.top_n)[0]                        # [Hkv,S]
-        n_vis = min(max((t - p.block) // p.stride + 1, 0), Nc)
-        scale = 1.0 / math.sqrt(Dk) if p.scale is None else p.scale
-        if n_vis > 0:
-            s = torch.einsum("hgd,chd->hgc", q_last.to(math_dtype).reshape(Hkv, -1, Dk),
-                             ck[:n_vis].to(math_dtype)) * scale
-            o_cmp = torch.einsum("hgc,chv->hgv", torch.softmax(s, -1), cv[:n_vis].to(math_dtype))
-            o_cmp = o_cmp.reshape(Hq, Dv)
-        else:
-            o_cmp = torch.zeros(Hq, Dv, dtype=math_dtype)
         parts["pooled"] = pooled[0]
     else:
         idx = torch.full((Hkv, p.top_n), -1, dtype=torch.int64)
+    n_vis = min(max((t - p.block) // p.stride + 1, 0), Nc) if t >= p.block else 0
+    if n_vis > 0:
+        s = torch.einsum("hgd,chd->hgc", q_last.to(math_dtype).reshape(Hkv, -1, Dk),
+                         ck[:n_vis].to(math_dtype)) * scale
+        o_cmp = torch.einsum("hgc,chv->hgv", torch.softmax(s, -1), cv[:n_vis].to(math_dtype))
+        o_cmp = o_cmp.reshape(Hq, Dv)
+    else:
         o_cmp = torch.zeros(Hq, Dv, dtype=math_dtype)
     scale = 1.0 / math.sqrt(Dk) if p.scale is None else p.scale
     G = Hq // Hkv

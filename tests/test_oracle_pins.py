@@ -275,3 +275,23 @@ def test_compare_selection_rule():
     assert O.compare_selection(torch.tensor([[[1, 0]]]), ref, pooled) == (1, 1, 0, 0)
     assert O.compare_selection(torch.tensor([[[0, 2]]]), ref, pooled) == (1, 0, 1, 0)
     assert O.compare_selection(torch.tensor([[[0, 3]]]), ref, pooled) == (1, 0, 0, 1)
+
+
+def test_row_subset_equals_full_run():
+    p = O.NSAParams(32, 16, 64, 3, 100)
+    q, k, v, gates = _cfg(700, 8, 2, 32, 16, 60)
+    full, fp = O.nsa_forward_single(q, k, v, gates, p, return_parts=True)
+    rows = torch.tensor([0, 1, 31, 32, 63, 64, 65, 300, 511, 512, 698, 699])
+    sub, sp = O.nsa_forward_single(q, k, v, gates, p, return_parts=True, rows=rows)
+    torch.testing.assert_close(sub, full[rows], rtol=1e-5, atol=1e-6)
+    for key in ("o_cmp", "o_slc", "o_swa", "pooled"):
+        torch.testing.assert_close(sp[key], fp[key][rows], rtol=1e-5, atol=1e-6)
+    assert torch.equal(sp["idx"], fp["idx"][rows])
+
+
+def test_short_sequence_has_compressed_branch_but_no_selection():
+    p = O.NSAParams(32, 16, 64, 2, 16)
+    q, k, v, gates = _cfg(64, 4, 2, 16, 16, 61)       # Nc = 3 < pool kernel 5
+    out, parts = O.nsa_forward_single(q, k, v, gates, p, return_parts=True)
+    assert (parts["idx"] == -1).all() and torch.count_nonzero(parts["o_slc"]) == 0
+    assert torch.count_nonzero(parts["o_cmp"][32:]) > 0 and torch.count_nonzero(parts["o_cmp"][:32]) == 0

@@ -28,3 +28,21 @@ def ragged_cu(lens):
     for x in lens:
         cu.append(cu[-1] + x)
     return cu
+
+
+def within(out, ref, dtype, large_values=False):
+    """max-abs bar of the dtype; with large_values (raw, un-activated gates make |out| > 4) one bf16
+    unit in the last place of the reference is allowed on top, since both sides round once to bf16."""
+    a, b = out.double().cpu(), ref.double().cpu()
+    bound = torch.full_like(b, TOL[dtype])
+    if large_values and dtype == torch.bfloat16:
+        bound = bound + b.abs() * 2.0 ** -7
+    return bool(((a - b).abs() <= bound).all())
+
+
+def sample_rows(T, n, seed, edges=(0, 1, 31, 32, 33, 63, 64, 65, 511, 512, 513)):
+    g = torch.Generator().manual_seed(seed)
+    r = set(int(x) for x in torch.randint(0, T, (n,), generator=g))
+    r.update(e for e in edges if e < T)
+    r.update((T - 1, T - 2, max(T - 65, 0)))
+    return torch.tensor(sorted(r))
