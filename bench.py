@@ -155,7 +155,8 @@ def main():
     valid = ((idx >= 0) & (idx.long() * SEL_BLOCK <= tok[:, None, None])).sum().item()
     fl = flops_model(lens, hq, hkv, dqk, dv, window, valid)
     f_eff = fl["cmp"] + fl["slc"] + fl["swa"]
-    stage_flops = {"cmp_select": fl["cmp"], "swa": fl["swa"], "slc_combine": fl["slc"]}
+    # block_select carries no credited flops: its score tiles are the uncredited non-causal pass
+    stage_flops = {"cmp_attn": fl["cmp"], "swa": fl["swa"], "slc_combine": fl["slc"]}
     dom = max(stage_flops, key=lambda n: stage_ms.get(n, 0.0))
     dom_tflops = stage_flops[dom] / (stage_ms[dom] * 1e-3) / 1e12
 

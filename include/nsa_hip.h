@@ -68,16 +68,30 @@ int nsa_transpose_fwd(const void* x, void* out, const int32_t* cu, int batch, in
  *   q [total, hq, dk]; ck rows at ck + (cu_cmp[b] + c)*ck_row_stride + h*ck_head_stride (dk elements);
  *   cvt transposed [hkv][dv][cvt_cols] over cu_cmp; o [total, hq, dv];
  *   indices [total, hkv, top_n] int32 or int64 (idx64), descending score, -1 where fewer bins exist;
- *   NULL skips the selection;  pooled (optional, float) [total, hkv, pooled_stride] block scores.
+ *   NULL skips the selection;  pooled (optional, float) [total, hkv, pooled_stride] block scores;
+ *   lse (float) [total, hq] receives the log-sum-exp of the raw scores q.ck over all compressed rows
+ *   (the reference's M without its mask and scale); required when indices is given.
  *   Compressed row c of a sequence is visible to token t iff c*stride + block <= t (causal != 0;
  *   causal == 0 makes every row visible).
  *   max_ns >= pooled bins of the longest sequence (sizes LDS). */
 int nsa_cmp_attn_select_fwd(const void* q, const void* ck, const void* cvt, void* o, void* indices,
-                            float* pooled, const int32_t* cu_seqlens, const int32_t* cu_cmp, int batch,
+                            float* pooled, float* lse, const int32_t* cu_seqlens, const int32_t* cu_cmp, int batch,
                             int total, int hq, int hkv, int dk, int dv, int64_t ck_row_stride,
                             int64_t ck_head_stride, int cvt_cols, int block, int stride, int pool_kernel,
                             int pool_stride, int pool_pad, int top_n, int max_ns, int pooled_stride,
                             float scale, int causal, int idx64, int dtype, nsa_stream_t stream);
+
+/* The two halves of nsa_cmp_attn_select_fwd as separate launches: compressed attention (writes o
+ * and lse) and block selection (reads lse).  Same arguments and meaning as above. */
+int nsa_cmp_attn_fwd(const void* q, const void* ck, const void* cvt, void* o, float* lse,
+                     const int32_t* cu_seqlens, const int32_t* cu_cmp, int batch, int total, int hq, int hkv,
+                     int dk, int dv, int64_t ck_row_stride, int64_t ck_head_stride, int cvt_cols, int block,
+                     int stride, float scale, int causal, int dtype, nsa_stream_t stream);
+int nsa_block_select_fwd(const void* q, const void* ck, const float* lse, void* indices, float* pooled,
+                         const int32_t* cu_seqlens, const int32_t* cu_cmp, int batch, int total, int hq, int hkv,
+                         int dk, int64_t ck_row_stride, int64_t ck_head_stride, int pool_kernel, int pool_stride,
+                         int pool_pad, int top_n, int max_ns, int pooled_stride, int idx64, int dtype,
+                         nsa_stream_t stream);
 
 /* Sliding window attention: token t attends keys [max(0, t-window+1), t] of its sequence.  Replaces
  * the window loop of nsa/selection_attn.py:483-517.  q [total,hq,dk], k [total,hkv,dk],

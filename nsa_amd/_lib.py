@@ -24,8 +24,11 @@ SIGNATURES = {
     "nsa_transposed_cols": (_I, [_I, _I]),
     "nsa_compress_fwd": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
     "nsa_transpose_fwd": (_I, [_P, _P, _P, _I, _I, _I, _L, _L, _I, _I, _P]),
-    "nsa_cmp_attn_select_fwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _L, _I,
+    "nsa_cmp_attn_select_fwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _L, _I,
                                      _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P]),
+    "nsa_cmp_attn_fwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _L, _I, _I, _I, _F, _I, _I, _P]),
+    "nsa_block_select_fwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _L, _L, _I, _I, _I, _I, _I, _I,
+                                  _I, _I, _P]),
     "nsa_swa_fwd": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P]),
     "nsa_slc_combine_fwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _L, _P, _P, _P, _P, _I, _I, _I, _I, _I,
                                  _I, _I, _I, _I, _F, _I, _I, _I, _P]),

@@ -1,422 +1,239 @@
-// The three attention branches of the NSA forward path on gfx950 MFMA.
+// Attention over a contiguous key stream shared by a whole token tile: the compressed branch
+// (keys = compressed rows, plus the log-sum-exp of the raw scores that the block-importance kernel
+// needs) and the sliding-window branch (keys = the union of the tile's windows).
 //
-// Row space. For one kv head the G query heads of a token are G consecutive "rows"; G is padded
-// to a power of two Gp <= 16 and 16 consecutive rows form one row group = the 16 columns of an
-// MFMA tile (G = 16: one token per group, G = 4: four tokens per group).  All heads of a group
-// share the K/V they read, which is what makes the GQA group the MFMA N dimension.
+// One workgroup of NW wavefronts owns NW*NG row groups (NW*NG*16 rows: 16 tokens for a GQA group
+// of 16).  Keys stream through LDS in chunks of CH rows, K row-major and V key-contiguous, double
+// buffered: the global loads of chunk i+1 are issued into registers before chunk i is computed and
+// written to the other buffer afterwards, one barrier per chunk.  Every wavefront reads each K/V
+// fragment from LDS once and feeds it to NG MFMAs (register blocking over row groups).
 //
-//   cmp_select_kernel  compressed attention (online softmax over the causally visible compressed
-//                      rows) + block importance: softmax of the raw q.ck over ALL compressed rows,
-//                      summed over the G heads, average-pooled into selection blocks, wavefront
-//                      top-n.  Pass 1 streams ck / cv^T through LDS once per token tile and also
-//                      accumulates the row-wise log-sum-exp of the raw scores; pass 2 recomputes the
-//                      score tiles in the un-transposed orientation so that the head sum is an
-//                      in-lane add plus two lane swaps, and bins exp(s - lse) in LDS.
-//   swa_kernel         sliding window attention; a token tile streams the union of its windows
-//                      through LDS once.
-//   slc_combine_kernel selected-block attention, one wavefront per row group reading its blocks
-//                      straight from global memory in fragment layout, and the gated combine of
-//                      the three branches in the epilogue.
-#include "common.h"
-#include "kernels.h"
+// Softmax bookkeeping per row: one running maximum of the raw scores.  In the compressed branch it
+// runs over ALL compressed rows (the importance softmax is not causal) and serves both sums:
+//   li += exp(s - M)                         every row      -> lse = M + log(li)
+//   l  += exp(scale*(s - M)), O += p V       visible rows   -> o = O / l
+// so each score tile costs one maximum reduction.  exp(scale*(s - M)) stays exact unless the
+// visible scores sit more than ~87/scale below the largest hidden one.
+//
+// The selected-block branch (one wavefront per row group, blocks read straight from global memory
+// in fragment layout) and the gated combine of the three branches live here as well.
+#include "tiles.h"
 
 namespace nsa {
 
-// ------------------------------------------------------------------------------------------------
-// tile pieces
-
-template <typename T, int DK, int DV, int NG>
-__device__ __forceinline__ void scores32(const T* __restrict__ a0p, const T* __restrict__ a1p,
-                                         const RowGroup<T, DK, DV> (&grp)[NG], f32x4_t (&s0)[NG],
-                                         f32x4_t (&s1)[NG]) {
-#pragma unroll
-  for (int j = 0; j < NG; ++j) {
-    s0[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    s1[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  }
-#pragma unroll
-  for (int kk = 0; kk < DK / 32; ++kk) {
-    const vec8_t<T> a0 = load8(a0p + 32 * kk);
-    const vec8_t<T> a1 = load8(a1p + 32 * kk);
-#pragma unroll
-    for (int j = 0; j < NG; ++j) {
-      s0[j] = mma16(a0, grp[j].q[kk], s0[j]);
-      s1[j] = mma16(a1, grp[j].q[kk], s1[j]);
-    }
-  }
-}
-
-template <typename T, int DK, int DV, int NG>
-__device__ __forceinline__ void pv32(const T* __restrict__ vp, long tile_stride,
-                                     RowGroup<T, DK, DV> (&grp)[NG], const vec8_t<T> (&pb)[NG],
-                                     const bool (&active)[NG]) {
-#pragma unroll
-  for (int t = 0; t < DV / 16; ++t) {
-    const vec8_t<T> av = load8(vp + t * tile_stride);
-#pragma unroll
-    for (int j = 0; j < NG; ++j)
-      if (active[j]) grp[j].o[t] = mma16(av, pb[j], grp[j].o[t]);
-  }
-}
-
-struct RowMap {
-  int tok;      // token of this lane's column (sequence local), may be >= len
-  int gidx;     // head inside the GQA group, may be >= G
-  bool valid;
+struct StreamParams {
+  const void* q; const void* k; const void* vt; void* o; float* lse;
+  const int32_t* cu_seq; const int32_t* cu_key;
+  int batch, hq, hkv;
+  long k_row_stride, k_head_stride; int vt_cols;
+  int block, stride, window, causal;
+  float scale;
 };
 
-__device__ __forceinline__ RowMap map_row(int t0, int group_in_tile, int n, int lgp, int G, int len) {
-  const int r = group_in_tile * 16 + n;
-  RowMap m;
-  m.tok = t0 + (r >> lgp);
-  m.gidx = r & ((1 << lgp) - 1);
-  m.valid = (m.tok < len) && (m.gidx < G);
-  return m;
-}
-
-template <typename T, int DK, int DV>
-__device__ __forceinline__ void load_q(RowGroup<T, DK, DV>& grp, const T* __restrict__ q, long start,
-                                       const RowMap& rm, int len, int hq, int h, int G, int g) {
-  const int tc = rm.tok < len ? rm.tok : len - 1;
-  const int gc = rm.gidx < G ? rm.gidx : G - 1;
-  const T* qp = q + ((start + tc) * hq + h * G + gc) * DK + 8 * g;
-#pragma unroll
-  for (int kk = 0; kk < DK / 32; ++kk) grp.q[kk] = load8(qp + 32 * kk);
-}
-
-// 16-byte pieces of `rows` rows of `row_elems` elements: global (row clamp) -> LDS [rows][ld].
-template <typename T>
-__device__ __forceinline__ void stage_rows(T* __restrict__ dst, int ld, const T* __restrict__ src,
-                                           long src_row_stride, int first_row, int last_valid_row,
-                                           int rows, int row_elems) {
-  const int pieces = row_elems / 8;
-  for (int p = threadIdx.x; p < rows * pieces; p += blockDim.x) {
-    const int r = p / pieces, pc = p % pieces;
-    int sr = first_row + r;
-    sr = sr > last_valid_row ? last_valid_row : sr;
-    store8(dst + r * ld + pc * 8, load8(src + (long)sr * src_row_stride + pc * 8));
-  }
-}
-
-template <typename T, int DV>
-__device__ __forceinline__ void store_rows(T* __restrict__ out_row, const f32x4_t (&o)[DV / 16], float inv,
-                                           int g) {
-#pragma unroll
-  for (int t = 0; t < DV / 16; ++t) {
-    T* p = out_row + t * 16 + 4 * g;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) p[i] = (T)(o[t][i] * inv);
-  }
-}
-
-__device__ __forceinline__ int ilog2(int x) { return 31 - __builtin_clz(x); }
-__device__ __forceinline__ int next_pow2(int x) {
-  int p = 1;
-  while (p < x) p <<= 1;
-  return p;
-}
-
-// ------------------------------------------------------------------------------------------------
-// compressed attention + block importance + top-n
-
-template <typename T, int DK, int DV, int NG, int CH>
-__global__ void __launch_bounds__(256)
-cmp_select_kernel(const CmpArgs a) {
-  constexpr int KLD = DK + 8, VLD = CH + 8, ROWS = 64 * NG;
+template <typename T, int DK, int DV, int NG, int CH, int NW, bool CMP>
+__global__ void __launch_bounds__(NW * 64)
+stream_attn_kernel(const StreamParams a) {
+  constexpr int KLD = DK + 8, VLD = CH + 8, ROWS = NW * NG * 16, NT = NW * 64;
+  constexpr int KPIECES = CH * DK / 8, VPIECES = DV * CH / 8;
+  constexpr int KPT = (KPIECES + NT - 1) / NT, VPT = (VPIECES + NT - 1) / NT;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  T* ldsK = reinterpret_cast<T*>(smem_raw);
-  T* ldsV = ldsK + CH * KLD;
-  float* bins = reinterpret_cast<float*>(ldsV + DV * VLD);
+  T* ldsK = reinterpret_cast<T*>(smem_raw);          // [2][CH][KLD]
+  T* ldsV = ldsK + 2 * CH * KLD;                     // [2][DV][VLD]
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n = lane & 15, g = lane >> 4;
   const int G = a.hq / a.hkv, Gp = next_pow2(G), lgp = ilog2(Gp);
   const int TQ = ROWS >> lgp;
   const SeqTile st = find_tile(a.cu_seq, a.batch, TQ, blockIdx.x);
   if (!st.valid) return;
   const int h = blockIdx.y;
-  const int coff = a.cu_cmp[st.b];
-  const int Nc = a.cu_cmp[st.b + 1] - coff;
-  const int ctoff = transposed_offset(coff, st.b);
-  int Ns = 0;
-  if (Nc > 0 && Nc + 2 * a.pool_p >= a.pool_k) {
-    Ns = (Nc + 2 * a.pool_p - a.pool_k + a.pool_s - 1) / a.pool_s + 1;
-    if ((Ns - 1) * a.pool_s >= Nc + a.pool_p) --Ns;
-  }
-  Ns = min(Ns, a.max_ns);   // LDS was sized for max_ns bins per token
   const int t_last = min(st.t0 + TQ, st.len) - 1;
-  const T* qb = reinterpret_cast<const T*>(a.q);
-  const T* ckb = reinterpret_cast<const T*>(a.ck) + (long)coff * a.ck_row_stride + (long)h * a.ck_head_stride;
-  const T* cvtb = reinterpret_cast<const T*>(a.cvt) + (long)h * DV * a.cvt_cols + ctoff;
 
-  RowGroup<T, DK, DV> grp[NG];
-  RowMap rm[NG];
-  int cmaxv[NG];      // last compressed row visible to this lane's column, -1 if none
-  int cmax_grp[NG];   // the same for the last token of the group (wave uniform)
-  float mi[NG], li[NG];
-#pragma unroll
-  for (int j = 0; j < NG; ++j) {
-    const int gi = wave * NG + j;
-    rm[j] = map_row(st.t0, gi, n, lgp, G, st.len);
-    load_q(grp[j], qb, (long)st.start, rm[j], st.len, a.hq, h, G, g);
-    group_reset(grp[j]);
-    cmaxv[j] = !a.causal ? Nc - 1 : (rm[j].tok >= a.block ? (rm[j].tok - a.block) / a.stride : -1);
-    const int tl = min(st.t0 + ((gi * 16 + 15) >> lgp), st.len - 1);
-    cmax_grp[j] = !a.causal ? Nc - 1 : (tl >= a.block ? (tl - a.block) / a.stride : -1);
-    mi[j] = kNegInf;
-    li[j] = 0.f;
+  // key space of this sequence
+  int nkeys, koff, vtoff;
+  if (CMP) {
+    koff = a.cu_key[st.b];
+    nkeys = a.cu_key[st.b + 1] - koff;
+    vtoff = transposed_offset(koff, st.b);
+  } else {
+    koff = st.start;
+    nkeys = st.len;
+    vtoff = transposed_offset(st.start, st.b);
   }
-  const int cmax_tile = !a.causal ? Nc - 1 : (t_last >= a.block ? (t_last - a.block) / a.stride : -1);
-  const float c_attn = a.scale * kLog2e;
-
-  // ---- pass 1: attention over visible rows, log-sum-exp of raw scores over all rows
-  for (int c0 = 0; c0 < Nc; c0 += CH) {
-    __syncthreads();
-    stage_rows(ldsK, KLD, ckb, a.ck_row_stride, c0, Nc - 1, CH, DK);
-    const bool need_v = c0 <= cmax_tile;
-    if (need_v) stage_rows(ldsV, VLD, cvtb + c0, (long)a.cvt_cols, 0, DV - 1, DV, CH);
-    __syncthreads();
-#pragma unroll
-    for (int sub = 0; sub < CH / 32; ++sub) {
-      const int cb = c0 + 32 * sub;
-      if (cb >= Nc) break;
-      f32x4_t s0[NG], s1[NG];
-      const T* ks = ldsK + 32 * sub * KLD + 8 * g;
-      scores32<T, DK, DV, NG>(ks + chunk_key_of_row(0, n) * KLD, ks + chunk_key_of_row(1, n) * KLD, grp, s0, s1);
-      vec8_t<T> pb[NG];
-      bool act[NG];
-#pragma unroll
-      for (int j = 0; j < NG; ++j) {
-        float s[8], sm[8], p[8];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) { s[i] = s0[j][i]; s[4 + i] = s1[j][i]; }
-        // importance statistics: every existing column, natural exponent
-        float mx = kNegInf;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const int c = cb + 8 * g + i;
-          sm[i] = c < Nc ? s[i] : kNegInf;
-          mx = fmaxf(mx, sm[i]);
-        }
-        mx = colgroup_max(mx);
-        const float m_new = fmaxf(mi[j], mx);   // finite: column cb exists
-        float sum = 0.f;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) sum += fast_exp2((sm[i] - m_new) * kLog2e);
-        li[j] = li[j] * fast_exp2((mi[j] - m_new) * kLog2e) + sum;
-        mi[j] = m_new;
-        // attention: causally visible columns only
-        act[j] = cb <= cmax_grp[j];
-        if (act[j]) {
-#pragma unroll
-          for (int i = 0; i < 8; ++i) {
-            const int c = cb + 8 * g + i;
-            sm[i] = (c <= cmaxv[j] && c < Nc) ? s[i] : kNegInf;
-          }
-          softmax_update(grp[j], sm, c_attn, p);
-          pb[j] = pack8<T>(p);
-        } else {
-          pb[j] = zero8<T>();
-        }
-      }
-      bool any = false;
-#pragma unroll
-      for (int j = 0; j < NG; ++j) any |= act[j];
-      if (any) pv32<T, DK, DV, NG>(ldsV + n * VLD + 32 * sub + 8 * g, 16 * VLD, grp, pb, act);
-    }
-  }
-
-  // ---- compressed-attention output
-  T* ob = reinterpret_cast<T*>(a.o);
-  float lse[NG];
-#pragma unroll
-  for (int j = 0; j < NG; ++j) {
-    const float lt = colgroup_sum(grp[j].l);
-    const float inv = lt > 0.f ? 1.0f / lt : 0.f;
-    if (rm[j].valid)
-      store_rows<T, DV>(ob + (((long)st.start + rm[j].tok) * a.hq + h * G + rm[j].gidx) * DV, grp[j].o, inv, g);
-    const float lit = colgroup_sum(li[j]);
-    lse[j] = rm[j].valid ? mi[j] + __logf(lit) : __builtin_huge_valf();   // +inf kills padded rows
-  }
-  if (a.indices == nullptr) return;
-
-  // ---- pass 2: importance bins
-  __syncthreads();
-  for (int i = threadIdx.x; i < TQ * Ns; i += 256) bins[i] = 0.f;
-  float lse_r[NG][4];   // lse of rows 4g+i (the rows this lane holds in the un-transposed tile)
-#pragma unroll
-  for (int j = 0; j < NG; ++j)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) lse_r[j][i] = __shfl(lse[j], 4 * g + i);
-
-  for (int c0 = 0; c0 < Nc && Ns > 0; c0 += CH) {
-    __syncthreads();
-    stage_rows(ldsK, KLD, ckb, a.ck_row_stride, c0, Nc - 1, CH, DK);
-    __syncthreads();
-#pragma unroll
-    for (int kt = 0; kt < CH / 16; ++kt) {
-      const int cb = c0 + 16 * kt;
-      if (cb >= Nc) break;
-      f32x4_t s[NG];
-#pragma unroll
-      for (int j = 0; j < NG; ++j) s[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-      const T* kp = ldsK + (16 * kt + n) * KLD + 8 * g;
-#pragma unroll
-      for (int kk = 0; kk < DK / 32; ++kk) {
-        const vec8_t<T> kb = load8(kp + 32 * kk);
-#pragma unroll
-        for (int j = 0; j < NG; ++j) s[j] = mma16(grp[j].q[kk], kb, s[j]);   // rows = heads, cols = keys
-      }
-      const int c = cb + n;
-      // bins that contain column c: j*s - p <= c < j*s - p + k
-      const int num = c + a.pool_p - a.pool_k + 1;
-      const int j_lo = num <= 0 ? 0 : (num + a.pool_s - 1) / a.pool_s;
-      const int j_hi = min((c + a.pool_p) / a.pool_s, Ns - 1);
-#pragma unroll
-      for (int j = 0; j < NG; ++j) {
-        const int gi = wave * NG + j;
-        float e[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) e[i] = fast_exp2((s[j][i] - lse_r[j][i]) * kLog2e);
-        if (lgp >= 2) {
-          float v = (e[0] + e[1]) + (e[2] + e[3]);
-          if (lgp >= 3) v += __shfl_xor(v, 16);
-          if (lgp >= 4) v += __shfl_xor(v, 32);
-          const bool adder = lgp >= 4 ? (g == 0) : (lgp == 3 ? ((g & 1) == 0) : true);
-          const int tl = (gi * 16 + 4 * g) >> lgp;
-          if (adder && c < Nc)
-            for (int b = j_lo; b <= j_hi; ++b) atomicAdd(&bins[tl * Ns + b], v);
-        } else {
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int tl = (gi * 16 + 4 * g + i) >> lgp;
-            if (c < Nc)
-              for (int b = j_lo; b <= j_hi; ++b) atomicAdd(&bins[tl * Ns + b], e[i]);
-          }
-        }
-      }
-    }
-  }
-  __syncthreads();
-
-  // ---- average (divisor rule of a ceil-mode pool with padding counted) and top-n per token
-  volatile float* vb = bins;
-  for (int tl = wave; tl < TQ; tl += 4) {
-    const int t = st.t0 + tl;
-    if (t >= st.len) break;
-    const long orow = ((long)st.start + t) * a.hkv + h;
-    for (int b = lane; b < Ns; b += 64) {
-      const int lo = b * a.pool_s - a.pool_p;
-      const int div = min(lo + a.pool_k, Nc + a.pool_p) - lo;
-      const float v = vb[tl * Ns + b] / (float)div;
-      vb[tl * Ns + b] = v;
-      if (a.pooled != nullptr) a.pooled[orow * a.pooled_stride + b] = v;
-    }
-    for (int r = 0; r < a.top_n; ++r) {
-      float best = -1.f;
-      int bi = 0x7fffffff;
-      for (int b = lane; b < Ns; b += 64) {
-        const float v = vb[tl * Ns + b];
-        if (v > best) { best = v; bi = b; }
-      }
-#pragma unroll
-      for (int off = 1; off < 64; off <<= 1) {
-        const float ov = __shfl_xor(best, off);
-        const int oi = __shfl_xor(bi, off);
-        if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
-      }
-      const bool found = best >= 0.f;
-      if (found && (bi & 63) == lane) vb[tl * Ns + bi] = -1.f;
-      if (lane == 0) {
-        const long pos = orow * a.top_n + r;
-        const int val = found ? bi : -1;
-        if (a.idx64) reinterpret_cast<int64_t*>(a.indices)[pos] = val;
-        else reinterpret_cast<int32_t*>(a.indices)[pos] = val;
-      }
-    }
-  }
-}
-
-// ------------------------------------------------------------------------------------------------
-// sliding window attention
-
-template <typename T, int DK, int DV, int NG, int CH>
-__global__ void __launch_bounds__(256)
-swa_kernel(const SwaArgs a) {
-  constexpr int KLD = DK + 8, VLD = CH + 8, ROWS = 64 * NG;
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  T* ldsK = reinterpret_cast<T*>(smem_raw);
-  T* ldsV = ldsK + CH * KLD;
-
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int n = lane & 15, g = lane >> 4;
-  const int G = a.hq / a.hkv, Gp = next_pow2(G), lgp = ilog2(Gp);
-  const int TQ = ROWS >> lgp;
-  const SeqTile st = find_tile(a.cu_seq, a.batch, TQ, blockIdx.x);
-  if (!st.valid) return;
-  const int h = blockIdx.y;
+  const T* kb = reinterpret_cast<const T*>(a.k) + (long)koff * a.k_row_stride + (long)h * a.k_head_stride;
+  const T* vtb = reinterpret_cast<const T*>(a.vt) + (long)h * DV * a.vt_cols + vtoff;
   const int W = a.window;
-  const int t_last = min(st.t0 + TQ, st.len) - 1;
-  const T* qb = reinterpret_cast<const T*>(a.q);
-  const T* kb = reinterpret_cast<const T*>(a.k) + ((long)st.start * a.hkv + h) * DK;
-  const T* vtb = reinterpret_cast<const T*>(a.vt) + (long)h * DV * a.vt_cols + transposed_offset(st.start, st.b);
+
+  auto last_visible = [&](int t) -> int {      // largest key index token t may attend
+    if (!CMP) return t;
+    if (!a.causal) return nkeys - 1;
+    return t >= a.block ? min((t - a.block) / a.stride, nkeys - 1) : -1;
+  };
 
   RowGroup<T, DK, DV> grp[NG];
   RowMap rm[NG];
-  int g_lo[NG], g_hi[NG];   // key range any column of the group may see (wave uniform)
+  int hi[NG], lo[NG];            // per lane: visible keys are lo..hi
+  int g_hi_max[NG], g_hi_min[NG], g_lo_min[NG], g_lo_max[NG];   // wave uniform bounds over the group
+  float li[NG];
 #pragma unroll
   for (int j = 0; j < NG; ++j) {
     const int gi = wave * NG + j;
     rm[j] = map_row(st.t0, gi, n, lgp, G, st.len);
-    load_q(grp[j], qb, (long)st.start, rm[j], st.len, a.hq, h, G, g);
+    load_q(grp[j], reinterpret_cast<const T*>(a.q), (long)st.start, rm[j], st.len, a.hq, h, G, g);
     group_reset(grp[j]);
+    li[j] = 0.f;
+    hi[j] = last_visible(rm[j].tok);
+    lo[j] = CMP ? 0 : rm[j].tok - W + 1;
     const int tf = st.t0 + ((gi * 16) >> lgp);
     const int tl = min(st.t0 + ((gi * 16 + 15) >> lgp), st.len - 1);
-    g_lo[j] = max(tf - W + 1, 0);
-    g_hi[j] = tl;   // < tf when the whole group lies past the sequence end
+    g_hi_min[j] = last_visible(tf);
+    g_hi_max[j] = last_visible(tl);          // below g_hi_min when the group lies past the sequence end
+    g_lo_min[j] = CMP ? 0 : tf - W + 1;
+    g_lo_max[j] = CMP ? 0 : tl - W + 1;
   }
   const float c_attn = a.scale * kLog2e;
-  const int k_lo = max(st.t0 - W + 1, 0);
+  const int attn_end = last_visible(t_last);                      // last key any row of the tile attends
+  const int c_begin = CMP ? 0 : (max(st.t0 - W + 1, 0) / CH) * CH;
+  const int c_end = CMP ? nkeys : t_last + 1;
 
-  for (int c0 = (k_lo / CH) * CH; c0 <= t_last; c0 += CH) {
-    __syncthreads();
-    stage_rows(ldsK, KLD, kb, (long)a.hkv * DK, c0, st.len - 1, CH, DK);
-    stage_rows(ldsV, VLD, vtb + c0, (long)a.vt_cols, 0, DV - 1, DV, CH);
-    __syncthreads();
+  vec8_t<T> kr[KPT], vr[VPT];
+  auto gload = [&](int c0, bool with_v) {
+#pragma unroll
+    for (int i = 0; i < KPT; ++i) {
+      const int p = tid + i * NT;
+      if (KPIECES % NT == 0 || p < KPIECES) {
+        const int r = p / (DK / 8), pc = p % (DK / 8);
+        const int sr = min(c0 + r, nkeys - 1);
+        kr[i] = load8(kb + (long)sr * a.k_row_stride + pc * 8);
+      }
+    }
+    if (with_v) {
+#pragma unroll
+      for (int i = 0; i < VPT; ++i) {
+        const int p = tid + i * NT;
+        if (VPIECES % NT == 0 || p < VPIECES) {
+          const int r = p / (CH / 8), pc = p % (CH / 8);
+          vr[i] = load8(vtb + (long)r * a.vt_cols + c0 + pc * 8);
+        }
+      }
+    }
+  };
+  auto lstore = [&](int buf, bool with_v) {
+    T* dk = ldsK + buf * CH * KLD;
+#pragma unroll
+    for (int i = 0; i < KPT; ++i) {
+      const int p = tid + i * NT;
+      if (KPIECES % NT == 0 || p < KPIECES) store8(dk + (p / (DK / 8)) * KLD + (p % (DK / 8)) * 8, kr[i]);
+    }
+    if (with_v) {
+      T* dv = ldsV + buf * DV * VLD;
+#pragma unroll
+      for (int i = 0; i < VPT; ++i) {
+        const int p = tid + i * NT;
+        if (VPIECES % NT == 0 || p < VPIECES) store8(dv + (p / (CH / 8)) * VLD + (p % (CH / 8)) * 8, vr[i]);
+      }
+    }
+  };
+
+  if (c_begin < c_end) {
+    const bool v0 = c_begin <= attn_end;
+    gload(c_begin, v0);
+    lstore(0, v0);
+  }
+  __syncthreads();
+  int buf = 0;
+  for (int c0 = c_begin; c0 < c_end; c0 += CH) {
+    const int cn = c0 + CH;
+    const bool has_next = cn < c_end;
+    const bool next_v = has_next && cn <= attn_end;
+    if (has_next) gload(cn, next_v);
+
+    const T* bk = ldsK + buf * CH * KLD;
+    const T* bv = ldsV + buf * DV * VLD;
 #pragma unroll
     for (int sub = 0; sub < CH / 32; ++sub) {
       const int cb = c0 + 32 * sub;
+      if (cb >= c_end) break;
       bool act[NG];
-      bool any = false;
+      bool any_act = false;
 #pragma unroll
       for (int j = 0; j < NG; ++j) {
-        act[j] = (cb <= g_hi[j]) && (cb + 31 >= g_lo[j]);
-        any |= act[j];
+        act[j] = cb <= g_hi_max[j] && (CMP || cb + 31 >= g_lo_min[j]);
+        any_act |= act[j];
       }
-      if (!any) continue;
+      if (!CMP && !any_act) continue;
       f32x4_t s0[NG], s1[NG];
-      const T* ks = ldsK + 32 * sub * KLD + 8 * g;
+      const T* ks = bk + 32 * sub * KLD + 8 * g;
       scores32<T, DK, DV, NG>(ks + chunk_key_of_row(0, n) * KLD, ks + chunk_key_of_row(1, n) * KLD, grp, s0, s1);
       vec8_t<T> pb[NG];
 #pragma unroll
       for (int j = 0; j < NG; ++j) {
-        if (act[j]) {
-          float s[8], p[8];
+        float s[8], p[8];
 #pragma unroll
-          for (int i = 0; i < 4; ++i) { s[i] = s0[j][i]; s[4 + i] = s1[j][i]; }
+        for (int i = 0; i < 4; ++i) { s[i] = s0[j][i]; s[4 + i] = s1[j][i]; }
+        const int key0 = cb + 8 * g;
+        const bool full = cb + 31 <= g_hi_min[j] && (CMP || cb >= g_lo_max[j]);
+        if (CMP) {
+          if (cb + 32 > nkeys) {
 #pragma unroll
-          for (int i = 0; i < 8; ++i) {
-            const int key = cb + 8 * g + i;
-            if (!(key <= rm[j].tok && key > rm[j].tok - W)) s[i] = kNegInf;
+            for (int i = 0; i < 8; ++i)
+              if (key0 + i >= nkeys) s[i] = kNegInf;
           }
-          softmax_update(grp[j], s, c_attn, p);
-          pb[j] = pack8<T>(p);
+          float mx = s[0];
+#pragma unroll
+          for (int i = 1; i < 8; ++i) mx = fmaxf(mx, s[i]);
+          mx = colgroup_max(mx);                       // finite: key cb exists
+          const float m_new = fmaxf(grp[j].m, mx);
+          if (__any(m_new > grp[j].m)) {
+            const float d = grp[j].m - m_new;          // -inf on the first chunk
+            li[j] *= fast_exp2(d * kLog2e);
+            const float alpha = fast_exp2(d * c_attn);
+            grp[j].l *= alpha;
+#pragma unroll
+            for (int t = 0; t < DV / 16; ++t) {
+              grp[j].o[t][0] *= alpha; grp[j].o[t][1] *= alpha; grp[j].o[t][2] *= alpha; grp[j].o[t][3] *= alpha;
+            }
+            grp[j].m = m_new;
+          }
+          const float m = grp[j].m;
+          float sum = 0.f;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) sum += fast_exp2(fmaf(s[i], kLog2e, -m * kLog2e));
+          li[j] += sum;
+          if (act[j]) {
+            sum = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+              float x = fast_exp2(fmaf(s[i], c_attn, -m * c_attn));
+              if (!full) x = (key0 + i <= hi[j]) ? x : 0.f;
+              p[i] = x;
+              sum += x;
+            }
+            grp[j].l += sum;
+            pb[j] = pack8<T>(p);
+          } else {
+            pb[j] = zero8<T>();
+          }
         } else {
-          pb[j] = zero8<T>();
+          if (act[j]) {
+            if (!full) {
+#pragma unroll
+              for (int i = 0; i < 8; ++i)
+                if (!(key0 + i <= hi[j] && key0 + i >= lo[j])) s[i] = kNegInf;
+            }
+            softmax_update(grp[j], s, c_attn, p);
+            pb[j] = pack8<T>(p);
+          } else {
+            pb[j] = zero8<T>();
+          }
         }
       }
-      pv32<T, DK, DV, NG>(ldsV + n * VLD + 32 * sub + 8 * g, 16 * VLD, grp, pb, act);
+      if (any_act) pv32<T, DK, DV, NG>(bv + n * VLD + 32 * sub + 8 * g, 16 * VLD, grp, pb, act);
     }
+
+    if (has_next) lstore(buf ^ 1, next_v);
+    __syncthreads();
+    buf ^= 1;
   }
 
   T* ob = reinterpret_cast<T*>(a.o);
@@ -424,8 +241,12 @@ swa_kernel(const SwaArgs a) {
   for (int j = 0; j < NG; ++j) {
     const float lt = colgroup_sum(grp[j].l);
     const float inv = lt > 0.f ? 1.0f / lt : 0.f;
-    if (rm[j].valid)
-      store_rows<T, DV>(ob + (((long)st.start + rm[j].tok) * a.hq + h * G + rm[j].gidx) * DV, grp[j].o, inv, g);
+    const long row = ((long)st.start + rm[j].tok) * a.hq + h * G + rm[j].gidx;
+    if (rm[j].valid) store_rows<T, DV>(ob + row * DV, grp[j].o, inv, g);
+    if (CMP && a.lse != nullptr) {
+      const float lit = colgroup_sum(li[j]);
+      if (rm[j].valid && g == 0) a.lse[row] = nkeys > 0 ? grp[j].m + __logf(lit) : 0.f;
+    }
   }
 }
 
@@ -528,13 +349,14 @@ slc_combine_kernel(const SlcArgs a) {
 // ------------------------------------------------------------------------------------------------
 // launchers
 
-template <typename T> struct Tile {
-  // groups per wave and keys per LDS chunk
+template <typename T> struct StreamTile {
+  // row groups per wavefront, keys per LDS chunk, wavefronts per workgroup
   static constexpr int NG = sizeof(T) == 2 ? 2 : 1;
   static constexpr int CH = sizeof(T) == 2 ? 64 : 32;
+  static constexpr int NW = 8;
 };
 
-static int set_smem(const void* fn, size_t bytes) {
+int set_smem(const void* fn, size_t bytes) {
   if (bytes > 160 * 1024) return -3;
   if (bytes > 48 * 1024) {
     if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess) return -4;
@@ -542,39 +364,38 @@ static int set_smem(const void* fn, size_t bytes) {
   return 0;
 }
 
-static int group_pow2(int G) {
+int group_pow2(int G) {
   int p = 1;
   while (p < G) p <<= 1;
   return p;
 }
 
-template <typename T, int DK, int DV>
-static int launch_cmp_t(const CmpArgs& a, hipStream_t st) {
-  constexpr int NG = Tile<T>::NG, CH = Tile<T>::CH;
+template <typename T, int DK, int DV, bool CMP>
+static int launch_stream_t(const StreamParams& a, int total, hipStream_t st) {
+  constexpr int NG = StreamTile<T>::NG, CH = StreamTile<T>::CH, NW = StreamTile<T>::NW;
   const int Gp = group_pow2(a.hq / a.hkv);
-  const int TQ = 64 * NG / Gp;
-  const size_t smem = (size_t)CH * (DK + 8) * sizeof(T) + (size_t)DV * (CH + 8) * sizeof(T) +
-                      (size_t)TQ * a.max_ns * sizeof(float);
-  auto fn = cmp_select_kernel<T, DK, DV, NG, CH>;
+  const int TQ = NW * NG * 16 / Gp;
+  const size_t smem = 2 * ((size_t)CH * (DK + 8) + (size_t)DV * (CH + 8)) * sizeof(T);
+  auto fn = stream_attn_kernel<T, DK, DV, NG, CH, NW, CMP>;
   const int rc = set_smem(reinterpret_cast<const void*>(fn), smem);
   if (rc) return rc;
-  const int tiles = a.total / TQ + a.batch;
-  hipLaunchKernelGGL(fn, dim3(tiles, a.hkv), dim3(256), smem, st, a);
+  const int tiles = total / TQ + a.batch;
+  hipLaunchKernelGGL(fn, dim3(tiles, a.hkv), dim3(NW * 64), smem, st, a);
   return 0;
 }
 
 template <typename T, int DK, int DV>
+static int launch_cmp_t(const CmpArgs& a, hipStream_t st) {
+  StreamParams p{a.q, a.ck, a.cvt, a.o, a.lse, a.cu_seq, a.cu_cmp, a.batch, a.hq, a.hkv, a.ck_row_stride,
+                 a.ck_head_stride, a.cvt_cols, a.block, a.stride, 0, a.causal, a.scale};
+  return launch_stream_t<T, DK, DV, true>(p, a.total, st);
+}
+
+template <typename T, int DK, int DV>
 static int launch_swa_t(const SwaArgs& a, hipStream_t st) {
-  constexpr int NG = Tile<T>::NG, CH = Tile<T>::CH;
-  const int Gp = group_pow2(a.hq / a.hkv);
-  const int TQ = 64 * NG / Gp;
-  const size_t smem = (size_t)CH * (DK + 8) * sizeof(T) + (size_t)DV * (CH + 8) * sizeof(T);
-  auto fn = swa_kernel<T, DK, DV, NG, CH>;
-  const int rc = set_smem(reinterpret_cast<const void*>(fn), smem);
-  if (rc) return rc;
-  const int tiles = a.total / TQ + a.batch;
-  hipLaunchKernelGGL(fn, dim3(tiles, a.hkv), dim3(256), smem, st, a);
-  return 0;
+  StreamParams p{a.q, a.k, a.vt, a.o, nullptr, a.cu_seq, a.cu_seq, a.batch, a.hq, a.hkv, (long)a.hkv * DK,
+                 (long)DK, a.vt_cols, 0, 0, a.window, 1, a.scale};
+  return launch_stream_t<T, DK, DV, false>(p, a.total, st);
 }
 
 template <typename T, int DK, int DV>
@@ -608,7 +429,7 @@ static int launch_slc_t(const SlcArgs& a, hipStream_t st) {
     }                                                                                 \
   } while (0)
 
-int launch_cmp_select(const CmpArgs& a, hipStream_t st) { NSA_DISPATCH(launch_cmp_t, a, st); }
+int launch_cmp_attn(const CmpArgs& a, hipStream_t st) { NSA_DISPATCH(launch_cmp_t, a, st); }
 int launch_swa(const SwaArgs& a, hipStream_t st) { NSA_DISPATCH(launch_swa_t, a, st); }
 int launch_slc_combine(const SlcArgs& a, hipStream_t st) { NSA_DISPATCH(launch_slc_t, a, st); }
 

@@ -77,32 +77,69 @@ int nsa_transpose_fwd(const void* x, void* out, const int32_t* cu, int batch, in
   return finish(nsa::launch_transpose(a, stream), "transpose");
 }
 
+static int cmp_common(const char* what, int stages, const void* q, const void* ck, const void* cvt, void* o,
+                      void* indices, float* pooled, float* lse, const int32_t* cu_seqlens, const int32_t* cu_cmp,
+                      int batch, int total, int hq, int hkv, int dk, int dv, int64_t ck_row_stride,
+                      int64_t ck_head_stride, int cvt_cols, int block, int stride, int pool_kernel, int pool_stride,
+                      int pool_pad, int top_n, int max_ns, int pooled_stride, float scale, int causal, int idx64,
+                      int dtype, nsa_stream_t stream) {
+  const bool attn = stages & 1, select = stages & 2;
+  if (!q || !ck || !cu_seqlens || !cu_cmp) return fail(NSA_ERR_INVALID, "%s: null pointer", what);
+  if (attn && (!cvt || !o)) return fail(NSA_ERR_INVALID, "%s: null pointer", what);
+  if (batch <= 0 || total <= 0 || block <= 0 || stride <= 0) return fail(NSA_ERR_INVALID, "%s: sizes must be positive", what);
+  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "%s: bad dtype", what);
+  if (int rc = check_heads(what, hq, hkv, dk, dv)) return rc;
+  if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "%s: scale must be positive", what);
+  if (ck_row_stride % 8 != 0 || ck_head_stride % 8 != 0 || (attn && cvt_cols % 64 != 0))
+    return fail(NSA_ERR_INVALID, "%s: ck strides must be multiples of 8, cvt_cols of 64", what);
+  if (!aligned16(q) || !aligned16(ck) || (attn && (!aligned16(cvt) || !aligned16(o))))
+    return fail(NSA_ERR_INVALID, "%s: pointers must be 16-byte aligned", what);
+  if (select) {
+    if (!indices || !lse) return fail(NSA_ERR_INVALID, "%s: the selection needs indices and the lse buffer", what);
+    if (pool_kernel <= 0 || pool_stride <= 0 || pool_pad < 0 || pool_pad >= pool_kernel || top_n <= 0 || max_ns < 0)
+      return fail(NSA_ERR_INVALID, "%s: bad pooling / top-n parameters", what);
+    if (pooled && pooled_stride < max_ns) return fail(NSA_ERR_INVALID, "%s: pooled_stride < max_ns", what);
+  } else {
+    max_ns = 0;
+  }
+  nsa::CmpArgs a{q, ck, cvt, o, indices, pooled, lse, cu_seqlens, cu_cmp, batch, total, hq, hkv, dk, dv,
+                 (long)ck_row_stride, (long)ck_head_stride, cvt_cols, block, stride, pool_kernel, pool_stride,
+                 pool_pad, top_n, max_ns, pooled_stride, scale, idx64, dtype, causal};
+  int rc = 0;
+  if (attn) rc = nsa::launch_cmp_attn(a, stream);
+  if (rc == 0 && select) rc = nsa::launch_select(a, stream);
+  return finish(rc, what);
+}
+
 int nsa_cmp_attn_select_fwd(const void* q, const void* ck, const void* cvt, void* o, void* indices,
-                            float* pooled, const int32_t* cu_seqlens, const int32_t* cu_cmp, int batch,
+                            float* pooled, float* lse, const int32_t* cu_seqlens, const int32_t* cu_cmp, int batch,
                             int total, int hq, int hkv, int dk, int dv, int64_t ck_row_stride,
                             int64_t ck_head_stride, int cvt_cols, int block, int stride, int pool_kernel,
                             int pool_stride, int pool_pad, int top_n, int max_ns, int pooled_stride,
                             float scale, int causal, int idx64, int dtype, nsa_stream_t stream) {
-  if (!q || !ck || !cvt || !o || !cu_seqlens || !cu_cmp) return fail(NSA_ERR_INVALID, "cmp_attn_select: null pointer");
-  if (batch <= 0 || total <= 0 || block <= 0 || stride <= 0) return fail(NSA_ERR_INVALID, "cmp_attn_select: sizes must be positive");
-  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "cmp_attn_select: bad dtype");
-  if (int rc = check_heads("cmp_attn_select", hq, hkv, dk, dv)) return rc;
-  if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "cmp_attn_select: scale must be positive");
-  if (ck_row_stride % 8 != 0 || ck_head_stride % 8 != 0 || cvt_cols % 64 != 0)
-    return fail(NSA_ERR_INVALID, "cmp_attn_select: ck strides must be multiples of 8, cvt_cols of 64");
-  if (!aligned16(q) || !aligned16(ck) || !aligned16(cvt) || !aligned16(o))
-    return fail(NSA_ERR_INVALID, "cmp_attn_select: pointers must be 16-byte aligned");
-  if (indices) {
-    if (pool_kernel <= 0 || pool_stride <= 0 || pool_pad < 0 || pool_pad >= pool_kernel || top_n <= 0 || max_ns < 0)
-      return fail(NSA_ERR_INVALID, "cmp_attn_select: bad pooling / top-n parameters");
-    if (pooled && pooled_stride < max_ns) return fail(NSA_ERR_INVALID, "cmp_attn_select: pooled_stride < max_ns");
-  } else {
-    max_ns = 0;
-  }
-  nsa::CmpArgs a{q, ck, cvt, o, indices, pooled, cu_seqlens, cu_cmp, batch, total, hq, hkv, dk, dv,
-                 (long)ck_row_stride, (long)ck_head_stride, cvt_cols, block, stride, pool_kernel, pool_stride,
-                 pool_pad, top_n, max_ns, pooled_stride, scale, idx64, dtype, causal};
-  return finish(nsa::launch_cmp_select(a, stream), "cmp_attn_select");
+  return cmp_common("cmp_attn_select", indices ? 3 : 1, q, ck, cvt, o, indices, pooled, lse, cu_seqlens, cu_cmp,
+                    batch, total, hq, hkv, dk, dv, ck_row_stride, ck_head_stride, cvt_cols, block, stride,
+                    pool_kernel, pool_stride, pool_pad, top_n, max_ns, pooled_stride, scale, causal, idx64, dtype,
+                    stream);
+}
+
+int nsa_cmp_attn_fwd(const void* q, const void* ck, const void* cvt, void* o, float* lse,
+                     const int32_t* cu_seqlens, const int32_t* cu_cmp, int batch, int total, int hq, int hkv,
+                     int dk, int dv, int64_t ck_row_stride, int64_t ck_head_stride, int cvt_cols, int block,
+                     int stride, float scale, int causal, int dtype, nsa_stream_t stream) {
+  return cmp_common("cmp_attn", 1, q, ck, cvt, o, nullptr, nullptr, lse, cu_seqlens, cu_cmp, batch, total, hq, hkv,
+                    dk, dv, ck_row_stride, ck_head_stride, cvt_cols, block, stride, 1, 1, 0, 1, 0, 0, scale, causal,
+                    0, dtype, stream);
+}
+
+int nsa_block_select_fwd(const void* q, const void* ck, const float* lse, void* indices, float* pooled,
+                         const int32_t* cu_seqlens, const int32_t* cu_cmp, int batch, int total, int hq, int hkv,
+                         int dk, int64_t ck_row_stride, int64_t ck_head_stride, int pool_kernel, int pool_stride,
+                         int pool_pad, int top_n, int max_ns, int pooled_stride, int idx64, int dtype,
+                         nsa_stream_t stream) {
+  return cmp_common("block_select", 2, q, ck, nullptr, nullptr, indices, pooled, const_cast<float*>(lse), cu_seqlens,
+                    cu_cmp, batch, total, hq, hkv, dk, 16, ck_row_stride, ck_head_stride, 0, 1, 1, pool_kernel,
+                    pool_stride, pool_pad, top_n, max_ns, pooled_stride, 1.0f, 1, idx64, dtype, stream);
 }
 
 int nsa_swa_fwd(const void* q, const void* k, const void* vt, void* o, const int32_t* cu_seqlens, int batch,

@@ -84,16 +84,31 @@ __device__ __forceinline__ int chunk_key_of_row(int tile, int m) {
   return 8 * (m >> 2) + (m & 3) + 4 * tile;
 }
 
-// Butterfly over the four lanes that share one tile column (lane%16).
+// All-reduce over the four lanes that share one tile column (lane%16): lanes n, n+16, n+32, n+48.
+// v_permlane16_swap exchanges the odd 16-lane rows of one operand with the even rows of the other,
+// v_permlane32_swap the upper half of one with the lower half of the other; fed the same value
+// twice they return the two partners of every lane, so each step is one VALU swap plus one op.
 __device__ __forceinline__ float colgroup_max(float x) {
-  x = fmaxf(x, __shfl_xor(x, 16));
-  x = fmaxf(x, __shfl_xor(x, 32));
-  return x;
+  unsigned u = __float_as_uint(x);
+  auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  x = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+  u = __float_as_uint(x);
+  r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
 }
 __device__ __forceinline__ float colgroup_sum(float x) {
-  x += __shfl_xor(x, 16);
-  x += __shfl_xor(x, 32);
-  return x;
+  unsigned u = __float_as_uint(x);
+  auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  x = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+  u = __float_as_uint(x);
+  r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+// Sum over the lane pairs (n, n+16) and (n+32, n+48) only.
+__device__ __forceinline__ float colpair_sum(float x) {
+  const unsigned u = __float_as_uint(x);
+  const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
 // Column offset of sequence b inside a key-contiguous ("transposed") buffer: every sequence starts
@@ -144,30 +159,41 @@ __device__ __forceinline__ void group_reset(RowGroup<T, DK, DV>& g) {
   g.l = 0.f;
 }
 
+// Raise the running maximum of a group to cover `mx` (already reduced over the column's four
+// lanes).  The accumulator and denominator are rescaled only when some lane's maximum grew, which
+// after the first few chunks is rare.  c = scale * log2(e).
+template <typename T, int DK, int DV>
+__device__ __forceinline__ void raise_max(RowGroup<T, DK, DV>& g, float mx, float c) {
+  const float m_new = fmaxf(g.m, mx);
+  if (__any(m_new > g.m)) {
+    const float mref = (m_new == kNegInf) ? 0.f : m_new;
+    const float alpha = fast_exp2((g.m - mref) * c);
+    g.l *= alpha;
+#pragma unroll
+    for (int i = 0; i < DV / 16; ++i) {
+      g.o[i][0] *= alpha; g.o[i][1] *= alpha; g.o[i][2] *= alpha; g.o[i][3] *= alpha;
+    }
+    g.m = m_new;
+  }
+}
+
 // Online-softmax update for the 8 scores a lane holds of one 32-key chunk (masked entries are
-// -inf).  Returns the probabilities in p (unnormalised) and rescales the accumulator.
+// -inf).  Returns the unnormalised probabilities in p.
 template <typename T, int DK, int DV>
 __device__ __forceinline__ void softmax_update(RowGroup<T, DK, DV>& g, const float (&s)[8], float c,
                                                float (&p)[8]) {
   float mx = s[0];
 #pragma unroll
   for (int i = 1; i < 8; ++i) mx = fmaxf(mx, s[i]);
-  mx = colgroup_max(mx);
-  const float m_new = fmaxf(g.m, mx);
-  const float mref = (m_new == kNegInf) ? 0.f : m_new;
-  const float alpha = fast_exp2((g.m - mref) * c);
+  raise_max(g, colgroup_max(mx), c);
+  const float off = (g.m == kNegInf) ? 0.f : -g.m * c;
   float sum = 0.f;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    p[i] = fast_exp2((s[i] - mref) * c);
+    p[i] = fast_exp2(fmaf(s[i], c, off));
     sum += p[i];
   }
-  g.l = g.l * alpha + sum;
-  g.m = m_new;
-#pragma unroll
-  for (int i = 0; i < DV / 16; ++i) {
-    g.o[i][0] *= alpha; g.o[i][1] *= alpha; g.o[i][2] *= alpha; g.o[i][3] *= alpha;
-  }
+  g.l += sum;
 }
 
 }  // namespace nsa

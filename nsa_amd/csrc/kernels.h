@@ -17,7 +17,7 @@ struct TransposeArgs {
 };
 
 struct CmpArgs {
-  const void* q; const void* ck; const void* cvt; void* o; void* indices; float* pooled;
+  const void* q; const void* ck; const void* cvt; void* o; void* indices; float* pooled; float* lse;
   const int32_t* cu_seq; const int32_t* cu_cmp;
   int batch, total, hq, hkv, dk, dv;
   long ck_row_stride, ck_head_stride; int cvt_cols;
@@ -40,7 +40,8 @@ struct SlcArgs {
 
 int launch_compress(const CompressArgs& a, hipStream_t st);
 int launch_transpose(const TransposeArgs& a, hipStream_t st);
-int launch_cmp_select(const CmpArgs& a, hipStream_t st);
+int launch_cmp_attn(const CmpArgs& a, hipStream_t st);
+int launch_select(const CmpArgs& a, hipStream_t st);
 int launch_swa(const SwaArgs& a, hipStream_t st);
 int launch_slc_combine(const SlcArgs& a, hipStream_t st);
 

@@ -107,10 +107,12 @@ class NSAAttention(nn.Module):
         max_nc = nc if nc is not None else conv_compressed_len(seq_len, self.compression_stride,
                                                                self.compression_block)
         cvt, vt = stage("transpose", lambda: (ops.transpose(cv, cu_cmp, batch), ops.transpose(v, cu, batch)))
-        o_cmp, idx, _ = stage("cmp_select", lambda: ops.cmp_attn_select(
+        o_cmp, lse = stage("cmp_attn", lambda: ops.cmp_attn(
             q, ck, cvt, cu, cu_cmp, batch, hkv, dv, ck.stride(0), ck.stride(1), self.compression_block,
-            self.compression_stride, self.pool_kernel_size, self.pool_stride, self.pool_padding,
-            self.selected_block_count, max_nc, scale, causal=bool(causal), select=True, idx64=False))
+            self.compression_stride, scale, causal=bool(causal)))
+        idx, _ = stage("block_select", lambda: ops.block_select(
+            q, ck, lse, cu, cu_cmp, batch, hkv, ck.stride(0), ck.stride(1), self.pool_kernel_size,
+            self.pool_stride, self.pool_padding, self.selected_block_count, max_nc, idx64=False))
         if gates is None:
             gates = self.gating(q)                       # [total, Hq, 3]
         g = gates.reshape(total * hq, 3)

@@ -122,18 +122,53 @@ def cmp_attn_select(q, ck, cvt, cu_seqlens, cu_cmp, batch, hkv, dv, ck_row_strid
     o = torch.empty(total, hq, dv, dtype=q.dtype, device=q.device)
     max_ns = pool_bins(max_nc, pool_kernel, pool_stride, pool_pad) if select else 0
     idx = pooled = None
+    lse = torch.empty(total, hq, dtype=torch.float32, device=q.device)
     if select:
         idx = torch.empty(total, hkv, top_n, dtype=torch.int64 if idx64 else torch.int32, device=q.device)
         if want_pooled:
             pooled = torch.zeros(total, hkv, max(max_ns, 1), dtype=torch.float32, device=q.device)
     lib = _lib.load()
     rc = lib.nsa_cmp_attn_select_fwd(
-        _ptr(q), _ptr(ck), _ptr(cvt), _ptr(o), _ptr(idx), _ptr(pooled), _ptr(cu_seqlens), _ptr(cu_cmp), batch,
+        _ptr(q), _ptr(ck), _ptr(cvt), _ptr(o), _ptr(idx), _ptr(pooled), _ptr(lse), _ptr(cu_seqlens), _ptr(cu_cmp),
+        batch,
         total, hq, hkv, dk, dv, ck_row_stride, ck_head_stride, cvt.shape[-1], block, stride, pool_kernel,
         pool_stride, pool_pad, max(top_n, 1), max_ns, max(max_ns, 1), float(scale), int(bool(causal)),
         int(idx64), _dtype_code(q), _stream())
     _lib.check(rc, "nsa_cmp_attn_select_fwd")
     return o, idx, pooled
+
+
+def cmp_attn(q, ck, cvt, cu_seqlens, cu_cmp, batch, hkv, dv, ck_row_stride, ck_head_stride, block, stride, scale,
+             causal=True):
+    """Compressed attention only.  Returns (o [total,Hq,dv], lse float32 [total,Hq])."""
+    _need_cuda(q, ck, cvt, cu_seqlens, cu_cmp)
+    q = _dense(q)
+    total, hq, dk = q.shape
+    o = torch.empty(total, hq, dv, dtype=q.dtype, device=q.device)
+    lse = torch.empty(total, hq, dtype=torch.float32, device=q.device)
+    rc = _lib.load().nsa_cmp_attn_fwd(_ptr(q), _ptr(ck), _ptr(cvt), _ptr(o), _ptr(lse), _ptr(cu_seqlens),
+                                      _ptr(cu_cmp), batch, total, hq, hkv, dk, dv, ck_row_stride, ck_head_stride,
+                                      cvt.shape[-1], block, stride, float(scale), int(bool(causal)),
+                                      _dtype_code(q), _stream())
+    _lib.check(rc, "nsa_cmp_attn_fwd")
+    return o, lse
+
+
+def block_select(q, ck, lse, cu_seqlens, cu_cmp, batch, hkv, ck_row_stride, ck_head_stride, pool_kernel,
+                 pool_stride, pool_pad, top_n, max_nc, idx64=True, want_pooled=False):
+    """Block importance + top-n from the lse that cmp_attn wrote.  Returns (indices, pooled or None)."""
+    _need_cuda(q, ck, lse, cu_seqlens, cu_cmp)
+    q = _dense(q)
+    total, hq, dk = q.shape
+    max_ns = pool_bins(max_nc, pool_kernel, pool_stride, pool_pad)
+    idx = torch.empty(total, hkv, top_n, dtype=torch.int64 if idx64 else torch.int32, device=q.device)
+    pooled = torch.zeros(total, hkv, max(max_ns, 1), dtype=torch.float32, device=q.device) if want_pooled else None
+    rc = _lib.load().nsa_block_select_fwd(_ptr(q), _ptr(ck), _ptr(lse), _ptr(idx), _ptr(pooled), _ptr(cu_seqlens),
+                                          _ptr(cu_cmp), batch, total, hq, hkv, dk, ck_row_stride, ck_head_stride,
+                                          pool_kernel, pool_stride, pool_pad, top_n, max_ns, max(max_ns, 1),
+                                          int(idx64), _dtype_code(q), _stream())
+    _lib.check(rc, "nsa_block_select_fwd")
+    return idx, pooled
 
 
 def swa(q, k, vt, cu_seqlens, batch, window, scale):
