@@ -31,7 +31,7 @@ struct StreamParams {
 };
 
 template <typename T, int DK, int DV, int NG, int CH, int NW, bool CMP>
-__global__ void __launch_bounds__(NW * 64)
+__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 stream_attn_kernel(const StreamParams a) {
   constexpr int KLD = DK + 8, VLD = CH + 8, ROWS = NW * NG * 16, NT = NW * 64;
   constexpr int KPIECES = CH * DK / 8, VPIECES = DV * CH / 8;
@@ -40,7 +40,8 @@ stream_attn_kernel(const StreamParams a) {
   T* ldsK = reinterpret_cast<T*>(smem_raw);          // [2][CH][KLD]
   T* ldsV = ldsK + 2 * CH * KLD;                     // [2][DV][VLD]
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: group bounds stay in SGPRs
   const int n = lane & 15, g = lane >> 4;
   const int G = a.hq / a.hkv, Gp = next_pow2(G), lgp = ilog2(Gp);
   const int TQ = ROWS >> lgp;
@@ -135,6 +136,7 @@ stream_attn_kernel(const StreamParams a) {
     }
   };
 
+  wait_all_loads();
   if (c_begin < c_end) {
     const bool v0 = c_begin <= attn_end;
     gload(c_begin, v0);
@@ -174,7 +176,8 @@ stream_attn_kernel(const StreamParams a) {
         const int key0 = cb + 8 * g;
         const bool full = cb + 31 <= g_hi_min[j] && (CMP || cb >= g_lo_max[j]);
         if (CMP) {
-          if (cb + 32 > nkeys) {
+          if (cb + 32 > nkeys) {                       // last chunk of the sequence only
+            asm volatile("" ::: "memory");
 #pragma unroll
             for (int i = 0; i < 8; ++i)
               if (key0 + i >= nkeys) s[i] = kNegInf;
@@ -196,19 +199,25 @@ stream_attn_kernel(const StreamParams a) {
             grp[j].m = m_new;
           }
           const float m = grp[j].m;
+          const float off_i = -m * kLog2e, off_a = -m * c_attn;
           float sum = 0.f;
 #pragma unroll
-          for (int i = 0; i < 8; ++i) sum += fast_exp2(fmaf(s[i], kLog2e, -m * kLog2e));
+          for (int i = 0; i < 8; ++i) sum += fast_exp2(fmaf(s[i], kLog2e, off_i));
           li[j] += sum;
           if (act[j]) {
             sum = 0.f;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-              float x = fast_exp2(fmaf(s[i], c_attn, -m * c_attn));
-              if (!full) x = (key0 + i <= hi[j]) ? x : 0.f;
-              p[i] = x;
-              sum += x;
+              p[i] = fast_exp2(fmaf(s[i], c_attn, off_a));
             }
+            if (!full) {                               // the one or two chunks on the causal edge
+              asm volatile("" ::: "memory");
+#pragma unroll
+              for (int i = 0; i < 8; ++i)
+                if (key0 + i > hi[j]) p[i] = 0.f;
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) sum += p[i];
             grp[j].l += sum;
             pb[j] = pack8<T>(p);
           } else {
@@ -216,7 +225,8 @@ stream_attn_kernel(const StreamParams a) {
           }
         } else {
           if (act[j]) {
-            if (!full) {
+            if (!full) {                               // window edges
+              asm volatile("" ::: "memory");
 #pragma unroll
               for (int i = 0; i < 8; ++i)
                 if (!(key0 + i <= hi[j] && key0 + i >= lo[j])) s[i] = kNegInf;
@@ -228,7 +238,11 @@ stream_attn_kernel(const StreamParams a) {
           }
         }
       }
-      if (any_act) pv32<T, DK, DV, NG>(bv + n * VLD + 32 * sub + 8 * g, 16 * VLD, grp, pb, act);
+      bool all_act = true;
+#pragma unroll
+      for (int j = 0; j < NG; ++j) all_act &= act[j];
+      if (all_act) pv32_all<T, DK, DV, NG>(bv + n * VLD + 32 * sub + 8 * g, 16 * VLD, grp, pb);
+      else if (any_act) pv32<T, DK, DV, NG>(bv + n * VLD + 32 * sub + 8 * g, 16 * VLD, grp, pb, act);
     }
 
     if (has_next) lstore(buf ^ 1, next_v);
@@ -257,21 +271,42 @@ __device__ __forceinline__ float gate_value(float x, int act) {
   return act == 1 ? 1.0f / (1.0f + __expf(-x)) : x;
 }
 
+// One wavefront per row group.  The usable blocks of a token are walked as a flat sequence of
+// 32-key chunks; the K fragments (two tiles) and V^T fragments of chunk i+1 are requested from
+// global memory before chunk i is multiplied, so a wavefront keeps one full chunk (K and V) in
+// flight while it computes.  Workgroups are dealt to kv heads so that, with the hardware's
+// round-robin placement of workgroups on the 8 XCDs, an XCD's L2 only ever holds one head's K/V.
 template <typename T, int DK, int DV>
 __global__ void __launch_bounds__(256)
 slc_combine_kernel(const SlcArgs a) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  constexpr int NK = DK / 32, NV = DV / 16;
+  constexpr bool PIPE = sizeof(T) == 2;       // fp32 fragments are twice as wide: no second buffer
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n = lane & 15, g = lane >> 4;
   const int G = a.hq / a.hkv, Gp = next_pow2(G), lgp = ilog2(Gp);
   const int TQ = 64 >> lgp;
-  const SeqTile st = find_tile(a.cu_seq, a.batch, TQ, blockIdx.x);
+  int h, tile;
+  {
+    const int id = blockIdx.x, hkv = a.hkv;
+    if (8 % hkv == 0) {
+      const int per = 8 / hkv, x = id & 7;
+      h = x % hkv;
+      tile = (id >> 3) * per + x / hkv;
+    } else {
+      h = id % hkv;
+      tile = id / hkv;
+    }
+  }
+  const SeqTile st = find_tile(a.cu_seq, a.batch, TQ, tile);
   if (!st.valid) return;
-  const int h = blockIdx.y;
   const int S = a.top_n, BS = a.block_size;
   const T* qb = reinterpret_cast<const T*>(a.q);
-  const T* kb = reinterpret_cast<const T*>(a.k) + ((long)st.start * a.hkv + h) * DK;
-  const T* vtb = reinterpret_cast<const T*>(a.vt) + (long)h * DV * a.vt_cols + transposed_offset(st.start, st.b);
+  const T* kb = reinterpret_cast<const T*>(a.k) + ((long)st.start * a.hkv + h) * DK + 8 * g;
+  const T* vtb = reinterpret_cast<const T*>(a.vt) + (long)h * DV * a.vt_cols + transposed_offset(st.start, st.b)
+                 + (long)n * a.vt_cols + 8 * g;
   const long krow = (long)a.hkv * DK;
+  const long vstep = 16L * a.vt_cols;
 
   RowGroup<T, DK, DV> grp[1];
   const RowMap rm = map_row(st.t0, wave, n, lgp, G, st.len);
@@ -280,6 +315,10 @@ slc_combine_kernel(const SlcArgs a) {
   const float c_attn = a.scale * kLog2e;
   const int tpg = lgp >= 4 ? 1 : (16 >> lgp);          // tokens per row group
   const int tfirst = st.t0 + ((wave * 16) >> lgp);
+  const int key_r0 = chunk_key_of_row(0, n), key_r1 = chunk_key_of_row(1, n);
+
+  struct Frags { vec8_t<T> k0[NK], k1[NK], v[NV]; };
+  wait_all_loads();
 
   for (int tk = 0; tk < tpg; ++tk) {
     const int tt = tfirst + tk;
@@ -288,34 +327,77 @@ slc_combine_kernel(const SlcArgs a) {
     int cnt = S;
     if (a.counts != nullptr) cnt = min(max(a.counts[irow], 0), S);
     long myidx = -1;
-    if (lane < S) {
+    if (lane < cnt) {
       myidx = a.idx64 ? reinterpret_cast<const int64_t*>(a.indices)[irow * S + lane]
                       : (long)reinterpret_cast<const int32_t*>(a.indices)[irow * S + lane];
     }
-    for (int i = 0; i < cnt; ++i) {
-      const long bi = __shfl(myidx, i);
-      if (bi < 0 || bi > tt) continue;                   // also keeps bi * BS inside int range
-      if (bi * BS > tt) continue;
-      const int k0 = (int)bi * BS;
-      const int k1 = min(k0 + BS - 1, tt);               // last key of the block this token may see
-      for (int cb = k0; cb <= k1; cb += 32) {
-        f32x4_t s0[1], s1[1];
-        const int r0 = min(cb + chunk_key_of_row(0, n), st.len - 1);
-        const int r1 = min(cb + chunk_key_of_row(1, n), st.len - 1);
-        scores32<T, DK, DV, 1>(kb + r0 * krow + 8 * g, kb + r1 * krow + 8 * g, grp, s0, s1);
-        float s[8], p[8];
+    const bool usable = myidx >= 0 && myidx <= tt && myidx * BS <= tt;   // bi <= tt keeps bi*BS in range
+    unsigned long long todo = __ballot(usable);
+    int cur = 0, cur_last = -1;                          // next chunk start / last visible key of the block
+    auto next_chunk = [&](int& cb, int& last) -> bool {
+      if (cur > cur_last) {
+        if (todo == 0) return false;
+        const int i = __ffsll((long long)todo) - 1;
+        todo &= todo - 1;
+        const int k0 = (int)__shfl(myidx, i) * BS;
+        cur = k0;
+        cur_last = min(k0 + BS - 1, tt);
+      }
+      cb = cur;
+      last = cur_last;
+      cur += 32;
+      return true;
+    };
+    auto issue = [&](Frags& f, int cb) {
+      const T* p0 = kb + (long)min(cb + key_r0, st.len - 1) * krow;
+      const T* p1 = kb + (long)min(cb + key_r1, st.len - 1) * krow;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) { s[e] = s0[0][e]; s[4 + e] = s1[0][e]; }
+      for (int kk = 0; kk < NK; ++kk) { f.k0[kk] = load8(p0 + 32 * kk); f.k1[kk] = load8(p1 + 32 * kk); }
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const int key = cb + 8 * g + e;
-          if (!(key <= k1 && rm.tok == tt)) s[e] = kNegInf;
-        }
-        softmax_update(grp[0], s, c_attn, p);
-        vec8_t<T> pb[1];
-        pb[0] = pack8<T>(p);
-        const bool act[1] = {true};
-        pv32<T, DK, DV, 1>(vtb + (long)n * a.vt_cols + cb + 8 * g, 16L * a.vt_cols, grp, pb, act);
+      for (int t = 0; t < NV; ++t) f.v[t] = load8(vtb + t * vstep + cb);
+    };
+    auto compute = [&](const Frags& f, int cb, int last) {
+      f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kk = 0; kk < NK; ++kk) {
+        s0 = mma16(f.k0[kk], grp[0].q[kk], s0);
+        s1 = mma16(f.k1[kk], grp[0].q[kk], s1);
+      }
+      float s[8], p[8];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { s[e] = s0[e]; s[4 + e] = s1[e]; }
+      if (cb + 31 > last || tpg > 1) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (!(cb + 8 * g + e <= last && rm.tok == tt)) s[e] = kNegInf;
+      }
+      softmax_update(grp[0], s, c_attn, p);
+      const vec8_t<T> pb = pack8<T>(p);
+#pragma unroll
+      for (int t = 0; t < NV; ++t) grp[0].o[t] = mma16(f.v[t], pb, grp[0].o[t]);
+    };
+
+    Frags fa;
+    int cba, lasta;
+    bool ha = next_chunk(cba, lasta);
+    if (ha) issue(fa, cba);
+    if (PIPE) {
+      Frags fb;
+      int cbb, lastb;
+      while (ha) {
+        const bool hb = next_chunk(cbb, lastb);
+        if (hb) issue(fb, cbb);
+        compute(fa, cba, lasta);
+        if (!hb) break;
+        ha = next_chunk(cba, lasta);
+        if (ha) issue(fa, cba);
+        compute(fb, cbb, lastb);
+      }
+    } else {
+      while (ha) {
+        compute(fa, cba, lasta);
+        ha = next_chunk(cba, lasta);
+        if (ha) issue(fa, cba);
       }
     }
   }
@@ -352,8 +434,8 @@ slc_combine_kernel(const SlcArgs a) {
 template <typename T> struct StreamTile {
   // row groups per wavefront, keys per LDS chunk, wavefronts per workgroup
   static constexpr int NG = sizeof(T) == 2 ? 2 : 1;
-  static constexpr int CH = sizeof(T) == 2 ? 64 : 32;
-  static constexpr int NW = 8;
+  static constexpr int CH = 32;
+  static constexpr int NW = 4;
 };
 
 int set_smem(const void* fn, size_t bytes) {
@@ -402,8 +484,9 @@ template <typename T, int DK, int DV>
 static int launch_slc_t(const SlcArgs& a, hipStream_t st) {
   const int Gp = group_pow2(a.hq / a.hkv);
   const int TQ = 64 / Gp;
-  const int tiles = a.total / TQ + a.batch;
-  hipLaunchKernelGGL((slc_combine_kernel<T, DK, DV>), dim3(tiles, a.hkv), dim3(256), 0, st, a);
+  int tiles = a.total / TQ + a.batch;
+  if (8 % a.hkv == 0) tiles = (tiles + 8 / a.hkv - 1) / (8 / a.hkv) * (8 / a.hkv);   // whole rounds of 8 workgroups
+  hipLaunchKernelGGL((slc_combine_kernel<T, DK, DV>), dim3(tiles * a.hkv), dim3(256), 0, st, a);
   return 0;
 }
 

@@ -79,6 +79,11 @@ template <typename T> __device__ __forceinline__ vec8_t<T> pack8(const float (&p
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Wait for every outstanding memory operation of this wavefront.  Placed after the one-time loads
+// (query fragments, statistics) and before a streaming loop, it keeps the compiler from guarding
+// those registers with waits inside the loop, which would also wait for the loop's own prefetches.
+__device__ __forceinline__ void wait_all_loads() { __builtin_amdgcn_s_waitcnt(0); }
+
 // A-operand row m of tile `tile` (0/1) of a 32-key chunk -> key offset inside the chunk.
 __device__ __forceinline__ int chunk_key_of_row(int tile, int m) {
   return 8 * (m >> 2) + (m & 3) + 4 * tile;
@@ -109,6 +114,12 @@ __device__ __forceinline__ float colpair_sum(float x) {
   const unsigned u = __float_as_uint(x);
   const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+// Data-parallel-primitive move inside a 16-lane row: CTRL 0x00-0xFF = quad_perm, 0x100+n = row_shl:n
+// (lane i reads lane i+n), 0x110+n = row_shr:n; lanes whose source is outside the row read 0.
+template <int CTRL> __device__ __forceinline__ float dpp_f32(float x) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xF, 0xF, true));
 }
 
 // Column offset of sequence b inside a key-contiguous ("transposed") buffer: every sequence starts

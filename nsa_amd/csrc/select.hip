@@ -13,7 +13,9 @@
 
 namespace nsa {
 
-template <typename T, int DK, int NG, int CH, int NW>
+// FAST: GQA group of 16 (one token per row group) and the default pooling (5 columns every 4, no
+// padding); everything else takes the generic path with LDS atomics.
+template <typename T, int DK, int NG, int CH, int NW, bool FAST>
 __global__ void __launch_bounds__(NW * 64)
 importance_select_kernel(const CmpArgs a) {
   constexpr int KLD = DK + 8, ROWS = NW * NG * 16, NT = NW * 64;
@@ -23,9 +25,10 @@ importance_select_kernel(const CmpArgs a) {
   T* ldsK = reinterpret_cast<T*>(smem_raw);                       // [2][CH][KLD]
   float* bins = reinterpret_cast<float*>(ldsK + 2 * CH * KLD);    // [TQ][Ns]
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 15, g = lane >> 4;
-  const int G = a.hq / a.hkv, Gp = next_pow2(G), lgp = ilog2(Gp);
+  const int G = a.hq / a.hkv, Gp = FAST ? 16 : next_pow2(G), lgp = FAST ? 4 : ilog2(Gp);
   const int TQ = ROWS >> lgp;
   const SeqTile st = find_tile(a.cu_seq, a.batch, TQ, blockIdx.x);
   if (!st.valid) return;
@@ -41,7 +44,7 @@ importance_select_kernel(const CmpArgs a) {
   const T* ckb = reinterpret_cast<const T*>(a.ck) + (long)coff * a.ck_row_stride + (long)h * a.ck_head_stride;
 
   vec8_t<T> qf[NG][DK / 32];
-  float lse_r[NG][4];        // lse of rows 4g+i of each group; +inf removes padded rows
+  float lse_r[NG][4];        // lse * log2(e) of rows 4g+i of each group; +inf removes padded rows
 #pragma unroll
   for (int j = 0; j < NG; ++j) {
     const int gi = wave * NG + j;
@@ -54,11 +57,17 @@ importance_select_kernel(const CmpArgs a) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const RowMap r4 = map_row(st.t0, gi, 4 * g + i, lgp, G, st.len);
-      lse_r[j][i] = r4.valid ? a.lse[((long)st.start + r4.tok) * a.hq + h * G + r4.gidx] : __builtin_huge_valf();
+      lse_r[j][i] = r4.valid ? a.lse[((long)st.start + r4.tok) * a.hq + h * G + r4.gidx] * kLog2e
+                             : __builtin_huge_valf();
     }
   }
 
   for (int i = tid; i < TQ * Ns; i += NT) bins[i] = 0.f;
+  wait_all_loads();
+
+  float pend[NG];   // FAST: the unfinished last bin of the previous tile (lane 12 of the g == 0 row)
+#pragma unroll
+  for (int j = 0; j < NG; ++j) pend[j] = 0.f;
 
   vec8_t<T> kr[KPT];
   auto gload = [&](int c0) {
@@ -106,6 +115,34 @@ importance_select_kernel(const CmpArgs a) {
         for (int j = 0; j < NG; ++j) s[j] = mma16(qf[j][kk], kf, s[j]);   // rows = heads, columns = keys
       }
       const int c = cb + n;
+      if (FAST) {
+        // One token per row group, windows of 5 columns every 4: after the head sum every lane of
+        // tile column n holds R[c].  Quad sums and the first column of the next quad come from DPP.
+        // Bins 4t..4t+2 of tile t are complete at once; bin 4t+3 waits in a register of lane 12 for
+        // the first column of the next tile.  Every bin is written exactly once by the g == 0 row.
+#pragma unroll
+        for (int j = 0; j < NG; ++j) {
+          float e[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) e[i] = fast_exp2(fmaf(s[j][i], kLog2e, -lse_r[j][i]));
+          float v = colgroup_sum((e[0] + e[1]) + (e[2] + e[3]));
+          v = c < Nc ? v : 0.f;
+          const float t2 = v + dpp_f32<0xB1>(v);            // quad_perm [1,0,3,2]
+          const float quad = t2 + dpp_f32<0x4E>(t2);        // quad_perm [2,3,0,1]
+          const float nextf = dpp_f32<0x104>(v);            // row_shl:4 -> R[c+4], 0 past the tile
+          const float first = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+          if (g == 0 && (n & 3) == 0) {
+            float* row = bins + (wave * NG + j) * Ns;
+            const int b = (cb >> 2) + (n >> 2);
+            if (n == 12) {
+              if (cb > 0 && (cb >> 2) - 1 < Ns) row[(cb >> 2) - 1] = pend[j] + first;
+              pend[j] = quad;
+            } else if (b < Ns) {
+              row[b] = quad + nextf;
+            }
+          }
+        }
+      } else {
       // bins that contain column c: b*s - p <= c < b*s - p + k
       const int num = c + a.pool_p - a.pool_k + 1;
       const int b_lo = num <= 0 ? 0 : (num + a.pool_s - 1) / a.pool_s;
@@ -115,7 +152,7 @@ importance_select_kernel(const CmpArgs a) {
         const int gi = wave * NG + j;
         float e[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) e[i] = fast_exp2((s[j][i] - lse_r[j][i]) * kLog2e);
+        for (int i = 0; i < 4; ++i) e[i] = fast_exp2(fmaf(s[j][i], kLog2e, -lse_r[j][i]));
         if (lgp >= 2) {
           float v = (e[0] + e[1]) + (e[2] + e[3]);
           if (lgp == 3) v = colpair_sum(v);
@@ -133,10 +170,17 @@ importance_select_kernel(const CmpArgs a) {
           }
         }
       }
+      }
     }
     if (has_next) lstore(buf ^ 1);
     __syncthreads();
     buf ^= 1;
+  }
+  if (FAST && c_end > 0 && g == 0 && n == 12) {
+    const int b = ((((c_end - 1) >> 4) << 4) >> 2) + 3;     // last bin of the last tile: no next column
+#pragma unroll
+    for (int j = 0; j < NG; ++j)
+      if (b < Ns) bins[(wave * NG + j) * Ns + b] = pend[j];
   }
   __syncthreads();
 
@@ -188,7 +232,8 @@ static int launch_select_ng(const CmpArgs& a, hipStream_t st) {
   const int TQ = NW * NG * 16 / Gp;
   const size_t smem = 2 * (size_t)CH * (DK + 8) * sizeof(T) + (size_t)TQ * a.max_ns * sizeof(float);
   if (smem > 160 * 1024) return -3;
-  auto fn = importance_select_kernel<T, DK, NG, CH, NW>;
+  const bool fast = Gp == 16 && a.pool_k == 5 && a.pool_s == 4 && a.pool_p == 0;
+  auto fn = fast ? importance_select_kernel<T, DK, NG, CH, NW, true> : importance_select_kernel<T, DK, NG, CH, NW, false>;
   const int rc = set_smem(reinterpret_cast<const void*>(fn), smem);
   if (rc) return rc;
   const int tiles = a.total / TQ + a.batch;

@@ -44,6 +44,17 @@ __device__ __forceinline__ void pv32(const T* __restrict__ vp, long tile_stride,
   }
 }
 
+template <typename T, int DK, int DV, int NG>
+__device__ __forceinline__ void pv32_all(const T* __restrict__ vp, long tile_stride,
+                                         RowGroup<T, DK, DV> (&grp)[NG], const vec8_t<T> (&pb)[NG]) {
+#pragma unroll
+  for (int t = 0; t < DV / 16; ++t) {
+    const vec8_t<T> av = load8(vp + t * tile_stride);
+#pragma unroll
+    for (int j = 0; j < NG; ++j) grp[j].o[t] = mma16(av, pb[j], grp[j].o[t]);
+  }
+}
+
 struct RowMap {
   int tok;      // token of this lane's column (sequence local), may be >= len
   int gidx;     // head inside the GQA group, may be >= G
