@@ -90,6 +90,55 @@ def cpu_baseline(q, k, v, gl, top_n, window, budget_s=20.0):
                        % (done_rows, spent, t_comp))
 
 
+def decode_bench(steps, warmup):
+    """BASELINE config 5: batch 64, one query token per sequence, 32768 cached tokens each (+ the
+    compressed caches), Hq64/Hkv4, D128, top-16 blocks of 64, window 512, bf16."""
+    import torch
+    from nsa_amd.decode import NSADecodeCache, nsa_decode_step
+    dev = "cuda:0"
+    B, ctx, hq, hkv, d, top_n, window = 64, 32768, 64, 4, 128, 16, 512
+    g = torch.Generator(device=dev).manual_seed(4)
+    cache = NSADecodeCache(B, ctx, hkv, d, d, dtype=torch.bfloat16, device=dev)
+    for b0 in range(0, B, 8):                                  # fill in slices to bound the temporaries
+        k = (torch.randn(8, ctx, hkv, d, device=dev, generator=g) * 0.5).bfloat16()
+        v = (torch.randn(8, ctx, hkv, d, device=dev, generator=g) * 0.5).bfloat16()
+        sub = NSADecodeCache(8, ctx, hkv, d, d, dtype=torch.bfloat16, device=dev)
+        sub.fill(k, v)
+        cache.k[b0:b0 + 8], cache.vt[b0:b0 + 8] = sub.k, sub.vt
+        cache.ck[b0:b0 + 8], cache.cvt[b0:b0 + 8] = sub.ck, sub.cvt
+        del sub, k, v
+    cache.ctx_lens.fill_(ctx)
+    q = (torch.randn(B, hq, d, device=dev, generator=g) * 0.5).bfloat16()
+    gl = torch.randn(B, hq, 3, device=dev, generator=g).bfloat16()
+    run = lambda: nsa_decode_step(q, cache, gl, SEL_BLOCK, top_n, window, gate_activation="sigmoid",
+                                  return_indices=True)
+    for _ in range(warmup):
+        run()
+    torch.cuda.synchronize()
+    beg, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    beg.record()
+    for _ in range(steps):
+        out, idx = run()
+    end.record()
+    torch.cuda.synchronize()
+    us = beg.elapsed_time(end) / steps * 1e3
+    assert torch.isfinite(out).all()
+    # algorithmic bytes: all compressed keys, visible compressed values, distinct selected/window rows, q/o/gates
+    nc = (ctx - BLOCK) // STRIDE + 1
+    n_vis = min((ctx - 1 - BLOCK) // STRIDE + 1, nc)
+    t = ctx - 1
+    blk_lo = (t - window + 1) // SEL_BLOCK                      # blocks that the window fully or partly covers
+    idx = idx.long()
+    valid = (idx >= 0) & (idx * SEL_BLOCK <= t)
+    outside = valid & (idx < blk_lo)                           # rows not already counted with the window
+    rows = outside.sum().item() * SEL_BLOCK + B * hkv * (t + 1 - blk_lo * SEL_BLOCK)
+    nbytes = B * hkv * (nc * d * 2 + n_vis * d * 2) + rows * (d + d) * 2 + B * hq * (d + d + 3) * 2
+    return {"us_per_step": us, "batch": B, "context": ctx, "algorithmic_bytes": nbytes,
+            "achieved_GBps": nbytes / (us * 1e-6) / 1e9, "hbm_peak_GBps": PEAK_HBM_GBS,
+            "hbm_frac": nbytes / (us * 1e-6) / 1e9 / PEAK_HBM_GBS,
+            "workload": "decode_cfg5: batch 64 x 1 token, ctx 32768, Hq64/Hkv4, D128, top-16 x 64, window 512, bf16"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -98,6 +147,7 @@ def main():
     ap.add_argument("--workload", default="prefill_cfg4", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-budget", type=float, default=20.0)
+    ap.add_argument("--no-decode", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures the one-GPU NSA forward path; --gpus %d is not supported (this build has no "
@@ -174,6 +224,10 @@ def main():
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": dom_tflops, "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": dom_tflops / PEAK_BF16_TFLOPS, "traffic": None},
     }
+    if not args.no_decode:
+        del qd, kd, vd, gd, out, idx
+        torch.cuda.empty_cache()
+        res["decode"] = decode_bench(max(args.steps, 20), args.warmup)
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(q, k, v, gl, top_n, window, args.cpu_budget)
     print(json.dumps(res))

@@ -114,6 +114,29 @@ int nsa_slc_combine_fwd(const void* q, const void* k, const void* vt, const void
                         int vt_cols, int top_n, int block_size, float scale, int idx64, int gate_act,
                         int dtype, nsa_stream_t stream);
 
+/* One-token decode step (no counterpart in the reference, which has no cache and no single-token
+ * path; defined as the last row of the prefill forward on the same keys/values, mean-pool
+ * compressor).  Cache layout, all zero-initialised by the owner:
+ *   k_cache [batch][ctx_cap][hkv][dk]      v_cache_t [batch][hkv][dv][ctx_cap]      (ctx_cap % 64 == 0)
+ *   ck_cache [batch][nc_cap][hkv][dk]      cv_cache_t [batch][hkv][dv][nc_cap]      (nc_cap % 64 == 0)
+ * ctx_lens int32[batch]: tokens in each cache including the current one; q [batch][hq][dk] is the
+ * query of that token; gates [batch][hq][3] (selected, sliding, compressed) or NULL (all ones);
+ * out [batch][hq][dv]; indices (optional) int32 [batch][hkv][top_n] receives the selected blocks.
+ * nc_cap <= nsa_decode_max_compressed(). */
+int nsa_decode_max_compressed(void);
+int nsa_decode_step(const void* q, const void* k_cache, const void* v_cache_t, const void* ck_cache,
+                    const void* cv_cache_t, const int32_t* ctx_lens, const void* gates, void* out, int32_t* indices,
+                    int batch, int hq, int hkv, int dk, int dv, int ctx_cap, int nc_cap, int block, int stride,
+                    int sel_block, int pool_kernel, int pool_stride, int pool_pad, int top_n, int window, float scale,
+                    int gate_act, int dtype, nsa_stream_t stream);
+
+/* Appends one token per sequence: k_new [batch][hkv][dk] -> row pos[b] of k_cache, v_new
+ * [batch][hkv][dv] -> column pos[b] of v_cache_t, and, when pos[b]+1 completes a compression block,
+ * the mean of the last `block` tokens as the next row / column of the compressed caches. */
+int nsa_decode_append(const void* k_new, const void* v_new, void* k_cache, void* v_cache_t, void* ck_cache,
+                      void* cv_cache_t, const int32_t* pos, int batch, int hkv, int dk, int dv, int ctx_cap, int nc_cap,
+                      int block, int stride, int dtype, nsa_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -38,11 +38,24 @@ struct SlcArgs {
   int idx64, gate_act, dtype;
 };
 
+struct DecodeArgs {
+  const void* q; const void* k_cache; const void* v_cache_t; const void* ck_cache; const void* cv_cache_t;
+  const int32_t* ctx_lens; const void* gates; void* out; int32_t* indices;
+  int batch, hq, hkv, dk, dv, ctx_cap, nc_cap;
+  int block, stride, sel_block, pool_k, pool_s, pool_p, top_n, window;
+  float scale; int gate_act, dtype;
+};
+
 int launch_compress(const CompressArgs& a, hipStream_t st);
 int launch_transpose(const TransposeArgs& a, hipStream_t st);
 int launch_cmp_attn(const CmpArgs& a, hipStream_t st);
 int launch_select(const CmpArgs& a, hipStream_t st);
 int launch_swa(const SwaArgs& a, hipStream_t st);
 int launch_slc_combine(const SlcArgs& a, hipStream_t st);
+int launch_decode(const DecodeArgs& a, hipStream_t st);
+int launch_decode_append(const void* k_new, const void* v_new, void* k_cache, void* v_cache_t, void* ck_cache,
+                         void* cv_cache_t, const int32_t* pos, int batch, int hkv, int dk, int dv, int ctx_cap,
+                         int nc_cap, int block, int stride, int dtype, hipStream_t st);
+int decode_max_nc();
 
 }  // namespace nsa

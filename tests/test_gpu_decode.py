@@ -1,0 +1,122 @@
+"""GPU parity of the decode step and the cache append, through the C ABI, against the CPU oracle
+(decode == last row of the prefill forward on the cached tokens)."""
+import math
+
+import pytest
+import torch
+
+from oracle import nsa_oracle as O
+from tests.util import TOL, max_abs, randn
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _make(B, T, Hq, Hkv, Dk, Dv, seed, dtype, scale=0.5):
+    q = randn(B, Hq, Dk, seed=seed, scale=scale, dtype=dtype)
+    k = randn(B, T, Hkv, Dk, seed=seed + 1, scale=scale, dtype=dtype)
+    v = randn(B, T, Hkv, Dv, seed=seed + 2, scale=scale, dtype=dtype)
+    gl = randn(B, Hq, 3, seed=seed + 3, dtype=dtype)
+    return q, k, v, gl
+
+
+def _check(dtype, ctxs, Hq, Hkv, Dk, Dv, S, W, seed, which=None):
+    from nsa_amd.decode import NSADecodeCache, nsa_decode_step
+    B, T = len(ctxs), max(ctxs)
+    q, k, v, gl = _make(B, T, Hq, Hkv, Dk, Dv, seed, dtype)
+    cache = NSADecodeCache(B, T, Hkv, Dk, Dv, dtype=dtype, device=DEV)
+    cache.fill(k.to(DEV), v.to(DEV))
+    cache.ctx_lens.copy_(torch.tensor(ctxs, dtype=torch.int32))
+    out, idx = nsa_decode_step(q.to(DEV), cache, gl.to(DEV), 64, S, W, gate_activation="sigmoid", return_indices=True)
+    out, idx = out.cpu(), idx.cpu().long()
+    p = O.NSAParams(32, 16, 64, S, W)
+    gates = torch.sigmoid(gl.float()).to(dtype)
+    worst, stats = 0.0, [0, 0, 0, 0]
+    for b in (range(B) if which is None else which):
+        c = ctxs[b]
+        ref, parts = O.nsa_decode_step(q[b], k[b, :c], v[b, :c], gates[b], p, return_parts=True)
+        same = torch.equal(idx[b].sort(-1).values, parts["idx"].sort(-1).values)
+        if "pooled" in parts:
+            r = O.compare_selection(idx[b][None], parts["idx"][None], parts["pooled"][None], 1e-3)
+            stats = [x + y for x, y in zip(stats, r)]
+            assert r[3] == 0
+        else:
+            assert (idx[b] == -1).all()
+        if same:                      # outputs are comparable only under the same picks
+            worst = max(worst, max_abs(out[b], ref))
+    print("decode", dtype, ctxs[:6], (Hq, Hkv, Dk, Dv, S, W), "max_abs", worst, "rows/exact/excused/fail", stats)
+    assert torch.isfinite(out).all()
+    assert worst <= TOL[dtype]
+    assert stats[1] >= 0.9 * stats[0]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_decode_small_ragged_contexts(dtype):
+    _check(dtype, [1024, 1000, 513, 64, 40, 33, 20, 1], 64, 4, 128, 128, 4, 128, seed=100)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_decode_gqa4_d64(dtype):
+    _check(dtype, [1024, 777], 4, 1, 64, 64, 4, 128, seed=110)
+
+
+def test_decode_dqk192():
+    _check(torch.bfloat16, [2048, 1536], 32, 2, 192, 128, 16, 512, seed=120)
+
+
+def test_decode_cfg5_context_subset():
+    """BASELINE config 5 shape per sequence (ctx 32768, Hq64/Hkv4, D128, top-16, window 512), batch 4."""
+    _check(torch.bfloat16, [32768, 32768, 32767, 32000], 64, 4, 128, 128, 16, 512, seed=130)
+
+
+def test_decode_equals_last_prefill_row_on_gpu():
+    from nsa_amd.decode import NSADecodeCache, nsa_decode_step
+    from nsa_amd.nsa import NSAAttention
+    T, Hq, Hkv, D, S, W = 2048, 64, 4, 128, 16, 512
+    dtype = torch.bfloat16
+    q = randn(T, Hq, D, seed=140, scale=0.5, dtype=dtype)
+    k = randn(T, Hkv, D, seed=141, scale=0.5, dtype=dtype)
+    v = randn(T, Hkv, D, seed=142, scale=0.5, dtype=dtype)
+    gl = randn(T, Hq, 3, seed=143, dtype=dtype)
+    m = NSAAttention(D, True, selected_block_count=S, sliding_window=W, dtype=dtype, compressor_mode="mean",
+                     gate_activation="sigmoid").to(DEV)
+    cu = torch.tensor([0, T], dtype=torch.int32, device=DEV)
+    full, idx_full = m(q.to(DEV), k.to(DEV), v.to(DEV), cu, 0, gates=gl.to(DEV), return_indices=True)
+    cache = NSADecodeCache(1, T, Hkv, D, D, dtype=dtype, device=DEV)
+    cache.fill(k[None].to(DEV), v[None].to(DEV))
+    out, idx = nsa_decode_step(q[-1:].to(DEV), cache, gl[-1:].to(DEV), 64, S, W, gate_activation="sigmoid",
+                               return_indices=True)
+    assert torch.equal(idx[0].sort(-1).values.cpu(), idx_full[-1].sort(-1).values.cpu().int())
+    err = max_abs(out[0], full[-1])
+    print("decode vs prefill last row max_abs", err)
+    assert err <= 2e-2
+
+
+def test_cache_append_matches_bulk_fill():
+    from nsa_amd.decode import NSADecodeCache, nsa_decode_step
+    B, T0, steps, Hkv, Dk, Dv = 3, 100, 45, 2, 64, 64
+    dtype = torch.bfloat16
+    k = randn(B, T0 + steps, Hkv, Dk, seed=150, dtype=dtype).to(DEV)
+    v = randn(B, T0 + steps, Hkv, Dv, seed=151, dtype=dtype).to(DEV)
+    inc = NSADecodeCache(B, T0 + steps, Hkv, Dk, Dv, dtype=dtype, device=DEV)
+    inc.fill(k[:, :T0], v[:, :T0])
+    for s in range(steps):
+        inc.append(k[:, T0 + s], v[:, T0 + s])
+    ref = NSADecodeCache(B, T0 + steps, Hkv, Dk, Dv, dtype=dtype, device=DEV)
+    ref.fill(k, v)
+    assert torch.equal(inc.ctx_lens, ref.ctx_lens)
+    assert torch.equal(inc.k, ref.k) and torch.equal(inc.vt, ref.vt)
+    assert max_abs(inc.ck, ref.ck) <= 4e-3 and max_abs(inc.cvt, ref.cvt) <= 4e-3
+    # and the caches are usable: a decode step on both gives the same result
+    q = randn(B, 8, Dk, seed=152, dtype=dtype).to(DEV)
+    a = nsa_decode_step(q, inc, None, 64, 2, 32)
+    b = nsa_decode_step(q, ref, None, 64, 2, 32)
+    assert max_abs(a, b) <= 2e-2
+
+
+def test_decode_rejects_long_caches():
+    from nsa_amd.decode import NSADecodeCache, nsa_decode_step
+    cache = NSADecodeCache(1, 65536, 1, 64, 64, dtype=torch.bfloat16, device=DEV)
+    q = torch.zeros(1, 4, 64, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(NotImplementedError):
+        nsa_decode_step(q, cache)
