@@ -106,13 +106,20 @@ int nsa_swa_fwd(const void* q, const void* k, const void* vt, void* o, const int
  *   token t is used iff i < counts[t,h] (counts NULL -> top_n), 0 <= idx and idx*block_size <= t.
  *   out = act(g_slc)*o_slc + act(g_swa)*o_swa + act(g_cmp)*o_cmp, where o_swa / o_cmp
  *   [total,hq,dv] may be NULL (term dropped), a NULL gate means 1, and gate (t,hq) is read at
- *   g[(t*hq + hq_idx)*gate_stride].  A token with no usable block has o_slc = 0. */
+ *   g[(t*hq + hq_idx)*gate_stride].  A token with no usable block has o_slc = 0.
+ *   workspace (optional, nsa_slc_workspace_bytes) switches to the block-major schedule: every K/V
+ *   block is loaded once and the queries that picked it are gathered, instead of gathering the
+ *   blocks per token; results agree to rounding.  NULL keeps the token-major kernel. */
 int nsa_slc_combine_fwd(const void* q, const void* k, const void* vt, const void* indices,
                         const int32_t* counts, const void* g_slc, const void* g_swa, const void* g_cmp,
                         int64_t gate_stride, const void* o_swa, const void* o_cmp, void* out,
                         const int32_t* cu_seqlens, int batch, int total, int hq, int hkv, int dk, int dv,
                         int vt_cols, int top_n, int block_size, float scale, int idx64, int gate_act,
-                        int dtype, nsa_stream_t stream);
+                        int dtype, void* workspace, int64_t workspace_bytes, nsa_stream_t stream);
+
+/* Bytes of the optional workspace of nsa_slc_combine_fwd; 0 when the shape has no block-major path
+ * (bf16, selection blocks of 64 keys only). */
+int64_t nsa_slc_workspace_bytes(int total, int batch, int hkv, int dk, int dv, int top_n, int block_size, int dtype);
 
 /* One-token decode step (no counterpart in the reference, which has no cache and no single-token
  * path; defined as the last row of the prefill forward on the same keys/values, mean-pool

@@ -514,6 +514,11 @@ static int launch_slc_t(const SlcArgs& a, hipStream_t st) {
 
 int launch_cmp_attn(const CmpArgs& a, hipStream_t st) { NSA_DISPATCH(launch_cmp_t, a, st); }
 int launch_swa(const SwaArgs& a, hipStream_t st) { NSA_DISPATCH(launch_swa_t, a, st); }
-int launch_slc_combine(const SlcArgs& a, hipStream_t st) { NSA_DISPATCH(launch_slc_t, a, st); }
+int launch_slc_combine(const SlcArgs& a, hipStream_t st) {
+  // block-major path when the caller lent a large enough workspace and the shape qualifies
+  if (a.workspace != nullptr && slc_block_major_ok(a) && a.workspace_bytes >= slc_workspace_bytes(a))
+    return launch_slc_block_major(a, a.workspace, st);
+  NSA_DISPATCH(launch_slc_t, a, st);
+}
 
 }  // namespace nsa

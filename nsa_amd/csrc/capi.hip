@@ -156,11 +156,20 @@ int nsa_swa_fwd(const void* q, const void* k, const void* vt, void* o, const int
   return finish(nsa::launch_swa(a, stream), "swa");
 }
 
+int64_t nsa_slc_workspace_bytes(int total, int batch, int hkv, int dk, int dv, int top_n, int block_size, int dtype) {
+  nsa::SlcArgs a{};
+  a.total = total; a.batch = batch; a.hkv = hkv; a.dk = dk; a.dv = dv; a.top_n = top_n; a.block_size = block_size;
+  a.dtype = dtype;
+  if (total <= 0 || batch <= 0 || hkv <= 0 || top_n <= 0 || !nsa::slc_block_major_ok(a)) return 0;
+  return nsa::slc_workspace_bytes(a);
+}
+
 int nsa_slc_combine_fwd(const void* q, const void* k, const void* vt, const void* indices, const int32_t* counts,
                         const void* g_slc, const void* g_swa, const void* g_cmp, int64_t gate_stride,
                         const void* o_swa, const void* o_cmp, void* out, const int32_t* cu_seqlens, int batch,
                         int total, int hq, int hkv, int dk, int dv, int vt_cols, int top_n, int block_size,
-                        float scale, int idx64, int gate_act, int dtype, nsa_stream_t stream) {
+                        float scale, int idx64, int gate_act, int dtype, void* workspace, int64_t workspace_bytes,
+                        nsa_stream_t stream) {
   if (!q || !k || !vt || !indices || !out || !cu_seqlens) return fail(NSA_ERR_INVALID, "slc_combine: null pointer");
   if (batch <= 0 || total <= 0) return fail(NSA_ERR_INVALID, "slc_combine: sizes must be positive");
   if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "slc_combine: bad dtype");
@@ -172,7 +181,9 @@ int nsa_slc_combine_fwd(const void* q, const void* k, const void* vt, const void
   if (gate_act != NSA_GATE_IDENTITY && gate_act != NSA_GATE_SIGMOID) return fail(NSA_ERR_INVALID, "slc_combine: bad gate activation");
   if (!aligned16(q) || !aligned16(k) || !aligned16(vt)) return fail(NSA_ERR_INVALID, "slc_combine: pointers must be 16-byte aligned");
   nsa::SlcArgs a{q, k, vt, indices, counts, g_slc, g_swa, g_cmp, (long)gate_stride, o_swa, o_cmp, out, cu_seqlens,
-                 batch, total, hq, hkv, dk, dv, vt_cols, top_n, block_size, scale, idx64, gate_act, dtype};
+                 batch, total, hq, hkv, dk, dv, vt_cols, top_n, block_size, scale, idx64, gate_act, dtype,
+                 workspace, (long)workspace_bytes};
+  if (workspace && !aligned16(workspace)) return fail(NSA_ERR_INVALID, "slc_combine: workspace must be 16-byte aligned");
   return finish(nsa::launch_slc_combine(a, stream), "slc_combine");
 }
 

@@ -36,6 +36,7 @@ struct SlcArgs {
   const void* o_swa; const void* o_cmp; void* out; const int32_t* cu_seq;
   int batch, total, hq, hkv, dk, dv, vt_cols, top_n, block_size; float scale;
   int idx64, gate_act, dtype;
+  void* workspace; long workspace_bytes;
 };
 
 struct DecodeArgs {
@@ -52,6 +53,9 @@ int launch_cmp_attn(const CmpArgs& a, hipStream_t st);
 int launch_select(const CmpArgs& a, hipStream_t st);
 int launch_swa(const SwaArgs& a, hipStream_t st);
 int launch_slc_combine(const SlcArgs& a, hipStream_t st);
+long slc_workspace_bytes(const SlcArgs& a);
+bool slc_block_major_ok(const SlcArgs& a);
+int launch_slc_block_major(const SlcArgs& a, void* workspace, hipStream_t st);
 int launch_decode(const DecodeArgs& a, hipStream_t st);
 int launch_decode_append(const void* k_new, const void* v_new, void* k_cache, void* v_cache_t, void* ck_cache,
                          void* cv_cache_t, const int32_t* pos, int batch, int hkv, int dk, int dv, int ctx_cap,

@@ -1,0 +1,367 @@
+// Block-major selected attention (bf16, selection blocks of 64 keys).
+//
+// The token-major kernel gathers every selected K/V block again for every token: 40 KB per
+// (token, kv head, block), 43 GB per forward at T = 32k, and a CU cannot pull more than ~15 B/clk
+// through its vector L1.  Here the loop is inverted: the (token, pick) pairs are bucketed by
+// (kv head, block); a wavefront loads one K/V block into registers as MFMA fragments ONCE and then
+// streams the queries that picked it (6 KB each), writing one normalised partial result
+// (o / l in bf16, plus max and denominator in fp32) per pair.  A second kernel merges the <= top_n
+// partials of every token, applies the gates and adds the other two branches.  Traffic per pair
+// drops from 40 KB to ~10 KB (query in, partial out) + 4 KB (partial back in).
+//
+// Workspace layout (caller allocated, nsa_slc_workspace_bytes): block bases per sequence, pair counts /
+// offsets / cursors per (head, block), work items (head, block, segment of 64 pairs), the bucketed
+// pair list, a slot map (token, head, pick) -> pair, and the partial results.
+#include "tiles.h"
+
+namespace nsa {
+
+constexpr int kSeg = 64;          // pairs of one block handled by one wavefront
+constexpr int kBlk = 64;          // keys per selection block (4 MFMA tiles)
+
+struct SlcWs {
+  int* blkbase; int* counts; int* offsets; int* cursor; int* items; int* n_items;
+  uint32_t* list; int* slotmap; float* ml; void* po;
+  int nb;          // bound on the number of 64-key blocks over all sequences
+  long pairs_cap;  // total * hkv * top_n
+  int items_cap;
+};
+
+__host__ __device__ inline long align_up(long x, long a) { return (x + a - 1) / a * a; }
+
+__host__ inline long carve(const SlcArgs& a, void* base, SlcWs* ws, size_t elem) {
+  const int nb = a.total / kBlk + a.batch;
+  const long pairs = (long)a.total * a.hkv * a.top_n;
+  const int items_cap = (int)(pairs / kSeg) + a.hkv * nb + 1;
+  long off = 0;
+  auto take = [&](long bytes) { const long o = off; off = align_up(off + bytes, 256); return o; };
+  const long o_blkbase = take((a.batch + 1) * 4L);
+  const long o_counts = take((long)a.hkv * nb * 4);
+  const long o_offsets = take((long)a.hkv * nb * 4);
+  const long o_cursor = take((long)a.hkv * nb * 4);
+  const long o_items = take((long)items_cap * 8);
+  const long o_nitems = take(4);
+  const long o_list = take(pairs * 4);
+  const long o_slot = take(pairs * 4);
+  const long o_ml = take(pairs * 2 * 16 * 4);
+  const long o_po = take(pairs * 16 * a.dv * (long)elem);
+  if (ws != nullptr) {
+    char* b = reinterpret_cast<char*>(base);
+    ws->blkbase = (int*)(b + o_blkbase); ws->counts = (int*)(b + o_counts); ws->offsets = (int*)(b + o_offsets);
+    ws->cursor = (int*)(b + o_cursor); ws->items = (int*)(b + o_items); ws->n_items = (int*)(b + o_nitems);
+    ws->list = (uint32_t*)(b + o_list); ws->slotmap = (int*)(b + o_slot); ws->ml = (float*)(b + o_ml);
+    ws->po = b + o_po;
+    ws->nb = nb; ws->pairs_cap = pairs; ws->items_cap = items_cap;
+  }
+  return off;
+}
+
+long slc_workspace_bytes(const SlcArgs& a) { return carve(a, nullptr, nullptr, a.dtype == 0 ? 2 : 4); }
+
+bool slc_block_major_ok(const SlcArgs& a) {
+  return a.dtype == 0 && a.block_size == kBlk && a.top_n <= 64 && a.total < (1 << 26) &&
+         (a.dk == 64 || a.dk == 128 || a.dk == 192) && (a.dv == 64 || a.dv == 128);
+}
+
+// ---- bucket the pairs ---------------------------------------------------------------------------
+
+__global__ void __launch_bounds__(256)
+slc_prep_kernel(const int32_t* __restrict__ cu, int batch, SlcWs ws, int hkv) {
+  if (threadIdx.x == 0) {
+    int acc = 0;
+    for (int b = 0; b < batch; ++b) {
+      ws.blkbase[b] = acc;
+      acc += (cu[b + 1] - cu[b] + kBlk - 1) / kBlk;
+    }
+    ws.blkbase[batch] = acc;
+    *ws.n_items = 0;
+  }
+  for (int i = threadIdx.x; i < hkv * ws.nb; i += 256) { ws.counts[i] = 0; ws.cursor[i] = 0; }
+}
+
+__device__ __forceinline__ int seq_of_token(const int32_t* __restrict__ cu, int batch, int t) {
+  int lo = 0, hi = batch;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (cu[mid] <= t) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+// FILL = false: count the pairs of every (head, block); FILL = true: place them.
+template <bool FILL>
+__global__ void __launch_bounds__(256)
+slc_bucket_kernel(const SlcArgs a, SlcWs ws) {
+  const long id = (long)blockIdx.x * 256 + threadIdx.x;          // (token, head, pick)
+  if (id >= (long)a.total * a.hkv * a.top_n) return;
+  const int i = (int)(id % a.top_n);
+  const long th = id / a.top_n;
+  const int h = (int)(th % a.hkv), tg = (int)(th / a.hkv);
+  const int b = seq_of_token(a.cu_seq, a.batch, tg);
+  const int t = tg - a.cu_seq[b];
+  int cnt = a.top_n;
+  if (a.counts != nullptr) cnt = min(max(a.counts[th], 0), a.top_n);
+  const long idx = a.idx64 ? reinterpret_cast<const int64_t*>(a.indices)[id]
+                           : (long)reinterpret_cast<const int32_t*>(a.indices)[id];
+  const bool ok = i < cnt && idx >= 0 && idx <= t && idx * kBlk <= t;
+  if (!ok) {
+    if (FILL) ws.slotmap[id] = -1;
+    return;
+  }
+  const int key = h * ws.nb + ws.blkbase[b] + (int)idx;
+  if (!FILL) {
+    atomicAdd(&ws.counts[key], 1);
+  } else {
+    const int p = ws.offsets[key] + atomicAdd(&ws.cursor[key], 1);
+    ws.list[p] = ((uint32_t)tg << 6) | (uint32_t)i;
+    ws.slotmap[id] = p;
+  }
+}
+
+// exclusive scan of the pair counts and the list of work items (one workgroup)
+__global__ void __launch_bounds__(1024)
+slc_scan_kernel(SlcWs ws, int hkv) {
+  __shared__ int s_cnt[1024], s_seg[1024];
+  __shared__ int carry_cnt, carry_seg;
+  if (threadIdx.x == 0) { carry_cnt = 0; carry_seg = 0; }
+  __syncthreads();
+  const int n = hkv * ws.nb;
+  for (int base = 0; base < n; base += 1024) {
+    const int i = base + threadIdx.x;
+    const int c = i < n ? ws.counts[i] : 0;
+    const int sg = (c + kSeg - 1) / kSeg;
+    s_cnt[threadIdx.x] = c;
+    s_seg[threadIdx.x] = sg;
+    __syncthreads();
+    for (int d = 1; d < 1024; d <<= 1) {          // Hillis-Steele inclusive scan
+      int vc = 0, vs = 0;
+      if ((int)threadIdx.x >= d) { vc = s_cnt[threadIdx.x - d]; vs = s_seg[threadIdx.x - d]; }
+      __syncthreads();
+      s_cnt[threadIdx.x] += vc;
+      s_seg[threadIdx.x] += vs;
+      __syncthreads();
+    }
+    const int ex_c = carry_cnt + s_cnt[threadIdx.x] - c;
+    const int ex_s = carry_seg + s_seg[threadIdx.x] - sg;
+    if (i < n) {
+      ws.offsets[i] = ex_c;
+      for (int k = 0; k < sg; ++k)
+        if (ex_s + k < ws.items_cap) { ws.items[2 * (ex_s + k)] = i; ws.items[2 * (ex_s + k) + 1] = k; }   // (head*nb + block, segment)
+    }
+    __syncthreads();
+    if (threadIdx.x == 1023) { carry_cnt += s_cnt[1023]; carry_seg += s_seg[1023]; }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) *ws.n_items = min(carry_seg, ws.items_cap);
+}
+
+// ---- one K/V block in registers, the queries that picked it streamed past ------------------------
+
+template <typename T, int DK, int DV>
+__global__ void __launch_bounds__(256)
+slc_block_kernel(const SlcArgs a, const SlcWs ws) {
+  constexpr int NK = DK / 32, NV = DV / 16, OLD = DV + 8;
+  __shared__ __attribute__((aligned(16))) T stage[4][16 * OLD];    // per wavefront: one partial, head-major
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int n = lane & 15, g = lane >> 4;
+  const int item_id = blockIdx.x * 4 + wave;
+  if (item_id >= *ws.n_items) return;
+  const int key = ws.items[2 * item_id], seg = ws.items[2 * item_id + 1];
+  const int h = key / ws.nb, gb = key % ws.nb;
+  const SeqTile st = find_tile(a.cu_seq, a.batch, kBlk, gb);      // st.t0 = first key of the block
+  if (!st.valid) return;
+  const int G = a.hq / a.hkv;
+  const int first = ws.offsets[key] + seg * kSeg;
+  const int count = min(ws.counts[key] - seg * kSeg, kSeg);
+  const float c_attn = a.scale * kLog2e;
+
+  // K block as A fragments: chunk c (32 keys) = tiles 2c, 2c+1 with permuted rows; V^T block per chunk
+  vec8_t<T> kf[4][NK], vf[2][NV];
+  {
+    const T* kb = reinterpret_cast<const T*>(a.k) + ((long)st.start * a.hkv + h) * DK + 8 * g;
+    const long krow = (long)a.hkv * DK;
+#pragma unroll
+    for (int tile = 0; tile < 4; ++tile) {
+      const int row = min(st.t0 + 32 * (tile >> 1) + chunk_key_of_row(tile & 1, n), st.len - 1);
+#pragma unroll
+      for (int kk = 0; kk < NK; ++kk) kf[tile][kk] = load8(kb + row * krow + 32 * kk);
+    }
+    const T* vtb = reinterpret_cast<const T*>(a.vt) + (long)h * DV * a.vt_cols + transposed_offset(st.start, st.b) +
+                   (long)n * a.vt_cols + st.t0 + 8 * g;
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int t = 0; t < NV; ++t) vf[c][t] = load8(vtb + t * 16L * a.vt_cols + 32 * c);
+  }
+
+  const T* qb = reinterpret_cast<const T*>(a.q);
+  T* pob = reinterpret_cast<T*>(ws.po);
+  const int gc = n < G ? n : G - 1;
+  vec8_t<T> qn[NK];
+  uint32_t ent = ws.list[first];
+  {
+    const T* qp = qb + ((long)(ent >> 6) * a.hq + h * G + gc) * DK + 8 * g;
+#pragma unroll
+    for (int kk = 0; kk < NK; ++kk) qn[kk] = load8(qp + 32 * kk);
+  }
+  for (int j = 0; j < count; ++j) {
+    vec8_t<T> qf[NK];
+#pragma unroll
+    for (int kk = 0; kk < NK; ++kk) qf[kk] = qn[kk];
+    const int tg = (int)(ent >> 6);
+    const int p = first + j;
+    if (j + 1 < count) {                                  // next query in flight while this one is multiplied
+      ent = ws.list[p + 1];
+      const T* qp = qb + ((long)(ent >> 6) * a.hq + h * G + gc) * DK + 8 * g;
+#pragma unroll
+      for (int kk = 0; kk < NK; ++kk) qn[kk] = load8(qp + 32 * kk);
+    }
+    const int t_loc = tg - st.start;                      // token position inside its sequence
+    float s[16];
+    {
+      f32x4_t acc[4];
+#pragma unroll
+      for (int tile = 0; tile < 4; ++tile) {
+        acc[tile] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < NK; ++kk) acc[tile] = mma16(kf[tile][kk], qf[kk], acc[tile]);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { s[i] = acc[0][i]; s[4 + i] = acc[1][i]; s[8 + i] = acc[2][i]; s[12 + i] = acc[3][i]; }
+    }
+    if (st.t0 + kBlk - 1 > t_loc) {                       // the block that contains the token itself
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        if (st.t0 + 32 * (i >> 3) + 8 * g + (i & 7) > t_loc) s[i] = kNegInf;
+    }
+    float mx = s[0];
+#pragma unroll
+    for (int i = 1; i < 16; ++i) mx = fmaxf(mx, s[i]);
+    mx = colgroup_max(mx);                                // finite: key t0 <= t_loc is visible
+    float pr[16], sum = 0.f;
+    const float off = -mx * c_attn;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) { pr[i] = fast_exp2(fmaf(s[i], c_attn, off)); sum += pr[i]; }
+    sum = colgroup_sum(sum);
+    float p0[8], p1[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { p0[i] = pr[i]; p1[i] = pr[8 + i]; }
+    const vec8_t<T> pb0 = pack8<T>(p0), pb1 = pack8<T>(p1);
+    const float inv = 1.0f / sum;
+    T* srow = &stage[wave][n * OLD + 4 * g];
+#pragma unroll
+    for (int t = 0; t < NV; ++t) {
+      f32x4_t o = {0.f, 0.f, 0.f, 0.f};
+      o = mma16(vf[0][t], pb0, o);
+      o = mma16(vf[1][t], pb1, o);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) srow[t * 16 + i] = (T)(o[i] * inv);
+    }
+    // head-major rows out of LDS: 16 lanes write one full row, a wavefront instruction 4 rows
+    {
+      T* dst = pob + (long)p * 16 * DV;
+      constexpr int PIECES = DV / 8;                       // 16-byte pieces per row
+#pragma unroll
+      for (int k = 0; k < 16 * PIECES / 64; ++k) {
+        const int e = lane + 64 * k;
+        const int r = e / PIECES, pc = e % PIECES;
+        store8(dst + r * DV + pc * 8, load8(&stage[wave][r * OLD + pc * 8]));
+      }
+    }
+    if (g == 0) {
+      ws.ml[((long)p * 2 + 0) * 16 + n] = mx;
+      ws.ml[((long)p * 2 + 1) * 16 + n] = sum;
+    }
+  }
+}
+
+// ---- merge the partials of every token, gate, add the other branches ---------------------------
+
+__device__ __forceinline__ float gate_of(float x, int act) { return act == 1 ? 1.0f / (1.0f + __expf(-x)) : x; }
+
+template <typename T, int DV>
+__global__ void __launch_bounds__(256)
+slc_merge_kernel(const SlcArgs a, const SlcWs ws) {
+  constexpr int PPR = DV / 8;                                     // 8-channel pieces per output row
+  const long id = (long)blockIdx.x * 256 + threadIdx.x;
+  if (id >= (long)a.total * a.hq * PPR) return;
+  const int pc = (int)(id % PPR);
+  const long row = id / PPR;                                      // token * hq + head
+  const int hq_i = (int)(row % a.hq);
+  const long tg = row / a.hq;
+  const int G = a.hq / a.hkv;
+  const int h = hq_i / G, n = hq_i % G;
+  const long base = (tg * a.hkv + h) * a.top_n;
+  const float c_attn = a.scale * kLog2e;
+  const T* pob = reinterpret_cast<const T*>(ws.po);
+  float M = kNegInf, den = 0.f, acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+#pragma unroll 8
+  for (int i = 0; i < a.top_n; ++i) {
+    const int p = ws.slotmap[base + i];
+    if (p < 0) continue;
+    const float m = ws.ml[((long)p * 2) * 16 + n];
+    const float l = ws.ml[((long)p * 2 + 1) * 16 + n];
+    const vec8_t<T> o = load8(pob + ((long)p * 16 + n) * DV + pc * 8);
+    const float m_new = fmaxf(M, m);
+    const float r_old = fast_exp2((M - m_new) * c_attn);          // 0 for the first partial
+    const float w = fast_exp2((m - m_new) * c_attn) * l;
+    den = den * r_old + w;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = acc[e] * r_old + w * (float)o[e];
+    M = m_new;
+  }
+  const float inv = den > 0.f ? 1.0f / den : 0.f;
+  const T* gs = reinterpret_cast<const T*>(a.g_slc);
+  const T* gw = reinterpret_cast<const T*>(a.g_swa);
+  const T* gcm = reinterpret_cast<const T*>(a.g_cmp);
+  const T* osw = reinterpret_cast<const T*>(a.o_swa);
+  const T* ocm = reinterpret_cast<const T*>(a.o_cmp);
+  const float w_slc = (gs ? gate_of((float)gs[row * a.gate_stride], a.gate_act) : 1.f) * inv;
+  float out[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) out[e] = acc[e] * w_slc;
+  if (osw) {
+    const float w = gw ? gate_of((float)gw[row * a.gate_stride], a.gate_act) : 1.f;
+    const vec8_t<T> o = load8(osw + row * DV + pc * 8);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) out[e] += w * (float)o[e];
+  }
+  if (ocm) {
+    const float w = gcm ? gate_of((float)gcm[row * a.gate_stride], a.gate_act) : 1.f;
+    const vec8_t<T> o = load8(ocm + row * DV + pc * 8);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) out[e] += w * (float)o[e];
+  }
+  store8(reinterpret_cast<T*>(a.out) + row * DV + pc * 8, pack8<T>(out));
+}
+
+template <typename T, int DK, int DV>
+static int launch_block_t(const SlcArgs& a, const SlcWs& ws, hipStream_t st) {
+  const long pairs = ws.pairs_cap;
+  hipLaunchKernelGGL(slc_prep_kernel, dim3(1), dim3(256), 0, st, a.cu_seq, a.batch, ws, a.hkv);
+  const int gb = (int)((pairs + 255) / 256);
+  hipLaunchKernelGGL(slc_bucket_kernel<false>, dim3(gb), dim3(256), 0, st, a, ws);
+  hipLaunchKernelGGL(slc_scan_kernel, dim3(1), dim3(1024), 0, st, ws, a.hkv);
+  hipLaunchKernelGGL(slc_bucket_kernel<true>, dim3(gb), dim3(256), 0, st, a, ws);
+  hipLaunchKernelGGL((slc_block_kernel<T, DK, DV>), dim3((ws.items_cap + 3) / 4), dim3(256), 0, st, a, ws);
+  const long threads = (long)a.total * a.hq * (DV / 8);
+  hipLaunchKernelGGL((slc_merge_kernel<T, DV>), dim3((int)((threads + 255) / 256)), dim3(256), 0, st, a, ws);
+  return 0;
+}
+
+int launch_slc_block_major(const SlcArgs& a, void* workspace, hipStream_t st) {
+  SlcWs ws;
+  carve(a, workspace, &ws, 2);
+  const int key = a.dk * 1000 + a.dv;
+  switch (key) {
+    case 64064: return launch_block_t<bf16_t, 64, 64>(a, ws, st);
+    case 128128: return launch_block_t<bf16_t, 128, 128>(a, ws, st);
+    case 192128: return launch_block_t<bf16_t, 192, 128>(a, ws, st);
+    default: return -2;
+  }
+}
+
+}  // namespace nsa

@@ -198,8 +198,13 @@ def _gate_views(gates, q):
     return [None if g is None else g.to(q.dtype).contiguous() for g in gates], 1
 
 
+SLC_WORKSPACE_LIMIT = 48 << 30      # bytes; larger problems keep the token-major kernel
+
+
 def slc_combine(q, k, vt, indices, counts, g_slc, g_swa, g_cmp, o_swa, o_cmp, cu_seqlens, batch, block_size,
-                scale, gate_act=0):
+                scale, gate_act=0, block_major=None):
+    """block_major: None = use the block-major schedule when the shape has one and its workspace
+    fits SLC_WORKSPACE_LIMIT; False = token-major kernel; True = require block-major."""
     _need_cuda(q, k, vt, indices, cu_seqlens)
     q, k = _dense(q), _dense(k)
     total, hq, dk = q.shape
@@ -215,9 +220,18 @@ def slc_combine(q, k, vt, indices, counts, g_slc, g_swa, g_cmp, o_swa, o_cmp, cu
     o_cmp = None if o_cmp is None else _dense(o_cmp)
     out = torch.empty(total, hq, dv, dtype=q.dtype, device=q.device)
     lib = _lib.load()
+    ws, ws_bytes = None, 0
+    if block_major is not False:
+        need = lib.nsa_slc_workspace_bytes(total, batch, hkv, dk, dv, top_n, block_size, _dtype_code(q))
+        if need > 0 and (block_major or need <= SLC_WORKSPACE_LIMIT):
+            ws = torch.empty(need, dtype=torch.uint8, device=q.device)
+            ws_bytes = need
+        elif block_major:
+            raise NotImplementedError("no block-major selected attention for this shape / dtype")
     rc = lib.nsa_slc_combine_fwd(
         _ptr(q), _ptr(k), _ptr(vt), _ptr(indices), _ptr(counts), _ptr(g_slc), _ptr(g_swa), _ptr(g_cmp), gs,
         _ptr(o_swa), _ptr(o_cmp), _ptr(out), _ptr(cu_seqlens), batch, total, hq, hkv, dk, dv, vt.shape[-1],
-        top_n, block_size, float(scale), int(indices.dtype == torch.int64), gate_act, _dtype_code(q), _stream())
+        top_n, block_size, float(scale), int(indices.dtype == torch.int64), gate_act, _dtype_code(q), _ptr(ws),
+        ws_bytes, _stream())
     _lib.check(rc, "nsa_slc_combine_fwd")
     return out

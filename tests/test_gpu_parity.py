@@ -210,17 +210,21 @@ def test_slc_only(dtype, lens, Hq, Hkv, Dk, Dv, S, bs):
     counts = torch.randint(0, S + 1, (T, Hkv), generator=g)
     vt = ops.transpose(v.to(DEV), cu, len(lens))
     scale = 1.0 / math.sqrt(Dk)
-    for use_counts, dt_idx in ((False, torch.int64), (True, torch.int32)):
+    has_block_major = dtype == torch.bfloat16 and bs == 64
+    modes = ((False, torch.int64, False), (True, torch.int32, False)) + \
+        (((False, torch.int32, True), (True, torch.int64, True)) if has_block_major else ())
+    for use_counts, dt_idx, block_major in modes:
         o = ops.slc_combine(q.to(DEV), k.to(DEV), vt, idx.to(dt_idx).to(DEV),
                             counts.to(DEV) if use_counts else None, None, None, None, None, None, cu,
-                            len(lens), bs, scale).cpu()
+                            len(lens), bs, scale, block_major=block_major).cpu()
         err = 0.0
         for s, e in zip(cuh[:-1], cuh[1:]):
             ref = O.selected_attention(q[s:e], k[s:e], v[s:e], idx[s:e], counts[s:e] if use_counts else None,
                                        bs, scale)
             err = max(err, max_abs(o[s:e], ref))
             assert torch.count_nonzero(o[s]) == 0                     # poisoned row: empty selection -> 0
-        print("slc", dtype, lens, (Hq, Hkv, Dk, Dv, S, bs), "counts", use_counts, "max_abs", err)
+        print("slc", dtype, lens, (Hq, Hkv, Dk, Dv, S, bs), "counts", use_counts, "block_major", block_major,
+              "max_abs", err)
         assert err <= TOL[dtype]
 
 

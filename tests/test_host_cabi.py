@@ -75,7 +75,7 @@ def test_argument_errors_do_not_launch(lib):
     rc = lib.nsa_swa_fwd(p, p, p, p, p, 1, 64, 4, 1, 64, 64, 128, 16, 0.1, 7, None)
     assert rc == -1
     rc = lib.nsa_slc_combine_fwd(p, p, p, p, None, None, None, None, 1, None, None, p, p, 1, 64, 4, 1, 64, 64, 128,
-                                 4, 60, 0.1, 1, 0, 0, None)
+                                 4, 60, 0.1, 1, 0, 0, None, 0, None)
     assert rc == -2 and b"block_size" in lib.nsa_last_error_string()
     rc = lib.nsa_compress_fwd(p, None, None, p, p, p, 1, 10, 2, 60, 32, 16, 0, None)
     assert rc == -2
