@@ -55,17 +55,39 @@ __device__ __forceinline__ void dec_scores(const T* __restrict__ k0p, const T* _
   for (int i = 0; i < 4; ++i) { s[i] = s0[i]; s[4 + i] = s1[i]; }
 }
 
-// one chunk of ordinary attention (window / selected block): keys [cb, cb+32) of the sequence,
-// visible keys are lo..hi
+// Fragments of one 32-key chunk of ordinary attention (window / selected block): two K tiles and
+// the V^T tiles, all requested together so that a chunk costs one memory round trip.
 template <typename T, int DK, int DV>
-__device__ __forceinline__ void dec_attend(DecState<T, DK, DV>& st, const vec8_t<T> (&q)[DK / 32],
-                                           const T* __restrict__ kseq, long krow, const T* __restrict__ vt,
-                                           long vstep, int cb, int lo, int hi, int last_row, float c_attn,
-                                           int n, int g) {
-  float s[8], p[8];
+struct ChunkFrags {
+  vec8_t<T> k0[DK / 32], k1[DK / 32], v[DV / 16];
+};
+
+template <typename T, int DK, int DV>
+__device__ __forceinline__ void chunk_issue(ChunkFrags<T, DK, DV>& f, const T* __restrict__ kseq, long krow,
+                                            const T* __restrict__ vt, long vstep, int cb, int last_row, int n,
+                                            int g) {
   const T* k0p = kseq + (long)min(cb + chunk_key_of_row(0, n), last_row) * krow + 8 * g;
   const T* k1p = kseq + (long)min(cb + chunk_key_of_row(1, n), last_row) * krow + 8 * g;
-  dec_scores<T, DK>(k0p, k1p, q, s);
+#pragma unroll
+  for (int kk = 0; kk < DK / 32; ++kk) { f.k0[kk] = load8(k0p + 32 * kk); f.k1[kk] = load8(k1p + 32 * kk); }
+#pragma unroll
+  for (int t = 0; t < DV / 16; ++t) f.v[t] = load8(vt + t * vstep + cb);
+}
+
+// keys [cb, cb+32) of the sequence, visible keys are lo..hi
+template <typename T, int DK, int DV>
+__device__ __forceinline__ void chunk_attend(DecState<T, DK, DV>& st, const ChunkFrags<T, DK, DV>& f,
+                                             const vec8_t<T> (&q)[DK / 32], int cb, int lo, int hi, float c_attn,
+                                             int g) {
+  f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int kk = 0; kk < DK / 32; ++kk) {
+    s0 = mma16(f.k0[kk], q[kk], s0);
+    s1 = mma16(f.k1[kk], q[kk], s1);
+  }
+  float s[8], p[8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { s[i] = s0[i]; s[4 + i] = s1[i]; }
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const int key = cb + 8 * g + i;
@@ -87,7 +109,7 @@ __device__ __forceinline__ void dec_attend(DecState<T, DK, DV>& st, const vec8_t
 #pragma unroll
   for (int t = 0; t < DV / 16; ++t) {
     st.o[t][0] *= alpha; st.o[t][1] *= alpha; st.o[t][2] *= alpha; st.o[t][3] *= alpha;
-    st.o[t] = mma16(load8(vt + t * vstep + cb), pb, st.o[t]);
+    st.o[t] = mma16(f.v[t], pb, st.o[t]);
   }
 }
 
@@ -98,7 +120,8 @@ decode_step_kernel(const DecodeArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   float* part = reinterpret_cast<float*>(smem_raw);            // [NW][DV][PLD] partial O^T of one branch
   float* pstat = part + NW * DV * PLD;                         // [NW][2][16]   (m, l) per wavefront
-  float* bins = pstat + NW * 2 * 16;                           // [Ns]
+  float* pstat1 = pstat + NW * 2 * 16;                         // [NW][2][16]   score statistics of phase 1
+  float* bins = pstat1 + NW * 2 * 16;                          // [Ns]
   int* sel = reinterpret_cast<int*>(bins + ((a.nc_cap + 3) / 4 + 4));   // [top_n]
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -175,94 +198,131 @@ decode_step_kernel(const DecodeArgs a) {
     }
   };
 
-  // ---- phase 1: compressed scores (registers) + sliding window
+  // ---- phase 0: sliding window, chunks dealt round-robin, next chunk in flight while one is multiplied
+  if (a.window > 0) {
+    DecState<T, DK, DV> swa;
+    dec_reset(swa);
+    const int w_lo = max(t - a.window + 1, 0);
+    ChunkFrags<T, DK, DV> fa, fb;
+    int cb = (w_lo / 32) * 32 + 32 * wave;
+    if (cb <= t) chunk_issue<T, DK, DV>(fa, kseq, krow, vt, vstep, cb, t, n, g);
+    while (cb <= t) {
+      const int cb2 = cb + 32 * NW;
+      if (cb2 <= t) chunk_issue<T, DK, DV>(fb, kseq, krow, vt, vstep, cb2, t, n, g);
+      chunk_attend<T, DK, DV>(swa, fa, qf, cb, w_lo, t, c_attn, g);
+      if (cb2 > t) break;
+      const int cb3 = cb2 + 32 * NW;
+      if (cb3 <= t) chunk_issue<T, DK, DV>(fa, kseq, krow, vt, vstep, cb3, t, n, g);
+      chunk_attend<T, DK, DV>(swa, fb, qf, cb2, w_lo, t, c_attn, g);
+      cb = cb3;
+    }
+    merge(swa, gate(1));
+  }
+
+  // ---- phase 1: compressed scores (kept in registers), next chunk's K fragments in flight
   float sc[MAXC][8];
   float mi = kNegInf, li = 0.f;
-#pragma unroll
-  for (int i = 0; i < MAXC; ++i) {
-    const int cb = 32 * (wave + NW * i);
-    if (cb < Nc) {
+  {
+    vec8_t<T> ka[2][DK / 32], kb2[2][DK / 32];
+    auto issue = [&](vec8_t<T> (&f)[2][DK / 32], int cb) {
       const T* k0p = ckseq + (long)min(cb + chunk_key_of_row(0, n), Nc - 1) * krow + 8 * g;
       const T* k1p = ckseq + (long)min(cb + chunk_key_of_row(1, n), Nc - 1) * krow + 8 * g;
-      dec_scores<T, DK>(k0p, k1p, qf, sc[i]);
-      float mx = kNegInf;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        if (cb + 8 * g + e >= Nc) sc[i][e] = kNegInf;
-        mx = fmaxf(mx, sc[i][e]);
+      for (int kk = 0; kk < DK / 32; ++kk) { f[0][kk] = load8(k0p + 32 * kk); f[1][kk] = load8(k1p + 32 * kk); }
+    };
+    if (32 * wave < Nc) issue(ka, 32 * wave);
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i) {
+      const int cb = 32 * (wave + NW * i);
+      vec8_t<T> (&cur)[2][DK / 32] = (i & 1) ? kb2 : ka;
+      vec8_t<T> (&nxt)[2][DK / 32] = (i & 1) ? ka : kb2;
+      if (i + 1 < MAXC && cb + 32 * NW < Nc) issue(nxt, cb + 32 * NW);
+      if (cb < Nc) {
+        f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < DK / 32; ++kk) {
+          s0 = mma16(cur[0][kk], qf[kk], s0);
+          s1 = mma16(cur[1][kk], qf[kk], s1);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { sc[i][e] = s0[e]; sc[i][4 + e] = s1[e]; }
+        float mx = kNegInf;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          if (cb + 8 * g + e >= Nc) sc[i][e] = kNegInf;
+          mx = fmaxf(mx, sc[i][e]);
+        }
+        mx = colgroup_max(mx);
+        const float m_new = fmaxf(mi, mx);              // finite: row cb exists
+        float sum = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sum += fast_exp2((sc[i][e] - m_new) * kLog2e);
+        li = li * fast_exp2((mi - m_new) * kLog2e) + sum;
+        mi = m_new;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sc[i][e] = kNegInf;
       }
-      mx = colgroup_max(mx);
-      const float m_new = fmaxf(mi, mx);              // finite: row cb exists
-      float sum = 0.f;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) sum += fast_exp2((sc[i][e] - m_new) * kLog2e);
-      li = li * fast_exp2((mi - m_new) * kLog2e) + sum;
-      mi = m_new;
-    } else {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) sc[i][e] = kNegInf;
     }
   }
-  DecState<T, DK, DV> swa;
-  dec_reset(swa);
-  if (a.window > 0) {
-    const int w_lo = max(t - a.window + 1, 0);
-    for (int cb = (w_lo / 32) * 32 + 32 * wave; cb <= t; cb += 32 * NW)
-      dec_attend<T, DK, DV>(swa, qf, kseq, krow, vt, vstep, cb, w_lo, t, t, c_attn, n, g);
-  }
   li = colgroup_sum(li);
-  if (g == 0) { pstat[(wave * 2 + 0) * 16 + n] = mi; pstat[(wave * 2 + 1) * 16 + n] = li; }
+  if (g == 0) { pstat1[(wave * 2 + 0) * 16 + n] = mi; pstat1[(wave * 2 + 1) * 16 + n] = li; }
   __syncthreads();
 
   // ---- phase 2: lse per head, importance bins, compressed attention
   float M = kNegInf;
 #pragma unroll
-  for (int w = 0; w < NW; ++w) M = fmaxf(M, pstat[(w * 2) * 16 + n]);
+  for (int w = 0; w < NW; ++w) M = fmaxf(M, pstat1[(w * 2) * 16 + n]);
   float Z = 0.f;
 #pragma unroll
   for (int w = 0; w < NW; ++w) {
-    const float mw = pstat[(w * 2) * 16 + n];
-    if (mw != kNegInf) Z += pstat[(w * 2 + 1) * 16 + n] * fast_exp2((mw - M) * kLog2e);
+    const float mw = pstat1[(w * 2) * 16 + n];
+    if (mw != kNegInf) Z += pstat1[(w * 2 + 1) * 16 + n] * fast_exp2((mw - M) * kLog2e);
   }
   const float lse2 = (Nc > 0 && n < G) ? (M + __logf(Z)) * kLog2e : __builtin_huge_valf();  // padding heads drop out
-  if (a.window > 0) merge(swa, gate(1));
-  DecState<T, DK, DV> cmp;
-  dec_reset(cmp);
+  // ---- phase 2a: importance bins from the registers (no memory traffic).  The head sum is a DPP
+  // all-reduce over the 16 lanes of a row; lane n == 0 of every row then owns 8 consecutive columns.
+  const bool fast_pool = a.pool_k == 5 && a.pool_s == 4 && a.pool_p == 0;
 #pragma unroll
   for (int i = 0; i < MAXC; ++i) {
     const int cb = 32 * (wave + NW * i);
-    if (cb < Nc) {
-      float p[8];
-      float psum = 0.f;
+    if (cb < Nc && Ns > 0) {
+      float v[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const int c = cb + 8 * g + e;
-        // importance: sum over the 16 lanes (heads) of this lane row
-        float v = fast_exp2(fmaf(sc[i][e], kLog2e, -lse2));
-        v += __shfl_xor(v, 1); v += __shfl_xor(v, 2); v += __shfl_xor(v, 4); v += __shfl_xor(v, 8);
-        if (n == 0 && c < Nc && Ns > 0) {
-          const int num = c + a.pool_p - a.pool_k + 1;
-          const int b_lo = num <= 0 ? 0 : (num + a.pool_s - 1) / a.pool_s;
-          const int b_hi = min((c + a.pool_p) / a.pool_s, Ns - 1);
-          for (int bb = b_lo; bb <= b_hi; ++bb) atomicAdd(&bins[bb], v);
-        }
-        // attention over the visible rows, reference M (>= every visible score)
-        p[e] = c <= cmaxv ? fast_exp2((sc[i][e] - M) * c_attn) : 0.f;
-        psum += p[e];
+        float x = fast_exp2(fmaf(sc[i][e], kLog2e, -lse2));
+        x += dpp_f32<0xB1>(x);          // quad_perm [1,0,3,2]
+        x += dpp_f32<0x4E>(x);          // quad_perm [2,3,0,1]
+        x += dpp_f32<0x141>(x);         // row_half_mirror
+        x += dpp_f32<0x140>(x);         // row_mirror
+        v[e] = x;
       }
-      if (cb <= cmaxv) {
-        cmp.l += psum;
-        const vec8_t<T> pb = pack8<T>(p);
+      const int c0 = cb + 8 * g;
+      if (n == 0 && c0 < Nc) {
+        if (fast_pool) {
+          // windows of 5 columns every 4: columns c0..c0+7 touch bins c0/4-1 (first column only),
+          // c0/4 and c0/4+1; columns past Nc carry 0
+          const int b0 = c0 >> 2;
+          if (b0 >= 1 && b0 - 1 < Ns) atomicAdd(&bins[b0 - 1], v[0]);
+          if (b0 < Ns) atomicAdd(&bins[b0], (v[0] + v[1]) + (v[2] + v[3]) + v[4]);
+          if (b0 + 1 < Ns) atomicAdd(&bins[b0 + 1], (v[4] + v[5]) + (v[6] + v[7]));
+        } else {
 #pragma unroll
-        for (int tt = 0; tt < DV / 16; ++tt) cmp.o[tt] = mma16(load8(cvt + tt * cvstep + cb), pb, cmp.o[tt]);
+          for (int e = 0; e < 8; ++e) {
+            const int c = c0 + e;
+            if (c >= Nc) break;
+            const int num = c + a.pool_p - a.pool_k + 1;
+            const int b_lo = num <= 0 ? 0 : (num + a.pool_s - 1) / a.pool_s;
+            const int b_hi = min((c + a.pool_p) / a.pool_s, Ns - 1);
+            for (int bb = b_lo; bb <= b_hi; ++bb) atomicAdd(&bins[bb], v[e]);
+          }
+        }
       }
     }
   }
-  cmp.m = cmaxv >= 0 ? M : kNegInf;   // every wavefront used the common reference M
-  merge(cmp, gate(2));               // its barriers also complete the bins
   __syncthreads();
 
-  // ---- phase 3: top-n blocks (wavefront 0); each lane owns the bins b == lane (mod 64)
+  // ---- phase 3 (wavefront 0 only): top-n blocks; each lane owns the bins b == lane (mod 64)
   if (wave == 0) {
     volatile float* vb = bins;
     for (int bb = lane; bb < Ns; bb += 64) {
@@ -270,45 +330,85 @@ decode_step_kernel(const DecodeArgs a) {
       const int div = min(lo + a.pool_k, Nc + a.pool_p) - lo;
       vb[bb] = vb[bb] / (float)div;
     }
-    for (int r = 0; r < a.top_n; ++r) {
-      float best = -1.f;
-      int bi = 0x7fffffff;
-      for (int bb = lane; bb < Ns; bb += 64) {
-        const float v = vb[bb];
-        if (v > best) { best = v; bi = bb; }
-      }
-#pragma unroll
-      for (int off = 1; off < 64; off <<= 1) {
-        const float ov = __shfl_xor(best, off);
-        const int oi = __shfl_xor(bi, off);
-        if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
-      }
-      const bool found = best >= 0.f;
-      if (found && (bi & 63) == lane) vb[bi] = -1.f;
+    wave_topn<(32 * kDecWaves * kDecMaxChunks / 4 + 63) / 64 + 1>(vb, Ns, a.top_n, lane, [&](int rr, int val) {
       if (lane == 0) {
-        sel[r] = found ? bi : -1;
-        if (a.indices != nullptr) a.indices[((long)b * a.hkv + h) * a.top_n + r] = found ? bi : -1;
+        sel[rr] = val;
+        if (a.indices != nullptr) a.indices[((long)b * a.hkv + h) * a.top_n + rr] = val;
+      }
+    });
+  }
+
+  // ---- phase 2b: compressed attention from the registers, cv^T fragments one chunk ahead
+  DecState<T, DK, DV> cmp;
+  dec_reset(cmp);
+  {
+    vec8_t<T> va[DV / 16], vb2[DV / 16];
+    auto issue = [&](vec8_t<T> (&f)[DV / 16], int cb) {
+#pragma unroll
+      for (int tt = 0; tt < DV / 16; ++tt) f[tt] = load8(cvt + tt * cvstep + cb);
+    };
+    if (32 * wave <= cmaxv) issue(va, 32 * wave);
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i) {
+      const int cb = 32 * (wave + NW * i);
+      vec8_t<T> (&cur)[DV / 16] = (i & 1) ? vb2 : va;
+      vec8_t<T> (&nxt)[DV / 16] = (i & 1) ? va : vb2;
+      if (i + 1 < MAXC && cb + 32 * NW <= cmaxv) issue(nxt, cb + 32 * NW);
+      if (cb <= cmaxv) {
+        float p[8], psum = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int c = cb + 8 * g + e;
+          p[e] = c <= cmaxv ? fast_exp2((sc[i][e] - M) * c_attn) : 0.f;   // reference M >= every visible score
+          psum += p[e];
+        }
+        cmp.l += psum;
+        const vec8_t<T> pb = pack8<T>(p);
+#pragma unroll
+        for (int tt = 0; tt < DV / 16; ++tt) cmp.o[tt] = mma16(cur[tt], pb, cmp.o[tt]);
       }
     }
   }
-  __syncthreads();
+  cmp.m = cmaxv >= 0 ? M : kNegInf;   // every wavefront used the common reference M
+  merge(cmp, gate(2));               // its barriers also publish the selected blocks
 
-  // ---- phase 4: selected blocks, 32-key chunks dealt round-robin
+  // ---- phase 4: selected blocks, 32-key chunks dealt round-robin, next chunk in flight
   DecState<T, DK, DV> slc;
   dec_reset(slc);
   {
-    int item = 0;
-    for (int r = 0; r < a.top_n; ++r) {
-      const int bi = sel[r];
-      if (bi < 0 || (long)bi * a.sel_block > t) continue;
-      const int k0 = bi * a.sel_block;
-      const int k1 = min(k0 + a.sel_block - 1, t);
-      for (int cb = k0; cb <= k1; cb += 32, ++item)
-        if ((item & (NW - 1)) == wave)
-          dec_attend<T, DK, DV>(slc, qf, kseq, krow, vt, vstep, cb, k0, k1, t, c_attn, n, g);
+    int rr = 0, item = 0, cur = 0, cur_last = -1, cur_k0 = 0;
+    // next 32-key chunk of this wavefront: (cb, k0, k1) of its block; false when the picks are exhausted
+    auto next_chunk = [&](int& cb, int& k0, int& k1) -> bool {
+      while (true) {
+        if (cur > cur_last) {
+          if (rr >= a.top_n) return false;
+          const int bi = sel[rr++];
+          if (bi < 0 || (long)bi * a.sel_block > t) continue;
+          cur_k0 = bi * a.sel_block;
+          cur = cur_k0;
+          cur_last = min(cur_k0 + a.sel_block - 1, t);
+        }
+        const bool mine = (item & (NW - 1)) == wave;
+        cb = cur; k0 = cur_k0; k1 = cur_last;
+        cur += 32;
+        ++item;
+        if (mine) return true;
+      }
+    };
+    ChunkFrags<T, DK, DV> fa, fb;
+    int cba, k0a, k1a, cbb, k0b, k1b;
+    bool ha = next_chunk(cba, k0a, k1a);
+    if (ha) chunk_issue<T, DK, DV>(fa, kseq, krow, vt, vstep, cba, t, n, g);
+    while (ha) {
+      const bool hb = next_chunk(cbb, k0b, k1b);
+      if (hb) chunk_issue<T, DK, DV>(fb, kseq, krow, vt, vstep, cbb, t, n, g);
+      chunk_attend<T, DK, DV>(slc, fa, qf, cba, k0a, k1a, c_attn, g);
+      if (!hb) break;
+      ha = next_chunk(cba, k0a, k1a);
+      if (ha) chunk_issue<T, DK, DV>(fa, kseq, krow, vt, vstep, cba, t, n, g);
+      chunk_attend<T, DK, DV>(slc, fb, qf, cbb, k0b, k1b, c_attn, g);
     }
   }
-
   merge(slc, gate(0));
   if (r < G && d0 < DV) {
     T* op = reinterpret_cast<T*>(a.out) + ((long)b * a.hq + h * G + r) * DV + d0;
@@ -355,7 +455,7 @@ int set_smem(const void* fn, size_t bytes);
 
 template <typename T, int DK, int DV>
 static int launch_decode_t(const DecodeArgs& a, hipStream_t st) {
-  const size_t smem = ((size_t)kDecWaves * DV * 17 + kDecWaves * 32 + (a.nc_cap + 3) / 4 + 4) * sizeof(float) +
+  const size_t smem = ((size_t)kDecWaves * DV * 17 + kDecWaves * 64 + (a.nc_cap + 3) / 4 + 4) * sizeof(float) +
                       (size_t)a.top_n * sizeof(int) + 64;
   auto fn = decode_step_kernel<T, DK, DV>;
   const int rc = set_smem(reinterpret_cast<const void*>(fn), smem);

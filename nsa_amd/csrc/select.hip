@@ -197,26 +197,32 @@ importance_select_kernel(const CmpArgs a) {
       vb[tl * Ns + b] = v;
       if (a.pooled != nullptr) a.pooled[orow * a.pooled_stride + b] = v;
     }
-    for (int r = 0; r < a.top_n; ++r) {
-      float best = -1.f;
-      int bi = 0x7fffffff;
-      for (int b = lane; b < Ns; b += 64) {
-        const float v = vb[tl * Ns + b];
-        if (v > best) { best = v; bi = b; }
-      }
-#pragma unroll
-      for (int off = 1; off < 64; off <<= 1) {
-        const float ov = __shfl_xor(best, off);
-        const int oi = __shfl_xor(bi, off);
-        if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
-      }
-      const bool found = best >= 0.f;
-      if (found && (bi & 63) == lane) vb[tl * Ns + bi] = -1.f;
+    auto emit = [&](int r, int val) {
       if (lane == 0) {
         const long pos = orow * a.top_n + r;
-        const int val = found ? bi : -1;
         if (a.idx64) reinterpret_cast<int64_t*>(a.indices)[pos] = val;
         else reinterpret_cast<int32_t*>(a.indices)[pos] = val;
+      }
+    };
+    if (Ns <= 64 * 8) {
+      wave_topn<8>(vb + tl * Ns, Ns, a.top_n, lane, emit);
+    } else {
+      for (int r = 0; r < a.top_n; ++r) {
+        float best = -1.f;
+        int bi = 0x7fffffff;
+        for (int b = lane; b < Ns; b += 64) {
+          const float v = vb[tl * Ns + b];
+          if (v > best) { best = v; bi = b; }
+        }
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+          const float ov = __shfl_xor(best, off);
+          const int oi = __shfl_xor(bi, off);
+          if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+        }
+        const bool found = best >= 0.f;
+        if (found && (bi & 63) == lane) vb[tl * Ns + bi] = -1.f;
+        emit(r, found ? bi : -1);
       }
     }
   }

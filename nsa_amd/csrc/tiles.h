@@ -105,6 +105,71 @@ __device__ __forceinline__ void store_rows(T* __restrict__ out_row, const f32x4_
   }
 }
 
+// Arg-max all-reduce over the 64 lanes of (score bits, tie key) packed as a signed 64-bit value:
+// non-negative floats order like their bit patterns, the "taken" marker -1.0f is negative.
+__device__ __forceinline__ long wave_max_i64(long key) {
+  auto step = [&](int lo_other, int hi_other) {
+    const long other = ((long)hi_other << 32) | (unsigned int)lo_other;
+    key = other > key ? other : key;
+  };
+  int lo = (int)key, hi = (int)(key >> 32);
+#define NSA_DPP_STEP(CTRL)                                                                       \
+  lo = (int)key; hi = (int)(key >> 32);                                                          \
+  step(__builtin_amdgcn_update_dpp(lo, lo, CTRL, 0xF, 0xF, false),                               \
+       __builtin_amdgcn_update_dpp(hi, hi, CTRL, 0xF, 0xF, false));
+  NSA_DPP_STEP(0xB1)    // quad_perm [1,0,3,2]
+  NSA_DPP_STEP(0x4E)    // quad_perm [2,3,0,1]
+  NSA_DPP_STEP(0x141)   // row_half_mirror
+  NSA_DPP_STEP(0x140)   // row_mirror
+#undef NSA_DPP_STEP
+  {
+    lo = (int)key; hi = (int)(key >> 32);
+    const auto a = __builtin_amdgcn_permlane16_swap((unsigned)lo, (unsigned)lo, false, false);
+    const auto b = __builtin_amdgcn_permlane16_swap((unsigned)hi, (unsigned)hi, false, false);
+    const long k0 = ((long)(int)b[0] << 32) | a[0], k1 = ((long)(int)b[1] << 32) | a[1];
+    key = k0 > k1 ? k0 : k1;
+  }
+  {
+    lo = (int)key; hi = (int)(key >> 32);
+    const auto a = __builtin_amdgcn_permlane32_swap((unsigned)lo, (unsigned)lo, false, false);
+    const auto b = __builtin_amdgcn_permlane32_swap((unsigned)hi, (unsigned)hi, false, false);
+    const long k0 = ((long)(int)b[0] << 32) | a[0], k1 = ((long)(int)b[1] << 32) | a[1];
+    key = k0 > k1 ? k0 : k1;
+  }
+  return key;
+}
+
+// Top-n of row[0..ns) (non-negative scores in LDS, ns <= 64*PER) by one wavefront: every lane keeps
+// its candidates b = lane + 64k in registers; each round is a local scan, one 64-lane arg-max
+// (ties go to the lower index) and the winner's lane retiring its entry.  emit(r, index or -1).
+template <int PER, typename Emit>
+__device__ __forceinline__ void wave_topn(const volatile float* row, int ns, int top_n, int lane, Emit emit) {
+  float v[PER];
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    const int b = lane + 64 * k;
+    v[k] = b < ns ? row[b] : -1.f;
+  }
+  for (int r = 0; r < top_n; ++r) {
+    float best = v[0];
+    int bk = 0;
+#pragma unroll
+    for (int k = 1; k < PER; ++k)
+      if (v[k] > best) { best = v[k]; bk = k; }
+    const int bi = lane + 64 * bk;
+    long key = ((long)__float_as_int(best) << 32) | (unsigned int)(0x7fffffff - bi);
+    key = wave_max_i64(key);
+    const bool found = (int)(key >> 32) >= 0;
+    const int win = 0x7fffffff - (int)(unsigned int)key;
+    if (found && (win & 63) == lane) {
+#pragma unroll
+      for (int k = 0; k < PER; ++k)
+        if (k == (win >> 6)) v[k] = -1.f;
+    }
+    emit(r, found ? win : -1);
+  }
+}
+
 __device__ __forceinline__ int ilog2(int x) { return 31 - __builtin_clz(x); }
 __device__ __forceinline__ int next_pow2(int x) {
   int p = 1;
