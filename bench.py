@@ -35,6 +35,8 @@ WORKLOADS = {
     "prefill_cfg2": ([8192], 64, 4, 128, 128, 16, 512, 1),
 }
 BLOCK, STRIDE, SEL_BLOCK = 32, 16, 64
+# bytes per launch: (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0) KiB, factors from a 1 GiB device copy in the same run
+MEASURED_TRAFFIC = {("prefill_cfg4", "cmp_attn"): int((565562.4 * 2.0 + 790751.4) * 1024)}
 
 
 def flops_model(lens, hq, hkv, dqk, dv, window, valid_blocks_total):
@@ -148,6 +150,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-budget", type=float, default=20.0)
     ap.add_argument("--no-decode", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 1 GiB device copy (reference point for FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures the one-GPU NSA forward path; --gpus %d is not supported (this build has no "
@@ -178,6 +182,13 @@ def main():
     def step():
         return m(qd, kd, vd, cu, max_len, gates=gd)
 
+    if args.copy_calibration:
+        src = torch.zeros(1 << 28, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(2):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -205,10 +216,16 @@ def main():
     valid = ((idx >= 0) & (idx.long() * SEL_BLOCK <= tok[:, None, None])).sum().item()
     fl = flops_model(lens, hq, hkv, dqk, dv, window, valid)
     f_eff = fl["cmp"] + fl["slc"] + fl["swa"]
-    # block_select carries no credited flops: its score tiles are the uncredited non-causal pass
+    # Per-stage credited flops.  block_select carries none (its score tiles are the uncredited
+    # non-causal importance pass); slc_combine is a chain of kernels (bucket, block, merge), the other
+    # stages are one kernel each, so the single dominant kernel is the longest of cmp_attn / swa.
     stage_flops = {"cmp_attn": fl["cmp"], "swa": fl["swa"], "slc_combine": fl["slc"]}
-    dom = max(stage_flops, key=lambda n: stage_ms.get(n, 0.0))
-    dom_tflops = stage_flops[dom] / (stage_ms[dom] * 1e-3) / 1e12
+    stage_tflops = {n: stage_flops[n] / (stage_ms[n] * 1e-3) / 1e12 for n in stage_flops if n in stage_ms}
+    dom = max(("cmp_attn", "swa"), key=lambda n: stage_ms.get(n, 0.0))
+    dom_tflops = stage_tflops[dom]
+    # HBM bytes per launch of that kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE (profiles/), only
+    # recorded for the default workload
+    traffic = MEASURED_TRAFFIC.get((args.workload, dom))
 
     res = {
         "metric": "nsa_prefill_fwd_tokens_per_s", "value": total / (ms * 1e-3), "unit": "tokens/s",
@@ -222,7 +239,8 @@ def main():
         "mfma_peak_frac_whole_step": f_eff / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
         "stage_ms": stage_ms,
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": dom_tflops, "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "frac": dom_tflops / PEAK_BF16_TFLOPS, "traffic": None},
+                     "unit": "TFLOP/s", "frac": dom_tflops / PEAK_BF16_TFLOPS, "traffic": traffic},
+        "stage_effective_tflops": stage_tflops,
     }
     if not args.no_decode:
         del qd, kd, vd, gd, out, idx

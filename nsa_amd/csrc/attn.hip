@@ -250,13 +250,33 @@ stream_attn_kernel(const StreamParams a) {
     buf ^= 1;
   }
 
+  // Output rows leave through LDS (the K buffers are free after the loop's last barrier): the
+  // accumulators hold 4 channels of 16 different rows per lane, whole 16-byte pieces of one row
+  // per lane make full cache lines.
   T* ob = reinterpret_cast<T*>(a.o);
+  constexpr int OLD = DV + 8;
+  static_assert(NW * 16 * OLD <= 2 * CH * KLD + 2 * DV * VLD, "output staging must fit the K/V buffers");
+  T* stage = ldsK + wave * 16 * OLD;
 #pragma unroll
   for (int j = 0; j < NG; ++j) {
     const float lt = colgroup_sum(grp[j].l);
     const float inv = lt > 0.f ? 1.0f / lt : 0.f;
     const long row = ((long)st.start + rm[j].tok) * a.hq + h * G + rm[j].gidx;
-    if (rm[j].valid) store_rows<T, DV>(ob + row * DV, grp[j].o, inv, g);
+    store_rows<T, DV>(stage + n * OLD, grp[j].o, inv, g);
+    {
+      constexpr int PIECES = DV / 8;
+      const int gi = wave * NG + j;
+#pragma unroll
+      for (int k = 0; k < (16 * PIECES + 63) / 64; ++k) {
+        const int e = lane + 64 * k;
+        const int r = e / PIECES, pc = e % PIECES;
+        if (16 * PIECES % 64 == 0 || r < 16) {
+          const RowMap rr = map_row(st.t0, gi, r, lgp, G, st.len);
+          if (rr.valid)
+            store8(ob + (((long)st.start + rr.tok) * a.hq + h * G + rr.gidx) * DV + pc * 8, load8(stage + r * OLD + pc * 8));
+        }
+      }
+    }
     if (CMP && a.lse != nullptr) {
       const float lit = colgroup_sum(li[j]);
       if (rm[j].valid && g == 0) a.lse[row] = nkeys > 0 ? grp[j].m + __logf(lit) : 0.f;
