@@ -97,26 +97,41 @@ stream_attn_kernel(const StreamParams a) {
   const int c_begin = CMP ? 0 : (max(st.t0 - W + 1, 0) / CH) * CH;
   const int c_end = CMP ? nkeys : t_last + 1;
 
+  // Per-thread element offsets of its staging pieces for chunk 0; a chunk adds one scalar.  Only the
+  // last chunk of a sequence needs the row clamp.
   vec8_t<T> kr[KPT], vr[VPT];
-  auto gload = [&](int c0, bool with_v) {
+  unsigned kpo[KPT], vpo[VPT];
 #pragma unroll
-    for (int i = 0; i < KPT; ++i) {
-      const int p = tid + i * NT;
-      if (KPIECES % NT == 0 || p < KPIECES) {
-        const int r = p / (DK / 8), pc = p % (DK / 8);
-        const int sr = min(c0 + r, nkeys - 1);
-        kr[i] = load8(kb + (long)sr * a.k_row_stride + pc * 8);
+  for (int i = 0; i < KPT; ++i) {
+    const int p = tid + i * NT;
+    kpo[i] = (unsigned)((p / (DK / 8)) * (int)a.k_row_stride + (p % (DK / 8)) * 8);
+  }
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int p = tid + i * NT;
+    vpo[i] = (unsigned)((p / (CH / 8)) * a.vt_cols + (p % (CH / 8)) * 8);
+  }
+  auto gload = [&](int c0, bool with_v) {
+    if (c0 + CH <= nkeys) {
+      const unsigned base = (unsigned)c0 * (unsigned)a.k_row_stride;
+#pragma unroll
+      for (int i = 0; i < KPT; ++i)
+        if (KPIECES % NT == 0 || tid + i * NT < KPIECES) kr[i] = load8(kb + (base + kpo[i]));
+    } else {
+#pragma unroll
+      for (int i = 0; i < KPT; ++i) {
+        const int p = tid + i * NT;
+        if (KPIECES % NT == 0 || p < KPIECES) {
+          const int r = p / (DK / 8), pc = p % (DK / 8);
+          const int sr = min(c0 + r, nkeys - 1);
+          kr[i] = load8(kb + (long)sr * a.k_row_stride + pc * 8);
+        }
       }
     }
     if (with_v) {
 #pragma unroll
-      for (int i = 0; i < VPT; ++i) {
-        const int p = tid + i * NT;
-        if (VPIECES % NT == 0 || p < VPIECES) {
-          const int r = p / (CH / 8), pc = p % (CH / 8);
-          vr[i] = load8(vtb + (long)r * a.vt_cols + c0 + pc * 8);
-        }
-      }
+      for (int i = 0; i < VPT; ++i)
+        if (VPIECES % NT == 0 || tid + i * NT < VPIECES) vr[i] = load8(vtb + ((unsigned)c0 + vpo[i]));
     }
   };
   auto lstore = [&](int buf, bool with_v) {
@@ -189,15 +204,14 @@ stream_attn_kernel(const StreamParams a) {
           const float m_new = fmaxf(grp[j].m, mx);
           if (__any(m_new > grp[j].m)) {
             const float d = grp[j].m - m_new;          // -inf on the first chunk
-            li[j] *= fast_exp2(d * kLog2e);
-            const float alpha = fast_exp2(d * c_attn);
-            grp[j].l *= alpha;
+            float beta = fast_exp2(d * kLog2e), alpha = fast_exp2(d * c_attn);
+            settle_factor(beta, alpha);
+            scale_inplace(li[j], beta);
+            scale_inplace(grp[j].l, alpha);
 #pragma unroll
-            for (int t = 0; t < DV / 16; ++t) {
-              grp[j].o[t][0] *= alpha; grp[j].o[t][1] *= alpha; grp[j].o[t][2] *= alpha; grp[j].o[t][3] *= alpha;
-            }
-            grp[j].m = m_new;
+            for (int t = 0; t < DV / 16; ++t) scale_inplace(grp[j].o[t], alpha);
           }
+          grp[j].m = m_new;
           const float m = grp[j].m;
           const float off_i = -m * kLog2e, off_a = -m * c_attn;
           float sum = 0.f;
@@ -238,11 +252,9 @@ stream_attn_kernel(const StreamParams a) {
           }
         }
       }
-      bool all_act = true;
-#pragma unroll
-      for (int j = 0; j < NG; ++j) all_act &= act[j];
-      if (all_act) pv32_all<T, DK, DV, NG>(bv + n * VLD + 32 * sub + 8 * g, 16 * VLD, grp, pb);
-      else if (any_act) pv32<T, DK, DV, NG>(bv + n * VLD + 32 * sub + 8 * g, 16 * VLD, grp, pb, act);
+      // a group without visible keys in this chunk carries all-zero probabilities: one MFMA chain
+      // for all groups keeps the accumulators in place (no per-group control flow around them)
+      if (any_act) pv32_all<T, DK, DV, NG>(bv + n * VLD + 32 * sub + 8 * g, 16 * VLD, grp, pb);
     }
 
     if (has_next) lstore(buf ^ 1, next_v);

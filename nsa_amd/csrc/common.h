@@ -170,6 +170,30 @@ __device__ __forceinline__ void group_reset(RowGroup<T, DK, DV>& g) {
   g.l = 0.f;
 }
 
+// x *= a with the result forced into the register x already lives in.  Used inside rarely taken
+// branches that rescale accumulators: a plain multiply lets the compiler put the products in new
+// registers, and the common not-taken path then pays one register move per accumulator.
+//
+// The compiler's hazard recogniser does not look inside inline assembly, so the wait states it
+// would insert between a transcendental (v_exp_f32) or MFMA result and an ordinary VALU consumer
+// are missing for these multiplies.  Every factor therefore has to pass through settle_factor()
+// first: it is ordered after the factor's computation and holds 12 wait states, which covers the
+// transcendental forwarding hazard (1) and an 8-pass MFMA write followed by a VALU read (11).
+__device__ __forceinline__ void settle_factor(float& a) {
+  asm volatile("s_nop 7\n\ts_nop 3" : "+v"(a));
+}
+__device__ __forceinline__ void settle_factor(float& a, float& b) {
+  asm volatile("s_nop 7\n\ts_nop 3" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ void scale_inplace(float& x, float a) {
+  asm volatile("v_mul_f32 %0, %1, %0" : "+v"(x) : "v"(a));
+}
+__device__ __forceinline__ void scale_inplace(f32x4_t& v, float a) {
+  float e0 = v[0], e1 = v[1], e2 = v[2], e3 = v[3];
+  scale_inplace(e0, a); scale_inplace(e1, a); scale_inplace(e2, a); scale_inplace(e3, a);
+  v[0] = e0; v[1] = e1; v[2] = e2; v[3] = e3;
+}
+
 // Raise the running maximum of a group to cover `mx` (already reduced over the column's four
 // lanes).  The accumulator and denominator are rescaled only when some lane's maximum grew, which
 // after the first few chunks is rare.  c = scale * log2(e).
@@ -178,14 +202,13 @@ __device__ __forceinline__ void raise_max(RowGroup<T, DK, DV>& g, float mx, floa
   const float m_new = fmaxf(g.m, mx);
   if (__any(m_new > g.m)) {
     const float mref = (m_new == kNegInf) ? 0.f : m_new;
-    const float alpha = fast_exp2((g.m - mref) * c);
-    g.l *= alpha;
+    float alpha = fast_exp2((g.m - mref) * c);
+    settle_factor(alpha);
+    scale_inplace(g.l, alpha);
 #pragma unroll
-    for (int i = 0; i < DV / 16; ++i) {
-      g.o[i][0] *= alpha; g.o[i][1] *= alpha; g.o[i][2] *= alpha; g.o[i][3] *= alpha;
-    }
-    g.m = m_new;
+    for (int i = 0; i < DV / 16; ++i) scale_inplace(g.o[i], alpha);
   }
+  g.m = m_new;
 }
 
 // Online-softmax update for the 8 scores a lane holds of one 32-key chunk (masked entries are

@@ -70,13 +70,26 @@ importance_select_kernel(const CmpArgs a) {
   for (int j = 0; j < NG; ++j) pend[j] = 0.f;
 
   vec8_t<T> kr[KPT];
-  auto gload = [&](int c0) {
+  unsigned koff[KPT];
 #pragma unroll
-    for (int i = 0; i < KPT; ++i) {
-      const int p = tid + i * NT;
-      if (KPIECES % NT == 0 || p < KPIECES) {
-        const int sr = min(c0 + p / (DK / 8), Nc - 1);
-        kr[i] = load8(ckb + (long)sr * a.ck_row_stride + (p % (DK / 8)) * 8);
+  for (int i = 0; i < KPT; ++i) {
+    const int p = tid + i * NT;
+    koff[i] = (unsigned)((p / (DK / 8)) * (int)a.ck_row_stride + (p % (DK / 8)) * 8);
+  }
+  auto gload = [&](int c0) {
+    if (c0 + CH <= Nc) {
+      const unsigned base = (unsigned)c0 * (unsigned)a.ck_row_stride;
+#pragma unroll
+      for (int i = 0; i < KPT; ++i)
+        if (KPIECES % NT == 0 || tid + i * NT < KPIECES) kr[i] = load8(ckb + (base + koff[i]));
+    } else {
+#pragma unroll
+      for (int i = 0; i < KPT; ++i) {
+        const int p = tid + i * NT;
+        if (KPIECES % NT == 0 || p < KPIECES) {
+          const int sr = min(c0 + p / (DK / 8), Nc - 1);
+          kr[i] = load8(ckb + (long)sr * a.ck_row_stride + (p % (DK / 8)) * 8);
+        }
       }
     }
   };
