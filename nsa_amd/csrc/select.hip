@@ -13,9 +13,8 @@
 
 namespace nsa {
 
-// FAST: GQA group of 16 (one token per row group) and the default pooling (5 columns every 4, no
-// padding); everything else takes the generic path with LDS atomics.
-template <typename T, int DK, int NG, int CH, int NW, bool FAST>
+// Any GQA group size up to 16 and any pooling window: column sums go into the bins with LDS atomics.
+template <typename T, int DK, int NG, int CH, int NW>
 __global__ void __launch_bounds__(NW * 64)
 importance_select_kernel(const CmpArgs a) {
   constexpr int KLD = DK + 8, ROWS = NW * NG * 16, NT = NW * 64;
@@ -28,7 +27,7 @@ importance_select_kernel(const CmpArgs a) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 15, g = lane >> 4;
-  const int G = a.hq / a.hkv, Gp = FAST ? 16 : next_pow2(G), lgp = FAST ? 4 : ilog2(Gp);
+  const int G = a.hq / a.hkv, Gp = next_pow2(G), lgp = ilog2(Gp);
   const int TQ = ROWS >> lgp;
   const SeqTile st = find_tile(a.cu_seq, a.batch, TQ, blockIdx.x);
   if (!st.valid) return;
@@ -64,10 +63,6 @@ importance_select_kernel(const CmpArgs a) {
 
   for (int i = tid; i < TQ * Ns; i += NT) bins[i] = 0.f;
   wait_all_loads();
-
-  float pend[NG];   // FAST: the unfinished last bin of the previous tile (lane 12 of the g == 0 row)
-#pragma unroll
-  for (int j = 0; j < NG; ++j) pend[j] = 0.f;
 
   vec8_t<T> kr[KPT];
   unsigned koff[KPT];
@@ -128,34 +123,6 @@ importance_select_kernel(const CmpArgs a) {
         for (int j = 0; j < NG; ++j) s[j] = mma16(qf[j][kk], kf, s[j]);   // rows = heads, columns = keys
       }
       const int c = cb + n;
-      if (FAST) {
-        // One token per row group, windows of 5 columns every 4: after the head sum every lane of
-        // tile column n holds R[c].  Quad sums and the first column of the next quad come from DPP.
-        // Bins 4t..4t+2 of tile t are complete at once; bin 4t+3 waits in a register of lane 12 for
-        // the first column of the next tile.  Every bin is written exactly once by the g == 0 row.
-#pragma unroll
-        for (int j = 0; j < NG; ++j) {
-          float e[4];
-#pragma unroll
-          for (int i = 0; i < 4; ++i) e[i] = fast_exp2(fmaf(s[j][i], kLog2e, -lse_r[j][i]));
-          float v = colgroup_sum((e[0] + e[1]) + (e[2] + e[3]));
-          v = c < Nc ? v : 0.f;
-          const float t2 = v + dpp_f32<0xB1>(v);            // quad_perm [1,0,3,2]
-          const float quad = t2 + dpp_f32<0x4E>(t2);        // quad_perm [2,3,0,1]
-          const float nextf = dpp_f32<0x104>(v);            // row_shl:4 -> R[c+4], 0 past the tile
-          const float first = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
-          if (g == 0 && (n & 3) == 0) {
-            float* row = bins + (wave * NG + j) * Ns;
-            const int b = (cb >> 2) + (n >> 2);
-            if (n == 12) {
-              if (cb > 0 && (cb >> 2) - 1 < Ns) row[(cb >> 2) - 1] = pend[j] + first;
-              pend[j] = quad;
-            } else if (b < Ns) {
-              row[b] = quad + nextf;
-            }
-          }
-        }
-      } else {
       // bins that contain column c: b*s - p <= c < b*s - p + k
       const int num = c + a.pool_p - a.pool_k + 1;
       const int b_lo = num <= 0 ? 0 : (num + a.pool_s - 1) / a.pool_s;
@@ -183,17 +150,10 @@ importance_select_kernel(const CmpArgs a) {
           }
         }
       }
-      }
     }
     if (has_next) lstore(buf ^ 1);
     __syncthreads();
     buf ^= 1;
-  }
-  if (FAST && c_end > 0 && g == 0 && n == 12) {
-    const int b = ((((c_end - 1) >> 4) << 4) >> 2) + 3;     // last bin of the last tile: no next column
-#pragma unroll
-    for (int j = 0; j < NG; ++j)
-      if (b < Ns) bins[(wave * NG + j) * Ns + b] = pend[j];
   }
   __syncthreads();
 
@@ -210,6 +170,8 @@ importance_select_kernel(const CmpArgs a) {
       vb[tl * Ns + b] = v;
       if (a.pooled != nullptr) a.pooled[orow * a.pooled_stride + b] = v;
     }
+    if (a.pooled != nullptr)
+      for (int b = Ns + lane; b < a.max_ns; b += 64) a.pooled[orow * a.pooled_stride + b] = 0.f;
     auto emit = [&](int r, int val) {
       if (lane == 0) {
         const long pos = orow * a.top_n + r;
@@ -241,6 +203,243 @@ importance_select_kernel(const CmpArgs a) {
   }
 }
 
+// Reduce-scatter of four per-lane partial column sums over the four 16-lane rows of a wavefront:
+// row g of the result holds the total of v_g.  Each step is one lane swap plus one add and needs no
+// copies, because the two swapped registers hold different values that are both consumed.
+__device__ __forceinline__ float row_reduce_scatter4(float v0, float v1, float v2, float v3) {
+  auto rs32 = [](float a, float b) {       // lower half: a summed over rows (g, g+2); upper half: b
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+  };
+  const float x = rs32(v0, v2), y = rs32(v1, v3);
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(y), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+// Block importance for the common shape: GQA group of 9..16 heads (one token per row group) and
+// the default pooling (windows of 5 columns every 4, no padding).  Writes the raw window sums to
+// a.pooled; topn_kernel below turns them into averages and picks the blocks.
+//
+// A workgroup of NW wavefronts owns NW*NG tokens of one kv head and streams ck through LDS in steps
+// of 64 rows, double buffered.  Per step and token a wavefront computes four 16x16 score tiles
+// (rows = heads, columns = compressed rows), exponentiates, adds the four heads each lane holds and
+// keeps one partial per tile; a 3-swap reduce-scatter then leaves lane i with the head sum R of
+// column c0 + i.  Bin b = R[4b .. 4b+4]: the quad sum comes from two DPP adds, the fifth column from
+// the next lane (wave_shl:1), so lanes 3, 7, .., 59 each store one finished bin and lane 63 carries
+// its quad to the next step, where it is completed with that step's first column.  Every bin is
+// written exactly once, 64 contiguous bytes per token and step, with no atomics.
+template <typename T, int DK, int NG, int NW>
+__global__ void __launch_bounds__(NW * 64)
+importance_stream_kernel(const CmpArgs a) {
+  constexpr int CH = 64, KLD = DK + 8, NT = NW * 64, TQ = NW * NG;
+  constexpr int KPIECES = CH * DK / 8;
+  constexpr int KPT = (KPIECES + NT - 1) / NT;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  T* ldsK = reinterpret_cast<T*>(smem_raw);                       // [2][CH][KLD]
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 15, g = lane >> 4;
+  const int G = a.hq / a.hkv;
+  const SeqTile st = find_tile(a.cu_seq, a.batch, TQ, blockIdx.x);
+  if (!st.valid) return;
+  const int h = blockIdx.y;
+  const int coff = a.cu_cmp[st.b];
+  const int Nc = a.cu_cmp[st.b + 1] - coff;
+  int Ns = 0;
+  if (Nc >= 5) {
+    Ns = (Nc - 5 + 3) / 4 + 1;
+    if ((Ns - 1) * 4 >= Nc) --Ns;
+  }
+  Ns = min(Ns, a.max_ns);
+  if (Ns == 0) return;
+  const T* ckb = reinterpret_cast<const T*>(a.ck) + (long)coff * a.ck_row_stride + (long)h * a.ck_head_stride;
+
+  vec8_t<T> qf[NG][DK / 32];
+  float lse_r[NG][4];        // lse * log2(e) of heads 4g+i of each token; +inf removes padded rows
+  float* prow[NG];           // this token's row of window sums
+  int ns_tok[NG];            // Ns, or 0 for a token past the end of the sequence: nothing is stored
+#pragma unroll
+  for (int j = 0; j < NG; ++j) {
+    const int tok = st.t0 + wave * NG + j;
+    const int tc = tok < st.len ? tok : st.len - 1;
+    const int gc = n < G ? n : G - 1;
+    const T* qp = reinterpret_cast<const T*>(a.q) + (((long)st.start + tc) * a.hq + h * G + gc) * DK + 8 * g;
+#pragma unroll
+    for (int kk = 0; kk < DK / 32; ++kk) qf[j][kk] = load8(qp + 32 * kk);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      lse_r[j][i] = (tok < st.len && 4 * g + i < G)
+                        ? a.lse[((long)st.start + tok) * a.hq + h * G + 4 * g + i] * kLog2e
+                        : __builtin_huge_valf();
+    prow[j] = a.pooled + (((long)st.start + tc) * a.hkv + h) * a.pooled_stride;
+    ns_tok[j] = tok < st.len ? Ns : 0;
+  }
+  wait_all_loads();
+
+  float pend[NG];            // lane 63: the quad sum of the previous step's last bin
+#pragma unroll
+  for (int j = 0; j < NG; ++j) pend[j] = 0.f;
+
+  vec8_t<T> kr[KPT];
+  unsigned koff[KPT];
+#pragma unroll
+  for (int i = 0; i < KPT; ++i) {
+    const int p = tid + i * NT;
+    koff[i] = (unsigned)((p / (DK / 8)) * (int)a.ck_row_stride + (p % (DK / 8)) * 8);
+  }
+  auto gload = [&](int c0) {
+    if (c0 + CH <= Nc) {
+      const unsigned base = (unsigned)c0 * (unsigned)a.ck_row_stride;
+#pragma unroll
+      for (int i = 0; i < KPT; ++i)
+        if (KPIECES % NT == 0 || tid + i * NT < KPIECES) kr[i] = load8(ckb + (base + koff[i]));
+    } else {                                         // last step: clamp the row
+#pragma unroll
+      for (int i = 0; i < KPT; ++i) {
+        const int p = tid + i * NT;
+        if (KPIECES % NT == 0 || p < KPIECES) {
+          const int sr = min(c0 + p / (DK / 8), Nc - 1);
+          kr[i] = load8(ckb + (long)sr * a.ck_row_stride + (p % (DK / 8)) * 8);
+        }
+      }
+    }
+  };
+  auto lstore = [&](int buf) {
+    T* dk = ldsK + buf * CH * KLD;
+#pragma unroll
+    for (int i = 0; i < KPT; ++i) {
+      const int p = tid + i * NT;
+      if (KPIECES % NT == 0 || p < KPIECES) store8(dk + (p / (DK / 8)) * KLD + (p % (DK / 8)) * 8, kr[i]);
+    }
+  };
+
+  gload(0);
+  lstore(0);
+  __syncthreads();
+  const bool writer = (lane & 3) == 3;
+  const bool carrier = lane == 63;
+  int buf = 0;
+  for (int c0 = 0; c0 < Nc; c0 += CH) {
+    const bool has_next = c0 + CH < Nc;
+    if (has_next) gload(c0 + CH);
+    const T* bk = ldsK + buf * CH * KLD;
+    float v[NG][4];
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) {
+      f32x4_t sc[NG];
+#pragma unroll
+      for (int j = 0; j < NG; ++j) sc[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      const T* kp = bk + (16 * kt + n) * KLD + 8 * g;
+#pragma unroll
+      for (int kk = 0; kk < DK / 32; ++kk) {
+        const vec8_t<T> kf = load8(kp + 32 * kk);
+#pragma unroll
+        for (int j = 0; j < NG; ++j) sc[j] = mma16(qf[j][kk], kf, sc[j]);   // rows = heads, columns = keys
+      }
+#pragma unroll
+      for (int j = 0; j < NG; ++j) {
+        float e[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) e[i] = fast_exp2(fmaf(sc[j][i], kLog2e, -lse_r[j][i]));
+        v[j][kt] = (e[0] + e[1]) + (e[2] + e[3]);
+      }
+    }
+    const bool live = c0 + lane < Nc;
+    const int idx = carrier ? (c0 >> 2) - 1 : (c0 >> 2) + (lane >> 2);
+#pragma unroll
+    for (int j = 0; j < NG; ++j) {
+      float r = row_reduce_scatter4(v[j][0], v[j][1], v[j][2], v[j][3]);   // lane i: column c0 + i
+      r = live ? r : 0.f;
+      const float t2 = r + dpp_f32<0xB1>(r);               // quad_perm [1,0,3,2]
+      const float quad = t2 + dpp_f32<0x4E>(t2);           // quad_perm [2,3,0,1]
+      const float nxt = dpp_f32<0x130>(r);                 // wave_shl:1 -> column c0 + i + 1 (0 in lane 63)
+      const float first = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(r), 0));
+      const float val = carrier ? pend[j] + first : quad + nxt;
+      if (writer && idx >= 0 && idx < ns_tok[j]) prow[j][idx] = val;
+      pend[j] = quad;
+    }
+    if (has_next) lstore(buf ^ 1);
+    __syncthreads();
+    buf ^= 1;
+  }
+  if (carrier) {
+    const int b = (((Nc - 1) >> 6) << 4) + 15;             // last bin of the last step: no next column
+#pragma unroll
+    for (int j = 0; j < NG; ++j)
+      if (b < ns_tok[j]) prow[j][b] = pend[j];
+  }
+}
+
+// One wavefront per (token, kv head): window sums -> averages (ceil-mode pool, padding counted in
+// the divisor, written back over the sums, bins past the sequence's last one zeroed) and the top_n
+// bins in descending order, ties to the lower index, -1 where the sequence has fewer bins.
+template <int PER>
+__global__ void __launch_bounds__(256)
+topn_kernel(const CmpArgs a) {
+  const int lane = threadIdx.x & 63;
+  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);       // token * hkv + head
+  if (row >= (long)a.total * a.hkv) return;
+  const int tg = (int)(row / a.hkv);
+  int sb = 0;
+  {
+    int hi = a.batch;
+    while (hi - sb > 1) {
+      const int mid = (sb + hi) >> 1;
+      if (a.cu_seq[mid] <= tg) sb = mid; else hi = mid;
+    }
+  }
+  const int Nc = a.cu_cmp[sb + 1] - a.cu_cmp[sb];
+  int Ns = 0;
+  if (Nc > 0 && Nc + 2 * a.pool_p >= a.pool_k) {
+    Ns = (Nc + 2 * a.pool_p - a.pool_k + a.pool_s - 1) / a.pool_s + 1;
+    if ((Ns - 1) * a.pool_s >= Nc + a.pool_p) --Ns;
+  }
+  Ns = min(Ns, a.max_ns);
+  float* prow = a.pooled + row * a.pooled_stride;
+  float v[PER];
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    const int b = lane + 64 * k;
+    v[k] = b < Ns ? prow[b] : -1.f;
+  }
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    const int b = lane + 64 * k;
+    if (b < Ns) {
+      const int lo = b * a.pool_s - a.pool_p;
+      const int div = min(lo + a.pool_k, Nc + a.pool_p) - lo;
+      v[k] = v[k] / (float)div;
+      prow[b] = v[k];
+    } else if (b < a.max_ns) {
+      prow[b] = 0.f;
+    }
+  }
+  for (int r = 0; r < a.top_n; ++r) {
+    float best = v[0];
+    int bk = 0;
+#pragma unroll
+    for (int k = 1; k < PER; ++k)
+      if (v[k] > best) { best = v[k]; bk = k; }
+    const int bi = lane + 64 * bk;
+    long key = ((long)__float_as_int(best) << 32) | (unsigned int)(0x7fffffff - bi);
+    key = wave_max_i64(key);
+    const bool found = (int)(key >> 32) >= 0;
+    const int win = 0x7fffffff - (int)(unsigned int)key;
+    if (found && (win & 63) == lane) {
+#pragma unroll
+      for (int k = 0; k < PER; ++k)
+        if (k == (win >> 6)) v[k] = -1.f;
+    }
+    if (lane == 0) {
+      const long pos = row * a.top_n + r;
+      const int val = found ? win : -1;
+      if (a.idx64) reinterpret_cast<int64_t*>(a.indices)[pos] = val;
+      else reinterpret_cast<int32_t*>(a.indices)[pos] = val;
+    }
+  }
+}
+
 int set_smem(const void* fn, size_t bytes);
 int group_pow2(int G);
 
@@ -251,8 +450,7 @@ static int launch_select_ng(const CmpArgs& a, hipStream_t st) {
   const int TQ = NW * NG * 16 / Gp;
   const size_t smem = 2 * (size_t)CH * (DK + 8) * sizeof(T) + (size_t)TQ * a.max_ns * sizeof(float);
   if (smem > 160 * 1024) return -3;
-  const bool fast = Gp == 16 && a.pool_k == 5 && a.pool_s == 4 && a.pool_p == 0;
-  auto fn = fast ? importance_select_kernel<T, DK, NG, CH, NW, true> : importance_select_kernel<T, DK, NG, CH, NW, false>;
+  auto fn = importance_select_kernel<T, DK, NG, CH, NW>;
   const int rc = set_smem(reinterpret_cast<const void*>(fn), smem);
   if (rc) return rc;
   const int tiles = a.total / TQ + a.batch;
@@ -260,8 +458,34 @@ static int launch_select_ng(const CmpArgs& a, hipStream_t st) {
   return 0;
 }
 
+#ifndef NSA_STREAM_NW
+#define NSA_STREAM_NW 8
+#endif
+#ifndef NSA_STREAM_NG
+#define NSA_STREAM_NG 2
+#endif
+
+// Two kernels: window sums into a.pooled, then averages + top-n per (token, head).
+template <typename T, int DK>
+static int launch_select_stream(const CmpArgs& a, hipStream_t st) {
+  constexpr int NW = NSA_STREAM_NW, NG = sizeof(T) == 2 ? NSA_STREAM_NG : NSA_STREAM_NG / 2, TQ = NW * NG;
+  const size_t smem = 2 * (size_t)64 * (DK + 8) * sizeof(T);
+  auto fn = importance_stream_kernel<T, DK, NG, NW>;
+  const int rc = set_smem(reinterpret_cast<const void*>(fn), smem);
+  if (rc) return rc;
+  const int tiles = a.total / TQ + a.batch;
+  hipLaunchKernelGGL(fn, dim3(tiles, a.hkv), dim3(NW * 64), smem, st, a);
+  const int rows = (int)(((long)a.total * a.hkv + 3) / 4);
+  if (a.max_ns <= 512) hipLaunchKernelGGL(topn_kernel<8>, dim3(rows), dim3(256), 0, st, a);
+  else hipLaunchKernelGGL(topn_kernel<16>, dim3(rows), dim3(256), 0, st, a);
+  return 0;
+}
+
 template <typename T, int DK>
 static int launch_select_t(const CmpArgs& a, hipStream_t st) {
+  if (a.pooled != nullptr && a.max_ns <= 1024 && group_pow2(a.hq / a.hkv) == 16 && a.pool_k == 5 &&
+      a.pool_s == 4 && a.pool_p == 0)
+    return launch_select_stream<T, DK>(a, st);
   // four row groups per wavefront unless the per-token bins of such a tile outgrow the LDS
   constexpr int NGBIG = sizeof(T) == 2 ? 4 : 2;
   const int rc = launch_select_ng<T, DK, NGBIG>(a, st);

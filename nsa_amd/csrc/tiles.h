@@ -170,6 +170,18 @@ __device__ __forceinline__ void wave_topn(const volatile float* row, int ns, int
   }
 }
 
+// Scheduling hint for the basic block it is placed in: alternate MF matrix instructions with VA
+// vector-ALU instructions, spread evenly (one MFMA, then its share of the VALU work, ...).
+template <int MF, int VA, int I = 0>
+__device__ __forceinline__ void interleave_mfma_valu() {
+  if constexpr (I < MF) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    constexpr int share = (VA * (I + 1)) / MF - (VA * I) / MF;
+    if constexpr (share > 0) __builtin_amdgcn_sched_group_barrier(0x002, share, 0);
+    interleave_mfma_valu<MF, VA, I + 1>();
+  }
+}
+
 __device__ __forceinline__ int ilog2(int x) { return 31 - __builtin_clz(x); }
 __device__ __forceinline__ int next_pow2(int x) {
   int p = 1;

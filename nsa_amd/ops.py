@@ -125,8 +125,8 @@ def cmp_attn_select(q, ck, cvt, cu_seqlens, cu_cmp, batch, hkv, dv, ck_row_strid
     lse = torch.empty(total, hq, dtype=torch.float32, device=q.device)
     if select:
         idx = torch.empty(total, hkv, top_n, dtype=torch.int64 if idx64 else torch.int32, device=q.device)
-        if want_pooled:
-            pooled = torch.zeros(total, hkv, max(max_ns, 1), dtype=torch.float32, device=q.device)
+        # always given: with it the library runs its two-kernel schedule (window sums, then top-n)
+        pooled = torch.empty(total, hkv, max(max_ns, 1), dtype=torch.float32, device=q.device)
     lib = _lib.load()
     rc = lib.nsa_cmp_attn_select_fwd(
         _ptr(q), _ptr(ck), _ptr(cvt), _ptr(o), _ptr(idx), _ptr(pooled), _ptr(lse), _ptr(cu_seqlens), _ptr(cu_cmp),
@@ -135,7 +135,7 @@ def cmp_attn_select(q, ck, cvt, cu_seqlens, cu_cmp, batch, hkv, dv, ck_row_strid
         pool_stride, pool_pad, max(top_n, 1), max_ns, max(max_ns, 1), float(scale), int(bool(causal)),
         int(idx64), _dtype_code(q), _stream())
     _lib.check(rc, "nsa_cmp_attn_select_fwd")
-    return o, idx, pooled
+    return o, idx, (pooled if want_pooled else None)
 
 
 def cmp_attn(q, ck, cvt, cu_seqlens, cu_cmp, batch, hkv, dv, ck_row_stride, ck_head_stride, block, stride, scale,
@@ -162,13 +162,14 @@ def block_select(q, ck, lse, cu_seqlens, cu_cmp, batch, hkv, ck_row_stride, ck_h
     total, hq, dk = q.shape
     max_ns = pool_bins(max_nc, pool_kernel, pool_stride, pool_pad)
     idx = torch.empty(total, hkv, top_n, dtype=torch.int64 if idx64 else torch.int32, device=q.device)
-    pooled = torch.zeros(total, hkv, max(max_ns, 1), dtype=torch.float32, device=q.device) if want_pooled else None
+    # always given: with it the library runs its two-kernel schedule (window sums, then top-n)
+    pooled = torch.empty(total, hkv, max(max_ns, 1), dtype=torch.float32, device=q.device)
     rc = _lib.load().nsa_block_select_fwd(_ptr(q), _ptr(ck), _ptr(lse), _ptr(idx), _ptr(pooled), _ptr(cu_seqlens),
                                           _ptr(cu_cmp), batch, total, hq, hkv, dk, ck_row_stride, ck_head_stride,
                                           pool_kernel, pool_stride, pool_pad, top_n, max_ns, max(max_ns, 1),
                                           int(idx64), _dtype_code(q), _stream())
     _lib.check(rc, "nsa_block_select_fwd")
-    return idx, pooled
+    return idx, (pooled if want_pooled else None)
 
 
 def swa(q, k, vt, cu_seqlens, batch, window, scale):
