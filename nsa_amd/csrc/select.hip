@@ -415,6 +415,74 @@ topn_kernel(const CmpArgs a) {
       prow[b] = 0.f;
     }
   }
+  // lane r keeps the r-th pick; one coalesced store per row at the end (top_n <= 64)
+  int picked = -1;
+  auto emit = [&](int r, int val) { picked = lane == r ? val : picked; };
+  auto flush = [&]() {
+    if (lane < a.top_n) {
+      const long pos = row * a.top_n + lane;
+      if (a.idx64) reinterpret_cast<int64_t*>(a.indices)[pos] = picked;
+      else reinterpret_cast<int32_t*>(a.indices)[pos] = picked;
+    }
+  };
+
+  // Shortlist.  Each of the 16 lane quads holds a maximum; the smallest of those, L, has at least
+  // 16 bins at or above it, so the 16 best bins are all >= L.  Typically fewer than a tenth of the
+  // bins pass; they are compacted in index order through LDS to at most two per lane, and the
+  // selection rounds then cost a fraction of rounds over all PER bins per lane.
+  __shared__ float cand_v[4][128];
+  __shared__ int cand_i[4][128];
+  const int w = threadIdx.x >> 6;
+  int total = 129;
+  if (a.top_n <= 16) {
+    float m = v[0];
+#pragma unroll
+    for (int k = 1; k < PER; ++k) m = fmaxf(m, v[k]);
+    m = fmaxf(m, dpp_f32<0xB1>(m));
+    m = fmaxf(m, dpp_f32<0x4E>(m));                       // quad maximum (-1 for a quad without bins)
+    const float L = wave_min_f32(m);
+    total = 0;
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      const bool c = v[k] >= L && v[k] >= 0.f;
+      const unsigned long long mask = __ballot(c);
+      const int pos = total + (int)__builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32),
+                                                             __builtin_amdgcn_mbcnt_lo((unsigned)mask, 0u));
+      if (c && pos < 128) {
+        cand_v[w][pos] = v[k];
+        cand_i[w][pos] = lane + 64 * k;
+      }
+      total += __popcll(mask);
+    }
+  }
+  if (total <= 128) {
+    __builtin_amdgcn_wave_barrier();
+    float c0 = lane < total ? cand_v[w][lane] : -1.f;
+    float c1 = lane + 64 < total ? cand_v[w][lane + 64] : -1.f;
+    const int i0 = cand_i[w][lane], i1 = cand_i[w][lane + 64];
+    for (int r = 0; r < a.top_n; ++r) {
+      const bool second = c1 > c0;                        // slot 0 has the lower index: it wins ties
+      const float best = second ? c1 : c0;
+      const int bi = second ? i1 : i0;
+      const float wmax = wave_max_f32(best);
+      int win = -1;
+      if (wmax >= 0.f) {
+        const unsigned long long tied = __ballot(best == wmax);
+        if (__popcll(tied) == 1) {
+          win = __builtin_amdgcn_readlane(bi, (int)__builtin_ctzll(tied));
+        } else {
+          win = wave_min_i32(best == wmax ? bi : 0x7fffffff);
+        }
+        if (bi == win) {                                  // indices are unique: exactly one lane
+          if (second) c1 = -1.f; else c0 = -1.f;
+        }
+      }
+      emit(r, win);
+    }
+    flush();
+    return;
+  }
+
   for (int r = 0; r < a.top_n; ++r) {
     float best = v[0];
     int bk = 0;
@@ -431,13 +499,9 @@ topn_kernel(const CmpArgs a) {
       for (int k = 0; k < PER; ++k)
         if (k == (win >> 6)) v[k] = -1.f;
     }
-    if (lane == 0) {
-      const long pos = row * a.top_n + r;
-      const int val = found ? win : -1;
-      if (a.idx64) reinterpret_cast<int64_t*>(a.indices)[pos] = val;
-      else reinterpret_cast<int32_t*>(a.indices)[pos] = val;
-    }
+    emit(r, found ? win : -1);
   }
+  flush();
 }
 
 int set_smem(const void* fn, size_t bytes);
@@ -483,7 +547,7 @@ static int launch_select_stream(const CmpArgs& a, hipStream_t st) {
 
 template <typename T, int DK>
 static int launch_select_t(const CmpArgs& a, hipStream_t st) {
-  if (a.pooled != nullptr && a.max_ns <= 1024 && group_pow2(a.hq / a.hkv) == 16 && a.pool_k == 5 &&
+  if (a.pooled != nullptr && a.max_ns <= 1024 && a.top_n <= 64 && group_pow2(a.hq / a.hkv) == 16 && a.pool_k == 5 &&
       a.pool_s == 4 && a.pool_p == 0)
     return launch_select_stream<T, DK>(a, st);
   // four row groups per wavefront unless the per-token bins of such a tile outgrow the LDS

@@ -170,6 +170,30 @@ __device__ __forceinline__ void wave_topn(const volatile float* row, int ns, int
   }
 }
 
+// Wavefront reductions that end in a scalar register: four DPP steps inside each 16-lane row, two
+// row broadcasts (lane 15 -> next row, lane 31 -> upper half), then lane 63 holds the result.
+// Written as one assembly block so that every step is a single DPP-modified instruction; the
+// compiler's hazard recogniser does not see inside it, so the wait states are spelled out: two
+// between a VALU write and a DPP read of the same register, and after v_readlane before use.
+#define NSA_WAVE_REDUCE(NAME, TYPE, OPCODE)                                                       \
+  __device__ __forceinline__ TYPE NAME(TYPE x) {                                                  \
+    TYPE r;                                                                                       \
+    asm volatile("s_nop 1\n\t"                                                                    \
+                 OPCODE " %1, %1, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\ts_nop 1\n\t" \
+                 OPCODE " %1, %1, %1 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\ts_nop 1\n\t" \
+                 OPCODE " %1, %1, %1 row_half_mirror row_mask:0xf bank_mask:0xf\n\ts_nop 1\n\t"     \
+                 OPCODE " %1, %1, %1 row_mirror row_mask:0xf bank_mask:0xf\n\ts_nop 1\n\t"          \
+                 OPCODE " %1, %1, %1 row_bcast:15 row_mask:0xa bank_mask:0xf\n\ts_nop 1\n\t"        \
+                 OPCODE " %1, %1, %1 row_bcast:31 row_mask:0xc bank_mask:0xf\n\ts_nop 1\n\t"        \
+                 "v_readlane_b32 %0, %1, 63\n\ts_nop 3"                                            \
+                 : "=s"(r), "+v"(x));                                                             \
+    return r;                                                                                     \
+  }
+NSA_WAVE_REDUCE(wave_max_f32, float, "v_max_f32_dpp")
+NSA_WAVE_REDUCE(wave_min_f32, float, "v_min_f32_dpp")
+NSA_WAVE_REDUCE(wave_min_i32, int, "v_min_i32_dpp")
+#undef NSA_WAVE_REDUCE
+
 // Scheduling hint for the basic block it is placed in: alternate MF matrix instructions with VA
 // vector-ALU instructions, spread evenly (one MFMA, then its share of the VALU work, ...).
 template <int MF, int VA, int I = 0>
