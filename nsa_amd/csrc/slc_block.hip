@@ -16,6 +16,8 @@
 
 namespace nsa {
 
+int set_smem(const void* fn, size_t bytes);
+
 constexpr int kSeg = 64;          // pairs of one block handled by one wavefront
 constexpr int kBlk = 64;          // keys per selection block (4 MFMA tiles)
 
@@ -31,14 +33,15 @@ __host__ __device__ inline long align_up(long x, long a) { return (x + a - 1) / 
 
 __host__ inline long carve(const SlcArgs& a, void* base, SlcWs* ws, size_t elem) {
   const int nb = a.total / kBlk + a.batch;
+  const long nkeys = (long)a.hkv * nb;
   const long pairs = (long)a.total * a.hkv * a.top_n;
-  const int items_cap = (int)(pairs / kSeg) + a.hkv * nb + 1;
+  const int items_cap = (int)(pairs / kSeg + nkeys) + 1;
   long off = 0;
   auto take = [&](long bytes) { const long o = off; off = align_up(off + bytes, 256); return o; };
   const long o_blkbase = take((a.batch + 1) * 4L);
-  const long o_counts = take((long)a.hkv * nb * 4);
-  const long o_offsets = take((long)a.hkv * nb * 4);
-  const long o_cursor = take((long)a.hkv * nb * 4);
+  const long o_counts = take(nkeys * 4);
+  const long o_offsets = take(nkeys * 4);
+  const long o_cursor = take(nkeys * 4);
   const long o_items = take((long)items_cap * 8);
   const long o_nitems = take(4);
   const long o_list = take(pairs * 4);
@@ -115,6 +118,66 @@ slc_bucket_kernel(const SlcArgs a, SlcWs ws) {
     const int p = ws.offsets[key] + atomicAdd(&ws.cursor[key], 1);
     ws.list[p] = ((uint32_t)tg << 6) | (uint32_t)i;
     ws.slotmap[id] = p;
+  }
+}
+
+// The same two passes with the histogram of a workgroup's tokens kept in LDS: one workgroup takes
+// kBucketTok consecutive tokens of one kv head, ranks its pairs per (head, block) with LDS atomics
+// and touches the global counters once per non-empty block instead of once per pair.  The pairs of
+// a block coming from one workgroup end up next to each other in the list, so a block's query
+// gathers walk the token axis in runs.
+constexpr int kBucketTok = 512;
+constexpr int kBucketMaxBins = 32768;      // LDS histogram: 4 bytes per 64-key block of the batch
+
+template <bool FILL>
+__global__ void __launch_bounds__(1024)
+slc_bucket_lds_kernel(const SlcArgs a, SlcWs ws) {
+  extern __shared__ int hist[];
+  const int h = blockIdx.y;
+  const int t_begin = blockIdx.x * kBucketTok;
+  const int t_end = min(a.total, t_begin + kBucketTok);
+  for (int i = threadIdx.x; i < ws.nb; i += 1024) hist[i] = 0;
+  __syncthreads();
+  const int entries = (t_end - t_begin) * a.top_n;
+  auto entry = [&](int e, long& id, int& tg, int& i) -> int {      // global block of the pair, or -1
+    tg = t_begin + e / a.top_n;
+    i = e % a.top_n;
+    const long th = (long)tg * a.hkv + h;
+    id = th * a.top_n + i;
+    const int b = seq_of_token(a.cu_seq, a.batch, tg);
+    const int t = tg - a.cu_seq[b];
+    int cnt = a.top_n;
+    if (a.counts != nullptr) cnt = min(max(a.counts[th], 0), a.top_n);
+    const long idx = a.idx64 ? reinterpret_cast<const int64_t*>(a.indices)[id]
+                             : (long)reinterpret_cast<const int32_t*>(a.indices)[id];
+    const bool ok = i < cnt && idx >= 0 && idx <= t && idx * kBlk <= t;
+    return ok ? ws.blkbase[b] + (int)idx : -1;
+  };
+  for (int e = threadIdx.x; e < entries; e += 1024) {
+    long id; int tg, i;
+    const int gb = entry(e, id, tg, i);
+    if (FILL) ws.slotmap[id] = gb >= 0 ? atomicAdd(&hist[gb], 1) : -1;     // rank inside this workgroup
+    else if (gb >= 0) atomicAdd(&hist[gb], 1);
+  }
+  __syncthreads();
+  for (int bin = threadIdx.x; bin < ws.nb; bin += 1024) {
+    const int c = hist[bin];
+    if (c > 0) {
+      const int key = h * ws.nb + bin;
+      if (FILL) hist[bin] = ws.offsets[key] + atomicAdd(&ws.cursor[key], c);
+      else atomicAdd(&ws.counts[key], c);
+    }
+  }
+  if (!FILL) return;
+  __syncthreads();
+  for (int e = threadIdx.x; e < entries; e += 1024) {
+    long id; int tg, i;
+    const int gb = entry(e, id, tg, i);
+    if (gb >= 0) {
+      const int p = hist[gb] + ws.slotmap[id];
+      ws.list[p] = ((uint32_t)tg << 6) | (uint32_t)i;
+      ws.slotmap[id] = p;
+    }
   }
 }
 
@@ -280,7 +343,10 @@ slc_block_kernel(const SlcArgs a, const SlcWs ws) {
 
 __device__ __forceinline__ float gate_of(float x, int act) { return act == 1 ? 1.0f / (1.0f + __expf(-x)) : x; }
 
-template <typename T, int DV>
+// One thread per (token, q head, 8 output channels).  TOPN > 0: the slot map of the token is read
+// with vector loads and all of its partials are requested before any is used, so a thread keeps
+// up to TOPN 16-byte loads in flight; TOPN = 0: any top_n, one partial at a time.
+template <typename T, int DV, int TOPN>
 __global__ void __launch_bounds__(256)
 slc_merge_kernel(const SlcArgs a, const SlcWs ws) {
   constexpr int PPR = DV / 8;                                     // 8-channel pieces per output row
@@ -295,23 +361,51 @@ slc_merge_kernel(const SlcArgs a, const SlcWs ws) {
   const long base = (tg * a.hkv + h) * a.top_n;
   const float c_attn = a.scale * kLog2e;
   const T* pob = reinterpret_cast<const T*>(ws.po);
-  float M = kNegInf, den = 0.f, acc[8];
+  float den = 0.f, acc[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-#pragma unroll 8
-  for (int i = 0; i < a.top_n; ++i) {
-    const int p = ws.slotmap[base + i];
-    if (p < 0) continue;
-    const float m = ws.ml[((long)p * 2) * 16 + n];
-    const float l = ws.ml[((long)p * 2 + 1) * 16 + n];
-    const vec8_t<T> o = load8(pob + ((long)p * 16 + n) * DV + pc * 8);
-    const float m_new = fmaxf(M, m);
-    const float r_old = fast_exp2((M - m_new) * c_attn);          // 0 for the first partial
-    const float w = fast_exp2((m - m_new) * c_attn) * l;
-    den = den * r_old + w;
+  if constexpr (TOPN > 0) {
+    int ps[TOPN];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] = acc[e] * r_old + w * (float)o[e];
-    M = m_new;
+    for (int i = 0; i < TOPN / 4; ++i) {
+      const int4 q4 = *reinterpret_cast<const int4*>(ws.slotmap + base + 4 * i);
+      ps[4 * i] = q4.x; ps[4 * i + 1] = q4.y; ps[4 * i + 2] = q4.z; ps[4 * i + 3] = q4.w;
+    }
+    float m[TOPN], l[TOPN];
+    vec8_t<T> o[TOPN];
+#pragma unroll
+    for (int i = 0; i < TOPN; ++i) {
+      const long p = ps[i] < 0 ? 0 : ps[i];                       // an unused slot re-reads pair 0, weight 0
+      m[i] = ws.ml[(p * 2) * 16 + n];
+      l[i] = ws.ml[(p * 2 + 1) * 16 + n];
+      o[i] = load8(pob + (p * 16 + n) * DV + pc * 8);
+    }
+    float M = kNegInf;
+#pragma unroll
+    for (int i = 0; i < TOPN; ++i) M = fmaxf(M, ps[i] < 0 ? kNegInf : m[i]);
+#pragma unroll
+    for (int i = 0; i < TOPN; ++i) {
+      const float w = ps[i] < 0 ? 0.f : fast_exp2((m[i] - M) * c_attn) * l[i];
+      den += w;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = fmaf(w, (float)o[i][e], acc[e]);
+    }
+  } else {
+    float M = kNegInf;
+    for (int i = 0; i < a.top_n; ++i) {
+      const int p = ws.slotmap[base + i];
+      if (p < 0) continue;
+      const float m = ws.ml[((long)p * 2) * 16 + n];
+      const float l = ws.ml[((long)p * 2 + 1) * 16 + n];
+      const vec8_t<T> o = load8(pob + ((long)p * 16 + n) * DV + pc * 8);
+      const float m_new = fmaxf(M, m);
+      const float r_old = fast_exp2((M - m_new) * c_attn);        // 0 for the first partial
+      const float w = fast_exp2((m - m_new) * c_attn) * l;
+      den = den * r_old + w;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = acc[e] * r_old + w * (float)o[e];
+      M = m_new;
+    }
   }
   const float inv = den > 0.f ? 1.0f / den : 0.f;
   const T* gs = reinterpret_cast<const T*>(a.g_slc);
@@ -342,13 +436,28 @@ template <typename T, int DK, int DV>
 static int launch_block_t(const SlcArgs& a, const SlcWs& ws, hipStream_t st) {
   const long pairs = ws.pairs_cap;
   hipLaunchKernelGGL(slc_prep_kernel, dim3(1), dim3(256), 0, st, a.cu_seq, a.batch, ws, a.hkv);
-  const int gb = (int)((pairs + 255) / 256);
-  hipLaunchKernelGGL(slc_bucket_kernel<false>, dim3(gb), dim3(256), 0, st, a, ws);
-  hipLaunchKernelGGL(slc_scan_kernel, dim3(1), dim3(1024), 0, st, ws, a.hkv);
-  hipLaunchKernelGGL(slc_bucket_kernel<true>, dim3(gb), dim3(256), 0, st, a, ws);
+  if (ws.nb <= kBucketMaxBins) {
+    const dim3 grid((a.total + kBucketTok - 1) / kBucketTok, a.hkv);
+    const size_t smem = (size_t)ws.nb * sizeof(int);
+    if (smem > 64 * 1024) {
+      int rc = set_smem(reinterpret_cast<const void*>(slc_bucket_lds_kernel<false>), smem);
+      if (rc == 0) rc = set_smem(reinterpret_cast<const void*>(slc_bucket_lds_kernel<true>), smem);
+      if (rc) return rc;
+    }
+    hipLaunchKernelGGL(slc_bucket_lds_kernel<false>, grid, dim3(1024), smem, st, a, ws);
+    hipLaunchKernelGGL(slc_scan_kernel, dim3(1), dim3(1024), 0, st, ws, a.hkv);
+    hipLaunchKernelGGL(slc_bucket_lds_kernel<true>, grid, dim3(1024), smem, st, a, ws);
+  } else {
+    const int gb = (int)((pairs + 255) / 256);
+    hipLaunchKernelGGL(slc_bucket_kernel<false>, dim3(gb), dim3(256), 0, st, a, ws);
+    hipLaunchKernelGGL(slc_scan_kernel, dim3(1), dim3(1024), 0, st, ws, a.hkv);
+    hipLaunchKernelGGL(slc_bucket_kernel<true>, dim3(gb), dim3(256), 0, st, a, ws);
+  }
   hipLaunchKernelGGL((slc_block_kernel<T, DK, DV>), dim3((ws.items_cap + 3) / 4), dim3(256), 0, st, a, ws);
   const long threads = (long)a.total * a.hq * (DV / 8);
-  hipLaunchKernelGGL((slc_merge_kernel<T, DV>), dim3((int)((threads + 255) / 256)), dim3(256), 0, st, a, ws);
+  const dim3 mg((int)((threads + 255) / 256));
+  if (a.top_n == 16) hipLaunchKernelGGL((slc_merge_kernel<T, DV, 16>), mg, dim3(256), 0, st, a, ws);
+  else hipLaunchKernelGGL((slc_merge_kernel<T, DV, 0>), mg, dim3(256), 0, st, a, ws);
   return 0;
 }
 
