@@ -229,7 +229,7 @@ __device__ __forceinline__ float row_reduce_scatter4(float v0, float v1, float v
 // its quad to the next step, where it is completed with that step's first column.  Every bin is
 // written exactly once, 64 contiguous bytes per token and step, with no atomics.
 template <typename T, int DK, int NG, int NW>
-__global__ void __launch_bounds__(NW * 64)
+__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(4, 4)))
 importance_stream_kernel(const CmpArgs a) {
   constexpr int CH = 64, KLD = DK + 8, NT = NW * 64, TQ = NW * NG;
   constexpr int KPIECES = CH * DK / 8;
@@ -319,32 +319,16 @@ importance_stream_kernel(const CmpArgs a) {
   __syncthreads();
   const bool writer = (lane & 3) == 3;
   const bool carrier = lane == 63;
-  int buf = 0;
-  for (int c0 = 0; c0 < Nc; c0 += CH) {
-    const bool has_next = c0 + CH < Nc;
-    if (has_next) gload(c0 + CH);
-    const T* bk = ldsK + buf * CH * KLD;
-    float v[NG][4];
+  // Software pipeline inside every wavefront: while the matrix unit multiplies score tile i, the
+  // vector ALU exponentiates tile i-1 (kept in `sp`), one or two operations after each MFMA.
+  // Without this the wavefronts of a SIMD drift into lockstep -- all multiplying, then all
+  // exponentiating -- and the two units take turns instead of working at the same time.
+  constexpr int NK = DK / 32, SLOTS = NK * NG, NOPS = NG * 7;
+  f32x4_t sp[NG];
+  float v[NG][4], e[NG][4], ea[NG], eb[NG];
 #pragma unroll
-    for (int kt = 0; kt < 4; ++kt) {
-      f32x4_t sc[NG];
-#pragma unroll
-      for (int j = 0; j < NG; ++j) sc[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-      const T* kp = bk + (16 * kt + n) * KLD + 8 * g;
-#pragma unroll
-      for (int kk = 0; kk < DK / 32; ++kk) {
-        const vec8_t<T> kf = load8(kp + 32 * kk);
-#pragma unroll
-        for (int j = 0; j < NG; ++j) sc[j] = mma16(qf[j][kk], kf, sc[j]);   // rows = heads, columns = keys
-      }
-#pragma unroll
-      for (int j = 0; j < NG; ++j) {
-        float e[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) e[i] = fast_exp2(fmaf(sc[j][i], kLog2e, -lse_r[j][i]));
-        v[j][kt] = (e[0] + e[1]) + (e[2] + e[3]);
-      }
-    }
+  for (int j = 0; j < NG; ++j) sp[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  auto pool_store = [&](int c0) {          // window sums of the step that started at column c0
     const bool live = c0 + lane < Nc;
     const int idx = carrier ? (c0 >> 2) - 1 : (c0 >> 2) + (lane >> 2);
 #pragma unroll
@@ -359,10 +343,53 @@ importance_stream_kernel(const CmpArgs a) {
       if (writer && idx >= 0 && idx < ns_tok[j]) prow[j][idx] = val;
       pend[j] = quad;
     }
+  };
+  // operation `op` of the exponentiation of tile `tp` held in sp: per group 4 x (fma, exp), 3 adds
+  auto exp_op = [&](int op, int tp) {
+    const int r = op / NG, j = op % NG;
+    // the empty asm pins the value to this point of the program: without it the optimiser sinks
+    // the whole computation down to its first use, behind all the MFMAs
+    if (r < 4) { e[j][r] = fast_exp2(fmaf(sp[j][r], kLog2e, -lse_r[j][r])); asm volatile("" : "+v"(e[j][r])); }
+    else if (r == 4) { ea[j] = e[j][0] + e[j][1]; asm volatile("" : "+v"(ea[j])); }
+    else if (r == 5) { eb[j] = e[j][2] + e[j][3]; asm volatile("" : "+v"(eb[j])); }
+    else { v[j][tp] = ea[j] + eb[j]; asm volatile("" : "+v"(v[j][tp])); }
+  };
+  int buf = 0;
+  for (int c0 = 0; c0 < Nc; c0 += CH) {
+    const bool has_next = c0 + CH < Nc;
+    if (has_next) gload(c0 + CH);
+    const T* bk = ldsK + buf * CH * KLD;
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) {
+      f32x4_t sc[NG];
+#pragma unroll
+      for (int j = 0; j < NG; ++j) sc[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      const T* kp = bk + (16 * kt + n) * KLD + 8 * g;
+      vec8_t<T> kf = load8(kp);
+#pragma unroll
+      for (int kk = 0; kk < NK; ++kk) {
+        const vec8_t<T> kcur = kf;
+        if (kk + 1 < NK) kf = load8(kp + 32 * (kk + 1));
+#pragma unroll
+        for (int j = 0; j < NG; ++j) {
+          sc[j] = mma16(qf[j][kk], kcur, sc[j]);            // rows = heads, columns = keys
+          const int slot = kk * NG + j;
+#pragma unroll
+          for (int op = slot * NOPS / SLOTS; op < (slot + 1) * NOPS / SLOTS; ++op) exp_op(op, (kt + 3) & 3);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      if (kt == 0 && c0 > 0) pool_store(c0 - CH);
+#pragma unroll
+      for (int j = 0; j < NG; ++j) sp[j] = sc[j];
+    }
     if (has_next) lstore(buf ^ 1);
     __syncthreads();
     buf ^= 1;
   }
+#pragma unroll
+  for (int op = 0; op < NOPS; ++op) exp_op(op, 3);
+  pool_store(((Nc - 1) >> 6) << 6);
   if (carrier) {
     const int b = (((Nc - 1) >> 6) << 4) + 15;             // last bin of the last step: no next column
 #pragma unroll
