@@ -68,7 +68,11 @@ int nsa_transpose_fwd(const void* x, void* out, const int32_t* cu, int batch, in
  *   q [total, hq, dk]; ck rows at ck + (cu_cmp[b] + c)*ck_row_stride + h*ck_head_stride (dk elements);
  *   cvt transposed [hkv][dv][cvt_cols] over cu_cmp; o [total, hq, dv];
  *   indices [total, hkv, top_n] int32 or int64 (idx64), descending score, -1 where fewer bins exist;
- *   NULL skips the selection;  pooled (optional, float) [total, hkv, pooled_stride] block scores;
+ *   NULL skips the selection;  pooled (optional, float) [total, hkv, pooled_stride] receives the
+ *   pooled block scores (bins past a sequence's last one up to max_ns are zeroed).  Pass it even when
+ *   the scores are not wanted: with it (and a GQA group of 9..16 heads, pooling 5/4/0, max_ns <= 1024,
+ *   top_n <= 64) the selection runs as two lean kernels that use it as their hand-over buffer, without
+ *   it as one slower kernel that keeps the bins in LDS;
  *   lse (float) [total, hq] receives the log-sum-exp of the raw scores q.ck over all compressed rows
  *   (the reference's M without its mask and scale); required when indices is given.
  *   Compressed row c of a sequence is visible to token t iff c*stride + block <= t (causal != 0;
