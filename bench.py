@@ -219,9 +219,12 @@ def main():
     # Per-stage credited flops.  block_select carries none (its score tiles are the uncredited
     # non-causal importance pass); slc_combine is a chain of kernels (bucket, block, merge), the other
     # stages are one kernel each, so the single dominant kernel is the longest of cmp_attn / swa.
-    stage_flops = {"cmp_attn": fl["cmp"], "swa": fl["swa"], "slc_combine": fl["slc"]}
+    # With the fused schedule the selected branch is "slc_blocks" (bucket + per-block partials) and the
+    # window branch "swa_combine" (window attention + merge of the partials + gated sum).
+    stage_flops = {"cmp_attn": fl["cmp"], "swa": fl["swa"], "slc_combine": fl["slc"],
+                   "swa_combine": fl["swa"], "slc_blocks": fl["slc"]}
     stage_tflops = {n: stage_flops[n] / (stage_ms[n] * 1e-3) / 1e12 for n in stage_flops if n in stage_ms}
-    dom = max(("cmp_attn", "swa"), key=lambda n: stage_ms.get(n, 0.0))
+    dom = max(("cmp_attn", "swa", "swa_combine"), key=lambda n: stage_ms.get(n, 0.0))
     dom_tflops = stage_tflops[dom]
     # HBM bytes per launch of that kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE (profiles/), only
     # recorded for the default workload

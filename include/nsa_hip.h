@@ -121,6 +121,29 @@ int nsa_slc_combine_fwd(const void* q, const void* k, const void* vt, const void
                         int vt_cols, int top_n, int block_size, float scale, int idx64, int gate_act,
                         int dtype, void* workspace, int64_t workspace_bytes, nsa_stream_t stream);
 
+/* The block-major selected attention in two steps, with the merge folded into the sliding-window
+ * kernel so that the window branch never goes to memory.  Same tensors, meaning and workspace
+ * (nsa_slc_workspace_bytes, required here) as nsa_slc_combine_fwd; stands behind the same reference
+ * lines plus the window loop nsa/selection_attn.py:483-517.
+ *   nsa_slc_partials_fwd   buckets the (token, pick) pairs by K/V block and leaves one partial
+ *                          softmax state per pair in the workspace;
+ *   nsa_swa_merge_fwd      sliding-window attention whose epilogue merges those partials and writes
+ *                          out = act(g_slc)*o_slc + act(g_swa)*o_swa + act(g_cmp)*o_cmp (o_cmp may be
+ *                          NULL).  Must follow nsa_slc_partials_fwd on the same stream with the same
+ *                          sizes; the workspace is only read (its slot map tells which picks have
+ *                          a partial).
+ * bf16, 64-key selection blocks; other shapes return NSA_ERR_UNSUPPORTED (use nsa_swa_fwd +
+ * nsa_slc_combine_fwd). */
+int nsa_slc_partials_fwd(const void* q, const void* k, const void* vt, const void* indices, const int32_t* counts,
+                         const int32_t* cu_seqlens, int batch, int total, int hq, int hkv, int dk, int dv,
+                         int vt_cols, int top_n, int block_size, float scale, int idx64, int dtype, void* workspace,
+                         int64_t workspace_bytes, nsa_stream_t stream);
+int nsa_swa_merge_fwd(const void* q, const void* k, const void* vt, const void* g_slc, const void* g_swa,
+                      const void* g_cmp, int64_t gate_stride, const void* o_cmp, void* out,
+                      const int32_t* cu_seqlens, int batch, int total, int hq, int hkv, int dk, int dv, int vt_cols,
+                      int window, int top_n, int block_size, float scale, int gate_act, int dtype,
+                      const void* workspace, int64_t workspace_bytes, nsa_stream_t stream);
+
 /* Bytes of the optional workspace of nsa_slc_combine_fwd; 0 when the shape has no block-major path
  * (bf16, selection blocks of 64 keys only). */
 int64_t nsa_slc_workspace_bytes(int total, int batch, int hkv, int dk, int dv, int top_n, int block_size, int dtype);

@@ -33,6 +33,8 @@ SIGNATURES = {
     "nsa_slc_combine_fwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _L, _P, _P, _P, _P, _I, _I, _I, _I, _I,
                                  _I, _I, _I, _I, _F, _I, _I, _I, _P, _L, _P]),
     "nsa_slc_workspace_bytes": (_L, [_I, _I, _I, _I, _I, _I, _I, _I]),
+    "nsa_slc_partials_fwd": (_I, [_P] * 6 + [_I] * 9 + [_F, _I, _I, _P, _L, _P]),
+    "nsa_swa_merge_fwd": (_I, [_P] * 6 + [_L, _P, _P, _P] + [_I] * 10 + [_F, _I, _I, _P, _L, _P]),
     "nsa_decode_max_compressed": (_I, []),
     "nsa_decode_step": (_I, [_P] * 9 + [_I] * 15 + [_F, _I, _I, _P]),
     "nsa_decode_append": (_I, [_P] * 7 + [_I] * 9 + [_P]),

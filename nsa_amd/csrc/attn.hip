@@ -17,7 +17,7 @@
 //
 // The selected-block branch (one wavefront per row group, blocks read straight from global memory
 // in fragment layout) and the gated combine of the three branches live here as well.
-#include "tiles.h"
+#include "slc_merge.h"
 
 namespace nsa {
 
@@ -28,9 +28,14 @@ struct StreamParams {
   long k_row_stride, k_head_stride; int vt_cols;
   int block, stride, window, causal;
   float scale;
+  MergeArgs mg;      // MERGE kernels only: the selected-attention partials and the other branches
 };
 
-template <typename T, int DK, int DV, int NG, int CH, int NW, bool CMP>
+// MERGE (sliding window only): 0 = write the branch output; otherwise the epilogue merges the
+// block-major selected-attention partials of its rows, applies the gates, adds the compressed
+// branch and writes the final output, so the window result never goes to memory (1 = any top_n,
+// 16 = top_n of exactly 16 with all partial loads in flight).
+template <typename T, int DK, int DV, int NG, int CH, int NW, bool CMP, int MERGE = 0>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 stream_attn_kernel(const StreamParams a) {
   constexpr int KLD = DK + 8, VLD = CH + 8, ROWS = NW * NG * 16, NT = NW * 64;
@@ -284,8 +289,17 @@ stream_attn_kernel(const StreamParams a) {
         const int r = e / PIECES, pc = e % PIECES;
         if (16 * PIECES % 64 == 0 || r < 16) {
           const RowMap rr = map_row(st.t0, gi, r, lgp, G, st.len);
-          if (rr.valid)
-            store8(ob + (((long)st.start + rr.tok) * a.hq + h * G + rr.gidx) * DV + pc * 8, load8(stage + r * OLD + pc * 8));
+          if (rr.valid) {
+            const long tg = (long)st.start + rr.tok;
+            const long orow = tg * a.hq + h * G + rr.gidx;
+            const vec8_t<T> piece = load8(stage + r * OLD + pc * 8);
+            if constexpr (MERGE == 0) {
+              store8(ob + orow * DV + pc * 8, piece);
+            } else {
+              const vec8_t<T> res = merge_piece<T, DV, (MERGE == 16 ? 16 : 0)>(a.mg, tg, h, rr.gidx, orow, pc, true, piece);
+              store8(reinterpret_cast<T*>(a.mg.out) + orow * DV + pc * 8, res);
+            }
+          }
         }
       }
     }
@@ -484,13 +498,13 @@ int group_pow2(int G) {
   return p;
 }
 
-template <typename T, int DK, int DV, bool CMP>
+template <typename T, int DK, int DV, bool CMP, int MERGE = 0>
 static int launch_stream_t(const StreamParams& a, int total, hipStream_t st) {
   constexpr int NG = StreamTile<T>::NG, CH = StreamTile<T>::CH, NW = StreamTile<T>::NW;
   const int Gp = group_pow2(a.hq / a.hkv);
   const int TQ = NW * NG * 16 / Gp;
   const size_t smem = 2 * ((size_t)CH * (DK + 8) + (size_t)DV * (CH + 8)) * sizeof(T);
-  auto fn = stream_attn_kernel<T, DK, DV, NG, CH, NW, CMP>;
+  auto fn = stream_attn_kernel<T, DK, DV, NG, CH, NW, CMP, MERGE>;
   const int rc = set_smem(reinterpret_cast<const void*>(fn), smem);
   if (rc) return rc;
   const int tiles = total / TQ + a.batch;
@@ -501,15 +515,23 @@ static int launch_stream_t(const StreamParams& a, int total, hipStream_t st) {
 template <typename T, int DK, int DV>
 static int launch_cmp_t(const CmpArgs& a, hipStream_t st) {
   StreamParams p{a.q, a.ck, a.cvt, a.o, a.lse, a.cu_seq, a.cu_cmp, a.batch, a.hq, a.hkv, a.ck_row_stride,
-                 a.ck_head_stride, a.cvt_cols, a.block, a.stride, 0, a.causal, a.scale};
+                 a.ck_head_stride, a.cvt_cols, a.block, a.stride, 0, a.causal, a.scale, MergeArgs{}};
   return launch_stream_t<T, DK, DV, true>(p, a.total, st);
 }
 
 template <typename T, int DK, int DV>
 static int launch_swa_t(const SwaArgs& a, hipStream_t st) {
   StreamParams p{a.q, a.k, a.vt, a.o, nullptr, a.cu_seq, a.cu_seq, a.batch, a.hq, a.hkv, (long)a.hkv * DK,
-                 (long)DK, a.vt_cols, 0, 0, a.window, 1, a.scale};
+                 (long)DK, a.vt_cols, 0, 0, a.window, 1, a.scale, MergeArgs{}};
   return launch_stream_t<T, DK, DV, false>(p, a.total, st);
+}
+
+template <int DK, int DV>
+static int launch_swa_merge_t(const SwaArgs& a, const MergeArgs& m, hipStream_t st) {
+  StreamParams p{a.q, a.k, a.vt, nullptr, nullptr, a.cu_seq, a.cu_seq, a.batch, a.hq, a.hkv, (long)a.hkv * DK,
+                 (long)DK, a.vt_cols, 0, 0, a.window, 1, a.scale, m};
+  if (m.top_n == 16) return launch_stream_t<bf16_t, DK, DV, false, 16>(p, a.total, st);
+  return launch_stream_t<bf16_t, DK, DV, false, 1>(p, a.total, st);
 }
 
 template <typename T, int DK, int DV>
@@ -546,6 +568,15 @@ static int launch_slc_t(const SlcArgs& a, hipStream_t st) {
 
 int launch_cmp_attn(const CmpArgs& a, hipStream_t st) { NSA_DISPATCH(launch_cmp_t, a, st); }
 int launch_swa(const SwaArgs& a, hipStream_t st) { NSA_DISPATCH(launch_swa_t, a, st); }
+int launch_swa_merge(const SwaArgs& a, const MergeArgs& m, hipStream_t st) {
+  if (a.dtype != 0) return -2;
+  switch (a.dk * 1000 + a.dv) {
+    case 64064: return launch_swa_merge_t<64, 64>(a, m, st);
+    case 128128: return launch_swa_merge_t<128, 128>(a, m, st);
+    case 192128: return launch_swa_merge_t<192, 128>(a, m, st);
+    default: return -2;
+  }
+}
 int launch_slc_combine(const SlcArgs& a, hipStream_t st) {
   // block-major path when the caller lent a large enough workspace and the shape qualifies
   if (a.workspace != nullptr && slc_block_major_ok(a) && a.workspace_bytes >= slc_workspace_bytes(a))

@@ -187,6 +187,55 @@ int nsa_slc_combine_fwd(const void* q, const void* k, const void* vt, const void
   return finish(nsa::launch_slc_combine(a, stream), "slc_combine");
 }
 
+static int slc_common_checks(const char* what, const void* q, const void* k, const void* vt, const int32_t* cu_seqlens,
+                             int batch, int total, int hq, int hkv, int dk, int dv, int vt_cols, int top_n,
+                             int block_size, float scale, int dtype, const void* workspace, int64_t workspace_bytes) {
+  if (!q || !k || !vt || !cu_seqlens || !workspace) return fail(NSA_ERR_INVALID, "%s: null pointer", what);
+  if (batch <= 0 || total <= 0) return fail(NSA_ERR_INVALID, "%s: sizes must be positive", what);
+  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "%s: bad dtype", what);
+  if (int rc = check_heads(what, hq, hkv, dk, dv)) return rc;
+  if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "%s: scale must be positive", what);
+  if (vt_cols % 64 != 0 || vt_cols < nsa_transposed_cols(total, batch)) return fail(NSA_ERR_INVALID, "%s: vt_cols too small or not a multiple of 64", what);
+  if (!aligned16(q) || !aligned16(k) || !aligned16(vt) || !aligned16(workspace)) return fail(NSA_ERR_INVALID, "%s: pointers must be 16-byte aligned", what);
+  const int64_t need = nsa_slc_workspace_bytes(total, batch, hkv, dk, dv, top_n, block_size, dtype);
+  if (need == 0) return fail(NSA_ERR_UNSUPPORTED, "%s: the block-major schedule needs bf16, 64-key blocks, top_n <= 64 and (dk,dv) in (64,64),(128,128),(192,128)", what);
+  if (workspace_bytes < need) return fail(NSA_ERR_INVALID, "%s: workspace smaller than nsa_slc_workspace_bytes", what);
+  return 0;
+}
+
+int nsa_slc_partials_fwd(const void* q, const void* k, const void* vt, const void* indices, const int32_t* counts,
+                         const int32_t* cu_seqlens, int batch, int total, int hq, int hkv, int dk, int dv,
+                         int vt_cols, int top_n, int block_size, float scale, int idx64, int dtype, void* workspace,
+                         int64_t workspace_bytes, nsa_stream_t stream) {
+  if (!indices) return fail(NSA_ERR_INVALID, "slc_partials: null pointer");
+  if (int rc = slc_common_checks("slc_partials", q, k, vt, cu_seqlens, batch, total, hq, hkv, dk, dv, vt_cols, top_n,
+                                 block_size, scale, dtype, workspace, workspace_bytes)) return rc;
+  nsa::SlcArgs a{q, k, vt, indices, counts, nullptr, nullptr, nullptr, 1, nullptr, nullptr, nullptr, cu_seqlens,
+                 batch, total, hq, hkv, dk, dv, vt_cols, top_n, block_size, scale, idx64, 0, dtype,
+                 workspace, (long)workspace_bytes};
+  return finish(nsa::launch_slc_partials(a, workspace, stream), "slc_partials");
+}
+
+int nsa_swa_merge_fwd(const void* q, const void* k, const void* vt, const void* g_slc, const void* g_swa,
+                      const void* g_cmp, int64_t gate_stride, const void* o_cmp, void* out,
+                      const int32_t* cu_seqlens, int batch, int total, int hq, int hkv, int dk, int dv, int vt_cols,
+                      int window, int top_n, int block_size, float scale, int gate_act, int dtype,
+                      const void* workspace, int64_t workspace_bytes, nsa_stream_t stream) {
+  if (!out) return fail(NSA_ERR_INVALID, "swa_merge: null pointer");
+  if (window <= 0) return fail(NSA_ERR_INVALID, "swa_merge: window must be positive");
+  if (gate_act != NSA_GATE_IDENTITY && gate_act != NSA_GATE_SIGMOID) return fail(NSA_ERR_INVALID, "swa_merge: bad gate activation");
+  if (int rc = slc_common_checks("swa_merge", q, k, vt, cu_seqlens, batch, total, hq, hkv, dk, dv, vt_cols, top_n,
+                                 block_size, scale, dtype, workspace, workspace_bytes)) return rc;
+  if (!aligned16(out) || (o_cmp && !aligned16(o_cmp))) return fail(NSA_ERR_INVALID, "swa_merge: pointers must be 16-byte aligned");
+  // the picks themselves are not needed here: the workspace's slot map says which have a partial
+  nsa::SlcArgs sa{q, k, vt, nullptr, nullptr, g_slc, g_swa, g_cmp, (long)gate_stride, nullptr, o_cmp, out, cu_seqlens,
+                  batch, total, hq, hkv, dk, dv, vt_cols, top_n, block_size, scale, 0, gate_act, dtype,
+                  const_cast<void*>(workspace), (long)workspace_bytes};
+  const nsa::MergeArgs m = nsa::slc_merge_args(sa, const_cast<void*>(workspace));
+  nsa::SwaArgs a{q, k, vt, nullptr, cu_seqlens, batch, total, hq, hkv, dk, dv, vt_cols, window, scale, dtype};
+  return finish(nsa::launch_swa_merge(a, m, stream), "swa_merge");
+}
+
 int nsa_decode_max_compressed(void) { return nsa::decode_max_nc(); }
 
 int nsa_decode_step(const void* q, const void* k_cache, const void* v_cache_t, const void* ck_cache,

@@ -39,6 +39,15 @@ struct SlcArgs {
   void* workspace; long workspace_bytes;
 };
 
+// Where the merge of the block-major partial results finds its inputs (all device pointers; the
+// first three live inside the selected-attention workspace).
+struct MergeArgs {
+  const int* slotmap; const float* ml; const void* po;
+  const void* g_slc; const void* g_swa; const void* g_cmp; long gate_stride;
+  const void* o_cmp; void* out;
+  int top_n, hq, hkv, gate_act; float scale;
+};
+
 struct DecodeArgs {
   const void* q; const void* k_cache; const void* v_cache_t; const void* ck_cache; const void* cv_cache_t;
   const int32_t* ctx_lens; const void* gates; void* out; int32_t* indices;
@@ -56,6 +65,9 @@ int launch_slc_combine(const SlcArgs& a, hipStream_t st);
 long slc_workspace_bytes(const SlcArgs& a);
 bool slc_block_major_ok(const SlcArgs& a);
 int launch_slc_block_major(const SlcArgs& a, void* workspace, hipStream_t st);
+int launch_slc_partials(const SlcArgs& a, void* workspace, hipStream_t st);
+MergeArgs slc_merge_args(const SlcArgs& a, void* workspace);
+int launch_swa_merge(const SwaArgs& a, const MergeArgs& m, hipStream_t st);
 int launch_decode(const DecodeArgs& a, hipStream_t st);
 int launch_decode_append(const void* k_new, const void* v_new, void* k_cache, void* v_cache_t, void* ck_cache,
                          void* cv_cache_t, const int32_t* pos, int batch, int hkv, int dk, int dv, int ctx_cap,

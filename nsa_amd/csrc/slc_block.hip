@@ -5,14 +5,14 @@
 // through its vector L1.  Here the loop is inverted: the (token, pick) pairs are bucketed by
 // (kv head, block); a wavefront loads one K/V block into registers as MFMA fragments ONCE and then
 // streams the queries that picked it (6 KB each), writing one normalised partial result
-// (o / l in bf16, plus max and denominator in fp32) per pair.  A second kernel merges the <= top_n
-// partials of every token, applies the gates and adds the other two branches.  Traffic per pair
-// drops from 40 KB to ~10 KB (query in, partial out) + 4 KB (partial back in).
+// (o / l in bf16, plus max and denominator in fp32) per pair, in pair order.  The merge of the <= top_n partials of every token, the gates and the sum with the other
+// two branches happen either in slc_merge_kernel or in the sliding-window kernel's epilogue.  Traffic
+// per pair drops from 40 KB to ~10 KB (query in, partial out) + 4 KB (partial back in).
 //
 // Workspace layout (caller allocated, nsa_slc_workspace_bytes): block bases per sequence, pair counts /
 // offsets / cursors per (head, block), work items (head, block, segment of 64 pairs), the bucketed
 // pair list, a slot map (token, head, pick) -> pair, and the partial results.
-#include "tiles.h"
+#include "slc_merge.h"
 
 namespace nsa {
 
@@ -341,14 +341,10 @@ slc_block_kernel(const SlcArgs a, const SlcWs ws) {
 
 // ---- merge the partials of every token, gate, add the other branches ---------------------------
 
-__device__ __forceinline__ float gate_of(float x, int act) { return act == 1 ? 1.0f / (1.0f + __expf(-x)) : x; }
-
-// One thread per (token, q head, 8 output channels).  TOPN > 0: the slot map of the token is read
-// with vector loads and all of its partials are requested before any is used, so a thread keeps
-// up to TOPN 16-byte loads in flight; TOPN = 0: any top_n, one partial at a time.
+// One thread per (token, q head, 8 output channels).
 template <typename T, int DV, int TOPN>
 __global__ void __launch_bounds__(256)
-slc_merge_kernel(const SlcArgs a, const SlcWs ws) {
+slc_merge_kernel(const SlcArgs a, const MergeArgs m) {
   constexpr int PPR = DV / 8;                                     // 8-channel pieces per output row
   const long id = (long)blockIdx.x * 256 + threadIdx.x;
   if (id >= (long)a.total * a.hq * PPR) return;
@@ -357,83 +353,21 @@ slc_merge_kernel(const SlcArgs a, const SlcWs ws) {
   const int hq_i = (int)(row % a.hq);
   const long tg = row / a.hq;
   const int G = a.hq / a.hkv;
-  const int h = hq_i / G, n = hq_i % G;
-  const long base = (tg * a.hkv + h) * a.top_n;
-  const float c_attn = a.scale * kLog2e;
-  const T* pob = reinterpret_cast<const T*>(ws.po);
-  float den = 0.f, acc[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-  if constexpr (TOPN > 0) {
-    int ps[TOPN];
-#pragma unroll
-    for (int i = 0; i < TOPN / 4; ++i) {
-      const int4 q4 = *reinterpret_cast<const int4*>(ws.slotmap + base + 4 * i);
-      ps[4 * i] = q4.x; ps[4 * i + 1] = q4.y; ps[4 * i + 2] = q4.z; ps[4 * i + 3] = q4.w;
-    }
-    float m[TOPN], l[TOPN];
-    vec8_t<T> o[TOPN];
-#pragma unroll
-    for (int i = 0; i < TOPN; ++i) {
-      const long p = ps[i] < 0 ? 0 : ps[i];                       // an unused slot re-reads pair 0, weight 0
-      m[i] = ws.ml[(p * 2) * 16 + n];
-      l[i] = ws.ml[(p * 2 + 1) * 16 + n];
-      o[i] = load8(pob + (p * 16 + n) * DV + pc * 8);
-    }
-    float M = kNegInf;
-#pragma unroll
-    for (int i = 0; i < TOPN; ++i) M = fmaxf(M, ps[i] < 0 ? kNegInf : m[i]);
-#pragma unroll
-    for (int i = 0; i < TOPN; ++i) {
-      const float w = ps[i] < 0 ? 0.f : fast_exp2((m[i] - M) * c_attn) * l[i];
-      den += w;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) acc[e] = fmaf(w, (float)o[i][e], acc[e]);
-    }
-  } else {
-    float M = kNegInf;
-    for (int i = 0; i < a.top_n; ++i) {
-      const int p = ws.slotmap[base + i];
-      if (p < 0) continue;
-      const float m = ws.ml[((long)p * 2) * 16 + n];
-      const float l = ws.ml[((long)p * 2 + 1) * 16 + n];
-      const vec8_t<T> o = load8(pob + ((long)p * 16 + n) * DV + pc * 8);
-      const float m_new = fmaxf(M, m);
-      const float r_old = fast_exp2((M - m_new) * c_attn);        // 0 for the first partial
-      const float w = fast_exp2((m - m_new) * c_attn) * l;
-      den = den * r_old + w;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) acc[e] = acc[e] * r_old + w * (float)o[e];
-      M = m_new;
-    }
-  }
-  const float inv = den > 0.f ? 1.0f / den : 0.f;
-  const T* gs = reinterpret_cast<const T*>(a.g_slc);
-  const T* gw = reinterpret_cast<const T*>(a.g_swa);
-  const T* gcm = reinterpret_cast<const T*>(a.g_cmp);
   const T* osw = reinterpret_cast<const T*>(a.o_swa);
-  const T* ocm = reinterpret_cast<const T*>(a.o_cmp);
-  const float w_slc = (gs ? gate_of((float)gs[row * a.gate_stride], a.gate_act) : 1.f) * inv;
-  float out[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e) out[e] = acc[e] * w_slc;
-  if (osw) {
-    const float w = gw ? gate_of((float)gw[row * a.gate_stride], a.gate_act) : 1.f;
-    const vec8_t<T> o = load8(osw + row * DV + pc * 8);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) out[e] += w * (float)o[e];
-  }
-  if (ocm) {
-    const float w = gcm ? gate_of((float)gcm[row * a.gate_stride], a.gate_act) : 1.f;
-    const vec8_t<T> o = load8(ocm + row * DV + pc * 8);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) out[e] += w * (float)o[e];
-  }
-  store8(reinterpret_cast<T*>(a.out) + row * DV + pc * 8, pack8<T>(out));
+  vec8_t<T> o_swa = zero8<T>();
+  if (osw) o_swa = load8(osw + row * DV + pc * 8);
+  const vec8_t<T> r = merge_piece<T, DV, TOPN>(m, tg, hq_i / G, hq_i % G, row, pc, osw != nullptr, o_swa);
+  store8(reinterpret_cast<T*>(a.out) + row * DV + pc * 8, r);
 }
 
+static MergeArgs merge_args_of(const SlcArgs& a, const SlcWs& ws) {
+  return MergeArgs{ws.slotmap, ws.ml, ws.po, a.g_slc, a.g_swa, a.g_cmp, a.gate_stride, a.o_cmp, a.out,
+                   a.top_n, a.hq, a.hkv, a.gate_act, a.scale};
+}
+
+// bucket the pairs, then one partial result per pair
 template <typename T, int DK, int DV>
-static int launch_block_t(const SlcArgs& a, const SlcWs& ws, hipStream_t st) {
+static int launch_partials_t(const SlcArgs& a, const SlcWs& ws, hipStream_t st) {
   const long pairs = ws.pairs_cap;
   hipLaunchKernelGGL(slc_prep_kernel, dim3(1), dim3(256), 0, st, a.cu_seq, a.batch, ws, a.hkv);
   if (ws.nb <= kBucketMaxBins) {
@@ -454,23 +388,42 @@ static int launch_block_t(const SlcArgs& a, const SlcWs& ws, hipStream_t st) {
     hipLaunchKernelGGL(slc_bucket_kernel<true>, dim3(gb), dim3(256), 0, st, a, ws);
   }
   hipLaunchKernelGGL((slc_block_kernel<T, DK, DV>), dim3((ws.items_cap + 3) / 4), dim3(256), 0, st, a, ws);
-  const long threads = (long)a.total * a.hq * (DV / 8);
-  const dim3 mg((int)((threads + 255) / 256));
-  if (a.top_n == 16) hipLaunchKernelGGL((slc_merge_kernel<T, DV, 16>), mg, dim3(256), 0, st, a, ws);
-  else hipLaunchKernelGGL((slc_merge_kernel<T, DV, 0>), mg, dim3(256), 0, st, a, ws);
   return 0;
 }
 
-int launch_slc_block_major(const SlcArgs& a, void* workspace, hipStream_t st) {
+template <typename T, int DV>
+static int launch_merge_t(const SlcArgs& a, const SlcWs& ws, hipStream_t st) {
+  const long threads = (long)a.total * a.hq * (DV / 8);
+  const dim3 mg((int)((threads + 255) / 256));
+  const MergeArgs m = merge_args_of(a, ws);
+  if (a.top_n == 16) hipLaunchKernelGGL((slc_merge_kernel<T, DV, 16>), mg, dim3(256), 0, st, a, m);
+  else hipLaunchKernelGGL((slc_merge_kernel<T, DV, 0>), mg, dim3(256), 0, st, a, m);
+  return 0;
+}
+
+int launch_slc_partials(const SlcArgs& a, void* workspace, hipStream_t st) {
   SlcWs ws;
   carve(a, workspace, &ws, 2);
-  const int key = a.dk * 1000 + a.dv;
-  switch (key) {
-    case 64064: return launch_block_t<bf16_t, 64, 64>(a, ws, st);
-    case 128128: return launch_block_t<bf16_t, 128, 128>(a, ws, st);
-    case 192128: return launch_block_t<bf16_t, 192, 128>(a, ws, st);
+  switch (a.dk * 1000 + a.dv) {
+    case 64064: return launch_partials_t<bf16_t, 64, 64>(a, ws, st);
+    case 128128: return launch_partials_t<bf16_t, 128, 128>(a, ws, st);
+    case 192128: return launch_partials_t<bf16_t, 192, 128>(a, ws, st);
     default: return -2;
   }
+}
+
+MergeArgs slc_merge_args(const SlcArgs& a, void* workspace) {
+  SlcWs ws;
+  carve(a, workspace, &ws, 2);
+  return merge_args_of(a, ws);
+}
+
+int launch_slc_block_major(const SlcArgs& a, void* workspace, hipStream_t st) {
+  const int rc = launch_slc_partials(a, workspace, st);
+  if (rc) return rc;
+  SlcWs ws;
+  carve(a, workspace, &ws, 2);
+  return a.dv == 64 ? launch_merge_t<bf16_t, 64>(a, ws, st) : launch_merge_t<bf16_t, 128>(a, ws, st);
 }
 
 }  // namespace nsa

@@ -1,0 +1,95 @@
+// Merge of the block-major selected-attention partials of one (token, q head, 8 output channels),
+// the gates and the sum of the three branches.  Shared by the stand-alone merge kernel and by the
+// sliding-window kernel's epilogue.
+#pragma once
+#include "tiles.h"
+
+namespace nsa {
+
+__device__ __forceinline__ float gate_of(float x, int act) { return act == 1 ? 1.0f / (1.0f + __expf(-x)) : x; }
+
+// slotmap[(tg*hkv + h)*top_n + i] = pair number of pick i, or -1 when the pick is unusable (past
+// the count, not a block, beyond the token).  TOPN > 0: the slot map is read with vector loads and
+// all partials of the piece are requested before any is used (up to TOPN 16-byte loads in flight
+// per lane); TOPN = 0: any top_n, one partial at a time.  n = head inside the GQA group,
+// row = token * hq + q head.
+// Returns g_slc * o_slc + g_swa * o_swa + g_cmp * o_cmp for the piece (o_swa given by the caller).
+template <typename T, int DV, int TOPN>
+__device__ __forceinline__ vec8_t<T> merge_piece(const MergeArgs& m, long tg, int h, int n, long row, int pc,
+                                                 bool has_swa, const vec8_t<T>& o_swa) {
+  const long base = (tg * m.hkv + h) * m.top_n;
+  const float c_attn = m.scale * kLog2e;
+  const T* pob = reinterpret_cast<const T*>(m.po);
+  float den = 0.f, acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  if constexpr (TOPN > 0) {
+    int ps[TOPN];
+#pragma unroll
+    for (int i = 0; i < TOPN / 4; ++i) {
+      const int4 q4 = *reinterpret_cast<const int4*>(m.slotmap + base + 4 * i);
+      ps[4 * i] = q4.x; ps[4 * i + 1] = q4.y; ps[4 * i + 2] = q4.z; ps[4 * i + 3] = q4.w;
+    }
+    float mx[TOPN], l[TOPN];
+    vec8_t<T> o[TOPN];
+#pragma unroll
+    for (int i = 0; i < TOPN; ++i) {
+      mx[i] = kNegInf; l[i] = 0.f; o[i] = zero8<T>();
+      if (ps[i] >= 0) {
+        const long p = ps[i];
+        mx[i] = m.ml[(p * 2) * 16 + n];
+        l[i] = m.ml[(p * 2 + 1) * 16 + n];
+        o[i] = load8(pob + (p * 16 + n) * DV + pc * 8);
+      }
+    }
+    float M = kNegInf;
+#pragma unroll
+    for (int i = 0; i < TOPN; ++i) M = fmaxf(M, mx[i]);
+#pragma unroll
+    for (int i = 0; i < TOPN; ++i) {
+      const float w = ps[i] >= 0 ? fast_exp2((mx[i] - M) * c_attn) * l[i] : 0.f;
+      den += w;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = fmaf(w, (float)o[i][e], acc[e]);
+    }
+  } else {
+    float M = kNegInf;
+    for (int i = 0; i < m.top_n; ++i) {
+      const long p = m.slotmap[base + i];
+      if (p < 0) continue;
+      const float mi = m.ml[(p * 2) * 16 + n];
+      const float l = m.ml[(p * 2 + 1) * 16 + n];
+      const vec8_t<T> o = load8(pob + (p * 16 + n) * DV + pc * 8);
+      const float m_new = fmaxf(M, mi);
+      const float r_old = fast_exp2((M - m_new) * c_attn);        // 0 for the first partial
+      const float w = fast_exp2((mi - m_new) * c_attn) * l;
+      den = den * r_old + w;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = acc[e] * r_old + w * (float)o[e];
+      M = m_new;
+    }
+  }
+  const float inv = den > 0.f ? 1.0f / den : 0.f;
+  const T* gs = reinterpret_cast<const T*>(m.g_slc);
+  const T* gw = reinterpret_cast<const T*>(m.g_swa);
+  const T* gcm = reinterpret_cast<const T*>(m.g_cmp);
+  const T* ocm = reinterpret_cast<const T*>(m.o_cmp);
+  const float w_slc = (gs ? gate_of((float)gs[row * m.gate_stride], m.gate_act) : 1.f) * inv;
+  float out[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) out[e] = acc[e] * w_slc;
+  if (has_swa) {
+    const float w = gw ? gate_of((float)gw[row * m.gate_stride], m.gate_act) : 1.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) out[e] += w * (float)o_swa[e];
+  }
+  if (ocm) {
+    const float w = gcm ? gate_of((float)gcm[row * m.gate_stride], m.gate_act) : 1.f;
+    const vec8_t<T> o = load8(ocm + row * DV + pc * 8);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) out[e] += w * (float)o[e];
+  }
+  return pack8<T>(out);
+}
+
+}  // namespace nsa

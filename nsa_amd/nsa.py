@@ -117,12 +117,22 @@ class NSAAttention(nn.Module):
             gates = self.gating(q)                       # [total, Hq, 3]
         g = gates.reshape(total * hq, 3)
         g_slc, g_swa, g_cmp = (g[:, i].view(total, hq) for i in range(3))
-        o_swa = stage("swa", lambda: ops.swa(q, k, vt, cu, batch, self.sliding_window, scale)) \
-            if self.sliding_window > 0 else None
         act = _lib.GATE_SIGMOID if self.gate_activation == "sigmoid" else _lib.GATE_IDENTITY
-        out = stage("slc_combine", lambda: ops.slc_combine(
-            q, k, vt, idx, None, g_slc, g_swa if o_swa is not None else None, g_cmp, o_swa, o_cmp, cu, batch,
-            self.selection_block_size, scale, gate_act=act))
+        ws = ops.slc_workspace(q, hkv, dv, idx.shape[-1], self.selection_block_size, batch) \
+            if self.sliding_window > 0 else None
+        if ws is not None:
+            # block-major selected attention, merged in the sliding-window kernel's epilogue
+            stage("slc_blocks", lambda: ops.slc_partials(q, k, vt, idx, None, cu, batch, self.selection_block_size,
+                                                         scale, ws))
+            out = stage("swa_combine", lambda: ops.swa_merge(
+                q, k, vt, ws, idx.shape[-1], g_slc, g_swa, g_cmp, o_cmp, cu, batch, self.selection_block_size,
+                self.sliding_window, scale, gate_act=act))
+        else:
+            o_swa = stage("swa", lambda: ops.swa(q, k, vt, cu, batch, self.sliding_window, scale)) \
+                if self.sliding_window > 0 else None
+            out = stage("slc_combine", lambda: ops.slc_combine(
+                q, k, vt, idx, None, g_slc, g_swa if o_swa is not None else None, g_cmp, o_swa, o_cmp, cu, batch,
+                self.selection_block_size, scale, gate_act=act))
         if return_indices:
             return out, idx
         return out

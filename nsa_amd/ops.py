@@ -236,3 +236,51 @@ def slc_combine(q, k, vt, indices, counts, g_slc, g_swa, g_cmp, o_swa, o_cmp, cu
         ws_bytes, _stream())
     _lib.check(rc, "nsa_slc_combine_fwd")
     return out
+
+
+def slc_workspace(q, hkv, dv, top_n, block_size, batch):
+    """Workspace tensor of the block-major selected attention, or None when the shape has none."""
+    total, hq, dk = q.shape
+    need = _lib.load().nsa_slc_workspace_bytes(total, batch, hkv, dk, dv, top_n, block_size, _dtype_code(q))
+    if need <= 0 or need > SLC_WORKSPACE_LIMIT:
+        return None
+    return torch.empty(need, dtype=torch.uint8, device=q.device)
+
+
+def slc_partials(q, k, vt, indices, counts, cu_seqlens, batch, block_size, scale, workspace):
+    """First half of the fused schedule: one partial softmax state per (token, pick) into `workspace`."""
+    _need_cuda(q, k, vt, indices, cu_seqlens, workspace)
+    q, k = _dense(q), _dense(k)
+    total, hq, dk = q.shape
+    hkv, dv = vt.shape[0], vt.shape[1]
+    if indices.dtype not in (torch.int32, torch.int64):
+        raise TypeError("block indices must be int32 or int64")
+    indices = indices.contiguous()
+    if counts is not None:
+        counts = counts.to(torch.int32).contiguous()
+    rc = _lib.load().nsa_slc_partials_fwd(
+        _ptr(q), _ptr(k), _ptr(vt), _ptr(indices), _ptr(counts), _ptr(cu_seqlens), batch, total, hq, hkv, dk, dv,
+        vt.shape[-1], indices.shape[-1], block_size, float(scale), int(indices.dtype == torch.int64),
+        _dtype_code(q), _ptr(workspace), workspace.numel(), _stream())
+    _lib.check(rc, "nsa_slc_partials_fwd")
+    return workspace
+
+
+def swa_merge(q, k, vt, workspace, top_n, g_slc, g_swa, g_cmp, o_cmp, cu_seqlens, batch, block_size, window,
+              scale, gate_act=0):
+    """Second half: sliding-window attention whose epilogue merges the partials slc_partials left in
+    `workspace` (same sizes, top_n picks per token and kv head), applies the gates and adds the
+    compressed branch.  Returns the final output [total,Hq,dv]."""
+    _need_cuda(q, k, vt, cu_seqlens, workspace)
+    q, k = _dense(q), _dense(k)
+    total, hq, dk = q.shape
+    hkv, dv = vt.shape[0], vt.shape[1]
+    (g_slc, g_swa, g_cmp), gs = _gate_views([g_slc, g_swa, g_cmp], q)
+    o_cmp = None if o_cmp is None else _dense(o_cmp)
+    out = torch.empty(total, hq, dv, dtype=q.dtype, device=q.device)
+    rc = _lib.load().nsa_swa_merge_fwd(
+        _ptr(q), _ptr(k), _ptr(vt), _ptr(g_slc), _ptr(g_swa), _ptr(g_cmp), gs, _ptr(o_cmp), _ptr(out),
+        _ptr(cu_seqlens), batch, total, hq, hkv, dk, dv, vt.shape[-1], window, top_n, block_size, float(scale),
+        gate_act, _dtype_code(q), _ptr(workspace), workspace.numel(), _stream())
+    _lib.check(rc, "nsa_swa_merge_fwd")
+    return out

@@ -228,6 +228,48 @@ def test_slc_only(dtype, lens, Hq, Hkv, Dk, Dv, S, bs):
         assert err <= TOL[dtype]
 
 
+@pytest.mark.parametrize("lens,Hq,Hkv,Dk,Dv,S,W", [([512, 100], 32, 2, 128, 128, 8, 128), ([200], 16, 1, 192, 128, 3, 64),
+                                                  ([384], 4, 1, 64, 64, 4, 512), ([700, 330], 24, 2, 64, 64, 16, 256)])
+def test_fused_partials_and_window_merge(lens, Hq, Hkv, Dk, Dv, S, W):
+    """nsa_slc_partials_fwd + nsa_swa_merge_fwd against nsa_swa_fwd + nsa_slc_combine_fwd (token-major
+    kernel) and against the oracle, with counts, invalid picks, gates and a compressed-branch input."""
+    ops = _ops()
+    dtype, bs = torch.bfloat16, 64
+    T = sum(lens)
+    q, k, v, gl = make_qkv(T, Hq, Hkv, Dk, Dv, 160, dtype, 0.7)
+    cu = _cu(lens)
+    cuh = ragged_cu(lens)
+    idx = torch.cat([_random_indices(e - s, Hkv, S, bs, 161 + s) for s, e in zip(cuh[:-1], cuh[1:])])
+    counts = torch.randint(0, S + 1, (T, Hkv), generator=torch.Generator().manual_seed(162))
+    o_cmp = randn(T, Hq, Dv, seed=163, dtype=dtype)
+    vt = ops.transpose(v.to(DEV), cu, len(lens))
+    scale = 1.0 / math.sqrt(Dk)
+    gd = gl.to(DEV)
+    g_slc, g_swa, g_cmp = (gd[..., i] for i in range(3))
+    qd, kd = q.to(DEV), k.to(DEV)
+    for use_counts, dt_idx in ((False, torch.int32), (True, torch.int64)):
+        cd = counts.to(DEV) if use_counts else None
+        idd = idx.to(dt_idx).to(DEV)
+        ws = ops.slc_workspace(qd, Hkv, Dv, S, bs, len(lens))
+        assert ws is not None
+        ops.slc_partials(qd, kd, vt, idd, cd, cu, len(lens), bs, scale, ws)
+        fused = ops.swa_merge(qd, kd, vt, ws, S, g_slc, g_swa, g_cmp, o_cmp.to(DEV), cu, len(lens), bs, W,
+                              scale, gate_act=1).cpu()
+        o_swa = ops.swa(qd, kd, vt, cu, len(lens), W, scale)
+        split = ops.slc_combine(qd, kd, vt, idd, cd, g_slc, g_swa, g_cmp, o_swa, o_cmp.to(DEV), cu, len(lens), bs,
+                                scale, gate_act=1, block_major=False).cpu()
+        sg = torch.sigmoid(gl.float())
+        err = 0.0
+        for s, e in zip(cuh[:-1], cuh[1:]):
+            slc = O.selected_attention(q[s:e], k[s:e], v[s:e], idx[s:e], counts[s:e] if use_counts else None, bs, scale)
+            swa = O.sliding_attention(q[s:e], k[s:e], v[s:e], W, scale)
+            ref = sg[s:e, :, 0:1] * slc.float() + sg[s:e, :, 1:2] * swa.float() + sg[s:e, :, 2:3] * o_cmp[s:e].float()
+            err = max(err, max_abs(fused[s:e], ref))
+        d = max_abs(fused, split)
+        print("fused", lens, (Hq, Hkv, Dk, Dv, S, W), "counts", use_counts, "vs oracle", err, "vs split kernels", d)
+        assert err <= TOL[dtype] and d <= TOL[dtype]
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_parallel_nsa_api_like_reference_test(dtype):
     """Shape of the reference's own test (B=2,T=64,H=1,HQ=16,D=32,S=2,bs=32,W=128, ones gates,
