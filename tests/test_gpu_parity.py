@@ -408,6 +408,17 @@ def test_module_cfg4_full_size_dqk192():
     _module_case(torch.bfloat16, [32768], 64, 4, 192, 128, 16, 512, seed=3, scale_in=0.5, rows_per_seq=96)
 
 
+def test_module_long_context_more_than_512_bins():
+    """T=40960: 2559 compressed rows, 640 pooled bins -> the 16-candidates-per-lane top-n kernel; one kv
+    head of 16 q heads keeps the sampled-row oracle cheap."""
+    _module_case(torch.bfloat16, [40960], 16, 1, 64, 64, 16, 512, seed=9, scale_in=0.5, rows_per_seq=96)
+
+
+def test_module_group_of_12_heads_ragged():
+    """GQA group of 12 (padded to 16 rows per token) with ragged sequences, one shorter than a bin."""
+    _module_case(torch.bfloat16, [1500, 70, 36, 900], 24, 2, 128, 128, 8, 256, seed=10, scale_in=0.5)
+
+
 def test_flash_attn_func_api():
     import nsa_amd
     from nsa_amd.compression_kv import KVCompressor
