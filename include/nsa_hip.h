@@ -97,6 +97,14 @@ int nsa_block_select_fwd(const void* q, const void* ck, const float* lse, void* 
                          int pool_pad, int top_n, int max_ns, int pooled_stride, int idx64, int dtype,
                          nsa_stream_t stream);
 
+/* Gate logits of the three branches: gates[row][o] = bias[o] + q[row] . weight[o], o = 0 (selected),
+ * 1 (sliding window), 2 (compressed).  Replaces the gating nn.Linear(head_dim, 3) of
+ * nsa/nsa.py:61 as applied at nsa/nsa.py:117.  q [rows = total*hq, dim], weight [3, dim] (the
+ * Linear's own layout), bias [3] or NULL, gates [rows, 3]; the activation is applied where the gates
+ * are used (gate_act of the combine calls). */
+int nsa_gate_fwd(const void* q, const void* weight, const void* bias, void* gates, int64_t rows, int dim, int dtype,
+                 nsa_stream_t stream);
+
 /* Sliding window attention: token t attends keys [max(0, t-window+1), t] of its sequence.  Replaces
  * the window loop of nsa/selection_attn.py:483-517.  q [total,hq,dk], k [total,hkv,dk],
  * vt transposed [hkv][dv][vt_cols] over cu_seqlens, o [total,hq,dv]. */

@@ -142,6 +142,15 @@ int nsa_block_select_fwd(const void* q, const void* ck, const float* lse, void* 
                     pool_stride, pool_pad, top_n, max_ns, pooled_stride, 1.0f, 1, idx64, dtype, stream);
 }
 
+int nsa_gate_fwd(const void* q, const void* weight, const void* bias, void* gates, int64_t rows, int dim, int dtype,
+                 nsa_stream_t stream) {
+  if (!q || !weight || !gates) return fail(NSA_ERR_INVALID, "gate: null pointer");
+  if (rows <= 0 || dim <= 0 || dim % 8 != 0) return fail(NSA_ERR_INVALID, "gate: rows must be positive and dim a positive multiple of 8");
+  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "gate: bad dtype");
+  if (!aligned16(q) || !aligned16(weight)) return fail(NSA_ERR_INVALID, "gate: pointers must be 16-byte aligned");
+  return finish(nsa::launch_gate(q, weight, bias, gates, (long)rows, dim, dtype, stream), "gate");
+}
+
 int nsa_swa_fwd(const void* q, const void* k, const void* vt, void* o, const int32_t* cu_seqlens, int batch,
                 int total, int hq, int hkv, int dk, int dv, int vt_cols, int window, float scale, int dtype,
                 nsa_stream_t stream) {

@@ -58,6 +58,8 @@ struct DecodeArgs {
 
 int launch_compress(const CompressArgs& a, hipStream_t st);
 int launch_transpose(const TransposeArgs& a, hipStream_t st);
+int launch_gate(const void* x, const void* w, const void* bias, void* out, long rows, int dim, int dtype,
+                hipStream_t st);
 int launch_cmp_attn(const CmpArgs& a, hipStream_t st);
 int launch_select(const CmpArgs& a, hipStream_t st);
 int launch_swa(const SwaArgs& a, hipStream_t st);

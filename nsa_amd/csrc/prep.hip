@@ -181,6 +181,48 @@ static int launch_transpose_t(const TransposeArgs& a, hipStream_t st) {
   return 0;
 }
 
+// Gate logits out[row][o] = bias[o] + sum_i x[row][i] * w[o][i], o = 0..2 (selected, sliding,
+// compressed): 16 lanes per (token, head) row, fp32 accumulation, one rounding at the end.
+template <typename T>
+__global__ void __launch_bounds__(256)
+gate_kernel(const T* __restrict__ x, const T* __restrict__ w, const T* __restrict__ bias, T* __restrict__ out,
+            long rows, int dim) {
+  const int l16 = threadIdx.x & 15;
+  const long row = (long)blockIdx.x * 16 + (threadIdx.x >> 4);
+  float acc[3] = {0.f, 0.f, 0.f};
+  if (row < rows) {
+    for (int p = l16; p < dim / 8; p += 16) {
+      const vec8_t<T> xv = load8(x + row * dim + 8 * p);
+#pragma unroll
+      for (int o = 0; o < 3; ++o) {
+        const vec8_t<T> wv = load8(w + (long)o * dim + 8 * p);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[o] = fmaf((float)xv[i], (float)wv[i], acc[o]);
+      }
+    }
+  }
+#pragma unroll
+  for (int o = 0; o < 3; ++o)
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) acc[o] += __shfl_xor(acc[o], off, 16);
+  if (row < rows && l16 < 3) {
+    const float v = l16 == 0 ? acc[0] : (l16 == 1 ? acc[1] : acc[2]);
+    out[row * 3 + l16] = (T)(v + (bias != nullptr ? (float)bias[l16] : 0.f));
+  }
+}
+
+int launch_gate(const void* x, const void* w, const void* bias, void* out, long rows, int dim, int dtype,
+                hipStream_t st) {
+  const dim3 grid((unsigned)((rows + 15) / 16));
+  if (dtype == 0)
+    hipLaunchKernelGGL(gate_kernel<bf16_t>, grid, dim3(256), 0, st, (const bf16_t*)x, (const bf16_t*)w,
+                       (const bf16_t*)bias, (bf16_t*)out, rows, dim);
+  else
+    hipLaunchKernelGGL(gate_kernel<float>, grid, dim3(256), 0, st, (const float*)x, (const float*)w,
+                       (const float*)bias, (float*)out, rows, dim);
+  return 0;
+}
+
 int launch_transpose(const TransposeArgs& a, hipStream_t st) {
   return a.dtype == 0 ? launch_transpose_t<bf16_t>(a, st) : launch_transpose_t<float>(a, st);
 }

@@ -114,7 +114,7 @@ class NSAAttention(nn.Module):
             q, ck, lse, cu, cu_cmp, batch, hkv, ck.stride(0), ck.stride(1), self.pool_kernel_size,
             self.pool_stride, self.pool_padding, self.selected_block_count, max_nc, idx64=False))
         if gates is None:
-            gates = self.gating(q)                       # [total, Hq, 3]
+            gates = stage("gates", lambda: ops.gate_logits(q, self.gating.weight, self.gating.bias))   # [total, Hq, 3]
         g = gates.reshape(total * hq, 3)
         g_slc, g_swa, g_cmp = (g[:, i].view(total, hq) for i in range(3))
         act = _lib.GATE_SIGMOID if self.gate_activation == "sigmoid" else _lib.GATE_IDENTITY

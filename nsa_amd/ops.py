@@ -284,3 +284,17 @@ def swa_merge(q, k, vt, workspace, top_n, g_slc, g_swa, g_cmp, o_cmp, cu_seqlens
         gate_act, _dtype_code(q), _ptr(workspace), workspace.numel(), _stream())
     _lib.check(rc, "nsa_swa_merge_fwd")
     return out
+
+
+def gate_logits(q, weight, bias=None):
+    """q [total,Hq,D], weight [3,D], bias [3] -> gate logits [total,Hq,3] (selected, sliding, compressed)."""
+    _need_cuda(q, weight)
+    q = _dense(q)
+    total, hq, dim = q.shape
+    weight = weight.to(q.dtype).contiguous()
+    bias = None if bias is None else bias.to(q.dtype).contiguous()
+    out = torch.empty(total, hq, 3, dtype=q.dtype, device=q.device)
+    rc = _lib.load().nsa_gate_fwd(_ptr(q), _ptr(weight), _ptr(bias), _ptr(out), total * hq, dim, _dtype_code(q),
+                                  _stream())
+    _lib.check(rc, "nsa_gate_fwd")
+    return out

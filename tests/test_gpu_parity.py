@@ -419,6 +419,44 @@ def test_module_group_of_12_heads_ragged():
     _module_case(torch.bfloat16, [1500, 70, 36, 900], 24, 2, 128, 128, 8, 256, seed=10, scale_in=0.5)
 
 
+@pytest.mark.parametrize("dtype,T,Hq,D", [(torch.bfloat16, 300, 16, 192), (torch.float32, 77, 4, 64),
+                                          (torch.bfloat16, 1000, 64, 128)])
+def test_gate_logits_match_linear(dtype, T, Hq, D):
+    """nsa_gate_fwd against the Linear it stands for, evaluated in fp64 on the bf16/fp32 values: one
+    rounding of the result is all that may differ."""
+    ops = _ops()
+    q = randn(T, Hq, D, seed=170, dtype=dtype)
+    w = randn(3, D, seed=171, scale=0.2, dtype=dtype)
+    b = randn(3, seed=172, dtype=dtype)
+    got = ops.gate_logits(q.to(DEV), w.to(DEV), b.to(DEV)).cpu()
+    ref = (q.double() @ w.double().t() + b.double())
+    err = (got.double() - ref).abs()
+    bar = ref.abs() * (2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -20) + 1e-6
+    print("gate", dtype, (T, Hq, D), "max_abs", err.max().item())
+    assert (err <= bar).all()
+    assert torch.equal(ops.gate_logits(q.to(DEV), w.to(DEV), None).cpu(),
+                       ops.gate_logits(q.to(DEV), w.to(DEV), torch.zeros(3, dtype=dtype).to(DEV)).cpu())
+
+
+def test_module_own_gating_equals_explicit_gates():
+    """forward(gates=None) runs the gate kernel on the module's Linear; feeding those logits back in
+    through gates= must give the same output bit for bit."""
+    from nsa_amd.nsa import NSAAttention
+    dtype, T, Hq, Hkv, D = torch.bfloat16, 640, 32, 2, 128
+    q, k, v, _ = make_qkv(T, Hq, Hkv, D, D, 173, dtype, 0.5)
+    torch.manual_seed(174)
+    m = NSAAttention(D, causal=True, selected_block_count=8, sliding_window=128, dtype=dtype, compressor_mode="mean",
+                     gate_activation="sigmoid").to(DEV)
+    cu = _cu([T])
+    a = m(q.to(DEV), k.to(DEV), v.to(DEV), cu, 0)
+    gl = _ops().gate_logits(q.to(DEV), m.gating.weight, m.gating.bias)
+    ref_gl = torch.nn.functional.linear(q.float(), m.gating.weight.detach().float().cpu(),
+                                        m.gating.bias.detach().float().cpu())
+    assert max_abs(gl.cpu(), ref_gl) <= 3e-2
+    b = m(q.to(DEV), k.to(DEV), v.to(DEV), cu, 0, gates=gl)
+    assert torch.equal(a, b)
+
+
 def test_flash_attn_func_api():
     import nsa_amd
     from nsa_amd.compression_kv import KVCompressor
