@@ -71,11 +71,19 @@ def parallel_nsa(q: torch.Tensor,
     nb = cu.numel() - 1
     qp, kp, vp = _packed(q, B, T), _packed(k, B, T), _packed(v, B, T)
     vt = ops.transpose(vp, cu, nb)
-    o_swa = ops.swa(qp, kp, vt, cu, nb, window_size, scale) if window_size > 0 else None
     counts = None if block_counts is None else block_counts.reshape(B * T, H)
-    o = ops.slc_combine(qp, kp, vt, block_indices.reshape(B * T, H, -1), counts,
-                        g_slc.reshape(B * T, HQ), g_swa.reshape(B * T, HQ) if o_swa is not None else None, None,
-                        o_swa, None, cu, nb, block_size, scale)
+    idx = block_indices.reshape(B * T, H, -1)
+    ws = ops.slc_workspace(qp, H, V, idx.shape[-1], block_size, nb) if window_size > 0 else None
+    if ws is not None:
+        # fused schedule: per-block partial results, merged in the window kernel's epilogue
+        ops.slc_partials(qp, kp, vt, idx, counts, cu, nb, block_size, scale, ws)
+        o = ops.swa_merge(qp, kp, vt, ws, idx.shape[-1], g_slc.reshape(B * T, HQ), g_swa.reshape(B * T, HQ), None,
+                          None, cu, nb, block_size, window_size, scale)
+    else:
+        o_swa = ops.swa(qp, kp, vt, cu, nb, window_size, scale) if window_size > 0 else None
+        o = ops.slc_combine(qp, kp, vt, idx, counts, g_slc.reshape(B * T, HQ),
+                            g_swa.reshape(B * T, HQ) if o_swa is not None else None, None, o_swa, None, cu, nb,
+                            block_size, scale)
     o = o.view(B, T, HQ, V)
     if head_first:
         o = o.transpose(1, 2)
