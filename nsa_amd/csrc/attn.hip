@@ -219,12 +219,13 @@ stream_attn_kernel(const StreamParams a) {
           grp[j].m = m_new;
           const float m = grp[j].m;
           const float off_i = -m * kLog2e, off_a = -m * c_attn;
-          float sum = 0.f;
+          {
+            float ei[8];
 #pragma unroll
-          for (int i = 0; i < 8; ++i) sum += fast_exp2(fmaf(s[i], kLog2e, off_i));
-          li[j] += sum;
+            for (int i = 0; i < 8; ++i) ei[i] = fast_exp2(fmaf(s[i], kLog2e, off_i));
+            li[j] += sum8(ei);
+          }
           if (act[j]) {
-            sum = 0.f;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
               p[i] = fast_exp2(fmaf(s[i], c_attn, off_a));
@@ -235,9 +236,7 @@ stream_attn_kernel(const StreamParams a) {
               for (int i = 0; i < 8; ++i)
                 if (key0 + i > hi[j]) p[i] = 0.f;
             }
-#pragma unroll
-            for (int i = 0; i < 8; ++i) sum += p[i];
-            grp[j].l += sum;
+            grp[j].l += sum8(p);
             pb[j] = pack8<T>(p);
           } else {
             pb[j] = zero8<T>();

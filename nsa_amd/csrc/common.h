@@ -211,6 +211,11 @@ __device__ __forceinline__ void raise_max(RowGroup<T, DK, DV>& g, float mx, floa
   g.m = m_new;
 }
 
+// Sum of 8 values as a balanced tree: three dependent adds instead of seven.
+__device__ __forceinline__ float sum8(const float (&x)[8]) {
+  return ((x[0] + x[1]) + (x[2] + x[3])) + ((x[4] + x[5]) + (x[6] + x[7]));
+}
+
 // Online-softmax update for the 8 scores a lane holds of one 32-key chunk (masked entries are
 // -inf).  Returns the unnormalised probabilities in p.
 template <typename T, int DK, int DV>
@@ -221,13 +226,9 @@ __device__ __forceinline__ void softmax_update(RowGroup<T, DK, DV>& g, const flo
   for (int i = 1; i < 8; ++i) mx = fmaxf(mx, s[i]);
   raise_max(g, colgroup_max(mx), c);
   const float off = (g.m == kNegInf) ? 0.f : -g.m * c;
-  float sum = 0.f;
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    p[i] = fast_exp2(fmaf(s[i], c, off));
-    sum += p[i];
-  }
-  g.l += sum;
+  for (int i = 0; i < 8; ++i) p[i] = fast_exp2(fmaf(s[i], c, off));
+  g.l += sum8(p);
 }
 
 }  // namespace nsa
