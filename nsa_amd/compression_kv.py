@@ -85,11 +85,11 @@ class KVCompressor(nn.Module):
         """Un-repeated result: (ck, cv [sum Nc, H, D], cu_cmp int32 [B+1], max Nc or None)."""
         cu = cu_seq_len.to(torch.int32)
         batch = cu.numel() - 1
-        if seq_len is not None:
-            nc = conv_compressed_len(seq_len, self.block_stride, self.block_size)
+        nc = conv_compressed_len(seq_len, self.block_stride, self.block_size) if seq_len is not None else None
+        if nc:
             cu_out = ops.uniform_cu(batch, nc, k.device)
             rows = nc * batch
-        else:
+        else:                       # ragged lengths, or sequences shorter than one block (no rows at all)
             cu_out = ops.compressed_offsets(cu, self.block_size, self.block_stride, extra=1)
             rows = k.shape[0] // self.block_stride + batch
             nc = None

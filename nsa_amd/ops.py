@@ -57,6 +57,8 @@ def transposed_cols(total_rows: int, batch: int) -> int:
 
 
 def uniform_cu(batch: int, length: int, device) -> torch.Tensor:
+    if length == 0:
+        return torch.zeros(batch + 1, dtype=torch.int32, device=device)
     return torch.arange(0, (batch + 1) * length, length, dtype=torch.int32, device=device)
 
 

@@ -457,6 +457,29 @@ def test_module_own_gating_equals_explicit_gates():
     assert torch.equal(a, b)
 
 
+def test_module_randomized_small_shapes():
+    """Seeded sweep over ragged lengths (down to a single token), group sizes 1..16, top-n, window and
+    both dtypes: every config is checked in full against the oracle."""
+    g = torch.Generator().manual_seed(2025)
+
+    def pick(options):
+        return options[int(torch.randint(0, len(options), (1,), generator=g))]
+
+    for case in range(28):
+        nseq = pick([1, 1, 2, 3, 4])
+        lens = [int(torch.randint(1, 400, (1,), generator=g)) for _ in range(nseq)]
+        if case % 7 == 0:
+            lens[0] = pick([1, 31, 32, 33, 47, 48, 63, 64, 65, 111, 112])
+        G = pick([1, 2, 3, 4, 8, 12, 16])
+        Hkv = pick([1, 2])
+        D = pick([64, 128])
+        S = pick([1, 2, 4, 7, 16])
+        W = pick([1, 5, 64, 100, 512])
+        dtype = pick([torch.bfloat16, torch.float32])
+        print("case", case, lens, G, Hkv, D, S, W, dtype)
+        _module_case(dtype, lens, G * Hkv, Hkv, D, D, S, W, seed=300 + case, scale_in=0.6)
+
+
 def test_flash_attn_func_api():
     import nsa_amd
     from nsa_amd.compression_kv import KVCompressor

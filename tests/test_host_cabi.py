@@ -117,3 +117,11 @@ def test_module_keeps_reference_parameter_names():
                      "gating.weight", "gating.bias"}
     assert m.compressor.compressor_k.weight.shape == (64, 64, 32) and m.gating.weight.shape == (3, 64)
     assert (m.pool_kernel_size, m.pool_stride, m.pool_padding) == (5, 4, 0)
+
+
+def test_uniform_cu_of_empty_sequences():
+    """A batch whose sequences have no compressed rows still gets a valid offsets tensor."""
+    import torch
+    from nsa_amd import ops
+    assert ops.uniform_cu(3, 0, "cpu").tolist() == [0, 0, 0, 0]
+    assert ops.uniform_cu(2, 5, "cpu").tolist() == [0, 5, 10]
