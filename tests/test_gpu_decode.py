@@ -120,3 +120,25 @@ def test_decode_rejects_long_caches():
     q = torch.zeros(1, 4, 64, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(NotImplementedError):
         nsa_decode_step(q, cache)
+
+
+def test_decode_randomized_sweep():
+    """Seeded sweep over ragged context lengths, group sizes, top-n and window, both dtypes."""
+    g = torch.Generator().manual_seed(77)
+
+    def pick(options):
+        return options[int(torch.randint(0, len(options), (1,), generator=g))]
+
+    for case in range(20):
+        B = pick([1, 2, 3, 5])
+        ctxs = [int(torch.randint(1, 900, (1,), generator=g)) for _ in range(B)]
+        if case % 5 == 0:
+            ctxs[0] = pick([1, 31, 32, 33, 63, 64, 65, 95, 96, 127, 128])
+        G, Hkv = pick([1, 2, 4, 8, 16]), pick([1, 2])
+        D = pick([64, 128])
+        S, W = pick([1, 3, 4, 16]), pick([1, 17, 64, 128, 512])
+        dtype = pick([torch.bfloat16, torch.float32])
+        if dtype == torch.float32 and D == 128 and G == 16:
+            G = 4                                  # keep the sweep to shapes every dtype is built for
+        print("case", case, ctxs, G, Hkv, D, S, W, dtype)
+        _check(dtype, ctxs, G * Hkv, Hkv, D, D, S, W, seed=400 + case)
