@@ -476,8 +476,10 @@ def test_module_randomized_small_shapes():
         S = pick([1, 2, 4, 7, 16])
         W = pick([1, 5, 64, 100, 512])
         dtype = pick([torch.bfloat16, torch.float32])
-        print("case", case, lens, G, Hkv, D, S, W, dtype)
-        _module_case(dtype, lens, G * Hkv, Hkv, D, D, S, W, seed=300 + case, scale_in=0.6)
+        mode = pick(["mean", "mean", "conv"])           # conv: the reference's learned Conv1d compressor
+        act = pick(["sigmoid", "sigmoid", None])        # None: raw gate logits as in the reference
+        print("case", case, lens, G, Hkv, D, S, W, dtype, mode, act)
+        _module_case(dtype, lens, G * Hkv, Hkv, D, D, S, W, seed=300 + case, scale_in=0.6, mode=mode, act=act)
 
 
 def test_flash_attn_func_api():
