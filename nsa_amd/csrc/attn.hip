@@ -98,6 +98,9 @@ stream_attn_kernel(const StreamParams a) {
     g_lo_max[j] = CMP ? 0 : tl - W + 1;
   }
   const float c_attn = a.scale * kLog2e;
+  // CMP runs two softmaxes off one reference (raw scores for the importance statistics, scaled ones
+  // for the attention): the slack, in raw score units, bounds the faster growing exponential
+  const float cmp_slack = kMaxSlackLog2 / fmaxf(kLog2e, c_attn);
   const int attn_end = last_visible(t_last);                      // last key any row of the tile attends
   const int c_begin = CMP ? 0 : (max(st.t0 - W + 1, 0) / CH) * CH;
   const int c_end = CMP ? nkeys : t_last + 1;
@@ -206,8 +209,8 @@ stream_attn_kernel(const StreamParams a) {
 #pragma unroll
           for (int i = 1; i < 8; ++i) mx = fmaxf(mx, s[i]);
           mx = colgroup_max(mx);                       // finite: key cb exists
-          const float m_new = fmaxf(grp[j].m, mx);
-          if (__any(m_new > grp[j].m)) {
+          if (__any(mx > grp[j].m + cmp_slack)) {
+            const float m_new = fmaxf(grp[j].m, mx);
             const float d = grp[j].m - m_new;          // -inf on the first chunk
             float beta = fast_exp2(d * kLog2e), alpha = fast_exp2(d * c_attn);
             settle_factor(beta, alpha);
@@ -215,8 +218,8 @@ stream_attn_kernel(const StreamParams a) {
             scale_inplace(grp[j].l, alpha);
 #pragma unroll
             for (int t = 0; t < DV / 16; ++t) scale_inplace(grp[j].o[t], alpha);
+            grp[j].m = m_new;
           }
-          grp[j].m = m_new;
           const float m = grp[j].m;
           const float off_i = -m * kLog2e, off_a = -m * c_attn;
           {

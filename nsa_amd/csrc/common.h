@@ -194,21 +194,29 @@ __device__ __forceinline__ void scale_inplace(f32x4_t& v, float a) {
   v[0] = e0; v[1] = e1; v[2] = e2; v[3] = e3;
 }
 
-// Raise the running maximum of a group to cover `mx` (already reduced over the column's four
-// lanes).  The accumulator and denominator are rescaled only when some lane's maximum grew, which
-// after the first few chunks is rare.  c = scale * log2(e).
+// How far (in powers of two of the resulting probability) a score may exceed the running reference
+// before the accumulators are rescaled.  The reference of an online softmax does not have to be the
+// exact maximum: any value within this slack of it keeps every exponential <= 2^kMaxSlackLog2, far
+// from overflow in fp32 sums and bf16 probabilities, and the final o / l is unchanged.  With 16 rows
+// sharing one branch, following the exact maximum would rescale on more than half of the chunks
+// (record-value statistics); with the slack it happens on the first chunk and hardly ever again.
+constexpr float kMaxSlackLog2 = 8.0f;
+
+// Move the running reference of a group up when `mx` (already reduced over the column's four
+// lanes) exceeds it by more than the slack; the accumulator and denominator are rescaled then.
+// c = scale * log2(e).
 template <typename T, int DK, int DV>
 __device__ __forceinline__ void raise_max(RowGroup<T, DK, DV>& g, float mx, float c) {
-  const float m_new = fmaxf(g.m, mx);
-  if (__any(m_new > g.m)) {
+  if (__any(mx * c > fmaf(g.m, c, kMaxSlackLog2))) {       // -inf reference: any finite score moves it
+    const float m_new = fmaxf(g.m, mx);
     const float mref = (m_new == kNegInf) ? 0.f : m_new;
     float alpha = fast_exp2((g.m - mref) * c);
     settle_factor(alpha);
     scale_inplace(g.l, alpha);
 #pragma unroll
     for (int i = 0; i < DV / 16; ++i) scale_inplace(g.o[i], alpha);
+    g.m = m_new;
   }
-  g.m = m_new;
 }
 
 // Sum of 8 values as a balanced tree: three dependent adds instead of seven.
