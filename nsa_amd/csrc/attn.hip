@@ -479,11 +479,13 @@ slc_combine_kernel(const SlcArgs a) {
 // ------------------------------------------------------------------------------------------------
 // launchers
 
-template <typename T> struct StreamTile {
-  // row groups per wavefront, keys per LDS chunk, wavefronts per workgroup
+template <typename T, bool CMP> struct StreamTile {
+  // row groups per wavefront, keys per LDS chunk, wavefronts per workgroup.  The compressed branch
+  // walks ~2000 keys per tile and gains from half as many barriers (64-key chunks, 16 tokens per
+  // workgroup); the window branch walks ~550 and is better off with small workgroups.
   static constexpr int NG = sizeof(T) == 2 ? 2 : 1;
-  static constexpr int CH = 32;
-  static constexpr int NW = 4;
+  static constexpr int CH = (CMP && sizeof(T) == 2) ? 64 : 32;
+  static constexpr int NW = (CMP && sizeof(T) == 2) ? 8 : 4;
 };
 
 int set_smem(const void* fn, size_t bytes) {
@@ -502,7 +504,7 @@ int group_pow2(int G) {
 
 template <typename T, int DK, int DV, bool CMP, int MERGE = 0>
 static int launch_stream_t(const StreamParams& a, int total, hipStream_t st) {
-  constexpr int NG = StreamTile<T>::NG, CH = StreamTile<T>::CH, NW = StreamTile<T>::NW;
+  constexpr int NG = StreamTile<T, CMP>::NG, CH = StreamTile<T, CMP>::CH, NW = StreamTile<T, CMP>::NW;
   const int Gp = group_pow2(a.hq / a.hkv);
   const int TQ = NW * NG * 16 / Gp;
   const size_t smem = 2 * ((size_t)CH * (DK + 8) + (size_t)DV * (CH + 8)) * sizeof(T);
