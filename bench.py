@@ -36,7 +36,7 @@ WORKLOADS = {
 }
 BLOCK, STRIDE, SEL_BLOCK = 32, 16, 64
 # bytes per launch: (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0) KiB, factors from a 1 GiB device copy in the same run
-MEASURED_TRAFFIC = {("prefill_cfg4", "cmp_attn"): int((432350.0 * 2.0 + 532480.0) * 1024)}
+MEASURED_TRAFFIC = {("prefill_cfg4", "cmp_attn"): int((443594.0 * 2.0 + 532480.0) * 1024)}
 
 
 def flops_model(lens, hq, hkv, dqk, dv, window, valid_blocks_total):
