@@ -47,10 +47,12 @@ __device__ __forceinline__ vec8_t<T> merge_piece(const MergeArgs& m, long tg, in
     for (int i = 0; i < TOPN; ++i) M = fmaxf(M, mx[i]);
 #pragma unroll
     for (int i = 0; i < TOPN; ++i) {
-      const float w = ps[i] >= 0 ? fast_exp2((mx[i] - M) * c_attn) * l[i] : 0.f;
-      den += w;
+      if (ps[i] >= 0) {          // the same for every lane that works on this token: unusable picks cost nothing
+        const float w = fast_exp2((mx[i] - M) * c_attn) * l[i];
+        den += w;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[e] = fmaf(w, (float)o[i][e], acc[e]);
+        for (int e = 0; e < 8; ++e) acc[e] = fmaf(w, (float)o[i][e], acc[e]);
+      }
     }
   } else {
     float M = kNegInf;
