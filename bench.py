@@ -93,7 +93,7 @@ def cpu_baseline(q, k, v, gl, top_n, window, budget_s=20.0):
 
 
 def decode_bench(steps, warmup):
-    """BASELINE config 5: batch 64, one query token per sequence, 32768 cached tokens each (+ the
+    """benchmark config 5: batch 64, one query token per sequence, 32768 cached tokens each (+ the
     compressed caches), Hq64/Hkv4, D128, top-16 blocks of 64, window 512, bf16."""
     import torch
     from nsa_amd.decode import NSADecodeCache, nsa_decode_step

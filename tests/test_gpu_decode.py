@@ -65,7 +65,7 @@ def test_decode_dqk192():
 
 
 def test_decode_cfg5_context_subset():
-    """BASELINE config 5 shape per sequence (ctx 32768, Hq64/Hkv4, D128, top-16, window 512), batch 4."""
+    """benchmark config 5 shape per sequence (ctx 32768, Hq64/Hkv4, D128, top-16, window 512), batch 4."""
     _check(torch.bfloat16, [32768, 32768, 32767, 32000], 64, 4, 128, 128, 16, 512, seed=130)
 
 

@@ -359,12 +359,12 @@ def _module_case(dtype, lens, Hq, Hkv, Dk, Dv, S, W, seed, scale_in, mode="mean"
 
 
 def test_module_cfg1_fp32():
-    """BASELINE config 1: B1, T1024, Hq4, Hkv1, D64, fp32, mean-pool 32/16, blocks of 64, top-4, window 128."""
+    """benchmark config 1: B1, T1024, Hq4, Hkv1, D64, fp32, mean-pool 32/16, blocks of 64, top-4, window 128."""
     _module_case(torch.float32, [1024], 4, 1, 64, 64, 4, 128, seed=0, scale_in=1.0)
 
 
 def test_module_cfg2_shape_reduced_bf16():
-    """BASELINE config 2 at T=2048 (the full T=8192 case is test_module_cfg2_full)."""
+    """benchmark config 2 at T=2048 (the full T=8192 case is test_module_cfg2_full)."""
     _module_case(torch.bfloat16, [2048], 64, 4, 128, 128, 16, 512, seed=1, scale_in=0.5)
 
 
@@ -383,12 +383,12 @@ def test_module_reference_defaults_conv_raw_gates():
 
 
 def test_module_cfg2_full_size():
-    """BASELINE config 2 at its real size (T=8192, Hq64/Hkv4, D128, bf16); sampled rows."""
+    """benchmark config 2 at its real size (T=8192, Hq64/Hkv4, D128, bf16); sampled rows."""
     _module_case(torch.bfloat16, [8192], 64, 4, 128, 128, 16, 512, seed=1, scale_in=0.5, rows_per_seq=160)
 
 
 def test_module_cfg3_full_size_varlen():
-    """BASELINE config 3: 8 sequences with seeded lengths in [1024, 16384], packed; sampled rows, and
+    """benchmark config 3: 8 sequences with seeded lengths in [1024, 16384], packed; sampled rows, and
     the packed result must equal, bit for bit, each sequence run on its own."""
     from nsa_amd.nsa import NSAAttention
     g = torch.Generator().manual_seed(2)
@@ -404,7 +404,7 @@ def test_module_cfg3_full_size_varlen():
 
 
 def test_module_cfg4_full_size_dqk192():
-    """BASELINE config 4 (T=32768, Dqk192/Dv128, bf16); sampled rows."""
+    """benchmark config 4 (T=32768, Dqk192/Dv128, bf16); sampled rows."""
     _module_case(torch.bfloat16, [32768], 64, 4, 192, 128, 16, 512, seed=3, scale_in=0.5, rows_per_seq=96)
 
 
