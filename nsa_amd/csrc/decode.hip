@@ -324,13 +324,21 @@ decode_step_kernel(const DecodeArgs a) {
 
   // ---- phase 3 (wavefront 0 only): top-n blocks; each lane owns the bins b == lane (mod 64)
   if (wave == 0) {
-    volatile float* vb = bins;
-    for (int bb = lane; bb < Ns; bb += 64) {
-      const int lo = bb * a.pool_s - a.pool_p;
-      const int div = min(lo + a.pool_k, Nc + a.pool_p) - lo;
-      vb[bb] = vb[bb] / (float)div;
+    constexpr int PER = (32 * kDecWaves * kDecMaxChunks / 4 + 63) / 64 + 1;
+    __shared__ float cand_v[128];
+    __shared__ int cand_i[128];
+    float v[PER];
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      const int bb = lane + 64 * k;
+      v[k] = -1.f;
+      if (bb < Ns) {
+        const int lo = bb * a.pool_s - a.pool_p;
+        const int div = min(lo + a.pool_k, Nc + a.pool_p) - lo;
+        v[k] = bins[bb] / (float)div;
+      }
     }
-    wave_topn<(32 * kDecWaves * kDecMaxChunks / 4 + 63) / 64 + 1>(vb, Ns, a.top_n, lane, [&](int rr, int val) {
+    wave_topn_shortlist<PER>(v, a.top_n, lane, cand_v, cand_i, [&](int rr, int val) {
       if (lane == 0) {
         sel[rr] = val;
         if (a.indices != nullptr) a.indices[((long)b * a.hkv + h) * a.top_n + rr] = val;

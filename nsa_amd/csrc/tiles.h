@@ -194,6 +194,85 @@ NSA_WAVE_REDUCE(wave_min_f32, float, "v_min_f32_dpp")
 NSA_WAVE_REDUCE(wave_min_i32, int, "v_min_i32_dpp")
 #undef NSA_WAVE_REDUCE
 
+// Top-n of the PER * 64 non-negative scores a wavefront holds in registers (v[k] of lane l is bin
+// l + 64k; -1 marks "no bin"), descending, ties to the lower index; emit(r, index or -1).
+//
+// Shortlist first: each of the 16 lane quads holds a maximum; the smallest of those, L, has at least
+// 16 bins at or above it, so the 16 best bins are all >= L.  Typically fewer than a tenth of the bins
+// pass; they are compacted in index order through `cand_v` / `cand_i` (128 entries each, private to
+// the wavefront) to at most two per lane, and the selection rounds then cost a fraction of rounds over
+// all PER bins per lane.  More than 16 picks or more than 128 candidates fall back to full rounds.
+template <int PER, typename Emit>
+__device__ __forceinline__ void wave_topn_shortlist(float (&v)[PER], int top_n, int lane, float* cand_v, int* cand_i,
+                                                    Emit emit) {
+  int total = 129;
+  if (top_n <= 16) {
+    float m = v[0];
+#pragma unroll
+    for (int k = 1; k < PER; ++k) m = fmaxf(m, v[k]);
+    m = fmaxf(m, dpp_f32<0xB1>(m));
+    m = fmaxf(m, dpp_f32<0x4E>(m));                       // quad maximum (-1 for a quad without bins)
+    const float L = wave_min_f32(m);
+    total = 0;
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      const bool c = v[k] >= L && v[k] >= 0.f;
+      const unsigned long long mask = __ballot(c);
+      const int pos = total + (int)__builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32),
+                                                             __builtin_amdgcn_mbcnt_lo((unsigned)mask, 0u));
+      if (c && pos < 128) {
+        cand_v[pos] = v[k];
+        cand_i[pos] = lane + 64 * k;
+      }
+      total += __popcll(mask);
+    }
+  }
+  if (total <= 128) {
+    __builtin_amdgcn_wave_barrier();
+    float c0 = lane < total ? cand_v[lane] : -1.f;
+    float c1 = lane + 64 < total ? cand_v[lane + 64] : -1.f;
+    const int i0 = cand_i[lane], i1 = cand_i[lane + 64];
+    for (int r = 0; r < top_n; ++r) {
+      const bool second = c1 > c0;                        // slot 0 has the lower index: it wins ties
+      const float best = second ? c1 : c0;
+      const int bi = second ? i1 : i0;
+      const float wmax = wave_max_f32(best);
+      int win = -1;
+      if (wmax >= 0.f) {
+        const unsigned long long tied = __ballot(best == wmax);
+        if (__popcll(tied) == 1) {
+          win = __builtin_amdgcn_readlane(bi, (int)__builtin_ctzll(tied));
+        } else {
+          win = wave_min_i32(best == wmax ? bi : 0x7fffffff);
+        }
+        if (bi == win) {                                  // indices are unique: exactly one lane
+          if (second) c1 = -1.f; else c0 = -1.f;
+        }
+      }
+      emit(r, win);
+    }
+    return;
+  }
+  for (int r = 0; r < top_n; ++r) {
+    float best = v[0];
+    int bk = 0;
+#pragma unroll
+    for (int k = 1; k < PER; ++k)
+      if (v[k] > best) { best = v[k]; bk = k; }
+    const int bi = lane + 64 * bk;
+    long key = ((long)__float_as_int(best) << 32) | (unsigned int)(0x7fffffff - bi);
+    key = wave_max_i64(key);
+    const bool found = (int)(key >> 32) >= 0;
+    const int win = 0x7fffffff - (int)(unsigned int)key;
+    if (found && (win & 63) == lane) {
+#pragma unroll
+      for (int k = 0; k < PER; ++k)
+        if (k == (win >> 6)) v[k] = -1.f;
+    }
+    emit(r, found ? win : -1);
+  }
+}
+
 // Scheduling hint for the basic block it is placed in: alternate MF matrix instructions with VA
 // vector-ALU instructions, spread evenly (one MFMA, then its share of the VALU work, ...).
 template <int MF, int VA, int I = 0>
