@@ -86,8 +86,11 @@ int nsa_cmp_attn_select_fwd(const void* q, const void* ck, const void* cvt, void
                             float scale, int causal, int idx64, int dtype, nsa_stream_t stream);
 
 /* The two halves of nsa_cmp_attn_select_fwd as separate launches: compressed attention (writes o
- * and lse) and block selection (reads lse).  Same arguments and meaning as above. */
-int nsa_cmp_attn_fwd(const void* q, const void* ck, const void* cvt, void* o, float* lse,
+ * and lse) and block selection (reads lse).  Same arguments and meaning as above.
+ *   lse_attn (optional, float [total, hq]) receives what the backward needs: the natural-log
+ *   log-sum-exp of the scaled scores over the rows visible to the token (the reference's M of
+ *   nsa/triton_attention.py:176-181 in natural log), +inf for a token that sees no row. */
+int nsa_cmp_attn_fwd(const void* q, const void* ck, const void* cvt, void* o, float* lse, float* lse_attn,
                      const int32_t* cu_seqlens, const int32_t* cu_cmp, int batch, int total, int hq, int hkv,
                      int dk, int dv, int64_t ck_row_stride, int64_t ck_head_stride, int cvt_cols, int block,
                      int stride, float scale, int causal, int dtype, nsa_stream_t stream);
@@ -107,8 +110,10 @@ int nsa_gate_fwd(const void* q, const void* weight, const void* bias, void* gate
 
 /* Sliding window attention: token t attends keys [max(0, t-window+1), t] of its sequence.  Replaces
  * the window loop of nsa/selection_attn.py:483-517.  q [total,hq,dk], k [total,hkv,dk],
- * vt transposed [hkv][dv][vt_cols] over cu_seqlens, o [total,hq,dv]. */
-int nsa_swa_fwd(const void* q, const void* k, const void* vt, void* o, const int32_t* cu_seqlens,
+ * vt transposed [hkv][dv][vt_cols] over cu_seqlens, o [total,hq,dv]; lse (optional, float
+ * [total,hq]) receives the log-sum-exp of the scaled window scores (lse_swa of
+ * nsa/selection_attn.py:492-515). */
+int nsa_swa_fwd(const void* q, const void* k, const void* vt, void* o, float* lse, const int32_t* cu_seqlens,
                 int batch, int total, int hq, int hkv, int dk, int dv, int vt_cols, int window,
                 float scale, int dtype, nsa_stream_t stream);
 
@@ -121,10 +126,13 @@ int nsa_swa_fwd(const void* q, const void* k, const void* vt, void* o, const int
  *   g[(t*hq + hq_idx)*gate_stride].  A token with no usable block has o_slc = 0.
  *   workspace (optional, nsa_slc_workspace_bytes) switches to the block-major schedule: every K/V
  *   block is loaded once and the queries that picked it are gathered, instead of gathering the
- *   blocks per token; results agree to rounding.  NULL keeps the token-major kernel. */
+ *   blocks per token; results agree to rounding.  NULL keeps the token-major kernel.
+ *   lse_slc (optional, float [total,hq]; block-major schedule only) receives the log-sum-exp of the
+ *   scaled scores over the token's selected keys (lse_slc of nsa/selection_attn.py:476-481), +inf
+ *   for a token without usable block. */
 int nsa_slc_combine_fwd(const void* q, const void* k, const void* vt, const void* indices,
                         const int32_t* counts, const void* g_slc, const void* g_swa, const void* g_cmp,
-                        int64_t gate_stride, const void* o_swa, const void* o_cmp, void* out,
+                        int64_t gate_stride, const void* o_swa, const void* o_cmp, void* out, float* lse_slc,
                         const int32_t* cu_seqlens, int batch, int total, int hq, int hkv, int dk, int dv,
                         int vt_cols, int top_n, int block_size, float scale, int idx64, int gate_act,
                         int dtype, void* workspace, int64_t workspace_bytes, nsa_stream_t stream);
@@ -155,6 +163,39 @@ int nsa_swa_merge_fwd(const void* q, const void* k, const void* vt, const void* 
 /* Bytes of the optional workspace of nsa_slc_combine_fwd; 0 when the shape has no block-major path
  * (bf16, selection blocks of 64 keys only). */
 int64_t nsa_slc_workspace_bytes(int total, int batch, int hkv, int dk, int dv, int top_n, int block_size, int dtype);
+
+/* Backward of the compressed attention.  Replaces nsa/triton_attention.py:478-546
+ * (_attention.backward: _attn_bwd_preprocess, _attn_bwd with its dkdv / dq halves, :184-416).
+ *   q [total,hq,dk], ck [cmp_rows,hkv,dk], cv [cmp_rows,hkv,dv] packed over cu_cmp (one row set per
+ *   kv head, not repeated per q head), o / d_o [total,hq,dv] the forward output and its gradient,
+ *   lse = lse_attn of nsa_cmp_attn_fwd.  Outputs dq [total,hq,dk], dck, dcv (shapes of ck, cv), all
+ *   fully overwritten.  The block selection has no gradient (indices are integers).
+ *   workspace: nsa_cmp_attn_bwd_workspace_bytes, caller allocated. */
+int64_t nsa_cmp_attn_bwd_workspace_bytes(int total, int cmp_rows, int hq, int hkv, int dk, int dv);
+int nsa_cmp_attn_bwd(const void* q, const void* ck, const void* cv, const void* o, const void* d_o, const float* lse,
+                     const int32_t* cu_seqlens, const int32_t* cu_cmp, int batch, int total, int cmp_rows, int hq,
+                     int hkv, int dk, int dv, int block, int stride, float scale, int causal, int dtype, void* dq,
+                     void* dck, void* dcv, void* workspace, int64_t workspace_bytes, nsa_stream_t stream);
+
+/* Backward of the selected and the sliding-window attention.  Replaces
+ * nsa/selection_attn.py:715-737 (ParallelNSAFunction.backward -> parallel_nsa_bwd :151-398 with
+ * parallel_nsa_bwd_kernel_preprocess, _dq, _dkv :520-676 and the block mask :60-87).
+ *   q [total,hq,dk], k [total,hkv,dk], v [total,hkv,dv] (row-major, not the transposed copy);
+ *   o_slc / d_o_slc / lse_slc: ungated output of the selected branch, its gradient, and lse_slc of
+ *   nsa_slc_combine_fwd; o_swa / d_o_swa / lse_swa likewise for the window (lse of nsa_swa_fwd).
+ *   A branch is skipped when its d_o is NULL.  indices / counts / idx64 / top_n / block_size as in
+ *   nsa_slc_combine_fwd (64-key blocks only).  dq [total,hq,dk], dk_out [total,hkv,dk], dv_out
+ *   [total,hkv,dv] receive the sums over the branches present and are fully overwritten.
+ *   workspace: nsa_slc_swa_bwd_workspace_bytes (pass top_n = 0 there when the selected branch is
+ *   skipped). */
+int64_t nsa_slc_swa_bwd_workspace_bytes(int total, int batch, int hq, int hkv, int dk, int dv, int top_n,
+                                        int block_size, int dtype);
+int nsa_slc_swa_bwd(const void* q, const void* k, const void* v, const void* o_slc, const void* o_swa,
+                    const void* d_o_slc, const void* d_o_swa, const float* lse_slc, const float* lse_swa,
+                    const void* indices, const int32_t* counts, const int32_t* cu_seqlens, int batch, int total, int hq,
+                    int hkv, int dk, int dv, int top_n, int block_size, int window, float scale, int idx64, int dtype,
+                    void* dq, void* dk_out, void* dv_out, void* workspace, int64_t workspace_bytes,
+                    nsa_stream_t stream);
 
 /* One-token decode step (no counterpart in the reference, which has no cache and no single-token
  * path; defined as the last row of the prefill forward on the same keys/values, mean-pool

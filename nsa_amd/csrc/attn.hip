@@ -29,6 +29,7 @@ struct StreamParams {
   int block, stride, window, causal;
   float scale;
   MergeArgs mg;      // MERGE kernels only: the selected-attention partials and the other branches
+  float* lse_attn;   // optional: log-sum-exp (natural log) of the scaled visible scores, for the backward
 };
 
 // MERGE (sliding window only): 0 = write the branch output; otherwise the epilogue merges the
@@ -305,6 +306,8 @@ stream_attn_kernel(const StreamParams a) {
         }
       }
     }
+    if (a.lse_attn != nullptr && rm[j].valid && g == 0)
+      a.lse_attn[row] = lt > 0.f ? fmaf(grp[j].m, a.scale, __logf(lt)) : __builtin_huge_valf();
     if (CMP && a.lse != nullptr) {
       const float lit = colgroup_sum(li[j]);
       if (rm[j].valid && g == 0) a.lse[row] = nkeys > 0 ? grp[j].m + __logf(lit) : 0.f;
@@ -519,21 +522,21 @@ static int launch_stream_t(const StreamParams& a, int total, hipStream_t st) {
 template <typename T, int DK, int DV>
 static int launch_cmp_t(const CmpArgs& a, hipStream_t st) {
   StreamParams p{a.q, a.ck, a.cvt, a.o, a.lse, a.cu_seq, a.cu_cmp, a.batch, a.hq, a.hkv, a.ck_row_stride,
-                 a.ck_head_stride, a.cvt_cols, a.block, a.stride, 0, a.causal, a.scale, MergeArgs{}};
+                 a.ck_head_stride, a.cvt_cols, a.block, a.stride, 0, a.causal, a.scale, MergeArgs{}, a.lse_attn};
   return launch_stream_t<T, DK, DV, true>(p, a.total, st);
 }
 
 template <typename T, int DK, int DV>
 static int launch_swa_t(const SwaArgs& a, hipStream_t st) {
   StreamParams p{a.q, a.k, a.vt, a.o, nullptr, a.cu_seq, a.cu_seq, a.batch, a.hq, a.hkv, (long)a.hkv * DK,
-                 (long)DK, a.vt_cols, 0, 0, a.window, 1, a.scale, MergeArgs{}};
+                 (long)DK, a.vt_cols, 0, 0, a.window, 1, a.scale, MergeArgs{}, a.lse};
   return launch_stream_t<T, DK, DV, false>(p, a.total, st);
 }
 
 template <int DK, int DV>
 static int launch_swa_merge_t(const SwaArgs& a, const MergeArgs& m, hipStream_t st) {
   StreamParams p{a.q, a.k, a.vt, nullptr, nullptr, a.cu_seq, a.cu_seq, a.batch, a.hq, a.hkv, (long)a.hkv * DK,
-                 (long)DK, a.vt_cols, 0, 0, a.window, 1, a.scale, m};
+                 (long)DK, a.vt_cols, 0, 0, a.window, 1, a.scale, m, nullptr};
   if (m.top_n == 16) return launch_stream_t<bf16_t, DK, DV, false, 16>(p, a.total, st);
   return launch_stream_t<bf16_t, DK, DV, false, 1>(p, a.total, st);
 }
@@ -585,6 +588,7 @@ int launch_slc_combine(const SlcArgs& a, hipStream_t st) {
   // block-major path when the caller lent a large enough workspace and the shape qualifies
   if (a.workspace != nullptr && slc_block_major_ok(a) && a.workspace_bytes >= slc_workspace_bytes(a))
     return launch_slc_block_major(a, a.workspace, st);
+  if (a.lse != nullptr) return -5;              // only the block-major schedule produces the log-sum-exp
   NSA_DISPATCH(launch_slc_t, a, st);
 }
 

@@ -1,0 +1,709 @@
+// Backward of the three attention branches (reference: nsa/triton_attention.py:184-416,478-546 for
+// the compressed branch, nsa/selection_attn.py:151-398,520-676 for the selected and sliding
+// branches).  Given dO, the forward's O and log-sum-exp per row:
+//   delta = rowsum(dO * O),  P = exp(scale*S - lse),  dP = dO V^T,  dS = P * (dP - delta)
+//   dV = P^T dO,  dK = scale * dS^T Q,  dQ = scale * dS K
+//
+// Two kernel shapes, both built on 16x16x32 MFMA tiles and the fragment convention of tiles.h:
+//
+//  * key-stationary (dK, dV): a wavefront keeps 16 keys as B operands (K rows for S = Q K^T, V rows
+//    for dP = dO V^T) and its dK^T / dV^T accumulators in registers; query rows stream through LDS in
+//    chunks of 32 rows (2 tokens x 16 heads of the GQA group), Q and dO row-major.  The score tile
+//    comes out with lane = key, registers = rows, which after the 8-row permutation of tiles.h is
+//    directly the B operand of dV^T = dO^T P and dK^T = Q^T dS.  Their A operands (Q^T, dO^T: rows =
+//    channels, depth = query rows) are read from the same row-major LDS tiles with the transposing
+//    LDS load of gfx950 (ds_read_b64_tr_b16), so no transposed copy of Q or dO exists anywhere.
+//    The three branches differ only in which tokens stream past a key tile: the tokens of a window
+//    (sliding), all later tokens in segments (compressed), the tokens that picked the block
+//    (selected, from the bucketed pair list of the block-major forward).  dK / dV are accumulated
+//    into fp32 buffers with atomics (a key tile is shared by several work items in two of the three).
+//    The selected branch also produces dQ here: dS goes through LDS to become a B operand with
+//    lane = query row, and dQ^T = K^T dS^T is written as one partial per (token, pick) pair, summed
+//    per token by slc_dq_merge_kernel.
+//
+//  * query-stationary (dQ of the compressed and sliding branches): a wavefront keeps one token's 16
+//    heads (Q and dO rows as B operands, dQ^T accumulators); keys stream through LDS in chunks of 32
+//    (K and V row-major; K^T for dQ^T = K^T dS^T again through the transposing load).
+#include "slc_ws.h"
+#include "tiles.h"
+
+namespace nsa {
+
+int set_smem(const void* fn, size_t bytes);
+
+constexpr int kBwdCmp = 0, kBwdSwa = 1, kBwdSlc = 2;
+constexpr int kCmpSplit = 1024;      // tokens of one compressed-branch work item
+
+struct BwdArgs {
+  const void* q; const void* d_o; const float* lse; const float* delta;    // rows: [total][hq][.]
+  const void* k; const void* v;                                          // keys: [key rows][hkv][.]
+  const int32_t* cu_seq; const int32_t* cu_key;
+  int batch, total, hq, hkv;
+  int block, stride, causal, window;
+  float scale;
+  void* dq;                       // query-stationary: [total][hq][dk]
+  float* dk_acc; float* dv_acc;   // key-stationary: fp32 [key rows][hkv][.]
+  SlcWs ws;                       // selected branch: bucketed pairs; ws.po = dq partials [pair][16][dk]
+};
+
+// ---- transposing fragment load ---------------------------------------------------------------------
+// tile points at element (row0, col0) of a row-major LDS tile with row pitch ld.  Lane (m = lane%16,
+// g = lane/16) receives tile[8g + j][m], j = 0..7: the A operand of a product whose depth runs over
+// the tile's rows.  bf16: two ds_read_b64_tr_b16, each transposing a 4 x 16 block per 16 lanes (lane
+// 4a+b supplies the address of row a, columns 4b..4b+3 and receives column 4a'+b' of rows 0..3).
+__device__ __forceinline__ bf16x8_t load8_tr(const bf16_t* tile, int ld, int lane) {
+  typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
+  typedef __attribute__((address_space(3))) bf16x4_t lds_bf16x4_t;
+  const int i = lane & 15, g = lane >> 4;
+  const bf16_t* p = tile + (8 * g + (i >> 2)) * ld + 4 * (i & 3);
+  const bf16x4_t a = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_t*)p);
+  const bf16x4_t b = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_t*)(p + 4 * ld));
+  bf16x8_t r;
+  r[0] = a[0]; r[1] = a[1]; r[2] = a[2]; r[3] = a[3];
+  r[4] = b[0]; r[5] = b[1]; r[6] = b[2]; r[7] = b[3];
+  return r;
+}
+__device__ __forceinline__ f32x8_t load8_tr(const float* tile, int ld, int lane) {
+  const int m = lane & 15, g = lane >> 4;
+  f32x8_t r;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) r[j] = tile[(8 * g + j) * ld + m];
+  return r;
+}
+
+// Two 16-row tiles of X[32 rows][D] (LDS, permuted rows) times the stationary fragments f[D/32].
+template <typename T, int D>
+__device__ __forceinline__ void tile_pair(const T* __restrict__ x, int ld, int n, int g, const vec8_t<T> (&f)[D / 32],
+                                          float (&out)[8]) {
+  f32x4_t t0 = {0.f, 0.f, 0.f, 0.f}, t1 = {0.f, 0.f, 0.f, 0.f};
+  const T* r0 = x + chunk_key_of_row(0, n) * ld + 8 * g;
+  const T* r1 = x + chunk_key_of_row(1, n) * ld + 8 * g;
+#pragma unroll
+  for (int kk = 0; kk < D / 32; ++kk) {
+    t0 = mma16(load8(r0 + 32 * kk), f[kk], t0);
+    t1 = mma16(load8(r1 + 32 * kk), f[kk], t1);
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { out[i] = t0[i]; out[4 + i] = t1[i]; }
+}
+
+__device__ __forceinline__ void store4(bf16_t* p, const f32x4_t& v, float s) {
+  typedef __bf16 bf16x4v __attribute__((ext_vector_type(4)));
+  bf16x4v r;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) r[i] = (bf16_t)(v[i] * s);
+  *reinterpret_cast<bf16x4v*>(p) = r;
+}
+__device__ __forceinline__ void store4(float* p, const f32x4_t& v, float s) {
+  f32x4_t r;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) r[i] = v[i] * s;
+  *reinterpret_cast<f32x4_t*>(p) = r;
+}
+
+// ---- key-stationary: dK, dV (and the dQ partials of the selected branch) ---------------------------
+
+template <typename T, int DK, int DV, int MODE, int NW>
+__global__ void __launch_bounds__(NW * 64)
+bwd_kv_kernel(const BwdArgs a) {
+  constexpr int QLD = DK + 8, OLD = DV + 8, NT = NW * 64, SLD = kBlk + 8;
+  constexpr int QP = 32 * DK / 8, OP = 32 * DV / 8;                 // 16-byte pieces of one chunk
+  constexpr int QPT = (QP + NT - 1) / NT, OPT = (OP + NT - 1) / NT;
+  constexpr int STAGE = 32 * QLD + 32 * OLD;
+  static_assert(MODE != kBwdSlc || NW * 16 == kBlk, "the selected branch keeps one 64-key block per workgroup");
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  T* lds = reinterpret_cast<T*>(smem_raw);                          // [2][Q 32 x QLD | dO 32 x OLD]
+  float* stat = reinterpret_cast<float*>(lds + 2 * STAGE);          // [2][lse2 32 | delta 32]
+  T* kblk = reinterpret_cast<T*>(stat + 128);                       // selected branch: K block [64][QLD]
+  T* dsl = kblk + kBlk * QLD;                                       //                  dS [32][SLD]
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 15, g = lane >> 4;
+  const int G = a.hq / a.hkv;
+
+  // ---- work item
+  int h, seq_start, key0, nkeys, key_base;
+  int t_begin = 0, t_end = 0, first = 0, count = 0, nchunks;
+  if (MODE == kBwdSlc) {
+    const int item = blockIdx.x;
+    if (item >= *a.ws.n_items) return;
+    const int key = a.ws.items[2 * item], seg = a.ws.items[2 * item + 1];
+    h = key / a.ws.nb;
+    const SeqTile st = find_tile(a.cu_seq, a.batch, kBlk, key % a.ws.nb);
+    if (!st.valid) return;
+    seq_start = st.start; key0 = st.t0; nkeys = st.len; key_base = st.start;
+    first = a.ws.offsets[key] + seg * kSeg;
+    count = min(a.ws.counts[key] - seg * kSeg, kSeg);
+    nchunks = (count + 1) >> 1;
+  } else if (MODE == kBwdSwa) {
+    const SeqTile st = find_tile(a.cu_seq, a.batch, NW * 16, blockIdx.x);
+    if (!st.valid) return;
+    h = blockIdx.y;
+    seq_start = st.start; key0 = st.t0; nkeys = st.len; key_base = st.start;
+    t_begin = key0;
+    t_end = min(key0 + NW * 16 + a.window - 1, st.len);
+    nchunks = (t_end - t_begin + 1) >> 1;
+  } else {
+    const SeqTile st = find_tile(a.cu_key, a.batch, NW * 16, blockIdx.y);
+    if (!st.valid) return;
+    h = blockIdx.z;
+    key0 = st.t0; nkeys = st.len; key_base = st.start;
+    seq_start = a.cu_seq[st.b];
+    const int seq_len = a.cu_seq[st.b + 1] - seq_start;
+    const int t_first = a.causal ? key0 * a.stride + a.block : 0;
+    t_begin = max((int)blockIdx.x * kCmpSplit, t_first) & ~1;
+    t_end = min(((int)blockIdx.x + 1) * kCmpSplit, seq_len);
+    if (t_begin >= t_end) return;
+    nchunks = (t_end - t_begin + 1) >> 1;
+  }
+  if (nchunks <= 0) return;
+
+  const T* qb = reinterpret_cast<const T*>(a.q);
+  const T* dob = reinterpret_cast<const T*>(a.d_o);
+
+  // tokens of chunk c: positions inside the sequence (pos*), validity of the second one
+  auto chunk_tokens = [&](int c, int& posA, int& posB, bool& vB) {
+    if (MODE == kBwdSlc) {
+      posA = (int)(a.ws.list[first + 2 * c] >> 6) - seq_start;
+      vB = 2 * c + 1 < count;
+      posB = vB ? (int)(a.ws.list[first + 2 * c + 1] >> 6) - seq_start : posA;
+    } else {
+      posA = t_begin + 2 * c;
+      vB = posA + 1 < t_end;
+      posB = vB ? posA + 1 : posA;
+    }
+  };
+
+  // ---- stationary fragments: 16 keys of this wavefront
+  const int keypos = key0 + 16 * wave + n;
+  const bool keyvalid = keypos < nkeys;
+  vec8_t<T> kf[DK / 32], vf[DV / 32];
+  {
+    const long krow = (long)(key_base + min(keypos, nkeys - 1)) * a.hkv + h;
+    const T* kp = reinterpret_cast<const T*>(a.k) + krow * DK + 8 * g;
+    const T* vp = reinterpret_cast<const T*>(a.v) + krow * DV + 8 * g;
+#pragma unroll
+    for (int kk = 0; kk < DK / 32; ++kk) kf[kk] = load8(kp + 32 * kk);
+#pragma unroll
+    for (int kk = 0; kk < DV / 32; ++kk) vf[kk] = load8(vp + 32 * kk);
+  }
+  if (MODE == kBwdSlc) {                      // the whole block row-major, for dQ^T = K^T dS^T
+    for (int p = tid; p < kBlk * DK / 8; p += NT) {
+      const int r = p / (DK / 8), pc = p % (DK / 8);
+      const long krow = (long)(key_base + min(key0 + r, nkeys - 1)) * a.hkv + h;
+      store8(kblk + r * QLD + pc * 8, load8(reinterpret_cast<const T*>(a.k) + krow * DK + pc * 8));
+    }
+  }
+  f32x4_t dk_acc[DK / 16], dv_acc[DV / 16];
+#pragma unroll
+  for (int t = 0; t < DK / 16; ++t) dk_acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int t = 0; t < DV / 16; ++t) dv_acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  // ---- staging of one chunk: global -> registers -> LDS
+  vec8_t<T> qr[QPT], orr[OPT];
+  float sr = 0.f;
+  auto gload = [&](int c) {
+    int posA, posB; bool vB;
+    chunk_tokens(c, posA, posB, vB);
+#pragma unroll
+    for (int i = 0; i < QPT; ++i) {
+      const int p = tid + i * NT;
+      if (QP % NT == 0 || p < QP) {
+        const int r = p / (DK / 8), pc = p % (DK / 8);
+        const long tg = seq_start + ((r >> 4) ? posB : posA);
+        qr[i] = load8(qb + (tg * a.hq + h * G + min(r & 15, G - 1)) * DK + pc * 8);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < OPT; ++i) {
+      const int p = tid + i * NT;
+      if (OP % NT == 0 || p < OP) {
+        const int r = p / (DV / 8), pc = p % (DV / 8);
+        const long tg = seq_start + ((r >> 4) ? posB : posA);
+        orr[i] = load8(dob + (tg * a.hq + h * G + min(r & 15, G - 1)) * DV + pc * 8);
+      }
+    }
+    if (tid < 64) {
+      const int r = tid & 31;
+      const long tg = seq_start + ((r >> 4) ? posB : posA);
+      const long row = tg * a.hq + h * G + min(r & 15, G - 1);
+      sr = tid < 32 ? a.lse[row] * kLog2e : a.delta[row];
+    }
+  };
+  auto lstore = [&](int buf) {
+    T* qs = lds + buf * STAGE;
+    T* os = qs + 32 * QLD;
+#pragma unroll
+    for (int i = 0; i < QPT; ++i) {
+      const int p = tid + i * NT;
+      if (QP % NT == 0 || p < QP) store8(qs + (p / (DK / 8)) * QLD + (p % (DK / 8)) * 8, qr[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < OPT; ++i) {
+      const int p = tid + i * NT;
+      if (OP % NT == 0 || p < OP) store8(os + (p / (DV / 8)) * OLD + (p % (DV / 8)) * 8, orr[i]);
+    }
+    if (tid < 64) stat[buf * 64 + tid] = sr;
+  };
+
+  const float c_attn = a.scale * kLog2e;
+  gload(0);
+  lstore(0);
+  __syncthreads();
+  int buf = 0;
+  for (int c = 0; c < nchunks; ++c) {
+    const bool has_next = c + 1 < nchunks;
+    if (has_next) gload(c + 1);
+
+    const T* qs = lds + buf * STAGE;
+    const T* os = qs + 32 * QLD;
+    const float* ss = stat + buf * 64;
+    int posA, posB; bool vB;
+    chunk_tokens(c, posA, posB, vB);
+    // the 8 rows of this lane (8g .. 8g+7) are heads 8(g&1) .. +7 of one token
+    const int tokpos = (g >> 1) ? posB : posA;
+    bool vis = keyvalid && ((g >> 1) == 0 || vB);
+    if (MODE == kBwdSwa) vis = vis && keypos <= tokpos && keypos > tokpos - a.window;
+    else if (MODE == kBwdSlc) vis = vis && keypos <= tokpos;
+    else if (a.causal) vis = vis && keypos * a.stride + a.block <= tokpos;
+
+    float s[8], dp[8], p[8], ds[8];
+    tile_pair<T, DK>(qs, QLD, n, g, kf, s);
+    tile_pair<T, DV>(os, OLD, n, g, vf, dp);
+    const f32x4_t l0 = *reinterpret_cast<const f32x4_t*>(ss + 8 * g);
+    const f32x4_t l1 = *reinterpret_cast<const f32x4_t*>(ss + 8 * g + 4);
+    const f32x4_t e0 = *reinterpret_cast<const f32x4_t*>(ss + 32 + 8 * g);
+    const f32x4_t e1 = *reinterpret_cast<const f32x4_t*>(ss + 32 + 8 * g + 4);
+    const int hbase = 8 * (g & 1);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float lse2 = j < 4 ? l0[j & 3] : l1[j & 3];
+      const float dl = j < 4 ? e0[j & 3] : e1[j & 3];
+      const bool ok = vis && hbase + j < G;
+      const float e = fast_exp2(fmaf(s[j], c_attn, -lse2));
+      p[j] = ok ? e : 0.f;
+      ds[j] = ok ? e * (dp[j] - dl) : 0.f;
+    }
+    const vec8_t<T> pb = pack8<T>(p), dsb = pack8<T>(ds);
+    if (MODE == kBwdSlc) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) dsl[(8 * g + j) * SLD + 16 * wave + n] = dsb[j];
+      __syncthreads();
+    }
+#pragma unroll
+    for (int t = 0; t < DV / 16; ++t) dv_acc[t] = mma16(load8_tr(os + 16 * t, OLD, lane), pb, dv_acc[t]);
+#pragma unroll
+    for (int t = 0; t < DK / 16; ++t) dk_acc[t] = mma16(load8_tr(qs + 16 * t, QLD, lane), dsb, dk_acc[t]);
+
+    if (MODE == kBwdSlc) {
+      // dQ^T[dk][row] = sum_key K[key][dk] dS[row][key]: this wavefront takes every NW-th 16-channel tile
+      T* part = reinterpret_cast<T*>(a.ws.po);
+#pragma unroll
+      for (int t = wave; t < DK / 16; t += NW) {
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+          if (r == 1 && !vB) break;
+          f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int step = 0; step < 2; ++step)
+            acc = mma16(load8_tr(kblk + 32 * step * QLD + 16 * t, QLD, lane),
+                        load8(dsl + (16 * r + n) * SLD + 32 * step + 8 * g), acc);
+          store4(part + ((long)(first + 2 * c + r) * 16 + n) * DK + 16 * t + 4 * g, acc, a.scale);
+        }
+      }
+    }
+
+    if (has_next) lstore(buf ^ 1);
+    __syncthreads();
+    buf ^= 1;
+  }
+
+  if (keyvalid) {
+    const long krow = (long)(key_base + keypos) * a.hkv + h;
+    float* dkp = a.dk_acc + krow * DK + 4 * g;
+    float* dvp = a.dv_acc + krow * DV + 4 * g;
+#pragma unroll
+    for (int t = 0; t < DK / 16; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) unsafeAtomicAdd(dkp + 16 * t + i, dk_acc[t][i] * a.scale);
+#pragma unroll
+    for (int t = 0; t < DV / 16; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) unsafeAtomicAdd(dvp + 16 * t + i, dv_acc[t][i]);
+  }
+}
+
+// ---- query-stationary: dQ of the compressed and sliding branches -----------------------------------
+
+template <typename T, int DK, int DV, int MODE, int NW>
+__global__ void __launch_bounds__(NW * 64)
+bwd_q_kernel(const BwdArgs a) {
+  constexpr int KLD = DK + 8, VLD = DV + 8, NT = NW * 64;
+  constexpr int KP = 32 * DK / 8, VP = 32 * DV / 8;
+  constexpr int KPT = (KP + NT - 1) / NT, VPT = (VP + NT - 1) / NT;
+  constexpr int STAGE = 32 * KLD + 32 * VLD;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  T* lds = reinterpret_cast<T*>(smem_raw);                          // [2][K 32 x KLD | V 32 x VLD]
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 15, g = lane >> 4;
+  const int G = a.hq / a.hkv;
+  const SeqTile st = find_tile(a.cu_seq, a.batch, NW, blockIdx.x);
+  if (!st.valid) return;
+  const int h = blockIdx.y;
+  const int tok = st.t0 + wave;
+  const bool tokvalid = tok < st.len;
+  const int t_last = min(st.t0 + NW, st.len) - 1;
+
+  int koff, nkeys;
+  if (MODE == kBwdCmp) { koff = a.cu_key[st.b]; nkeys = a.cu_key[st.b + 1] - koff; }
+  else { koff = st.start; nkeys = st.len; }
+  auto last_visible = [&](int t) -> int {
+    if (MODE == kBwdSwa) return t;
+    if (!a.causal) return nkeys - 1;
+    return t >= a.block ? min((t - a.block) / a.stride, nkeys - 1) : -1;
+  };
+  const int c_begin = MODE == kBwdSwa ? (max(st.t0 - a.window + 1, 0) & ~31) : 0;
+  const int c_end = last_visible(t_last) + 1;
+  const int my_hi = tokvalid ? last_visible(tok) : -1;
+  const int my_lo = MODE == kBwdSwa ? tok - a.window + 1 : 0;
+
+  vec8_t<T> qf[DK / 32], dof[DV / 32];
+  float lse2, dl;
+  {
+    const long row = ((long)st.start + min(tok, st.len - 1)) * a.hq + h * G + min(n, G - 1);
+    const T* qp = reinterpret_cast<const T*>(a.q) + row * DK + 8 * g;
+    const T* dp = reinterpret_cast<const T*>(a.d_o) + row * DV + 8 * g;
+#pragma unroll
+    for (int kk = 0; kk < DK / 32; ++kk) qf[kk] = load8(qp + 32 * kk);
+#pragma unroll
+    for (int kk = 0; kk < DV / 32; ++kk) dof[kk] = load8(dp + 32 * kk);
+    lse2 = a.lse[row] * kLog2e;
+    dl = a.delta[row];
+  }
+  f32x4_t acc[DK / 16];
+#pragma unroll
+  for (int t = 0; t < DK / 16; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  const T* kb = reinterpret_cast<const T*>(a.k) + ((long)koff * a.hkv + h) * DK;
+  const T* vb = reinterpret_cast<const T*>(a.v) + ((long)koff * a.hkv + h) * DV;
+  vec8_t<T> kr[KPT], vr[VPT];
+  auto gload = [&](int c0) {
+#pragma unroll
+    for (int i = 0; i < KPT; ++i) {
+      const int p = tid + i * NT;
+      if (KP % NT == 0 || p < KP) {
+        const int r = min(c0 + p / (DK / 8), nkeys - 1);
+        kr[i] = load8(kb + (long)r * a.hkv * DK + (p % (DK / 8)) * 8);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int p = tid + i * NT;
+      if (VP % NT == 0 || p < VP) {
+        const int r = min(c0 + p / (DV / 8), nkeys - 1);
+        vr[i] = load8(vb + (long)r * a.hkv * DV + (p % (DV / 8)) * 8);
+      }
+    }
+  };
+  auto lstore = [&](int buf) {
+    T* ks = lds + buf * STAGE;
+    T* vs = ks + 32 * KLD;
+#pragma unroll
+    for (int i = 0; i < KPT; ++i) {
+      const int p = tid + i * NT;
+      if (KP % NT == 0 || p < KP) store8(ks + (p / (DK / 8)) * KLD + (p % (DK / 8)) * 8, kr[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int p = tid + i * NT;
+      if (VP % NT == 0 || p < VP) store8(vs + (p / (DV / 8)) * VLD + (p % (DV / 8)) * 8, vr[i]);
+    }
+  };
+
+  const float c_attn = a.scale * kLog2e;
+  if (c_begin < c_end) {
+    gload(c_begin);
+    lstore(0);
+  }
+  __syncthreads();
+  int buf = 0;
+  for (int c0 = c_begin; c0 < c_end; c0 += 32) {
+    const bool has_next = c0 + 32 < c_end;
+    if (has_next) gload(c0 + 32);
+    if (c0 <= my_hi && c0 + 31 >= my_lo) {           // wavefront uniform: one token per wavefront
+      const T* ks = lds + buf * STAGE;
+      const T* vs = ks + 32 * KLD;
+      float s[8], dp[8], ds[8];
+      tile_pair<T, DK>(ks, KLD, n, g, qf, s);
+      tile_pair<T, DV>(vs, VLD, n, g, dof, dp);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int key = c0 + 8 * g + j;
+        const bool ok = key >= my_lo && key <= my_hi && n < G;
+        const float e = fast_exp2(fmaf(s[j], c_attn, -lse2));
+        ds[j] = ok ? e * (dp[j] - dl) : 0.f;
+      }
+      const vec8_t<T> dsb = pack8<T>(ds);
+#pragma unroll
+      for (int t = 0; t < DK / 16; ++t) acc[t] = mma16(load8_tr(ks + 16 * t, KLD, lane), dsb, acc[t]);
+    }
+    if (has_next) lstore(buf ^ 1);
+    __syncthreads();
+    buf ^= 1;
+  }
+
+  if (tokvalid && n < G) {
+    T* dqp = reinterpret_cast<T*>(a.dq) + (((long)st.start + tok) * a.hq + h * G + n) * DK + 4 * g;
+#pragma unroll
+    for (int t = 0; t < DK / 16; ++t) store4(dqp + 16 * t, acc[t], a.scale);
+  }
+}
+
+// ---- small kernels ------------------------------------------------------------------------------
+
+// delta[row] = sum_v o[row][v] * d_o[row][v]; 16 lanes per row
+template <typename T>
+__global__ void __launch_bounds__(256)
+bwd_delta_kernel(const T* __restrict__ o, const T* __restrict__ d_o, float* __restrict__ delta, long rows, int dv) {
+  const long row = ((long)blockIdx.x * 256 + threadIdx.x) >> 4;
+  const int sub = threadIdx.x & 15;
+  float acc = 0.f;
+  if (row < rows) {
+    for (int c = sub * 8; c < dv; c += 128) {
+      const vec8_t<T> x = load8(o + row * dv + c), y = load8(d_o + row * dv + c);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc = fmaf((float)x[i], (float)y[i], acc);
+    }
+  }
+#pragma unroll
+  for (int d = 1; d < 16; d <<= 1) acc += __shfl_xor(acc, d, 16);
+  if (row < rows && sub == 0) delta[row] = acc;
+}
+
+__global__ void __launch_bounds__(256)
+bwd_fill_kernel(float* __restrict__ p, long n4) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i < n4) reinterpret_cast<f32x4_t*>(p)[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+bwd_cast_kernel(const float* __restrict__ src, T* __restrict__ dst, long n8) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n8) return;
+  float v[8];
+  const f32x8_t x = load8(src + i * 8);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) v[e] = x[e];
+  store8(dst + i * 8, pack8<T>(v));
+}
+
+// dq[token][head][8 channels] = (dq_in) + sum over the token's usable picks of the pair partials
+template <typename T, int DK>
+__global__ void __launch_bounds__(256)
+slc_dq_merge_kernel(const int* __restrict__ slotmap, const T* __restrict__ part, const T* __restrict__ dq_in,
+                    T* __restrict__ dq, long total, int hq, int hkv, int top_n) {
+  constexpr int PPR = DK / 8;
+  const long id = (long)blockIdx.x * 256 + threadIdx.x;
+  if (id >= total * hq * PPR) return;
+  const int pc = (int)(id % PPR);
+  const long row = id / PPR;
+  const int hq_i = (int)(row % hq);
+  const long tg = row / hq;
+  const int G = hq / hkv;
+  const int h = hq_i / G, n = hq_i % G;
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  if (dq_in != nullptr) {
+    const vec8_t<T> x = load8(dq_in + row * DK + pc * 8);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = (float)x[e];
+  }
+  const long base = (tg * hkv + h) * top_n;
+  for (int i = 0; i < top_n; ++i) {
+    const long p = slotmap[base + i];
+    if (p < 0) continue;
+    const vec8_t<T> x = load8(part + (p * 16 + n) * DK + pc * 8);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] += (float)x[e];
+  }
+  store8(dq + row * DK + pc * 8, pack8<T>(acc));
+}
+
+// ---- launchers ------------------------------------------------------------------------------------
+
+template <typename T, int DK, int DV, int MODE, int NW>
+static int launch_kv_t(const BwdArgs& a, int key_rows, hipStream_t st) {
+  size_t smem = 2 * (size_t)(32 * (DK + 8) + 32 * (DV + 8)) * sizeof(T) + 128 * sizeof(float);
+  if (MODE == kBwdSlc) smem += ((size_t)kBlk * (DK + 8) + 32 * (kBlk + 8)) * sizeof(T);
+  auto fn = bwd_kv_kernel<T, DK, DV, MODE, NW>;
+  const int rc = set_smem(reinterpret_cast<const void*>(fn), smem);
+  if (rc) return rc;
+  dim3 grid;
+  if (MODE == kBwdSlc) grid = dim3(a.ws.items_cap);
+  else if (MODE == kBwdSwa) grid = dim3(key_rows / (NW * 16) + a.batch, a.hkv);
+  else grid = dim3((a.total + kCmpSplit - 1) / kCmpSplit, key_rows / (NW * 16) + a.batch, a.hkv);
+  hipLaunchKernelGGL(fn, grid, dim3(NW * 64), smem, st, a);
+  return 0;
+}
+
+template <typename T, int DK, int DV, int MODE>
+static int launch_q_t(const BwdArgs& a, hipStream_t st) {
+  constexpr int NW = 8;
+  const size_t smem = 2 * (size_t)(32 * (DK + 8) + 32 * (DV + 8)) * sizeof(T);
+  auto fn = bwd_q_kernel<T, DK, DV, MODE, NW>;
+  const int rc = set_smem(reinterpret_cast<const void*>(fn), smem);
+  if (rc) return rc;
+  hipLaunchKernelGGL(fn, dim3(a.total / NW + a.batch, a.hkv), dim3(NW * 64), smem, st, a);
+  return 0;
+}
+
+static void fill_zero(float* p, long n, hipStream_t st) {        // n is a multiple of 4
+  const long n4 = n / 4;
+  if (n4 > 0) hipLaunchKernelGGL(bwd_fill_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, st, p, n4);
+}
+template <typename T>
+static void cast_out(const float* src, void* dst, long n, hipStream_t st) {   // n is a multiple of 8
+  const long n8 = n / 8;
+  if (n8 > 0)
+    hipLaunchKernelGGL((bwd_cast_kernel<T>), dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, st, src,
+                       reinterpret_cast<T*>(dst), n8);
+}
+template <typename T>
+static void launch_delta(const void* o, const void* d_o, float* delta, long rows, int dv, hipStream_t st) {
+  hipLaunchKernelGGL((bwd_delta_kernel<T>), dim3((unsigned)((rows * 16 + 255) / 256)), dim3(256), 0, st,
+                     reinterpret_cast<const T*>(o), reinterpret_cast<const T*>(d_o), delta, rows, dv);
+}
+
+static long take(long& off, long bytes) { const long o = off; off = slc_align_up(off + bytes, 256); return o; }
+
+// compressed branch -----------------------------------------------------------------------------------
+
+long cmp_bwd_workspace_bytes(const CmpBwdArgs& a) {
+  long off = 0;
+  take(off, (long)a.total * a.hq * 4);
+  take(off, (long)a.cmp_rows * a.hkv * a.dk * 4);
+  take(off, (long)a.cmp_rows * a.hkv * a.dv * 4);
+  return off;
+}
+
+template <typename T, int DK, int DV>
+static int launch_cmp_bwd_t(const CmpBwdArgs& c, hipStream_t st) {
+  char* base = reinterpret_cast<char*>(c.workspace);
+  long off = 0;
+  float* delta = (float*)(base + take(off, (long)c.total * c.hq * 4));
+  float* dk_acc = (float*)(base + take(off, (long)c.cmp_rows * c.hkv * DK * 4));
+  float* dv_acc = (float*)(base + take(off, (long)c.cmp_rows * c.hkv * DV * 4));
+  launch_delta<T>(c.o, c.d_o, delta, (long)c.total * c.hq, DV, st);
+  BwdArgs a{};
+  a.q = c.q; a.d_o = c.d_o; a.lse = c.lse; a.delta = delta; a.k = c.ck; a.v = c.cv;
+  a.cu_seq = c.cu_seq; a.cu_key = c.cu_cmp; a.batch = c.batch; a.total = c.total; a.hq = c.hq; a.hkv = c.hkv;
+  a.block = c.block; a.stride = c.stride; a.causal = c.causal; a.window = 0; a.scale = c.scale;
+  a.dq = c.dq; a.dk_acc = dk_acc; a.dv_acc = dv_acc;
+  int rc = launch_q_t<T, DK, DV, kBwdCmp>(a, st);
+  if (rc) return rc;
+  if (c.cmp_rows > 0) {
+    fill_zero(dk_acc, (long)c.cmp_rows * c.hkv * DK, st);
+    fill_zero(dv_acc, (long)c.cmp_rows * c.hkv * DV, st);
+    rc = launch_kv_t<T, DK, DV, kBwdCmp, 8>(a, c.cmp_rows, st);
+    if (rc) return rc;
+    cast_out<T>(dk_acc, c.dck, (long)c.cmp_rows * c.hkv * DK, st);
+    cast_out<T>(dv_acc, c.dcv, (long)c.cmp_rows * c.hkv * DV, st);
+  }
+  return 0;
+}
+
+// selected + sliding branches ------------------------------------------------------------------------
+
+static SlcArgs slc_args_of(const SlcSwaBwdArgs& c) {
+  SlcArgs s{};
+  s.indices = c.indices; s.counts = c.counts; s.cu_seq = c.cu_seq; s.batch = c.batch; s.total = c.total;
+  s.hq = c.hq; s.hkv = c.hkv; s.dk = c.dk; s.dv = c.dv; s.top_n = c.top_n; s.block_size = c.block_size;
+  s.idx64 = c.idx64; s.dtype = c.dtype;
+  return s;
+}
+
+long slc_swa_bwd_workspace_bytes(const SlcSwaBwdArgs& c) {
+  long off = 0;
+  take(off, (long)c.total * c.hq * 4);
+  take(off, (long)c.total * c.hq * 4);
+  take(off, (long)c.total * c.hkv * c.dk * 4);
+  take(off, (long)c.total * c.hkv * c.dv * 4);
+  if (c.top_n > 0) off += slc_carve(slc_args_of(c), nullptr, nullptr, c.dtype == 0 ? 2 : 4, c.dk);
+  return off;
+}
+
+template <typename T, int DK, int DV>
+static int launch_slc_swa_bwd_t(const SlcSwaBwdArgs& c, hipStream_t st) {
+  char* base = reinterpret_cast<char*>(c.workspace);
+  long off = 0;
+  float* delta_slc = (float*)(base + take(off, (long)c.total * c.hq * 4));
+  float* delta_swa = (float*)(base + take(off, (long)c.total * c.hq * 4));
+  float* dk_acc = (float*)(base + take(off, (long)c.total * c.hkv * DK * 4));
+  float* dv_acc = (float*)(base + take(off, (long)c.total * c.hkv * DV * 4));
+  const bool slc = c.top_n > 0 && c.d_o_slc != nullptr, swa = c.window > 0 && c.d_o_swa != nullptr;
+  fill_zero(dk_acc, (long)c.total * c.hkv * DK, st);
+  fill_zero(dv_acc, (long)c.total * c.hkv * DV, st);
+  BwdArgs a{};
+  a.q = c.q; a.k = c.k; a.v = c.v; a.cu_seq = c.cu_seq; a.cu_key = c.cu_seq; a.batch = c.batch; a.total = c.total;
+  a.hq = c.hq; a.hkv = c.hkv; a.causal = 1; a.window = c.window; a.scale = c.scale;
+  a.dq = c.dq; a.dk_acc = dk_acc; a.dv_acc = dv_acc;
+  int rc = 0;
+  if (swa) {
+    launch_delta<T>(c.o_swa, c.d_o_swa, delta_swa, (long)c.total * c.hq, DV, st);
+    a.d_o = c.d_o_swa; a.lse = c.lse_swa; a.delta = delta_swa;
+    rc = launch_q_t<T, DK, DV, kBwdSwa>(a, st);
+    if (rc == 0) rc = launch_kv_t<T, DK, DV, kBwdSwa, 8>(a, c.total, st);
+    if (rc) return rc;
+  }
+  if (slc) {
+    const SlcArgs s = slc_args_of(c);
+    SlcWs ws;
+    slc_carve(s, base + off, &ws, sizeof(T), DK);
+    rc = launch_slc_bucket(s, ws, st);
+    if (rc) return rc;
+    launch_delta<T>(c.o_slc, c.d_o_slc, delta_slc, (long)c.total * c.hq, DV, st);
+    a.d_o = c.d_o_slc; a.lse = c.lse_slc; a.delta = delta_slc; a.ws = ws;
+    rc = launch_kv_t<T, DK, DV, kBwdSlc, 4>(a, c.total, st);
+    if (rc) return rc;
+    const long threads = (long)c.total * c.hq * (DK / 8);
+    hipLaunchKernelGGL((slc_dq_merge_kernel<T, DK>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st,
+                       ws.slotmap, reinterpret_cast<const T*>(ws.po),
+                       swa ? reinterpret_cast<const T*>(c.dq) : nullptr, reinterpret_cast<T*>(c.dq),
+                       (long)c.total, c.hq, c.hkv, c.top_n);
+  } else if (!swa) {
+    fill_zero(reinterpret_cast<float*>(c.dq), (long)c.total * c.hq * DK * (long)sizeof(T) / 4, st);
+  }
+  cast_out<T>(dk_acc, c.dk_out, (long)c.total * c.hkv * DK, st);
+  cast_out<T>(dv_acc, c.dv_out, (long)c.total * c.hkv * DV, st);
+  return 0;
+}
+
+#define NSA_BWD_DISPATCH(FN, ARGS, ST)                                                \
+  do {                                                                                \
+    const int key = (ARGS).dk * 1000 + (ARGS).dv;                                     \
+    if ((ARGS).dtype == 0) {                                                          \
+      switch (key) {                                                                  \
+        case 64064: return FN<bf16_t, 64, 64>(ARGS, ST);                              \
+        case 128128: return FN<bf16_t, 128, 128>(ARGS, ST);                           \
+        case 192128: return FN<bf16_t, 192, 128>(ARGS, ST);                           \
+        default: return -2;                                                           \
+      }                                                                               \
+    } else {                                                                          \
+      switch (key) {                                                                  \
+        case 64064: return FN<float, 64, 64>(ARGS, ST);                               \
+        case 128128: return FN<float, 128, 128>(ARGS, ST);                            \
+        default: return -2;                                                           \
+      }                                                                               \
+    }                                                                                 \
+  } while (0)
+
+int launch_cmp_bwd(const CmpBwdArgs& a, hipStream_t st) { NSA_BWD_DISPATCH(launch_cmp_bwd_t, a, st); }
+int launch_slc_swa_bwd(const SlcSwaBwdArgs& a, hipStream_t st) { NSA_BWD_DISPATCH(launch_slc_swa_bwd_t, a, st); }
+
+}  // namespace nsa

@@ -78,8 +78,8 @@ int nsa_transpose_fwd(const void* x, void* out, const int32_t* cu, int batch, in
 }
 
 static int cmp_common(const char* what, int stages, const void* q, const void* ck, const void* cvt, void* o,
-                      void* indices, float* pooled, float* lse, const int32_t* cu_seqlens, const int32_t* cu_cmp,
-                      int batch, int total, int hq, int hkv, int dk, int dv, int64_t ck_row_stride,
+                      void* indices, float* pooled, float* lse, float* lse_attn, const int32_t* cu_seqlens,
+                      const int32_t* cu_cmp, int batch, int total, int hq, int hkv, int dk, int dv, int64_t ck_row_stride,
                       int64_t ck_head_stride, int cvt_cols, int block, int stride, int pool_kernel, int pool_stride,
                       int pool_pad, int top_n, int max_ns, int pooled_stride, float scale, int causal, int idx64,
                       int dtype, nsa_stream_t stream) {
@@ -104,7 +104,7 @@ static int cmp_common(const char* what, int stages, const void* q, const void* c
   }
   nsa::CmpArgs a{q, ck, cvt, o, indices, pooled, lse, cu_seqlens, cu_cmp, batch, total, hq, hkv, dk, dv,
                  (long)ck_row_stride, (long)ck_head_stride, cvt_cols, block, stride, pool_kernel, pool_stride,
-                 pool_pad, top_n, max_ns, pooled_stride, scale, idx64, dtype, causal};
+                 pool_pad, top_n, max_ns, pooled_stride, scale, idx64, dtype, causal, lse_attn};
   int rc = 0;
   if (attn) rc = nsa::launch_cmp_attn(a, stream);
   if (rc == 0 && select) rc = nsa::launch_select(a, stream);
@@ -117,17 +117,17 @@ int nsa_cmp_attn_select_fwd(const void* q, const void* ck, const void* cvt, void
                             int64_t ck_head_stride, int cvt_cols, int block, int stride, int pool_kernel,
                             int pool_stride, int pool_pad, int top_n, int max_ns, int pooled_stride,
                             float scale, int causal, int idx64, int dtype, nsa_stream_t stream) {
-  return cmp_common("cmp_attn_select", indices ? 3 : 1, q, ck, cvt, o, indices, pooled, lse, cu_seqlens, cu_cmp,
+  return cmp_common("cmp_attn_select", indices ? 3 : 1, q, ck, cvt, o, indices, pooled, lse, nullptr, cu_seqlens, cu_cmp,
                     batch, total, hq, hkv, dk, dv, ck_row_stride, ck_head_stride, cvt_cols, block, stride,
                     pool_kernel, pool_stride, pool_pad, top_n, max_ns, pooled_stride, scale, causal, idx64, dtype,
                     stream);
 }
 
-int nsa_cmp_attn_fwd(const void* q, const void* ck, const void* cvt, void* o, float* lse,
+int nsa_cmp_attn_fwd(const void* q, const void* ck, const void* cvt, void* o, float* lse, float* lse_attn,
                      const int32_t* cu_seqlens, const int32_t* cu_cmp, int batch, int total, int hq, int hkv,
                      int dk, int dv, int64_t ck_row_stride, int64_t ck_head_stride, int cvt_cols, int block,
                      int stride, float scale, int causal, int dtype, nsa_stream_t stream) {
-  return cmp_common("cmp_attn", 1, q, ck, cvt, o, nullptr, nullptr, lse, cu_seqlens, cu_cmp, batch, total, hq, hkv,
+  return cmp_common("cmp_attn", 1, q, ck, cvt, o, nullptr, nullptr, lse, lse_attn, cu_seqlens, cu_cmp, batch, total, hq, hkv,
                     dk, dv, ck_row_stride, ck_head_stride, cvt_cols, block, stride, 1, 1, 0, 1, 0, 0, scale, causal,
                     0, dtype, stream);
 }
@@ -137,7 +137,7 @@ int nsa_block_select_fwd(const void* q, const void* ck, const float* lse, void* 
                          int dk, int64_t ck_row_stride, int64_t ck_head_stride, int pool_kernel, int pool_stride,
                          int pool_pad, int top_n, int max_ns, int pooled_stride, int idx64, int dtype,
                          nsa_stream_t stream) {
-  return cmp_common("block_select", 2, q, ck, nullptr, nullptr, indices, pooled, const_cast<float*>(lse), cu_seqlens,
+  return cmp_common("block_select", 2, q, ck, nullptr, nullptr, indices, pooled, const_cast<float*>(lse), nullptr, cu_seqlens,
                     cu_cmp, batch, total, hq, hkv, dk, 16, ck_row_stride, ck_head_stride, 0, 1, 1, pool_kernel,
                     pool_stride, pool_pad, top_n, max_ns, pooled_stride, 1.0f, 1, idx64, dtype, stream);
 }
@@ -151,7 +151,7 @@ int nsa_gate_fwd(const void* q, const void* weight, const void* bias, void* gate
   return finish(nsa::launch_gate(q, weight, bias, gates, (long)rows, dim, dtype, stream), "gate");
 }
 
-int nsa_swa_fwd(const void* q, const void* k, const void* vt, void* o, const int32_t* cu_seqlens, int batch,
+int nsa_swa_fwd(const void* q, const void* k, const void* vt, void* o, float* lse, const int32_t* cu_seqlens, int batch,
                 int total, int hq, int hkv, int dk, int dv, int vt_cols, int window, float scale, int dtype,
                 nsa_stream_t stream) {
   if (!q || !k || !vt || !o || !cu_seqlens) return fail(NSA_ERR_INVALID, "swa: null pointer");
@@ -161,7 +161,7 @@ int nsa_swa_fwd(const void* q, const void* k, const void* vt, void* o, const int
   if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "swa: scale must be positive");
   if (vt_cols % 64 != 0 || vt_cols < nsa_transposed_cols(total, batch)) return fail(NSA_ERR_INVALID, "swa: vt_cols too small or not a multiple of 64");
   if (!aligned16(q) || !aligned16(k) || !aligned16(vt) || !aligned16(o)) return fail(NSA_ERR_INVALID, "swa: pointers must be 16-byte aligned");
-  nsa::SwaArgs a{q, k, vt, o, cu_seqlens, batch, total, hq, hkv, dk, dv, vt_cols, window, scale, dtype};
+  nsa::SwaArgs a{q, k, vt, o, cu_seqlens, batch, total, hq, hkv, dk, dv, vt_cols, window, scale, dtype, lse};
   return finish(nsa::launch_swa(a, stream), "swa");
 }
 
@@ -175,8 +175,8 @@ int64_t nsa_slc_workspace_bytes(int total, int batch, int hkv, int dk, int dv, i
 
 int nsa_slc_combine_fwd(const void* q, const void* k, const void* vt, const void* indices, const int32_t* counts,
                         const void* g_slc, const void* g_swa, const void* g_cmp, int64_t gate_stride,
-                        const void* o_swa, const void* o_cmp, void* out, const int32_t* cu_seqlens, int batch,
-                        int total, int hq, int hkv, int dk, int dv, int vt_cols, int top_n, int block_size,
+                        const void* o_swa, const void* o_cmp, void* out, float* lse_slc, const int32_t* cu_seqlens,
+                        int batch, int total, int hq, int hkv, int dk, int dv, int vt_cols, int top_n, int block_size,
                         float scale, int idx64, int gate_act, int dtype, void* workspace, int64_t workspace_bytes,
                         nsa_stream_t stream) {
   if (!q || !k || !vt || !indices || !out || !cu_seqlens) return fail(NSA_ERR_INVALID, "slc_combine: null pointer");
@@ -191,9 +191,11 @@ int nsa_slc_combine_fwd(const void* q, const void* k, const void* vt, const void
   if (!aligned16(q) || !aligned16(k) || !aligned16(vt)) return fail(NSA_ERR_INVALID, "slc_combine: pointers must be 16-byte aligned");
   nsa::SlcArgs a{q, k, vt, indices, counts, g_slc, g_swa, g_cmp, (long)gate_stride, o_swa, o_cmp, out, cu_seqlens,
                  batch, total, hq, hkv, dk, dv, vt_cols, top_n, block_size, scale, idx64, gate_act, dtype,
-                 workspace, (long)workspace_bytes};
+                 workspace, (long)workspace_bytes, lse_slc};
   if (workspace && !aligned16(workspace)) return fail(NSA_ERR_INVALID, "slc_combine: workspace must be 16-byte aligned");
-  return finish(nsa::launch_slc_combine(a, stream), "slc_combine");
+  const int rc = nsa::launch_slc_combine(a, stream);
+  if (rc == -5) return fail(NSA_ERR_UNSUPPORTED, "slc_combine: lse_slc needs the block-major schedule (bf16, 64-key blocks, a workspace)");
+  return finish(rc, "slc_combine");
 }
 
 static int slc_common_checks(const char* what, const void* q, const void* k, const void* vt, const int32_t* cu_seqlens,
@@ -221,7 +223,7 @@ int nsa_slc_partials_fwd(const void* q, const void* k, const void* vt, const voi
                                  block_size, scale, dtype, workspace, workspace_bytes)) return rc;
   nsa::SlcArgs a{q, k, vt, indices, counts, nullptr, nullptr, nullptr, 1, nullptr, nullptr, nullptr, cu_seqlens,
                  batch, total, hq, hkv, dk, dv, vt_cols, top_n, block_size, scale, idx64, 0, dtype,
-                 workspace, (long)workspace_bytes};
+                 workspace, (long)workspace_bytes, nullptr};
   return finish(nsa::launch_slc_partials(a, workspace, stream), "slc_partials");
 }
 
@@ -239,10 +241,81 @@ int nsa_swa_merge_fwd(const void* q, const void* k, const void* vt, const void* 
   // the picks themselves are not needed here: the workspace's slot map says which have a partial
   nsa::SlcArgs sa{q, k, vt, nullptr, nullptr, g_slc, g_swa, g_cmp, (long)gate_stride, nullptr, o_cmp, out, cu_seqlens,
                   batch, total, hq, hkv, dk, dv, vt_cols, top_n, block_size, scale, 0, gate_act, dtype,
-                  const_cast<void*>(workspace), (long)workspace_bytes};
+                  const_cast<void*>(workspace), (long)workspace_bytes, nullptr};
   const nsa::MergeArgs m = nsa::slc_merge_args(sa, const_cast<void*>(workspace));
-  nsa::SwaArgs a{q, k, vt, nullptr, cu_seqlens, batch, total, hq, hkv, dk, dv, vt_cols, window, scale, dtype};
+  nsa::SwaArgs a{q, k, vt, nullptr, cu_seqlens, batch, total, hq, hkv, dk, dv, vt_cols, window, scale, dtype, nullptr};
   return finish(nsa::launch_swa_merge(a, m, stream), "swa_merge");
+}
+
+int64_t nsa_cmp_attn_bwd_workspace_bytes(int total, int cmp_rows, int hq, int hkv, int dk, int dv) {
+  if (total <= 0 || cmp_rows < 0 || hq <= 0 || hkv <= 0 || dk <= 0 || dv <= 0) return 0;
+  nsa::CmpBwdArgs a{};
+  a.total = total; a.cmp_rows = cmp_rows; a.hq = hq; a.hkv = hkv; a.dk = dk; a.dv = dv;
+  return nsa::cmp_bwd_workspace_bytes(a);
+}
+
+int nsa_cmp_attn_bwd(const void* q, const void* ck, const void* cv, const void* o, const void* d_o, const float* lse,
+                     const int32_t* cu_seqlens, const int32_t* cu_cmp, int batch, int total, int cmp_rows, int hq,
+                     int hkv, int dk, int dv, int block, int stride, float scale, int causal, int dtype, void* dq,
+                     void* dck, void* dcv, void* workspace, int64_t workspace_bytes, nsa_stream_t stream) {
+  if (!q || !o || !d_o || !lse || !cu_seqlens || !cu_cmp || !dq || !workspace)
+    return fail(NSA_ERR_INVALID, "cmp_attn_bwd: null pointer");
+  if (cmp_rows > 0 && (!ck || !cv || !dck || !dcv)) return fail(NSA_ERR_INVALID, "cmp_attn_bwd: null pointer");
+  if (batch <= 0 || total <= 0 || cmp_rows < 0 || block <= 0 || stride <= 0)
+    return fail(NSA_ERR_INVALID, "cmp_attn_bwd: sizes must be positive");
+  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "cmp_attn_bwd: bad dtype");
+  if (int rc = check_heads("cmp_attn_bwd", hq, hkv, dk, dv)) return rc;
+  if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "cmp_attn_bwd: scale must be positive");
+  if (!aligned16(q) || !aligned16(ck) || !aligned16(cv) || !aligned16(o) || !aligned16(d_o) || !aligned16(dq) ||
+      !aligned16(dck) || !aligned16(dcv) || !aligned16(workspace))
+    return fail(NSA_ERR_INVALID, "cmp_attn_bwd: pointers must be 16-byte aligned");
+  if (workspace_bytes < nsa_cmp_attn_bwd_workspace_bytes(total, cmp_rows, hq, hkv, dk, dv))
+    return fail(NSA_ERR_INVALID, "cmp_attn_bwd: workspace smaller than nsa_cmp_attn_bwd_workspace_bytes");
+  nsa::CmpBwdArgs a{q, ck, cv, o, d_o, lse, cu_seqlens, cu_cmp, batch, total, cmp_rows, hq, hkv, dk, dv, block, stride,
+                    causal, scale, dtype, dq, dck, dcv, workspace};
+  const int rc = nsa::launch_cmp_bwd(a, stream);
+  if (rc == -2) return fail(NSA_ERR_UNSUPPORTED, "cmp_attn_bwd: head dims not built (dk,dv in (64,64),(128,128),(192,128); fp32: no 192)");
+  return finish(rc, "cmp_attn_bwd");
+}
+
+int64_t nsa_slc_swa_bwd_workspace_bytes(int total, int batch, int hq, int hkv, int dk, int dv, int top_n,
+                                        int block_size, int dtype) {
+  if (total <= 0 || batch <= 0 || hq <= 0 || hkv <= 0 || dk <= 0 || dv <= 0 || top_n < 0) return 0;
+  nsa::SlcSwaBwdArgs a{};
+  a.total = total; a.batch = batch; a.hq = hq; a.hkv = hkv; a.dk = dk; a.dv = dv; a.top_n = top_n;
+  a.block_size = block_size; a.dtype = dtype;
+  return nsa::slc_swa_bwd_workspace_bytes(a);
+}
+
+int nsa_slc_swa_bwd(const void* q, const void* k, const void* v, const void* o_slc, const void* o_swa,
+                    const void* d_o_slc, const void* d_o_swa, const float* lse_slc, const float* lse_swa,
+                    const void* indices, const int32_t* counts, const int32_t* cu_seqlens, int batch, int total, int hq,
+                    int hkv, int dk, int dv, int top_n, int block_size, int window, float scale, int idx64, int dtype,
+                    void* dq, void* dk_out, void* dv_out, void* workspace, int64_t workspace_bytes,
+                    nsa_stream_t stream) {
+  if (!q || !k || !v || !cu_seqlens || !dq || !dk_out || !dv_out || !workspace)
+    return fail(NSA_ERR_INVALID, "slc_swa_bwd: null pointer");
+  const bool slc = d_o_slc != nullptr, swa = d_o_swa != nullptr;
+  if (slc && (!o_slc || !lse_slc || !indices || top_n <= 0)) return fail(NSA_ERR_INVALID, "slc_swa_bwd: the selected branch needs o_slc, lse_slc, indices and top_n > 0");
+  if (swa && (!o_swa || !lse_swa || window <= 0)) return fail(NSA_ERR_INVALID, "slc_swa_bwd: the sliding branch needs o_swa, lse_swa and window > 0");
+  if (batch <= 0 || total <= 0) return fail(NSA_ERR_INVALID, "slc_swa_bwd: sizes must be positive");
+  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "slc_swa_bwd: bad dtype");
+  if (int rc = check_heads("slc_swa_bwd", hq, hkv, dk, dv)) return rc;
+  if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "slc_swa_bwd: scale must be positive");
+  if (slc && (block_size != 64 || top_n > 64 || total >= (1 << 26)))
+    return fail(NSA_ERR_UNSUPPORTED, "slc_swa_bwd: the selected branch is built for 64-key blocks, top_n <= 64");
+  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(dq) || !aligned16(dk_out) || !aligned16(dv_out) ||
+      !aligned16(workspace) || (slc && (!aligned16(o_slc) || !aligned16(d_o_slc))) ||
+      (swa && (!aligned16(o_swa) || !aligned16(d_o_swa))))
+    return fail(NSA_ERR_INVALID, "slc_swa_bwd: pointers must be 16-byte aligned");
+  if (workspace_bytes < nsa_slc_swa_bwd_workspace_bytes(total, batch, hq, hkv, dk, dv, slc ? top_n : 0, block_size, dtype))
+    return fail(NSA_ERR_INVALID, "slc_swa_bwd: workspace smaller than nsa_slc_swa_bwd_workspace_bytes");
+  nsa::SlcSwaBwdArgs a{q, k, v, o_slc, o_swa, d_o_slc, d_o_swa, lse_slc, lse_swa, indices, counts, cu_seqlens, batch,
+                       total, hq, hkv, dk, dv, slc ? top_n : 0, block_size, swa ? window : 0, scale, idx64, dtype, dq,
+                       dk_out, dv_out, workspace};
+  const int rc = nsa::launch_slc_swa_bwd(a, stream);
+  if (rc == -2) return fail(NSA_ERR_UNSUPPORTED, "slc_swa_bwd: head dims not built (dk,dv in (64,64),(128,128),(192,128); fp32: no 192)");
+  return finish(rc, "slc_swa_bwd");
 }
 
 int nsa_decode_max_compressed(void) { return nsa::decode_max_nc(); }

@@ -23,11 +23,13 @@ struct CmpArgs {
   long ck_row_stride, ck_head_stride; int cvt_cols;
   int block, stride, pool_k, pool_s, pool_p, top_n, max_ns, pooled_stride;
   float scale; int idx64, dtype, causal;
+  float* lse_attn;   // optional: natural-log log-sum-exp of the scaled visible scores (+inf: no key visible)
 };
 
 struct SwaArgs {
   const void* q; const void* k; const void* vt; void* o; const int32_t* cu_seq;
   int batch, total, hq, hkv, dk, dv, vt_cols, window; float scale; int dtype;
+  float* lse;        // optional, as CmpArgs::lse_attn
 };
 
 struct SlcArgs {
@@ -37,6 +39,7 @@ struct SlcArgs {
   int batch, total, hq, hkv, dk, dv, vt_cols, top_n, block_size; float scale;
   int idx64, gate_act, dtype;
   void* workspace; long workspace_bytes;
+  float* lse;        // optional (block-major schedule only), as CmpArgs::lse_attn
 };
 
 // Where the merge of the block-major partial results finds its inputs (all device pointers; the
@@ -46,6 +49,27 @@ struct MergeArgs {
   const void* g_slc; const void* g_swa; const void* g_cmp; long gate_stride;
   const void* o_cmp; void* out;
   int top_n, hq, hkv, gate_act; float scale;
+  float* lse;        // optional: log-sum-exp of the selected branch per (token, q head)
+};
+
+// Backward of the compressed branch: all tensors packed and contiguous; lse is the natural-log
+// log-sum-exp of the scaled visible scores of every row (+inf for rows that see nothing).
+struct CmpBwdArgs {
+  const void* q; const void* ck; const void* cv; const void* o; const void* d_o; const float* lse;
+  const int32_t* cu_seq; const int32_t* cu_cmp;
+  int batch, total, cmp_rows, hq, hkv, dk, dv, block, stride, causal; float scale; int dtype;
+  void* dq; void* dck; void* dcv; void* workspace;
+};
+
+// Backward of the selected and sliding branches (either may be absent: top_n == 0 / d_o_slc null,
+// window == 0 / d_o_swa null).  dq, dk_out, dv_out receive the sums over the present branches.
+struct SlcSwaBwdArgs {
+  const void* q; const void* k; const void* v;
+  const void* o_slc; const void* o_swa; const void* d_o_slc; const void* d_o_swa;
+  const float* lse_slc; const float* lse_swa;
+  const void* indices; const int32_t* counts; const int32_t* cu_seq;
+  int batch, total, hq, hkv, dk, dv, top_n, block_size, window; float scale; int idx64, dtype;
+  void* dq; void* dk_out; void* dv_out; void* workspace;
 };
 
 struct DecodeArgs {
@@ -70,6 +94,10 @@ int launch_slc_block_major(const SlcArgs& a, void* workspace, hipStream_t st);
 int launch_slc_partials(const SlcArgs& a, void* workspace, hipStream_t st);
 MergeArgs slc_merge_args(const SlcArgs& a, void* workspace);
 int launch_swa_merge(const SwaArgs& a, const MergeArgs& m, hipStream_t st);
+long cmp_bwd_workspace_bytes(const CmpBwdArgs& a);
+int launch_cmp_bwd(const CmpBwdArgs& a, hipStream_t st);
+long slc_swa_bwd_workspace_bytes(const SlcSwaBwdArgs& a);
+int launch_slc_swa_bwd(const SlcSwaBwdArgs& a, hipStream_t st);
 int launch_decode(const DecodeArgs& a, hipStream_t st);
 int launch_decode_append(const void* k_new, const void* v_new, void* k_cache, void* v_cache_t, void* ck_cache,
                          void* cv_cache_t, const int32_t* pos, int batch, int hkv, int dk, int dv, int ctx_cap,

@@ -13,31 +13,19 @@
 // offsets / cursors per (head, block), work items (head, block, segment of 64 pairs), the bucketed
 // pair list, a slot map (token, head, pick) -> pair, and the partial results.
 #include "slc_merge.h"
+#include "slc_ws.h"
 
 namespace nsa {
 
 int set_smem(const void* fn, size_t bytes);
 
-constexpr int kSeg = 64;          // pairs of one block handled by one wavefront
-constexpr int kBlk = 64;          // keys per selection block (4 MFMA tiles)
-
-struct SlcWs {
-  int* blkbase; int* counts; int* offsets; int* cursor; int* items; int* n_items;
-  uint32_t* list; int* slotmap; float* ml; void* po;
-  int nb;          // bound on the number of 64-key blocks over all sequences
-  long pairs_cap;  // total * hkv * top_n
-  int items_cap;
-};
-
-__host__ __device__ inline long align_up(long x, long a) { return (x + a - 1) / a * a; }
-
-__host__ inline long carve(const SlcArgs& a, void* base, SlcWs* ws, size_t elem) {
+long slc_carve(const SlcArgs& a, void* base, SlcWs* ws, size_t elem, int part_width) {
   const int nb = a.total / kBlk + a.batch;
   const long nkeys = (long)a.hkv * nb;
   const long pairs = (long)a.total * a.hkv * a.top_n;
   const int items_cap = (int)(pairs / kSeg + nkeys) + 1;
   long off = 0;
-  auto take = [&](long bytes) { const long o = off; off = align_up(off + bytes, 256); return o; };
+  auto take = [&](long bytes) { const long o = off; off = slc_align_up(off + bytes, 256); return o; };
   const long o_blkbase = take((a.batch + 1) * 4L);
   const long o_counts = take(nkeys * 4);
   const long o_offsets = take(nkeys * 4);
@@ -47,7 +35,7 @@ __host__ inline long carve(const SlcArgs& a, void* base, SlcWs* ws, size_t elem)
   const long o_list = take(pairs * 4);
   const long o_slot = take(pairs * 4);
   const long o_ml = take(pairs * 2 * 16 * 4);
-  const long o_po = take(pairs * 16 * a.dv * (long)elem);
+  const long o_po = take(pairs * 16 * part_width * (long)elem);
   if (ws != nullptr) {
     char* b = reinterpret_cast<char*>(base);
     ws->blkbase = (int*)(b + o_blkbase); ws->counts = (int*)(b + o_counts); ws->offsets = (int*)(b + o_offsets);
@@ -58,6 +46,8 @@ __host__ inline long carve(const SlcArgs& a, void* base, SlcWs* ws, size_t elem)
   }
   return off;
 }
+
+static long carve(const SlcArgs& a, void* base, SlcWs* ws, size_t elem) { return slc_carve(a, base, ws, elem, a.dv); }
 
 long slc_workspace_bytes(const SlcArgs& a) { return carve(a, nullptr, nullptr, a.dtype == 0 ? 2 : 4); }
 
@@ -358,16 +348,16 @@ slc_merge_kernel(const SlcArgs a, const MergeArgs m) {
   if (osw) o_swa = load8(osw + row * DV + pc * 8);
   const vec8_t<T> r = merge_piece<T, DV, TOPN>(m, tg, hq_i / G, hq_i % G, row, pc, osw != nullptr, o_swa);
   store8(reinterpret_cast<T*>(a.out) + row * DV + pc * 8, r);
+  if (m.lse != nullptr && pc == 0) m.lse[row] = merge_lse(m, tg, hq_i / G, hq_i % G);
 }
 
 static MergeArgs merge_args_of(const SlcArgs& a, const SlcWs& ws) {
   return MergeArgs{ws.slotmap, ws.ml, ws.po, a.g_slc, a.g_swa, a.g_cmp, a.gate_stride, a.o_cmp, a.out,
-                   a.top_n, a.hq, a.hkv, a.gate_act, a.scale};
+                   a.top_n, a.hq, a.hkv, a.gate_act, a.scale, a.lse};
 }
 
-// bucket the pairs, then one partial result per pair
-template <typename T, int DK, int DV>
-static int launch_partials_t(const SlcArgs& a, const SlcWs& ws, hipStream_t st) {
+// bucket the (token, pick) pairs by (kv head, block): counts, offsets, pair list, slot map, work items
+int launch_slc_bucket(const SlcArgs& a, const SlcWs& ws, hipStream_t st) {
   const long pairs = ws.pairs_cap;
   hipLaunchKernelGGL(slc_prep_kernel, dim3(1), dim3(256), 0, st, a.cu_seq, a.batch, ws, a.hkv);
   if (ws.nb <= kBucketMaxBins) {
@@ -387,6 +377,14 @@ static int launch_partials_t(const SlcArgs& a, const SlcWs& ws, hipStream_t st) 
     hipLaunchKernelGGL(slc_scan_kernel, dim3(1), dim3(1024), 0, st, ws, a.hkv);
     hipLaunchKernelGGL(slc_bucket_kernel<true>, dim3(gb), dim3(256), 0, st, a, ws);
   }
+  return 0;
+}
+
+// bucket the pairs, then one partial result per pair
+template <typename T, int DK, int DV>
+static int launch_partials_t(const SlcArgs& a, const SlcWs& ws, hipStream_t st) {
+  const int rc = launch_slc_bucket(a, ws, st);
+  if (rc) return rc;
   hipLaunchKernelGGL((slc_block_kernel<T, DK, DV>), dim3((ws.items_cap + 3) / 4), dim3(256), 0, st, a, ws);
   return 0;
 }

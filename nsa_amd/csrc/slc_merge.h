@@ -94,4 +94,22 @@ __device__ __forceinline__ vec8_t<T> merge_piece(const MergeArgs& m, long tg, in
   return pack8<T>(out);
 }
 
+// Log-sum-exp (natural log) of the scaled scores over all usable picks of (token tg, kv head h,
+// head n of the group); +inf when the token has no usable pick.
+__device__ __forceinline__ float merge_lse(const MergeArgs& m, long tg, int h, int n) {
+  const long base = (tg * m.hkv + h) * m.top_n;
+  const float c_attn = m.scale * kLog2e;
+  float M = kNegInf, den = 0.f;
+  for (int i = 0; i < m.top_n; ++i) {
+    const long p = m.slotmap[base + i];
+    if (p < 0) continue;
+    const float mi = m.ml[(p * 2) * 16 + n];
+    const float l = m.ml[(p * 2 + 1) * 16 + n];
+    const float m_new = fmaxf(M, mi);
+    den = den * fast_exp2((M - m_new) * c_attn) + l * fast_exp2((mi - m_new) * c_attn);
+    M = m_new;
+  }
+  return den > 0.f ? fmaf(M, m.scale, __logf(den)) : __builtin_huge_valf();
+}
+
 }  // namespace nsa

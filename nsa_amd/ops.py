@@ -141,19 +141,22 @@ def cmp_attn_select(q, ck, cvt, cu_seqlens, cu_cmp, batch, hkv, dv, ck_row_strid
 
 
 def cmp_attn(q, ck, cvt, cu_seqlens, cu_cmp, batch, hkv, dv, ck_row_stride, ck_head_stride, block, stride, scale,
-             causal=True):
-    """Compressed attention only.  Returns (o [total,Hq,dv], lse float32 [total,Hq])."""
+             causal=True, want_lse_attn=False):
+    """Compressed attention only.  Returns (o [total,Hq,dv], lse float32 [total,Hq]) where lse is the
+    log-sum-exp of the raw scores over all compressed rows (what block_select reads); with
+    want_lse_attn a third tensor: the log-sum-exp of the scaled visible scores (what the backward reads)."""
     _need_cuda(q, ck, cvt, cu_seqlens, cu_cmp)
     q = _dense(q)
     total, hq, dk = q.shape
     o = torch.empty(total, hq, dv, dtype=q.dtype, device=q.device)
     lse = torch.empty(total, hq, dtype=torch.float32, device=q.device)
-    rc = _lib.load().nsa_cmp_attn_fwd(_ptr(q), _ptr(ck), _ptr(cvt), _ptr(o), _ptr(lse), _ptr(cu_seqlens),
-                                      _ptr(cu_cmp), batch, total, hq, hkv, dk, dv, ck_row_stride, ck_head_stride,
-                                      cvt.shape[-1], block, stride, float(scale), int(bool(causal)),
+    lse_attn = torch.empty(total, hq, dtype=torch.float32, device=q.device) if want_lse_attn else None
+    rc = _lib.load().nsa_cmp_attn_fwd(_ptr(q), _ptr(ck), _ptr(cvt), _ptr(o), _ptr(lse), _ptr(lse_attn),
+                                      _ptr(cu_seqlens), _ptr(cu_cmp), batch, total, hq, hkv, dk, dv, ck_row_stride,
+                                      ck_head_stride, cvt.shape[-1], block, stride, float(scale), int(bool(causal)),
                                       _dtype_code(q), _stream())
     _lib.check(rc, "nsa_cmp_attn_fwd")
-    return o, lse
+    return (o, lse, lse_attn) if want_lse_attn else (o, lse)
 
 
 def block_select(q, ck, lse, cu_seqlens, cu_cmp, batch, hkv, ck_row_stride, ck_head_stride, pool_kernel,
@@ -174,17 +177,19 @@ def block_select(q, ck, lse, cu_seqlens, cu_cmp, batch, hkv, ck_row_stride, ck_h
     return idx, (pooled if want_pooled else None)
 
 
-def swa(q, k, vt, cu_seqlens, batch, window, scale):
+def swa(q, k, vt, cu_seqlens, batch, window, scale, want_lse=False):
+    """Sliding-window attention; with want_lse returns (o, lse float32 [total,Hq])."""
     _need_cuda(q, k, vt, cu_seqlens)
     q, k = _dense(q), _dense(k)
     total, hq, dk = q.shape
     hkv, dv = vt.shape[0], vt.shape[1]
     o = torch.empty(total, hq, dv, dtype=q.dtype, device=q.device)
+    lse = torch.empty(total, hq, dtype=torch.float32, device=q.device) if want_lse else None
     lib = _lib.load()
-    rc = lib.nsa_swa_fwd(_ptr(q), _ptr(k), _ptr(vt), _ptr(o), _ptr(cu_seqlens), batch, total, hq, hkv, dk, dv,
-                         vt.shape[-1], window, float(scale), _dtype_code(q), _stream())
+    rc = lib.nsa_swa_fwd(_ptr(q), _ptr(k), _ptr(vt), _ptr(o), _ptr(lse), _ptr(cu_seqlens), batch, total, hq, hkv,
+                         dk, dv, vt.shape[-1], window, float(scale), _dtype_code(q), _stream())
     _lib.check(rc, "nsa_swa_fwd")
-    return o
+    return (o, lse) if want_lse else o
 
 
 def _gate_views(gates, q):
@@ -205,9 +210,10 @@ SLC_WORKSPACE_LIMIT = 48 << 30      # bytes; larger problems keep the token-majo
 
 
 def slc_combine(q, k, vt, indices, counts, g_slc, g_swa, g_cmp, o_swa, o_cmp, cu_seqlens, batch, block_size,
-                scale, gate_act=0, block_major=None):
+                scale, gate_act=0, block_major=None, want_lse=False):
     """block_major: None = use the block-major schedule when the shape has one and its workspace
-    fits SLC_WORKSPACE_LIMIT; False = token-major kernel; True = require block-major."""
+    fits SLC_WORKSPACE_LIMIT; False = token-major kernel; True = require block-major.
+    want_lse (block-major only): returns (out, lse float32 [total,Hq] of the selected branch)."""
     _need_cuda(q, k, vt, indices, cu_seqlens)
     q, k = _dense(q), _dense(k)
     total, hq, dk = q.shape
@@ -222,6 +228,7 @@ def slc_combine(q, k, vt, indices, counts, g_slc, g_swa, g_cmp, o_swa, o_cmp, cu
     o_swa = None if o_swa is None else _dense(o_swa)
     o_cmp = None if o_cmp is None else _dense(o_cmp)
     out = torch.empty(total, hq, dv, dtype=q.dtype, device=q.device)
+    lse = torch.empty(total, hq, dtype=torch.float32, device=q.device) if want_lse else None
     lib = _lib.load()
     ws, ws_bytes = None, 0
     if block_major is not False:
@@ -233,11 +240,11 @@ def slc_combine(q, k, vt, indices, counts, g_slc, g_swa, g_cmp, o_swa, o_cmp, cu
             raise NotImplementedError("no block-major selected attention for this shape / dtype")
     rc = lib.nsa_slc_combine_fwd(
         _ptr(q), _ptr(k), _ptr(vt), _ptr(indices), _ptr(counts), _ptr(g_slc), _ptr(g_swa), _ptr(g_cmp), gs,
-        _ptr(o_swa), _ptr(o_cmp), _ptr(out), _ptr(cu_seqlens), batch, total, hq, hkv, dk, dv, vt.shape[-1],
-        top_n, block_size, float(scale), int(indices.dtype == torch.int64), gate_act, _dtype_code(q), _ptr(ws),
-        ws_bytes, _stream())
+        _ptr(o_swa), _ptr(o_cmp), _ptr(out), _ptr(lse), _ptr(cu_seqlens), batch, total, hq, hkv, dk, dv,
+        vt.shape[-1], top_n, block_size, float(scale), int(indices.dtype == torch.int64), gate_act, _dtype_code(q),
+        _ptr(ws), ws_bytes, _stream())
     _lib.check(rc, "nsa_slc_combine_fwd")
-    return out
+    return (out, lse) if want_lse else out
 
 
 def slc_workspace(q, hkv, dv, top_n, block_size, batch):
@@ -300,3 +307,58 @@ def gate_logits(q, weight, bias=None):
                                   _stream())
     _lib.check(rc, "nsa_gate_fwd")
     return out
+
+
+def cmp_attn_bwd(q, ck, cv, o, d_o, lse_attn, cu_seqlens, cu_cmp, batch, block, stride, scale, causal=True):
+    """Backward of the compressed attention.  q [total,Hq,Dk], ck [rows,Hkv,Dk], cv [rows,Hkv,Dv]
+    (packed over cu_cmp), o / d_o [total,Hq,Dv], lse_attn from cmp_attn(want_lse_attn=True).
+    Returns (dq, dck, dcv)."""
+    _need_cuda(q, ck, cv, o, d_o, lse_attn, cu_seqlens, cu_cmp)
+    q, ck, cv, o, d_o = (_dense(t) for t in (q, ck, cv, o, d_o))
+    total, hq, dk = q.shape
+    rows, hkv, dv = cv.shape
+    dq, dck, dcv = torch.empty_like(q), torch.empty_like(ck), torch.empty_like(cv)
+    lib = _lib.load()
+    need = lib.nsa_cmp_attn_bwd_workspace_bytes(total, rows, hq, hkv, dk, dv)
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
+    rc = lib.nsa_cmp_attn_bwd(_ptr(q), _ptr(ck), _ptr(cv), _ptr(o), _ptr(d_o), _ptr(lse_attn), _ptr(cu_seqlens),
+                              _ptr(cu_cmp), batch, total, rows, hq, hkv, dk, dv, block, stride, float(scale),
+                              int(bool(causal)), _dtype_code(q), _ptr(dq), _ptr(dck), _ptr(dcv), _ptr(ws),
+                              ws.numel(), _stream())
+    _lib.check(rc, "nsa_cmp_attn_bwd")
+    return dq, dck, dcv
+
+
+def slc_swa_bwd(q, k, v, o_slc, d_o_slc, lse_slc, o_swa, d_o_swa, lse_swa, indices, counts, cu_seqlens, batch,
+                block_size, window, scale):
+    """Backward of the selected (o_slc / d_o_slc / lse_slc, or None) and sliding (o_swa / d_o_swa /
+    lse_swa, or None) branches.  v is the row-major [total,Hkv,Dv] tensor.  Returns (dq, dk, dv), each
+    the sum over the branches given."""
+    _need_cuda(q, k, v, cu_seqlens)
+    q, k, v = _dense(q), _dense(k), _dense(v)
+    total, hq, dk = q.shape
+    hkv, dv = v.shape[1], v.shape[2]
+    slc, swa_ = d_o_slc is not None, d_o_swa is not None
+    top_n = 0
+    if slc:
+        if indices.dtype not in (torch.int32, torch.int64):
+            raise TypeError("block indices must be int32 or int64")
+        indices = indices.contiguous()
+        top_n = indices.shape[-1]
+        counts = None if counts is None else counts.to(torch.int32).contiguous()
+        o_slc, d_o_slc = _dense(o_slc), _dense(d_o_slc)
+    if swa_:
+        o_swa, d_o_swa = _dense(o_swa), _dense(d_o_swa)
+    dq, dk_out, dv_out = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    lib = _lib.load()
+    need = lib.nsa_slc_swa_bwd_workspace_bytes(total, batch, hq, hkv, dk, dv, top_n, block_size, _dtype_code(q))
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
+    rc = lib.nsa_slc_swa_bwd(
+        _ptr(q), _ptr(k), _ptr(v), _ptr(o_slc if slc else None), _ptr(o_swa if swa_ else None),
+        _ptr(d_o_slc if slc else None), _ptr(d_o_swa if swa_ else None), _ptr(lse_slc if slc else None),
+        _ptr(lse_swa if swa_ else None), _ptr(indices if slc else None), _ptr(counts if slc else None),
+        _ptr(cu_seqlens), batch, total, hq, hkv, dk, dv, top_n, block_size, window if swa_ else 0, float(scale),
+        int(slc and indices.dtype == torch.int64), _dtype_code(q), _ptr(dq), _ptr(dk_out), _ptr(dv_out), _ptr(ws),
+        ws.numel(), _stream())
+    _lib.check(rc, "nsa_slc_swa_bwd")
+    return dq, dk_out, dv_out

@@ -64,17 +64,17 @@ def test_host_helpers(lib):
 
 def test_argument_errors_do_not_launch(lib):
     # null pointers / bad sizes are rejected before any HIP call, so this runs without a GPU
-    rc = lib.nsa_swa_fwd(None, None, None, None, None, 1, 64, 4, 1, 64, 64, 128, 16, 0.1, 0, None)
+    rc = lib.nsa_swa_fwd(None, None, None, None, None, None, 1, 64, 4, 1, 64, 64, 128, 16, 0.1, 0, None)
     assert rc == -1 and b"null" in lib.nsa_last_error_string()
     buf = ctypes.create_string_buffer(4096)
     p = ctypes.c_void_p((ctypes.addressof(buf) + 15) & ~15)
-    rc = lib.nsa_swa_fwd(p, p, p, p, p, 1, 64, 64, 2, 64, 64, 128, 16, 0.1, 0, None)
+    rc = lib.nsa_swa_fwd(p, p, p, p, None, p, 1, 64, 64, 2, 64, 64, 128, 16, 0.1, 0, None)
     assert rc == -2 and b"group size" in lib.nsa_last_error_string()
-    rc = lib.nsa_swa_fwd(p, p, p, p, p, 1, 64, 4, 1, 48, 64, 128, 16, 0.1, 0, None)
+    rc = lib.nsa_swa_fwd(p, p, p, p, None, p, 1, 64, 4, 1, 48, 64, 128, 16, 0.1, 0, None)
     assert rc == -2
-    rc = lib.nsa_swa_fwd(p, p, p, p, p, 1, 64, 4, 1, 64, 64, 128, 16, 0.1, 7, None)
+    rc = lib.nsa_swa_fwd(p, p, p, p, None, p, 1, 64, 4, 1, 64, 64, 128, 16, 0.1, 7, None)
     assert rc == -1
-    rc = lib.nsa_slc_combine_fwd(p, p, p, p, None, None, None, None, 1, None, None, p, p, 1, 64, 4, 1, 64, 64, 128,
+    rc = lib.nsa_slc_combine_fwd(p, p, p, p, None, None, None, None, 1, None, None, p, None, p, 1, 64, 4, 1, 64, 64, 128,
                                  4, 60, 0.1, 1, 0, 0, None, 0, None)
     assert rc == -2 and b"block_size" in lib.nsa_last_error_string()
     rc = lib.nsa_compress_fwd(p, None, None, p, p, p, 1, 10, 2, 60, 32, 16, 0, None)
