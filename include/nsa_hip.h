@@ -62,6 +62,19 @@ int nsa_transpose_fwd(const void* x, void* out, const int32_t* cu, int batch, in
                       int64_t row_stride, int64_t head_stride, int out_cols, int dtype,
                       nsa_stream_t stream);
 
+/* Backward of nsa_compress_fwd.  Replaces nsa/compression_kv.py:220-266 (_compress_kv.backward with
+ * the kernels _compress_bwd_dx / _compress_bwd_dw, :62-171); for the Conv1d compressor (:292-312,
+ * differentiated by autograd in the reference) it also yields the bias gradient.
+ *   d_out [out rows, heads, dim] gradient of the compressed rows; dx [total, heads, dim] is fully
+ *   overwritten.  w_lin NULL = mean pooling.  Otherwise w_lin is the weight as [block*dim][dim]
+ *   (row j*dim + i = tap j, input channel i; column = output channel: the layout of the reference's
+ *   k_weight / v_weight, i.e. the TRANSPOSE of what nsa_compress_fwd takes), x [total, heads, dim] the
+ *   forward input, dw float [block*dim][dim] and dbias float [dim] (either may be NULL) are
+ *   overwritten with the weight / bias gradients in fp32. */
+int nsa_compress_bwd(const void* x, const void* w_lin, const void* d_out, void* dx, float* dw, float* dbias,
+                     const int32_t* cu_seqlens, const int32_t* cu_out, int batch, int total, int out_rows_bound,
+                     int heads, int dim, int block, int stride, int dtype, nsa_stream_t stream);
+
 /* Compressed attention fused with block-importance scoring and top-n selection.  Replaces
  * nsa/triton_attention.py:419-476 (_attention.forward: _attn_fwd, softmax_kernel, sum / avg_pool1d /
  * topk) with the semantics of nsa/torch_attention.py:66-163 (attention_ref, get_indices).

@@ -1,0 +1,104 @@
+"""torch.autograd glue over the backward entry points of the C ABI.  Every Function works on packed
+tensors ([total, heads, dim]); the forward calls the same kernels as the inference path (asking them
+for the log-sum-exp per row), the backward calls nsa_compress_bwd / nsa_cmp_attn_bwd /
+nsa_slc_swa_bwd.  No arithmetic happens here.
+
+Counterparts in the reference: _compress_kv (nsa/compression_kv.py:178-266), _attention
+(nsa/triton_attention.py:419-546), ParallelNSAFunction (nsa/selection_attn.py:679-737)."""
+from __future__ import annotations
+
+import torch
+
+from . import ops
+
+
+def needs_grad(*tensors) -> bool:
+    return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
+
+
+class CompressFn(torch.autograd.Function):
+    """x [total,H,D] -> [rows,H,D].  w_lin None = mean pooling, else [block*D, D] (row j*D+i, column o)
+    with an optional bias [D]."""
+
+    @staticmethod
+    def forward(ctx, x, w_lin, bias, cu, cu_out, rows, block, stride):
+        wt = None if w_lin is None else w_lin.detach().t().contiguous()
+        out = ops.compress(x, cu, cu_out, rows, block, stride, wt, None if bias is None else bias.detach())
+        ctx.save_for_backward(x, w_lin, bias, cu, cu_out)
+        ctx.geom = (block, stride)
+        return out
+
+    @staticmethod
+    def backward(ctx, d_out):
+        x, w_lin, bias, cu, cu_out = ctx.saved_tensors
+        block, stride = ctx.geom
+        if w_lin is None:
+            dx = ops.compress_bwd(d_out, cu, cu_out, x.shape[0], block, stride)
+            return dx, None, None, None, None, None, None, None
+        dx, dw, db = ops.compress_bwd(d_out, cu, cu_out, x.shape[0], block, stride, x=x, w_lin=w_lin.detach(),
+                                      want_dw=ctx.needs_input_grad[1],
+                                      want_dbias=bias is not None and ctx.needs_input_grad[2])
+        dw = None if dw is None else dw.to(w_lin.dtype)
+        db = None if db is None else db.to(bias.dtype)
+        return dx, dw, db, None, None, None, None, None
+
+
+class CmpAttnFn(torch.autograd.Function):
+    """Compressed attention (+ block selection, which has no gradient).  q [total,Hq,Dk], ck
+    [rows,Hkv,Dk], cv [rows,Hkv,Dv] packed over cu_cmp.  select = None or (pool_kernel, pool_stride,
+    pool_pad, top_n, max_nc, idx64).  Returns (o, indices or None)."""
+
+    @staticmethod
+    def forward(ctx, q, ck, cv, cu, cu_cmp, batch, block, stride, scale, causal, select):
+        q, ck, cv = q.contiguous(), ck.contiguous(), cv.contiguous()
+        hkv, dk, dv = ck.shape[1], ck.shape[2], cv.shape[2]
+        cvt = ops.transpose(cv, cu_cmp, batch)
+        o, lse_raw, lse = ops.cmp_attn(q, ck, cvt, cu, cu_cmp, batch, hkv, dv, hkv * dk, dk, block, stride, scale,
+                                       causal=causal, want_lse_attn=True)
+        idx = None
+        if select is not None:
+            pk, ps, pp, top_n, max_nc, idx64 = select
+            idx, _ = ops.block_select(q, ck, lse_raw, cu, cu_cmp, batch, hkv, hkv * dk, dk, pk, ps, pp, top_n, max_nc,
+                                      idx64=idx64)
+            ctx.mark_non_differentiable(idx)
+        ctx.save_for_backward(q, ck, cv, o, lse, cu, cu_cmp)
+        ctx.geom = (batch, block, stride, scale, causal)
+        return o, idx
+
+    @staticmethod
+    def backward(ctx, d_o, _d_idx=None):
+        q, ck, cv, o, lse, cu, cu_cmp = ctx.saved_tensors
+        batch, block, stride, scale, causal = ctx.geom
+        dq, dck, dcv = ops.cmp_attn_bwd(q, ck, cv, o, d_o, lse, cu, cu_cmp, batch, block, stride, scale, causal=causal)
+        return dq, dck, dcv, None, None, None, None, None, None, None, None
+
+
+class SlcSwaFn(torch.autograd.Function):
+    """Selected-block attention (idx not None) and sliding-window attention (window > 0), ungated.
+    q [total,Hq,Dk], k [total,Hkv,Dk], v [total,Hkv,Dv].  Returns (o_slc or None, o_swa or None)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, idx, counts, cu, batch, block_size, window, scale):
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        vt = ops.transpose(v, cu, batch)
+        o_slc = lse_slc = o_swa = lse_swa = None
+        if idx is not None:
+            o_slc, lse_slc = ops.slc_combine(q, k, vt, idx, counts, None, None, None, None, None, cu, batch,
+                                             block_size, scale, block_major=True, want_lse=True)
+        if window > 0:
+            o_swa, lse_swa = ops.swa(q, k, vt, cu, batch, window, scale, want_lse=True)
+        ctx.save_for_backward(q, k, v, o_slc, lse_slc, o_swa, lse_swa, idx, counts, cu)
+        ctx.geom = (batch, block_size, window, scale)
+        return o_slc, o_swa
+
+    @staticmethod
+    def backward(ctx, d_slc, d_swa):
+        q, k, v, o_slc, lse_slc, o_swa, lse_swa, idx, counts, cu = ctx.saved_tensors
+        batch, block_size, window, scale = ctx.geom
+        if o_slc is None:
+            d_slc = None
+        if o_swa is None:
+            d_swa = None
+        dq, dk, dv = ops.slc_swa_bwd(q, k, v, o_slc, d_slc, lse_slc, o_swa, d_swa, lse_swa, idx, counts, cu, batch,
+                                     block_size, window, scale)
+        return dq, dk, dv, None, None, None, None, None, None, None

@@ -1,7 +1,9 @@
 """Compressed attention + block selection with the interface of the reference's
 nsa/triton_attention.py::flash_attn_func (:419-476, :549).  Semantics are those of the reference's
 torch path (nsa/torch_attention.py:66-163): the importance softmax is over all compressed rows of
-the raw, unscaled scores.  Forward only."""
+the raw, unscaled scores.  When q, k or v requires grad the call goes through an autograd function
+whose backward (nsa/triton_attention.py:478-546 in the reference) is nsa_cmp_attn_bwd; the block
+indices carry no gradient."""
 from __future__ import annotations
 
 import math
@@ -9,9 +11,9 @@ import math
 import torch
 
 from . import ops
+from .autograd import CmpAttnFn, needs_grad
 
 
-@torch.no_grad()
 def flash_attn_func(q, k, v, block_stride, block_size, causal, sm_scale, pool_num_kv_head=0,
                     pool_kernel_size=0, pool_stride=0, pool_padding=0, select_block_count=0):
     """q [B,T,Hq,D]; k, v = compressed keys/values [B,Nc,H,D] with H = Hq (each kv head repeated
@@ -28,6 +30,23 @@ def flash_attn_func(q, k, v, block_stride, block_size, causal, sm_scale, pool_nu
     select = select_block_count > 0 and pool_kernel_size > 0
     cu = ops.uniform_cu(B, T, q.device)
     cu_cmp = ops.uniform_cu(B, Nc, q.device)
+    if needs_grad(q, k, v):
+        # one row set per kv head; the gradient of a head-repeated k / v lands on the head that is read
+        ckp = k[:, :, ::rep].reshape(B * Nc, hkv, D)
+        cvp = v[:, :, ::rep].reshape(B * Nc, hkv, Dv)
+        sel = (pool_kernel_size, pool_stride, pool_padding, select_block_count, Nc, True) if select else None
+        o, idx = CmpAttnFn.apply(q.reshape(B * T, Hq, D), ckp, cvp, cu, cu_cmp, B, block_size, block_stride,
+                                 float(sm_scale), bool(causal), sel)
+        return o.view(B, T, Hq, Dv), (None if idx is None else idx.view(B, T, hkv, select_block_count))
+    with torch.no_grad():
+        return _flash_attn_nograd(q, k, v, cu, cu_cmp, hkv, rep, block_stride, block_size, causal, sm_scale,
+                                  pool_kernel_size, pool_stride, pool_padding, select_block_count, select)
+
+
+def _flash_attn_nograd(q, k, v, cu, cu_cmp, hkv, rep, block_stride, block_size, causal, sm_scale, pool_kernel_size,
+                       pool_stride, pool_padding, select_block_count, select):
+    B, T, Hq, D = q.shape
+    _, Nc, H, Dv = v.shape
     if (k.stride(-1) != 1 or k.stride(0) != Nc * k.stride(1) or k.data_ptr() % 16 or k.stride(1) % 8
             or k.stride(2) % 8):
         k = k.contiguous()

@@ -2,7 +2,8 @@
 
 calc_compressed_len (compression_kv.py:9-10), compress_kv (:178-217, :269), KVCompressorVarlen
 (:272-289) and KVCompressor (:292-312) keep their names, argument order, parameter names/shapes and
-return arity.  The arithmetic runs in the HIP kernels of libnsa_hip.so; forward only.
+return arity.  The arithmetic runs in the HIP kernels of libnsa_hip.so, forward and backward (the
+backward of :220-266 through nsa_compress_bwd when an input or a parameter requires grad).
 """
 from __future__ import annotations
 
@@ -14,6 +15,7 @@ import torch.nn as nn
 from torch.nn import init
 
 from . import ops
+from .autograd import CompressFn, needs_grad
 
 
 def calc_compressed_len(x, stride, size):
@@ -26,13 +28,23 @@ def conv_compressed_len(x, stride, size):
     return 0 if x < size else (x - size) // stride + 1
 
 
-@torch.no_grad()
 def compress_kv(k, v, w_k, w_v, cu_seq_len, block_stride, block_size):
     """k, v [total, H, D]; w_* [block_size*D, D] (row j*D+i); cu_seq_len int32 [B+1].
     Returns (ck, cv, cu_out_len): bf16 [sum Nc', H, D] with Nc' = (T - block_size)//block_stride."""
     cu = cu_seq_len.to(torch.int32)
     cu_out = ops.compressed_offsets(cu, block_size, block_stride, extra=0)
     out_rows = int(cu_out[-1].item())      # the reference syncs here as well (cu_seq_len.tolist())
+    if needs_grad(k, v, w_k, w_v):
+        kk = k if k.dtype in (torch.bfloat16, torch.float32) else k.to(torch.bfloat16)
+        vv = v if v.dtype in (torch.bfloat16, torch.float32) else v.to(torch.bfloat16)
+        ck = CompressFn.apply(kk, w_k.to(kk.dtype), None, cu, cu_out, out_rows, block_size, block_stride)
+        cv = CompressFn.apply(vv, w_v.to(vv.dtype), None, cu, cu_out, out_rows, block_size, block_stride)
+        return ck.to(torch.bfloat16), cv.to(torch.bfloat16), cu_out
+    with torch.no_grad():
+        return _compress_kv_nograd(k, v, w_k, w_v, cu, cu_out, out_rows, block_stride, block_size)
+
+
+def _compress_kv_nograd(k, v, w_k, w_v, cu, cu_out, out_rows, block_stride, block_size):
     wk_t = w_k.detach().t().contiguous()
     wv_t = w_v.detach().t().contiguous()
     kk = k if k.dtype in (torch.bfloat16, torch.float32) else k.to(torch.bfloat16)
@@ -80,9 +92,21 @@ class KVCompressor(nn.Module):
         w = conv.weight.detach()
         return w.permute(0, 2, 1).reshape(w.shape[0], -1).contiguous()
 
-    @torch.no_grad()
+    @staticmethod
+    def _w_lin(conv: nn.Conv1d) -> torch.Tensor:
+        # [o, i, j] -> [j*D + i, o], differentiable
+        w = conv.weight
+        return w.permute(2, 1, 0).reshape(-1, w.shape[0])
+
     def compress_packed(self, k, v, cu_seq_len, seq_len: Optional[int] = None):
         """Un-repeated result: (ck, cv [sum Nc, H, D], cu_cmp int32 [B+1], max Nc or None)."""
+        params = () if self.mode == "mean" else tuple(self.parameters())
+        if needs_grad(k, v, *params):
+            return self._compress_packed(k, v, cu_seq_len, seq_len, True)
+        with torch.no_grad():
+            return self._compress_packed(k, v, cu_seq_len, seq_len, False)
+
+    def _compress_packed(self, k, v, cu_seq_len, seq_len, train):
         cu = cu_seq_len.to(torch.int32)
         batch = cu.numel() - 1
         nc = conv_compressed_len(seq_len, self.block_stride, self.block_size) if seq_len is not None else None
@@ -93,7 +117,15 @@ class KVCompressor(nn.Module):
             cu_out = ops.compressed_offsets(cu, self.block_size, self.block_stride, extra=1)
             rows = k.shape[0] // self.block_stride + batch
             nc = None
-        if self.mode == "mean":
+        if train:
+            if self.mode == "mean":
+                wk = wv = bk = bv = None
+            else:
+                wk, wv = self._w_lin(self.compressor_k).to(k.dtype), self._w_lin(self.compressor_v).to(v.dtype)
+                bk, bv = self.compressor_k.bias, self.compressor_v.bias
+            ck = CompressFn.apply(k, wk, bk, cu, cu_out, rows, self.block_size, self.block_stride)
+            cv = CompressFn.apply(v, wv, bv, cu, cu_out, rows, self.block_size, self.block_stride)
+        elif self.mode == "mean":
             ck = ops.compress(k, cu, cu_out, rows, self.block_size, self.block_stride)
             cv = ops.compress(v, cu, cu_out, rows, self.block_size, self.block_stride)
         else:

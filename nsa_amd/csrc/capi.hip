@@ -65,6 +65,25 @@ int nsa_compress_fwd(const void* x, const void* wt, const void* bias, void* out,
   return finish(rc, "compress");
 }
 
+int nsa_compress_bwd(const void* x, const void* w_lin, const void* d_out, void* dx, float* dw, float* dbias,
+                     const int32_t* cu_seqlens, const int32_t* cu_out, int batch, int total, int out_rows_bound,
+                     int heads, int dim, int block, int stride, int dtype, nsa_stream_t stream) {
+  if (!d_out || !dx || !cu_seqlens || !cu_out) return fail(NSA_ERR_INVALID, "compress_bwd: null pointer");
+  if ((dw || dbias) && !w_lin) return fail(NSA_ERR_INVALID, "compress_bwd: weight gradients need the weight");
+  if (dw && !x) return fail(NSA_ERR_INVALID, "compress_bwd: the weight gradient needs x");
+  if (batch <= 0 || total <= 0 || heads <= 0 || block <= 0 || stride <= 0 || out_rows_bound < 0)
+    return fail(NSA_ERR_INVALID, "compress_bwd: sizes must be positive");
+  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "compress_bwd: bad dtype");
+  if (dim % 8 != 0) return fail(NSA_ERR_UNSUPPORTED, "compress_bwd: dim must be a multiple of 8");
+  if (!aligned16(d_out) || !aligned16(dx) || (x && !aligned16(x)) || (w_lin && !aligned16(w_lin)))
+    return fail(NSA_ERR_INVALID, "compress_bwd: pointers must be 16-byte aligned");
+  nsa::CompressBwdArgs a{x, w_lin, d_out, dx, dw, dbias, cu_seqlens, cu_out, batch, total, out_rows_bound, heads, dim,
+                         block, stride, dtype};
+  const int rc = nsa::launch_compress_bwd(a, stream);
+  if (rc == -2) return fail(NSA_ERR_UNSUPPORTED, "compress_bwd: weighted path is built for dim 32/64/128/192");
+  return finish(rc, "compress_bwd");
+}
+
 int nsa_transpose_fwd(const void* x, void* out, const int32_t* cu, int batch, int heads, int dim,
                       int64_t row_stride, int64_t head_stride, int out_cols, int dtype, nsa_stream_t stream) {
   if (!x || !out || !cu) return fail(NSA_ERR_INVALID, "transpose: null pointer");

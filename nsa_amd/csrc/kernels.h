@@ -11,6 +11,14 @@ struct CompressArgs {
   int batch, out_rows_bound, heads, dim, block, stride, dtype;
 };
 
+// Backward of the compression.  w_lin == nullptr: mean pooling (only dx).  w_lin is the weight in the
+// functional layout [block*dim][dim] (row j*dim + i, column o); dw (same layout) and dbias are fp32.
+struct CompressBwdArgs {
+  const void* x; const void* w_lin; const void* d_out; void* dx; float* dw; float* dbias;
+  const int32_t* cu_seq; const int32_t* cu_out;
+  int batch, total, out_rows_bound, heads, dim, block, stride, dtype;
+};
+
 struct TransposeArgs {
   const void* x; void* out; const int32_t* cu;
   int batch, heads, dim; long row_stride, head_stride; int out_cols, dtype;
@@ -81,6 +89,7 @@ struct DecodeArgs {
 };
 
 int launch_compress(const CompressArgs& a, hipStream_t st);
+int launch_compress_bwd(const CompressBwdArgs& a, hipStream_t st);
 int launch_transpose(const TransposeArgs& a, hipStream_t st);
 int launch_gate(const void* x, const void* w, const void* bias, void* out, long rows, int dim, int dtype,
                 hipStream_t st);

@@ -8,12 +8,16 @@ import torch
 from torch import nn
 
 from . import _lib, ops
+from .autograd import CmpAttnFn, SlcSwaFn, needs_grad
 from .compression_kv import KVCompressor, conv_compressed_len
 
 
 class NSAAttention(nn.Module):
-    """Native Sparse Attention forward: compress -> compressed attention + block selection ->
-    selected + sliding-window attention -> gated sum, all on hand-written gfx950 kernels.
+    """Native Sparse Attention: compress -> compressed attention + block selection ->
+    selected + sliding-window attention -> gated sum, all on hand-written gfx950 kernels.  Without
+    grad the fused inference schedule runs; when an input or a parameter requires grad the branches run
+    un-fused through autograd functions whose backward is hand-written as well (the gating Linear and
+    the gated sum then go through torch ops, as in the reference).
 
     Parameters follow the reference (`compressor.compressor_k/v.{weight,bias}`,
     `gating.{weight,bias}`), so its state_dict loads.  Two build-owned switches:
@@ -60,7 +64,6 @@ class NSAAttention(nn.Module):
         self.gating = nn.Linear(head_dim, 3, device=device, dtype=dtype)
         self.gate_activation = gate_activation
 
-    @torch.no_grad()
     def forward(
         self,
         q: torch.Tensor,
@@ -91,6 +94,39 @@ class NSAAttention(nn.Module):
             scale = 1.0 / math.sqrt(dk)
         uniform = not max_seqlen
         seq_len = total // batch if uniform else int(max_seqlen)
+        params = [self.gating.weight, self.gating.bias]
+        if self.compressor.mode != "mean":
+            params += list(self.compressor.parameters())
+        if needs_grad(q, k, v, gates, *params):
+            return self._forward_train(q, k, v, cu, batch, scale, bool(causal), seq_len, uniform, gates,
+                                       return_indices)
+        with torch.no_grad():
+            return self._forward_infer(q, k, v, cu, batch, scale, causal, seq_len, uniform, gates, stage_times,
+                                       return_indices)
+
+    def _forward_train(self, q, k, v, cu, batch, scale, causal, seq_len, uniform, gates, return_indices):
+        ck, cv, cu_cmp, nc = self.compressor.compress_packed(k, v, cu, seq_len=seq_len if uniform else None)
+        max_nc = nc if nc is not None else conv_compressed_len(seq_len, self.compression_stride,
+                                                               self.compression_block)
+        sel = (self.pool_kernel_size, self.pool_stride, self.pool_padding, self.selected_block_count, max_nc, False)
+        o_cmp, idx = CmpAttnFn.apply(q, ck, cv, cu, cu_cmp, batch, self.compression_block,
+                                     self.compression_stride, float(scale), causal, sel)
+        o_slc, o_swa = SlcSwaFn.apply(q, k, v, idx, None, cu, batch, self.selection_block_size,
+                                      self.sliding_window, float(scale))
+        if gates is None:
+            gates = torch.nn.functional.linear(q, self.gating.weight.to(q.dtype), self.gating.bias.to(q.dtype))
+        g = torch.sigmoid(gates) if self.gate_activation == "sigmoid" else gates
+        out = g[..., 0:1] * o_slc + g[..., 2:3] * o_cmp
+        if o_swa is not None:
+            out = out + g[..., 1:2] * o_swa
+        if return_indices:
+            return out, idx
+        return out
+
+    def _forward_infer(self, q, k, v, cu, batch, scale, causal, seq_len, uniform, gates, stage_times,
+                       return_indices):
+        total, hq, dk = q.shape
+        hkv, dv = v.shape[1], v.shape[2]
 
         def stage(name, fn):
             if stage_times is None:

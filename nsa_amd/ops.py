@@ -362,3 +362,36 @@ def slc_swa_bwd(q, k, v, o_slc, d_o_slc, lse_slc, o_swa, d_o_swa, lse_swa, indic
         ws.numel(), _stream())
     _lib.check(rc, "nsa_slc_swa_bwd")
     return dq, dk_out, dv_out
+
+
+def compress_bwd(d_out, cu_seqlens, cu_out, total, block, stride, x=None, w_lin=None, want_dw=True,
+                 want_dbias=False):
+    """Backward of compress().  d_out [rows, H, D].  Mean pooling: w_lin None -> returns dx.  Weighted:
+    w_lin [block*D, D] (row j*D+i, column o), x the forward input -> (dx, dw float32 or None,
+    dbias float32 or None)."""
+    _need_cuda(d_out, cu_seqlens, cu_out)
+    d_out = _dense(d_out)
+    rows, H, D = d_out.shape
+    dx = torch.empty(total, H, D, dtype=d_out.dtype, device=d_out.device)
+    dw = dbias = None
+    if w_lin is not None:
+        w_lin = _dense(w_lin.to(d_out.dtype))
+        if tuple(w_lin.shape) != (block * D, D):
+            raise ValueError("weight must be [block*dim, dim], got %s" % (tuple(w_lin.shape),))
+        if want_dw:
+            x = _dense(x)
+            dw = torch.empty(block * D, D, dtype=torch.float32, device=d_out.device)
+        if want_dbias:
+            dbias = torch.empty(D, dtype=torch.float32, device=d_out.device)
+    if rows == 0:
+        dx.zero_()
+        for t in (dw, dbias):
+            if t is not None:
+                t.zero_()
+    else:
+        rc = _lib.load().nsa_compress_bwd(_ptr(x if dw is not None else None), _ptr(w_lin), _ptr(d_out), _ptr(dx),
+                                          _ptr(dw), _ptr(dbias), _ptr(cu_seqlens), _ptr(cu_out),
+                                          cu_seqlens.numel() - 1, total, rows, H, D, block, stride,
+                                          _dtype_code(d_out), _stream())
+        _lib.check(rc, "nsa_compress_bwd")
+    return dx if w_lin is None else (dx, dw, dbias)

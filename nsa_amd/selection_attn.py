@@ -1,5 +1,7 @@
 """Selected-block + sliding-window attention with the interface of the reference's
-nsa/selection_attn.py::parallel_nsa (:740-814).  Forward only."""
+nsa/selection_attn.py::parallel_nsa (:740-814).  When q, k, v or a gate requires grad the two
+branches run un-fused through an autograd function (backward: nsa_slc_swa_bwd, the counterpart of
+nsa/selection_attn.py:715-737) and the gates are applied with torch ops as in :808-811."""
 from __future__ import annotations
 
 from typing import Optional, Union
@@ -7,13 +9,13 @@ from typing import Optional, Union
 import torch
 
 from . import ops
+from .autograd import SlcSwaFn, needs_grad
 
 
 def _packed(x, B, T):
     return x.reshape(B * T, *x.shape[2:])
 
 
-@torch.no_grad()
 def sliding_window_attn(q, k, v, window_size: int, scale: Optional[float] = None,
                         cu_seqlens: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Token t attends the last `window_size` tokens up to and including itself.
@@ -27,12 +29,16 @@ def sliding_window_attn(q, k, v, window_size: int, scale: Optional[float] = None
     else:
         cu = ops.uniform_cu(B, T, q.device)
     nb = cu.numel() - 1
-    vt = ops.transpose(_packed(v, B, T), cu, nb)
-    o = ops.swa(_packed(q, B, T), _packed(k, B, T), vt, cu, nb, window_size, scale)
+    if needs_grad(q, k, v):
+        _, o = SlcSwaFn.apply(_packed(q, B, T), _packed(k, B, T), _packed(v, B, T), None, None, cu, nb, 64,
+                              window_size, float(scale))
+        return o.view(B, T, HQ, v.shape[-1])
+    with torch.no_grad():
+        vt = ops.transpose(_packed(v, B, T), cu, nb)
+        o = ops.swa(_packed(q, B, T), _packed(k, B, T), vt, cu, nb, window_size, scale)
     return o.view(B, T, HQ, v.shape[-1])
 
 
-@torch.no_grad()
 def parallel_nsa(q: torch.Tensor,
                  k: torch.Tensor,
                  v: torch.Tensor,
@@ -70,21 +76,35 @@ def parallel_nsa(q: torch.Tensor,
     cu = cu_seqlens.to(torch.int32) if cu_seqlens is not None else ops.uniform_cu(B, T, q.device)
     nb = cu.numel() - 1
     qp, kp, vp = _packed(q, B, T), _packed(k, B, T), _packed(v, B, T)
-    vt = ops.transpose(vp, cu, nb)
     counts = None if block_counts is None else block_counts.reshape(B * T, H)
     idx = block_indices.reshape(B * T, H, -1)
+    if needs_grad(q, k, v, g_slc, g_swa):
+        o_slc, o_swa = SlcSwaFn.apply(qp, kp, vp, idx, counts, cu, nb, block_size, window_size, float(scale))
+        o = o_slc * g_slc.reshape(B * T, HQ, 1)
+        if o_swa is not None:
+            o = o + o_swa * g_swa.reshape(B * T, HQ, 1)
+    else:
+        with torch.no_grad():
+            o = _parallel_nsa_nograd(qp, kp, vp, idx, counts, g_slc, g_swa, cu, nb, block_size, window_size, scale)
+    o = o.view(B, T, HQ, V)
+    if head_first:
+        o = o.transpose(1, 2)
+    return o
+
+
+def _parallel_nsa_nograd(qp, kp, vp, idx, counts, g_slc, g_swa, cu, nb, block_size, window_size, scale):
+    total, HQ = qp.shape[0], qp.shape[1]
+    H, V = kp.shape[1], vp.shape[-1]
+    vt = ops.transpose(vp, cu, nb)
     ws = ops.slc_workspace(qp, H, V, idx.shape[-1], block_size, nb) if window_size > 0 else None
     if ws is not None:
         # fused schedule: per-block partial results, merged in the window kernel's epilogue
         ops.slc_partials(qp, kp, vt, idx, counts, cu, nb, block_size, scale, ws)
-        o = ops.swa_merge(qp, kp, vt, ws, idx.shape[-1], g_slc.reshape(B * T, HQ), g_swa.reshape(B * T, HQ), None,
+        o = ops.swa_merge(qp, kp, vt, ws, idx.shape[-1], g_slc.reshape(total, HQ), g_swa.reshape(total, HQ), None,
                           None, cu, nb, block_size, window_size, scale)
     else:
         o_swa = ops.swa(qp, kp, vt, cu, nb, window_size, scale) if window_size > 0 else None
-        o = ops.slc_combine(qp, kp, vt, idx, counts, g_slc.reshape(B * T, HQ),
-                            g_swa.reshape(B * T, HQ) if o_swa is not None else None, None, o_swa, None, cu, nb,
+        o = ops.slc_combine(qp, kp, vt, idx, counts, g_slc.reshape(total, HQ),
+                            g_swa.reshape(total, HQ) if o_swa is not None else None, None, o_swa, None, cu, nb,
                             block_size, scale)
-    o = o.view(B, T, HQ, V)
-    if head_first:
-        o = o.transpose(1, 2)
     return o

@@ -32,11 +32,11 @@ def _oracle_grads(fn, inputs, d_o):
     return [x.grad if x.grad is not None else torch.zeros_like(x) for x in ins]
 
 
-def _check(name, got, ref, dtype):
+def _check(name, got, ref, dtype, floor=1.0):
     a, b = got.double().cpu(), ref.double()
     assert torch.isfinite(a).all(), name + ": non-finite gradient"
     err = float((a - b).abs().max()) if a.numel() else 0.0
-    mag = max(1.0, float(b.abs().max()) if b.numel() else 0.0)
+    mag = max(floor, float(b.abs().max()) if b.numel() else 0.0)
     print("   %-4s max_abs %.3e  (max|ref| %.3f)" % (name, err, mag))
     assert err <= GTOL[dtype] * mag, "%s: %.3e > %.1e * %.3f" % (name, err, GTOL[dtype], mag)
 
@@ -174,3 +174,213 @@ def test_slc_swa_bwd(lens, Hq, Hkv, Dk, Dv, S, W):
             _check("dq", dq[s:e], rq, dtype)
             _check("dk", dk[s:e], rk, dtype)
             _check("dv", dv[s:e], rv, dtype)
+
+
+# ------------------------------------------------------------------------------ compression
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("lens,H,D,l,d", [([300], 1, 64, 32, 16), ([300, 31, 64, 1000], 4, 128, 32, 16),
+                                          ([200, 77], 2, 192, 64, 16), ([90], 2, 32, 8, 4)])
+def test_compress_mean_bwd(dtype, lens, H, D, l, d):
+    ops = _ops()
+    T = sum(lens)
+    ncs = [O.compressed_len_conv(t, l, d) for t in lens]
+    d_out = randn(sum(ncs), H, D, seed=180, dtype=dtype)
+    cu, cu_out = _cu(lens), _cu(ncs)
+    dx = ops.compress_bwd(d_out.to(DEV), cu, cu_out, T, l, d)
+    cuh, cuc = ragged_cu(lens), ragged_cu(ncs)
+    print("compress_mean_bwd", dtype, lens, (H, D, l, d))
+    for s, e, cs, ce, n in zip(cuh[:-1], cuh[1:], cuc[:-1], cuc[1:], ncs):
+        if n == 0:                                     # shorter than one block: no window, no gradient
+            assert torch.count_nonzero(dx[s:e]) == 0
+            continue
+        x = torch.zeros(e - s, H, D)
+        (rx,) = _oracle_grads(lambda a: O.compress_meanpool(a, l, d, n, math_dtype=torch.float64), [x], d_out[cs:ce])
+        _check("dx", dx[s:e], rx, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("lens,H,D,l,d,extra", [([256, 100], 2, 64, 32, 16, 1), ([1024] * 2, 2, 128, 64, 16, 0),
+                                                ([90, 7], 1, 32, 8, 4, 1), ([700], 4, 192, 32, 16, 1)])
+def test_compress_weighted_bwd(dtype, lens, H, D, l, d, extra):
+    ops = _ops()
+    T = sum(lens)
+    ncs = [O.compressed_len_conv(t, l, d) if extra else O.compressed_len_functional(t, l, d) for t in lens]
+    x = randn(T, H, D, seed=181, dtype=dtype)
+    w_lin = randn(l * D, D, seed=182, scale=1.0 / math.sqrt(l * D), dtype=dtype)
+    bias = randn(D, seed=183, dtype=dtype) if extra else None
+    d_out = randn(sum(ncs), H, D, seed=184, dtype=dtype)
+    cu, cu_out = _cu(lens), _cu(ncs)
+    dx, dw, db = ops.compress_bwd(d_out.to(DEV), cu, cu_out, T, l, d, x=x.to(DEV), w_lin=w_lin.to(DEV),
+                                  want_dbias=bool(extra))
+    cuh, cuc = ragged_cu(lens), ragged_cu(ncs)
+    print("compress_weighted_bwd", dtype, lens, (H, D, l, d, extra))
+    rw = torch.zeros(l * D, D, dtype=torch.float64)
+    rb = torch.zeros(D, dtype=torch.float64)
+    for s, e, cs, ce, n in zip(cuh[:-1], cuh[1:], cuc[:-1], cuc[1:], ncs):
+        ins = [x[s:e], w_lin] + ([bias] if extra else [])
+        fn = (lambda a, w, b: O.compress_weighted(a, w, b, l, d, n, math_dtype=torch.float64)) if extra else \
+            (lambda a, w: O.compress_weighted(a, w, None, l, d, n, math_dtype=torch.float64))
+        g = _oracle_grads(fn, ins, d_out[cs:ce])
+        _check("dx", dx[s:e], g[0], dtype)
+        rw += g[1]
+        if extra:
+            rb += g[2]
+    _check("dw", dw, rw, dtype)
+    if extra:
+        _check("db", db, rb, dtype)
+
+
+# ------------------------------------------------------------------------------ host API (autograd functions)
+def _leaf(t):
+    return t.to(DEV).requires_grad_(True)
+
+
+@pytest.mark.parametrize("mode,lens,Hq,Hkv,Dk,Dv", [("mean", [600], 16, 1, 64, 64), ("mean", [300, 200, 40], 32, 2, 128, 128),
+                                                    ("conv", [500], 16, 1, 64, 64), ("mean", [400], 16, 1, 192, 128)])
+def test_module_backward(mode, lens, Hq, Hkv, Dk, Dv):
+    """NSAAttention end to end: gradients of every input and parameter against autograd through the
+    oracle forward (float64, the module's own block picks forced so that score ties cannot differ)."""
+    from nsa_amd.nsa import NSAAttention
+    dtype = torch.bfloat16
+    T = sum(lens)
+    p = O.NSAParams(block=32, stride=16, sel_block=64, top_n=4, window=64, scale=1.0 / math.sqrt(Dk))
+    torch.manual_seed(5)
+    mod = NSAAttention(Dk, causal=True, compression_stride=16, compression_block=32, selection_block=64,
+                       selected_block_count=4, sliding_window=64, device=DEV, dtype=dtype, compressor_mode=mode,
+                       gate_activation="sigmoid")
+    if mode == "conv" and Dk != Dv:
+        pytest.skip("the Conv1d compressor has one head_dim")
+    q, k, v, _ = make_qkv(T, Hq, Hkv, Dk, Dv, 190, dtype, 0.7)
+    d_o = randn(T, Hq, Dv, seed=191, dtype=dtype)
+    qd, kd, vd = _leaf(q), _leaf(k), _leaf(v)
+    cu = _cu(lens)
+    out, idx = mod(qd, kd, vd, cu, max_seqlen=max(lens), return_indices=True)
+    out.backward(d_o.to(DEV))
+    assert out.requires_grad and idx.dtype == torch.int32
+
+    # oracle: same parameters, float64
+    gw = mod.gating.weight.detach().cpu().double().requires_grad_(True)
+    gb = mod.gating.bias.detach().cpu().double().requires_grad_(True)
+    comp = None
+    if mode == "conv":
+        def lin(conv):
+            w = conv.weight.detach().cpu().double()
+            return w.permute(2, 1, 0).reshape(-1, w.shape[0]).requires_grad_(True)
+        comp = {"wk": lin(mod.compressor.compressor_k), "wv": lin(mod.compressor.compressor_v),
+                "bk": mod.compressor.compressor_k.bias.detach().cpu().double().requires_grad_(True),
+                "bv": mod.compressor.compressor_v.bias.detach().cpu().double().requires_grad_(True)}
+    qr, kr, vr = (t.double().clone().requires_grad_(True) for t in (q, k, v))
+    cuh = ragged_cu(lens)
+    outs = []
+    for s, e in zip(cuh[:-1], cuh[1:]):
+        gates = torch.sigmoid(qr[s:e] @ gw.t() + gb)
+        outs.append(O.nsa_forward_single(qr[s:e], kr[s:e], vr[s:e], gates, p, comp, math_dtype=torch.float64,
+                                         force_idx=idx[s:e].cpu()))
+    ref = torch.cat(outs)
+    ref.backward(d_o.double())
+    print("module_bwd", mode, lens, (Hq, Hkv, Dk, Dv))
+    _check("out", out.detach(), ref.detach(), dtype)
+    _check("dq", qd.grad, qr.grad, dtype)
+    _check("dk", kd.grad, kr.grad, dtype)
+    _check("dv", vd.grad, vr.grad, dtype)
+    _check("dgw", mod.gating.weight.grad, gw.grad, dtype)
+    _check("dgb", mod.gating.bias.grad, gb.grad, dtype)
+    if mode == "conv":
+        for name, conv in (("k", mod.compressor.compressor_k), ("v", mod.compressor.compressor_v)):
+            w = comp["w" + name].grad                                  # [j*D+i, o] -> [o, i, j]
+            D = conv.weight.shape[0]
+            _check("dw" + name, conv.weight.grad, w.reshape(-1, D, D).permute(2, 1, 0), dtype)
+            # the bias gradient is a sum of bf16-rounded rows that nearly cancel (shifting every key by a
+            # constant does not change the attention): its error scales with the terms, as dw's does
+            _check("db" + name, conv.bias.grad, comp["b" + name].grad, dtype, floor=float(w.abs().max()))
+
+
+def test_module_no_grad_path_unchanged():
+    """Without grad the fused inference schedule runs and agrees with the training-path output."""
+    from nsa_amd.nsa import NSAAttention
+    dtype, T, Hq, Hkv, D = torch.bfloat16, 700, 32, 2, 128
+    mod = NSAAttention(D, causal=True, selected_block_count=4, sliding_window=128, device=DEV, dtype=dtype,
+                       compressor_mode="mean", gate_activation="sigmoid")
+    q, k, v, _ = make_qkv(T, Hq, Hkv, D, D, 195, dtype, 0.7)
+    cu = _cu([T])
+    with torch.no_grad():
+        a = mod(q.to(DEV), k.to(DEV), v.to(DEV), cu)
+    b = mod(_leaf(q), k.to(DEV), v.to(DEV), cu)
+    assert not a.requires_grad and b.requires_grad
+    assert float((a.float() - b.detach().float()).abs().max()) <= 2e-2
+
+
+def test_parallel_nsa_and_flash_attn_backward():
+    """The two functional entry points with the reference's tensor layouts ([B,T,H,D], head-repeated
+    compressed keys): gradients of q, k, v and the gates."""
+    import nsa_amd
+    dtype, B, T, Hq, Hkv, D, S, W, bs = torch.bfloat16, 2, 256, 32, 2, 64, 3, 32, 64
+    scale = 1.0 / math.sqrt(D)
+    q = randn(B, T, Hq, D, seed=200, scale=0.7, dtype=dtype)
+    k = randn(B, T, Hkv, D, seed=201, scale=0.7, dtype=dtype)
+    v = randn(B, T, Hkv, D, seed=202, scale=0.7, dtype=dtype)
+    g1 = torch.sigmoid(randn(B, T, Hq, seed=203)).to(dtype)
+    g2 = torch.sigmoid(randn(B, T, Hq, seed=204)).to(dtype)
+    d_o = randn(B, T, Hq, D, seed=205, dtype=dtype)
+    idx = torch.stack([_random_indices(T, Hkv, S, bs, 206 + b) for b in range(B)])
+    leaves = [_leaf(t) for t in (q, k, v, g1, g2)]
+    o = nsa_amd.parallel_nsa(*leaves, idx.to(DEV), block_size=bs, window_size=W, scale=scale)
+    o.backward(d_o.to(DEV))
+    refs = [t.double().clone().requires_grad_(True) for t in (q, k, v, g1, g2)]
+    outs = []
+    for b in range(B):
+        o_slc = O.selected_attention(refs[0][b], refs[1][b], refs[2][b], idx[b], None, bs, scale, math_dtype=torch.float64)
+        o_swa = O.sliding_attention(refs[0][b], refs[1][b], refs[2][b], W, scale, math_dtype=torch.float64)
+        outs.append(O.gated_combine(refs[3][b], o_slc, refs[4][b], o_swa))
+    ref = torch.stack(outs)
+    ref.backward(d_o.double())
+    print("parallel_nsa_bwd")
+    _check("out", o.detach(), ref.detach(), dtype)
+    for name, a, r in zip(("dq", "dk", "dv", "dg1", "dg2"), leaves, refs):
+        _check(name, a.grad, r.grad, dtype)
+
+    # compressed attention on head-repeated compressed keys, as KVCompressor(group=...) hands them over
+    Nc, l, d = O.compressed_len_conv(T, 32, 16), 32, 16
+    ck = randn(B, Nc, Hkv, D, seed=207, scale=0.7, dtype=dtype)
+    cv = randn(B, Nc, Hkv, D, seed=208, scale=0.7, dtype=dtype)
+    qd, ckd, cvd = _leaf(q), _leaf(ck), _leaf(cv)
+    G = Hq // Hkv
+    o2, idx2 = nsa_amd.flash_attn_func(qd, ckd.repeat_interleave(G, dim=2), cvd.repeat_interleave(G, dim=2), d, l, True,
+                                       scale, Hkv, 5, 4, 0, 2)
+    o2.backward(d_o.to(DEV))
+    assert idx2.shape == (B, T, Hkv, 2) and not idx2.requires_grad
+    rq, rck, rcv = (t.double().clone().requires_grad_(True) for t in (q, ck, cv))
+    ref2 = torch.stack([O.compressed_attention(rq[b], rck[b], rcv[b], l, d, scale, math_dtype=torch.float64)
+                        for b in range(B)])
+    ref2.backward(d_o.double())
+    print("flash_attn_func_bwd")
+    _check("out", o2.detach(), ref2.detach(), dtype)
+    _check("dq", qd.grad, rq.grad, dtype)
+    _check("dck", ckd.grad, rck.grad, dtype)
+    _check("dcv", cvd.grad, rcv.grad, dtype)
+
+
+def test_compress_kv_backward():
+    """compress_kv (functional, learned weights) and KVCompressorVarlen: gradients of k, v and the weights."""
+    from nsa_amd.compression_kv import KVCompressorVarlen
+    dtype, lens, H, D, l, d = torch.bfloat16, [200, 90], 2, 64, 32, 16
+    T = sum(lens)
+    mod = KVCompressorVarlen(d, l, D, DEV, dtype)
+    k, v = randn(T, H, D, seed=210, dtype=dtype), randn(T, H, D, seed=211, dtype=dtype)
+    kd, vd = _leaf(k), _leaf(v)
+    ck, cv, cu_out = mod(kd, vd, _cu(lens))
+    ncs = [O.compressed_len_functional(t, l, d) for t in lens]
+    assert cu_out.cpu().tolist() == ragged_cu(ncs)
+    d1, d2 = randn(sum(ncs), H, D, seed=212, dtype=dtype), randn(sum(ncs), H, D, seed=213, dtype=dtype)
+    (ck.float() * d1.to(DEV).float()).sum().backward(retain_graph=True)
+    (cv.float() * d2.to(DEV).float()).sum().backward()
+    cuh, cuc = ragged_cu(lens), ragged_cu(ncs)
+    for x, xd, w, dd, name in ((k, kd, mod.k_weight, d1, "k"), (v, vd, mod.v_weight, d2, "v")):
+        wr = w.detach().cpu().double().requires_grad_(True)
+        xr = x.double().clone().requires_grad_(True)
+        ref = torch.cat([O.compress_weighted(xr[s:e], wr, None, l, d, n, math_dtype=torch.float64)
+                         for s, e, n in zip(cuh[:-1], cuh[1:], ncs)])
+        ref.backward(dd.double())
+        print("compress_kv_bwd", name)
+        _check("dx", xd.grad, xr.grad, dtype)
+        _check("dw", w.grad, wr.grad, dtype)
