@@ -6,13 +6,15 @@ One "step" is one pass of the NSA forward path (compress -> compressed attention
 already resident in HBM.  Prints ONE JSON line.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload prefill_cfg4|prefill_cfg2|prefill_32k_d128]
-                  [--no-cpu-baseline]
+                  [--no-cpu-baseline] [--no-decode] [--no-backward]
 
 roofline: taken for the kernel stage with the largest share of the step; its algorithmic flops
 (causal compressed rows, whole valid selected blocks, exact window; nothing for exp / pooling /
 top-n or for the non-causal part of the importance scores) divided by its mean duration measured
 with events on the launch stream.  cpu_baseline: the CPU oracle (a port of the reference's naive
 torch path) on a bounded sample of query rows of the same workload, on this host's cores.
+train_step (extra, not the headline metric): forward + backward of the same workload through the
+module's autograd path.
 """
 import argparse
 import json
@@ -141,6 +143,43 @@ def decode_bench(steps, warmup):
             "workload": "decode_cfg5: batch 64 x 1 token, ctx 32768, Hq64/Hkv4, D128, top-16 x 64, window 512, bf16"}
 
 
+def train_bench(m, q, k, v, gl, cu, max_len, total, f_eff, steps, warmup):
+    """Forward + backward through the module's training path (un-fused forward that keeps the
+    per-branch outputs and log-sum-exps, hand-written backward kernels) on the same workload.
+    Model flops of the step: 3.5 x the forward's effective flops (two GEMMs forward, five backward)."""
+    import torch
+    qg, kg, vg, gg = (t.detach().clone().requires_grad_(True) for t in (q, k, v, gl))
+    d_o = torch.randn(total, q.shape[1], v.shape[2], device=q.device, generator=torch.Generator(q.device).manual_seed(9))
+    d_o = d_o.bfloat16()
+
+    def fwd():
+        return m(qg, kg, vg, cu, max_len, gates=gg)
+
+    def timed(fn, n):
+        beg, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        beg.record()
+        for _ in range(n):
+            fn()
+        end.record()
+        torch.cuda.synchronize()
+        return beg.elapsed_time(end) / n
+
+    def both():
+        for t in (qg, kg, vg, gg):
+            t.grad = None
+        fwd().backward(d_o)
+
+    for _ in range(warmup):
+        both()
+    ms_both = timed(both, steps)
+    ms_fwd = timed(fwd, steps)
+    assert all(torch.isfinite(t.grad).all() for t in (qg, kg, vg, gg))
+    return {"ms_fwd_bwd": ms_both, "ms_fwd_training_path": ms_fwd, "ms_bwd": ms_both - ms_fwd,
+            "tokens_per_s": total / (ms_both * 1e-3), "model_tflops": 3.5 * f_eff / (ms_both * 1e-3) / 1e12,
+            "mfma_peak_frac": 3.5 * f_eff / (ms_both * 1e-3) / 1e12 / PEAK_BF16_TFLOPS}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -150,6 +189,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-budget", type=float, default=20.0)
     ap.add_argument("--no-decode", action="store_true")
+    ap.add_argument("--no-backward", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (reference point for FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -245,6 +285,8 @@ def main():
                      "unit": "TFLOP/s", "frac": dom_tflops / PEAK_BF16_TFLOPS, "traffic": traffic},
         "stage_effective_tflops": stage_tflops,
     }
+    if not args.no_backward:
+        res["train_step"] = train_bench(m, qd, kd, vd, gd, cu, max_len, total, f_eff, max(2, min(args.steps, 5)), 2)
     if not args.no_decode:
         del qd, kd, vd, gd, out, idx
         torch.cuda.empty_cache()

@@ -94,7 +94,7 @@ class NSAAttention(nn.Module):
             scale = 1.0 / math.sqrt(dk)
         uniform = not max_seqlen
         seq_len = total // batch if uniform else int(max_seqlen)
-        params = [self.gating.weight, self.gating.bias]
+        params = [] if gates is not None else [self.gating.weight, self.gating.bias]
         if self.compressor.mode != "mean":
             params += list(self.compressor.parameters())
         if needs_grad(q, k, v, gates, *params):
@@ -105,6 +105,10 @@ class NSAAttention(nn.Module):
                                        return_indices)
 
     def _forward_train(self, q, k, v, cu, batch, scale, causal, seq_len, uniform, gates, return_indices):
+        if q.dtype != torch.bfloat16 or self.selection_block_size != 64:
+            raise NotImplementedError(
+                "the NSA backward kernels are built for bfloat16 and 64-key selection blocks; run inference under "
+                "torch.no_grad() (an input or a parameter of this call requires grad)")
         ck, cv, cu_cmp, nc = self.compressor.compress_packed(k, v, cu, seq_len=seq_len if uniform else None)
         max_nc = nc if nc is not None else conv_compressed_len(seq_len, self.compression_stride,
                                                                self.compression_block)

@@ -332,7 +332,8 @@ def _module_case(dtype, lens, Hq, Hkv, Dk, Dv, S, W, seed, scale_in, mode="mean"
     m = m.to(DEV)
     uniform = len(set(lens)) == 1
     cu = _cu(lens)
-    out, idx = m(q.to(DEV), k.to(DEV), v.to(DEV), cu, 0 if uniform else max(lens), gates=gl.to(DEV),
+    with torch.no_grad():       # parameters require grad: without this the un-fused training path would run
+        out, idx = m(q.to(DEV), k.to(DEV), v.to(DEV), cu, 0 if uniform else max(lens), gates=gl.to(DEV),
                  return_indices=True)
     out, idx = out.cpu(), idx.cpu().long()
     gates = torch.sigmoid(gl.float()).to(dtype) if act == "sigmoid" else gl
@@ -448,7 +449,8 @@ def test_module_own_gating_equals_explicit_gates():
     m = NSAAttention(D, causal=True, selected_block_count=8, sliding_window=128, dtype=dtype, compressor_mode="mean",
                      gate_activation="sigmoid").to(DEV)
     cu = _cu([T])
-    a = m(q.to(DEV), k.to(DEV), v.to(DEV), cu, 0)
+    with torch.no_grad():
+        a = m(q.to(DEV), k.to(DEV), v.to(DEV), cu, 0)
     gl = _ops().gate_logits(q.to(DEV), m.gating.weight, m.gating.bias)
     ref_gl = torch.nn.functional.linear(q.float(), m.gating.weight.detach().float().cpu(),
                                         m.gating.bias.detach().float().cpu())

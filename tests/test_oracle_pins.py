@@ -295,3 +295,63 @@ def test_short_sequence_has_compressed_branch_but_no_selection():
     out, parts = O.nsa_forward_single(q, k, v, gates, p, return_parts=True)
     assert (parts["idx"] == -1).all() and torch.count_nonzero(parts["o_slc"]) == 0
     assert torch.count_nonzero(parts["o_cmp"][32:]) > 0 and torch.count_nonzero(parts["o_cmp"][:32]) == 0
+
+
+# ----------------------------------------------------------------------------- gradients
+# The backward kernels are checked against autograd through the oracle's forward in float64.  These
+# pins show that this is the right derivative: finite differences on tiny inputs (a dropped term or a
+# wrong sign in any branch fails them) and the library's own attention gradient on the dense cases.
+
+def _tiny(T=7, Hq=4, Hkv=2, Dk=4, Dv=3, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    mk = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64).requires_grad_(True)
+    return mk(T, Hq, Dk), mk(T, Hkv, Dk), mk(T, Hkv, Dv)
+
+
+def test_oracle_gradients_pass_finite_differences():
+    q, k, v = _tiny()
+    assert torch.autograd.gradcheck(lambda a, b, c: O.sliding_attention(a, b, c, 3, 0.5, math_dtype=torch.float64),
+                                    (q, k, v), eps=1e-6, atol=1e-6)
+    idx = torch.tensor([[[0, 1]], [[1, 0]], [[0, 5]], [[1, -1]], [[2, 0]], [[0, 1]], [[3, 1]]]).expand(7, 2, 2)
+    assert torch.autograd.gradcheck(
+        lambda a, b, c: O.selected_attention(a, b, c, idx, None, 2, 0.5, math_dtype=torch.float64),
+        (q, k, v), eps=1e-6, atol=1e-6)
+    g = torch.Generator().manual_seed(1)
+    ck = torch.randn(3, 2, 4, generator=g, dtype=torch.float64).requires_grad_(True)
+    cv = torch.randn(3, 2, 3, generator=g, dtype=torch.float64).requires_grad_(True)
+    assert torch.autograd.gradcheck(
+        lambda a, b, c: O.compressed_attention(a, b, c, 2, 2, 0.5, math_dtype=torch.float64),
+        (q, ck, cv), eps=1e-6, atol=1e-6)
+    x = torch.randn(9, 2, 3, generator=g, dtype=torch.float64).requires_grad_(True)
+    w = torch.randn(4 * 3, 3, generator=g, dtype=torch.float64).requires_grad_(True)
+    b = torch.randn(3, generator=g, dtype=torch.float64).requires_grad_(True)
+    assert torch.autograd.gradcheck(lambda a, ww, bb: O.compress_weighted(a, ww, bb, 4, 2, 3, math_dtype=torch.float64),
+                                    (x, w, b), eps=1e-6, atol=1e-6)
+    assert torch.autograd.gradcheck(lambda a: O.compress_meanpool(a, 4, 2, 3, math_dtype=torch.float64), (x,),
+                                    eps=1e-6, atol=1e-6)
+
+
+def test_oracle_gradients_match_library_attention_on_dense_cases():
+    """A window that covers the sequence, and all blocks selected, are plain causal attention: the
+    oracle's gradients must equal those of F.scaled_dot_product_attention."""
+    T, Hq, Hkv, D = 12, 4, 2, 8
+    q, k, v = _tiny(T, Hq, Hkv, D, D, seed=3)
+    d_o = torch.randn(T, Hq, D, generator=torch.Generator().manual_seed(4), dtype=torch.float64)
+
+    def grads(fn):
+        ins = [t.detach().clone().requires_grad_(True) for t in (q, k, v)]
+        fn(*ins).backward(d_o)
+        return [t.grad for t in ins]
+
+    def sdpa(a, b, c):
+        kk, vv = b.repeat_interleave(Hq // Hkv, 1), c.repeat_interleave(Hq // Hkv, 1)
+        o = F.scaled_dot_product_attention(a.transpose(0, 1), kk.transpose(0, 1), vv.transpose(0, 1), is_causal=True,
+                                           scale=0.3)
+        return o.transpose(0, 1)
+
+    ref = grads(sdpa)
+    idx = torch.arange(3).expand(T, Hkv, 3)
+    for fn in (lambda a, b, c: O.sliding_attention(a, b, c, T, 0.3, math_dtype=torch.float64),
+               lambda a, b, c: O.selected_attention(a, b, c, idx, None, 4, 0.3, math_dtype=torch.float64)):
+        for got, want in zip(grads(fn), ref):
+            assert float((got - want).abs().max()) < 1e-10
