@@ -121,6 +121,25 @@ int nsa_block_select_fwd(const void* q, const void* ck, const float* lse, void* 
 int nsa_gate_fwd(const void* q, const void* weight, const void* bias, void* gates, int64_t rows, int dim, int dtype,
                  nsa_stream_t stream);
 
+/* Backward of nsa_gate_fwd (autograd of the gating nn.Linear, nsa/nsa.py:61,117, in the reference):
+ * d_gates [rows, 3] -> dq [rows, dim] = d_gates . weight (fully overwritten; the caller adds it to
+ * the attention branches' dq), dweight float [3, dim] and dbias float [3] (NULL to skip), both
+ * overwritten. */
+int nsa_gate_bwd(const void* q, const void* weight, const void* d_gates, void* dq, float* dweight, float* dbias,
+                 int64_t rows, int dim, int dtype, nsa_stream_t stream);
+
+/* The gated sum on its own, for the training path, and its backward.  Replace the addcmul chain of
+ * nsa/selection_attn.py:808-811 and nsa/nsa.py:133 and its autograd.
+ *   gate_logits [rows, 3] (selected, sliding, compressed), pre-activation; o_* [rows, dv] (o_swa,
+ *   o_cmp may be NULL: term dropped);  out = sum_b act(gate_b) * o_b.
+ *   backward: d_b = act(gate_b) * d_out for every branch given, d_gate_logits[row][b] =
+ *   act'(gate_b) * <d_out[row], o_b[row]> (0 for a missing branch). */
+int nsa_gate_combine_fwd(const void* gate_logits, const void* o_slc, const void* o_swa, const void* o_cmp, void* out,
+                         int64_t rows, int dv, int gate_act, int dtype, nsa_stream_t stream);
+int nsa_gate_combine_bwd(const void* gate_logits, const void* d_out, const void* o_slc, const void* o_swa,
+                         const void* o_cmp, void* d_slc, void* d_swa, void* d_cmp, void* d_gate_logits, int64_t rows,
+                         int dv, int gate_act, int dtype, nsa_stream_t stream);
+
 /* Sliding window attention: token t attends keys [max(0, t-window+1), t] of its sequence.  Replaces
  * the window loop of nsa/selection_attn.py:483-517.  q [total,hq,dk], k [total,hkv,dk],
  * vt transposed [hkv][dv][vt_cols] over cu_seqlens, o [total,hq,dv]; lse (optional, float

@@ -31,6 +31,9 @@ SIGNATURES = {
     "nsa_block_select_fwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _L, _L, _I, _I, _I, _I, _I, _I,
                                   _I, _I, _P]),
     "nsa_gate_fwd": (_I, [_P, _P, _P, _P, _L, _I, _I, _P]),
+    "nsa_gate_bwd": (_I, [_P] * 6 + [_L, _I, _I, _P]),
+    "nsa_gate_combine_fwd": (_I, [_P] * 5 + [_L, _I, _I, _I, _P]),
+    "nsa_gate_combine_bwd": (_I, [_P] * 9 + [_L, _I, _I, _I, _P]),
     "nsa_swa_fwd": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P]),
     "nsa_slc_combine_fwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I,
                                  _I, _I, _I, _I, _F, _I, _I, _I, _P, _L, _P]),

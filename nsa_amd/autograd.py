@@ -102,3 +102,35 @@ class SlcSwaFn(torch.autograd.Function):
         dq, dk, dv = ops.slc_swa_bwd(q, k, v, o_slc, d_slc, lse_slc, o_swa, d_swa, lse_swa, idx, counts, cu, batch,
                                      block_size, window, scale)
         return dq, dk, dv, None, None, None, None, None, None, None
+
+
+class GateLinearFn(torch.autograd.Function):
+    """Gate logits [total,Hq,3] = q . weight^T + bias (the gating nn.Linear of nsa/nsa.py:61)."""
+
+    @staticmethod
+    def forward(ctx, q, weight, bias):
+        q = q.contiguous()
+        ctx.save_for_backward(q, weight, bias)
+        return ops.gate_logits(q, weight.detach(), None if bias is None else bias.detach())
+
+    @staticmethod
+    def backward(ctx, d_gates):
+        q, weight, bias = ctx.saved_tensors
+        dq, dw, db = ops.gate_bwd(q, weight.detach(), d_gates, want_dbias=bias is not None)
+        return dq, dw.to(weight.dtype), None if db is None else db.to(bias.dtype)
+
+
+class GateCombineFn(torch.autograd.Function):
+    """out = sum_b act(gate_logits[..., b]) * o_b, b = (selected, sliding, compressed)."""
+
+    @staticmethod
+    def forward(ctx, gate_logits, o_slc, o_swa, o_cmp, gate_act):
+        ctx.save_for_backward(gate_logits, o_slc, o_swa, o_cmp)
+        ctx.gate_act = gate_act
+        return ops.gate_combine(gate_logits, o_slc, o_swa, o_cmp, gate_act)
+
+    @staticmethod
+    def backward(ctx, d_out):
+        gate_logits, o_slc, o_swa, o_cmp = ctx.saved_tensors
+        d_slc, d_swa, d_cmp, d_gl = ops.gate_combine_bwd(gate_logits, d_out, o_slc, o_swa, o_cmp, ctx.gate_act)
+        return d_gl.to(gate_logits.dtype), d_slc, d_swa, d_cmp, None

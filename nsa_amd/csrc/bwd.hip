@@ -33,6 +33,7 @@ int set_smem(const void* fn, size_t bytes);
 
 constexpr int kBwdCmp = 0, kBwdSwa = 1, kBwdSlc = 2;
 constexpr int kCmpSplit = 1024;      // tokens of one compressed-branch work item
+constexpr int kSegGroup = 4;         // selected branch: consecutive 64-pair segments of a block per workgroup
 
 struct BwdArgs {
   const void* q; const void* d_o; const float* lse; const float* delta;    // rows: [total][hq][.]
@@ -104,7 +105,7 @@ __device__ __forceinline__ void store4(float* p, const f32x4_t& v, float s) {
 // ---- key-stationary: dK, dV (and the dQ partials of the selected branch) ---------------------------
 
 template <typename T, int DK, int DV, int MODE, int NW>
-__global__ void __launch_bounds__(NW * 64)
+__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 bwd_kv_kernel(const BwdArgs a) {
   constexpr int QLD = DK + 8, OLD = DV + 8, NT = NW * 64, SLD = kBlk + 8;
   constexpr int QP = 32 * DK / 8, OP = 32 * DV / 8;                 // 16-byte pieces of one chunk
@@ -129,12 +130,13 @@ bwd_kv_kernel(const BwdArgs a) {
     const int item = blockIdx.x;
     if (item >= *a.ws.n_items) return;
     const int key = a.ws.items[2 * item], seg = a.ws.items[2 * item + 1];
+    if (seg % kSegGroup != 0) return;         // the workgroup of segment 4i also takes 4i+1 .. 4i+3
     h = key / a.ws.nb;
     const SeqTile st = find_tile(a.cu_seq, a.batch, kBlk, key % a.ws.nb);
     if (!st.valid) return;
     seq_start = st.start; key0 = st.t0; nkeys = st.len; key_base = st.start;
     first = a.ws.offsets[key] + seg * kSeg;
-    count = min(a.ws.counts[key] - seg * kSeg, kSeg);
+    count = min(a.ws.counts[key] - seg * kSeg, kSegGroup * kSeg);
     nchunks = (count + 1) >> 1;
   } else if (MODE == kBwdSwa) {
     const SeqTile st = find_tile(a.cu_seq, a.batch, NW * 16, blockIdx.x);

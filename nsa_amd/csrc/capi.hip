@@ -170,6 +170,46 @@ int nsa_gate_fwd(const void* q, const void* weight, const void* bias, void* gate
   return finish(nsa::launch_gate(q, weight, bias, gates, (long)rows, dim, dtype, stream), "gate");
 }
 
+int nsa_gate_bwd(const void* q, const void* weight, const void* d_gates, void* dq, float* dweight, float* dbias,
+                 int64_t rows, int dim, int dtype, nsa_stream_t stream) {
+  if (!q || !weight || !d_gates || !dq || !dweight) return fail(NSA_ERR_INVALID, "gate_bwd: null pointer");
+  if (rows <= 0 || dim <= 0 || dim % 8 != 0) return fail(NSA_ERR_INVALID, "gate_bwd: rows must be positive and dim a positive multiple of 8");
+  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "gate_bwd: bad dtype");
+  if (!aligned16(q) || !aligned16(weight) || !aligned16(dq)) return fail(NSA_ERR_INVALID, "gate_bwd: pointers must be 16-byte aligned");
+  const int rc = nsa::launch_gate_bwd(q, weight, d_gates, dq, dweight, dbias, (long)rows, dim, dtype, stream);
+  if (rc == -2) return fail(NSA_ERR_UNSUPPORTED, "gate_bwd: built for dim 32/64/128/192/256");
+  return finish(rc, "gate_bwd");
+}
+
+static int gate_combine_common(const char* what, const nsa::GateCombineArgs& a, nsa_stream_t stream) {
+  if (!a.gate_logits || !a.o_slc) return fail(NSA_ERR_INVALID, "%s: null pointer", what);
+  if (a.rows <= 0 || a.dv <= 0 || a.dv % 8 != 0) return fail(NSA_ERR_INVALID, "%s: rows must be positive and dv a positive multiple of 8", what);
+  if (a.dtype != NSA_BF16 && a.dtype != NSA_F32) return fail(NSA_ERR_INVALID, "%s: bad dtype", what);
+  if (a.act != NSA_GATE_IDENTITY && a.act != NSA_GATE_SIGMOID) return fail(NSA_ERR_INVALID, "%s: bad gate activation", what);
+  const void* ptrs[] = {a.o_slc, a.o_swa, a.o_cmp, a.out, a.d_out, a.d_slc, a.d_swa, a.d_cmp};
+  for (const void* p : ptrs)
+    if (p && !aligned16(p)) return fail(NSA_ERR_INVALID, "%s: pointers must be 16-byte aligned", what);
+  return finish(nsa::launch_gate_combine(a, stream), what);
+}
+
+int nsa_gate_combine_fwd(const void* gate_logits, const void* o_slc, const void* o_swa, const void* o_cmp, void* out,
+                         int64_t rows, int dv, int gate_act, int dtype, nsa_stream_t stream) {
+  if (!out) return fail(NSA_ERR_INVALID, "gate_combine: null pointer");
+  nsa::GateCombineArgs a{gate_logits, o_slc, o_swa, o_cmp, out, nullptr, nullptr, nullptr, nullptr, nullptr,
+                         (long)rows, dv, gate_act, dtype};
+  return gate_combine_common("gate_combine", a, stream);
+}
+
+int nsa_gate_combine_bwd(const void* gate_logits, const void* d_out, const void* o_slc, const void* o_swa,
+                         const void* o_cmp, void* d_slc, void* d_swa, void* d_cmp, void* d_gate_logits, int64_t rows,
+                         int dv, int gate_act, int dtype, nsa_stream_t stream) {
+  if (!d_out || !d_slc || !d_gate_logits || (o_swa && !d_swa) || (o_cmp && !d_cmp))
+    return fail(NSA_ERR_INVALID, "gate_combine_bwd: null pointer");
+  nsa::GateCombineArgs a{gate_logits, o_slc, o_swa, o_cmp, nullptr, d_out, d_slc, d_swa, d_cmp, d_gate_logits,
+                         (long)rows, dv, gate_act, dtype};
+  return gate_combine_common("gate_combine_bwd", a, stream);
+}
+
 int nsa_swa_fwd(const void* q, const void* k, const void* vt, void* o, float* lse, const int32_t* cu_seqlens, int batch,
                 int total, int hq, int hkv, int dk, int dv, int vt_cols, int window, float scale, int dtype,
                 nsa_stream_t stream) {

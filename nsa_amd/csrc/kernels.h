@@ -80,6 +80,15 @@ struct SlcSwaBwdArgs {
   void* dq; void* dk_out; void* dv_out; void* workspace;
 };
 
+// Gated sum of the branches (d_out == nullptr: forward into out) or its backward (d_out given:
+// d_slc / d_swa / d_cmp = act(gate) * d_out and d_gate_logits).  gate_logits [rows][3] (selected,
+// sliding, compressed), branch tensors [rows][dv]; o_swa / o_cmp (and their gradients) may be null.
+struct GateCombineArgs {
+  const void* gate_logits; const void* o_slc; const void* o_swa; const void* o_cmp; void* out;
+  const void* d_out; void* d_slc; void* d_swa; void* d_cmp; void* d_gate_logits;
+  long rows; int dv, act, dtype;
+};
+
 struct DecodeArgs {
   const void* q; const void* k_cache; const void* v_cache_t; const void* ck_cache; const void* cv_cache_t;
   const int32_t* ctx_lens; const void* gates; void* out; int32_t* indices;
@@ -93,6 +102,9 @@ int launch_compress_bwd(const CompressBwdArgs& a, hipStream_t st);
 int launch_transpose(const TransposeArgs& a, hipStream_t st);
 int launch_gate(const void* x, const void* w, const void* bias, void* out, long rows, int dim, int dtype,
                 hipStream_t st);
+int launch_gate_combine(const GateCombineArgs& a, hipStream_t st);
+int launch_gate_bwd(const void* q, const void* w, const void* d_gl, void* dq, float* dw, float* db, long rows,
+                    int dim, int dtype, hipStream_t st);
 int launch_cmp_attn(const CmpArgs& a, hipStream_t st);
 int launch_select(const CmpArgs& a, hipStream_t st);
 int launch_swa(const SwaArgs& a, hipStream_t st);

@@ -8,7 +8,7 @@ import torch
 from torch import nn
 
 from . import _lib, ops
-from .autograd import CmpAttnFn, SlcSwaFn, needs_grad
+from .autograd import CmpAttnFn, GateCombineFn, GateLinearFn, SlcSwaFn, needs_grad
 from .compression_kv import KVCompressor, conv_compressed_len
 
 
@@ -16,8 +16,7 @@ class NSAAttention(nn.Module):
     """Native Sparse Attention: compress -> compressed attention + block selection ->
     selected + sliding-window attention -> gated sum, all on hand-written gfx950 kernels.  Without
     grad the fused inference schedule runs; when an input or a parameter requires grad the branches run
-    un-fused through autograd functions whose backward is hand-written as well (the gating Linear and
-    the gated sum then go through torch ops, as in the reference).
+    un-fused through autograd functions whose backward kernels are hand-written as well.
 
     Parameters follow the reference (`compressor.compressor_k/v.{weight,bias}`,
     `gating.{weight,bias}`), so its state_dict loads.  Two build-owned switches:
@@ -118,11 +117,9 @@ class NSAAttention(nn.Module):
         o_slc, o_swa = SlcSwaFn.apply(q, k, v, idx, None, cu, batch, self.selection_block_size,
                                       self.sliding_window, float(scale))
         if gates is None:
-            gates = torch.nn.functional.linear(q, self.gating.weight.to(q.dtype), self.gating.bias.to(q.dtype))
-        g = torch.sigmoid(gates) if self.gate_activation == "sigmoid" else gates
-        out = g[..., 0:1] * o_slc + g[..., 2:3] * o_cmp
-        if o_swa is not None:
-            out = out + g[..., 1:2] * o_swa
+            gates = GateLinearFn.apply(q, self.gating.weight, self.gating.bias)
+        act = _lib.GATE_SIGMOID if self.gate_activation == "sigmoid" else _lib.GATE_IDENTITY
+        out = GateCombineFn.apply(gates, o_slc, o_swa, o_cmp, act)
         if return_indices:
             return out, idx
         return out

@@ -395,3 +395,53 @@ def compress_bwd(d_out, cu_seqlens, cu_out, total, block, stride, x=None, w_lin=
                                           _dtype_code(d_out), _stream())
         _lib.check(rc, "nsa_compress_bwd")
     return dx if w_lin is None else (dx, dw, dbias)
+
+
+def gate_bwd(q, weight, d_gates, want_dbias=True):
+    """Backward of gate_logits: returns (dq [total,Hq,D], dweight float32 [3,D], dbias float32 [3] or None)."""
+    _need_cuda(q, weight, d_gates)
+    q = _dense(q)
+    total, hq, dim = q.shape
+    weight = weight.to(q.dtype).contiguous()
+    d_gates = d_gates.to(q.dtype).contiguous()
+    dq = torch.empty_like(q)
+    dw = torch.empty(3, dim, dtype=torch.float32, device=q.device)
+    db = torch.empty(3, dtype=torch.float32, device=q.device) if want_dbias else None
+    rc = _lib.load().nsa_gate_bwd(_ptr(q), _ptr(weight), _ptr(d_gates), _ptr(dq), _ptr(dw), _ptr(db), total * hq, dim,
+                                  _dtype_code(q), _stream())
+    _lib.check(rc, "nsa_gate_bwd")
+    return dq, dw, db
+
+
+def gate_combine(gate_logits, o_slc, o_swa, o_cmp, gate_act=0):
+    """out = sum_b act(gate_logits[..., b]) * o_b over (selected, sliding, compressed); o_swa / o_cmp may be None."""
+    _need_cuda(gate_logits, o_slc)
+    gl = _dense(gate_logits.to(o_slc.dtype))
+    o_slc = _dense(o_slc)
+    o_swa = None if o_swa is None else _dense(o_swa)
+    o_cmp = None if o_cmp is None else _dense(o_cmp)
+    total, hq, dv = o_slc.shape
+    out = torch.empty_like(o_slc)
+    rc = _lib.load().nsa_gate_combine_fwd(_ptr(gl), _ptr(o_slc), _ptr(o_swa), _ptr(o_cmp), _ptr(out), total * hq, dv,
+                                          gate_act, _dtype_code(o_slc), _stream())
+    _lib.check(rc, "nsa_gate_combine_fwd")
+    return out
+
+
+def gate_combine_bwd(gate_logits, d_out, o_slc, o_swa, o_cmp, gate_act=0):
+    """Returns (d_o_slc, d_o_swa or None, d_o_cmp or None, d_gate_logits [total,Hq,3])."""
+    _need_cuda(gate_logits, d_out, o_slc)
+    gl = _dense(gate_logits.to(o_slc.dtype))
+    d_out, o_slc = _dense(d_out), _dense(o_slc)
+    o_swa = None if o_swa is None else _dense(o_swa)
+    o_cmp = None if o_cmp is None else _dense(o_cmp)
+    total, hq, dv = o_slc.shape
+    d_slc = torch.empty_like(o_slc)
+    d_swa = None if o_swa is None else torch.empty_like(o_slc)
+    d_cmp = None if o_cmp is None else torch.empty_like(o_slc)
+    d_gl = torch.empty(total, hq, 3, dtype=o_slc.dtype, device=o_slc.device)
+    rc = _lib.load().nsa_gate_combine_bwd(_ptr(gl), _ptr(d_out), _ptr(o_slc), _ptr(o_swa), _ptr(o_cmp), _ptr(d_slc),
+                                          _ptr(d_swa), _ptr(d_cmp), _ptr(d_gl), total * hq, dv, gate_act,
+                                          _dtype_code(o_slc), _stream())
+    _lib.check(rc, "nsa_gate_combine_bwd")
+    return d_slc, d_swa, d_cmp, d_gl

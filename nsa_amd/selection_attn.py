@@ -9,7 +9,7 @@ from typing import Optional, Union
 import torch
 
 from . import ops
-from .autograd import SlcSwaFn, needs_grad
+from .autograd import GateCombineFn, SlcSwaFn, needs_grad
 
 
 def _packed(x, B, T):
@@ -80,9 +80,9 @@ def parallel_nsa(q: torch.Tensor,
     idx = block_indices.reshape(B * T, H, -1)
     if needs_grad(q, k, v, g_slc, g_swa):
         o_slc, o_swa = SlcSwaFn.apply(qp, kp, vp, idx, counts, cu, nb, block_size, window_size, float(scale))
-        o = o_slc * g_slc.reshape(B * T, HQ, 1)
-        if o_swa is not None:
-            o = o + o_swa * g_swa.reshape(B * T, HQ, 1)
+        gs = g_slc.reshape(B * T, HQ).to(q.dtype)
+        gw = g_swa.reshape(B * T, HQ).to(q.dtype) if o_swa is not None else torch.zeros_like(gs)
+        o = GateCombineFn.apply(torch.stack((gs, gw, torch.zeros_like(gs)), -1), o_slc, o_swa, None, 0)
     else:
         with torch.no_grad():
             o = _parallel_nsa_nograd(qp, kp, vp, idx, counts, g_slc, g_swa, cu, nb, block_size, window_size, scale)

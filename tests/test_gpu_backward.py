@@ -384,3 +384,44 @@ def test_compress_kv_backward():
         print("compress_kv_bwd", name)
         _check("dx", xd.grad, xr.grad, dtype)
         _check("dw", w.grad, wr.grad, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("T,Hq,D,Dv,act", [(300, 16, 64, 64, 1), (257, 6, 192, 128, 0), (64, 4, 128, 128, 1)])
+def test_gate_and_combine_kernels(dtype, T, Hq, D, Dv, act):
+    """nsa_gate_combine_fwd / _bwd and nsa_gate_bwd against the same arithmetic in torch float64."""
+    ops = _ops()
+    q = randn(T, Hq, D, seed=220, scale=0.7, dtype=dtype)
+    w = randn(3, D, seed=221, scale=0.2, dtype=dtype)
+    gl = randn(T, Hq, 3, seed=222, dtype=dtype)
+    o = [randn(T, Hq, Dv, seed=223 + i, dtype=dtype) for i in range(3)]
+    d_out = randn(T, Hq, Dv, seed=227, dtype=dtype)
+    d_gl_in = randn(T, Hq, 3, seed=228, dtype=dtype)
+    f = torch.sigmoid if act else (lambda x: x)
+    for with_swa, with_cmp in ((True, True), (False, True), (True, False)):
+        od = [o[0].to(DEV), o[1].to(DEV) if with_swa else None, o[2].to(DEV) if with_cmp else None]
+        out = ops.gate_combine(gl.to(DEV), od[0], od[1], od[2], act)
+        d_slc, d_swa, d_cmp, d_gl = ops.gate_combine_bwd(gl.to(DEV), d_out.to(DEV), od[0], od[1], od[2], act)
+        glr = gl.double().requires_grad_(True)
+        orr = [t.double().requires_grad_(True) for t in o]
+        g = f(glr)
+        ref = g[..., 0:1] * orr[0]
+        if with_swa:
+            ref = ref + g[..., 1:2] * orr[1]
+        if with_cmp:
+            ref = ref + g[..., 2:3] * orr[2]
+        ref.backward(d_out.double())
+        _check("out", out, ref.detach(), dtype)
+        _check("dslc", d_slc, orr[0].grad, dtype)
+        if with_swa:
+            _check("dswa", d_swa, orr[1].grad, dtype)
+        if with_cmp:
+            _check("dcmp", d_cmp, orr[2].grad, dtype)
+        _check("dgl", d_gl, glr.grad, dtype, floor=float(glr.grad.abs().max()) if dtype == torch.bfloat16 else 1.0)
+    dq, dw, db = ops.gate_bwd(q.to(DEV), w.to(DEV), d_gl_in.to(DEV))
+    qr, wr = q.double().requires_grad_(True), w.double().requires_grad_(True)
+    br = torch.zeros(3, dtype=torch.float64, requires_grad=True)
+    (qr @ wr.t() + br).backward(d_gl_in.double())
+    _check("dq", dq, qr.grad, dtype)
+    _check("dw", dw, wr.grad, dtype)
+    _check("db", db, br.grad, dtype)
