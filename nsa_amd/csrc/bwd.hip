@@ -31,8 +31,14 @@ namespace nsa {
 
 int set_smem(const void* fn, size_t bytes);
 
+#ifndef NSA_CMP_SPLIT
+#define NSA_CMP_SPLIT 256
+#endif
+#ifndef NSA_KV_NW
+#define NSA_KV_NW 4
+#endif
 constexpr int kBwdCmp = 0, kBwdSwa = 1, kBwdSlc = 2;
-constexpr int kCmpSplit = 1024;      // tokens of one compressed-branch work item
+constexpr int kCmpSplit = NSA_CMP_SPLIT;     // tokens of one compressed-branch work item
 constexpr int kSegGroup = 4;         // selected branch: consecutive 64-pair segments of a block per workgroup
 
 struct BwdArgs {
@@ -353,7 +359,9 @@ bwd_q_kernel(const BwdArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 15, g = lane >> 4;
   const int G = a.hq / a.hkv;
-  const SeqTile st = find_tile(a.cu_seq, a.batch, NW, blockIdx.x);
+  // compressed branch: the work of a tile grows with its position, so the last tiles start first
+  const int tile_id = MODE == kBwdCmp ? (int)(gridDim.x - 1 - blockIdx.x) : (int)blockIdx.x;
+  const SeqTile st = find_tile(a.cu_seq, a.batch, NW, tile_id);
   if (!st.valid) return;
   const int h = blockIdx.y;
   const int tok = st.t0 + wave;
@@ -612,7 +620,7 @@ static int launch_cmp_bwd_t(const CmpBwdArgs& c, hipStream_t st) {
   if (c.cmp_rows > 0) {
     fill_zero(dk_acc, (long)c.cmp_rows * c.hkv * DK, st);
     fill_zero(dv_acc, (long)c.cmp_rows * c.hkv * DV, st);
-    rc = launch_kv_t<T, DK, DV, kBwdCmp, 8>(a, c.cmp_rows, st);
+    rc = launch_kv_t<T, DK, DV, kBwdCmp, NSA_KV_NW>(a, c.cmp_rows, st);
     if (rc) return rc;
     cast_out<T>(dk_acc, c.dck, (long)c.cmp_rows * c.hkv * DK, st);
     cast_out<T>(dv_acc, c.dcv, (long)c.cmp_rows * c.hkv * DV, st);
@@ -660,7 +668,7 @@ static int launch_slc_swa_bwd_t(const SlcSwaBwdArgs& c, hipStream_t st) {
     launch_delta<T>(c.o_swa, c.d_o_swa, delta_swa, (long)c.total * c.hq, DV, st);
     a.d_o = c.d_o_swa; a.lse = c.lse_swa; a.delta = delta_swa;
     rc = launch_q_t<T, DK, DV, kBwdSwa>(a, st);
-    if (rc == 0) rc = launch_kv_t<T, DK, DV, kBwdSwa, 8>(a, c.total, st);
+    if (rc == 0) rc = launch_kv_t<T, DK, DV, kBwdSwa, NSA_KV_NW>(a, c.total, st);
     if (rc) return rc;
   }
   if (slc) {
