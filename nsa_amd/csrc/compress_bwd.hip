@@ -12,8 +12,7 @@
 // from global memory (the weights are L2 resident).  Every dx row is written exactly once.
 // dW: contraction over the (window, head) rows, so both operands are read with the transposing
 // fragment load from row-major LDS tiles; one workgroup per (j, 256-row chunk), fp32 atomics.
-#include "common.h"
-#include "kernels.h"
+#include "tiles.h"
 
 namespace nsa {
 
@@ -24,26 +23,6 @@ __device__ __forceinline__ int upper_seq_of(const int32_t* __restrict__ cu, int 
     if (cu[mid] <= r) lo = mid; else hi = mid;
   }
   return lo;
-}
-
-__device__ __forceinline__ bf16x8_t frag_tr(const bf16_t* tile, int ld, int lane) {
-  typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
-  typedef __attribute__((address_space(3))) bf16x4_t lds_bf16x4_t;
-  const int i = lane & 15, g = lane >> 4;
-  const bf16_t* p = tile + (8 * g + (i >> 2)) * ld + 4 * (i & 3);
-  const bf16x4_t a = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_t*)p);
-  const bf16x4_t b = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_t*)(p + 4 * ld));
-  bf16x8_t r;
-  r[0] = a[0]; r[1] = a[1]; r[2] = a[2]; r[3] = a[3];
-  r[4] = b[0]; r[5] = b[1]; r[6] = b[2]; r[7] = b[3];
-  return r;
-}
-__device__ __forceinline__ f32x8_t frag_tr(const float* tile, int ld, int lane) {
-  const int m = lane & 15, g = lane >> 4;
-  f32x8_t r;
-#pragma unroll
-  for (int j = 0; j < 8; ++j) r[j] = tile[(8 * g + j) * ld + m];
-  return r;
 }
 
 // ---- dx, mean pooling: one thread per (token, 8 channels of the heads*dim row)
@@ -184,12 +163,12 @@ compress_dw_kernel(const T* __restrict__ x, const T* __restrict__ d_out, float* 
     __syncthreads();
     vec8_t<T> bfr[TO];
 #pragma unroll
-    for (int t = 0; t < TO; ++t) bfr[t] = frag_tr(ds + 16 * t, LD, lane);
+    for (int t = 0; t < TO; ++t) bfr[t] = load8_tr(ds + 16 * t, LD, lane);
 #pragma unroll
     for (int a = 0; a < TI; ++a) {
       const int ti = wave + 4 * a;
       if (ti < DIM / 16) {
-        const vec8_t<T> af = frag_tr(xs + 16 * ti, LD, lane);
+        const vec8_t<T> af = load8_tr(xs + 16 * ti, LD, lane);
 #pragma unroll
         for (int t = 0; t < TO; ++t) acc[a][t] = mma16(af, bfr[t], acc[a][t]);
       }

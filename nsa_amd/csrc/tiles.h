@@ -55,6 +55,32 @@ __device__ __forceinline__ void pv32_all(const T* __restrict__ vp, long tile_str
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// transposing fragment load
+// tile points at element (row0, col0) of a row-major LDS tile with row pitch ld.  Lane (m = lane%16,
+// g = lane/16) receives tile[8g + j][m], j = 0..7: the A operand of a product whose depth runs over
+// the tile's rows.  bf16: two ds_read_b64_tr_b16, each transposing a 4 x 16 block per 16 lanes (lane
+// 4a+b supplies the address of row a, columns 4b..4b+3 and receives column 4a'+b' of rows 0..3).
+__device__ __forceinline__ bf16x8_t load8_tr(const bf16_t* tile, int ld, int lane) {
+  typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
+  typedef __attribute__((address_space(3))) bf16x4_t lds_bf16x4_t;
+  const int i = lane & 15, g = lane >> 4;
+  const bf16_t* p = tile + (8 * g + (i >> 2)) * ld + 4 * (i & 3);
+  const bf16x4_t a = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_t*)p);
+  const bf16x4_t b = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_t*)(p + 4 * ld));
+  bf16x8_t r;
+  r[0] = a[0]; r[1] = a[1]; r[2] = a[2]; r[3] = a[3];
+  r[4] = b[0]; r[5] = b[1]; r[6] = b[2]; r[7] = b[3];
+  return r;
+}
+__device__ __forceinline__ f32x8_t load8_tr(const float* tile, int ld, int lane) {
+  const int m = lane & 15, g = lane >> 4;
+  f32x8_t r;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) r[j] = tile[(8 * g + j) * ld + m];
+  return r;
+}
+
 struct RowMap {
   int tok;      // token of this lane's column (sequence local), may be >= len
   int gidx;     // head inside the GQA group, may be >= G
