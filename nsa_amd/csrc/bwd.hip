@@ -320,8 +320,11 @@ bwd_kv_kernel(const BwdArgs a) {
 
 // ---- query-stationary: dQ of the compressed and sliding branches -----------------------------------
 
+#ifndef NSA_Q_WPE
+#define NSA_Q_WPE 4
+#endif
 template <typename T, int DK, int DV, int MODE, int NW>
-__global__ void __launch_bounds__(NW * 64)
+__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NSA_Q_WPE, NSA_Q_WPE)))
 bwd_q_kernel(const BwdArgs a) {
   constexpr int KLD = DK + 8, VLD = DV + 8, NT = NW * 64;
   constexpr int KP = 32 * DK / 8, VP = 32 * DV / 8;
@@ -539,7 +542,10 @@ static int launch_kv_t(const BwdArgs& a, int key_rows, hipStream_t st) {
 
 template <typename T, int DK, int DV, int MODE>
 static int launch_q_t(const BwdArgs& a, hipStream_t st) {
-  constexpr int NW = 8;
+#ifndef NSA_Q_NW
+#define NSA_Q_NW 16
+#endif
+  constexpr int NW = NSA_Q_NW;
   const size_t smem = 2 * (size_t)(32 * (DK + 8) + 32 * (DV + 8)) * sizeof(T);
   auto fn = bwd_q_kernel<T, DK, DV, MODE, NW>;
   const int rc = set_smem(reinterpret_cast<const void*>(fn), smem);
