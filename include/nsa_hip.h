@@ -1,8 +1,10 @@
-/* C ABI of libnsa_hip.so: the gfx950 kernels behind the NSA forward path.
+/* C ABI of libnsa_hip.so: the gfx950 kernels behind the NSA forward path and its backward.
  *
  * Conventions
  *   - every pointer is a DEVICE pointer unless stated otherwise; the library never allocates, frees
  *     or synchronises; work is enqueued on `stream` and outputs are fully overwritten
+ *   - the backward entry points (nsa_*_bwd) accumulate dK / dV with fp32 atomics inside their workspace:
+ *     results agree from run to run to rounding, not bit for bit
  *   - tensors are packed ("varlen"): rows of all sequences back to back, `cu_seqlens` int32[batch+1]
  *     with cu_seqlens[0] == 0 holds the row offsets; a batch of equal lengths is the special case
  *     cu_seqlens[b] = b*T

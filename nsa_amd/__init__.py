@@ -1,7 +1,7 @@
-"""MI355X-native Native Sparse Attention forward path (hand-written gfx950 kernels behind a C ABI).
+"""MI355X-native Native Sparse Attention, forward and backward (hand-written gfx950 kernels behind a C ABI).
 
-Module layout mirrors the reference package so that `import nsa_amd as nsa` is a drop-in for the
-forward path: nsa.selection_attention, nsa.nsa.NSAAttention, nsa.compression_kv.*,
+Module layout mirrors the reference package so that `import nsa_amd as nsa` is a drop-in for that
+path: nsa.selection_attention, nsa.nsa.NSAAttention, nsa.compression_kv.*,
 nsa.triton_attention.flash_attn_func, nsa.selection_attn.parallel_nsa."""
 from .selection_attn import parallel_nsa as selection_attention  # noqa: F401
 from .selection_attn import parallel_nsa, sliding_window_attn  # noqa: F401

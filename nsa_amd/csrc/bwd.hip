@@ -31,14 +31,11 @@ namespace nsa {
 
 int set_smem(const void* fn, size_t bytes);
 
-#ifndef NSA_CMP_SPLIT
-#define NSA_CMP_SPLIT 256
-#endif
-#ifndef NSA_KV_NW
-#define NSA_KV_NW 4
-#endif
 constexpr int kBwdCmp = 0, kBwdSwa = 1, kBwdSlc = 2;
-constexpr int kCmpSplit = NSA_CMP_SPLIT;     // tokens of one compressed-branch work item
+// Launch shapes, chosen by measurement on T = 32768, Hq64/Hkv4, Dk192/Dv128:
+constexpr int kCmpSplit = 256;       // tokens of one compressed-branch work item (1024: 8.6 ms, 256: 5.4 ms)
+constexpr int kKvWaves = 4;          // key-stationary: wavefronts (x16 keys) per workgroup, two workgroups per CU
+constexpr int kQWaves = 16;          // query-stationary: tokens per workgroup (8: 3.7 ms, 16: 3.3 ms)
 constexpr int kSegGroup = 4;         // selected branch: consecutive 64-pair segments of a block per workgroup
 
 struct BwdArgs {
@@ -85,6 +82,8 @@ __device__ __forceinline__ void store4(float* p, const f32x4_t& v, float s) {
 
 // ---- key-stationary: dK, dV (and the dQ partials of the selected branch) ---------------------------
 
+// Two wavefronts per SIMD: left alone the compiler takes 264 registers (one wavefront per SIMD); a budget of
+// 168 (three) spills the accumulators and more than doubles the run time.
 template <typename T, int DK, int DV, int MODE, int NW>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 bwd_kv_kernel(const BwdArgs a) {
@@ -320,11 +319,9 @@ bwd_kv_kernel(const BwdArgs a) {
 
 // ---- query-stationary: dQ of the compressed and sliding branches -----------------------------------
 
-#ifndef NSA_Q_WPE
-#define NSA_Q_WPE 4
-#endif
+// Four wavefronts per SIMD (128 registers, a few of them spilled at Dk = 192): faster than two or three.
 template <typename T, int DK, int DV, int MODE, int NW>
-__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NSA_Q_WPE, NSA_Q_WPE)))
+__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(4, 4)))
 bwd_q_kernel(const BwdArgs a) {
   constexpr int KLD = DK + 8, VLD = DV + 8, NT = NW * 64;
   constexpr int KP = 32 * DK / 8, VP = 32 * DV / 8;
@@ -542,10 +539,7 @@ static int launch_kv_t(const BwdArgs& a, int key_rows, hipStream_t st) {
 
 template <typename T, int DK, int DV, int MODE>
 static int launch_q_t(const BwdArgs& a, hipStream_t st) {
-#ifndef NSA_Q_NW
-#define NSA_Q_NW 16
-#endif
-  constexpr int NW = NSA_Q_NW;
+  constexpr int NW = kQWaves;
   const size_t smem = 2 * (size_t)(32 * (DK + 8) + 32 * (DV + 8)) * sizeof(T);
   auto fn = bwd_q_kernel<T, DK, DV, MODE, NW>;
   const int rc = set_smem(reinterpret_cast<const void*>(fn), smem);
@@ -601,7 +595,7 @@ static int launch_cmp_bwd_t(const CmpBwdArgs& c, hipStream_t st) {
   if (c.cmp_rows > 0) {
     fill_zero(dk_acc, (long)c.cmp_rows * c.hkv * DK, st);
     fill_zero(dv_acc, (long)c.cmp_rows * c.hkv * DV, st);
-    rc = launch_kv_t<T, DK, DV, kBwdCmp, NSA_KV_NW>(a, c.cmp_rows, st);
+    rc = launch_kv_t<T, DK, DV, kBwdCmp, kKvWaves>(a, c.cmp_rows, st);
     if (rc) return rc;
     cast_out<T>(dk_acc, c.dck, (long)c.cmp_rows * c.hkv * DK, st);
     cast_out<T>(dv_acc, c.dcv, (long)c.cmp_rows * c.hkv * DV, st);
@@ -649,7 +643,7 @@ static int launch_slc_swa_bwd_t(const SlcSwaBwdArgs& c, hipStream_t st) {
     launch_delta<T>(c.o_swa, c.d_o_swa, delta_swa, (long)c.total * c.hq, DV, st);
     a.d_o = c.d_o_swa; a.lse = c.lse_swa; a.delta = delta_swa;
     rc = launch_q_t<T, DK, DV, kBwdSwa>(a, st);
-    if (rc == 0) rc = launch_kv_t<T, DK, DV, kBwdSwa, NSA_KV_NW>(a, c.total, st);
+    if (rc == 0) rc = launch_kv_t<T, DK, DV, kBwdSwa, kKvWaves>(a, c.total, st);
     if (rc) return rc;
   }
   if (slc) {
