@@ -15,8 +15,8 @@
 //    LDS load of gfx950 (ds_read_b64_tr_b16), so no transposed copy of Q or dO exists anywhere.
 //    The three branches differ only in which tokens stream past a key tile: the tokens of a window
 //    (sliding), all later tokens in segments (compressed), the tokens that picked the block
-//    (selected, from the bucketed pair list of the block-major forward).  dK / dV are accumulated
-//    into fp32 buffers with atomics (a key tile is shared by several work items in two of the three).
+//    (selected, from the bucketed pair list of the block-major forward).  dK / dV go to fp32 buffers:
+//    plain stores in the window mode (one work item per key tile), atomics in the other two.
 //    The selected branch also produces dQ here: dS goes through LDS to become a B operand with
 //    lane = query row, and dQ^T = K^T dS^T is written as one partial per (token, pick) pair, summed
 //    per token by slc_dq_merge_kernel.
@@ -306,14 +306,28 @@ bwd_kv_kernel(const BwdArgs a) {
     const long krow = (long)(key_base + keypos) * a.hkv + h;
     float* dkp = a.dk_acc + krow * DK + 4 * g;
     float* dvp = a.dv_acc + krow * DV + 4 * g;
+    if (MODE == kBwdSwa) {
+      // every key row belongs to exactly one workgroup of this mode: plain stores, which also initialise
+      // the accumulators for the selected branch's atomics that follow on the same stream
 #pragma unroll
-    for (int t = 0; t < DK / 16; ++t)
+      for (int t = 0; t < DK / 16; ++t) {
+        f32x4_t v = dk_acc[t];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) unsafeAtomicAdd(dkp + 16 * t + i, dk_acc[t][i] * a.scale);
+        for (int i = 0; i < 4; ++i) v[i] *= a.scale;
+        *reinterpret_cast<f32x4_t*>(dkp + 16 * t) = v;
+      }
 #pragma unroll
-    for (int t = 0; t < DV / 16; ++t)
+      for (int t = 0; t < DV / 16; ++t) *reinterpret_cast<f32x4_t*>(dvp + 16 * t) = dv_acc[t];
+    } else {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) unsafeAtomicAdd(dvp + 16 * t + i, dv_acc[t][i]);
+      for (int t = 0; t < DK / 16; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) unsafeAtomicAdd(dkp + 16 * t + i, dk_acc[t][i] * a.scale);
+#pragma unroll
+      for (int t = 0; t < DV / 16; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) unsafeAtomicAdd(dvp + 16 * t + i, dv_acc[t][i]);
+    }
   }
 }
 
@@ -632,8 +646,10 @@ static int launch_slc_swa_bwd_t(const SlcSwaBwdArgs& c, hipStream_t st) {
   float* dk_acc = (float*)(base + take(off, (long)c.total * c.hkv * DK * 4));
   float* dv_acc = (float*)(base + take(off, (long)c.total * c.hkv * DV * 4));
   const bool slc = c.top_n > 0 && c.d_o_slc != nullptr, swa = c.window > 0 && c.d_o_swa != nullptr;
-  fill_zero(dk_acc, (long)c.total * c.hkv * DK, st);
-  fill_zero(dv_acc, (long)c.total * c.hkv * DV, st);
+  if (!swa) {                      // the window kernel stores every row of the accumulators itself
+    fill_zero(dk_acc, (long)c.total * c.hkv * DK, st);
+    fill_zero(dv_acc, (long)c.total * c.hkv * DV, st);
+  }
   BwdArgs a{};
   a.q = c.q; a.k = c.k; a.v = c.v; a.cu_seq = c.cu_seq; a.cu_key = c.cu_seq; a.batch = c.batch; a.total = c.total;
   a.hq = c.hq; a.hkv = c.hkv; a.causal = 1; a.window = c.window; a.scale = c.scale;
