@@ -6,7 +6,8 @@
 //   rows; the second use hits L2. Algorithmic bytes: rows_in*heads*dim*sizeof(T) read +
 //   rows_out*heads*dim*sizeof(T) written.
 // compress (weighted): out[n][o] = b[o] + sum_{j,i} x[n*stride+j][i] * Wt[o][j*dim+i] as an MFMA
-//   GEMM with the [dim_out x block*dim] weight (L2 resident) as the A operand.
+//   GEMM with the [dim_out x block*dim] weight (L2 resident) as the A operand, split over the taps j
+//   between the wavefronts of a workgroup and summed in LDS.
 // transpose: out[h][d][col] = x[row(col)][h][d], 64-column tiles through LDS.
 #include "common.h"
 #include "kernels.h"
@@ -51,50 +52,72 @@ compress_mean_kernel(const T* __restrict__ x, T* __restrict__ out, const int32_t
   store8(out + (long)r * heads * dim + piece * 8, pack8<T>(acc));
 }
 
+// One workgroup per (32 output rows, head).  The block's taps are dealt to the 4 wavefronts (split-K):
+// each multiplies its taps' weight slices (A operand, straight from L2) with the rows' inputs (B operand,
+// two 16-row groups per weight fragment) and adds its [32 x DIM] partial sum into an fp32 LDS tile, from
+// which whole rows are written with the bias.  4 x the wavefronts of a one-wavefront-per-tile layout:
+// the GEMM is small (Nc x l*D x D) and otherwise leaves most SIMDs idle, waiting on L2 latency.
 template <typename T, int DIM>
 __global__ void __launch_bounds__(256)
 compress_weighted_kernel(const T* __restrict__ x, const T* __restrict__ wt, const T* __restrict__ bias,
                          T* __restrict__ out, const int32_t* __restrict__ cu_seq,
                          const int32_t* __restrict__ cu_out, int batch, int heads, int block, int stride) {
-  const int lane = threadIdx.x & 63;
+  constexpr int NG = 2, LD = DIM + 4;
+  __shared__ float tile[NG * 16 * LD];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n = lane & 15, g = lane >> 4;
-  const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
   const int total_out = cu_out[batch];
-  const int ntile = (total_out + 15) / 16;
-  const int tile = wave / heads, h = wave % heads;
-  if (tile >= ntile) return;
-  const int r = tile * 16 + n;
-  const bool live = r < total_out;
-  const int rc = live ? r : total_out - 1;
-  const int b = upper_seq(cu_out, batch, rc);
-  const T* xrow = x + (((long)cu_seq[b] + (long)(rc - cu_out[b]) * stride) * heads + h) * DIM;
-  f32x4_t acc[DIM / 16];
+  const int r0 = blockIdx.x * NG * 16, h = blockIdx.y;
+  if (r0 >= total_out) return;
+  for (int e = tid; e < NG * 16 * LD; e += 256) tile[e] = 0.f;
+  const T* xrow[NG];
 #pragma unroll
-  for (int i = 0; i < DIM / 16; ++i) acc[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int gi = 0; gi < NG; ++gi) {
+    const int rc = min(r0 + gi * 16 + n, total_out - 1);
+    const int b = upper_seq(cu_out, batch, rc);
+    xrow[gi] = x + (((long)cu_seq[b] + (long)(rc - cu_out[b]) * stride) * heads + h) * DIM + 8 * g;
+  }
+  f32x4_t acc[NG][DIM / 16];
+#pragma unroll
+  for (int gi = 0; gi < NG; ++gi)
+#pragma unroll
+    for (int t = 0; t < DIM / 16; ++t) acc[gi][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   const int K = block * DIM;
-  for (int j = 0; j < block; ++j) {
+  __syncthreads();
+  for (int j = wave; j < block; j += 4) {
+    vec8_t<T> xb[NG][DIM / 32];
 #pragma unroll
-    for (int i0 = 0; i0 < DIM; i0 += 32) {
-      const vec8_t<T> xb = load8(xrow + (long)j * heads * DIM + i0 + 8 * g);
-      const int k0 = j * DIM + i0 + 8 * g;
+    for (int gi = 0; gi < NG; ++gi)
 #pragma unroll
-      for (int t = 0; t < DIM / 16; ++t) {
-        const vec8_t<T> wa = load8(wt + (long)(t * 16 + n) * K + k0);
-        acc[t] = mma16(wa, xb, acc[t]);
+      for (int kk = 0; kk < DIM / 32; ++kk) xb[gi][kk] = load8(xrow[gi] + (long)j * heads * DIM + 32 * kk);
+#pragma unroll
+    for (int t = 0; t < DIM / 16; ++t) {
+      const T* wrow = wt + (long)(t * 16 + n) * K + j * DIM + 8 * g;
+#pragma unroll
+      for (int kk = 0; kk < DIM / 32; ++kk) {
+        const vec8_t<T> wa = load8(wrow + 32 * kk);
+#pragma unroll
+        for (int gi = 0; gi < NG; ++gi) acc[gi][t] = mma16(wa, xb[gi][kk], acc[gi][t]);
       }
     }
   }
-  if (!live) return;
-  T* orow = out + ((long)r * heads + h) * DIM;
 #pragma unroll
-  for (int t = 0; t < DIM / 16; ++t) {
+  for (int gi = 0; gi < NG; ++gi)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int o = t * 16 + 4 * g + i;
-      float v = acc[t][i];
-      if (bias != nullptr) v += (float)bias[o];
-      orow[o] = (T)v;
+    for (int t = 0; t < DIM / 16; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) atomicAdd(&tile[(gi * 16 + n) * LD + 16 * t + 4 * g + i], acc[gi][t][i]);
+  __syncthreads();
+  for (int p = tid; p < NG * 16 * (DIM / 8); p += 256) {
+    const int r = p / (DIM / 8), pc = p % (DIM / 8);
+    if (r0 + r >= total_out) continue;
+    float v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      v[e] = tile[r * LD + pc * 8 + e];
+      if (bias != nullptr) v[e] += (float)bias[pc * 8 + e];
     }
+    store8(out + ((long)(r0 + r) * heads + h) * DIM + pc * 8, pack8<T>(v));
   }
 }
 
@@ -151,10 +174,9 @@ static int launch_compress_t(const CompressArgs& a, hipStream_t st) {
                        a.cu_seq, a.cu_out, a.batch, a.heads, a.dim, a.block, a.stride);
     return 0;
   }
-  const int waves = ((a.out_rows_bound + 15) / 16) * a.heads;
-  const int grid = (waves + 3) / 4;
+  const dim3 grid((a.out_rows_bound + 31) / 32, a.heads);
 #define NSA_WEIGHTED(D)                                                                              \
-  hipLaunchKernelGGL((compress_weighted_kernel<T, D>), dim3(grid), dim3(256), 0, st, (const T*)a.x, \
+  hipLaunchKernelGGL((compress_weighted_kernel<T, D>), grid, dim3(256), 0, st, (const T*)a.x, \
                      (const T*)a.wt, (const T*)a.bias, (T*)a.out, a.cu_seq, a.cu_out, a.batch,      \
                      a.heads, a.block, a.stride)
   switch (a.dim) {
