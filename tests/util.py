@@ -20,7 +20,7 @@ def make_qkv(T, Hq, Hkv, Dk, Dv, seed, dtype, scale=1.0):
 
 
 def max_abs(a, b):
-    return float((a.double().cpu() - b.double().cpu()).abs().max()) if a.numel() else 0.0
+    return float((a.detach().double().cpu() - b.detach().double().cpu()).abs().max()) if a.numel() else 0.0
 
 
 def ragged_cu(lens):
