@@ -135,12 +135,15 @@ int nsa_gate_bwd(const void* q, const void* weight, const void* d_gates, void* d
  *   gate_logits [rows, 3] (selected, sliding, compressed), pre-activation; o_* [rows, dv] (o_swa,
  *   o_cmp may be NULL: term dropped);  out = sum_b act(gate_b) * o_b.
  *   backward: d_b = act(gate_b) * d_out for every branch given, d_gate_logits[row][b] =
- *   act'(gate_b) * <d_out[row], o_b[row]> (0 for a missing branch). */
+ *   act'(gate_b) * <d_out[row], o_b[row]> (0 for a missing branch).  stats (optional, float [6][rows])
+ *   receives <d_out[row], o_b[row]> for b = selected, sliding, compressed and then act(gate_b): the
+ *   delta / rowscale inputs of the attention backward entry points; with stats given the scaled copies
+ *   d_slc / d_swa / d_cmp may be NULL (not written). */
 int nsa_gate_combine_fwd(const void* gate_logits, const void* o_slc, const void* o_swa, const void* o_cmp, void* out,
                          int64_t rows, int dv, int gate_act, int dtype, nsa_stream_t stream);
 int nsa_gate_combine_bwd(const void* gate_logits, const void* d_out, const void* o_slc, const void* o_swa,
-                         const void* o_cmp, void* d_slc, void* d_swa, void* d_cmp, void* d_gate_logits, int64_t rows,
-                         int dv, int gate_act, int dtype, nsa_stream_t stream);
+                         const void* o_cmp, void* d_slc, void* d_swa, void* d_cmp, void* d_gate_logits, float* stats,
+                         int64_t rows, int dv, int gate_act, int dtype, nsa_stream_t stream);
 
 /* Sliding window attention: token t attends keys [max(0, t-window+1), t] of its sequence.  Replaces
  * the window loop of nsa/selection_attn.py:483-517.  q [total,hq,dk], k [total,hkv,dk],
@@ -204,10 +207,14 @@ int64_t nsa_slc_workspace_bytes(int total, int batch, int hkv, int dk, int dv, i
  *   kv head, not repeated per q head), o / d_o [total,hq,dv] the forward output and its gradient,
  *   lse = lse_attn of nsa_cmp_attn_fwd.  Outputs dq [total,hq,dk], dck, dcv (shapes of ck, cv), all
  *   fully overwritten.  The block selection has no gradient (indices are integers).
+ *   delta (optional, float [total,hq]): rowsum(o * d_o) when the caller already has it (o may then be
+ *   NULL);  rowscale (optional, float [total,hq]): a per-row gate g — the results are those for the output
+ *   gradient g * d_o with delta = rowsum(o * d_o) still the unscaled sum, so a gated sum of branches
+ *   needs no scaled copy of d_o (nsa_gate_combine_bwd writes both arrays).
  *   workspace: nsa_cmp_attn_bwd_workspace_bytes, caller allocated. */
 int64_t nsa_cmp_attn_bwd_workspace_bytes(int total, int cmp_rows, int hq, int hkv, int dk, int dv);
 int nsa_cmp_attn_bwd(const void* q, const void* ck, const void* cv, const void* o, const void* d_o, const float* lse,
-                     const int32_t* cu_seqlens, const int32_t* cu_cmp, int batch, int total, int cmp_rows, int hq,
+                     const float* delta, const float* rowscale, const int32_t* cu_seqlens, const int32_t* cu_cmp, int batch, int total, int cmp_rows, int hq,
                      int hkv, int dk, int dv, int block, int stride, float scale, int causal, int dtype, void* dq,
                      void* dck, void* dcv, void* workspace, int64_t workspace_bytes, nsa_stream_t stream);
 
@@ -220,13 +227,16 @@ int nsa_cmp_attn_bwd(const void* q, const void* ck, const void* cv, const void* 
  *   A branch is skipped when its d_o is NULL.  indices / counts / idx64 / top_n / block_size as in
  *   nsa_slc_combine_fwd (64-key blocks only).  dq [total,hq,dk], dk_out [total,hkv,dk], dv_out
  *   [total,hkv,dv] receive the sums over the branches present and are fully overwritten.
+ *   delta_* / rowscale_* (optional, float [total,hq]) as in nsa_cmp_attn_bwd, per branch.
  *   workspace: nsa_slc_swa_bwd_workspace_bytes (pass top_n = 0 there when the selected branch is
  *   skipped). */
 int64_t nsa_slc_swa_bwd_workspace_bytes(int total, int batch, int hq, int hkv, int dk, int dv, int top_n,
                                         int block_size, int dtype);
 int nsa_slc_swa_bwd(const void* q, const void* k, const void* v, const void* o_slc, const void* o_swa,
                     const void* d_o_slc, const void* d_o_swa, const float* lse_slc, const float* lse_swa,
-                    const void* indices, const int32_t* counts, const int32_t* cu_seqlens, int batch, int total, int hq,
+                    const float* delta_slc, const float* delta_swa, const float* rowscale_slc,
+                    const float* rowscale_swa, const void* indices, const int32_t* counts,
+                    const int32_t* cu_seqlens, int batch, int total, int hq,
                     int hkv, int dk, int dv, int top_n, int block_size, int window, float scale, int idx64, int dtype,
                     void* dq, void* dk_out, void* dv_out, void* workspace, int64_t workspace_bytes,
                     nsa_stream_t stream);

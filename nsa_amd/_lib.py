@@ -33,7 +33,7 @@ SIGNATURES = {
     "nsa_gate_fwd": (_I, [_P, _P, _P, _P, _L, _I, _I, _P]),
     "nsa_gate_bwd": (_I, [_P] * 6 + [_L, _I, _I, _P]),
     "nsa_gate_combine_fwd": (_I, [_P] * 5 + [_L, _I, _I, _I, _P]),
-    "nsa_gate_combine_bwd": (_I, [_P] * 9 + [_L, _I, _I, _I, _P]),
+    "nsa_gate_combine_bwd": (_I, [_P] * 10 + [_L, _I, _I, _I, _P]),
     "nsa_swa_fwd": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P]),
     "nsa_slc_combine_fwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I,
                                  _I, _I, _I, _I, _F, _I, _I, _I, _P, _L, _P]),
@@ -41,9 +41,9 @@ SIGNATURES = {
     "nsa_slc_partials_fwd": (_I, [_P] * 6 + [_I] * 9 + [_F, _I, _I, _P, _L, _P]),
     "nsa_swa_merge_fwd": (_I, [_P] * 6 + [_L, _P, _P, _P] + [_I] * 10 + [_F, _I, _I, _P, _L, _P]),
     "nsa_cmp_attn_bwd_workspace_bytes": (_L, [_I] * 6),
-    "nsa_cmp_attn_bwd": (_I, [_P] * 8 + [_I] * 9 + [_F, _I, _I, _P, _P, _P, _P, _L, _P]),
+    "nsa_cmp_attn_bwd": (_I, [_P] * 10 + [_I] * 9 + [_F, _I, _I, _P, _P, _P, _P, _L, _P]),
     "nsa_slc_swa_bwd_workspace_bytes": (_L, [_I] * 9),
-    "nsa_slc_swa_bwd": (_I, [_P] * 12 + [_I] * 9 + [_F, _I, _I, _P, _P, _P, _P, _L, _P]),
+    "nsa_slc_swa_bwd": (_I, [_P] * 16 + [_I] * 9 + [_F, _I, _I, _P, _P, _P, _P, _L, _P]),
     "nsa_decode_max_compressed": (_I, []),
     "nsa_decode_step": (_I, [_P] * 9 + [_I] * 15 + [_F, _I, _I, _P]),
     "nsa_decode_append": (_I, [_P] * 7 + [_I] * 9 + [_P]),

@@ -134,3 +134,50 @@ class GateCombineFn(torch.autograd.Function):
         gate_logits, o_slc, o_swa, o_cmp = ctx.saved_tensors
         d_slc, d_swa, d_cmp, d_gl = ops.gate_combine_bwd(gate_logits, d_out, o_slc, o_swa, o_cmp, ctx.gate_act)
         return d_gl.to(gate_logits.dtype), d_slc, d_swa, d_cmp, None
+
+
+class NSACoreFn(torch.autograd.Function):
+    """The three branches and their gated sum as one node (what NSAAttention's training path runs):
+    q [total,Hq,Dk], ck / cv [rows,Hkv,D] packed over cu_cmp, k / v [total,Hkv,D], gate_logits
+    [total,Hq,3] -> (out [total,Hq,Dv], indices int32 [total,Hkv,S]).  One node lets the backward hand
+    the gates to the attention kernels as per-row scales together with the unscaled row sums
+    <d_out, o_b>, so neither scaled copies of d_out nor separate row-sum passes are needed."""
+
+    @staticmethod
+    def forward(ctx, q, ck, cv, k, v, gate_logits, cu, cu_cmp, batch, block, stride, sel_block, window, scale,
+                causal, select, gate_act):
+        q, ck, cv, k, v = (t.contiguous() for t in (q, ck, cv, k, v))
+        hkv, dk, dv = ck.shape[1], ck.shape[2], cv.shape[2]
+        cvt, vt = ops.transpose(cv, cu_cmp, batch), ops.transpose(v, cu, batch)
+        o_cmp, lse_raw, lse_cmp = ops.cmp_attn(q, ck, cvt, cu, cu_cmp, batch, hkv, dv, hkv * dk, dk, block, stride,
+                                               scale, causal=causal, want_lse_attn=True)
+        pk, ps, pp, top_n, max_nc = select
+        idx, _ = ops.block_select(q, ck, lse_raw, cu, cu_cmp, batch, hkv, hkv * dk, dk, pk, ps, pp, top_n, max_nc,
+                                  idx64=False)
+        o_slc, lse_slc = ops.slc_combine(q, k, vt, idx, None, None, None, None, None, None, cu, batch, sel_block,
+                                         scale, block_major=True, want_lse=True)
+        o_swa = lse_swa = None
+        if window > 0:
+            o_swa, lse_swa = ops.swa(q, k, vt, cu, batch, window, scale, want_lse=True)
+        out = ops.gate_combine(gate_logits, o_slc, o_swa, o_cmp, gate_act)
+        ctx.save_for_backward(q, ck, cv, k, v, gate_logits, o_cmp, lse_cmp, o_slc, lse_slc, o_swa, lse_swa, idx, cu,
+                              cu_cmp)
+        ctx.geom = (batch, block, stride, sel_block, window, scale, causal, gate_act)
+        ctx.mark_non_differentiable(idx)
+        return out, idx
+
+    @staticmethod
+    def backward(ctx, d_out, _d_idx=None):
+        q, ck, cv, k, v, gate_logits, o_cmp, lse_cmp, o_slc, lse_slc, o_swa, lse_swa, idx, cu, cu_cmp = \
+            ctx.saved_tensors
+        batch, block, stride, sel_block, window, scale, causal, gate_act = ctx.geom
+        d_out = d_out.contiguous()
+        _, _, _, d_gl, st = ops.gate_combine_bwd(gate_logits, d_out, o_slc, o_swa, o_cmp, gate_act, want_scaled=False,
+                                                 want_stats=True)
+        dq_c, dck, dcv = ops.cmp_attn_bwd(q, ck, cv, None, d_out, lse_cmp, cu, cu_cmp, batch, block, stride, scale,
+                                          causal=causal, delta=st[2], rowscale=st[5])
+        dq, dk, dv = ops.slc_swa_bwd(q, k, v, None, d_out, lse_slc, None, d_out if o_swa is not None else None,
+                                     lse_swa, idx, None, cu, batch, sel_block, window, scale, delta_slc=st[0],
+                                     delta_swa=st[1], rowscale_slc=st[3], rowscale_swa=st[4])
+        dq += dq_c
+        return (dq, dck, dcv, dk, dv, d_gl.to(gate_logits.dtype)) + (None,) * 11

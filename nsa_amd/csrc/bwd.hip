@@ -40,6 +40,8 @@ constexpr int kSegGroup = 4;         // selected branch: consecutive 64-pair seg
 
 struct BwdArgs {
   const void* q; const void* d_o; const float* lse; const float* delta;    // rows: [total][hq][.]
+  const float* rowscale;          // optional [total][hq]: the branch's gate g; folded into the row statistics
+                                  // (lse - ln|g| scales P and dS, sign(g) flips delta and the dO rows)
   const void* k; const void* v;                                          // keys: [key rows][hkv][.]
   const int32_t* cu_seq; const int32_t* cu_key;
   int batch, total, hq, hkv;
@@ -185,7 +187,9 @@ bwd_kv_kernel(const BwdArgs a) {
 
   // ---- staging of one chunk: global -> registers -> LDS
   vec8_t<T> qr[QPT], orr[OPT];
-  float sr = 0.f;
+  float ors[OPT], sr = 0.f, srs = 1.f;       // the gates of the staged rows (1 without a.rowscale)
+#pragma unroll
+  for (int i = 0; i < OPT; ++i) ors[i] = 1.f;
   auto gload = [&](int c) {
     int posA, posB; bool vB;
     chunk_tokens(c, posA, posB, vB);
@@ -204,14 +208,17 @@ bwd_kv_kernel(const BwdArgs a) {
       if (OP % NT == 0 || p < OP) {
         const int r = p / (DV / 8), pc = p % (DV / 8);
         const long tg = seq_start + ((r >> 4) ? posB : posA);
-        orr[i] = load8(dob + (tg * a.hq + h * G + min(r & 15, G - 1)) * DV + pc * 8);
+        const long row = tg * a.hq + h * G + min(r & 15, G - 1);
+        orr[i] = load8(dob + row * DV + pc * 8);
+        if (a.rowscale != nullptr) ors[i] = a.rowscale[row];       // used in lstore: nothing here waits for a load
       }
     }
     if (tid < 64) {
       const int r = tid & 31;
       const long tg = seq_start + ((r >> 4) ? posB : posA);
       const long row = tg * a.hq + h * G + min(r & 15, G - 1);
-      sr = tid < 32 ? a.lse[row] * kLog2e : a.delta[row];
+      sr = tid < 32 ? a.lse[row] : a.delta[row];
+      if (a.rowscale != nullptr) srs = a.rowscale[row];
     }
   };
   auto lstore = [&](int buf) {
@@ -225,9 +232,12 @@ bwd_kv_kernel(const BwdArgs a) {
 #pragma unroll
     for (int i = 0; i < OPT; ++i) {
       const int p = tid + i * NT;
-      if (OP % NT == 0 || p < OP) store8(os + (p / (DV / 8)) * OLD + (p % (DV / 8)) * 8, orr[i]);
+      if (OP % NT == 0 || p < OP)
+        store8(os + (p / (DV / 8)) * OLD + (p % (DV / 8)) * 8, ors[i] < 0.f ? -orr[i] : orr[i]);
     }
-    if (tid < 64) stat[buf * 64 + tid] = sr;
+    // fold the gate g of a row: lse - ln|g| scales P and dS, sign(g) flips delta and (above) the dO row
+    if (tid < 32) stat[buf * 64 + tid] = sr * kLog2e - __log2f(fabsf(srs));
+    else if (tid < 64) stat[buf * 64 + tid] = srs < 0.f ? -sr : sr;
   };
 
   const float c_attn = a.scale * kLog2e;
@@ -382,6 +392,15 @@ bwd_q_kernel(const BwdArgs a) {
     for (int kk = 0; kk < DV / 32; ++kk) dof[kk] = load8(dp + 32 * kk);
     lse2 = a.lse[row] * kLog2e;
     dl = a.delta[row];
+    if (a.rowscale != nullptr) {            // fold the gate as in the key-stationary kernel
+      const float rs = a.rowscale[row];
+      lse2 -= __log2f(fabsf(rs));
+      if (rs < 0.f) {
+        dl = -dl;
+#pragma unroll
+        for (int kk = 0; kk < DV / 32; ++kk) dof[kk] = -dof[kk];
+      }
+    }
   }
   f32x4_t acc[DK / 16];
 #pragma unroll
@@ -598,9 +617,10 @@ static int launch_cmp_bwd_t(const CmpBwdArgs& c, hipStream_t st) {
   float* delta = (float*)(base + take(off, (long)c.total * c.hq * 4));
   float* dk_acc = (float*)(base + take(off, (long)c.cmp_rows * c.hkv * DK * 4));
   float* dv_acc = (float*)(base + take(off, (long)c.cmp_rows * c.hkv * DV * 4));
-  launch_delta<T>(c.o, c.d_o, delta, (long)c.total * c.hq, DV, st);
+  if (c.delta == nullptr) launch_delta<T>(c.o, c.d_o, delta, (long)c.total * c.hq, DV, st);
   BwdArgs a{};
-  a.q = c.q; a.d_o = c.d_o; a.lse = c.lse; a.delta = delta; a.k = c.ck; a.v = c.cv;
+  a.q = c.q; a.d_o = c.d_o; a.lse = c.lse; a.delta = c.delta ? c.delta : delta; a.rowscale = c.rowscale;
+  a.k = c.ck; a.v = c.cv;
   a.cu_seq = c.cu_seq; a.cu_key = c.cu_cmp; a.batch = c.batch; a.total = c.total; a.hq = c.hq; a.hkv = c.hkv;
   a.block = c.block; a.stride = c.stride; a.causal = c.causal; a.window = 0; a.scale = c.scale;
   a.dq = c.dq; a.dk_acc = dk_acc; a.dv_acc = dv_acc;
@@ -656,8 +676,9 @@ static int launch_slc_swa_bwd_t(const SlcSwaBwdArgs& c, hipStream_t st) {
   a.dq = c.dq; a.dk_acc = dk_acc; a.dv_acc = dv_acc;
   int rc = 0;
   if (swa) {
-    launch_delta<T>(c.o_swa, c.d_o_swa, delta_swa, (long)c.total * c.hq, DV, st);
-    a.d_o = c.d_o_swa; a.lse = c.lse_swa; a.delta = delta_swa;
+    if (c.delta_swa == nullptr) launch_delta<T>(c.o_swa, c.d_o_swa, delta_swa, (long)c.total * c.hq, DV, st);
+    a.d_o = c.d_o_swa; a.lse = c.lse_swa; a.delta = c.delta_swa ? c.delta_swa : delta_swa;
+    a.rowscale = c.rowscale_swa;
     rc = launch_q_t<T, DK, DV, kBwdSwa>(a, st);
     if (rc == 0) rc = launch_kv_t<T, DK, DV, kBwdSwa, kKvWaves>(a, c.total, st);
     if (rc) return rc;
@@ -668,8 +689,9 @@ static int launch_slc_swa_bwd_t(const SlcSwaBwdArgs& c, hipStream_t st) {
     slc_carve(s, base + off, &ws, sizeof(T), DK);
     rc = launch_slc_bucket(s, ws, st);
     if (rc) return rc;
-    launch_delta<T>(c.o_slc, c.d_o_slc, delta_slc, (long)c.total * c.hq, DV, st);
-    a.d_o = c.d_o_slc; a.lse = c.lse_slc; a.delta = delta_slc; a.ws = ws;
+    if (c.delta_slc == nullptr) launch_delta<T>(c.o_slc, c.d_o_slc, delta_slc, (long)c.total * c.hq, DV, st);
+    a.d_o = c.d_o_slc; a.lse = c.lse_slc; a.delta = c.delta_slc ? c.delta_slc : delta_slc;
+    a.rowscale = c.rowscale_slc; a.ws = ws;
     rc = launch_kv_t<T, DK, DV, kBwdSlc, 4>(a, c.total, st);
     if (rc) return rc;
     const long threads = (long)c.total * c.hq * (DK / 8);

@@ -196,17 +196,18 @@ int nsa_gate_combine_fwd(const void* gate_logits, const void* o_slc, const void*
                          int64_t rows, int dv, int gate_act, int dtype, nsa_stream_t stream) {
   if (!out) return fail(NSA_ERR_INVALID, "gate_combine: null pointer");
   nsa::GateCombineArgs a{gate_logits, o_slc, o_swa, o_cmp, out, nullptr, nullptr, nullptr, nullptr, nullptr,
-                         (long)rows, dv, gate_act, dtype};
+                         (long)rows, dv, gate_act, dtype, nullptr};
   return gate_combine_common("gate_combine", a, stream);
 }
 
 int nsa_gate_combine_bwd(const void* gate_logits, const void* d_out, const void* o_slc, const void* o_swa,
-                         const void* o_cmp, void* d_slc, void* d_swa, void* d_cmp, void* d_gate_logits, int64_t rows,
-                         int dv, int gate_act, int dtype, nsa_stream_t stream) {
-  if (!d_out || !d_slc || !d_gate_logits || (o_swa && !d_swa) || (o_cmp && !d_cmp))
-    return fail(NSA_ERR_INVALID, "gate_combine_bwd: null pointer");
+                         const void* o_cmp, void* d_slc, void* d_swa, void* d_cmp, void* d_gate_logits, float* stats,
+                         int64_t rows, int dv, int gate_act, int dtype, nsa_stream_t stream) {
+  if (!d_out || !d_gate_logits) return fail(NSA_ERR_INVALID, "gate_combine_bwd: null pointer");
+  if (!stats && (!d_slc || (o_swa && !d_swa) || (o_cmp && !d_cmp)))
+    return fail(NSA_ERR_INVALID, "gate_combine_bwd: null pointer (every branch given needs its gradient buffer unless stats is requested)");
   nsa::GateCombineArgs a{gate_logits, o_slc, o_swa, o_cmp, nullptr, d_out, d_slc, d_swa, d_cmp, d_gate_logits,
-                         (long)rows, dv, gate_act, dtype};
+                         (long)rows, dv, gate_act, dtype, stats};
   return gate_combine_common("gate_combine_bwd", a, stream);
 }
 
@@ -314,10 +315,10 @@ int64_t nsa_cmp_attn_bwd_workspace_bytes(int total, int cmp_rows, int hq, int hk
 }
 
 int nsa_cmp_attn_bwd(const void* q, const void* ck, const void* cv, const void* o, const void* d_o, const float* lse,
-                     const int32_t* cu_seqlens, const int32_t* cu_cmp, int batch, int total, int cmp_rows, int hq,
+                     const float* delta, const float* rowscale, const int32_t* cu_seqlens, const int32_t* cu_cmp, int batch, int total, int cmp_rows, int hq,
                      int hkv, int dk, int dv, int block, int stride, float scale, int causal, int dtype, void* dq,
                      void* dck, void* dcv, void* workspace, int64_t workspace_bytes, nsa_stream_t stream) {
-  if (!q || !o || !d_o || !lse || !cu_seqlens || !cu_cmp || !dq || !workspace)
+  if (!q || (!o && !delta) || !d_o || !lse || !cu_seqlens || !cu_cmp || !dq || !workspace)
     return fail(NSA_ERR_INVALID, "cmp_attn_bwd: null pointer");
   if (cmp_rows > 0 && (!ck || !cv || !dck || !dcv)) return fail(NSA_ERR_INVALID, "cmp_attn_bwd: null pointer");
   if (batch <= 0 || total <= 0 || cmp_rows < 0 || block <= 0 || stride <= 0)
@@ -325,13 +326,13 @@ int nsa_cmp_attn_bwd(const void* q, const void* ck, const void* cv, const void* 
   if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "cmp_attn_bwd: bad dtype");
   if (int rc = check_heads("cmp_attn_bwd", hq, hkv, dk, dv)) return rc;
   if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "cmp_attn_bwd: scale must be positive");
-  if (!aligned16(q) || !aligned16(ck) || !aligned16(cv) || !aligned16(o) || !aligned16(d_o) || !aligned16(dq) ||
+  if (!aligned16(q) || !aligned16(ck) || !aligned16(cv) || (o && !aligned16(o)) || !aligned16(d_o) || !aligned16(dq) ||
       !aligned16(dck) || !aligned16(dcv) || !aligned16(workspace))
     return fail(NSA_ERR_INVALID, "cmp_attn_bwd: pointers must be 16-byte aligned");
   if (workspace_bytes < nsa_cmp_attn_bwd_workspace_bytes(total, cmp_rows, hq, hkv, dk, dv))
     return fail(NSA_ERR_INVALID, "cmp_attn_bwd: workspace smaller than nsa_cmp_attn_bwd_workspace_bytes");
   nsa::CmpBwdArgs a{q, ck, cv, o, d_o, lse, cu_seqlens, cu_cmp, batch, total, cmp_rows, hq, hkv, dk, dv, block, stride,
-                    causal, scale, dtype, dq, dck, dcv, workspace};
+                    causal, scale, dtype, dq, dck, dcv, workspace, delta, rowscale};
   const int rc = nsa::launch_cmp_bwd(a, stream);
   if (rc == -2) return fail(NSA_ERR_UNSUPPORTED, "cmp_attn_bwd: head dims not built (dk,dv in (64,64),(128,128),(192,128); fp32: no 192)");
   return finish(rc, "cmp_attn_bwd");
@@ -348,15 +349,17 @@ int64_t nsa_slc_swa_bwd_workspace_bytes(int total, int batch, int hq, int hkv, i
 
 int nsa_slc_swa_bwd(const void* q, const void* k, const void* v, const void* o_slc, const void* o_swa,
                     const void* d_o_slc, const void* d_o_swa, const float* lse_slc, const float* lse_swa,
-                    const void* indices, const int32_t* counts, const int32_t* cu_seqlens, int batch, int total, int hq,
+                    const float* delta_slc, const float* delta_swa, const float* rowscale_slc,
+                    const float* rowscale_swa, const void* indices, const int32_t* counts,
+                    const int32_t* cu_seqlens, int batch, int total, int hq,
                     int hkv, int dk, int dv, int top_n, int block_size, int window, float scale, int idx64, int dtype,
                     void* dq, void* dk_out, void* dv_out, void* workspace, int64_t workspace_bytes,
                     nsa_stream_t stream) {
   if (!q || !k || !v || !cu_seqlens || !dq || !dk_out || !dv_out || !workspace)
     return fail(NSA_ERR_INVALID, "slc_swa_bwd: null pointer");
   const bool slc = d_o_slc != nullptr, swa = d_o_swa != nullptr;
-  if (slc && (!o_slc || !lse_slc || !indices || top_n <= 0)) return fail(NSA_ERR_INVALID, "slc_swa_bwd: the selected branch needs o_slc, lse_slc, indices and top_n > 0");
-  if (swa && (!o_swa || !lse_swa || window <= 0)) return fail(NSA_ERR_INVALID, "slc_swa_bwd: the sliding branch needs o_swa, lse_swa and window > 0");
+  if (slc && ((!o_slc && !delta_slc) || !lse_slc || !indices || top_n <= 0)) return fail(NSA_ERR_INVALID, "slc_swa_bwd: the selected branch needs o_slc, lse_slc, indices and top_n > 0");
+  if (swa && ((!o_swa && !delta_swa) || !lse_swa || window <= 0)) return fail(NSA_ERR_INVALID, "slc_swa_bwd: the sliding branch needs o_swa, lse_swa and window > 0");
   if (batch <= 0 || total <= 0) return fail(NSA_ERR_INVALID, "slc_swa_bwd: sizes must be positive");
   if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "slc_swa_bwd: bad dtype");
   if (int rc = check_heads("slc_swa_bwd", hq, hkv, dk, dv)) return rc;
@@ -364,14 +367,14 @@ int nsa_slc_swa_bwd(const void* q, const void* k, const void* v, const void* o_s
   if (slc && (block_size != 64 || top_n > 64 || total >= (1 << 26)))
     return fail(NSA_ERR_UNSUPPORTED, "slc_swa_bwd: the selected branch is built for 64-key blocks, top_n <= 64");
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(dq) || !aligned16(dk_out) || !aligned16(dv_out) ||
-      !aligned16(workspace) || (slc && (!aligned16(o_slc) || !aligned16(d_o_slc))) ||
-      (swa && (!aligned16(o_swa) || !aligned16(d_o_swa))))
+      !aligned16(workspace) || (slc && ((o_slc && !aligned16(o_slc)) || !aligned16(d_o_slc))) ||
+      (swa && ((o_swa && !aligned16(o_swa)) || !aligned16(d_o_swa))))
     return fail(NSA_ERR_INVALID, "slc_swa_bwd: pointers must be 16-byte aligned");
   if (workspace_bytes < nsa_slc_swa_bwd_workspace_bytes(total, batch, hq, hkv, dk, dv, slc ? top_n : 0, block_size, dtype))
     return fail(NSA_ERR_INVALID, "slc_swa_bwd: workspace smaller than nsa_slc_swa_bwd_workspace_bytes");
   nsa::SlcSwaBwdArgs a{q, k, v, o_slc, o_swa, d_o_slc, d_o_swa, lse_slc, lse_swa, indices, counts, cu_seqlens, batch,
                        total, hq, hkv, dk, dv, slc ? top_n : 0, block_size, swa ? window : 0, scale, idx64, dtype, dq,
-                       dk_out, dv_out, workspace};
+                       dk_out, dv_out, workspace, delta_slc, delta_swa, rowscale_slc, rowscale_swa};
   const int rc = nsa::launch_slc_swa_bwd(a, stream);
   if (rc == -2) return fail(NSA_ERR_UNSUPPORTED, "slc_swa_bwd: head dims not built (dk,dv in (64,64),(128,128),(192,128); fp32: no 192)");
   return finish(rc, "slc_swa_bwd");

@@ -1,7 +1,9 @@
 // Gated sum of the three branches as stand-alone kernels, and the backward of the gates, for the
 // training path (the inference path folds the sum into the attention epilogues).
 //   forward   out = act(x_slc) o_slc + act(x_swa) o_swa + act(x_cmp) o_cmp      (nsa/nsa.py:117-133)
-//   backward  d_o_b = act(x_b) d_out,  d_x_b = act'(x_b) <d_out, o_b>
+//   backward  d_o_b = act(x_b) d_out,  d_x_b = act'(x_b) <d_out, o_b>;  on request the row sums <d_out, o_b> and
+//             the gates act(x_b) are written out instead of (or next to) the scaled copies d_o_b, for attention
+//             backward kernels that take d_out itself plus a per-row scale
 //   gating Linear x = W q + b (nsa/nsa.py:61,117):  dq = d_x W,  dW = d_x^T q,  db = sum d_x
 // All three are HBM streaming kernels: every operand is read once, 16 lanes share one (token, head) row.
 #include "common.h"
@@ -39,8 +41,8 @@ template <typename T>
 __global__ void __launch_bounds__(256)
 gate_combine_bwd_kernel(const T* __restrict__ gl, const T* __restrict__ d_out, const T* __restrict__ o_slc,
                         const T* __restrict__ o_swa, const T* __restrict__ o_cmp, T* __restrict__ d_slc,
-                        T* __restrict__ d_swa, T* __restrict__ d_cmp, T* __restrict__ d_gl, long rows, int dv,
-                        int act) {
+                        T* __restrict__ d_swa, T* __restrict__ d_cmp, T* __restrict__ d_gl, float* __restrict__ stats,
+                        long rows, int dv, int act) {
   const long row = ((long)blockIdx.x * 256 + threadIdx.x) >> 4;
   const int sub = threadIdx.x & 15;
   const bool live = row < rows;
@@ -65,7 +67,7 @@ gate_combine_bwd_kernel(const T* __restrict__ gl, const T* __restrict__ d_out, c
           dot[b] = fmaf((float)d[e], (float)o[e], dot[b]);
           s[e] = g[b] * (float)d[e];
         }
-        store8(grad[b] + row * dv + c, pack8<T>(s));
+        if (grad[b] != nullptr) store8(grad[b] + row * dv + c, pack8<T>(s));
       }
     }
   }
@@ -77,6 +79,10 @@ gate_combine_bwd_kernel(const T* __restrict__ gl, const T* __restrict__ d_out, c
     const float dg = sub == 0 ? dot[0] : (sub == 1 ? dot[1] : dot[2]);
     const float gg = sub == 0 ? g[0] : (sub == 1 ? g[1] : g[2]);
     d_gl[row * 3 + sub] = (T)(act == 1 ? dg * gg * (1.0f - gg) : dg);
+    if (stats != nullptr) {
+      stats[(long)sub * rows + row] = dg;
+      stats[(long)(3 + sub) * rows + row] = gg;
+    }
   }
 }
 
@@ -164,7 +170,7 @@ static int gate_combine_t(const GateCombineArgs& a, hipStream_t st) {
   } else {
     hipLaunchKernelGGL((gate_combine_bwd_kernel<T>), dim3((unsigned)((a.rows * 16 + 255) / 256)), dim3(256), 0, st,
                        gl, (const T*)a.d_out, (const T*)a.o_slc, (const T*)a.o_swa, (const T*)a.o_cmp, (T*)a.d_slc,
-                       (T*)a.d_swa, (T*)a.d_cmp, (T*)a.d_gate_logits, a.rows, a.dv, a.act);
+                       (T*)a.d_swa, (T*)a.d_cmp, (T*)a.d_gate_logits, a.stats, a.rows, a.dv, a.act);
   }
   return 0;
 }

@@ -67,6 +67,9 @@ struct CmpBwdArgs {
   const int32_t* cu_seq; const int32_t* cu_cmp;
   int batch, total, cmp_rows, hq, hkv, dk, dv, block, stride, causal; float scale; int dtype;
   void* dq; void* dck; void* dcv; void* workspace;
+  // optional: delta = rowsum(o * d_o) computed by the caller (o may then be null), and a per-row gate:
+  // the gradients are those for d_o scaled by rowscale[row], with delta the unscaled row sum
+  const float* delta; const float* rowscale;
 };
 
 // Backward of the selected and sliding branches (either may be absent: top_n == 0 / d_o_slc null,
@@ -78,6 +81,7 @@ struct SlcSwaBwdArgs {
   const void* indices; const int32_t* counts; const int32_t* cu_seq;
   int batch, total, hq, hkv, dk, dv, top_n, block_size, window; float scale; int idx64, dtype;
   void* dq; void* dk_out; void* dv_out; void* workspace;
+  const float* delta_slc; const float* delta_swa; const float* rowscale_slc; const float* rowscale_swa;   // as above
 };
 
 // Gated sum of the branches (d_out == nullptr: forward into out) or its backward (d_out given:
@@ -87,6 +91,7 @@ struct GateCombineArgs {
   const void* gate_logits; const void* o_slc; const void* o_swa; const void* o_cmp; void* out;
   const void* d_out; void* d_slc; void* d_swa; void* d_cmp; void* d_gate_logits;
   long rows; int dv, act, dtype;
+  float* stats;      // optional (backward): [6][rows] = <d_out, o_b> for b = slc, swa, cmp, then act(gate_b)
 };
 
 struct DecodeArgs {

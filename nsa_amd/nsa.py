@@ -8,7 +8,7 @@ import torch
 from torch import nn
 
 from . import _lib, ops
-from .autograd import CmpAttnFn, GateCombineFn, GateLinearFn, SlcSwaFn, needs_grad
+from .autograd import GateLinearFn, NSACoreFn, needs_grad
 from .compression_kv import KVCompressor, conv_compressed_len
 
 
@@ -111,15 +111,13 @@ class NSAAttention(nn.Module):
         ck, cv, cu_cmp, nc = self.compressor.compress_packed(k, v, cu, seq_len=seq_len if uniform else None)
         max_nc = nc if nc is not None else conv_compressed_len(seq_len, self.compression_stride,
                                                                self.compression_block)
-        sel = (self.pool_kernel_size, self.pool_stride, self.pool_padding, self.selected_block_count, max_nc, False)
-        o_cmp, idx = CmpAttnFn.apply(q, ck, cv, cu, cu_cmp, batch, self.compression_block,
-                                     self.compression_stride, float(scale), causal, sel)
-        o_slc, o_swa = SlcSwaFn.apply(q, k, v, idx, None, cu, batch, self.selection_block_size,
-                                      self.sliding_window, float(scale))
+        sel = (self.pool_kernel_size, self.pool_stride, self.pool_padding, self.selected_block_count, max_nc)
         if gates is None:
             gates = GateLinearFn.apply(q, self.gating.weight, self.gating.bias)
         act = _lib.GATE_SIGMOID if self.gate_activation == "sigmoid" else _lib.GATE_IDENTITY
-        out = GateCombineFn.apply(gates, o_slc, o_swa, o_cmp, act)
+        out, idx = NSACoreFn.apply(q, ck, cv, k, v, gates, cu, cu_cmp, batch, self.compression_block,
+                                   self.compression_stride, self.selection_block_size, self.sliding_window,
+                                   float(scale), causal, sel, act)
         if return_indices:
             return out, idx
         return out

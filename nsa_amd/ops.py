@@ -309,20 +309,23 @@ def gate_logits(q, weight, bias=None):
     return out
 
 
-def cmp_attn_bwd(q, ck, cv, o, d_o, lse_attn, cu_seqlens, cu_cmp, batch, block, stride, scale, causal=True):
+def cmp_attn_bwd(q, ck, cv, o, d_o, lse_attn, cu_seqlens, cu_cmp, batch, block, stride, scale, causal=True,
+                 delta=None, rowscale=None):
     """Backward of the compressed attention.  q [total,Hq,Dk], ck [rows,Hkv,Dk], cv [rows,Hkv,Dv]
     (packed over cu_cmp), o / d_o [total,Hq,Dv], lse_attn from cmp_attn(want_lse_attn=True).
-    Returns (dq, dck, dcv)."""
-    _need_cuda(q, ck, cv, o, d_o, lse_attn, cu_seqlens, cu_cmp)
-    q, ck, cv, o, d_o = (_dense(t) for t in (q, ck, cv, o, d_o))
+    delta (float32 [total,Hq]) = rowsum(o*d_o) if already known (o may then be None); rowscale (float32
+    [total,Hq]) = a per-row gate applied to d_o inside the kernels.  Returns (dq, dck, dcv)."""
+    _need_cuda(q, ck, cv, d_o, lse_attn, cu_seqlens, cu_cmp)
+    q, ck, cv, d_o = (_dense(t) for t in (q, ck, cv, d_o))
+    o = None if o is None else _dense(o)
     total, hq, dk = q.shape
     rows, hkv, dv = cv.shape
     dq, dck, dcv = torch.empty_like(q), torch.empty_like(ck), torch.empty_like(cv)
     lib = _lib.load()
     need = lib.nsa_cmp_attn_bwd_workspace_bytes(total, rows, hq, hkv, dk, dv)
     ws = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
-    rc = lib.nsa_cmp_attn_bwd(_ptr(q), _ptr(ck), _ptr(cv), _ptr(o), _ptr(d_o), _ptr(lse_attn), _ptr(cu_seqlens),
-                              _ptr(cu_cmp), batch, total, rows, hq, hkv, dk, dv, block, stride, float(scale),
+    rc = lib.nsa_cmp_attn_bwd(_ptr(q), _ptr(ck), _ptr(cv), _ptr(o), _ptr(d_o), _ptr(lse_attn), _ptr(delta),
+                              _ptr(rowscale), _ptr(cu_seqlens), _ptr(cu_cmp), batch, total, rows, hq, hkv, dk, dv, block, stride, float(scale),
                               int(bool(causal)), _dtype_code(q), _ptr(dq), _ptr(dck), _ptr(dcv), _ptr(ws),
                               ws.numel(), _stream())
     _lib.check(rc, "nsa_cmp_attn_bwd")
@@ -330,10 +333,11 @@ def cmp_attn_bwd(q, ck, cv, o, d_o, lse_attn, cu_seqlens, cu_cmp, batch, block, 
 
 
 def slc_swa_bwd(q, k, v, o_slc, d_o_slc, lse_slc, o_swa, d_o_swa, lse_swa, indices, counts, cu_seqlens, batch,
-                block_size, window, scale):
+                block_size, window, scale, delta_slc=None, delta_swa=None, rowscale_slc=None, rowscale_swa=None):
     """Backward of the selected (o_slc / d_o_slc / lse_slc, or None) and sliding (o_swa / d_o_swa /
-    lse_swa, or None) branches.  v is the row-major [total,Hkv,Dv] tensor.  Returns (dq, dk, dv), each
-    the sum over the branches given."""
+    lse_swa, or None) branches.  v is the row-major [total,Hkv,Dv] tensor.  delta_* / rowscale_* as in
+    cmp_attn_bwd (with delta_* the matching o_* may be None).  Returns (dq, dk, dv), each the sum over
+    the branches given."""
     _need_cuda(q, k, v, cu_seqlens)
     q, k, v = _dense(q), _dense(k), _dense(v)
     total, hq, dk = q.shape
@@ -346,9 +350,9 @@ def slc_swa_bwd(q, k, v, o_slc, d_o_slc, lse_slc, o_swa, d_o_swa, lse_swa, indic
         indices = indices.contiguous()
         top_n = indices.shape[-1]
         counts = None if counts is None else counts.to(torch.int32).contiguous()
-        o_slc, d_o_slc = _dense(o_slc), _dense(d_o_slc)
+        o_slc, d_o_slc = (None if o_slc is None else _dense(o_slc)), _dense(d_o_slc)
     if swa_:
-        o_swa, d_o_swa = _dense(o_swa), _dense(d_o_swa)
+        o_swa, d_o_swa = (None if o_swa is None else _dense(o_swa)), _dense(d_o_swa)
     dq, dk_out, dv_out = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     lib = _lib.load()
     need = lib.nsa_slc_swa_bwd_workspace_bytes(total, batch, hq, hkv, dk, dv, top_n, block_size, _dtype_code(q))
@@ -356,7 +360,9 @@ def slc_swa_bwd(q, k, v, o_slc, d_o_slc, lse_slc, o_swa, d_o_swa, lse_swa, indic
     rc = lib.nsa_slc_swa_bwd(
         _ptr(q), _ptr(k), _ptr(v), _ptr(o_slc if slc else None), _ptr(o_swa if swa_ else None),
         _ptr(d_o_slc if slc else None), _ptr(d_o_swa if swa_ else None), _ptr(lse_slc if slc else None),
-        _ptr(lse_swa if swa_ else None), _ptr(indices if slc else None), _ptr(counts if slc else None),
+        _ptr(lse_swa if swa_ else None), _ptr(delta_slc if slc else None), _ptr(delta_swa if swa_ else None),
+        _ptr(rowscale_slc if slc else None), _ptr(rowscale_swa if swa_ else None),
+        _ptr(indices if slc else None), _ptr(counts if slc else None),
         _ptr(cu_seqlens), batch, total, hq, hkv, dk, dv, top_n, block_size, window if swa_ else 0, float(scale),
         int(slc and indices.dtype == torch.int64), _dtype_code(q), _ptr(dq), _ptr(dk_out), _ptr(dv_out), _ptr(ws),
         ws.numel(), _stream())
@@ -428,20 +434,26 @@ def gate_combine(gate_logits, o_slc, o_swa, o_cmp, gate_act=0):
     return out
 
 
-def gate_combine_bwd(gate_logits, d_out, o_slc, o_swa, o_cmp, gate_act=0):
-    """Returns (d_o_slc, d_o_swa or None, d_o_cmp or None, d_gate_logits [total,Hq,3])."""
+def gate_combine_bwd(gate_logits, d_out, o_slc, o_swa, o_cmp, gate_act=0, want_scaled=True, want_stats=False):
+    """Returns (d_o_slc, d_o_swa or None, d_o_cmp or None, d_gate_logits [total,Hq,3]) and, with want_stats,
+    a fifth tensor float32 [6, total, Hq]: <d_out, o_b> for b = selected, sliding, compressed, then the
+    activated gates (the delta / rowscale inputs of the attention backward).  want_scaled=False skips the
+    scaled copies (they come back as None)."""
     _need_cuda(gate_logits, d_out, o_slc)
     gl = _dense(gate_logits.to(o_slc.dtype))
     d_out, o_slc = _dense(d_out), _dense(o_slc)
     o_swa = None if o_swa is None else _dense(o_swa)
     o_cmp = None if o_cmp is None else _dense(o_cmp)
     total, hq, dv = o_slc.shape
-    d_slc = torch.empty_like(o_slc)
-    d_swa = None if o_swa is None else torch.empty_like(o_slc)
-    d_cmp = None if o_cmp is None else torch.empty_like(o_slc)
+    if not (want_scaled or want_stats):
+        raise ValueError("gate_combine_bwd: nothing requested")
+    d_slc = torch.empty_like(o_slc) if want_scaled else None
+    d_swa = None if o_swa is None or not want_scaled else torch.empty_like(o_slc)
+    d_cmp = None if o_cmp is None or not want_scaled else torch.empty_like(o_slc)
     d_gl = torch.empty(total, hq, 3, dtype=o_slc.dtype, device=o_slc.device)
+    stats = torch.empty(6, total, hq, dtype=torch.float32, device=o_slc.device) if want_stats else None
     rc = _lib.load().nsa_gate_combine_bwd(_ptr(gl), _ptr(d_out), _ptr(o_slc), _ptr(o_swa), _ptr(o_cmp), _ptr(d_slc),
-                                          _ptr(d_swa), _ptr(d_cmp), _ptr(d_gl), total * hq, dv, gate_act,
+                                          _ptr(d_swa), _ptr(d_cmp), _ptr(d_gl), _ptr(stats), total * hq, dv, gate_act,
                                           _dtype_code(o_slc), _stream())
     _lib.check(rc, "nsa_gate_combine_bwd")
-    return d_slc, d_swa, d_cmp, d_gl
+    return (d_slc, d_swa, d_cmp, d_gl, stats) if want_stats else (d_slc, d_swa, d_cmp, d_gl)

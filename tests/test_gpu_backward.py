@@ -235,9 +235,12 @@ def _leaf(t):
     return t.to(DEV).requires_grad_(True)
 
 
-@pytest.mark.parametrize("mode,lens,Hq,Hkv,Dk,Dv", [("mean", [600], 16, 1, 64, 64), ("mean", [300, 200, 40], 32, 2, 128, 128),
-                                                    ("conv", [500], 16, 1, 64, 64), ("mean", [400], 16, 1, 192, 128)])
-def test_module_backward(mode, lens, Hq, Hkv, Dk, Dv):
+@pytest.mark.parametrize("mode,lens,Hq,Hkv,Dk,Dv,act", [("mean", [600], 16, 1, 64, 64, "sigmoid"),
+                                                        ("mean", [300, 200, 40], 32, 2, 128, 128, "sigmoid"),
+                                                        ("conv", [500], 16, 1, 64, 64, "sigmoid"),
+                                                        ("mean", [400], 16, 1, 192, 128, "sigmoid"),
+                                                        ("mean", [450], 32, 2, 64, 64, None)])
+def test_module_backward(mode, lens, Hq, Hkv, Dk, Dv, act):
     """NSAAttention end to end: gradients of every input and parameter against autograd through the
     oracle forward (float64, the module's own block picks forced so that score ties cannot differ)."""
     from nsa_amd.nsa import NSAAttention
@@ -247,7 +250,7 @@ def test_module_backward(mode, lens, Hq, Hkv, Dk, Dv):
     torch.manual_seed(5)
     mod = NSAAttention(Dk, causal=True, compression_stride=16, compression_block=32, selection_block=64,
                        selected_block_count=4, sliding_window=64, device=DEV, dtype=dtype, compressor_mode=mode,
-                       gate_activation="sigmoid")
+                       gate_activation=act)       # None: raw gates of either sign, as in the reference
     if mode == "conv" and Dk != Dv:
         pytest.skip("the Conv1d compressor has one head_dim")
     q, k, v, _ = make_qkv(T, Hq, Hkv, Dk, Dv, 190, dtype, 0.7)
@@ -273,7 +276,8 @@ def test_module_backward(mode, lens, Hq, Hkv, Dk, Dv):
     cuh = ragged_cu(lens)
     outs = []
     for s, e in zip(cuh[:-1], cuh[1:]):
-        gates = torch.sigmoid(qr[s:e] @ gw.t() + gb)
+        gates = qr[s:e] @ gw.t() + gb
+        gates = torch.sigmoid(gates) if act == "sigmoid" else gates
         outs.append(O.nsa_forward_single(qr[s:e], kr[s:e], vr[s:e], gates, p, comp, math_dtype=torch.float64,
                                          force_idx=idx[s:e].cpu()))
     ref = torch.cat(outs)
@@ -418,6 +422,14 @@ def test_gate_and_combine_kernels(dtype, T, Hq, D, Dv, act):
         if with_cmp:
             _check("dcmp", d_cmp, orr[2].grad, dtype)
         _check("dgl", d_gl, glr.grad, dtype, floor=float(glr.grad.abs().max()) if dtype == torch.bfloat16 else 1.0)
+        # the same call asked for the row sums and gates instead of the scaled copies
+        n1, n2, n3, d_gl2, st = ops.gate_combine_bwd(gl.to(DEV), d_out.to(DEV), od[0], od[1], od[2], act,
+                                                     want_scaled=False, want_stats=True)
+        assert n1 is None and n2 is None and n3 is None and torch.equal(d_gl2, d_gl)
+        for b, present in enumerate((True, with_swa, with_cmp)):
+            dots = (d_out.double() * o[b].double()).sum(-1) if present else torch.zeros(T, Hq, dtype=torch.float64)
+            _check("dot%d" % b, st[b], dots, torch.float32, floor=float(dots.abs().max()) * (64 if dtype == torch.bfloat16 else 1))
+            _check("g%d" % b, st[3 + b], f(gl.double()[..., b]), torch.float32)
     dq, dw, db = ops.gate_bwd(q.to(DEV), w.to(DEV), d_gl_in.to(DEV))
     qr, wr = q.double().requires_grad_(True), w.double().requires_grad_(True)
     br = torch.zeros(3, dtype=torch.float64, requires_grad=True)

@@ -131,19 +131,19 @@ def test_backward_argument_errors_do_not_launch(lib):
     buf = ctypes.create_string_buffer(4096)
     p = ctypes.c_void_p((ctypes.addressof(buf) + 15) & ~15)
     # compressed attention backward
-    rc = lib.nsa_cmp_attn_bwd(None, p, p, p, p, p, p, p, 1, 64, 2, 16, 1, 64, 64, 32, 16, 0.1, 1, 0, p, p, p, p, 1 << 20, None)
+    rc = lib.nsa_cmp_attn_bwd(None, p, p, p, p, p, None, None, p, p, 1, 64, 2, 16, 1, 64, 64, 32, 16, 0.1, 1, 0, p, p, p, p, 1 << 20, None)
     assert rc == -1 and b"null" in lib.nsa_last_error_string()
-    rc = lib.nsa_cmp_attn_bwd(p, p, p, p, p, p, p, p, 1, 64, 2, 16, 1, 64, 64, 32, 16, 0.1, 1, 0, p, p, p, p, 8, None)
+    rc = lib.nsa_cmp_attn_bwd(p, p, p, p, p, p, None, None, p, p, 1, 64, 2, 16, 1, 64, 64, 32, 16, 0.1, 1, 0, p, p, p, p, 8, None)
     assert rc == -1 and b"workspace" in lib.nsa_last_error_string()
     assert lib.nsa_cmp_attn_bwd_workspace_bytes(64, 2, 16, 1, 64, 64) >= 64 * 16 * 4 + 2 * 2 * 64 * 4
     # selected + sliding backward: a branch needs its saved tensors, the selected one 64-key blocks
-    rc = lib.nsa_slc_swa_bwd(p, p, p, None, None, p, None, None, None, None, None, p, 1, 64, 16, 1, 64, 64, 4, 64, 0, 0.1, 1,
+    rc = lib.nsa_slc_swa_bwd(p, p, p, None, None, p, None, None, None, None, None, None, None, None, None, p, 1, 64, 16, 1, 64, 64, 4, 64, 0, 0.1, 1,
                              0, p, p, p, p, 1 << 30, None)
     assert rc == -1 and b"selected branch" in lib.nsa_last_error_string()
-    rc = lib.nsa_slc_swa_bwd(p, p, p, p, None, p, None, p, None, p, None, p, 1, 64, 16, 1, 64, 64, 4, 32, 0, 0.1, 1, 0, p, p,
+    rc = lib.nsa_slc_swa_bwd(p, p, p, p, None, p, None, p, None, None, None, None, None, p, None, p, 1, 64, 16, 1, 64, 64, 4, 32, 0, 0.1, 1, 0, p, p,
                              p, p, 1 << 30, None)
     assert rc == -2 and b"64-key" in lib.nsa_last_error_string()
-    rc = lib.nsa_slc_swa_bwd(p, p, p, None, p, None, p, None, p, None, None, p, 1, 64, 16, 1, 64, 64, 0, 64, 0, 0.1, 1, 0, p, p,
+    rc = lib.nsa_slc_swa_bwd(p, p, p, None, p, None, p, None, p, None, None, None, None, None, None, p, 1, 64, 16, 1, 64, 64, 0, 64, 0, 0.1, 1, 0, p, p,
                              p, p, 1 << 30, None)
     assert rc == -1 and b"sliding branch" in lib.nsa_last_error_string()
     need = lib.nsa_slc_swa_bwd_workspace_bytes(64, 1, 16, 1, 64, 64, 4, 64, 0)
@@ -155,7 +155,7 @@ def test_backward_argument_errors_do_not_launch(lib):
     assert rc == -1
     rc = lib.nsa_gate_combine_fwd(p, p, None, None, p, 64, 60, 0, 0, None)
     assert rc == -1 and b"multiple of 8" in lib.nsa_last_error_string()
-    rc = lib.nsa_gate_combine_bwd(p, p, p, p, None, p, None, None, p, 64, 64, 0, 0, None)
+    rc = lib.nsa_gate_combine_bwd(p, p, p, p, None, p, None, None, p, None, 64, 64, 0, 0, None)
     assert rc == -1 and b"null" in lib.nsa_last_error_string()
 
 
