@@ -102,6 +102,7 @@ stream_attn_kernel(const StreamParams a) {
   // CMP runs two softmaxes off one reference (raw scores for the importance statistics, scaled ones
   // for the attention): the slack, in raw score units, bounds the faster growing exponential
   const float cmp_slack = kMaxSlackLog2 / fmaxf(kLog2e, c_attn);
+  const float cmp_probe = fast_exp2(cmp_slack * kLog2e);          // exp of the slack in raw-score units
   const int attn_end = last_visible(t_last);                      // last key any row of the tile attends
   const int c_begin = CMP ? 0 : (max(st.t0 - W + 1, 0) / CH) * CH;
   const int c_end = CMP ? nkeys : t_last + 1;
@@ -180,6 +181,7 @@ stream_attn_kernel(const StreamParams a) {
     for (int sub = 0; sub < CH / 32; ++sub) {
       const int cb = c0 + 32 * sub;
       if (cb >= c_end) break;
+      const bool first_sub = CMP && cb == c_begin;
       bool act[NG];
       bool any_act = false;
 #pragma unroll
@@ -206,11 +208,25 @@ stream_attn_kernel(const StreamParams a) {
             for (int i = 0; i < 8; ++i)
               if (key0 + i >= nkeys) s[i] = kNegInf;
           }
-          float mx = s[0];
+          // The raw-score exponentials are needed anyway (importance log-sum-exp), so they double as the
+          // overflow probe: a score more than the slack above the reference makes its exponential, and
+          // with it the lane's sum of 8, exceed 2^slack.  Only then (and on the very first chunk, while
+          // the reference is still -inf) is the maximum taken and the reference moved; the common case
+          // pays neither the 8-way maximum nor its reduction over the column's four lanes.
+          float ei[8], si = 0.f;
+          bool redo = first_sub;
+          if (!first_sub) {
+            const float off_i = -grp[j].m * kLog2e;
 #pragma unroll
-          for (int i = 1; i < 8; ++i) mx = fmaxf(mx, s[i]);
-          mx = colgroup_max(mx);                       // finite: key cb exists
-          if (__any(mx > grp[j].m + cmp_slack)) {
+            for (int i = 0; i < 8; ++i) ei[i] = fast_exp2(fmaf(s[i], kLog2e, off_i));
+            si = sum8(ei);
+            redo = __any(si > cmp_probe);
+          }
+          if (redo) {
+            float mx = s[0];
+#pragma unroll
+            for (int i = 1; i < 8; ++i) mx = fmaxf(mx, s[i]);
+            mx = colgroup_max(mx);                     // finite: key cb exists
             const float m_new = fmaxf(grp[j].m, mx);
             const float d = grp[j].m - m_new;          // -inf on the first chunk
             float beta = fast_exp2(d * kLog2e), alpha = fast_exp2(d * c_attn);
@@ -220,15 +236,13 @@ stream_attn_kernel(const StreamParams a) {
 #pragma unroll
             for (int t = 0; t < DV / 16; ++t) scale_inplace(grp[j].o[t], alpha);
             grp[j].m = m_new;
-          }
-          const float m = grp[j].m;
-          const float off_i = -m * kLog2e, off_a = -m * c_attn;
-          {
-            float ei[8];
+            const float off_i = -m_new * kLog2e;
 #pragma unroll
             for (int i = 0; i < 8; ++i) ei[i] = fast_exp2(fmaf(s[i], kLog2e, off_i));
-            li[j] += sum8(ei);
+            si = sum8(ei);
           }
+          li[j] += si;
+          const float off_a = -grp[j].m * c_attn;
           if (act[j]) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
