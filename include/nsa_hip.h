@@ -257,6 +257,24 @@ int nsa_decode_step(const void* q, const void* k_cache, const void* v_cache_t, c
                     int sel_block, int pool_kernel, int pool_stride, int pool_pad, int top_n, int window, float scale,
                     int gate_act, int dtype, nsa_stream_t stream);
 
+/* The same step on a paged K/V cache (pages of 64 tokens = one selection block):
+ *   k_pool [pages][64][hkv][dk]      v_pool_t [pages][hkv][dv][64]
+ *   block_table int32 [batch][max_pages]: page i of sequence b holds its tokens [64 i, 64 i + 64)
+ * The compressed caches stay contiguous per sequence as above.  Results are bit-identical to
+ * nsa_decode_step on the same tokens.  Every table entry up to the page of token ctx_lens[b]-1 must
+ * name a page of the pool; the library cannot check this.  Neither call has a counterpart in the
+ * reference (it has no cache). */
+int nsa_decode_step_paged(const void* q, const void* k_pool, const void* v_pool_t, const int32_t* block_table,
+                          int max_pages, const void* ck_cache, const void* cv_cache_t, const int32_t* ctx_lens,
+                          const void* gates, void* out, int32_t* indices, int batch, int hq, int hkv, int dk, int dv,
+                          int nc_cap, int block, int stride, int sel_block, int pool_kernel, int pool_stride,
+                          int pool_pad, int top_n, int window, float scale, int gate_act, int dtype,
+                          nsa_stream_t stream);
+int nsa_decode_append_paged(const void* k_new, const void* v_new, void* k_pool, void* v_pool_t,
+                            const int32_t* block_table, int max_pages, void* ck_cache, void* cv_cache_t,
+                            const int32_t* pos, int batch, int hkv, int dk, int dv, int nc_cap, int block, int stride,
+                            int dtype, nsa_stream_t stream);
+
 /* Appends one token per sequence: k_new [batch][hkv][dk] -> row pos[b] of k_cache, v_new
  * [batch][hkv][dv] -> column pos[b] of v_cache_t, and, when pos[b]+1 completes a compression block,
  * the mean of the last `block` tokens as the next row / column of the compressed caches. */

@@ -47,6 +47,8 @@ SIGNATURES = {
     "nsa_decode_max_compressed": (_I, []),
     "nsa_decode_step": (_I, [_P] * 9 + [_I] * 15 + [_F, _I, _I, _P]),
     "nsa_decode_append": (_I, [_P] * 7 + [_I] * 9 + [_P]),
+    "nsa_decode_step_paged": (_I, [_P] * 4 + [_I] + [_P] * 6 + [_I] * 14 + [_F, _I, _I, _P]),
+    "nsa_decode_append_paged": (_I, [_P] * 5 + [_I] + [_P] * 3 + [_I] * 8 + [_P]),
 }
 
 _lib = None

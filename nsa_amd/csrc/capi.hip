@@ -380,35 +380,72 @@ int nsa_slc_swa_bwd(const void* q, const void* k, const void* v, const void* o_s
   return finish(rc, "slc_swa_bwd");
 }
 
+int nsa_decode_append_paged(const void* k_new, const void* v_new, void* k_pool, void* v_pool_t,
+                            const int32_t* block_table, int max_pages, void* ck_cache, void* cv_cache_t,
+                            const int32_t* pos, int batch, int hkv, int dk, int dv, int nc_cap, int block, int stride,
+                            int dtype, nsa_stream_t stream) {
+  if (!k_new || !v_new || !k_pool || !v_pool_t || !block_table || !ck_cache || !cv_cache_t || !pos)
+    return fail(NSA_ERR_INVALID, "decode_append_paged: null pointer");
+  if (batch <= 0 || hkv <= 0 || dk <= 0 || dv <= 0 || max_pages <= 0 || nc_cap <= 0 || block <= 0 || stride <= 0)
+    return fail(NSA_ERR_INVALID, "decode_append_paged: sizes must be positive");
+  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "decode_append_paged: bad dtype");
+  return finish(nsa::launch_decode_append_paged(k_new, v_new, k_pool, v_pool_t, block_table, max_pages, ck_cache,
+                                                cv_cache_t, pos, batch, hkv, dk, dv, nc_cap, block, stride, dtype,
+                                                stream), "decode_append_paged");
+}
+
 int nsa_decode_max_compressed(void) { return nsa::decode_max_nc(); }
+
+static int decode_common(const char* what, const void* q, const void* k_cache, const void* v_cache_t,
+                         const int32_t* block_table, int max_pages, const void* ck_cache, const void* cv_cache_t,
+                         const int32_t* ctx_lens, const void* gates, void* out, int32_t* indices, int batch, int hq,
+                         int hkv, int dk, int dv, int ctx_cap, int nc_cap, int block, int stride, int sel_block,
+                         int pool_kernel, int pool_stride, int pool_pad, int top_n, int window, float scale,
+                         int gate_act, int dtype, nsa_stream_t stream) {
+  if (!q || !k_cache || !v_cache_t || !ck_cache || !cv_cache_t || !ctx_lens || !out)
+    return fail(NSA_ERR_INVALID, "%s: null pointer", what);
+  if (batch <= 0 || ctx_cap <= 0 || nc_cap <= 0 || block <= 0 || stride <= 0 || window < 0)
+    return fail(NSA_ERR_INVALID, "%s: sizes must be positive", what);
+  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "%s: bad dtype", what);
+  if (int rc = check_heads(what, hq, hkv, dk, dv)) return rc;
+  if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "%s: scale must be positive", what);
+  if (ctx_cap % 64 != 0 || nc_cap % 64 != 0) return fail(NSA_ERR_INVALID, "%s: cache capacities must be multiples of 64", what);
+  if (nc_cap > nsa::decode_max_nc())
+    return fail(NSA_ERR_UNSUPPORTED, "%s: at most %d compressed rows per sequence are built", what, nsa::decode_max_nc());
+  if (sel_block <= 0 || sel_block % 32 != 0) return fail(NSA_ERR_UNSUPPORTED, "%s: selection block must be a multiple of 32", what);
+  if (pool_kernel <= 0 || pool_stride <= 0 || pool_pad < 0 || pool_pad >= pool_kernel || top_n <= 0)
+    return fail(NSA_ERR_INVALID, "%s: bad pooling / top-n parameters", what);
+  if (gate_act != NSA_GATE_IDENTITY && gate_act != NSA_GATE_SIGMOID) return fail(NSA_ERR_INVALID, "%s: bad gate activation", what);
+  if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache_t) || !aligned16(ck_cache) || !aligned16(cv_cache_t))
+    return fail(NSA_ERR_INVALID, "%s: pointers must be 16-byte aligned", what);
+  nsa::DecodeArgs a{q, k_cache, v_cache_t, ck_cache, cv_cache_t, ctx_lens, gates, out, indices, batch, hq, hkv, dk, dv,
+                    ctx_cap, nc_cap, block, stride, sel_block, pool_kernel, pool_stride, pool_pad, top_n, window, scale,
+                    gate_act, dtype, block_table, max_pages};
+  const int rc = nsa::launch_decode(a, stream);
+  if (rc == -2) return fail(NSA_ERR_UNSUPPORTED, "%s: head dims not built (dk,dv in (64,64),(128,128),(192,128); fp32: no 192)", what);
+  return finish(rc, what);
+}
 
 int nsa_decode_step(const void* q, const void* k_cache, const void* v_cache_t, const void* ck_cache,
                     const void* cv_cache_t, const int32_t* ctx_lens, const void* gates, void* out, int32_t* indices,
                     int batch, int hq, int hkv, int dk, int dv, int ctx_cap, int nc_cap, int block, int stride,
                     int sel_block, int pool_kernel, int pool_stride, int pool_pad, int top_n, int window, float scale,
                     int gate_act, int dtype, nsa_stream_t stream) {
-  if (!q || !k_cache || !v_cache_t || !ck_cache || !cv_cache_t || !ctx_lens || !out)
-    return fail(NSA_ERR_INVALID, "decode_step: null pointer");
-  if (batch <= 0 || ctx_cap <= 0 || nc_cap <= 0 || block <= 0 || stride <= 0 || window < 0)
-    return fail(NSA_ERR_INVALID, "decode_step: sizes must be positive");
-  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "decode_step: bad dtype");
-  if (int rc = check_heads("decode_step", hq, hkv, dk, dv)) return rc;
-  if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "decode_step: scale must be positive");
-  if (ctx_cap % 64 != 0 || nc_cap % 64 != 0) return fail(NSA_ERR_INVALID, "decode_step: cache capacities must be multiples of 64");
-  if (nc_cap > nsa::decode_max_nc())
-    return fail(NSA_ERR_UNSUPPORTED, "decode_step: at most %d compressed rows per sequence are built", nsa::decode_max_nc());
-  if (sel_block <= 0 || sel_block % 32 != 0) return fail(NSA_ERR_UNSUPPORTED, "decode_step: selection block must be a multiple of 32");
-  if (pool_kernel <= 0 || pool_stride <= 0 || pool_pad < 0 || pool_pad >= pool_kernel || top_n <= 0)
-    return fail(NSA_ERR_INVALID, "decode_step: bad pooling / top-n parameters");
-  if (gate_act != NSA_GATE_IDENTITY && gate_act != NSA_GATE_SIGMOID) return fail(NSA_ERR_INVALID, "decode_step: bad gate activation");
-  if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache_t) || !aligned16(ck_cache) || !aligned16(cv_cache_t))
-    return fail(NSA_ERR_INVALID, "decode_step: pointers must be 16-byte aligned");
-  nsa::DecodeArgs a{q, k_cache, v_cache_t, ck_cache, cv_cache_t, ctx_lens, gates, out, indices, batch, hq, hkv, dk, dv,
-                    ctx_cap, nc_cap, block, stride, sel_block, pool_kernel, pool_stride, pool_pad, top_n, window, scale,
-                    gate_act, dtype};
-  const int rc = nsa::launch_decode(a, stream);
-  if (rc == -2) return fail(NSA_ERR_UNSUPPORTED, "decode_step: head dims not built (dk,dv in (64,64),(128,128),(192,128); fp32: no 192)");
-  return finish(rc, "decode_step");
+  return decode_common("decode_step", q, k_cache, v_cache_t, nullptr, 0, ck_cache, cv_cache_t, ctx_lens, gates, out,
+                       indices, batch, hq, hkv, dk, dv, ctx_cap, nc_cap, block, stride, sel_block, pool_kernel,
+                       pool_stride, pool_pad, top_n, window, scale, gate_act, dtype, stream);
+}
+
+int nsa_decode_step_paged(const void* q, const void* k_pool, const void* v_pool_t, const int32_t* block_table,
+                          int max_pages, const void* ck_cache, const void* cv_cache_t, const int32_t* ctx_lens,
+                          const void* gates, void* out, int32_t* indices, int batch, int hq, int hkv, int dk, int dv,
+                          int nc_cap, int block, int stride, int sel_block, int pool_kernel, int pool_stride,
+                          int pool_pad, int top_n, int window, float scale, int gate_act, int dtype,
+                          nsa_stream_t stream) {
+  if (!block_table || max_pages <= 0) return fail(NSA_ERR_INVALID, "decode_step_paged: needs a block table");
+  return decode_common("decode_step_paged", q, k_pool, v_pool_t, block_table, max_pages, ck_cache, cv_cache_t, ctx_lens,
+                       gates, out, indices, batch, hq, hkv, dk, dv, max_pages * 64, nc_cap, block, stride, sel_block,
+                       pool_kernel, pool_stride, pool_pad, top_n, window, scale, gate_act, dtype, stream);
 }
 
 int nsa_decode_append(const void* k_new, const void* v_new, void* k_cache, void* v_cache_t, void* ck_cache,

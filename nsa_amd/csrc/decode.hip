@@ -6,7 +6,11 @@
 //   ck_cache   [B][nc_cap][Hkv][Dk]    compressed keys,  row n = mean of tokens [n*stride, n*stride+block)
 //   cv_cache_t [B][Hkv][Dv][nc_cap]    compressed values, key-contiguous (nc_cap a multiple of 64)
 // so every MFMA operand of the step is a plain 16-byte global load: K fragments are rows, V^T
-// fragments are 8 contiguous keys of one channel.  The step is bound by HBM: per sequence and kv
+// fragments are 8 contiguous keys of one channel.
+// Paged variant: k / v live in a pool of 64-token pages (one selection block = one page),
+//   k_pool [page][64][Hkv][Dk],  v_pool_t [page][Hkv][Dv][64],  block_table [B][max_pages]
+// and a 32-key chunk looks its page up (a wavefront-uniform scalar load) before requesting its
+// fragments; the compressed caches stay contiguous.  The step is bound by HBM: per sequence and kv
 // head it reads all compressed keys once (block importance is scored over every compressed row),
 // the visible compressed values, the selected blocks and the window.
 //
@@ -113,7 +117,7 @@ __device__ __forceinline__ void chunk_attend(DecState<T, DK, DV>& st, const Chun
   }
 }
 
-template <typename T, int DK, int DV>
+template <typename T, int DK, int DV, bool PAGED>
 __global__ void __launch_bounds__(kDecWaves * 64)
 decode_step_kernel(const DecodeArgs a) {
   constexpr int NW = kDecWaves, MAXC = kDecMaxChunks, PLD = 17;
@@ -141,10 +145,21 @@ decode_step_kernel(const DecodeArgs a) {
   const int cmaxv = t >= a.block ? min((t - a.block) / a.stride, Nc - 1) : -1;   // last visible compressed row
   const float c_attn = a.scale * kLog2e;
 
-  const T* kseq = reinterpret_cast<const T*>(a.k_cache) + ((long)b * a.ctx_cap * a.hkv + h) * DK;
+  const T* kseq = reinterpret_cast<const T*>(a.k_cache) + (PAGED ? (long)h * DK : ((long)b * a.ctx_cap * a.hkv + h) * DK);
   const long krow = (long)a.hkv * DK;
-  const T* vt = reinterpret_cast<const T*>(a.v_cache_t) + (((long)b * a.hkv + h) * DV + n) * a.ctx_cap + 8 * g;
-  const long vstep = 16L * a.ctx_cap;
+  const T* vt = reinterpret_cast<const T*>(a.v_cache_t) +
+                (PAGED ? ((long)h * DV + n) * 64 + 8 * g : (((long)b * a.hkv + h) * DV + n) * a.ctx_cap + 8 * g);
+  const long vstep = PAGED ? 16L * 64 : 16L * a.ctx_cap;
+  // fragments of keys [cb, cb+32) of this sequence (rows past the newest token t are clamped to it)
+  auto issue_kv = [&](ChunkFrags<T, DK, DV>& f, int cb) {
+    if constexpr (PAGED) {
+      const long pg = a.block_table[(long)b * a.max_pages + (cb >> 6)];
+      chunk_issue<T, DK, DV>(f, kseq + pg * 64 * krow, krow, vt + pg * a.hkv * DV * 64, vstep, cb & 63,
+                             min(t - (cb & ~63), 63), n, g);
+    } else {
+      chunk_issue<T, DK, DV>(f, kseq, krow, vt, vstep, cb, t, n, g);
+    }
+  };
   const T* ckseq = reinterpret_cast<const T*>(a.ck_cache) + ((long)b * a.nc_cap * a.hkv + h) * DK;
   const T* cvt = reinterpret_cast<const T*>(a.cv_cache_t) + (((long)b * a.hkv + h) * DV + n) * a.nc_cap + 8 * g;
   const long cvstep = 16L * a.nc_cap;
@@ -205,14 +220,14 @@ decode_step_kernel(const DecodeArgs a) {
     const int w_lo = max(t - a.window + 1, 0);
     ChunkFrags<T, DK, DV> fa, fb;
     int cb = (w_lo / 32) * 32 + 32 * wave;
-    if (cb <= t) chunk_issue<T, DK, DV>(fa, kseq, krow, vt, vstep, cb, t, n, g);
+    if (cb <= t) issue_kv(fa, cb);
     while (cb <= t) {
       const int cb2 = cb + 32 * NW;
-      if (cb2 <= t) chunk_issue<T, DK, DV>(fb, kseq, krow, vt, vstep, cb2, t, n, g);
+      if (cb2 <= t) issue_kv(fb, cb2);
       chunk_attend<T, DK, DV>(swa, fa, qf, cb, w_lo, t, c_attn, g);
       if (cb2 > t) break;
       const int cb3 = cb2 + 32 * NW;
-      if (cb3 <= t) chunk_issue<T, DK, DV>(fa, kseq, krow, vt, vstep, cb3, t, n, g);
+      if (cb3 <= t) issue_kv(fa, cb3);
       chunk_attend<T, DK, DV>(swa, fb, qf, cb2, w_lo, t, c_attn, g);
       cb = cb3;
     }
@@ -406,14 +421,14 @@ decode_step_kernel(const DecodeArgs a) {
     ChunkFrags<T, DK, DV> fa, fb;
     int cba, k0a, k1a, cbb, k0b, k1b;
     bool ha = next_chunk(cba, k0a, k1a);
-    if (ha) chunk_issue<T, DK, DV>(fa, kseq, krow, vt, vstep, cba, t, n, g);
+    if (ha) issue_kv(fa, cba);
     while (ha) {
       const bool hb = next_chunk(cbb, k0b, k1b);
-      if (hb) chunk_issue<T, DK, DV>(fb, kseq, krow, vt, vstep, cbb, t, n, g);
+      if (hb) issue_kv(fb, cbb);
       chunk_attend<T, DK, DV>(slc, fa, qf, cba, k0a, k1a, c_attn, g);
       if (!hb) break;
       ha = next_chunk(cba, k0a, k1a);
-      if (ha) chunk_issue<T, DK, DV>(fa, kseq, krow, vt, vstep, cba, t, n, g);
+      if (ha) issue_kv(fa, cba);
       chunk_attend<T, DK, DV>(slc, fb, qf, cbb, k0b, k1b, c_attn, g);
     }
   }
@@ -459,13 +474,61 @@ decode_append_kernel(const T* __restrict__ k_new, const T* __restrict__ v_new, T
   }
 }
 
+// The same for the paged pool: the token goes to slot pos % 64 of page block_table[b][pos / 64]; a
+// compression window may straddle two pages.
+template <typename T>
+__global__ void __launch_bounds__(256)
+decode_append_paged_kernel(const T* __restrict__ k_new, const T* __restrict__ v_new, T* __restrict__ k_pool,
+                           T* __restrict__ v_pool_t, const int32_t* __restrict__ block_table, int max_pages,
+                           T* __restrict__ ck_cache, T* __restrict__ cv_cache_t, const int32_t* __restrict__ pos,
+                           int hkv, int dk, int dv, int nc_cap, int block, int stride) {
+  const int b = blockIdx.x;
+  const int p = pos[b];
+  if (p < 0 || p >= max_pages * 64) return;
+  const int32_t* table = block_table + (long)b * max_pages;
+  const long pg = table[p >> 6];
+  T* krow = k_pool + (pg * 64 + (p & 63)) * hkv * dk;
+  for (int i = threadIdx.x; i < hkv * dk; i += 256) krow[i] = k_new[(long)b * hkv * dk + i];
+  for (int i = threadIdx.x; i < hkv * dv; i += 256)
+    v_pool_t[(pg * hkv * dv + i) * 64 + (p & 63)] = v_new[(long)b * hkv * dv + i];
+  const int ctx = p + 1;
+  if (ctx < block || (ctx - block) % stride != 0) return;
+  const int nrow = (ctx - block) / stride;
+  if (nrow >= nc_cap) return;
+  __syncthreads();   // the row and column written above are part of the window below
+  const float inv = 1.0f / (float)block;
+  for (int i = threadIdx.x; i < hkv * dk; i += 256) {
+    float s = 0.f;
+    for (int j = 0; j < block; ++j) {
+      const int tk = ctx - block + j;
+      s += (float)k_pool[((long)table[tk >> 6] * 64 + (tk & 63)) * hkv * dk + i];
+    }
+    ck_cache[((long)b * nc_cap + nrow) * hkv * dk + i] = (T)(s * inv);
+  }
+  for (int i = threadIdx.x; i < hkv * dv; i += 256) {
+    float s = 0.f;
+    for (int j = 0; j < block; ++j) {
+      const int tk = ctx - block + j;
+      s += (float)v_pool_t[((long)table[tk >> 6] * hkv * dv + i) * 64 + (tk & 63)];
+    }
+    cv_cache_t[((long)b * hkv * dv + i) * nc_cap + nrow] = (T)(s * inv);
+  }
+}
+
 int set_smem(const void* fn, size_t bytes);
 
 template <typename T, int DK, int DV>
 static int launch_decode_t(const DecodeArgs& a, hipStream_t st) {
   const size_t smem = ((size_t)kDecWaves * DV * 17 + kDecWaves * 64 + (a.nc_cap + 3) / 4 + 4) * sizeof(float) +
                       (size_t)a.top_n * sizeof(int) + 64;
-  auto fn = decode_step_kernel<T, DK, DV>;
+  if (a.block_table != nullptr) {
+    auto fn = decode_step_kernel<T, DK, DV, true>;
+    const int rc = set_smem(reinterpret_cast<const void*>(fn), smem);
+    if (rc) return rc;
+    hipLaunchKernelGGL(fn, dim3(a.batch * a.hkv), dim3(kDecWaves * 64), smem, st, a);
+    return 0;
+  }
+  auto fn = decode_step_kernel<T, DK, DV, false>;
   const int rc = set_smem(reinterpret_cast<const void*>(fn), smem);
   if (rc) return rc;
   hipLaunchKernelGGL(fn, dim3(a.batch * a.hkv), dim3(kDecWaves * 64), smem, st, a);
@@ -500,6 +563,21 @@ int launch_decode_append(const void* k_new, const void* v_new, void* k_cache, vo
     hipLaunchKernelGGL(decode_append_kernel<float>, dim3(batch), dim3(256), 0, st, (const float*)k_new,
                        (const float*)v_new, (float*)k_cache, (float*)v_cache_t, (float*)ck_cache,
                        (float*)cv_cache_t, pos, hkv, dk, dv, ctx_cap, nc_cap, block, stride);
+  return 0;
+}
+
+int launch_decode_append_paged(const void* k_new, const void* v_new, void* k_pool, void* v_pool_t,
+                               const int32_t* block_table, int max_pages, void* ck_cache, void* cv_cache_t,
+                               const int32_t* pos, int batch, int hkv, int dk, int dv, int nc_cap, int block,
+                               int stride, int dtype, hipStream_t st) {
+  if (dtype == 0)
+    hipLaunchKernelGGL(decode_append_paged_kernel<bf16_t>, dim3(batch), dim3(256), 0, st, (const bf16_t*)k_new,
+                       (const bf16_t*)v_new, (bf16_t*)k_pool, (bf16_t*)v_pool_t, block_table, max_pages,
+                       (bf16_t*)ck_cache, (bf16_t*)cv_cache_t, pos, hkv, dk, dv, nc_cap, block, stride);
+  else
+    hipLaunchKernelGGL(decode_append_paged_kernel<float>, dim3(batch), dim3(256), 0, st, (const float*)k_new,
+                       (const float*)v_new, (float*)k_pool, (float*)v_pool_t, block_table, max_pages,
+                       (float*)ck_cache, (float*)cv_cache_t, pos, hkv, dk, dv, nc_cap, block, stride);
   return 0;
 }
 

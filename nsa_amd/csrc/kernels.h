@@ -100,6 +100,10 @@ struct DecodeArgs {
   int batch, hq, hkv, dk, dv, ctx_cap, nc_cap;
   int block, stride, sel_block, pool_k, pool_s, pool_p, top_n, window;
   float scale; int gate_act, dtype;
+  // paged K/V (block_table != nullptr): k_cache is a pool of 64-token pages [page][64][hkv][dk], v_cache_t a
+  // pool [page][hkv][dv][64]; page i of sequence b is block_table[b * max_pages + i]; ctx_cap is unused.
+  // The compressed caches stay contiguous per sequence (1/16 of the K/V).
+  const int32_t* block_table; int max_pages;
 };
 
 int launch_compress(const CompressArgs& a, hipStream_t st);
@@ -128,6 +132,10 @@ int launch_decode(const DecodeArgs& a, hipStream_t st);
 int launch_decode_append(const void* k_new, const void* v_new, void* k_cache, void* v_cache_t, void* ck_cache,
                          void* cv_cache_t, const int32_t* pos, int batch, int hkv, int dk, int dv, int ctx_cap,
                          int nc_cap, int block, int stride, int dtype, hipStream_t st);
+int launch_decode_append_paged(const void* k_new, const void* v_new, void* k_pool, void* v_pool_t,
+                               const int32_t* block_table, int max_pages, void* ck_cache, void* cv_cache_t,
+                               const int32_t* pos, int batch, int hkv, int dk, int dv, int nc_cap, int block,
+                               int stride, int dtype, hipStream_t st);
 int decode_max_nc();
 
 }  // namespace nsa

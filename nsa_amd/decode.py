@@ -65,12 +65,142 @@ class NSADecodeCache:
         self.ctx_lens += 1
 
 
+class NSAPagedDecodeCache:
+    """The same caches with K and V in a pool of 64-token pages shared by all sequences (one page =
+    one selection block of the default configuration), so that sequences of very different lengths
+    do not reserve their maximum.  Layout per page: keys [64, Hkv, Dk] row-major, values
+    [Hkv, Dv, 64] key-contiguous.  block_table[b, i] is the page that holds tokens [64 i, 64 i + 64)
+    of sequence b; unused entries point at page 0, which is never handed out and stays zero.  The
+    compressed caches are small (1/stride of the tokens) and stay contiguous per sequence.
+
+    Page bookkeeping (free list, lengths) lives on the host, so no call here waits for the GPU."""
+
+    PAGE = 64
+
+    def __init__(self, batch, num_pages, max_ctx, hkv, dk, dv, block=32, stride=16, dtype=torch.bfloat16,
+                 device="cuda"):
+        if block > self.PAGE:
+            raise ValueError("the compression block may span at most one page boundary (block <= 64)")
+        self.batch, self.hkv, self.dk, self.dv = batch, hkv, dk, dv
+        self.block, self.stride = block, stride
+        self.max_pages = _round_up(max_ctx, self.PAGE) // self.PAGE
+        self.ctx_cap = self.max_pages * self.PAGE
+        nc = (self.ctx_cap - block) // stride + 1 if self.ctx_cap >= block else 1
+        self.nc_cap = _round_up(nc, 64)
+        z = dict(dtype=dtype, device=device)
+        self.num_pages = num_pages + 1                           # page 0 is the shared all-zero page
+        self.k_pool = torch.zeros(self.num_pages, self.PAGE, hkv, dk, **z)
+        self.v_pool_t = torch.zeros(self.num_pages, hkv, dv, self.PAGE, **z)
+        self.ck = torch.zeros(batch, self.nc_cap, hkv, dk, **z)
+        self.cvt = torch.zeros(batch, hkv, dv, self.nc_cap, **z)
+        self.block_table = torch.zeros(batch, self.max_pages, dtype=torch.int32, device=device)
+        self.ctx_lens = torch.zeros(batch, dtype=torch.int32, device=device)
+        self._free = list(range(self.num_pages - 1, 0, -1))
+        self._pages = [[] for _ in range(batch)]
+        self._lens = [0] * batch
+
+    @property
+    def free_pages(self) -> int:
+        return len(self._free)
+
+    def _grow(self, b: int, new_len: int):
+        """Makes sure sequence b owns pages for new_len tokens; returns the (slot, page) pairs added."""
+        need = (new_len + self.PAGE - 1) // self.PAGE
+        if need > self.max_pages:
+            raise RuntimeError(f"sequence {b} would exceed the cache capacity of {self.ctx_cap} tokens")
+        added = []
+        while len(self._pages[b]) < need:
+            if not self._free:
+                raise RuntimeError("the K/V page pool is exhausted")
+            pg = self._free.pop()
+            added.append((len(self._pages[b]), pg))
+            self._pages[b].append(pg)
+        return added
+
+    def _publish(self, entries):
+        """entries: (sequence, slot, page) triples to write into the device block table."""
+        if not entries:
+            return
+        e = torch.tensor(entries, dtype=torch.int64)
+        self.block_table[e[:, 0].to(self.block_table.device), e[:, 1].to(self.block_table.device)] = \
+            e[:, 2].to(device=self.block_table.device, dtype=torch.int32)
+
+    def release(self, b: int):
+        """Returns the pages of sequence b to the pool and empties it."""
+        self._free.extend(reversed(self._pages[b]))
+        self._pages[b] = []
+        self._lens[b] = 0
+        self.block_table[b].zero_()
+        self.ctx_lens[b] = 0
+
+    @torch.no_grad()
+    def fill(self, k: torch.Tensor, v: torch.Tensor, seq: Optional[int] = None):
+        """Loads a prefilled context.  k [B,T,Hkv,Dk], v [B,T,Hkv,Dv] for every sequence (seq None,
+        B == batch), or k [T,Hkv,Dk], v [T,Hkv,Dv] for sequence `seq` alone."""
+        from . import ops
+        if seq is not None:
+            k, v, seqs = k.unsqueeze(0), v.unsqueeze(0), [seq]
+        else:
+            seqs = list(range(self.batch))
+        B, T = k.shape[:2]
+        entries = []
+        for b in seqs:
+            if self._lens[b]:
+                self.release(b)
+            entries += [(b, slot, pg) for slot, pg in self._grow(b, T)]
+            self._lens[b] = T
+        self._publish(entries)
+        P, Tp = self.PAGE, _round_up(T, self.PAGE)
+        if T > 0:
+            pages = torch.tensor([self._pages[b][:Tp // P] for b in seqs], dtype=torch.int64, device=k.device)
+            kp = torch.zeros(B, Tp, self.hkv, self.dk, dtype=k.dtype, device=k.device)
+            vp = torch.zeros(B, Tp, self.hkv, self.dv, dtype=v.dtype, device=v.device)
+            kp[:, :T], vp[:, :T] = k, v
+            self.k_pool[pages.reshape(-1)] = kp.view(B * (Tp // P), P, self.hkv, self.dk)
+            self.v_pool_t[pages.reshape(-1)] = vp.view(B * (Tp // P), P, self.hkv, self.dv).permute(0, 2, 3, 1)
+        nc = (T - self.block) // self.stride + 1 if T >= self.block else 0
+        sq = torch.tensor(seqs, dtype=torch.int64, device=k.device)
+        if nc > 0:
+            cu = ops.uniform_cu(B, T, k.device)
+            cu_out = ops.uniform_cu(B, nc, k.device)
+            ck = ops.compress(k.reshape(B * T, self.hkv, self.dk).contiguous(), cu, cu_out, B * nc, self.block,
+                              self.stride)
+            cv = ops.compress(v.reshape(B * T, self.hkv, self.dv).contiguous(), cu, cu_out, B * nc, self.block,
+                              self.stride)
+            self.ck[sq, :nc] = ck.view(B, nc, self.hkv, self.dk)
+            self.cvt[sq, :, :, :nc] = cv.view(B, nc, self.hkv, self.dv).permute(0, 2, 3, 1)
+        self.ctx_lens[sq] = T
+
+    @torch.no_grad()
+    def append(self, k_new: torch.Tensor, v_new: torch.Tensor):
+        """k_new [B,Hkv,Dk], v_new [B,Hkv,Dv]: the next token of every sequence."""
+        fresh = sum(self._lens[b] % self.PAGE == 0 for b in range(self.batch))
+        if fresh > len(self._free):
+            raise RuntimeError("the K/V page pool is exhausted")       # before any sequence has grown
+        if max(self._lens) >= self.ctx_cap:
+            raise RuntimeError(f"a sequence would exceed the cache capacity of {self.ctx_cap} tokens")
+        entries = []
+        for b in range(self.batch):
+            entries += [(b, slot, pg) for slot, pg in self._grow(b, self._lens[b] + 1)]
+            self._lens[b] += 1
+        self._publish(entries)
+        pos = self.ctx_lens.clone()
+        k_new, v_new = k_new.contiguous(), v_new.contiguous()
+        rc = _lib.load().nsa_decode_append_paged(_ptr(k_new), _ptr(v_new), _ptr(self.k_pool), _ptr(self.v_pool_t),
+                                                 _ptr(self.block_table), self.max_pages, _ptr(self.ck),
+                                                 _ptr(self.cvt), _ptr(pos), self.batch, self.hkv, self.dk, self.dv,
+                                                 self.nc_cap, self.block, self.stride, _dtype_code(self.k_pool),
+                                                 _stream())
+        _lib.check(rc, "nsa_decode_append_paged")
+        self.ctx_lens += 1
+
+
 @torch.no_grad()
-def nsa_decode_step(q: torch.Tensor, cache: NSADecodeCache, gates: Optional[torch.Tensor] = None,
+def nsa_decode_step(q: torch.Tensor, cache, gates: Optional[torch.Tensor] = None,
                     selection_block: int = 64, selected_block_count: int = 16, sliding_window: int = 512,
                     scale: Optional[float] = None, gate_activation: Optional[str] = None,
                     return_indices: bool = False):
-    """q [B,Hq,Dk]: queries of the newest cached token.  gates [B,Hq,3] (selected, sliding,
+    """q [B,Hq,Dk]: queries of the newest cached token; cache: NSADecodeCache or NSAPagedDecodeCache.  gates [B,Hq,3] (selected, sliding,
     compressed; pre-activation if gate_activation == "sigmoid").  Returns out [B,Hq,Dv]
     (and int32 block indices [B,Hkv,S])."""
     if not q.is_cuda:
@@ -88,6 +218,14 @@ def nsa_decode_step(q: torch.Tensor, cache: NSADecodeCache, gates: Optional[torc
     pool_s = selection_block // cache.stride
     pool_p = cache.block // cache.stride - 2
     act = _lib.GATE_SIGMOID if gate_activation == "sigmoid" else _lib.GATE_IDENTITY
+    if isinstance(cache, NSAPagedDecodeCache):
+        rc = _lib.load().nsa_decode_step_paged(
+            _ptr(q), _ptr(cache.k_pool), _ptr(cache.v_pool_t), _ptr(cache.block_table), cache.max_pages,
+            _ptr(cache.ck), _ptr(cache.cvt), _ptr(cache.ctx_lens), _ptr(gates), _ptr(out), _ptr(idx), B, hq,
+            cache.hkv, dk, cache.dv, cache.nc_cap, cache.block, cache.stride, selection_block, pool_k, pool_s,
+            pool_p, selected_block_count, sliding_window, float(scale), act, _dtype_code(q), _stream())
+        _lib.check(rc, "nsa_decode_step_paged")
+        return (out, idx) if return_indices else out
     rc = _lib.load().nsa_decode_step(
         _ptr(q), _ptr(cache.k), _ptr(cache.vt), _ptr(cache.ck), _ptr(cache.cvt), _ptr(cache.ctx_lens), _ptr(gates),
         _ptr(out), _ptr(idx), B, hq, cache.hkv, dk, cache.dv, cache.ctx_cap, cache.nc_cap, cache.block, cache.stride,

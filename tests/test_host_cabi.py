@@ -165,3 +165,24 @@ def test_training_path_is_taken_only_when_something_requires_grad():
     assert not needs_grad(a, None) and needs_grad(a, b)
     with torch.no_grad():
         assert not needs_grad(a, b)
+
+
+def test_paged_cache_bookkeeping_on_host():
+    """Free list, growth, release and capacity errors of the paged cache need no GPU."""
+    from nsa_amd.decode import NSAPagedDecodeCache
+    c = NSAPagedDecodeCache(2, 5, 200, 1, 64, 64, dtype=torch.float32, device="cpu")
+    assert (c.max_pages, c.ctx_cap, c.free_pages) == (4, 256, 5)
+    assert c._grow(0, 65) == [(0, 1), (1, 2)]
+    assert c._grow(0, 128) == []
+    assert c._grow(1, 1) == [(0, 3)]
+    c._publish([(0, 0, 1), (0, 1, 2), (1, 0, 3)])
+    assert c.block_table.tolist() == [[1, 2, 0, 0], [3, 0, 0, 0]]
+    with pytest.raises(RuntimeError, match="capacity"):
+        c._grow(0, 257)
+    c._grow(1, 192)
+    with pytest.raises(RuntimeError, match="exhausted"):
+        c._grow(0, 192)
+    c.release(1)
+    assert c.free_pages == 3 and c.block_table[1].tolist() == [0, 0, 0, 0]
+    with pytest.raises(ValueError):
+        NSAPagedDecodeCache(1, 4, 256, 1, 64, 64, block=128, device="cpu")
