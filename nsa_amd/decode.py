@@ -171,9 +171,9 @@ class NSAPagedDecodeCache:
             self.cvt[sq, :, :, :nc] = cv.view(B, nc, self.hkv, self.dv).permute(0, 2, 3, 1)
         self.ctx_lens[sq] = T
 
-    @torch.no_grad()
-    def append(self, k_new: torch.Tensor, v_new: torch.Tensor):
-        """k_new [B,Hkv,Dk], v_new [B,Hkv,Dv]: the next token of every sequence."""
+    def reserve_next(self):
+        """Host half of append(): makes sure every sequence owns the page of its next token and
+        publishes new table entries.  Separate so that the device half can live in a captured graph."""
         fresh = sum(self._lens[b] % self.PAGE == 0 for b in range(self.batch))
         if fresh > len(self._free):
             raise RuntimeError("the K/V page pool is exhausted")       # before any sequence has grown
@@ -184,6 +184,10 @@ class NSAPagedDecodeCache:
             entries += [(b, slot, pg) for slot, pg in self._grow(b, self._lens[b] + 1)]
             self._lens[b] += 1
         self._publish(entries)
+
+    @torch.no_grad()
+    def append_reserved(self, k_new: torch.Tensor, v_new: torch.Tensor):
+        """Device half of append(): writes the token (and a compressed row when one completes)."""
         pos = self.ctx_lens.clone()
         k_new, v_new = k_new.contiguous(), v_new.contiguous()
         rc = _lib.load().nsa_decode_append_paged(_ptr(k_new), _ptr(v_new), _ptr(self.k_pool), _ptr(self.v_pool_t),
@@ -193,6 +197,11 @@ class NSAPagedDecodeCache:
                                                  _stream())
         _lib.check(rc, "nsa_decode_append_paged")
         self.ctx_lens += 1
+
+    def append(self, k_new: torch.Tensor, v_new: torch.Tensor):
+        """k_new [B,Hkv,Dk], v_new [B,Hkv,Dv]: the next token of every sequence."""
+        self.reserve_next()
+        self.append_reserved(k_new, v_new)
 
 
 @torch.no_grad()
@@ -233,3 +242,70 @@ def nsa_decode_step(q: torch.Tensor, cache, gates: Optional[torch.Tensor] = None
         _dtype_code(q), _stream())
     _lib.check(rc, "nsa_decode_step")
     return (out, idx) if return_indices else out
+
+
+class NSADecodeGraph:
+    """One decode iteration (cache append of the new token, then the attention step for its query)
+    captured as a HIP graph and replayed per token, so that a serving loop pays one graph launch
+    instead of the launches and allocations of the eager path.  Inputs are copied into fixed
+    buffers; the result is returned as a view of a fixed buffer that the next call overwrites.
+
+    Works on both cache kinds; with a paged cache the page bookkeeping (host only, plus a small
+    table update when a sequence crosses a page boundary) runs before the replay, outside the
+    graph.  The graph holds no memset nodes: the kernels clear what they need themselves."""
+
+    def __init__(self, cache, hq: int, selection_block: int = 64, selected_block_count: int = 16,
+                 sliding_window: int = 512, scale: Optional[float] = None, gate_activation: Optional[str] = None,
+                 use_gates: bool = True, return_indices: bool = False):
+        self.cache = cache
+        self.paged = isinstance(cache, NSAPagedDecodeCache)
+        dt = (cache.k_pool if self.paged else cache.k).dtype
+        dev = cache.ctx_lens.device
+        B = cache.batch
+        self.q = torch.zeros(B, hq, cache.dk, dtype=dt, device=dev)
+        self.k_new = torch.zeros(B, cache.hkv, cache.dk, dtype=dt, device=dev)
+        self.v_new = torch.zeros(B, cache.hkv, cache.dv, dtype=dt, device=dev)
+        self.gates = torch.zeros(B, hq, 3, dtype=dt, device=dev) if use_gates else None
+        self._kw = dict(selection_block=selection_block, selected_block_count=selected_block_count,
+                        sliding_window=sliding_window, scale=scale, gate_activation=gate_activation,
+                        return_indices=return_indices)
+        self.graph = None
+        self.out = self.indices = None
+
+    def _iteration(self):
+        if self.paged:
+            self.cache.append_reserved(self.k_new, self.v_new)
+        else:
+            self.cache.append(self.k_new, self.v_new)
+        r = nsa_decode_step(self.q, self.cache, self.gates, **self._kw)
+        self.out, self.indices = r if self._kw["return_indices"] else (r, None)
+
+    @torch.no_grad()
+    def step(self, q=None, k_new=None, v_new=None, gates=None):
+        """q [B,Hq,Dk], k_new [B,Hkv,Dk], v_new [B,Hkv,Dv] of the next token, gates [B,Hq,3]; None
+        for an operand that the caller has already written into self.q / k_new / v_new / gates."""
+        if self.paged:
+            self.cache.reserve_next()
+        elif int(self.cache.ctx_cap) <= self._host_len():
+            raise RuntimeError(f"a sequence would exceed the cache capacity of {self.cache.ctx_cap} tokens")
+        for buf, src in ((self.q, q), (self.k_new, k_new), (self.v_new, v_new), (self.gates, gates)):
+            if buf is not None and src is not None and src is not buf:
+                buf.copy_(src)       # producers that write into the buffers themselves pass None (or the buffer)
+        if self.graph is None:
+            # the capture itself does not execute, so it stands for no token: replayed below
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                self._iteration()
+            self.graph = g
+        self.graph.replay()
+        self._steps += 1
+        return (self.out, self.indices) if self._kw["return_indices"] else self.out
+
+    _steps = 0
+    _base_len = None
+
+    def _host_len(self) -> int:
+        """Longest sequence, tracked on the host (one read of the device lengths at the first call)."""
+        if self._base_len is None:
+            self._base_len = int(self.cache.ctx_lens.max())
+        return self._base_len + self._steps

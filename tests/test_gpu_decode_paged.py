@@ -108,3 +108,40 @@ def test_paged_append_matches_bulk_fill_and_recycles_pages():
     with pytest.raises(RuntimeError, match="exhausted"):
         for _ in range(200):
             inc.append(k[:, 0], v[:, 0])
+
+
+@pytest.mark.parametrize("paged", [False, True])
+def test_decode_graph_replays_match_eager_steps(paged):
+    """append + step captured once and replayed per token: every replay must equal the eager
+    iteration on a twin cache, with eager work and synchronisations between the replays."""
+    from nsa_amd.decode import NSADecodeCache, NSADecodeGraph, nsa_decode_step
+    B, T0, steps, Hq, Hkv, D = 3, 500, 80, 16, 2, 128
+    dtype = torch.bfloat16
+    k = randn(B, T0 + steps, Hkv, D, seed=730, scale=0.5, dtype=dtype).to(DEV)
+    v = randn(B, T0 + steps, Hkv, D, seed=731, scale=0.5, dtype=dtype).to(DEV)
+    q = randn(steps, B, Hq, D, seed=732, scale=0.5, dtype=dtype).to(DEV)
+    gl = randn(steps, B, Hq, 3, seed=733, dtype=dtype).to(DEV)
+
+    def make():
+        if paged:
+            return _paged(B, B * 10 + 2, T0 + steps, Hkv, D, D, dtype, seed=4)
+        return NSADecodeCache(B, T0 + steps, Hkv, D, D, dtype=dtype, device=DEV)
+
+    ca, cb = make(), make()
+    ca.fill(k[:, :T0], v[:, :T0])
+    cb.fill(k[:, :T0], v[:, :T0])
+    graph = NSADecodeGraph(ca, Hq, 64, 4, 128, gate_activation="sigmoid", return_indices=True)
+    for s in range(steps):
+        out, idx = graph.step(q[s], k[:, T0 + s], v[:, T0 + s], gl[s])
+        cb.append(k[:, T0 + s], v[:, T0 + s])
+        ref, ref_idx = nsa_decode_step(q[s], cb, gl[s], 64, 4, 128, gate_activation="sigmoid", return_indices=True)
+        torch.cuda.synchronize()
+        assert torch.equal(idx, ref_idx), s
+        assert torch.equal(out, ref), s
+    assert torch.equal(ca.ctx_lens, cb.ctx_lens) and int(ca.ctx_lens[0]) == T0 + steps
+    assert torch.equal(ca.ck, cb.ck) and torch.equal(ca.cvt, cb.cvt)
+    if not paged:
+        assert torch.equal(ca.k, cb.k) and torch.equal(ca.vt, cb.vt)
+        with pytest.raises(RuntimeError, match="capacity"):
+            for _ in range(64):
+                graph.step(q[0], k[:, 0], v[:, 0], gl[0])
