@@ -6,7 +6,7 @@ One "step" is one pass of the NSA forward path (compress -> compressed attention
 already resident in HBM.  Prints ONE JSON line.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload prefill_cfg4|prefill_cfg2|prefill_32k_d128]
-                  [--no-cpu-baseline] [--no-decode] [--no-backward]
+                  [--no-cpu-baseline] [--no-decode] [--no-backward] [--no-layer]
 
 roofline: taken for the kernel stage with the largest share of the step; its algorithmic flops
 (causal compressed rows, whole valid selected blocks, exact window; nothing for exp / pooling /
@@ -14,7 +14,8 @@ top-n or for the non-causal part of the importance scores) divided by its mean d
 with events on the launch stream.  cpu_baseline: the CPU oracle (a port of the reference's naive
 torch path) on a bounded sample of query rows of the same workload, on this host's cores.
 train_step (extra, not the headline metric): forward + backward of the same workload through the
-module's autograd path.
+module's autograd path.  layer (extra): the attention layer (projections, rotary embedding, NSA,
+output projection) around the same workload.
 """
 import argparse
 import json
@@ -180,6 +181,44 @@ def train_bench(m, q, k, v, gl, cu, max_len, total, f_eff, steps, warmup):
             "mfma_peak_frac": 3.5 * f_eff / (ms_both * 1e-3) / 1e12 / PEAK_BF16_TFLOPS}
 
 
+def layer_bench(total, hq, hkv, dqk, dv, top_n, window, steps, warmup, hidden=4096, rope_dim=64):
+    """The attention layer around the same workload (extra, not the headline metric): fused q/k/v/gate
+    projection GEMM (hipBLASLt through torch), split + rotary embedding in one HIP pass, NSA forward,
+    output projection.  The split kernel is HBM-bound: bytes = one read and one write of the packed row."""
+    import torch
+    from nsa_amd import ops
+    from nsa_amd.layer import NSAAttentionLayer
+    layer = NSAAttentionLayer(hidden, hq, hkv, dqk, dv, rope_dim=rope_dim, selected_block_count=top_n,
+                              sliding_window=window, compressor_mode="mean", gate_activation="sigmoid",
+                              dtype=torch.bfloat16).cuda()
+    x = torch.randn(1, total, hidden, device="cuda", dtype=torch.bfloat16,
+                    generator=torch.Generator("cuda").manual_seed(11))
+
+    def timed(fn, n):
+        for _ in range(warmup):
+            fn()
+        beg, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        beg.record()
+        for _ in range(n):
+            fn()
+        end.record()
+        torch.cuda.synchronize()
+        return beg.elapsed_time(end) / n
+
+    with torch.no_grad():
+        w, b = layer._fused_cached()
+        packed = torch.nn.functional.linear(x.view(total, hidden), w, b)
+        cu = ops.uniform_cu(1, total, "cuda")
+        ms_split = timed(lambda: ops.qkv_rope_split(packed, hq, hkv, dqk, dv, layer.offsets, layer.inv_freq, None,
+                                                    cu, dqk - rope_dim, rope_dim), steps)
+        ms_layer = timed(lambda: layer(x), steps)
+    nbytes = 2 * 2 * total * (hq * dqk + hkv * dqk + hkv * dv + 3 * hq)
+    return {"hidden": hidden, "rope_dim": rope_dim, "ms_layer_fwd": ms_layer, "tokens_per_s": total / (ms_layer * 1e-3),
+            "ms_split_rope": ms_split, "split_rope_GBps": nbytes / (ms_split * 1e-3) / 1e9,
+            "split_rope_hbm_frac": nbytes / (ms_split * 1e-3) / 1e9 / PEAK_HBM_GBS}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -190,6 +229,7 @@ def main():
     ap.add_argument("--cpu-budget", type=float, default=20.0)
     ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--no-backward", action="store_true")
+    ap.add_argument("--no-layer", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (reference point for FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -287,6 +327,8 @@ def main():
     }
     if not args.no_backward:
         res["train_step"] = train_bench(m, qd, kd, vd, gd, cu, max_len, total, f_eff, max(2, min(args.steps, 5)), 2)
+    if not args.no_layer and len(lens) == 1:
+        res["layer"] = layer_bench(total, hq, hkv, dqk, dv, top_n, window, max(2, min(args.steps, 10)), 2)
     if not args.no_decode:
         del qd, kd, vd, gd, out, idx
         torch.cuda.empty_cache()

@@ -115,6 +115,22 @@ int nsa_block_select_fwd(const void* q, const void* ck, const float* lse, void* 
                          int pool_pad, int top_n, int max_ns, int pooled_stride, int idx64, int dtype,
                          nsa_stream_t stream);
 
+/* Model integration: the glue between a layer's fused q/k/v(/gate) projection GEMM and the kernels
+ * above.  The reference leaves this to its caller (nsa/nsa.py:83-135 receives q, k, v already split and
+ * rotated) and computes the gate logits with a separate Linear (nsa/nsa.py:61,117); here the gating
+ * weights are folded into the projection by the host, and one pass splits the packed GEMM rows
+ *   packed [total][ld] = [ ... q (hq*dk) ... k (hkv*dk) ... v (hkv*dv) ... gate logits (3*hq) ... ]
+ * into q [total][hq][dk], k [total][hkv][dk], v [total][hkv][dv], gates [total][hq][3] (gates may be
+ * NULL), rotating channels [rope_off, rope_off + rope_dim) of every q and k head by the angles
+ * position * inv_freq[i] (inv_freq fp32 [rope_dim/2], NULL = no rotation; interleaved = 0 pairs
+ * channel i with i + rope_dim/2, 1 pairs 2i with 2i+1).  positions int32 [total], or NULL for the
+ * offset inside the sequence given by cu_seqlens.  pack = 1 runs the transpose: gathers gradients
+ * of the four tensors into packed rows with the inverse rotation.  Offsets and ld in elements. */
+int nsa_qkv_rope(void* packed, void* q, void* k, void* v, void* gates, const float* inv_freq,
+                 const int32_t* positions, const int32_t* cu_seqlens, int batch, int64_t total, int ld, int q_off,
+                 int k_off, int v_off, int g_off, int hq, int hkv, int dk, int dv, int rope_off, int rope_dim,
+                 int interleaved, int pack, int dtype, nsa_stream_t stream);
+
 /* Gate logits of the three branches: gates[row][o] = bias[o] + q[row] . weight[o], o = 0 (selected),
  * 1 (sliding window), 2 (compressed).  Replaces the gating nn.Linear(head_dim, 3) of
  * nsa/nsa.py:61 as applied at nsa/nsa.py:117.  q [rows = total*hq, dim], weight [3, dim] (the

@@ -181,3 +181,36 @@ class NSACoreFn(torch.autograd.Function):
                                      delta_swa=st[1], rowscale_slc=st[3], rowscale_swa=st[4])
         dq += dq_c
         return (dq, dck, dcv, dk, dv, d_gl.to(gate_logits.dtype)) + (None,) * 11
+
+
+class QkvRopeFn(torch.autograd.Function):
+    """Packed projection rows -> (q, k, v, gate logits or None) with the rotary embedding on q and k;
+    the backward gathers the four gradients into packed rows with the inverse rotation."""
+
+    @staticmethod
+    def forward(ctx, packed, hq, hkv, dk, dv, offsets, inv_freq, positions, cu, rope_off, rope_dim, interleaved,
+                with_gates):
+        ctx.rows, ctx.like = packed.shape[0], (packed.dtype, packed.device)
+        ctx.meta = (packed.shape[1], offsets, inv_freq, positions, cu, rope_off, rope_dim, interleaved, with_gates,
+                    (hq, hkv, dk, dv))
+        q, k, v, g = ops.qkv_rope_split(packed, hq, hkv, dk, dv, offsets, inv_freq, positions, cu, rope_off, rope_dim,
+                                        interleaved, with_gates)
+        if g is None:
+            return q, k, v
+        return q, k, v, g
+
+    @staticmethod
+    def backward(ctx, dq, dk_, dv_, dg=None):
+        ld, offsets, inv_freq, positions, cu, rope_off, rope_dim, interleaved, with_gates, (hq, hkv, dk, dv) = ctx.meta
+
+        def dense(g, heads, dim):
+            if g is not None:
+                return g
+            return torch.zeros(ctx.rows, heads, dim, dtype=ctx.like[0], device=ctx.like[1])
+
+        dq, dk_, dv_ = dense(dq, hq, dk), dense(dk_, hkv, dk), dense(dv_, hkv, dv)
+        if with_gates:
+            dg = dense(dg, hq, 3)
+        d_packed = ops.qkv_rope_pack(dq, dk_, dv_, dg if with_gates else None, ld, offsets, inv_freq, positions, cu,
+                                     rope_off, rope_dim, interleaved)
+        return (d_packed,) + (None,) * 12

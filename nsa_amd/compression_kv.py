@@ -78,14 +78,16 @@ class KVCompressor(nn.Module):
     mode="conv" is the reference; mode="mean" ignores the parameters and averages each window
     (the conv with eye/block weights and zero bias)."""
 
-    def __init__(self, block_stride, block_size, head_dim, device=None, dtype=None, mode: str = "conv"):
+    def __init__(self, block_stride, block_size, head_dim, device=None, dtype=None, mode: str = "conv",
+                 v_head_dim: Optional[int] = None):
         super().__init__()
         factory_kwargs = {"device": device, "dtype": dtype}
         self.block_stride = block_stride
         self.block_size = block_size
         self.mode = mode
+        v_head_dim = head_dim if v_head_dim is None else v_head_dim     # the reference has one head_dim for both
         self.compressor_k = nn.Conv1d(head_dim, head_dim, block_size, block_stride, **factory_kwargs)
-        self.compressor_v = nn.Conv1d(head_dim, head_dim, block_size, block_stride, **factory_kwargs)
+        self.compressor_v = nn.Conv1d(v_head_dim, v_head_dim, block_size, block_stride, **factory_kwargs)
 
     def _wt(self, conv: nn.Conv1d) -> torch.Tensor:
         # [o, i, j] -> [o, j*D + i]

@@ -161,6 +161,35 @@ int nsa_block_select_fwd(const void* q, const void* ck, const float* lse, void* 
                     pool_stride, pool_pad, top_n, max_ns, pooled_stride, 1.0f, 1, idx64, dtype, stream);
 }
 
+int nsa_qkv_rope(void* packed, void* q, void* k, void* v, void* gates, const float* inv_freq,
+                 const int32_t* positions, const int32_t* cu_seqlens, int batch, int64_t total, int ld, int q_off,
+                 int k_off, int v_off, int g_off, int hq, int hkv, int dk, int dv, int rope_off, int rope_dim,
+                 int interleaved, int pack, int dtype, nsa_stream_t stream) {
+  if (!packed || !q || !k || !v) return fail(NSA_ERR_INVALID, "qkv_rope: null pointer");
+  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "qkv_rope: bad dtype");
+  if (total <= 0 || hq <= 0 || hkv <= 0 || dk <= 0 || dv <= 0 || dk % 8 != 0 || dv % 8 != 0)
+    return fail(NSA_ERR_INVALID, "qkv_rope: sizes must be positive and head dims multiples of 8");
+  if (ld % 8 != 0 || q_off % 8 != 0 || k_off % 8 != 0 || v_off % 8 != 0 || q_off < 0 || k_off < 0 || v_off < 0 ||
+      q_off + hq * dk > ld || k_off + hkv * dk > ld || v_off + hkv * dv > ld)
+    return fail(NSA_ERR_INVALID, "qkv_rope: column offsets and row stride must be multiples of 8 inside the row");
+  if (gates && (g_off < 0 || g_off + 3 * hq > ld)) return fail(NSA_ERR_INVALID, "qkv_rope: gate columns outside the row");
+  if (inv_freq) {
+    if (rope_dim <= 0 || rope_off < 0 || rope_off % 8 != 0 || rope_off + rope_dim > dk ||
+        rope_dim % (interleaved ? 8 : 16) != 0)
+      return fail(NSA_ERR_INVALID, "qkv_rope: rotary channels must be an 8-aligned range inside the head "
+                                   "(length a multiple of 16, or of 8 when interleaved)");
+    if (!positions && (!cu_seqlens || batch <= 0))
+      return fail(NSA_ERR_INVALID, "qkv_rope: needs positions or cu_seqlens");
+  }
+  if (!aligned16(packed) || !aligned16(q) || !aligned16(k) || !aligned16(v))
+    return fail(NSA_ERR_INVALID, "qkv_rope: pointers must be 16-byte aligned");
+  nsa::QkvRopeArgs a{packed, q, k, v, gates, inv_freq, positions, cu_seqlens, batch, (long)total, ld, q_off, k_off,
+                     v_off, g_off, hq, hkv, dk, dv, rope_off, rope_dim, interleaved ? 1 : 0, pack ? 1 : 0, dtype};
+  const int rc = nsa::launch_qkv_rope(a, stream);
+  if (rc == -2) return fail(NSA_ERR_UNSUPPORTED, "qkv_rope: more than 2^31-1 rows, 2^24 row elements or 256 rotary channels");
+  return finish(rc, "qkv_rope");
+}
+
 int nsa_gate_fwd(const void* q, const void* weight, const void* bias, void* gates, int64_t rows, int dim, int dtype,
                  nsa_stream_t stream) {
   if (!q || !weight || !gates) return fail(NSA_ERR_INVALID, "gate: null pointer");

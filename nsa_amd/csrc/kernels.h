@@ -106,6 +106,18 @@ struct DecodeArgs {
   const int32_t* block_table; int max_pages;
 };
 
+// Split of a projection GEMM's packed rows [q | k | v | gate logits] into the attention operands with
+// the rotary embedding applied to q and k (pack == 0), or the reverse gather of their gradients with
+// the inverse rotation (pack == 1).  Column offsets and ld in elements, multiples of 8 except g_off.
+struct QkvRopeArgs {
+  void* packed; void* q; void* k; void* v; void* gates;   // gates may be null
+  const float* inv_freq;                                   // [rope_dim / 2], null = no rotation
+  const int32_t* positions;                                // [total], null = position within the sequence
+  const int32_t* cu_seq; int batch;
+  long total; int ld, q_off, k_off, v_off, g_off, hq, hkv, dk, dv, rope_off, rope_dim, interleaved, pack, dtype;
+};
+int launch_qkv_rope(const QkvRopeArgs& a, hipStream_t st);
+
 int launch_compress(const CompressArgs& a, hipStream_t st);
 int launch_compress_bwd(const CompressBwdArgs& a, hipStream_t st);
 int launch_transpose(const TransposeArgs& a, hipStream_t st);

@@ -22,6 +22,7 @@ class NSAAttention(nn.Module):
     `gating.{weight,bias}`), so its state_dict loads.  Two build-owned switches:
       compressor_mode  "conv" (reference: learned Conv1d) | "mean" (average each window)
       gate_activation  None (reference: raw Linear output) | "sigmoid"
+      v_head_dim       value head size when it differs from head_dim (e.g. 192 / 128)
     Unlike the reference, ragged `cu_seqlens` are honoured (each sequence is attended on its own)."""
 
     def __init__(
@@ -40,6 +41,7 @@ class NSAAttention(nn.Module):
         dtype=None,
         compressor_mode: str = "conv",
         gate_activation: Optional[str] = None,
+        v_head_dim: Optional[int] = None,
     ):
         super().__init__()
         if attention_dropout not in (0, 0.0, None):
@@ -56,7 +58,7 @@ class NSAAttention(nn.Module):
         self.compression_stride = compression_stride
         self.compression_block = compression_block
         self.compressor = KVCompressor(compression_stride, compression_block, head_dim, device, dtype,
-                                       mode=compressor_mode)
+                                       mode=compressor_mode, v_head_dim=v_head_dim)
         self.pool_kernel_size = selection_block // compression_stride + 1
         self.pool_padding = compression_block // compression_stride - 2
         self.pool_stride = selection_block // compression_stride

@@ -457,3 +457,64 @@ def gate_combine_bwd(gate_logits, d_out, o_slc, o_swa, o_cmp, gate_act=0, want_s
                                           _dtype_code(o_slc), _stream())
     _lib.check(rc, "nsa_gate_combine_bwd")
     return (d_slc, d_swa, d_cmp, d_gl, stats) if want_stats else (d_slc, d_swa, d_cmp, d_gl)
+
+
+def _qkv_rope(packed, q, k, v, gates, offsets, inv_freq, positions, cu_seqlens, rope_off, rope_dim, interleaved,
+              pack):
+    total, hq, dk = q.shape
+    hkv, dv = v.shape[1], v.shape[2]
+    q_off, k_off, v_off, g_off = offsets
+    batch = 0 if cu_seqlens is None else cu_seqlens.numel() - 1
+    rc = _lib.load().nsa_qkv_rope(_ptr(packed), _ptr(q), _ptr(k), _ptr(v), _ptr(gates), _ptr(inv_freq),
+                                  _ptr(positions), _ptr(cu_seqlens), batch, total, packed.shape[1], q_off, k_off,
+                                  v_off, g_off, hq, hkv, dk, dv, rope_off, rope_dim, int(bool(interleaved)),
+                                  int(pack), _dtype_code(packed), _stream())
+    _lib.check(rc, "nsa_qkv_rope")
+
+
+def _rope_operands(inv_freq, positions, cu_seqlens, ref):
+    if inv_freq is not None:
+        inv_freq = inv_freq.to(device=ref.device, dtype=torch.float32).contiguous()
+        if positions is not None:
+            positions = positions.to(device=ref.device, dtype=torch.int32).contiguous()
+        elif cu_seqlens is None:
+            raise ValueError("a rotation needs positions or cu_seqlens")
+    if cu_seqlens is not None:
+        cu_seqlens = cu_seqlens.to(device=ref.device, dtype=torch.int32).contiguous()
+    return inv_freq, positions, cu_seqlens
+
+
+def qkv_rope_split(packed, hq, hkv, dk, dv, offsets, inv_freq=None, positions=None, cu_seqlens=None, rope_off=0,
+                   rope_dim=0, interleaved=False, with_gates=True):
+    """packed [total, ld] (a projection GEMM's output: q, k, v and 3*hq gate-logit columns at the
+    element offsets (q_off, k_off, v_off, g_off)) -> q [total,hq,dk], k [total,hkv,dk], v
+    [total,hkv,dv], gates [total,hq,3] or None; channels [rope_off, rope_off+rope_dim) of every q and
+    k head are rotated by position * inv_freq[i] (positions int32 [total], or the offset inside the
+    sequence from cu_seqlens)."""
+    _need_cuda(packed)
+    packed = _dense(packed)
+    total = packed.shape[0]
+    inv_freq, positions, cu_seqlens = _rope_operands(inv_freq, positions, cu_seqlens, packed)
+    z = dict(dtype=packed.dtype, device=packed.device)
+    q, k, v = torch.empty(total, hq, dk, **z), torch.empty(total, hkv, dk, **z), torch.empty(total, hkv, dv, **z)
+    gates = torch.empty(total, hq, 3, **z) if with_gates else None
+    _qkv_rope(packed, q, k, v, gates, offsets, inv_freq, positions, cu_seqlens, rope_off, rope_dim, interleaved, 0)
+    return q, k, v, gates
+
+
+def qkv_rope_pack(dq, dk_, dv_, dgates, ld, offsets, inv_freq=None, positions=None, cu_seqlens=None, rope_off=0,
+                  rope_dim=0, interleaved=False):
+    """Transpose of qkv_rope_split: gradients of q, k, v (and gate logits, or None) -> gradient of the
+    packed rows [total, ld] (columns outside the four ranges are zero), inverse rotation applied."""
+    _need_cuda(dq, dk_, dv_)
+    dq, dk_, dv_ = _dense(dq), _dense(dk_), _dense(dv_)
+    dgates = None if dgates is None else _dense(dgates)
+    inv_freq, positions, cu_seqlens = _rope_operands(inv_freq, positions, cu_seqlens, dq)
+    total, hq, dk = dq.shape
+    hkv, dv = dv_.shape[1], dv_.shape[2]
+    covered = hq * dk + hkv * dk + hkv * dv + (0 if dgates is None else 3 * hq)
+    alloc = torch.empty if covered == ld else torch.zeros
+    packed = alloc(total, ld, dtype=dq.dtype, device=dq.device)
+    _qkv_rope(packed, dq, dk_, dv_, dgates, offsets, inv_freq, positions, cu_seqlens, rope_off, rope_dim,
+              interleaved, 1)
+    return packed

@@ -186,3 +186,55 @@ def test_paged_cache_bookkeeping_on_host():
     assert c.free_pages == 3 and c.block_table[1].tolist() == [0, 0, 0, 0]
     with pytest.raises(ValueError):
         NSAPagedDecodeCache(1, 4, 256, 1, 64, 64, block=128, device="cpu")
+
+
+def test_qkv_rope_argument_errors_do_not_launch(lib):
+    buf = ctypes.create_string_buffer(4096)
+    p = (ctypes.addressof(buf) + 63) // 64 * 64
+    base = dict(packed=p, q=p, k=p, v=p, gates=p, inv_freq=p, positions=None, cu=p, batch=1, total=4, ld=120,
+                q_off=0, k_off=64, v_off=80, g_off=96, hq=4, hkv=1, dk=16, dv=16, rope_off=0, rope_dim=16,
+                interleaved=0, pack=0, dtype=0)
+
+    def call(**kw):
+        a = dict(base, **kw)
+        return lib.nsa_qkv_rope(a["packed"], a["q"], a["k"], a["v"], a["gates"], a["inv_freq"], a["positions"],
+                                a["cu"], a["batch"], a["total"], a["ld"], a["q_off"], a["k_off"], a["v_off"],
+                                a["g_off"], a["hq"], a["hkv"], a["dk"], a["dv"], a["rope_off"], a["rope_dim"],
+                                a["interleaved"], a["pack"], a["dtype"], None)
+
+    for bad in (dict(packed=None), dict(dtype=7), dict(total=0), dict(dk=12), dict(ld=100), dict(k_off=60),
+                dict(v_off=112), dict(g_off=110), dict(rope_dim=8), dict(rope_dim=24, interleaved=1),
+                dict(rope_off=4), dict(rope_off=8, rope_dim=16), dict(cu=None), dict(q=p + 4)):
+        assert call(**bad) == -1, bad
+        assert b"qkv_rope" in lib.nsa_last_error_string()
+
+
+def test_layer_folds_the_gating_linear_into_the_projection():
+    """Pure host arithmetic: the gate columns of the fused GEMM equal gating(q_proj(x)), and the
+    q / k / v columns are the three projections, with and without biases."""
+    from nsa_amd.layer import NSAAttentionLayer
+    torch.manual_seed(0)
+    for bias in (False, True):
+        layer = NSAAttentionLayer(40, 6, 2, qk_head_dim=24, v_head_dim=16, rope_dim=16, bias=bias,
+                                  dtype=torch.float64)
+        w, b = layer.fused_projection()
+        assert w.shape == (layer.ld, 40) and layer.ld % 8 == 0 and layer.ld >= 6 * 24 + 2 * 24 + 2 * 16 + 18
+        x = torch.randn(11, 40, dtype=torch.float64)
+        packed = torch.nn.functional.linear(x, w, b)
+        q = layer.q_proj(x)
+        o = layer.offsets
+        assert torch.allclose(packed[:, :o[1]], q)
+        assert torch.allclose(packed[:, o[1]:o[2]], layer.k_proj(x))
+        assert torch.allclose(packed[:, o[2]:o[3]], layer.v_proj(x))
+        gates = layer.attn.gating(q.view(11, 6, 24))
+        assert torch.allclose(packed[:, o[3]:o[3] + 18].view(11, 6, 3), gates, atol=1e-12)
+        assert (packed[:, o[3] + 18:] == 0).all()
+    names = set(layer.state_dict())
+    assert {"q_proj.weight", "o_proj.weight", "attn.gating.weight", "attn.compressor.compressor_k.weight"} <= names
+    assert layer.attn.compressor.compressor_v.weight.shape[0] == 16
+    with pytest.raises(ValueError):
+        NSAAttentionLayer(40, 6, 4)
+    with pytest.raises(ValueError):
+        NSAAttentionLayer(40, 6, 2, qk_head_dim=24, rope_dim=12)
+    with pytest.raises(NotImplementedError):
+        layer(torch.zeros(1, 4, 40, dtype=torch.float64), attention_mask=torch.ones(1, 4))

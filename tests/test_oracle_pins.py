@@ -355,3 +355,70 @@ def test_oracle_gradients_match_library_attention_on_dense_cases():
                lambda a, b, c: O.selected_attention(a, b, c, idx, None, 4, 0.3, math_dtype=torch.float64)):
         for got, want in zip(grads(fn), ref):
             assert float((got - want).abs().max()) < 1e-10
+
+
+# ------------------------------------------------------------------------------ rotary embedding / layer
+def _rope_inputs(interleaved, seed=0):
+    from oracle import layer_oracle as L
+    g = torch.Generator().manual_seed(seed)
+    T, H, D, off, rd = 37, 3, 48, 16, 32
+    x = torch.randn(T, H, D, generator=g, dtype=torch.float64)
+    pos = torch.randint(0, 5000, (T,), generator=g)
+    inv = 1.0 / (10000.0 ** (torch.arange(0, rd, 2, dtype=torch.float32) / rd))
+    return L, x, pos, inv, off, rd
+
+
+@pytest.mark.parametrize("interleaved", [False, True])
+def test_rope_oracle_is_complex_multiplication(interleaved):
+    """Rotation of a channel pair == multiplication of a + ib by exp(i * angle)."""
+    L, x, pos, inv, off, rd = _rope_inputs(interleaved)
+    y = L.rope_rotate(x, pos, inv, off, rd, interleaved, math_dtype=torch.float64)
+    ang = (pos.float()[:, None] * inv[None, :]).double()
+    unit = torch.polar(torch.ones_like(ang), ang)[:, None, :]
+    r = x[..., off:off + rd]
+    z = torch.complex(r[..., 0::2], r[..., 1::2]) if interleaved else torch.complex(r[..., :rd // 2], r[..., rd // 2:])
+    z = z * unit
+    want = torch.stack([z.real, z.imag], -1).flatten(-2) if interleaved else torch.cat([z.real, z.imag], -1)
+    assert torch.allclose(y[..., off:off + rd], want, atol=1e-12)
+    assert torch.equal(y[..., :off], x[..., :off])
+
+
+def test_rope_oracle_invariants():
+    L, x, pos, inv, off, rd = _rope_inputs(False, seed=1)
+    kw = dict(math_dtype=torch.float64)
+    y = L.rope_rotate(x, pos, inv, off, rd, False, **kw)
+    # the two pairings are the same rotation up to the channel permutation between them
+    perm = torch.arange(rd).view(2, rd // 2).t().reshape(-1)            # half layout -> interleaved layout
+    xi = x.clone()
+    xi[..., off:off + rd] = x[..., off:off + rd][..., perm]
+    yi = L.rope_rotate(xi, pos, inv, off, rd, True, **kw)
+    assert torch.allclose(yi[..., off:off + rd], y[..., off:off + rd][..., perm], atol=1e-12)
+    # position 0 is the identity, norms are preserved, the inverse undoes it
+    assert torch.equal(L.rope_rotate(x, torch.zeros_like(pos), inv, off, rd, False, **kw), x)
+    assert torch.allclose(y.norm(dim=-1), x.norm(dim=-1), atol=1e-12)
+    assert torch.allclose(L.rope_rotate(y, pos, inv, off, rd, False, inverse=True, **kw), x, atol=1e-12)
+    # scores depend on the distance only (dyadic inv_freq and small positions: the fp32 angles are exact)
+    inv2 = 2.0 ** -torch.arange(rd // 2, dtype=torch.float32)
+    q, k = x[:1], x[1:2]
+    def score(m, n):
+        qm = L.rope_rotate(q, torch.tensor([m]), inv2, off, rd, False, **kw)
+        kn = L.rope_rotate(k, torch.tensor([n]), inv2, off, rd, False, **kw)
+        return (qm * kn).sum(-1)
+    assert torch.allclose(score(70, 50), score(25, 5), atol=1e-10)
+    assert not torch.allclose(score(70, 50), score(70, 49), atol=1e-3)
+
+
+def test_layer_oracle_without_rope_is_the_reference_module_on_projected_inputs():
+    """With no rotation the layer oracle is Linear -> (gating on q, NSA forward) -> Linear."""
+    from oracle import layer_oracle as L
+    g = torch.Generator().manual_seed(3)
+    T, hidden, hq, hkv, d = 96, 32, 4, 2, 16
+    x = torch.randn(T, hidden, generator=g)
+    wq, wk, wv = (torch.randn(n * d, hidden, generator=g) * 0.2 for n in (hq, hkv, hkv))
+    wo = torch.randn(hidden, hq * d, generator=g) * 0.2
+    gw, gb = torch.randn(3, d, generator=g), torch.randn(3, generator=g)
+    p = O.NSAParams(8, 4, 16, 2, 16)
+    out = L.layer_forward(x, wq, wk, wv, wo, gw, gb, [0, 60, T], p, hq, hkv, d, d)
+    q, k, v = (F.linear(x, w).view(T, -1, d) for w in (wq, wk, wv))
+    o = O.nsa_forward_varlen(q, k, v, F.linear(q, gw, gb), [0, 60, T], p)
+    assert torch.allclose(out, F.linear(o.reshape(T, -1), wo), atol=1e-5)
