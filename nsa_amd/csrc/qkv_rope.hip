@@ -39,10 +39,37 @@ qkv_rope_kernel(const QkvRopeArgs a) {
   const int ppt = pq + pk + pv + (ng + 7) / 8;
   const long t = blockIdx.x;
   const int p = blockIdx.y * 256 + threadIdx.x;
+  T* prow = reinterpret_cast<T*>(a.packed) + t * a.ld;
+  // 0: nothing, 1: copy, 2: rotate; the loads are issued before the angles are worked out
+  int kind = 0, r = 0;
+  const T* src = nullptr;
+  T* dst = nullptr;
+  vec8_t<T> x = zero8<T>(), xp = zero8<T>();
+  const int half = a.rope_dim / 2;
+  if (p < pq + pk + pv) {
+    T* split;
+    int c, dim, poff;
+    bool rot = a.inv_freq != nullptr;
+    if (p < pq) { split = reinterpret_cast<T*>(a.q) + t * a.hq * a.dk; c = 8 * p; dim = a.dk; poff = a.q_off; }
+    else if (p < pq + pk) { split = reinterpret_cast<T*>(a.k) + t * a.hkv * a.dk; c = 8 * (p - pq); dim = a.dk; poff = a.k_off; }
+    else { split = reinterpret_cast<T*>(a.v) + t * a.hkv * a.dv; c = 8 * (p - pq - pk); dim = a.dv; poff = a.v_off; rot = false; }
+    src = PACK ? split + c : prow + poff + c;
+    dst = PACK ? prow + poff + c : split + c;
+    x = load8(src);
+    r = c % dim - a.rope_off;               // first rotary channel of this piece (multiple of 8)
+    kind = (rot && r >= 0 && r < a.rope_dim) ? 2 : 1;
+    if (kind == 2 && !a.interleaved) xp = load8(src + (r < half ? half : -half));
+  } else if (p < ppt) {                     // gate logits: plain columns, any alignment
+    T* g = reinterpret_cast<T*>(a.gates) + t * ng;
+    const int c0 = 8 * (p - pq - pk - pv);
+    for (int e = 0; e < 8 && c0 + e < ng; ++e) {
+      if (PACK) prow[a.g_off + c0 + e] = g[c0 + e];
+      else g[c0 + e] = prow[a.g_off + c0 + e];
+    }
+  }
   // slices past the q and k pieces hold nothing to rotate
-  const bool rot_block = a.inv_freq != nullptr && blockIdx.y * 256 < pq + pk;
-  if (rot_block) {
-    if (threadIdx.x < a.rope_dim / 2) {
+  if (a.inv_freq != nullptr && blockIdx.y * 256 < pq + pk) {
+    if (threadIdx.x < half) {
       const float pos = (float)position_of(a, t);
       float s, co;
       sincosf(pos * a.inv_freq[threadIdx.x], &s, &co);
@@ -51,28 +78,8 @@ qkv_rope_kernel(const QkvRopeArgs a) {
     }
     __syncthreads();
   }
-  if (p >= ppt) return;
-  T* prow = reinterpret_cast<T*>(a.packed) + t * a.ld;
-  if (p >= pq + pk + pv) {                  // gate logits: plain columns, any alignment
-    T* g = reinterpret_cast<T*>(a.gates) + t * ng;
-    const int c0 = 8 * (p - pq - pk - pv);
-    for (int e = 0; e < 8 && c0 + e < ng; ++e) {
-      if (PACK) prow[a.g_off + c0 + e] = g[c0 + e];
-      else g[c0 + e] = prow[a.g_off + c0 + e];
-    }
-    return;
-  }
-  T* split;
-  int c, dim, poff;
-  bool rot = a.inv_freq != nullptr;
-  if (p < pq) { split = reinterpret_cast<T*>(a.q) + t * a.hq * a.dk; c = 8 * p; dim = a.dk; poff = a.q_off; }
-  else if (p < pq + pk) { split = reinterpret_cast<T*>(a.k) + t * a.hkv * a.dk; c = 8 * (p - pq); dim = a.dk; poff = a.k_off; }
-  else { split = reinterpret_cast<T*>(a.v) + t * a.hkv * a.dv; c = 8 * (p - pq - pk); dim = a.dv; poff = a.v_off; rot = false; }
-  const T* src = PACK ? split + c : prow + poff + c;
-  T* dst = PACK ? prow + poff + c : split + c;
-  const vec8_t<T> x = load8(src);
-  const int r = c % dim - a.rope_off;       // first rotary channel of this piece (multiple of 8)
-  if (!rot || r < 0 || r >= a.rope_dim) {
+  if (kind == 0) return;
+  if (kind == 1) {
     store8(dst, x);
     return;
   }
@@ -86,9 +93,7 @@ qkv_rope_kernel(const QkvRopeArgs a) {
       y[2 * i + 1] = x1 * co + x0 * s;
     }
   } else {
-    const int half = a.rope_dim / 2;
     const bool first = r < half;
-    const vec8_t<T> xp = load8(src + (first ? half : -half));
     const int f0 = first ? r : r - half;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
