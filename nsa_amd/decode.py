@@ -104,14 +104,15 @@ class NSAPagedDecodeCache:
         return len(self._free)
 
     def _grow(self, b: int, new_len: int):
-        """Makes sure sequence b owns pages for new_len tokens; returns the (slot, page) pairs added."""
+        """Makes sure sequence b owns pages for new_len tokens; returns the (slot, page) pairs added.
+        All or nothing: on an error the sequence keeps exactly the pages it had."""
         need = (new_len + self.PAGE - 1) // self.PAGE
         if need > self.max_pages:
             raise RuntimeError(f"sequence {b} would exceed the cache capacity of {self.ctx_cap} tokens")
+        if need - len(self._pages[b]) > len(self._free):
+            raise RuntimeError("the K/V page pool is exhausted")
         added = []
         while len(self._pages[b]) < need:
-            if not self._free:
-                raise RuntimeError("the K/V page pool is exhausted")
             pg = self._free.pop()
             added.append((len(self._pages[b]), pg))
             self._pages[b].append(pg)
@@ -143,6 +144,11 @@ class NSAPagedDecodeCache:
         else:
             seqs = list(range(self.batch))
         B, T = k.shape[:2]
+        if B != len(seqs):
+            raise ValueError(f"fill() got {B} sequences for {len(seqs)} cache slots")
+        held = sum(len(self._pages[b]) for b in seqs)
+        if len(seqs) * ((T + self.PAGE - 1) // self.PAGE) > len(self._free) + held:
+            raise RuntimeError("the K/V page pool is exhausted")       # before any sequence is touched
         entries = []
         for b in seqs:
             if self._lens[b]:

@@ -253,3 +253,18 @@ def test_layer_backward_matches_oracle_autograd(mode, act, rd, lens):
         conv = layer.attn.compressor.compressor_k
         w = comp["wk"].grad
         check("dconv_k.w", conv.weight.grad, w.reshape(-1, dk, dk).permute(2, 1, 0))
+
+
+def test_layer_explicit_position_ids_equal_derived_positions():
+    hidden, hq, hkv, dk, dv, rd = 128, 8, 2, 64, 64, 32
+    layer = _layer(torch.bfloat16, hidden, hq, hkv, dk, dv, rd, "mean", "sigmoid", 2, 32).to(DEV)
+    lens = [200, 1, 90]
+    cu = ragged_cu(lens)
+    x = randn(sum(lens), hidden, seed=860, dtype=torch.bfloat16).to(DEV)
+    cud = torch.tensor(cu, dtype=torch.int32, device=DEV)
+    with torch.no_grad():
+        a, _ = layer(x, cu_seqlens=cud, max_seqlen=max(lens))
+        b, _ = layer(x, cu_seqlens=cud, position_ids=L.positions_from_cu(cu).to(DEV))
+        c, _ = layer(x, cu_seqlens=cud, position_ids=L.positions_from_cu(cu).to(DEV) + 7)
+    assert torch.equal(a, b)
+    assert not torch.equal(a, c)      # content channels make absolute positions matter (rope_dim < head dim)

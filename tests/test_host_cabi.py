@@ -182,6 +182,7 @@ def test_paged_cache_bookkeeping_on_host():
     c._grow(1, 192)
     with pytest.raises(RuntimeError, match="exhausted"):
         c._grow(0, 192)
+    assert len(c._pages[0]) == 2 and c.free_pages == 0          # a failed growth takes nothing
     c.release(1)
     assert c.free_pages == 3 and c.block_table[1].tolist() == [0, 0, 0, 0]
     with pytest.raises(ValueError):
