@@ -194,41 +194,52 @@ stream_attn_kernel(const StreamParams a) {
       const T* ks = bk + 32 * sub * KLD + 8 * g;
       scores32<T, DK, DV, NG>(ks + chunk_key_of_row(0, n) * KLD, ks + chunk_key_of_row(1, n) * KLD, grp, s0, s1);
       vec8_t<T> pb[NG];
+      if constexpr (CMP) {
+        // Scores of all groups first, so that the probe below is one branch per sub-chunk and the
+        // exponentials of the groups are independent straight-line work.
+        float s[NG][8], si[NG];
 #pragma unroll
-      for (int j = 0; j < NG; ++j) {
-        float s[8], p[8];
+        for (int j = 0; j < NG; ++j) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) { s[i] = s0[j][i]; s[4 + i] = s1[j][i]; }
+          for (int i = 0; i < 4; ++i) { s[j][i] = s0[j][i]; s[j][4 + i] = s1[j][i]; }
+        }
         const int key0 = cb + 8 * g;
-        const bool full = cb + 31 <= g_hi_min[j] && (CMP || cb >= g_lo_max[j]);
-        if (CMP) {
-          if (cb + 32 > nkeys) {                       // last chunk of the sequence only
-            asm volatile("" ::: "memory");
+        if (cb + 32 > nkeys) {                         // last chunk of the sequence only
+          asm volatile("" ::: "memory");
+#pragma unroll
+          for (int j = 0; j < NG; ++j)
 #pragma unroll
             for (int i = 0; i < 8; ++i)
-              if (key0 + i >= nkeys) s[i] = kNegInf;
-          }
-          // The raw-score exponentials are needed anyway (importance log-sum-exp), so they double as the
-          // overflow probe: a score more than the slack above the reference makes its exponential, and
-          // with it the lane's sum of 8, exceed 2^slack.  Only then (and on the very first chunk, while
-          // the reference is still -inf) is the maximum taken and the reference moved; the common case
-          // pays neither the 8-way maximum nor its reduction over the column's four lanes.
-          float ei[8], si = 0.f;
-          bool redo = first_sub;
-          if (!first_sub) {
+              if (key0 + i >= nkeys) s[j][i] = kNegInf;
+        }
+        // The raw-score exponentials are needed anyway (importance log-sum-exp), so they double as the
+        // overflow probe: a score more than the slack above the reference makes its exponential, and
+        // with it the lane's sum of 8, exceed 2^slack.  Only then (and on the very first chunk, while
+        // the reference is still -inf) is the maximum taken and the reference moved; the common case
+        // pays neither the 8-way maximum nor its reduction over the column's four lanes.
+        bool redo = first_sub;
+        if (!first_sub) {
+          bool over = false;
+#pragma unroll
+          for (int j = 0; j < NG; ++j) {
             const float off_i = -grp[j].m * kLog2e;
+            float ei[8];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) ei[i] = fast_exp2(fmaf(s[i], kLog2e, off_i));
-            si = sum8(ei);
-            redo = __any(si > cmp_probe);
+            for (int i = 0; i < 8; ++i) ei[i] = fast_exp2(fmaf(s[j][i], kLog2e, off_i));
+            si[j] = sum8(ei);
+            over |= si[j] > cmp_probe;
           }
-          if (redo) {
-            float mx = s[0];
+          redo = __any(over);
+        }
+        if (redo) {
 #pragma unroll
-            for (int i = 1; i < 8; ++i) mx = fmaxf(mx, s[i]);
+          for (int j = 0; j < NG; ++j) {
+            float mx = s[j][0];
+#pragma unroll
+            for (int i = 1; i < 8; ++i) mx = fmaxf(mx, s[j][i]);
             mx = colgroup_max(mx);                     // finite: key cb exists
             const float m_new = fmaxf(grp[j].m, mx);
-            const float d = grp[j].m - m_new;          // -inf on the first chunk
+            const float d = grp[j].m - m_new;          // -inf on the first chunk, 0 when nothing moved
             float beta = fast_exp2(d * kLog2e), alpha = fast_exp2(d * c_attn);
             settle_factor(beta, alpha);
             scale_inplace(li[j], beta);
@@ -237,17 +248,21 @@ stream_attn_kernel(const StreamParams a) {
             for (int t = 0; t < DV / 16; ++t) scale_inplace(grp[j].o[t], alpha);
             grp[j].m = m_new;
             const float off_i = -m_new * kLog2e;
+            float ei[8];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) ei[i] = fast_exp2(fmaf(s[i], kLog2e, off_i));
-            si = sum8(ei);
+            for (int i = 0; i < 8; ++i) ei[i] = fast_exp2(fmaf(s[j][i], kLog2e, off_i));
+            si[j] = sum8(ei);
           }
-          li[j] += si;
-          const float off_a = -grp[j].m * c_attn;
-          if (act[j]) {
+        }
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-              p[i] = fast_exp2(fmaf(s[i], c_attn, off_a));
-            }
+        for (int j = 0; j < NG; ++j) {
+          li[j] += si[j];
+          if (act[j]) {
+            const float off_a = -grp[j].m * c_attn;
+            const bool full = cb + 31 <= g_hi_min[j];
+            float p[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) p[i] = fast_exp2(fmaf(s[j][i], c_attn, off_a));
             if (!full) {                               // the one or two chunks on the causal edge
               asm volatile("" ::: "memory");
 #pragma unroll
@@ -259,7 +274,15 @@ stream_attn_kernel(const StreamParams a) {
           } else {
             pb[j] = zero8<T>();
           }
-        } else {
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < NG; ++j) {
+          float s[8], p[8];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) { s[i] = s0[j][i]; s[4 + i] = s1[j][i]; }
+          const int key0 = cb + 8 * g;
+          const bool full = cb + 31 <= g_hi_min[j] && cb >= g_lo_max[j];
           if (act[j]) {
             if (!full) {                               // window edges
               asm volatile("" ::: "memory");
