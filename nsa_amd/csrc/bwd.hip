@@ -52,13 +52,25 @@ struct BwdArgs {
   SlcWs ws;                       // selected branch: bucketed pairs; ws.po = dq partials [pair][16][dk]
 };
 
-// Two 16-row tiles of X[32 rows][D] (LDS, permuted rows) times the stationary fragments f[D/32].
-template <typename T, int D>
+// Two LDS layouts of a 32-row chunk.  X32: rows padded by 32 bytes, row ownership of lane_row32; no bank
+// conflicts on either kind of read.  Otherwise: rows padded by 8 elements, lane group g owns rows 8g .. 8g+7
+// (two-way conflicts on most reads).  The selected-block mode keeps the second one: it is bound by its global
+// traffic, and with the first layout it measured 5 % slower although its LDS time halved.
+template <typename T, bool X32> constexpr int kLdsPad = X32 ? 32 / (int)sizeof(T) : 8;
+template <bool X32> __device__ __forceinline__ int chunk_row(int g, int j) { return X32 ? lane_row32(g, j) : 8 * g + j; }
+template <bool X32, typename T> __device__ __forceinline__ vec8_t<T> chunk_tr(const T* tile, int ld, int lane) {
+  if constexpr (X32) return load8_tr32(tile, ld, lane);
+  else return load8_tr(tile, ld, lane);
+}
+
+// Two 16-row tiles of X[32 rows][D] (LDS) times the stationary fragments f[D/32]; lane group g receives the
+// rows lane_row32(g, 0..7).
+template <typename T, int D, bool X32>
 __device__ __forceinline__ void tile_pair(const T* __restrict__ x, int ld, int n, int g, const vec8_t<T> (&f)[D / 32],
                                           float (&out)[8]) {
   f32x4_t t0 = {0.f, 0.f, 0.f, 0.f}, t1 = {0.f, 0.f, 0.f, 0.f};
-  const T* r0 = x + chunk_key_of_row(0, n) * ld + 8 * g;
-  const T* r1 = x + chunk_key_of_row(1, n) * ld + 8 * g;
+  const T* r0 = x + (X32 ? tile_row32(0, n) : chunk_key_of_row(0, n)) * ld + 8 * g;
+  const T* r1 = r0 + (X32 ? 8 : 4) * ld;
 #pragma unroll
   for (int kk = 0; kk < D / 32; ++kk) {
     t0 = mma16(load8(r0 + 32 * kk), f[kk], t0);
@@ -89,7 +101,8 @@ __device__ __forceinline__ void store4(float* p, const f32x4_t& v, float s) {
 template <typename T, int DK, int DV, int MODE, int NW>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 bwd_kv_kernel(const BwdArgs a) {
-  constexpr int QLD = DK + 8, OLD = DV + 8, NT = NW * 64, SLD = kBlk + 8;
+  constexpr bool X32 = MODE != kBwdSlc;
+  constexpr int QLD = DK + kLdsPad<T, X32>, OLD = DV + kLdsPad<T, X32>, NT = NW * 64, SLD = kBlk + 8;
   constexpr int QP = 32 * DK / 8, OP = 32 * DV / 8;                 // 16-byte pieces of one chunk
   constexpr int QPT = (QP + NT - 1) / NT, OPT = (OP + NT - 1) / NT;
   constexpr int STAGE = 32 * QLD + 32 * OLD;
@@ -254,7 +267,7 @@ bwd_kv_kernel(const BwdArgs a) {
     const float* ss = stat + buf * 64;
     int posA, posB; bool vB;
     chunk_tokens(c, posA, posB, vB);
-    // the 8 rows of this lane (8g .. 8g+7) are heads 8(g&1) .. +7 of one token
+    // the 8 rows of this lane (chunk_row(g, 0..7)) are heads of one token
     const int tokpos = (g >> 1) ? posB : posA;
     bool vis = keyvalid && ((g >> 1) == 0 || vB);
     if (MODE == kBwdSwa) vis = vis && keypos <= tokpos && keypos > tokpos - a.window;
@@ -262,18 +275,18 @@ bwd_kv_kernel(const BwdArgs a) {
     else if (a.causal) vis = vis && keypos * a.stride + a.block <= tokpos;
 
     float s[8], dp[8], p[8], ds[8];
-    tile_pair<T, DK>(qs, QLD, n, g, kf, s);
-    tile_pair<T, DV>(os, OLD, n, g, vf, dp);
-    const f32x4_t l0 = *reinterpret_cast<const f32x4_t*>(ss + 8 * g);
-    const f32x4_t l1 = *reinterpret_cast<const f32x4_t*>(ss + 8 * g + 4);
-    const f32x4_t e0 = *reinterpret_cast<const f32x4_t*>(ss + 32 + 8 * g);
-    const f32x4_t e1 = *reinterpret_cast<const f32x4_t*>(ss + 32 + 8 * g + 4);
-    const int hbase = 8 * (g & 1);
+    tile_pair<T, DK, X32>(qs, QLD, n, g, kf, s);
+    tile_pair<T, DV, X32>(os, OLD, n, g, vf, dp);
+    const int rlo = chunk_row<X32>(g, 0), rhi = chunk_row<X32>(g, 4);
+    const f32x4_t l0 = *reinterpret_cast<const f32x4_t*>(ss + rlo);
+    const f32x4_t l1 = *reinterpret_cast<const f32x4_t*>(ss + rhi);
+    const f32x4_t e0 = *reinterpret_cast<const f32x4_t*>(ss + 32 + rlo);
+    const f32x4_t e1 = *reinterpret_cast<const f32x4_t*>(ss + 32 + rhi);
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const float lse2 = j < 4 ? l0[j & 3] : l1[j & 3];
       const float dl = j < 4 ? e0[j & 3] : e1[j & 3];
-      const bool ok = vis && hbase + j < G;
+      const bool ok = vis && (chunk_row<X32>(g, j) & 15) < G;
       const float e = fast_exp2(fmaf(s[j], c_attn, -lse2));
       p[j] = ok ? e : 0.f;
       ds[j] = ok ? e * (dp[j] - dl) : 0.f;
@@ -281,13 +294,13 @@ bwd_kv_kernel(const BwdArgs a) {
     const vec8_t<T> pb = pack8<T>(p), dsb = pack8<T>(ds);
     if (MODE == kBwdSlc) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) dsl[(8 * g + j) * SLD + 16 * wave + n] = dsb[j];
+      for (int j = 0; j < 8; ++j) dsl[chunk_row<X32>(g, j) * SLD + 16 * wave + n] = dsb[j];
       __syncthreads();
     }
 #pragma unroll
-    for (int t = 0; t < DV / 16; ++t) dv_acc[t] = mma16(load8_tr(os + 16 * t, OLD, lane), pb, dv_acc[t]);
+    for (int t = 0; t < DV / 16; ++t) dv_acc[t] = mma16(chunk_tr<X32>(os + 16 * t, OLD, lane), pb, dv_acc[t]);
 #pragma unroll
-    for (int t = 0; t < DK / 16; ++t) dk_acc[t] = mma16(load8_tr(qs + 16 * t, QLD, lane), dsb, dk_acc[t]);
+    for (int t = 0; t < DK / 16; ++t) dk_acc[t] = mma16(chunk_tr<X32>(qs + 16 * t, QLD, lane), dsb, dk_acc[t]);
 
     if (MODE == kBwdSlc) {
       // dQ^T[dk][row] = sum_key K[key][dk] dS[row][key]: this wavefront takes every NW-th 16-channel tile
@@ -347,7 +360,7 @@ bwd_kv_kernel(const BwdArgs a) {
 template <typename T, int DK, int DV, int MODE, int NW>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(4, 4)))
 bwd_q_kernel(const BwdArgs a) {
-  constexpr int KLD = DK + 8, VLD = DV + 8, NT = NW * 64;
+  constexpr int KLD = DK + kLdsPad<T, true>, VLD = DV + kLdsPad<T, true>, NT = NW * 64;
   constexpr int KP = 32 * DK / 8, VP = 32 * DV / 8;
   constexpr int KPT = (KP + NT - 1) / NT, VPT = (VP + NT - 1) / NT;
   constexpr int STAGE = 32 * KLD + 32 * VLD;
@@ -456,18 +469,18 @@ bwd_q_kernel(const BwdArgs a) {
       const T* ks = lds + buf * STAGE;
       const T* vs = ks + 32 * KLD;
       float s[8], dp[8], ds[8];
-      tile_pair<T, DK>(ks, KLD, n, g, qf, s);
-      tile_pair<T, DV>(vs, VLD, n, g, dof, dp);
+      tile_pair<T, DK, true>(ks, KLD, n, g, qf, s);
+      tile_pair<T, DV, true>(vs, VLD, n, g, dof, dp);
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        const int key = c0 + 8 * g + j;
+        const int key = c0 + lane_row32(g, j);
         const bool ok = key >= my_lo && key <= my_hi && n < G;
         const float e = fast_exp2(fmaf(s[j], c_attn, -lse2));
         ds[j] = ok ? e * (dp[j] - dl) : 0.f;
       }
       const vec8_t<T> dsb = pack8<T>(ds);
 #pragma unroll
-      for (int t = 0; t < DK / 16; ++t) acc[t] = mma16(load8_tr(ks + 16 * t, KLD, lane), dsb, acc[t]);
+      for (int t = 0; t < DK / 16; ++t) acc[t] = mma16(load8_tr32(ks + 16 * t, KLD, lane), dsb, acc[t]);
     }
     if (has_next) lstore(buf ^ 1);
     __syncthreads();
@@ -557,8 +570,9 @@ slc_dq_merge_kernel(const int* __restrict__ slotmap, const T* __restrict__ part,
 
 template <typename T, int DK, int DV, int MODE, int NW>
 static int launch_kv_t(const BwdArgs& a, int key_rows, hipStream_t st) {
-  size_t smem = 2 * (size_t)(32 * (DK + 8) + 32 * (DV + 8)) * sizeof(T) + 128 * sizeof(float);
-  if (MODE == kBwdSlc) smem += ((size_t)kBlk * (DK + 8) + 32 * (kBlk + 8)) * sizeof(T);
+  constexpr int XP = kLdsPad<T, MODE != kBwdSlc>;
+  size_t smem = 2 * (size_t)(32 * (DK + XP) + 32 * (DV + XP)) * sizeof(T) + 128 * sizeof(float);
+  if (MODE == kBwdSlc) smem += ((size_t)kBlk * (DK + XP) + 32 * (kBlk + 8)) * sizeof(T);
   auto fn = bwd_kv_kernel<T, DK, DV, MODE, NW>;
   const int rc = set_smem(reinterpret_cast<const void*>(fn), smem);
   if (rc) return rc;
@@ -573,7 +587,7 @@ static int launch_kv_t(const BwdArgs& a, int key_rows, hipStream_t st) {
 template <typename T, int DK, int DV, int MODE>
 static int launch_q_t(const BwdArgs& a, hipStream_t st) {
   constexpr int NW = kQWaves;
-  const size_t smem = 2 * (size_t)(32 * (DK + 8) + 32 * (DV + 8)) * sizeof(T);
+  const size_t smem = 2 * (size_t)(32 * (DK + kLdsPad<T, true>) + 32 * (DV + kLdsPad<T, true>)) * sizeof(T);
   auto fn = bwd_q_kernel<T, DK, DV, MODE, NW>;
   const int rc = set_smem(reinterpret_cast<const void*>(fn), smem);
   if (rc) return rc;

@@ -81,6 +81,36 @@ __device__ __forceinline__ f32x8_t load8_tr(const float* tile, int ld, int lane)
   return r;
 }
 
+// Row of a 32-row LDS tile behind value j (0..7) of lane group g (lane / 16) wherever a 32-row tile feeds
+// two products, once row-major (rows = MFMA rows, two 16-row tiles) and once transposed (rows = depth):
+// group g owns rows {b, .., b+3} and {b+8, .., b+11} with b = 4 (g & 1) + 16 (g >> 1).  With rows padded by
+// 32 bytes both kinds of read are free of bank conflicts: the row-major tiles are rows {0..7, 16..23} and
+// {8..15, 24..31}, and each half-wavefront's transposing read touches 8 rows that differ modulo 8.
+__device__ __forceinline__ int lane_row32(int g, int j) { return 4 * (g & 1) + 16 * (g >> 1) + j + 4 * (j >> 2); }
+// LDS row read by MFMA row m of row-major tile `tile` (0/1) of such a 32-row tile.
+__device__ __forceinline__ int tile_row32(int tile, int m) { return m + 8 * (m >> 3) + 8 * tile; }
+
+// The transposing read for that row ownership: lane (g, m) receives tile[lane_row32(g, j)][m], j = 0..7.
+__device__ __forceinline__ bf16x8_t load8_tr32(const bf16_t* tile, int ld, int lane) {
+  typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
+  typedef __attribute__((address_space(3))) bf16x4_t lds_bf16x4_t;
+  const int i = lane & 15, g = lane >> 4;
+  const bf16_t* p = tile + (4 * (g & 1) + 16 * (g >> 1) + (i >> 2)) * ld + 4 * (i & 3);
+  const bf16x4_t a = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_t*)p);
+  const bf16x4_t b = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_t*)(p + 8 * ld));
+  bf16x8_t r;
+  r[0] = a[0]; r[1] = a[1]; r[2] = a[2]; r[3] = a[3];
+  r[4] = b[0]; r[5] = b[1]; r[6] = b[2]; r[7] = b[3];
+  return r;
+}
+__device__ __forceinline__ f32x8_t load8_tr32(const float* tile, int ld, int lane) {
+  const int m = lane & 15, g = lane >> 4;
+  f32x8_t r;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) r[j] = tile[lane_row32(g, j) * ld + m];
+  return r;
+}
+
 struct RowMap {
   int tok;      // token of this lane's column (sequence local), may be >= len
   int gidx;     // head inside the GQA group, may be >= G
