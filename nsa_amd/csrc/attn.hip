@@ -39,7 +39,7 @@ struct StreamParams {
 template <typename T, int DK, int DV, int NG, int CH, int NW, bool CMP, int MERGE = 0>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 stream_attn_kernel(const StreamParams a) {
-  constexpr int KLD = DK + 8, VLD = CH + 8, ROWS = NW * NG * 16, NT = NW * 64;
+  constexpr int KLD = DK + kLdsRowPad<T>, VLD = CH + kLdsRowPad<T>, ROWS = NW * NG * 16, NT = NW * 64;
   constexpr int KPIECES = CH * DK / 8, VPIECES = DV * CH / 8;
   constexpr int KPT = (KPIECES + NT - 1) / NT, VPT = (VPIECES + NT - 1) / NT;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -156,7 +156,18 @@ stream_attn_kernel(const StreamParams a) {
 #pragma unroll
       for (int i = 0; i < VPT; ++i) {
         const int p = tid + i * NT;
-        if (VPIECES % NT == 0 || p < VPIECES) store8(dv + (p / (CH / 8)) * VLD + (p % (CH / 8)) * 8, vr[i]);
+        if (VPIECES % NT == 0 || p < VPIECES) {
+          // keys 16..31 of every 32-key sub-chunk: the two 4-key halves trade places (see lds_key_of_row)
+          const int pc = p % (CH / 8);
+          vec8_t<T> x = vr[i];
+          if (pc & 2) {
+            vec8_t<T> y;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) y[e] = x[e ^ 4];
+            x = y;
+          }
+          store8(dv + (p / (CH / 8)) * VLD + pc * 8, x);
+        }
       }
     }
   };
@@ -192,7 +203,8 @@ stream_attn_kernel(const StreamParams a) {
       if (!CMP && !any_act) continue;
       f32x4_t s0[NG], s1[NG];
       const T* ks = bk + 32 * sub * KLD + 8 * g;
-      scores32<T, DK, DV, NG>(ks + chunk_key_of_row(0, n) * KLD, ks + chunk_key_of_row(1, n) * KLD, grp, s0, s1);
+      scores32<T, DK, DV, NG>(ks + lds_key_of_row(0, n) * KLD, ks + lds_key_of_row(1, n) * KLD, grp, s0, s1);
+      const int swp = lds_key_swap(g);       // value i of this lane belongs to key cb + 8g + (i ^ swp)
       vec8_t<T> pb[NG];
       if constexpr (CMP) {
         // Scores of all groups first, so that the probe below is one branch per sub-chunk and the
@@ -210,7 +222,7 @@ stream_attn_kernel(const StreamParams a) {
           for (int j = 0; j < NG; ++j)
 #pragma unroll
             for (int i = 0; i < 8; ++i)
-              if (key0 + i >= nkeys) s[j][i] = kNegInf;
+              if (key0 + (i ^ swp) >= nkeys) s[j][i] = kNegInf;
         }
         // The raw-score exponentials are needed anyway (importance log-sum-exp), so they double as the
         // overflow probe: a score more than the slack above the reference makes its exponential, and
@@ -267,7 +279,7 @@ stream_attn_kernel(const StreamParams a) {
               asm volatile("" ::: "memory");
 #pragma unroll
               for (int i = 0; i < 8; ++i)
-                if (key0 + i > hi[j]) p[i] = 0.f;
+                if (key0 + (i ^ swp) > hi[j]) p[i] = 0.f;
             }
             grp[j].l += sum8(p);
             pb[j] = pack8<T>(p);
@@ -288,7 +300,7 @@ stream_attn_kernel(const StreamParams a) {
               asm volatile("" ::: "memory");
 #pragma unroll
               for (int i = 0; i < 8; ++i)
-                if (!(key0 + i <= hi[j] && key0 + i >= lo[j])) s[i] = kNegInf;
+                if (!(key0 + (i ^ swp) <= hi[j] && key0 + (i ^ swp) >= lo[j])) s[i] = kNegInf;
             }
             softmax_update(grp[j], s, c_attn, p);
             pb[j] = pack8<T>(p);
@@ -547,7 +559,7 @@ static int launch_stream_t(const StreamParams& a, int total, hipStream_t st) {
   constexpr int NG = StreamTile<T, CMP>::NG, CH = StreamTile<T, CMP>::CH, NW = StreamTile<T, CMP>::NW;
   const int Gp = group_pow2(a.hq / a.hkv);
   const int TQ = NW * NG * 16 / Gp;
-  const size_t smem = 2 * ((size_t)CH * (DK + 8) + (size_t)DV * (CH + 8)) * sizeof(T);
+  const size_t smem = 2 * ((size_t)CH * (DK + kLdsRowPad<T>) + (size_t)DV * (CH + kLdsRowPad<T>)) * sizeof(T);
   auto fn = stream_attn_kernel<T, DK, DV, NG, CH, NW, CMP, MERGE>;
   const int rc = set_smem(reinterpret_cast<const void*>(fn), smem);
   if (rc) return rc;

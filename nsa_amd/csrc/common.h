@@ -89,6 +89,17 @@ __device__ __forceinline__ int chunk_key_of_row(int tile, int m) {
   return 8 * (m >> 2) + (m & 3) + 4 * tile;
 }
 
+// LDS tiles: rows are padded by 32 bytes, which spreads 16 consecutive rows (and the row sets below) over
+// all banks for 16-byte reads; a padding of 16 bytes costs a second pass on most reads.
+template <typename T> constexpr int kLdsRowPad = 32 / (int)sizeof(T);
+// The same map for a chunk staged in LDS: lane groups 2 and 3 (m >= 8) take their two tiles in the
+// opposite order, so that the 16 rows of one tile are distinct modulo 16 (no bank conflicts).  Value i
+// (0..7, tile 0 first) of lane group g then belongs to key 8g + (i ^ lds_key_swap(g)).
+__device__ __forceinline__ int lds_key_of_row(int tile, int m) {
+  return 8 * (m >> 2) + (m & 3) + 4 * (tile ^ (m >> 3));
+}
+__device__ __forceinline__ int lds_key_swap(int g) { return (g >> 1) << 2; }
+
 // All-reduce over the four lanes that share one tile column (lane%16): lanes n, n+16, n+32, n+48.
 // v_permlane16_swap exchanges the odd 16-lane rows of one operand with the even rows of the other,
 // v_permlane32_swap the upper half of one with the lower half of the other; fed the same value

@@ -17,7 +17,7 @@ namespace nsa {
 template <typename T, int DK, int NG, int CH, int NW>
 __global__ void __launch_bounds__(NW * 64)
 importance_select_kernel(const CmpArgs a) {
-  constexpr int KLD = DK + 8, ROWS = NW * NG * 16, NT = NW * 64;
+  constexpr int KLD = DK + kLdsRowPad<T>, ROWS = NW * NG * 16, NT = NW * 64;
   constexpr int KPIECES = CH * DK / 8;
   constexpr int KPT = (KPIECES + NT - 1) / NT;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -231,7 +231,7 @@ __device__ __forceinline__ float row_reduce_scatter4(float v0, float v1, float v
 template <typename T, int DK, int NG, int NW>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(4, 4)))
 importance_stream_kernel(const CmpArgs a) {
-  constexpr int CH = 64, KLD = DK + 8, NT = NW * 64, TQ = NW * NG;
+  constexpr int CH = 64, KLD = DK + kLdsRowPad<T>, NT = NW * 64, TQ = NW * NG;
   constexpr int KPIECES = CH * DK / 8;
   constexpr int KPT = (KPIECES + NT - 1) / NT;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -468,7 +468,7 @@ static int launch_select_ng(const CmpArgs& a, hipStream_t st) {
   constexpr int CH = 32, NW = 4;
   const int Gp = group_pow2(a.hq / a.hkv);
   const int TQ = NW * NG * 16 / Gp;
-  const size_t smem = 2 * (size_t)CH * (DK + 8) * sizeof(T) + (size_t)TQ * a.max_ns * sizeof(float);
+  const size_t smem = 2 * (size_t)CH * (DK + kLdsRowPad<T>) * sizeof(T) + (size_t)TQ * a.max_ns * sizeof(float);
   if (smem > 160 * 1024) return -3;
   auto fn = importance_select_kernel<T, DK, NG, CH, NW>;
   const int rc = set_smem(reinterpret_cast<const void*>(fn), smem);
@@ -489,7 +489,7 @@ static int launch_select_ng(const CmpArgs& a, hipStream_t st) {
 template <typename T, int DK>
 static int launch_select_stream(const CmpArgs& a, hipStream_t st) {
   constexpr int NW = NSA_STREAM_NW, NG = sizeof(T) == 2 ? NSA_STREAM_NG : NSA_STREAM_NG / 2, TQ = NW * NG;
-  const size_t smem = 2 * (size_t)64 * (DK + 8) * sizeof(T);
+  const size_t smem = 2 * (size_t)64 * (DK + kLdsRowPad<T>) * sizeof(T);
   auto fn = importance_stream_kernel<T, DK, NG, NW>;
   const int rc = set_smem(reinterpret_cast<const void*>(fn), smem);
   if (rc) return rc;
