@@ -133,10 +133,11 @@ decode_step_kernel(const DecodeArgs a) {
   const int n = lane & 15, g = lane >> 4;
   const int b = blockIdx.x / a.hkv, h = blockIdx.x % a.hkv;
   const int G = a.hq / a.hkv;
-  const int ctx = a.ctx_lens[b];
+  // a length beyond the cache would index past the K/V rows (or the page table): clamp it
+  const int ctx = min(a.ctx_lens[b], PAGED ? a.max_pages * 64 : a.ctx_cap);
   if (ctx <= 0) return;
   const int t = ctx - 1;
-  const int Nc = ctx >= a.block ? (ctx - a.block) / a.stride + 1 : 0;
+  const int Nc = ctx >= a.block ? min((ctx - a.block) / a.stride + 1, a.nc_cap) : 0;
   int Ns = 0;
   if (Nc > 0 && Nc + 2 * a.pool_p >= a.pool_k) {
     Ns = (Nc + 2 * a.pool_p - a.pool_k + a.pool_s - 1) / a.pool_s + 1;
