@@ -277,6 +277,8 @@ class NSADecodeGraph:
                         return_indices=return_indices)
         self.graph = None
         self.out = self.indices = None
+        self._steps = 0             # tokens appended through this object
+        self._base_len = None       # longest sequence at the first call (read from the device once)
 
     def _iteration(self):
         if self.paged:
@@ -307,11 +309,9 @@ class NSADecodeGraph:
         self._steps += 1
         return (self.out, self.indices) if self._kw["return_indices"] else self.out
 
-    _steps = 0
-    _base_len = None
-
     def _host_len(self) -> int:
-        """Longest sequence, tracked on the host (one read of the device lengths at the first call)."""
+        """Longest sequence, tracked on the host (one read of the device lengths at the first call;
+        appends made behind this object's back are not seen)."""
         if self._base_len is None:
             self._base_len = int(self.cache.ctx_lens.max())
         return self._base_len + self._steps
