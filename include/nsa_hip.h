@@ -291,6 +291,19 @@ int nsa_decode_append_paged(const void* k_new, const void* v_new, void* k_pool, 
                             const int32_t* pos, int batch, int hkv, int dk, int dv, int nc_cap, int block, int stride,
                             int dtype, nsa_stream_t stream);
 
+/* The same step for small batches: the work of every (sequence, kv head) pair is spread over `splits`
+ * workgroups (three launches: compressed slices, selection + window / selected chunks, merge), because one
+ * workgroup per pair leaves most of the chip idle below ~128 pairs.  block_table NULL = contiguous caches
+ * (ctx_cap used), else the paged pool (max_pages used).  Pooling 5 / 4 / 0 only.  The workspace holds
+ * partial results only; calls that share it must not overlap.  No counterpart in the reference. */
+int64_t nsa_decode_split_workspace_bytes(int batch, int hkv, int dv, int nc_cap, int splits);
+int nsa_decode_step_split(const void* q, const void* k_cache, const void* v_cache_t, const int32_t* block_table,
+                          int max_pages, const void* ck_cache, const void* cv_cache_t, const int32_t* ctx_lens,
+                          const void* gates, void* out, int32_t* indices, int batch, int hq, int hkv, int dk, int dv,
+                          int ctx_cap, int nc_cap, int block, int stride, int sel_block, int pool_kernel,
+                          int pool_stride, int pool_pad, int top_n, int window, float scale, int gate_act, int dtype,
+                          int splits, void* workspace, int64_t workspace_bytes, nsa_stream_t stream);
+
 /* Appends one token per sequence: k_new [batch][hkv][dk] -> row pos[b] of k_cache, v_new
  * [batch][hkv][dv] -> column pos[b] of v_cache_t, and, when pos[b]+1 completes a compression block,
  * the mean of the last `block` tokens as the next row / column of the compressed caches. */

@@ -430,7 +430,8 @@ static int decode_common(const char* what, const void* q, const void* k_cache, c
                          const int32_t* ctx_lens, const void* gates, void* out, int32_t* indices, int batch, int hq,
                          int hkv, int dk, int dv, int ctx_cap, int nc_cap, int block, int stride, int sel_block,
                          int pool_kernel, int pool_stride, int pool_pad, int top_n, int window, float scale,
-                         int gate_act, int dtype, nsa_stream_t stream) {
+                         int gate_act, int dtype, nsa_stream_t stream, int splits = 0, void* workspace = nullptr,
+                         int64_t workspace_bytes = 0) {
   if (!q || !k_cache || !v_cache_t || !ck_cache || !cv_cache_t || !ctx_lens || !out)
     return fail(NSA_ERR_INVALID, "%s: null pointer", what);
   if (batch <= 0 || ctx_cap <= 0 || nc_cap <= 0 || block <= 0 || stride <= 0 || window < 0)
@@ -450,9 +451,42 @@ static int decode_common(const char* what, const void* q, const void* k_cache, c
   nsa::DecodeArgs a{q, k_cache, v_cache_t, ck_cache, cv_cache_t, ctx_lens, gates, out, indices, batch, hq, hkv, dk, dv,
                     ctx_cap, nc_cap, block, stride, sel_block, pool_kernel, pool_stride, pool_pad, top_n, window, scale,
                     gate_act, dtype, block_table, max_pages};
+  if (splits > 0) {
+    if (splits > 16) return fail(NSA_ERR_INVALID, "%s: at most 16 splits", what);
+    if (pool_kernel != 5 || pool_stride != 4 || pool_pad != 0)
+      return fail(NSA_ERR_UNSUPPORTED, "%s: the split step is built for pooling windows of 5 every 4 without padding", what);
+    if (top_n > 64) return fail(NSA_ERR_UNSUPPORTED, "%s: at most 64 selected blocks", what);
+    if (!workspace || !aligned16(workspace) || workspace_bytes < nsa::decode_split_workspace_bytes(a, splits))
+      return fail(NSA_ERR_INVALID, "%s: workspace missing, misaligned or smaller than nsa_decode_split_workspace_bytes", what);
+    const int rc = nsa::launch_decode_split(a, splits, workspace, stream);
+    if (rc == -2) return fail(NSA_ERR_UNSUPPORTED, "%s: head dims or split count not built", what);
+    return finish(rc, what);
+  }
   const int rc = nsa::launch_decode(a, stream);
   if (rc == -2) return fail(NSA_ERR_UNSUPPORTED, "%s: head dims not built (dk,dv in (64,64),(128,128),(192,128); fp32: no 192)", what);
   return finish(rc, what);
+}
+
+int64_t nsa_decode_split_workspace_bytes(int batch, int hkv, int dv, int nc_cap, int splits) {
+  if (batch <= 0 || hkv <= 0 || dv <= 0 || nc_cap <= 0 || splits <= 0) return 0;
+  nsa::DecodeArgs a{};
+  a.batch = batch; a.hkv = hkv; a.dv = dv; a.nc_cap = nc_cap;
+  return nsa::decode_split_workspace_bytes(a, splits);
+}
+
+int nsa_decode_step_split(const void* q, const void* k_cache, const void* v_cache_t, const int32_t* block_table,
+                          int max_pages, const void* ck_cache, const void* cv_cache_t, const int32_t* ctx_lens,
+                          const void* gates, void* out, int32_t* indices, int batch, int hq, int hkv, int dk, int dv,
+                          int ctx_cap, int nc_cap, int block, int stride, int sel_block, int pool_kernel,
+                          int pool_stride, int pool_pad, int top_n, int window, float scale, int gate_act, int dtype,
+                          int splits, void* workspace, int64_t workspace_bytes, nsa_stream_t stream) {
+  if (splits <= 0) return fail(NSA_ERR_INVALID, "decode_step_split: splits must be positive");
+  if (block_table && max_pages <= 0) return fail(NSA_ERR_INVALID, "decode_step_split: a block table needs max_pages");
+  return decode_common("decode_step_split", q, k_cache, v_cache_t, block_table, block_table ? max_pages : 0, ck_cache,
+                       cv_cache_t, ctx_lens, gates, out, indices, batch, hq, hkv, dk, dv,
+                       block_table ? max_pages * 64 : ctx_cap, nc_cap, block, stride, sel_block, pool_kernel,
+                       pool_stride, pool_pad, top_n, window, scale, gate_act, dtype, stream, splits, workspace,
+                       workspace_bytes);
 }
 
 int nsa_decode_step(const void* q, const void* k_cache, const void* v_cache_t, const void* ck_cache,

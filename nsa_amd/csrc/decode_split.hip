@@ -1,0 +1,542 @@
+// Decode step for small batches: the work of one (sequence, kv head) spread over many workgroups.
+//
+// The one-workgroup kernel streams 1.8 MB through a single CU, which takes ~60 us however few sequences
+// there are; with fewer than 128 (sequence, kv head) pairs most of the chip idles.  Here the step runs as
+// three launches on the same stream, each over (pair, split) workgroups of 4 wavefronts:
+//   A  compressed rows cut into SA slices: raw scores, per-slice max / sum per head, per-head pooled
+//      window sums relative to the slice maximum (the head sum needs every head's global normaliser, which
+//      only B knows), partial compressed attention of the visible rows
+//   B  every workgroup rebuilds the global statistics from the SA slices (a few KB), normalises and adds the
+//      window sums, takes the top-n blocks (all SB workgroups get the same answer), then attends its share
+//      of the 32-key chunks of the window and of the selected blocks; partial states per branch
+//   C  merges the partial states of the three branches, gates, stores
+// Same arithmetic as the one-workgroup kernel up to the order of fp32 sums.  Pooling 5 / 4 / 0 only
+// (windows of 5 compressed rows every 4, the default geometry).
+#include "decode_common.h"
+
+namespace nsa {
+
+constexpr int kSplitWaves = 4;
+constexpr int kSplitMaxChunks = 3;                                   // compressed 32-row chunks per wavefront of a slice
+constexpr int kSplitMaxSlice = 32 * kSplitWaves * kSplitMaxChunks;   // 384 rows
+
+// floats per (sequence, kv head) in the workspace
+struct SplitLayout {
+  int sa, sb, slice, nb, dv;
+  __host__ __device__ long stat() const { return 0; }                                   // [sa][2][16]
+  __host__ __device__ long bins() const { return (long)sa * 32; }                       // [sa][nb][16]
+  __host__ __device__ long cmp() const { return bins() + (long)sa * nb * 16; }          // [sa][1 + dv][16]
+  __host__ __device__ long att() const { return cmp() + (long)sa * (1 + dv) * 16; }     // [2][sb][2 + dv][16]
+  __host__ __device__ long total() const { return att() + 2L * sb * (2 + dv) * 16; }
+};
+
+static SplitLayout split_layout(const DecodeArgs& a, int splits) {
+  SplitLayout l;
+  l.sa = max(splits, (a.nc_cap + kSplitMaxSlice - 1) / kSplitMaxSlice);
+  l.slice = ((a.nc_cap + l.sa - 1) / l.sa + 31) / 32 * 32;
+  l.sb = splits;
+  l.nb = l.slice / 4 + 2;
+  l.dv = a.dv;
+  return l;
+}
+
+long decode_split_workspace_bytes(const DecodeArgs& a, int splits) {
+  return split_layout(a, splits).total() * (long)a.batch * a.hkv * (long)sizeof(float);
+}
+
+// ---- A: compressed rows of one slice ---------------------------------------------------------------
+template <typename T, int DK, int DV>
+__global__ void __launch_bounds__(kSplitWaves * 64)
+decode_split_cmp_kernel(const DecodeArgs a, const SplitLayout L, float* __restrict__ ws) {
+  constexpr int NW = kSplitWaves, MAXC = kSplitMaxChunks, PLD = 17;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  float* part = reinterpret_cast<float*>(smem_raw);            // [NW][DV][PLD]
+  float* pstat = part + NW * DV * PLD;                         // [NW][2][16]
+  float* pl = pstat + NW * 2 * 16;                             // [NW][16]
+  float* binsL = pl + NW * 16;                                 // [nb][16]
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 15, g = lane >> 4;
+  const int bh = blockIdx.x, s = blockIdx.y;
+  const int b = bh / a.hkv, h = bh % a.hkv;
+  const int G = a.hq / a.hkv;
+  float* wsp = ws + (long)bh * L.total();
+  float* w_stat = wsp + L.stat() + (long)s * 32;
+  float* w_bins = wsp + L.bins() + (long)s * L.nb * 16;
+  float* w_cmp = wsp + L.cmp() + (long)s * (1 + DV) * 16;
+
+  const int cap = a.block_table != nullptr ? a.max_pages * 64 : a.ctx_cap;
+  const int ctx = min(a.ctx_lens[b], cap);
+  const int t = ctx - 1;
+  const int Nc = ctx >= a.block ? min((ctx - a.block) / a.stride + 1, a.nc_cap) : 0;
+  const int c_lo = s * L.slice, c_hi = min(c_lo + L.slice, Nc);
+  if (c_lo >= c_hi) {                        // nothing in this slice: neutral statistics, no partial
+    if (tid < 16) { w_stat[tid] = kNegInf; w_stat[16 + tid] = 0.f; w_cmp[tid] = 0.f; }
+    return;
+  }
+  const int cmaxv = t >= a.block ? min((t - a.block) / a.stride, Nc - 1) : -1;   // last visible compressed row
+  const float c_attn = a.scale * kLog2e;
+  const long krow = (long)a.hkv * DK;
+  const T* ckseq = reinterpret_cast<const T*>(a.ck_cache) + ((long)b * a.nc_cap * a.hkv + h) * DK;
+  const T* cvt = reinterpret_cast<const T*>(a.cv_cache_t) + (((long)b * a.hkv + h) * DV + n) * a.nc_cap + 8 * g;
+  const long cvstep = 16L * a.nc_cap;
+
+  vec8_t<T> qf[DK / 32];
+  {
+    const int gc = n < G ? n : G - 1;
+    const T* qp = reinterpret_cast<const T*>(a.q) + ((long)b * a.hq + h * G + gc) * DK + 8 * g;
+#pragma unroll
+    for (int kk = 0; kk < DK / 32; ++kk) qf[kk] = load8(qp + 32 * kk);
+  }
+  for (int i = tid; i < L.nb * 16; i += NW * 64) binsL[i] = 0.f;
+
+  // raw scores of this wavefront's chunks, all K fragments requested before the first product
+  vec8_t<T> kf[MAXC][2][DK / 32];
+#pragma unroll
+  for (int i = 0; i < MAXC; ++i) {
+    const int cb = c_lo + 32 * (wave + NW * i);
+    if (cb < c_hi) {
+      const T* k0p = ckseq + (long)min(cb + chunk_key_of_row(0, n), Nc - 1) * krow + 8 * g;
+      const T* k1p = ckseq + (long)min(cb + chunk_key_of_row(1, n), Nc - 1) * krow + 8 * g;
+#pragma unroll
+      for (int kk = 0; kk < DK / 32; ++kk) { kf[i][0][kk] = load8(k0p + 32 * kk); kf[i][1][kk] = load8(k1p + 32 * kk); }
+    }
+  }
+  float sc[MAXC][8];
+  float mi = kNegInf, li = 0.f;
+#pragma unroll
+  for (int i = 0; i < MAXC; ++i) {
+    const int cb = c_lo + 32 * (wave + NW * i);
+    if (cb < c_hi) {
+      f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kk = 0; kk < DK / 32; ++kk) {
+        s0 = mma16(kf[i][0][kk], qf[kk], s0);
+        s1 = mma16(kf[i][1][kk], qf[kk], s1);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { sc[i][e] = s0[e]; sc[i][4 + e] = s1[e]; }
+      float mx = kNegInf;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        if (cb + 8 * g + e >= c_hi) sc[i][e] = kNegInf;
+        mx = fmaxf(mx, sc[i][e]);
+      }
+      mx = colgroup_max(mx);                            // finite: row cb exists
+      const float m_new = fmaxf(mi, mx);
+      float sum = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sum += fast_exp2((sc[i][e] - m_new) * kLog2e);
+      li = li * fast_exp2((mi - m_new) * kLog2e) + sum;
+      mi = m_new;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sc[i][e] = kNegInf;
+    }
+  }
+  // the visible chunks' value fragments: requested now, used after the statistics are combined
+  vec8_t<T> vf[MAXC][DV / 16];
+#pragma unroll
+  for (int i = 0; i < MAXC; ++i) {
+    const int cb = c_lo + 32 * (wave + NW * i);
+    if (cb < c_hi && cb <= cmaxv) {
+#pragma unroll
+      for (int tt = 0; tt < DV / 16; ++tt) vf[i][tt] = load8(cvt + tt * cvstep + cb);
+    }
+  }
+  li = colgroup_sum(li);
+  if (g == 0) { pstat[(wave * 2 + 0) * 16 + n] = mi; pstat[(wave * 2 + 1) * 16 + n] = li; }
+  __syncthreads();                                      // also: binsL is zero
+  float M = kNegInf;
+#pragma unroll
+  for (int w = 0; w < NW; ++w) M = fmaxf(M, pstat[(w * 2) * 16 + n]);
+  float Z = 0.f;
+#pragma unroll
+  for (int w = 0; w < NW; ++w) {
+    const float mw = pstat[(w * 2) * 16 + n];
+    if (mw != kNegInf) Z += pstat[(w * 2 + 1) * 16 + n] * fast_exp2((mw - M) * kLog2e);
+  }
+  if (tid < 16) { w_stat[tid] = M; w_stat[16 + tid] = Z; }          // head n = tid (wavefront 0, g = 0)
+
+  // pooled window sums per head, relative to the slice maximum: rows 4j .. 4j+4 make bin j; local bin
+  // index = j - (c_lo / 4 - 1), so that the bin a slice's first row completes is local bin 0
+  const float Ml2 = M * kLog2e;
+#pragma unroll
+  for (int i = 0; i < MAXC; ++i) {
+    const int cb = c_lo + 32 * (wave + NW * i);
+    if (cb < c_hi) {
+      float v[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = fast_exp2(fmaf(sc[i][e], kLog2e, -Ml2));     // 0 past c_hi
+      const int c0 = cb + 8 * g;
+      if (c0 < c_hi) {
+        const int b0 = (c0 - c_lo) / 4 + 1;
+        atomicAdd(&binsL[(b0 - 1) * 16 + n], v[0]);
+        atomicAdd(&binsL[b0 * 16 + n], (v[0] + v[1]) + (v[2] + v[3]) + v[4]);
+        atomicAdd(&binsL[(b0 + 1) * 16 + n], (v[4] + v[5]) + (v[6] + v[7]));
+      }
+    }
+  }
+
+  // partial compressed attention of the visible rows, reference = the slice maximum
+  DecState<T, DK, DV> cmp;
+  dec_reset(cmp);
+#pragma unroll
+  for (int i = 0; i < MAXC; ++i) {
+    const int cb = c_lo + 32 * (wave + NW * i);
+    if (cb < c_hi && cb <= cmaxv) {
+      float p[8], psum = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int c = cb + 8 * g + e;
+        p[e] = (c <= cmaxv && c < c_hi) ? fast_exp2((sc[i][e] - M) * c_attn) : 0.f;
+        psum += p[e];
+      }
+      cmp.l += psum;
+      const vec8_t<T> pb = pack8<T>(p);
+#pragma unroll
+      for (int tt = 0; tt < DV / 16; ++tt) cmp.o[tt] = mma16(vf[i][tt], pb, cmp.o[tt]);
+    }
+  }
+#pragma unroll
+  for (int tt = 0; tt < DV / 16; ++tt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) part[(wave * DV + tt * 16 + 4 * g + i) * PLD + n] = cmp.o[tt][i];
+  const float lt = colgroup_sum(cmp.l);
+  if (g == 0) pl[wave * 16 + n] = lt;
+  __syncthreads();
+  for (int i = tid; i < L.nb * 16; i += NW * 64) w_bins[i] = binsL[i];
+  // every wavefront used the same reference: the partial states just add up
+  const int r = tid & 15;
+  if (tid < 16) {
+    float l = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) l += pl[w * 16 + tid];
+    w_cmp[tid] = l;
+  }
+  for (int d = tid >> 4; d < DV; d += NW * 4) {
+    float o = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) o += part[(w * DV + d) * PLD + r];
+    w_cmp[(1 + d) * 16 + r] = o;
+  }
+}
+
+// ---- B: selection, then window and selected chunks ---------------------------------------------------
+template <typename T, int DK, int DV, bool PAGED>
+__global__ void __launch_bounds__(kSplitWaves * 64)
+decode_split_attend_kernel(const DecodeArgs a, const SplitLayout L, float* __restrict__ ws) {
+  constexpr int NW = kSplitWaves, PLD = 17;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  float* part = reinterpret_cast<float*>(smem_raw);            // [NW][DV][PLD]
+  float* pstat = part + NW * DV * PLD;                         // [NW][2][16]
+  float* fac = pstat + NW * 2 * 16;                            // [sa][16]
+  float* pooled = fac + L.sa * 16;                             // [Ns]
+  int* sel = reinterpret_cast<int*>(pooled + ((a.nc_cap + 3) / 4 + 4));   // [top_n]
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 15, g = lane >> 4;
+  const int bh = blockIdx.x, sb = blockIdx.y;
+  const int b = bh / a.hkv, h = bh % a.hkv;
+  const int G = a.hq / a.hkv;
+  float* wsp = ws + (long)bh * L.total();
+  const float* w_stat = wsp + L.stat();
+  const float* w_bins = wsp + L.bins();
+
+  const int cap = PAGED ? a.max_pages * 64 : a.ctx_cap;
+  const int ctx = min(a.ctx_lens[b], cap);
+  if (ctx <= 0) return;
+  const int t = ctx - 1;
+  const int Nc = ctx >= a.block ? min((ctx - a.block) / a.stride + 1, a.nc_cap) : 0;
+  int Ns = 0;
+  if (Nc >= 5) {
+    Ns = (Nc - 5 + 3) / 4 + 1;
+    if ((Ns - 1) * 4 >= Nc) --Ns;
+  }
+  const float c_attn = a.scale * kLog2e;
+
+  // ---- this workgroup's share of the 32-key chunks: item k goes to workgroup k % sb, wavefront (k / sb) % NW
+  const T* kseq = reinterpret_cast<const T*>(a.k_cache) + (PAGED ? (long)h * DK : ((long)b * a.ctx_cap * a.hkv + h) * DK);
+  const long krow = (long)a.hkv * DK;
+  const T* vt = reinterpret_cast<const T*>(a.v_cache_t) +
+                (PAGED ? ((long)h * DV + n) * 64 + 8 * g : (((long)b * a.hkv + h) * DV + n) * a.ctx_cap + 8 * g);
+  const long vstep = PAGED ? 16L * 64 : 16L * a.ctx_cap;
+  auto issue_kv = [&](ChunkFrags<T, DK, DV>& f, int cb) {
+    if constexpr (PAGED) {
+      const long pg = a.block_table[(long)b * a.max_pages + (cb >> 6)];
+      chunk_issue<T, DK, DV>(f, kseq + pg * 64 * krow, krow, vt + pg * a.hkv * DV * 64, vstep, cb & 63,
+                             min(t - (cb & ~63), 63), n, g);
+    } else {
+      chunk_issue<T, DK, DV>(f, kseq, krow, vt, vstep, cb, t, n, g);
+    }
+  };
+  vec8_t<T> qf[DK / 32];
+  {
+    const int gc = n < G ? n : G - 1;
+    const T* qp = reinterpret_cast<const T*>(a.q) + ((long)b * a.hq + h * G + gc) * DK + 8 * g;
+#pragma unroll
+    for (int kk = 0; kk < DK / 32; ++kk) qf[kk] = load8(qp + 32 * kk);
+  }
+  const int r = tid & 15;
+  // partial state of a branch: wavefronts merged through LDS, left un-normalised for kernel C
+  auto put = [&](const DecState<T, DK, DV>& st, int branch) {
+    float* dst = wsp + L.att() + ((long)branch * L.sb + sb) * (2 + DV) * 16;
+    __syncthreads();
+#pragma unroll
+    for (int tt = 0; tt < DV / 16; ++tt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) part[(wave * DV + tt * 16 + 4 * g + i) * PLD + n] = st.o[tt][i];
+    const float lt = colgroup_sum(st.l);
+    if (g == 0) { pstat[(wave * 2 + 0) * 16 + n] = st.m; pstat[(wave * 2 + 1) * 16 + n] = lt; }
+    __syncthreads();
+    float mm = kNegInf;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) mm = fmaxf(mm, pstat[(w * 2) * 16 + r]);
+    float wgt[NW], den = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      const float mw = pstat[(w * 2) * 16 + r];
+      wgt[w] = mw == kNegInf ? 0.f : fast_exp2((mw - mm) * c_attn);
+      den += wgt[w] * pstat[(w * 2 + 1) * 16 + r];
+    }
+    if (tid < 16) { dst[tid] = mm; dst[16 + tid] = den; }
+    for (int d = tid >> 4; d < DV; d += NW * 4) {
+      float o = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) o += wgt[w] * part[(w * DV + d) * PLD + r];
+      dst[(2 + d) * 16 + r] = o;
+    }
+  };
+
+  // chunk items are numbered window first, then the selected blocks in pick order; this wavefront takes the
+  // items sb + L.sb * (wave + NW * i), i = 0, 1, ...
+  const int item_step = L.sb * NW;
+  int next = sb + L.sb * wave;
+  // The window does not depend on the selection: this wavefront's first window chunk is requested before the
+  // statistics and the top-n (which only wavefront 0 computes) and attended while they are under way.
+  ChunkFrags<T, DK, DV> f;
+  const int w_lo = max(t - a.window + 1, 0);
+  const int w_first = (w_lo / 32) * 32;
+  const int nwin = a.window > 0 ? (t - w_first) / 32 + 1 : 0;
+  const int my_win = next < nwin ? next : -1;                // first window item of this wavefront
+  if (my_win >= 0) issue_kv(f, w_first + 32 * my_win);
+
+  // global log-sum-exp of the raw scores per head, and each slice's factor exp(M_s - lse).  One thread per
+  // (slice, statistic, head) fetches its value (sa <= 16: at most 512 of them) so that the 16 threads that
+  // combine them read LDS, not a chain of dependent global loads.
+  float* st_l = part;                                          // [sa][32], free until the first put()
+  for (int i = tid; i < L.sa * 32; i += NW * 64) st_l[i] = w_stat[i];
+  __syncthreads();
+  if (tid < 16) {
+    float M = kNegInf;
+    for (int s = 0; s < L.sa; ++s) M = fmaxf(M, st_l[s * 32 + tid]);
+    float Z = 0.f;
+    for (int s = 0; s < L.sa; ++s) {
+      const float ms = st_l[s * 32 + tid];
+      if (ms != kNegInf) Z += st_l[s * 32 + 16 + tid] * fast_exp2((ms - M) * kLog2e);
+    }
+    const float lse2 = (Nc > 0 && tid < G) ? (M + __logf(Z)) * kLog2e : __builtin_huge_valf();   // padding heads drop out
+    for (int s = 0; s < L.sa; ++s) {
+      const float ms = st_l[s * 32 + tid];
+      fac[s * 16 + tid] = ms == kNegInf ? 0.f : fast_exp2(fmaf(ms, kLog2e, -lse2));
+    }
+  }
+  for (int i = tid; i < Ns; i += NW * 64) pooled[i] = 0.f;
+  __syncthreads();
+  for (int base = 0; base < L.sa * L.nb; base += 4 * NW * 64) {
+    f32x4_t x[4][4];
+    int js[4], ss[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {                     // all loads of this round first
+      const int idx = base + u * NW * 64 + tid;
+      const int s = idx / L.nb, lb = idx % L.nb;
+      const int j = s * (L.slice / 4) - 1 + lb;
+      const bool ok = idx < L.sa * L.nb && j >= 0 && j < Ns && s * L.slice < Nc;
+      js[u] = ok ? j : -1;
+      ss[u] = s;
+      if (ok) {
+        const float* src = w_bins + ((long)s * L.nb + lb) * 16;
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) x[u][q4] = *reinterpret_cast<const f32x4_t*>(src + 4 * q4);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (js[u] >= 0) {
+        float v = 0.f;
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          const f32x4_t fc = *reinterpret_cast<const f32x4_t*>(fac + ss[u] * 16 + 4 * q4);
+          v += x[u][q4][0] * fc[0] + x[u][q4][1] * fc[1] + x[u][q4][2] * fc[2] + x[u][q4][3] * fc[3];
+        }
+        atomicAdd(&pooled[js[u]], v);
+      }
+    }
+  }
+  __syncthreads();
+  if (wave == 0) {
+    constexpr int PER = (32 * kDecWaves * kDecMaxChunks / 4 + 63) / 64 + 1;
+    __shared__ float cand_v[128];
+    __shared__ int cand_i[128];
+    float v[PER];
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      const int bb = lane + 64 * k;
+      v[k] = -1.f;
+      if (bb < Ns) v[k] = pooled[bb] / (float)(min(4 * bb + 5, Nc) - 4 * bb);
+    }
+    wave_topn_shortlist<PER>(v, a.top_n, lane, cand_v, cand_i, [&](int rr, int val) {
+      if (lane == 0) {
+        sel[rr] = val;
+        if (a.indices != nullptr && sb == 0) a.indices[((long)b * a.hkv + h) * a.top_n + rr] = val;
+      }
+    });
+  }
+  {
+    DecState<T, DK, DV> swa;
+    dec_reset(swa);
+    for (; next < nwin; next += item_step) {
+      const int cb = w_first + 32 * next;
+      if (next != my_win) issue_kv(f, cb);
+      chunk_attend<T, DK, DV>(swa, f, qf, cb, w_lo, t, c_attn, g);
+    }
+    put(swa, 1);                                             // its barriers also publish the selected blocks
+  }
+
+  // selected blocks: their chunks continue the item count of the window
+  {
+    DecState<T, DK, DV> slc;
+    dec_reset(slc);
+    int item = nwin;
+    for (int rr = 0; rr < a.top_n; ++rr) {
+      const int bi = sel[rr];
+      if (bi < 0 || (long)bi * a.sel_block > t) continue;
+      const int k0 = bi * a.sel_block, k1 = min(k0 + a.sel_block - 1, t);
+      for (int cb = k0; cb <= k1; cb += 32, ++item) {
+        if (item != next) continue;
+        next += item_step;
+        issue_kv(f, cb);
+        chunk_attend<T, DK, DV>(slc, f, qf, cb, k0, k1, c_attn, g);
+      }
+    }
+    put(slc, 0);
+  }
+}
+
+// ---- C: merge of the partial states, gates, output ---------------------------------------------------
+// grid (pair, DV / 16): thread = (head r, channel d).  The weights of all partial states go through LDS first
+// (one thread per state and head), and the weighted sums are unrolled over the most states there can be, so
+// that every load of a thread is in flight at once: the launch is pure latency otherwise.
+constexpr int kSplitMaxStates = 16;
+
+template <typename T, int DV>
+__global__ void __launch_bounds__(256)
+decode_split_merge_kernel(const DecodeArgs a, const SplitLayout L, const float* __restrict__ ws) {
+  constexpr int MAXS = kSplitMaxStates;
+  __shared__ float sm[3][MAXS][16], sl[3][MAXS][16];           // branch 0 selected, 1 window, 2 compressed
+  const int tid = threadIdx.x, r = tid & 15, dg = tid >> 4;
+  const int bh = blockIdx.x, d = blockIdx.y * 16 + dg;
+  const int b = bh / a.hkv, h = bh % a.hkv;
+  const int G = a.hq / a.hkv;
+  const float* wsp = ws + (long)bh * L.total();
+  const int cap = a.block_table != nullptr ? a.max_pages * 64 : a.ctx_cap;
+  if (min(a.ctx_lens[b], cap) <= 0) return;
+  const float c_attn = a.scale * kLog2e;
+  for (int i = tid; i < 3 * MAXS * 16; i += 256) {
+    const int br = i / (MAXS * 16), s = (i / 16) % MAXS, hh = i % 16;
+    float m = kNegInf, l = 0.f;
+    if (br < 2) {
+      if (s < L.sb) {
+        const float* p = wsp + L.att() + ((long)br * L.sb + s) * (2 + DV) * 16;
+        m = p[hh]; l = p[16 + hh];
+      }
+    } else if (s < L.sa) {
+      m = wsp[L.stat() + s * 32 + hh];
+      l = wsp[L.cmp() + (long)s * (1 + DV) * 16 + hh];
+    }
+    sm[br][s][hh] = m; sl[br][s][hh] = l;
+  }
+  __syncthreads();
+  if (r >= G) return;
+  const T* gp = reinterpret_cast<const T*>(a.gates);
+  float acc = 0.f;
+#pragma unroll
+  for (int br = 0; br < 3; ++br) {
+    float mm = kNegInf;
+#pragma unroll
+    for (int s = 0; s < MAXS; ++s) mm = fmaxf(mm, sm[br][s][r]);
+    float w[MAXS], den = 0.f;
+#pragma unroll
+    for (int s = 0; s < MAXS; ++s) {
+      const float ms = sm[br][s][r];
+      w[s] = ms == kNegInf ? 0.f : fast_exp2((ms - mm) * c_attn);
+      den += w[s] * sl[br][s][r];
+    }
+    const float* p = br < 2 ? wsp + L.att() + (long)br * L.sb * (2 + DV) * 16 + (2 + d) * 16 + r
+                            : wsp + L.cmp() + (1 + d) * 16 + r;
+    const long step = br < 2 ? (2 + DV) * 16 : (1 + DV) * 16;
+    float x[MAXS];
+#pragma unroll
+    for (int s = 0; s < MAXS; ++s) x[s] = w[s] != 0.f ? p[s * step] : 0.f;    // zero weight: unwritten or empty state
+    float num = 0.f;
+#pragma unroll
+    for (int s = 0; s < MAXS; ++s) num += w[s] * x[s];
+    float gate = 1.f;
+    if (gp != nullptr) {
+      const float gx = (float)gp[((long)b * a.hq + h * G + r) * 3 + br];
+      gate = a.gate_act == 1 ? 1.0f / (1.0f + __expf(-gx)) : gx;
+    }
+    if (den > 0.f) acc += num * gate / den;
+  }
+  reinterpret_cast<T*>(a.out)[((long)b * a.hq + h * G + r) * DV + d] = (T)acc;
+}
+
+int set_smem(const void* fn, size_t bytes);
+
+template <typename T, int DK, int DV>
+static int launch_decode_split_t(const DecodeArgs& a, int splits, float* ws, hipStream_t st) {
+  const SplitLayout L = split_layout(a, splits);
+  if (L.sa > 16 || L.sb > 16) return -2;
+  const int pairs = a.batch * a.hkv;
+  const size_t base = ((size_t)kSplitWaves * DV * 17 + kSplitWaves * 32) * sizeof(float);
+  const size_t smem_a = base + ((size_t)kSplitWaves * 16 + (size_t)L.nb * 16) * sizeof(float);
+  const size_t smem_b = base + ((size_t)L.sa * 16 + (a.nc_cap + 3) / 4 + 4) * sizeof(float) + (size_t)a.top_n * sizeof(int) + 64;
+  {
+    auto fn = decode_split_cmp_kernel<T, DK, DV>;
+    if (int rc = set_smem(reinterpret_cast<const void*>(fn), smem_a)) return rc;
+    hipLaunchKernelGGL(fn, dim3(pairs, L.sa), dim3(kSplitWaves * 64), smem_a, st, a, L, ws);
+  }
+  if (a.block_table != nullptr) {
+    auto fn = decode_split_attend_kernel<T, DK, DV, true>;
+    if (int rc = set_smem(reinterpret_cast<const void*>(fn), smem_b)) return rc;
+    hipLaunchKernelGGL(fn, dim3(pairs, L.sb), dim3(kSplitWaves * 64), smem_b, st, a, L, ws);
+  } else {
+    auto fn = decode_split_attend_kernel<T, DK, DV, false>;
+    if (int rc = set_smem(reinterpret_cast<const void*>(fn), smem_b)) return rc;
+    hipLaunchKernelGGL(fn, dim3(pairs, L.sb), dim3(kSplitWaves * 64), smem_b, st, a, L, ws);
+  }
+  hipLaunchKernelGGL((decode_split_merge_kernel<T, DV>), dim3(pairs, DV / 16), dim3(256), 0, st, a, L, ws);
+  return 0;
+}
+
+int launch_decode_split(const DecodeArgs& a, int splits, void* workspace, hipStream_t st) {
+  float* ws = reinterpret_cast<float*>(workspace);
+  const int key = a.dk * 1000 + a.dv;
+  if (a.dtype == 0) {
+    switch (key) {
+      case 64064: return launch_decode_split_t<bf16_t, 64, 64>(a, splits, ws, st);
+      case 128128: return launch_decode_split_t<bf16_t, 128, 128>(a, splits, ws, st);
+      case 192128: return launch_decode_split_t<bf16_t, 192, 128>(a, splits, ws, st);
+      default: return -2;
+    }
+  }
+  switch (key) {
+    case 64064: return launch_decode_split_t<float, 64, 64>(a, splits, ws, st);
+    case 128128: return launch_decode_split_t<float, 128, 128>(a, splits, ws, st);
+    default: return -2;
+  }
+}
+
+}  // namespace nsa

@@ -214,10 +214,15 @@ class NSAPagedDecodeCache:
 def nsa_decode_step(q: torch.Tensor, cache, gates: Optional[torch.Tensor] = None,
                     selection_block: int = 64, selected_block_count: int = 16, sliding_window: int = 512,
                     scale: Optional[float] = None, gate_activation: Optional[str] = None,
-                    return_indices: bool = False):
+                    return_indices: bool = False, splits: Optional[int] = None):
     """q [B,Hq,Dk]: queries of the newest cached token; cache: NSADecodeCache or NSAPagedDecodeCache.  gates [B,Hq,3] (selected, sliding,
     compressed; pre-activation if gate_activation == "sigmoid").  Returns out [B,Hq,Dv]
-    (and int32 block indices [B,Hkv,S])."""
+    (and int32 block indices [B,Hkv,S]).
+
+    splits: how many workgroups share one (sequence, kv head) pair.  0 = one (the kernel the batch-64
+    benchmark runs); None = chosen from the batch: up to 64 pairs a single workgroup per pair leaves
+    most of the chip idle and its ~60 us critical path sets the step time, so the work is split 8 ways
+    (three launches, partial results in a workspace kept on the cache object)."""
     if not q.is_cuda:
         raise RuntimeError("NSA kernels run on the GPU only")
     B, hq, dk = q.shape
@@ -233,7 +238,28 @@ def nsa_decode_step(q: torch.Tensor, cache, gates: Optional[torch.Tensor] = None
     pool_s = selection_block // cache.stride
     pool_p = cache.block // cache.stride - 2
     act = _lib.GATE_SIGMOID if gate_activation == "sigmoid" else _lib.GATE_IDENTITY
-    if isinstance(cache, NSAPagedDecodeCache):
+    paged = isinstance(cache, NSAPagedDecodeCache)
+    if splits is None:
+        pairs = B * cache.hkv
+        # measured at 32k context: 8 splits halve the step up to 32 pairs and still win at 64 (46 vs 64 us);
+        # at 128 pairs one workgroup per pair is as fast and needs no workspace
+        splits = 8 if pairs <= 64 and (pool_k, pool_s, pool_p) == (5, 4, 0) and selected_block_count <= 64 else 0
+    if splits:
+        lib = _lib.load()
+        need = lib.nsa_decode_split_workspace_bytes(B, cache.hkv, cache.dv, cache.nc_cap, splits)
+        ws = getattr(cache, "_split_ws", None)
+        if ws is None or ws.numel() < need:
+            ws = cache._split_ws = torch.empty(need, dtype=torch.uint8, device=q.device)
+        k_c, v_c = (cache.k_pool, cache.v_pool_t) if paged else (cache.k, cache.vt)
+        rc = lib.nsa_decode_step_split(
+            _ptr(q), _ptr(k_c), _ptr(v_c), _ptr(cache.block_table) if paged else None,
+            cache.max_pages if paged else 0, _ptr(cache.ck), _ptr(cache.cvt), _ptr(cache.ctx_lens), _ptr(gates),
+            _ptr(out), _ptr(idx), B, hq, cache.hkv, dk, cache.dv, cache.ctx_cap, cache.nc_cap, cache.block,
+            cache.stride, selection_block, pool_k, pool_s, pool_p, selected_block_count, sliding_window,
+            float(scale), act, _dtype_code(q), splits, _ptr(ws), ws.numel(), _stream())
+        _lib.check(rc, "nsa_decode_step_split")
+        return (out, idx) if return_indices else out
+    if paged:
         rc = _lib.load().nsa_decode_step_paged(
             _ptr(q), _ptr(cache.k_pool), _ptr(cache.v_pool_t), _ptr(cache.block_table), cache.max_pages,
             _ptr(cache.ck), _ptr(cache.cvt), _ptr(cache.ctx_lens), _ptr(gates), _ptr(out), _ptr(idx), B, hq,

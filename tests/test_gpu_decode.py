@@ -142,3 +142,50 @@ def test_decode_randomized_sweep():
             G = 4                                  # keep the sweep to shapes every dtype is built for
         print("case", case, ctxs, G, Hkv, D, S, W, dtype)
         _check(dtype, ctxs, G * Hkv, Hkv, D, D, S, W, seed=400 + case)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("splits", [1, 2, 3, 8, 16])
+def test_split_step_equals_one_workgroup_step(dtype, splits):
+    """The small-batch schedule (work of a pair spread over `splits` workgroups, three launches) against
+    the one-workgroup kernel: same block picks, outputs equal up to the order of fp32 sums."""
+    from nsa_amd.decode import NSADecodeCache, nsa_decode_step
+    ctxs = [2048, 1500, 1025, 513, 96, 64, 33, 31, 5, 1]
+    B, T = len(ctxs), max(ctxs)
+    Hq, Hkv, D, S, W = 32, 2, 128, 4, 128
+    q, k, v, gl = _make(B, T, Hq, Hkv, D, D, 900, dtype)
+    cache = NSADecodeCache(B, T, Hkv, D, D, dtype=dtype, device=DEV)
+    cache.fill(k.to(DEV), v.to(DEV))
+    cache.ctx_lens.copy_(torch.tensor(ctxs, dtype=torch.int32))
+    kw = dict(selection_block=64, selected_block_count=S, sliding_window=W, gate_activation="sigmoid",
+              return_indices=True)
+    ref, ref_idx = nsa_decode_step(q.to(DEV), cache, gl.to(DEV), splits=0, **kw)
+    out, idx = nsa_decode_step(q.to(DEV), cache, gl.to(DEV), splits=splits, **kw)
+    assert torch.equal(idx, ref_idx)
+    err = max_abs(out, ref)
+    print("split", splits, dtype, "max_abs vs one workgroup", err)
+    assert err <= (1e-5 if dtype == torch.float32 else 8e-3)
+
+
+def test_split_step_long_context_and_paged():
+    """ctx 32768 (2047 compressed rows, every slice and bin boundary in use), contiguous and paged, group 16."""
+    import random
+    from nsa_amd.decode import NSADecodeCache, NSAPagedDecodeCache, nsa_decode_step
+    B, T, Hq, Hkv, D = 2, 32768, 64, 4, 128
+    dtype = torch.bfloat16
+    q, k, v, gl = _make(B, T, Hq, Hkv, D, D, 910, dtype)
+    flat = NSADecodeCache(B, T, Hkv, D, D, dtype=dtype, device=DEV)
+    flat.fill(k.to(DEV), v.to(DEV))
+    paged = NSAPagedDecodeCache(B, B * T // 64, T, Hkv, D, D, dtype=dtype, device=DEV)
+    random.Random(5).shuffle(paged._free)
+    paged.fill(k.to(DEV), v.to(DEV))
+    kw = dict(selection_block=64, selected_block_count=16, sliding_window=512, gate_activation="sigmoid",
+              return_indices=True)
+    ref, ref_idx = nsa_decode_step(q.to(DEV), flat, gl.to(DEV), splits=0, **kw)
+    for cache in (flat, paged):
+        for splits in (6, 8):
+            out, idx = nsa_decode_step(q.to(DEV), cache, gl.to(DEV), splits=splits, **kw)
+            assert torch.equal(idx, ref_idx)
+            assert max_abs(out, ref) <= 8e-3
+    auto, _ = nsa_decode_step(q.to(DEV), flat, gl.to(DEV), **kw)           # 8 pairs: the split path by default
+    assert max_abs(auto, ref) <= 8e-3

@@ -239,3 +239,24 @@ def test_layer_folds_the_gating_linear_into_the_projection():
         NSAAttentionLayer(40, 6, 2, qk_head_dim=24, rope_dim=12)
     with pytest.raises(NotImplementedError):
         layer(torch.zeros(1, 4, 40, dtype=torch.float64), attention_mask=torch.ones(1, 4))
+
+
+def test_split_decode_argument_errors_do_not_launch(lib):
+    assert lib.nsa_decode_split_workspace_bytes(0, 4, 128, 2048, 8) == 0
+    need = lib.nsa_decode_split_workspace_bytes(2, 4, 128, 2048, 8)
+    assert need > 0 and need % 4 == 0
+    assert lib.nsa_decode_split_workspace_bytes(2, 4, 128, 2048, 2) <= need      # fewer splits never need more
+    buf = ctypes.create_string_buffer(4096)
+    p = (ctypes.addressof(buf) + 63) // 64 * 64
+
+    def call(splits=8, pool=(5, 4, 0), ws=p, ws_bytes=1 << 40, top_n=16):
+        return lib.nsa_decode_step_split(p, p, p, None, 0, p, p, p, None, p, None, 2, 64, 4, 128, 128, 2048, 2048, 32,
+                                         16, 64, pool[0], pool[1], pool[2], top_n, 512, 0.1, 0, 0, splits, ws,
+                                         ws_bytes, None)
+
+    assert call(splits=0) == -1
+    assert call(splits=17) == -1
+    assert call(pool=(3, 2, 0)) == -2 and b"pooling" in lib.nsa_last_error_string()
+    assert call(ws=None) == -1
+    assert call(ws_bytes=16) == -1 and b"workspace" in lib.nsa_last_error_string()
+    assert call(top_n=65) == -2
