@@ -14,7 +14,8 @@ top-n or for the non-causal part of the importance scores) divided by its mean d
 with events on the launch stream.  cpu_baseline: the CPU oracle (a port of the reference's naive
 torch path) on a bounded sample of query rows of the same workload, on this host's cores.
 train_step (extra, not the headline metric): forward + backward of the same workload through the
-module's autograd path.  layer (extra): the attention layer (projections, rotary embedding, NSA,
+module's autograd path.  decode / decode_small_batch (extra): the decode step of benchmark config 5 at
+batch 64 and at batch 8.  layer (extra): the attention layer (projections, rotary embedding, NSA,
 output projection) around the same workload.
 """
 import argparse
@@ -181,6 +182,38 @@ def train_bench(m, q, k, v, gl, cu, max_len, total, f_eff, steps, warmup):
             "mfma_peak_frac": 3.5 * f_eff / (ms_both * 1e-3) / 1e12 / PEAK_BF16_TFLOPS}
 
 
+def decode_small_bench(batch=8, steps=200, warmup=10):
+    """The same decode step at a small batch (extra): 32 (sequence, kv head) pairs cannot fill 256 CUs with
+    one workgroup each, so the step is spread over 8 workgroups per pair; both schedules are timed."""
+    import torch
+    from nsa_amd.decode import NSADecodeCache, nsa_decode_step
+    dev = "cuda:0"
+    ctx, hq, hkv, d, top_n, window = 32768, 64, 4, 128, 16, 512
+    g = torch.Generator(device=dev).manual_seed(5)
+    cache = NSADecodeCache(batch, ctx, hkv, d, d, dtype=torch.bfloat16, device=dev)
+    k = (torch.randn(batch, ctx, hkv, d, device=dev, generator=g) * 0.5).bfloat16()
+    v = (torch.randn(batch, ctx, hkv, d, device=dev, generator=g) * 0.5).bfloat16()
+    cache.fill(k, v)
+    del k, v
+    q = (torch.randn(batch, hq, d, device=dev, generator=g) * 0.5).bfloat16()
+    gl = torch.randn(batch, hq, 3, device=dev, generator=g).bfloat16()
+    res = {"batch": batch, "context": ctx}
+    for name, splits in (("us_per_step", None), ("us_per_step_one_workgroup_per_pair", 0)):
+        run = lambda: nsa_decode_step(q, cache, gl, SEL_BLOCK, top_n, window, gate_activation="sigmoid", splits=splits)
+        for _ in range(warmup):
+            run()
+        torch.cuda.synchronize()
+        beg, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        beg.record()
+        for _ in range(steps):
+            out = run()
+        end.record()
+        torch.cuda.synchronize()
+        assert torch.isfinite(out).all()
+        res[name] = beg.elapsed_time(end) / steps * 1e3
+    return res
+
+
 def layer_bench(total, hq, hkv, dqk, dv, top_n, window, steps, warmup, hidden=4096, rope_dim=64):
     """The attention layer around the same workload (extra, not the headline metric): fused q/k/v/gate
     projection GEMM (hipBLASLt through torch), split + rotary embedding in one HIP pass, NSA forward,
@@ -247,6 +280,8 @@ def main():
     decode_res = None
     if not args.no_decode:
         decode_res = decode_bench(max(args.steps, 200), max(args.warmup, 10))
+        torch.cuda.empty_cache()
+        decode_small = decode_small_bench()
         torch.cuda.empty_cache()
     lens, hq, hkv, dqk, dv, top_n, window, seed = WORKLOADS[args.workload]
     total = sum(lens)
@@ -337,6 +372,7 @@ def main():
         res["layer"] = layer_bench(total, hq, hkv, dqk, dv, top_n, window, max(2, min(args.steps, 10)), 2)
     if decode_res is not None:
         res["decode"] = decode_res
+        res["decode_small_batch"] = decode_small
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(q, k, v, gl, top_n, window, args.cpu_budget)
     print(json.dumps(res))
