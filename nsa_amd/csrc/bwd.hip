@@ -33,7 +33,8 @@ int set_smem(const void* fn, size_t bytes);
 
 constexpr int kBwdCmp = 0, kBwdSwa = 1, kBwdSlc = 2;
 // Launch shapes, chosen by measurement on T = 32768, Hq64/Hkv4, Dk192/Dv128:
-constexpr int kCmpSplit = 256;       // tokens of one compressed-branch work item (1024: 8.6 ms, 256: 5.4 ms)
+constexpr int kCmpSplit = 384;       // tokens of one compressed-branch work item (1024: 8.6 ms, 256: 5.4 ms; with conflict-free
+                                     // LDS the whole backward call: 128: 9.48, 256: 7.89, 320: 7.87, 384: 7.71, 448: 7.68, 512: 7.75)
 constexpr int kKvWaves = 4;          // key-stationary: wavefronts (x16 keys) per workgroup, two workgroups per CU
 constexpr int kQWaves = 16;          // query-stationary: tokens per workgroup (8: 3.7 ms, 16: 3.3 ms)
 constexpr int kSegGroup = 4;         // selected branch: consecutive 64-pair segments of a block per workgroup
