@@ -189,3 +189,21 @@ def test_split_step_long_context_and_paged():
             assert max_abs(out, ref) <= 8e-3
     auto, _ = nsa_decode_step(q.to(DEV), flat, gl.to(DEV), **kw)           # 8 pairs: the split path by default
     assert max_abs(auto, ref) <= 8e-3
+
+
+@pytest.mark.parametrize("S,W", [(1, 0), (64, 0), (64, 2048), (16, 1)])
+def test_split_step_extreme_selection_and_window(S, W):
+    """No window at all, one pick, more picks than blocks, a window longer than the context."""
+    from nsa_amd.decode import NSADecodeCache, nsa_decode_step
+    ctxs = [1999, 640, 70]
+    B, T, Hq, Hkv, D = len(ctxs), max(ctxs), 16, 2, 64
+    dtype = torch.float32
+    q, k, v, gl = _make(B, T, Hq, Hkv, D, D, 920, dtype)
+    cache = NSADecodeCache(B, T, Hkv, D, D, dtype=dtype, device=DEV)
+    cache.fill(k.to(DEV), v.to(DEV))
+    cache.ctx_lens.copy_(torch.tensor(ctxs, dtype=torch.int32))
+    kw = dict(selection_block=64, selected_block_count=S, sliding_window=W, return_indices=True)
+    ref, ref_idx = nsa_decode_step(q.to(DEV), cache, gl.to(DEV), splits=0, **kw)
+    out, idx = nsa_decode_step(q.to(DEV), cache, gl.to(DEV), splits=8, **kw)
+    assert torch.equal(idx, ref_idx)
+    assert torch.isfinite(out).all() and max_abs(out, ref) <= 1e-5
