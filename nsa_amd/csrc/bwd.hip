@@ -35,6 +35,7 @@ constexpr int kBwdCmp = 0, kBwdSwa = 1, kBwdSlc = 2;
 // Launch shapes, chosen by measurement on T = 32768, Hq64/Hkv4, Dk192/Dv128:
 constexpr int kCmpSplit = 384;       // tokens of one compressed-branch work item (1024: 8.6 ms, 256: 5.4 ms; with conflict-free
                                      // LDS the whole backward call: 128: 9.48, 256: 7.89, 320: 7.87, 384: 7.71, 448: 7.68, 512: 7.75)
+constexpr int kXcds = 8;             // accelerator dies; workgroup w of a launch runs on die w % 8
 constexpr int kKvWaves = 4;          // key-stationary: wavefronts (x16 keys) per workgroup, two workgroups per CU
 constexpr int kQWaves = 16;          // query-stationary: tokens per workgroup (8: 3.7 ms, 16: 3.3 ms)
 constexpr int kSegGroup = 4;         // selected branch: consecutive 64-pair segments of a block per workgroup
@@ -51,6 +52,7 @@ struct BwdArgs {
   void* dq;                       // query-stationary: [total][hq][dk]
   float* dk_acc; float* dv_acc;   // key-stationary: fp32 [key rows][hkv][.]
   SlcWs ws;                       // selected branch: bucketed pairs; ws.po = dq partials [pair][16][dk]
+  int tiles, items;               // key-stationary launch: key tiles, token items (compressed branch)
 };
 
 // Two LDS layouts of a 32-row chunk.  X32: rows padded by 32 bytes, row ownership of lane_row32; no bank
@@ -135,23 +137,38 @@ bwd_kv_kernel(const BwdArgs a) {
     count = min(a.ws.counts[key] - seg * kSeg, kSegGroup * kSeg);
     nchunks = (count + 1) >> 1;
   } else if (MODE == kBwdSwa) {
-    const SeqTile st = find_tile(a.cu_seq, a.batch, NW * 16, blockIdx.x);
+    // Workgroup w runs on XCD w % 8 (each XCD has its own L2).  Neighbouring key tiles stream almost the same
+    // tokens (a 64-key tile and its 512-token window), so every XCD takes a contiguous run of key tiles: the
+    // q / dO rows its resident workgroups stream are then fetched into that L2 once, not once per key tile.
+    const int per_xcd = (a.tiles + kXcds - 1) / kXcds;
+    const int xcd = blockIdx.x % kXcds, s = blockIdx.x / kXcds;
+    h = s / per_xcd;
+    const int tile = xcd * per_xcd + s % per_xcd;
+    if (tile >= a.tiles) return;
+    const SeqTile st = find_tile(a.cu_seq, a.batch, NW * 16, tile);
     if (!st.valid) return;
-    h = blockIdx.y;
     seq_start = st.start; key0 = st.t0; nkeys = st.len; key_base = st.start;
     t_begin = key0;
     t_end = min(key0 + NW * 16 + a.window - 1, st.len);
     nchunks = (t_end - t_begin + 1) >> 1;
   } else {
-    const SeqTile st = find_tile(a.cu_key, a.batch, NW * 16, blockIdx.y);
+    // The same idea for the compressed branch: all key tiles of one token item stream the same q / dO rows,
+    // so inside an XCD the key tile runs fastest and the token items are dealt to the XCDs round-robin.
+    const int xcd = blockIdx.x % kXcds, s = blockIdx.x / kXcds;
+    const int kt = s % a.tiles;
+    const int per_xcd = (a.items + kXcds - 1) / kXcds;
+    const int ti_local = (s / a.tiles) % per_xcd;
+    h = s / (a.tiles * per_xcd);
+    const int ti = ti_local * kXcds + xcd;
+    if (ti >= a.items) return;
+    const SeqTile st = find_tile(a.cu_key, a.batch, NW * 16, kt);
     if (!st.valid) return;
-    h = blockIdx.z;
     key0 = st.t0; nkeys = st.len; key_base = st.start;
     seq_start = a.cu_seq[st.b];
     const int seq_len = a.cu_seq[st.b + 1] - seq_start;
     const int t_first = a.causal ? key0 * a.stride + a.block : 0;
-    t_begin = max((int)blockIdx.x * kCmpSplit, t_first) & ~1;
-    t_end = min(((int)blockIdx.x + 1) * kCmpSplit, seq_len);
+    t_begin = max(ti * kCmpSplit, t_first) & ~1;
+    t_end = min((ti + 1) * kCmpSplit, seq_len);
     if (t_begin >= t_end) return;
     nchunks = (t_end - t_begin + 1) >> 1;
   }
@@ -578,10 +595,14 @@ static int launch_kv_t(const BwdArgs& a, int key_rows, hipStream_t st) {
   const int rc = set_smem(reinterpret_cast<const void*>(fn), smem);
   if (rc) return rc;
   dim3 grid;
+  BwdArgs b = a;
+  b.tiles = key_rows / (NW * 16) + a.batch;
+  b.items = (a.total + kCmpSplit - 1) / kCmpSplit;
+  const int tiles_per_xcd = (b.tiles + kXcds - 1) / kXcds, items_per_xcd = (b.items + kXcds - 1) / kXcds;
   if (MODE == kBwdSlc) grid = dim3(a.ws.items_cap);
-  else if (MODE == kBwdSwa) grid = dim3(key_rows / (NW * 16) + a.batch, a.hkv);
-  else grid = dim3((a.total + kCmpSplit - 1) / kCmpSplit, key_rows / (NW * 16) + a.batch, a.hkv);
-  hipLaunchKernelGGL(fn, grid, dim3(NW * 64), smem, st, a);
+  else if (MODE == kBwdSwa) grid = dim3(kXcds * tiles_per_xcd * a.hkv);
+  else grid = dim3(kXcds * b.tiles * items_per_xcd * a.hkv);
+  hipLaunchKernelGGL(fn, grid, dim3(NW * 64), smem, st, b);
   return 0;
 }
 
