@@ -123,7 +123,7 @@ bwd_kv_kernel(const BwdArgs a) {
 
   // ---- work item
   int h, seq_start, key0, nkeys, key_base;
-  int t_begin = 0, t_end = 0, first = 0, count = 0, nchunks;
+  int t_begin = 0, t_end = 0, first = 0, count = 0, nchunks, rot = 0;
   if (MODE == kBwdSlc) {
     const int item = blockIdx.x;
     if (item >= *a.ws.n_items) return;
@@ -151,6 +151,13 @@ bwd_kv_kernel(const BwdArgs a) {
     t_begin = key0;
     t_end = min(key0 + NW * 16 + a.window - 1, st.len);
     nchunks = (t_end - t_begin + 1) >> 1;
+    // The key tiles resident on an XCD are 64 tokens apart, so in plain order tile i would stream a token 32
+    // chunks after tile i + 1 did, long after it left the L2.  A full window spans `period` chunks and so holds
+    // every chunk number modulo `period` once: each tile starts at its multiple of `period` and wraps around,
+    // which makes the workgroups that run side by side stream the same tokens at the same time.
+    const int period = (NW * 16 + a.window) >> 1;
+    rot = (period - (t_begin >> 1) % period) % period;
+    if (rot >= nchunks) rot = 0;
   } else {
     // The same idea for the compressed branch: all key tiles of one token item stream the same q / dO rows,
     // so inside an XCD the key tile runs fastest and the token items are dealt to the XCDs round-robin.
@@ -184,6 +191,7 @@ bwd_kv_kernel(const BwdArgs a) {
       vB = 2 * c + 1 < count;
       posB = vB ? (int)(a.ws.list[first + 2 * c + 1] >> 6) - seq_start : posA;
     } else {
+      if (MODE == kBwdSwa) { c += rot; if (c >= nchunks) c -= nchunks; }
       posA = t_begin + 2 * c;
       vB = posA + 1 < t_end;
       posB = vB ? posA + 1 : posA;
