@@ -33,8 +33,9 @@ int set_smem(const void* fn, size_t bytes);
 
 constexpr int kBwdCmp = 0, kBwdSwa = 1, kBwdSlc = 2;
 // Launch shapes, chosen by measurement on T = 32768, Hq64/Hkv4, Dk192/Dv128:
-constexpr int kCmpSplit = 384;       // tokens of one compressed-branch work item (1024: 8.6 ms, 256: 5.4 ms; with conflict-free
-                                     // LDS the whole backward call: 128: 9.48, 256: 7.89, 320: 7.87, 384: 7.71, 448: 7.68, 512: 7.75)
+constexpr int kCmpSplit = 512;       // tokens of one compressed-branch work item (1024: 8.6 ms, 256: 5.4 ms; with conflict-free
+                                     // LDS the whole backward call: 128: 9.48, 256: 7.89, 320: 7.87, 384: 7.71, 448: 7.68, 512: 7.75;
+                                     // with the XCD-aware order 256: 7.25, 384: 7.2-7.4, 512: 7.07, 768: 7.74, 1024: 7.40)
 constexpr int kXcds = 8;             // accelerator dies; workgroup w of a launch runs on die w % 8
 constexpr int kKvWaves = 4;          // key-stationary: wavefronts (x16 keys) per workgroup, two workgroups per CU
 constexpr int kQWaves = 16;          // query-stationary: tokens per workgroup (8: 3.7 ms, 16: 3.3 ms)
