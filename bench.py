@@ -11,7 +11,8 @@ already resident in HBM.  Prints ONE JSON line.
 roofline: taken for the kernel stage with the largest share of the step; its algorithmic flops
 (causal compressed rows, whole valid selected blocks, exact window; nothing for exp / pooling /
 top-n or for the non-causal part of the importance scores) divided by its mean duration measured
-with events on the launch stream.  cpu_baseline: the CPU oracle (a port of the reference's naive
+with events on the launch stream; `executed` (extra) is the same with the uncredited QK^T of the keys
+a token cannot see, which the kernel multiplies for the importance normaliser.  cpu_baseline: the CPU oracle (a port of the reference's naive
 torch path) on a bounded sample of query rows of the same workload, on this host's cores.
 train_step (extra, not the headline metric): forward + backward of the same workload through the
 module's autograd path.  decode / decode_small_batch (extra): the decode step of benchmark config 5 at
@@ -350,6 +351,13 @@ def main():
     # HBM bytes per launch of that kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE (profiles/), only
     # recorded for the default workload
     traffic = MEASURED_TRAFFIC.get((args.workload, dom))
+    # The compressed-attention kernel also multiplies q with the compressed keys a token cannot see: the
+    # importance softmax is normalised over all of them.  `executed` adds that uncredited part of QK^T.
+    executed = None
+    if dom == "cmp_attn":
+        qk_all = sum(2.0 * hq * dqk * x * max((x - BLOCK) // STRIDE + 1, 0) for x in lens)
+        qk_seen = fl["cmp"] * dqk / (dqk + dv)
+        executed = (fl["cmp"] + max(qk_all - qk_seen, 0.0)) / (stage_ms[dom] * 1e-3) / 1e12
 
     res = {
         "metric": "nsa_prefill_fwd_tokens_per_s", "value": total / (ms * 1e-3), "unit": "tokens/s",
@@ -363,7 +371,8 @@ def main():
         "mfma_peak_frac_whole_step": f_eff / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
         "stage_ms": stage_ms,
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": dom_tflops, "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "frac": dom_tflops / PEAK_BF16_TFLOPS, "traffic": traffic},
+                     "unit": "TFLOP/s", "frac": dom_tflops / PEAK_BF16_TFLOPS, "traffic": traffic,
+                     "executed": executed},
         "stage_effective_tflops": stage_tflops,
     }
     if not args.no_backward:
