@@ -45,7 +45,9 @@ def _check(name, got, ref, dtype, floor=1.0):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("lens,Hq,Hkv,Dk,Dv,W", [([300], 16, 1, 64, 64, 128), ([257, 40, 130], 32, 2, 128, 128, 100),
                                                  ([200], 16, 1, 192, 128, 64), ([130], 8, 2, 64, 64, 1),
-                                                 ([150], 6, 2, 64, 64, 1000)])
+                                                 ([150], 6, 2, 64, 64, 1000),
+                                                 # 36 key tiles: several per XCD, windows that wrap around
+                                                 ([1500, 700], 16, 2, 64, 64, 200)])
 def test_swa_bwd(dtype, lens, Hq, Hkv, Dk, Dv, W):
     if dtype == torch.float32 and Dk == 192:
         pytest.skip("fp32 backward is built for head dims 64 and 128")
@@ -81,7 +83,9 @@ def test_swa_bwd(dtype, lens, Hq, Hkv, Dk, Dv, W):
                                                           ([1300, 20, 333], 32, 2, 128, 128, 32, 16, True),
                                                           ([2500], 16, 1, 192, 128, 32, 16, True),
                                                           ([260], 8, 2, 64, 64, 64, 16, True),
-                                                          ([200], 4, 1, 64, 64, 32, 16, False)])
+                                                          ([200], 4, 1, 64, 64, 32, 16, False),
+                                                          # 10 token items: more than one per XCD
+                                                          ([5000], 16, 1, 64, 64, 32, 16, True)])
 def test_cmp_attn_bwd(dtype, lens, Hq, Hkv, Dk, Dv, l, d, causal):
     if dtype == torch.float32 and Dk == 192:
         pytest.skip("fp32 backward is built for head dims 64 and 128")
