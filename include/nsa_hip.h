@@ -244,6 +244,8 @@ int nsa_cmp_attn_bwd(const void* q, const void* ck, const void* cv, const void* 
  *   nsa_slc_combine_fwd (64-key blocks only).  dq [total,hq,dk], dk_out [total,hkv,dk], dv_out
  *   [total,hkv,dv] receive the sums over the branches present and are fully overwritten.
  *   delta_* / rowscale_* (optional, float [total,hq]) as in nsa_cmp_attn_bwd, per branch.
+ *   dq_add (optional, [total,hq,dk], must not overlap dq): added to dq in the kernel that writes it, e.g. the
+ *   dq of nsa_cmp_attn_bwd, so that the sum over all three branches needs no further pass.
  *   workspace: nsa_slc_swa_bwd_workspace_bytes (pass top_n = 0 there when the selected branch is
  *   skipped). */
 int64_t nsa_slc_swa_bwd_workspace_bytes(int total, int batch, int hq, int hkv, int dk, int dv, int top_n,
@@ -254,7 +256,7 @@ int nsa_slc_swa_bwd(const void* q, const void* k, const void* v, const void* o_s
                     const float* rowscale_swa, const void* indices, const int32_t* counts,
                     const int32_t* cu_seqlens, int batch, int total, int hq,
                     int hkv, int dk, int dv, int top_n, int block_size, int window, float scale, int idx64, int dtype,
-                    void* dq, void* dk_out, void* dv_out, void* workspace, int64_t workspace_bytes,
+                    const void* dq_add, void* dq, void* dk_out, void* dv_out, void* workspace, int64_t workspace_bytes,
                     nsa_stream_t stream);
 
 /* One-token decode step (no counterpart in the reference, which has no cache and no single-token

@@ -178,8 +178,7 @@ class NSACoreFn(torch.autograd.Function):
                                           causal=causal, delta=st[2], rowscale=st[5])
         dq, dk, dv = ops.slc_swa_bwd(q, k, v, None, d_out, lse_slc, None, d_out if o_swa is not None else None,
                                      lse_swa, idx, None, cu, batch, sel_block, window, scale, delta_slc=st[0],
-                                     delta_swa=st[1], rowscale_slc=st[3], rowscale_swa=st[4])
-        dq += dq_c
+                                     delta_swa=st[1], rowscale_slc=st[3], rowscale_swa=st[4], dq_add=dq_c)
         return (dq, dck, dcv, dk, dv, d_gl.to(gate_logits.dtype)) + (None,) * 11
 
 

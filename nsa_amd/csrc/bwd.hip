@@ -560,11 +560,13 @@ bwd_cast_kernel(const float* __restrict__ src, T* __restrict__ dst, long n8) {
   store8(dst + i * 8, pack8<T>(v));
 }
 
-// dq[token][head][8 channels] = (dq_in) + sum over the token's usable picks of the pair partials
-template <typename T, int DK>
+// dq[token][head][8 channels] = (dq_in) + (dq_add) + sum over the token's usable picks of the pair partials.
+// TOPN > 0: top_n == TOPN, the slot map is read with vector loads and all partials of the piece are
+// requested before any is summed; TOPN = 0: any top_n (0 included), one partial at a time.
+template <typename T, int DK, int TOPN>
 __global__ void __launch_bounds__(256)
 slc_dq_merge_kernel(const int* __restrict__ slotmap, const T* __restrict__ part, const T* __restrict__ dq_in,
-                    T* __restrict__ dq, long total, int hq, int hkv, int top_n) {
+                    const T* __restrict__ dq_add, T* __restrict__ dq, long total, int hq, int hkv, int top_n) {
   constexpr int PPR = DK / 8;
   const long id = (long)blockIdx.x * 256 + threadIdx.x;
   if (id >= total * hq * PPR) return;
@@ -577,19 +579,38 @@ slc_dq_merge_kernel(const int* __restrict__ slotmap, const T* __restrict__ part,
   float acc[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-  if (dq_in != nullptr) {
-    const vec8_t<T> x = load8(dq_in + row * DK + pc * 8);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] = (float)x[e];
-  }
+  vec8_t<T> x0 = zero8<T>(), x1 = zero8<T>();
+  if (dq_in != nullptr) x0 = load8(dq_in + row * DK + pc * 8);
+  if (dq_add != nullptr) x1 = load8(dq_add + row * DK + pc * 8);
   const long base = (tg * hkv + h) * top_n;
-  for (int i = 0; i < top_n; ++i) {
-    const long p = slotmap[base + i];
-    if (p < 0) continue;
-    const vec8_t<T> x = load8(part + (p * 16 + n) * DK + pc * 8);
+  if constexpr (TOPN > 0) {
+    int ps[TOPN];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] += (float)x[e];
+    for (int i = 0; i < TOPN / 4; ++i) {
+      const int4 q4 = *reinterpret_cast<const int4*>(slotmap + base + 4 * i);
+      ps[4 * i] = q4.x; ps[4 * i + 1] = q4.y; ps[4 * i + 2] = q4.z; ps[4 * i + 3] = q4.w;
+    }
+    vec8_t<T> x[TOPN];
+#pragma unroll
+    for (int i = 0; i < TOPN; ++i) {
+      x[i] = zero8<T>();
+      if (ps[i] >= 0) x[i] = load8(part + ((long)ps[i] * 16 + n) * DK + pc * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < TOPN; ++i)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += (float)x[i][e];
+  } else {
+    for (int i = 0; i < top_n; ++i) {
+      const long p = slotmap[base + i];
+      if (p < 0) continue;
+      const vec8_t<T> x = load8(part + (p * 16 + n) * DK + pc * 8);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += (float)x[e];
+    }
   }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] += (float)x0[e] + (float)x1[e];
   store8(dq + row * DK + pc * 8, pack8<T>(acc));
 }
 
@@ -728,9 +749,9 @@ static int launch_slc_swa_bwd_t(const SlcSwaBwdArgs& c, hipStream_t st) {
     if (rc == 0) rc = launch_kv_t<T, DK, DV, kBwdSwa, kKvWaves>(a, c.total, st);
     if (rc) return rc;
   }
+  SlcWs ws{};
   if (slc) {
     const SlcArgs s = slc_args_of(c);
-    SlcWs ws;
     slc_carve(s, base + off, &ws, sizeof(T), DK);
     rc = launch_slc_bucket(s, ws, st);
     if (rc) return rc;
@@ -739,11 +760,22 @@ static int launch_slc_swa_bwd_t(const SlcSwaBwdArgs& c, hipStream_t st) {
     a.rowscale = c.rowscale_slc; a.ws = ws;
     rc = launch_kv_t<T, DK, DV, kBwdSlc, 4>(a, c.total, st);
     if (rc) return rc;
+  }
+  if (slc || c.dq_add != nullptr) {          // dq = window dQ + partials of the selected branch + dq_add
     const long threads = (long)c.total * c.hq * (DK / 8);
-    hipLaunchKernelGGL((slc_dq_merge_kernel<T, DK>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st,
-                       ws.slotmap, reinterpret_cast<const T*>(ws.po),
-                       swa ? reinterpret_cast<const T*>(c.dq) : nullptr, reinterpret_cast<T*>(c.dq),
-                       (long)c.total, c.hq, c.hkv, c.top_n);
+    const dim3 grid((unsigned)((threads + 255) / 256));
+    const int* slotmap = slc ? ws.slotmap : nullptr;
+    const T* part = slc ? reinterpret_cast<const T*>(ws.po) : nullptr;
+    const T* dq_in = swa ? reinterpret_cast<const T*>(c.dq) : nullptr;
+    const int top_n = slc ? c.top_n : 0;
+    if (top_n == 16)
+      hipLaunchKernelGGL((slc_dq_merge_kernel<T, DK, 16>), grid, dim3(256), 0, st, slotmap, part, dq_in,
+                         reinterpret_cast<const T*>(c.dq_add), reinterpret_cast<T*>(c.dq), (long)c.total, c.hq, c.hkv,
+                         top_n);
+    else
+      hipLaunchKernelGGL((slc_dq_merge_kernel<T, DK, 0>), grid, dim3(256), 0, st, slotmap, part, dq_in,
+                         reinterpret_cast<const T*>(c.dq_add), reinterpret_cast<T*>(c.dq), (long)c.total, c.hq, c.hkv,
+                         top_n);
   } else if (!swa) {
     fill_zero(reinterpret_cast<float*>(c.dq), (long)c.total * c.hq * DK * (long)sizeof(T) / 4, st);
   }

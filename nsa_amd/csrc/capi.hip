@@ -382,10 +382,12 @@ int nsa_slc_swa_bwd(const void* q, const void* k, const void* v, const void* o_s
                     const float* rowscale_swa, const void* indices, const int32_t* counts,
                     const int32_t* cu_seqlens, int batch, int total, int hq,
                     int hkv, int dk, int dv, int top_n, int block_size, int window, float scale, int idx64, int dtype,
-                    void* dq, void* dk_out, void* dv_out, void* workspace, int64_t workspace_bytes,
-                    nsa_stream_t stream) {
+                    const void* dq_add, void* dq, void* dk_out, void* dv_out, void* workspace,
+                    int64_t workspace_bytes, nsa_stream_t stream) {
   if (!q || !k || !v || !cu_seqlens || !dq || !dk_out || !dv_out || !workspace)
     return fail(NSA_ERR_INVALID, "slc_swa_bwd: null pointer");
+  if (dq_add && (dq_add == dq || !aligned16(dq_add)))
+    return fail(NSA_ERR_INVALID, "slc_swa_bwd: dq_add must be 16-byte aligned and must not be dq");
   const bool slc = d_o_slc != nullptr, swa = d_o_swa != nullptr;
   if (slc && ((!o_slc && !delta_slc) || !lse_slc || !indices || top_n <= 0)) return fail(NSA_ERR_INVALID, "slc_swa_bwd: the selected branch needs o_slc, lse_slc, indices and top_n > 0");
   if (swa && ((!o_swa && !delta_swa) || !lse_swa || window <= 0)) return fail(NSA_ERR_INVALID, "slc_swa_bwd: the sliding branch needs o_swa, lse_swa and window > 0");
@@ -403,7 +405,7 @@ int nsa_slc_swa_bwd(const void* q, const void* k, const void* v, const void* o_s
     return fail(NSA_ERR_INVALID, "slc_swa_bwd: workspace smaller than nsa_slc_swa_bwd_workspace_bytes");
   nsa::SlcSwaBwdArgs a{q, k, v, o_slc, o_swa, d_o_slc, d_o_swa, lse_slc, lse_swa, indices, counts, cu_seqlens, batch,
                        total, hq, hkv, dk, dv, slc ? top_n : 0, block_size, swa ? window : 0, scale, idx64, dtype, dq,
-                       dk_out, dv_out, workspace, delta_slc, delta_swa, rowscale_slc, rowscale_swa};
+                       dk_out, dv_out, workspace, delta_slc, delta_swa, rowscale_slc, rowscale_swa, dq_add};
   const int rc = nsa::launch_slc_swa_bwd(a, stream);
   if (rc == -2) return fail(NSA_ERR_UNSUPPORTED, "slc_swa_bwd: head dims not built (dk,dv in (64,64),(128,128),(192,128); fp32: no 192)");
   return finish(rc, "slc_swa_bwd");

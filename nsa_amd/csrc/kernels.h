@@ -82,6 +82,7 @@ struct SlcSwaBwdArgs {
   int batch, total, hq, hkv, dk, dv, top_n, block_size, window; float scale; int idx64, dtype;
   void* dq; void* dk_out; void* dv_out; void* workspace;
   const float* delta_slc; const float* delta_swa; const float* rowscale_slc; const float* rowscale_swa;   // as above
+  const void* dq_add;        // optional [total][hq][dk]: added to dq (the compressed branch's dQ); not dq itself
 };
 
 // Gated sum of the branches (d_out == nullptr: forward into out) or its backward (d_out given:

@@ -333,10 +333,12 @@ def cmp_attn_bwd(q, ck, cv, o, d_o, lse_attn, cu_seqlens, cu_cmp, batch, block, 
 
 
 def slc_swa_bwd(q, k, v, o_slc, d_o_slc, lse_slc, o_swa, d_o_swa, lse_swa, indices, counts, cu_seqlens, batch,
-                block_size, window, scale, delta_slc=None, delta_swa=None, rowscale_slc=None, rowscale_swa=None):
+                block_size, window, scale, delta_slc=None, delta_swa=None, rowscale_slc=None, rowscale_swa=None,
+                dq_add=None):
     """Backward of the selected (o_slc / d_o_slc / lse_slc, or None) and sliding (o_swa / d_o_swa /
     lse_swa, or None) branches.  v is the row-major [total,Hkv,Dv] tensor.  delta_* / rowscale_* as in
-    cmp_attn_bwd (with delta_* the matching o_* may be None).  Returns (dq, dk, dv), each the sum over
+    cmp_attn_bwd (with delta_* the matching o_* may be None).  dq_add (optional, shape of q): added to dq
+    by the kernel that writes it (the compressed branch's dq).  Returns (dq, dk, dv), each the sum over
     the branches given."""
     _need_cuda(q, k, v, cu_seqlens)
     q, k, v = _dense(q), _dense(k), _dense(v)
@@ -354,6 +356,10 @@ def slc_swa_bwd(q, k, v, o_slc, d_o_slc, lse_slc, o_swa, d_o_swa, lse_swa, indic
     if swa_:
         o_swa, d_o_swa = (None if o_swa is None else _dense(o_swa)), _dense(d_o_swa)
     dq, dk_out, dv_out = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    if dq_add is not None:
+        if dq_add.shape != q.shape or dq_add.dtype != q.dtype:
+            raise ValueError("dq_add must have the shape and dtype of q")
+        dq_add = _dense(dq_add)
     lib = _lib.load()
     need = lib.nsa_slc_swa_bwd_workspace_bytes(total, batch, hq, hkv, dk, dv, top_n, block_size, _dtype_code(q))
     ws = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
@@ -364,7 +370,8 @@ def slc_swa_bwd(q, k, v, o_slc, d_o_slc, lse_slc, o_swa, d_o_swa, lse_swa, indic
         _ptr(rowscale_slc if slc else None), _ptr(rowscale_swa if swa_ else None),
         _ptr(indices if slc else None), _ptr(counts if slc else None),
         _ptr(cu_seqlens), batch, total, hq, hkv, dk, dv, top_n, block_size, window if swa_ else 0, float(scale),
-        int(slc and indices.dtype == torch.int64), _dtype_code(q), _ptr(dq), _ptr(dk_out), _ptr(dv_out), _ptr(ws),
+        int(slc and indices.dtype == torch.int64), _dtype_code(q), _ptr(dq_add), _ptr(dq), _ptr(dk_out), _ptr(dv_out),
+        _ptr(ws),
         ws.numel(), _stream())
     _lib.check(rc, "nsa_slc_swa_bwd")
     return dq, dk_out, dv_out

@@ -182,6 +182,45 @@ def test_slc_swa_bwd(lens, Hq, Hkv, Dk, Dv, S, W):
 
 # ------------------------------------------------------------------------------ compression
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("S,W", [(16, 100), (4, 0), (0, 64)])
+def test_slc_swa_bwd_dq_add(dtype, S, W):
+    """dq_add is summed into dq by the kernel that writes it: dk / dv unchanged, dq = plain result + dq_add (to
+    one rounding of the output type).  top_n 16 takes the unrolled merge, 4 the loop, 0 the window-only path."""
+    if dtype == torch.float32 and S > 0:
+        pytest.skip("the selected branch saves its log-sum-exp on the bf16 path only")
+    lens, Hq, Hkv, D, bs = [300, 77], 16, 1, 64, 64
+    ops = _ops()
+    T = sum(lens)
+    q, k, v, _ = make_qkv(T, Hq, Hkv, D, D, 180, dtype, 0.7)
+    d_o = randn(T, Hq, D, seed=181, dtype=dtype).to(DEV)
+    extra = randn(T, Hq, D, seed=182, dtype=dtype).to(DEV)
+    cu, cuh = _cu(lens), ragged_cu(lens)
+    scale = 1.0 / math.sqrt(D)
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    vt = ops.transpose(vd, cu, len(lens))
+    idx = o_slc = lse_slc = o_swa = lse_swa = None
+    if S > 0:
+        idx = torch.cat([_random_indices(e - s, Hkv, S, bs, 183 + s) for s, e in zip(cuh[:-1], cuh[1:])]).to(DEV)
+        o_slc, lse_slc = ops.slc_combine(qd, kd, vt, idx, None, None, None, None, None, None, cu, len(lens), bs, scale,
+                                         block_major=True, want_lse=True)
+    if W > 0:
+        o_swa, lse_swa = ops.swa(qd, kd, vt, cu, len(lens), W, scale, want_lse=True)
+    args = (qd, kd, vd, o_slc, d_o if S > 0 else None, lse_slc, o_swa, d_o if W > 0 else None, lse_swa, idx, None, cu,
+            len(lens), bs, W, scale)
+    dq0, dk0, dv0 = ops.slc_swa_bwd(*args)
+    dq1, dk1, dv1 = ops.slc_swa_bwd(*args, dq_add=extra)
+    tol = 2.0 ** -7 if dtype == torch.bfloat16 else 1e-5
+    for a, b in ((dk0, dk1), (dv0, dv1)):      # fp32 atomics: the order of the sums differs from run to run
+        assert float((a.double() - b.double()).abs().max()) <= tol * max(1.0, float(a.abs().max()))
+    ref = dq0.double() + extra.double()
+    err = float((dq1.double() - ref).abs().max())
+    mag = max(1.0, float(ref.abs().max()))
+    assert err <= tol * mag, err
+    with pytest.raises(ValueError):
+        ops.slc_swa_bwd(*args, dq_add=extra[:, :, :32])
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("lens,H,D,l,d", [([300], 1, 64, 32, 16), ([300, 31, 64, 1000], 4, 128, 32, 16),
                                           ([200, 77], 2, 192, 64, 16), ([90], 2, 32, 8, 4)])
 def test_compress_mean_bwd(dtype, lens, H, D, l, d):

@@ -138,14 +138,18 @@ def test_backward_argument_errors_do_not_launch(lib):
     assert lib.nsa_cmp_attn_bwd_workspace_bytes(64, 2, 16, 1, 64, 64) >= 64 * 16 * 4 + 2 * 2 * 64 * 4
     # selected + sliding backward: a branch needs its saved tensors, the selected one 64-key blocks
     rc = lib.nsa_slc_swa_bwd(p, p, p, None, None, p, None, None, None, None, None, None, None, None, None, p, 1, 64, 16, 1, 64, 64, 4, 64, 0, 0.1, 1,
-                             0, p, p, p, p, 1 << 30, None)
+                             0, None, p, p, p, p, 1 << 30, None)
     assert rc == -1 and b"selected branch" in lib.nsa_last_error_string()
-    rc = lib.nsa_slc_swa_bwd(p, p, p, p, None, p, None, p, None, None, None, None, None, p, None, p, 1, 64, 16, 1, 64, 64, 4, 32, 0, 0.1, 1, 0, p, p,
+    rc = lib.nsa_slc_swa_bwd(p, p, p, p, None, p, None, p, None, None, None, None, None, p, None, p, 1, 64, 16, 1, 64, 64, 4, 32, 0, 0.1, 1, 0, None, p, p,
                              p, p, 1 << 30, None)
     assert rc == -2 and b"64-key" in lib.nsa_last_error_string()
-    rc = lib.nsa_slc_swa_bwd(p, p, p, None, p, None, p, None, p, None, None, None, None, None, None, p, 1, 64, 16, 1, 64, 64, 0, 64, 0, 0.1, 1, 0, p, p,
+    rc = lib.nsa_slc_swa_bwd(p, p, p, None, p, None, p, None, p, None, None, None, None, None, None, p, 1, 64, 16, 1, 64, 64, 0, 64, 0, 0.1, 1, 0, None, p, p,
                              p, p, 1 << 30, None)
     assert rc == -1 and b"sliding branch" in lib.nsa_last_error_string()
+    # dq_add must not be the output itself
+    rc = lib.nsa_slc_swa_bwd(p, p, p, None, p, None, p, None, p, None, None, None, None, None, None, p, 1, 64, 16, 1, 64, 64, 0, 64, 64, 0.1, 1, 0, p, p,
+                             p, p, p, 1 << 30, None)
+    assert rc == -1 and b"dq_add" in lib.nsa_last_error_string()
     need = lib.nsa_slc_swa_bwd_workspace_bytes(64, 1, 16, 1, 64, 64, 4, 64, 0)
     assert need > lib.nsa_slc_swa_bwd_workspace_bytes(64, 1, 16, 1, 64, 64, 0, 64, 0) > 0
     # compression, gates
