@@ -200,7 +200,10 @@ int nsa_slc_combine_fwd(const void* q, const void* k, const void* vt, const void
  *                          out = act(g_slc)*o_slc + act(g_swa)*o_swa + act(g_cmp)*o_cmp (o_cmp may be
  *                          NULL).  Must follow nsa_slc_partials_fwd on the same stream with the same
  *                          sizes; the workspace is only read (its slot map tells which picks have
- *                          a partial).
+ *                          a partial).  Optional outputs for a backward pass, written by the same
+ *                          epilogue: o_slc_out / o_swa_out [total,hq,dv] (ungated branch outputs),
+ *                          lse_slc_out / lse_swa_out (float [total,hq], as lse_slc above and lse of
+ *                          nsa_swa_fwd).
  * bf16, 64-key selection blocks; other shapes return NSA_ERR_UNSUPPORTED (use nsa_swa_fwd +
  * nsa_slc_combine_fwd). */
 int nsa_slc_partials_fwd(const void* q, const void* k, const void* vt, const void* indices, const int32_t* counts,
@@ -211,6 +214,7 @@ int nsa_swa_merge_fwd(const void* q, const void* k, const void* vt, const void* 
                       const void* g_cmp, int64_t gate_stride, const void* o_cmp, void* out,
                       const int32_t* cu_seqlens, int batch, int total, int hq, int hkv, int dk, int dv, int vt_cols,
                       int window, int top_n, int block_size, float scale, int gate_act, int dtype,
+                      void* o_slc_out, void* o_swa_out, float* lse_slc_out, float* lse_swa_out,
                       const void* workspace, int64_t workspace_bytes, nsa_stream_t stream);
 
 /* Bytes of the optional workspace of nsa_slc_combine_fwd; 0 when the shape has no block-major path

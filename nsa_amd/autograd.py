@@ -154,12 +154,23 @@ class NSACoreFn(torch.autograd.Function):
         pk, ps, pp, top_n, max_nc = select
         idx, _ = ops.block_select(q, ck, lse_raw, cu, cu_cmp, batch, hkv, hkv * dk, dk, pk, ps, pp, top_n, max_nc,
                                   idx64=False)
-        o_slc, lse_slc = ops.slc_combine(q, k, vt, idx, None, None, None, None, None, None, cu, batch, sel_block,
-                                         scale, block_major=True, want_lse=True)
-        o_swa = lse_swa = None
-        if window > 0:
-            o_swa, lse_swa = ops.swa(q, k, vt, cu, batch, window, scale, want_lse=True)
-        out = ops.gate_combine(gate_logits, o_slc, o_swa, o_cmp, gate_act)
+        ws = ops.slc_workspace(q, hkv, dv, idx.shape[-1], sel_block, batch) if window > 0 else None
+        gl = gate_logits.reshape(-1, 3)
+        if ws is not None and gl.dtype == q.dtype:
+            # the inference schedule (partials per block, merged in the window kernel's epilogue), which also
+            # leaves the ungated branch outputs and their log-sum-exps for the backward
+            ops.slc_partials(q, k, vt, idx, None, cu, batch, sel_block, scale, ws)
+            g_slc, g_swa, g_cmp = (gl[:, i].view(q.shape[0], q.shape[1]) for i in range(3))
+            out, o_slc, o_swa, lse_slc, lse_swa = ops.swa_merge(
+                q, k, vt, ws, idx.shape[-1], g_slc, g_swa, g_cmp, o_cmp, cu, batch, sel_block, window, scale,
+                gate_act=gate_act, want_branches=True)
+        else:
+            o_slc, lse_slc = ops.slc_combine(q, k, vt, idx, None, None, None, None, None, None, cu, batch, sel_block,
+                                             scale, block_major=True, want_lse=True)
+            o_swa = lse_swa = None
+            if window > 0:
+                o_swa, lse_swa = ops.swa(q, k, vt, cu, batch, window, scale, want_lse=True)
+            out = ops.gate_combine(gate_logits, o_slc, o_swa, o_cmp, gate_act)
         ctx.save_for_backward(q, ck, cv, k, v, gate_logits, o_cmp, lse_cmp, o_slc, lse_slc, o_swa, lse_swa, idx, cu,
                               cu_cmp)
         ctx.geom = (batch, block, stride, sel_block, window, scale, causal, gate_act)

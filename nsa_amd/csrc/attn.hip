@@ -585,7 +585,7 @@ static int launch_swa_t(const SwaArgs& a, hipStream_t st) {
 template <int DK, int DV>
 static int launch_swa_merge_t(const SwaArgs& a, const MergeArgs& m, hipStream_t st) {
   StreamParams p{a.q, a.k, a.vt, nullptr, nullptr, a.cu_seq, a.cu_seq, a.batch, a.hq, a.hkv, (long)a.hkv * DK,
-                 (long)DK, a.vt_cols, 0, 0, a.window, 1, a.scale, m, nullptr};
+                 (long)DK, a.vt_cols, 0, 0, a.window, 1, a.scale, m, a.lse};
   if (m.top_n == 16) return launch_stream_t<bf16_t, DK, DV, false, 16>(p, a.total, st);
   return launch_stream_t<bf16_t, DK, DV, false, 1>(p, a.total, st);
 }

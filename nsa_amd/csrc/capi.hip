@@ -320,8 +320,11 @@ int nsa_swa_merge_fwd(const void* q, const void* k, const void* vt, const void* 
                       const void* g_cmp, int64_t gate_stride, const void* o_cmp, void* out,
                       const int32_t* cu_seqlens, int batch, int total, int hq, int hkv, int dk, int dv, int vt_cols,
                       int window, int top_n, int block_size, float scale, int gate_act, int dtype,
+                      void* o_slc_out, void* o_swa_out, float* lse_slc_out, float* lse_swa_out,
                       const void* workspace, int64_t workspace_bytes, nsa_stream_t stream) {
   if (!out) return fail(NSA_ERR_INVALID, "swa_merge: null pointer");
+  if ((o_slc_out && !aligned16(o_slc_out)) || (o_swa_out && !aligned16(o_swa_out)))
+    return fail(NSA_ERR_INVALID, "swa_merge: pointers must be 16-byte aligned");
   if (window <= 0) return fail(NSA_ERR_INVALID, "swa_merge: window must be positive");
   if (gate_act != NSA_GATE_IDENTITY && gate_act != NSA_GATE_SIGMOID) return fail(NSA_ERR_INVALID, "swa_merge: bad gate activation");
   if (int rc = slc_common_checks("swa_merge", q, k, vt, cu_seqlens, batch, total, hq, hkv, dk, dv, vt_cols, top_n,
@@ -331,8 +334,10 @@ int nsa_swa_merge_fwd(const void* q, const void* k, const void* vt, const void* 
   nsa::SlcArgs sa{q, k, vt, nullptr, nullptr, g_slc, g_swa, g_cmp, (long)gate_stride, nullptr, o_cmp, out, cu_seqlens,
                   batch, total, hq, hkv, dk, dv, vt_cols, top_n, block_size, scale, 0, gate_act, dtype,
                   const_cast<void*>(workspace), (long)workspace_bytes, nullptr};
-  const nsa::MergeArgs m = nsa::slc_merge_args(sa, const_cast<void*>(workspace));
-  nsa::SwaArgs a{q, k, vt, nullptr, cu_seqlens, batch, total, hq, hkv, dk, dv, vt_cols, window, scale, dtype, nullptr};
+  nsa::MergeArgs m = nsa::slc_merge_args(sa, const_cast<void*>(workspace));
+  m.o_slc_out = o_slc_out; m.o_swa_out = o_swa_out; m.lse_slc_out = lse_slc_out;
+  nsa::SwaArgs a{q, k, vt, nullptr, cu_seqlens, batch, total, hq, hkv, dk, dv, vt_cols, window, scale, dtype,
+                 lse_swa_out};
   return finish(nsa::launch_swa_merge(a, m, stream), "swa_merge");
 }
 

@@ -58,6 +58,9 @@ struct MergeArgs {
   const void* o_cmp; void* out;
   int top_n, hq, hkv, gate_act; float scale;
   float* lse;        // optional: log-sum-exp of the selected branch per (token, q head)
+  // optional, written by merge_piece (what a backward pass keeps): the ungated, normalised selected and
+  // sliding outputs [total,hq,dv] and the selected branch's log-sum-exp
+  void* o_slc_out; void* o_swa_out; float* lse_slc_out;
 };
 
 // Backward of the compressed branch: all tensors packed and contiguous; lse is the natural-log

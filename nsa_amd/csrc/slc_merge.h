@@ -20,7 +20,7 @@ __device__ __forceinline__ vec8_t<T> merge_piece(const MergeArgs& m, long tg, in
   const long base = (tg * m.hkv + h) * m.top_n;
   const float c_attn = m.scale * kLog2e;
   const T* pob = reinterpret_cast<const T*>(m.po);
-  float den = 0.f, acc[8];
+  float den = 0.f, acc[8], M = kNegInf;
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.f;
   if constexpr (TOPN > 0) {
@@ -42,7 +42,6 @@ __device__ __forceinline__ vec8_t<T> merge_piece(const MergeArgs& m, long tg, in
         o[i] = load8(pob + (p * 16 + n) * DV + pc * 8);
       }
     }
-    float M = kNegInf;
 #pragma unroll
     for (int i = 0; i < TOPN; ++i) M = fmaxf(M, mx[i]);
 #pragma unroll
@@ -55,7 +54,6 @@ __device__ __forceinline__ vec8_t<T> merge_piece(const MergeArgs& m, long tg, in
       }
     }
   } else {
-    float M = kNegInf;
     for (int i = 0; i < m.top_n; ++i) {
       const long p = m.slotmap[base + i];
       if (p < 0) continue;
@@ -72,6 +70,15 @@ __device__ __forceinline__ vec8_t<T> merge_piece(const MergeArgs& m, long tg, in
     }
   }
   const float inv = den > 0.f ? 1.0f / den : 0.f;
+  if (m.o_slc_out != nullptr) {
+    float os[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) os[e] = acc[e] * inv;
+    store8(reinterpret_cast<T*>(m.o_slc_out) + row * DV + pc * 8, pack8<T>(os));
+  }
+  if (m.o_swa_out != nullptr && has_swa) store8(reinterpret_cast<T*>(m.o_swa_out) + row * DV + pc * 8, o_swa);
+  if (m.lse_slc_out != nullptr && pc == 0)
+    m.lse_slc_out[row] = den > 0.f ? fmaf(M, m.scale, __logf(den)) : __builtin_huge_valf();
   const T* gs = reinterpret_cast<const T*>(m.g_slc);
   const T* gw = reinterpret_cast<const T*>(m.g_swa);
   const T* gcm = reinterpret_cast<const T*>(m.g_cmp);

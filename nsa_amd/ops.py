@@ -276,10 +276,12 @@ def slc_partials(q, k, vt, indices, counts, cu_seqlens, batch, block_size, scale
 
 
 def swa_merge(q, k, vt, workspace, top_n, g_slc, g_swa, g_cmp, o_cmp, cu_seqlens, batch, block_size, window,
-              scale, gate_act=0):
+              scale, gate_act=0, want_branches=False):
     """Second half: sliding-window attention whose epilogue merges the partials slc_partials left in
     `workspace` (same sizes, top_n picks per token and kv head), applies the gates and adds the
-    compressed branch.  Returns the final output [total,Hq,dv]."""
+    compressed branch.  Returns the final output [total,Hq,dv]; with want_branches also what a backward
+    pass keeps: (out, o_slc, o_swa, lse_slc, lse_swa), the ungated branch outputs and their float32
+    [total,Hq] log-sum-exps."""
     _need_cuda(q, k, vt, cu_seqlens, workspace)
     q, k = _dense(q), _dense(k)
     total, hq, dk = q.shape
@@ -287,12 +289,18 @@ def swa_merge(q, k, vt, workspace, top_n, g_slc, g_swa, g_cmp, o_cmp, cu_seqlens
     (g_slc, g_swa, g_cmp), gs = _gate_views([g_slc, g_swa, g_cmp], q)
     o_cmp = None if o_cmp is None else _dense(o_cmp)
     out = torch.empty(total, hq, dv, dtype=q.dtype, device=q.device)
+    o_slc = o_swa = lse_slc = lse_swa = None
+    if want_branches:
+        o_slc, o_swa = torch.empty_like(out), torch.empty_like(out)
+        lse_slc = torch.empty(total, hq, dtype=torch.float32, device=q.device)
+        lse_swa = torch.empty_like(lse_slc)
     rc = _lib.load().nsa_swa_merge_fwd(
         _ptr(q), _ptr(k), _ptr(vt), _ptr(g_slc), _ptr(g_swa), _ptr(g_cmp), gs, _ptr(o_cmp), _ptr(out),
         _ptr(cu_seqlens), batch, total, hq, hkv, dk, dv, vt.shape[-1], window, top_n, block_size, float(scale),
-        gate_act, _dtype_code(q), _ptr(workspace), workspace.numel(), _stream())
+        gate_act, _dtype_code(q), _ptr(o_slc), _ptr(o_swa), _ptr(lse_slc), _ptr(lse_swa), _ptr(workspace),
+        workspace.numel(), _stream())
     _lib.check(rc, "nsa_swa_merge_fwd")
-    return out
+    return (out, o_slc, o_swa, lse_slc, lse_swa) if want_branches else out
 
 
 def gate_logits(q, weight, bias=None):

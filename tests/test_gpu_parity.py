@@ -268,6 +268,18 @@ def test_fused_partials_and_window_merge(lens, Hq, Hkv, Dk, Dv, S, W):
         d = max_abs(fused, split)
         print("fused", lens, (Hq, Hkv, Dk, Dv, S, W), "counts", use_counts, "vs oracle", err, "vs split kernels", d)
         assert err <= TOL[dtype] and d <= TOL[dtype]
+        # the same launch can also leave what a backward pass keeps: the ungated branch outputs and their
+        # log-sum-exps, equal to those of the stand-alone kernels
+        out2, b_slc, b_swa, l_slc, l_swa = ops.swa_merge(qd, kd, vt, ws, S, g_slc, g_swa, g_cmp, o_cmp.to(DEV), cu,
+                                                         len(lens), bs, W, scale, gate_act=1, want_branches=True)
+        r_slc, rl_slc = ops.slc_combine(qd, kd, vt, idd, cd, None, None, None, None, None, cu, len(lens), bs, scale,
+                                        block_major=True, want_lse=True)
+        r_swa, rl_swa = ops.swa(qd, kd, vt, cu, len(lens), W, scale, want_lse=True)
+        assert torch.equal(out2.cpu(), fused)
+        assert torch.equal(b_slc, r_slc) and torch.equal(b_swa, r_swa) and torch.equal(l_swa, rl_swa)
+        fin = torch.isfinite(rl_slc)
+        assert torch.equal(fin, torch.isfinite(l_slc)) and torch.equal(l_slc[~fin], rl_slc[~fin])
+        assert float((l_slc[fin] - rl_slc[fin]).abs().max()) <= 1e-5 if fin.any() else True
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
