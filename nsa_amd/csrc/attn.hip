@@ -332,9 +332,29 @@ stream_attn_kernel(const StreamParams a) {
     const float inv = lt > 0.f ? 1.0f / lt : 0.f;
     const long row = ((long)st.start + rm[j].tok) * a.hq + h * G + rm[j].gidx;
     store_rows<T, DV>(stage + n * OLD, grp[j].o, inv, g);
-    {
-      constexpr int PIECES = DV / 8;
-      const int gi = wave * NG + j;
+    constexpr int PIECES = DV / 8;
+    const int gi = wave * NG + j;
+    if constexpr (MERGE == 16) {
+      // a lane takes two pieces (pc, pc + PIECES / 2) of one row, so that 32 partial loads are in flight per lane
+      constexpr int HALF = PIECES / 2;
+#pragma unroll
+      for (int k = 0; k < (16 * HALF + 63) / 64; ++k) {
+        const int e = lane + 64 * k;
+        const int r = e / HALF, pc = e % HALF;
+        if (16 * HALF % 64 == 0 || r < 16) {
+          const RowMap rr = map_row(st.t0, gi, r, lgp, G, st.len);
+          if (rr.valid) {
+            const long tg = (long)st.start + rr.tok;
+            const long orow = tg * a.hq + h * G + rr.gidx;
+            const vec8_t<T> pa = load8(stage + r * OLD + pc * 8), pb = load8(stage + r * OLD + (pc + HALF) * 8);
+            vec8_t<T> ra, rb;
+            merge_two<T, DV, 16>(a.mg, tg, h, rr.gidx, orow, pc, pc + HALF, pa, pb, ra, rb);
+            store8(reinterpret_cast<T*>(a.mg.out) + orow * DV + pc * 8, ra);
+            store8(reinterpret_cast<T*>(a.mg.out) + orow * DV + (pc + HALF) * 8, rb);
+          }
+        }
+      }
+    } else {
 #pragma unroll
       for (int k = 0; k < (16 * PIECES + 63) / 64; ++k) {
         const int e = lane + 64 * k;
@@ -348,7 +368,7 @@ stream_attn_kernel(const StreamParams a) {
             if constexpr (MERGE == 0) {
               store8(ob + orow * DV + pc * 8, piece);
             } else {
-              const vec8_t<T> res = merge_piece<T, DV, (MERGE == 16 ? 16 : 0)>(a.mg, tg, h, rr.gidx, orow, pc, true, piece);
+              const vec8_t<T> res = merge_piece<T, DV, 0>(a.mg, tg, h, rr.gidx, orow, pc, true, piece);
               store8(reinterpret_cast<T*>(a.mg.out) + orow * DV + pc * 8, res);
             }
           }

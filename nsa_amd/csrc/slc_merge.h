@@ -101,6 +101,96 @@ __device__ __forceinline__ vec8_t<T> merge_piece(const MergeArgs& m, long tg, in
   return pack8<T>(out);
 }
 
+// Two pieces (pc_a, pc_b) of one row at once, TOPN > 0 only: the slot map, the maxima and the sums are
+// read once, and 2 * TOPN partial loads are in flight per lane before the first is used.  The epilogue
+// that calls this is bound by the latency of those loads, not by their bytes.
+template <typename T, int DV, int TOPN>
+__device__ __forceinline__ void merge_two(const MergeArgs& m, long tg, int h, int n, long row, int pc_a, int pc_b,
+                                          const vec8_t<T>& swa_a, const vec8_t<T>& swa_b, vec8_t<T>& res_a,
+                                          vec8_t<T>& res_b) {
+  static_assert(TOPN > 0 && TOPN % 4 == 0, "unrolled merge only");
+  const long base = (tg * m.hkv + h) * m.top_n;
+  const float c_attn = m.scale * kLog2e;
+  const T* pob = reinterpret_cast<const T*>(m.po);
+  int ps[TOPN];
+#pragma unroll
+  for (int i = 0; i < TOPN / 4; ++i) {
+    const int4 q4 = *reinterpret_cast<const int4*>(m.slotmap + base + 4 * i);
+    ps[4 * i] = q4.x; ps[4 * i + 1] = q4.y; ps[4 * i + 2] = q4.z; ps[4 * i + 3] = q4.w;
+  }
+  float mx[TOPN], l[TOPN];
+  vec8_t<T> oa[TOPN], ob[TOPN];
+#pragma unroll
+  for (int i = 0; i < TOPN; ++i) {
+    mx[i] = kNegInf; l[i] = 0.f; oa[i] = zero8<T>(); ob[i] = zero8<T>();
+    if (ps[i] >= 0) {
+      const long p = ps[i];
+      mx[i] = m.ml[(p * 2) * 16 + n];
+      l[i] = m.ml[(p * 2 + 1) * 16 + n];
+      oa[i] = load8(pob + (p * 16 + n) * DV + pc_a * 8);
+      ob[i] = load8(pob + (p * 16 + n) * DV + pc_b * 8);
+    }
+  }
+  float M = kNegInf, den = 0.f, acc_a[8], acc_b[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) { acc_a[e] = 0.f; acc_b[e] = 0.f; }
+#pragma unroll
+  for (int i = 0; i < TOPN; ++i) M = fmaxf(M, mx[i]);
+#pragma unroll
+  for (int i = 0; i < TOPN; ++i) {
+    if (ps[i] >= 0) {
+      const float w = fast_exp2((mx[i] - M) * c_attn) * l[i];
+      den += w;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        acc_a[e] = fmaf(w, (float)oa[i][e], acc_a[e]);
+        acc_b[e] = fmaf(w, (float)ob[i][e], acc_b[e]);
+      }
+    }
+  }
+  const float inv = den > 0.f ? 1.0f / den : 0.f;
+  if (m.o_slc_out != nullptr) {
+    float os[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) os[e] = acc_a[e] * inv;
+    store8(reinterpret_cast<T*>(m.o_slc_out) + row * DV + pc_a * 8, pack8<T>(os));
+#pragma unroll
+    for (int e = 0; e < 8; ++e) os[e] = acc_b[e] * inv;
+    store8(reinterpret_cast<T*>(m.o_slc_out) + row * DV + pc_b * 8, pack8<T>(os));
+  }
+  if (m.o_swa_out != nullptr) {
+    store8(reinterpret_cast<T*>(m.o_swa_out) + row * DV + pc_a * 8, swa_a);
+    store8(reinterpret_cast<T*>(m.o_swa_out) + row * DV + pc_b * 8, swa_b);
+  }
+  if (m.lse_slc_out != nullptr && pc_a == 0)
+    m.lse_slc_out[row] = den > 0.f ? fmaf(M, m.scale, __logf(den)) : __builtin_huge_valf();
+  const T* gs = reinterpret_cast<const T*>(m.g_slc);
+  const T* gw = reinterpret_cast<const T*>(m.g_swa);
+  const T* gcm = reinterpret_cast<const T*>(m.g_cmp);
+  const T* ocm = reinterpret_cast<const T*>(m.o_cmp);
+  const float w_slc = (gs ? gate_of((float)gs[row * m.gate_stride], m.gate_act) : 1.f) * inv;
+  const float w_swa = gw ? gate_of((float)gw[row * m.gate_stride], m.gate_act) : 1.f;
+  float out_a[8], out_b[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    out_a[e] = acc_a[e] * w_slc;
+    out_b[e] = acc_b[e] * w_slc;
+    out_a[e] += w_swa * (float)swa_a[e];
+    out_b[e] += w_swa * (float)swa_b[e];
+  }
+  if (ocm) {
+    const float w = gcm ? gate_of((float)gcm[row * m.gate_stride], m.gate_act) : 1.f;
+    const vec8_t<T> ca = load8(ocm + row * DV + pc_a * 8), cb = load8(ocm + row * DV + pc_b * 8);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      out_a[e] += w * (float)ca[e];
+      out_b[e] += w * (float)cb[e];
+    }
+  }
+  res_a = pack8<T>(out_a);
+  res_b = pack8<T>(out_b);
+}
+
 // Log-sum-exp (natural log) of the scaled scores over all usable picks of (token tg, kv head h,
 // head n of the group); +inf when the token has no usable pick.
 __device__ __forceinline__ float merge_lse(const MergeArgs& m, long tg, int h, int n) {
