@@ -230,9 +230,7 @@ bwd_kv_kernel(const BwdArgs a) {
   float ors[OPT], sr = 0.f, srs = 1.f;       // the gates of the staged rows (1 without a.rowscale)
 #pragma unroll
   for (int i = 0; i < OPT; ++i) ors[i] = 1.f;
-  auto gload = [&](int c) {
-    int posA, posB; bool vB;
-    chunk_tokens(c, posA, posB, vB);
+  auto gload = [&](int posA, int posB) {
 #pragma unroll
     for (int i = 0; i < QPT; ++i) {
       const int p = tid + i * NT;
@@ -281,19 +279,24 @@ bwd_kv_kernel(const BwdArgs a) {
   };
 
   const float c_attn = a.scale * kLog2e;
-  gload(0);
+  // The selected mode reads its token positions from the pair list.  Those of chunk c + 2 are requested at the
+  // end of iteration c and first used at the end of iteration c + 1, so neither the gathers of a chunk nor its
+  // masks wait for the list.  (Requested right after the gathers instead, the kernel is 10 % slower.)
+  int posA, posB, nxtA = 0, nxtB = 0, aftA = 0, aftB = 0;
+  bool vB, nxtV = false, aftV = false;
+  chunk_tokens(0, posA, posB, vB);
+  if (nchunks > 1) chunk_tokens(1, nxtA, nxtB, nxtV);
+  gload(posA, posB);
   lstore(0);
   __syncthreads();
   int buf = 0;
   for (int c = 0; c < nchunks; ++c) {
     const bool has_next = c + 1 < nchunks;
-    if (has_next) gload(c + 1);
+    if (has_next) gload(nxtA, nxtB);
 
     const T* qs = lds + buf * STAGE;
     const T* os = qs + 32 * QLD;
     const float* ss = stat + buf * 64;
-    int posA, posB; bool vB;
-    chunk_tokens(c, posA, posB, vB);
     // the 8 rows of this lane (chunk_row(g, 0..7)) are heads of one token
     const int tokpos = (g >> 1) ? posB : posA;
     bool vis = keyvalid && ((g >> 1) == 0 || vB);
@@ -302,7 +305,14 @@ bwd_kv_kernel(const BwdArgs a) {
     else if (a.causal) vis = vis && keypos * a.stride + a.block <= tokpos;
 
     float s[8], dp[8], p[8], ds[8];
-    tile_pair<T, DK, X32>(qs, QLD, n, g, kf, s);
+    if (MODE == kBwdSlc) {                    // K fragments from the block copy in LDS instead of 24 registers
+      vec8_t<T> kl[DK / 32];
+#pragma unroll
+      for (int kk = 0; kk < DK / 32; ++kk) kl[kk] = load8(kblk + (16 * wave + n) * QLD + 32 * kk + 8 * g);
+      tile_pair<T, DK, X32>(qs, QLD, n, g, kl, s);
+    } else {
+      tile_pair<T, DK, X32>(qs, QLD, n, g, kf, s);
+    }
     tile_pair<T, DV, X32>(os, OLD, n, g, vf, dp);
     const int rlo = chunk_row<X32>(g, 0), rhi = chunk_row<X32>(g, 4);
     const f32x4_t l0 = *reinterpret_cast<const f32x4_t*>(ss + rlo);
@@ -350,6 +360,9 @@ bwd_kv_kernel(const BwdArgs a) {
     if (has_next) lstore(buf ^ 1);
     __syncthreads();
     buf ^= 1;
+    if (c + 2 < nchunks) chunk_tokens(c + 2, aftA, aftB, aftV);
+    posA = nxtA; posB = nxtB; vB = nxtV;
+    nxtA = aftA; nxtB = aftB; nxtV = aftV;
   }
 
   if (keyvalid) {
