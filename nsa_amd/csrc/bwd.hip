@@ -279,13 +279,22 @@ bwd_kv_kernel(const BwdArgs a) {
   };
 
   const float c_attn = a.scale * kLog2e;
-  // The selected mode reads its token positions from the pair list.  Those of chunk c + 2 are requested at the
-  // end of iteration c and first used at the end of iteration c + 1, so neither the gathers of a chunk nor its
-  // masks wait for the list.  (Requested right after the gathers instead, the kernel is 10 % slower.)
-  int posA, posB, nxtA = 0, nxtB = 0, aftA = 0, aftB = 0;
-  bool vB, nxtV = false, aftV = false;
+  // Token positions are carried in registers: pos = chunk c, nxt = chunk c + 1.
+  int posA, posB, nxtA = 0, nxtB = 0;
+  bool vB, nxtV = false;
+  // selected mode: even lanes read the pair-list entry of a chunk's first token, odd lanes that of its second
+  // (the first again when the chunk has one), as one load whose value is only split into the two positions
+  // where they are used: a load from a wave-uniform address would be waited for where it is issued.
+  unsigned aftv = 0;
+  auto list_entry = [&](int c) { return a.ws.list[first + min(2 * c + (lane & 1), count - 1)]; };
+  auto list_split = [&](unsigned v, int c, int& pA, int& pB, bool& vb) {
+    pA = (int)(__builtin_amdgcn_readlane(v, 0) >> 6) - seq_start;
+    pB = (int)(__builtin_amdgcn_readlane(v, 1) >> 6) - seq_start;
+    vb = 2 * c + 1 < count;
+  };
   chunk_tokens(0, posA, posB, vB);
   if (nchunks > 1) chunk_tokens(1, nxtA, nxtB, nxtV);
+  if (MODE == kBwdSlc && nchunks > 2) aftv = list_entry(2);
   gload(posA, posB);
   lstore(0);
   __syncthreads();
@@ -339,6 +348,14 @@ bwd_kv_kernel(const BwdArgs a) {
 #pragma unroll
     for (int t = 0; t < DK / 16; ++t) dk_acc[t] = mma16(chunk_tr<X32>(qs + 16 * t, QLD, lane), dsb, dk_acc[t]);
 
+    // The next chunk goes to LDS before this chunk's dQ partials are stored: the counter that says "the gathers
+    // have arrived" also counts stores, in order, so after the stores it would wait for their write round trip.
+    if (has_next) lstore(buf ^ 1);
+    // aftv (chunk c + 2) was requested an iteration ago; it is split here, before the stores below, for the same
+    // reason
+    int splA = 0, splB = 0;
+    bool splV = false;
+    if (MODE == kBwdSlc) list_split(aftv, c + 2, splA, splB, splV);
     if (MODE == kBwdSlc) {
       // dQ^T[dk][row] = sum_key K[key][dk] dS[row][key]: this wavefront takes every NW-th 16-channel tile
       T* part = reinterpret_cast<T*>(a.ws.po);
@@ -357,12 +374,15 @@ bwd_kv_kernel(const BwdArgs a) {
       }
     }
 
-    if (has_next) lstore(buf ^ 1);
     __syncthreads();
     buf ^= 1;
-    if (c + 2 < nchunks) chunk_tokens(c + 2, aftA, aftB, aftV);
     posA = nxtA; posB = nxtB; vB = nxtV;
-    nxtA = aftA; nxtB = aftB; nxtV = aftV;
+    if (MODE == kBwdSlc) {
+      nxtA = splA; nxtB = splB; nxtV = splV;
+      if (c + 3 < nchunks) aftv = list_entry(c + 3);      // first touched an iteration from here
+    } else if (c + 2 < nchunks) {
+      chunk_tokens(c + 2, nxtA, nxtB, nxtV);
+    }
   }
 
   if (keyvalid) {
