@@ -300,8 +300,11 @@ bwd_kv_kernel(const BwdArgs a) {
   __syncthreads();
   int buf = 0;
   for (int c = 0; c < nchunks; ++c) {
+    // The last iteration stages its own chunk once more instead of branching around the loads and the LDS
+    // stores: with both unconditional the compiler knows that nothing is in flight at the top of the loop and
+    // puts no wait there (one that would also cover the dQ partial stores just issued).
     const bool has_next = c + 1 < nchunks;
-    if (has_next) gload(nxtA, nxtB);
+    gload(has_next ? nxtA : posA, has_next ? nxtB : posB);
 
     const T* qs = lds + buf * STAGE;
     const T* os = qs + 32 * QLD;
@@ -350,7 +353,7 @@ bwd_kv_kernel(const BwdArgs a) {
 
     // The next chunk goes to LDS before this chunk's dQ partials are stored: the counter that says "the gathers
     // have arrived" also counts stores, in order, so after the stores it would wait for their write round trip.
-    if (has_next) lstore(buf ^ 1);
+    lstore(buf ^ 1);
     // aftv (chunk c + 2) was requested an iteration ago; it is split here, before the stores below, for the same
     // reason
     int splA = 0, splB = 0;
