@@ -626,6 +626,10 @@ slc_dq_merge_kernel(const int* __restrict__ slotmap, const T* __restrict__ part,
       const int4 q4 = *reinterpret_cast<const int4*>(slotmap + base + 4 * i);
       ps[4 * i] = q4.x; ps[4 * i + 1] = q4.y; ps[4 * i + 2] = q4.z; ps[4 * i + 3] = q4.w;
     }
+    // all of the slot map before the first partial is requested (the conditional loads below would otherwise be
+    // split into batches by a wait for the later parts of the map)
+#pragma unroll
+    for (int i = 0; i < TOPN; ++i) asm volatile("" ::"v"(ps[i]));
     vec8_t<T> x[TOPN];
 #pragma unroll
     for (int i = 0; i < TOPN; ++i) {

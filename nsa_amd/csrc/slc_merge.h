@@ -30,6 +30,10 @@ __device__ __forceinline__ vec8_t<T> merge_piece(const MergeArgs& m, long tg, in
       const int4 q4 = *reinterpret_cast<const int4*>(m.slotmap + base + 4 * i);
       ps[4 * i] = q4.x; ps[4 * i + 1] = q4.y; ps[4 * i + 2] = q4.z; ps[4 * i + 3] = q4.w;
     }
+    // all of the slot map before the first partial is requested (the conditional loads below would otherwise be
+    // split into batches by a wait for the later parts of the map)
+#pragma unroll
+    for (int i = 0; i < TOPN; ++i) asm volatile("" ::"v"(ps[i]));
     float mx[TOPN], l[TOPN];
     vec8_t<T> o[TOPN];
 #pragma unroll
@@ -118,6 +122,11 @@ __device__ __forceinline__ void merge_two(const MergeArgs& m, long tg, int h, in
     const int4 q4 = *reinterpret_cast<const int4*>(m.slotmap + base + 4 * i);
     ps[4 * i] = q4.x; ps[4 * i + 1] = q4.y; ps[4 * i + 2] = q4.z; ps[4 * i + 3] = q4.w;
   }
+  // All of the slot map before the first partial is requested: the partial loads below are conditional, so the
+  // in-order memory counter could otherwise only be waited down to zero when a later part of the map is needed,
+  // which would split the loads into batches.
+#pragma unroll
+  for (int i = 0; i < TOPN; ++i) asm volatile("" ::"v"(ps[i]));
   float mx[TOPN], l[TOPN];
   vec8_t<T> oa[TOPN], ob[TOPN];
 #pragma unroll
