@@ -252,12 +252,27 @@ slc_block_kernel(const SlcArgs a, const SlcWs ws) {
   T* pob = reinterpret_cast<T*>(ws.po);
   const int gc = n < G ? n : G - 1;
   vec8_t<T> qn[NK];
-  uint32_t ent = ws.list[first];
+  // The segment's pair-list entries (at most one per lane) in one load; entry j is taken out with readlane.  A
+  // load from a wave-uniform address inside the loop would be waited for where it is issued, and on this
+  // hardware that wait (loads and stores share one in-order counter) also covers the stores of the pair before.
+  const uint32_t ents = ws.list[first + min(lane, count - 1)];
+  uint32_t ent = __builtin_amdgcn_readlane(ents, 0);
   {
     const T* qp = qb + ((long)(ent >> 6) * a.hq + h * G + gc) * DK + 8 * g;
 #pragma unroll
     for (int kk = 0; kk < NK; ++kk) qn[kk] = load8(qp + 32 * kk);
   }
+  // The K / V fragments are waited for here, once (an empty asm that takes each of them): left to the compiler,
+  // their waits sit inside the loop, where the fragments are first used, and, counting down to zero, would there
+  // also wait for the query just requested.
+#pragma unroll
+  for (int tile = 0; tile < 4; ++tile)
+#pragma unroll
+    for (int kk = 0; kk < NK; ++kk) asm volatile("" ::"v"(kf[tile][kk]));
+#pragma unroll
+  for (int c = 0; c < 2; ++c)
+#pragma unroll
+    for (int t = 0; t < NV; ++t) asm volatile("" ::"v"(vf[c][t]));
   for (int j = 0; j < count; ++j) {
     vec8_t<T> qf[NK];
 #pragma unroll
@@ -265,7 +280,7 @@ slc_block_kernel(const SlcArgs a, const SlcWs ws) {
     const int tg = (int)(ent >> 6);
     const int p = first + j;
     if (j + 1 < count) {                                  // next query in flight while this one is multiplied
-      ent = ws.list[p + 1];
+      ent = __builtin_amdgcn_readlane(ents, j + 1);
       const T* qp = qb + ((long)(ent >> 6) * a.hq + h * G + gc) * DK + 8 * g;
 #pragma unroll
       for (int kk = 0; kk < NK; ++kk) qn[kk] = load8(qp + 32 * kk);
@@ -322,10 +337,10 @@ slc_block_kernel(const SlcArgs a, const SlcWs ws) {
         store8(dst + r * DV + pc * 8, load8(&stage[wave][r * OLD + pc * 8]));
       }
     }
-    if (g == 0) {
-      ws.ml[((long)p * 2 + 0) * 16 + n] = mx;
-      ws.ml[((long)p * 2 + 1) * 16 + n] = sum;
-    }
+    // every lane group holds the same mx / sum; all four store them (same values to the same addresses) so that
+    // the stores are unconditional and the compiler can count them when it waits for the next query's loads
+    ws.ml[((long)p * 2 + 0) * 16 + n] = mx;
+    ws.ml[((long)p * 2 + 1) * 16 + n] = sum;
   }
 }
 
