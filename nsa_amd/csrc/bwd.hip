@@ -38,7 +38,9 @@ constexpr int kCmpSplit = 512;       // tokens of one compressed-branch work ite
                                      // with the XCD-aware order 256: 7.25, 384: 7.2-7.4, 512: 7.07, 768: 7.74, 1024: 7.40)
 constexpr int kXcds = 8;             // accelerator dies; workgroup w of a launch runs on die w % 8
 constexpr int kKvWaves = 4;          // key-stationary: wavefronts (x16 keys) per workgroup, two workgroups per CU
-constexpr int kQWaves = 16;          // query-stationary: tokens per workgroup (8: 3.7 ms, 16: 3.3 ms)
+constexpr int kQWaves = 12;          // query-stationary: tokens per workgroup = wavefronts, kQWaves / 4 per SIMD (8: 3.7 ms;
+                                     // 16: 3.3 ms at 128 registers with the staged chunk spilled; 12: 170 registers, nothing
+                                     // spilled, compressed / sliding calls 0.7 % / 3 % faster than 16)
 constexpr int kSegGroup = 4;         // selected branch: consecutive 64-pair segments of a block per workgroup
 
 struct BwdArgs {
@@ -419,9 +421,9 @@ bwd_kv_kernel(const BwdArgs a) {
 
 // ---- query-stationary: dQ of the compressed and sliding branches -----------------------------------
 
-// Four wavefronts per SIMD (128 registers, a few of them spilled at Dk = 192): faster than two or three.
+// kQWaves / 4 wavefronts per SIMD.
 template <typename T, int DK, int DV, int MODE, int NW>
-__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(4, 4)))
+__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW / 4, NW / 4)))
 bwd_q_kernel(const BwdArgs a) {
   constexpr int KLD = DK + kLdsPad<T, true>, VLD = DV + kLdsPad<T, true>, NT = NW * 64;
   constexpr int KP = 32 * DK / 8, VP = 32 * DV / 8;
