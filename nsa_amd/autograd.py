@@ -82,11 +82,21 @@ class SlcSwaFn(torch.autograd.Function):
         q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
         vt = ops.transpose(v, cu, batch)
         o_slc = lse_slc = o_swa = lse_swa = None
-        if idx is not None:
-            o_slc, lse_slc = ops.slc_combine(q, k, vt, idx, counts, None, None, None, None, None, cu, batch,
-                                             block_size, scale, block_major=True, want_lse=True)
-        if window > 0:
-            o_swa, lse_swa = ops.swa(q, k, vt, cu, batch, window, scale, want_lse=True)
+        ws = None
+        if idx is not None and window > 0:
+            ws = ops.slc_workspace(q, k.shape[1], v.shape[2], idx.shape[-1], block_size, batch)
+        if ws is not None:
+            # both branches: the fused schedule (partials per block, merged in the window kernel's epilogue),
+            # which leaves the two ungated outputs and their log-sum-exps; its gated sum is not used here
+            ops.slc_partials(q, k, vt, idx, counts, cu, batch, block_size, scale, ws)
+            _, o_slc, o_swa, lse_slc, lse_swa = ops.swa_merge(q, k, vt, ws, idx.shape[-1], None, None, None, None, cu,
+                                                               batch, block_size, window, scale, want_branches=True)
+        else:
+            if idx is not None:
+                o_slc, lse_slc = ops.slc_combine(q, k, vt, idx, counts, None, None, None, None, None, cu, batch,
+                                                 block_size, scale, block_major=True, want_lse=True)
+            if window > 0:
+                o_swa, lse_swa = ops.swa(q, k, vt, cu, batch, window, scale, want_lse=True)
         ctx.save_for_backward(q, k, v, o_slc, lse_slc, o_swa, lse_swa, idx, counts, cu)
         ctx.geom = (batch, block_size, window, scale)
         return o_slc, o_swa
