@@ -427,6 +427,12 @@ def test_module_long_context_more_than_512_bins():
     _module_case(torch.bfloat16, [40960], 16, 1, 64, 64, 16, 512, seed=9, scale_in=0.5, rows_per_seq=96)
 
 
+def test_module_long_context_131072():
+    """T=131072: 8191 compressed rows, 2048 pooled bins -> the generic selection kernel with its window sums in
+    LDS; sampled rows."""
+    _module_case(torch.bfloat16, [131072], 16, 1, 64, 64, 16, 512, seed=11, scale_in=0.5, rows_per_seq=48)
+
+
 def test_module_group_of_12_heads_ragged():
     """GQA group of 12 (padded to 16 rows per token) with ragged sequences, one shorter than a bin."""
     _module_case(torch.bfloat16, [1500, 70, 36, 900], 24, 2, 128, 128, 8, 256, seed=10, scale_in=0.5)
