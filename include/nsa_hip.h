@@ -85,7 +85,7 @@ int nsa_compress_bwd(const void* x, const void* w_lin, const void* d_out, void* 
  *   indices [total, hkv, top_n] int32 or int64 (idx64), descending score, -1 where fewer bins exist;
  *   NULL skips the selection;  pooled (optional, float) [total, hkv, pooled_stride] receives the
  *   pooled block scores (bins past a sequence's last one up to max_ns are zeroed).  Pass it even when
- *   the scores are not wanted: with it (and a GQA group of 9..16 heads, pooling 5/4/0, max_ns <= 1024,
+ *   the scores are not wanted: with it (and a GQA group of 9..16 heads, pooling 5/4/0, max_ns <= 4096,
  *   top_n <= 64) the selection runs as two lean kernels that use it as their hand-over buffer, without
  *   it as one slower kernel that keeps the bins in LDS;
  *   lse (float) [total, hq] receives the log-sum-exp of the raw scores q.ck over all compressed rows

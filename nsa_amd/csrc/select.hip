@@ -497,13 +497,15 @@ static int launch_select_stream(const CmpArgs& a, hipStream_t st) {
   hipLaunchKernelGGL(fn, dim3(tiles, a.hkv), dim3(NW * 64), smem, st, a);
   const int rows = (int)(((long)a.total * a.hkv + 3) / 4);
   if (a.max_ns <= 512) hipLaunchKernelGGL(topn_kernel<8>, dim3(rows), dim3(256), 0, st, a);
-  else hipLaunchKernelGGL(topn_kernel<16>, dim3(rows), dim3(256), 0, st, a);
+  else if (a.max_ns <= 1024) hipLaunchKernelGGL(topn_kernel<16>, dim3(rows), dim3(256), 0, st, a);
+  else if (a.max_ns <= 2048) hipLaunchKernelGGL(topn_kernel<32>, dim3(rows), dim3(256), 0, st, a);
+  else hipLaunchKernelGGL(topn_kernel<64>, dim3(rows), dim3(256), 0, st, a);
   return 0;
 }
 
 template <typename T, int DK>
 static int launch_select_t(const CmpArgs& a, hipStream_t st) {
-  if (a.pooled != nullptr && a.max_ns <= 1024 && a.top_n <= 64 && group_pow2(a.hq / a.hkv) == 16 && a.pool_k == 5 &&
+  if (a.pooled != nullptr && a.max_ns <= 4096 && a.top_n <= 64 && group_pow2(a.hq / a.hkv) == 16 && a.pool_k == 5 &&
       a.pool_s == 4 && a.pool_p == 0)
     return launch_select_stream<T, DK>(a, st);
   // four row groups per wavefront unless the per-token bins of such a tile outgrow the LDS

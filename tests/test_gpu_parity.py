@@ -427,10 +427,10 @@ def test_module_long_context_more_than_512_bins():
     _module_case(torch.bfloat16, [40960], 16, 1, 64, 64, 16, 512, seed=9, scale_in=0.5, rows_per_seq=96)
 
 
-def test_module_long_context_131072():
-    """T=131072: 8191 compressed rows, 2048 pooled bins -> the generic selection kernel with its window sums in
-    LDS; sampled rows."""
-    _module_case(torch.bfloat16, [131072], 16, 1, 64, 64, 16, 512, seed=11, scale_in=0.5, rows_per_seq=48)
+@pytest.mark.parametrize("T", [131072, 262144])
+def test_module_long_context_beyond_1024_bins(T):
+    """T=131072 / 262144: 2048 / 4096 pooled bins -> 32 / 64 top-n candidates per lane; sampled rows."""
+    _module_case(torch.bfloat16, [T], 16, 1, 64, 64, 16, 512, seed=11, scale_in=0.5, rows_per_seq=48)
 
 
 def test_module_group_of_12_heads_ragged():
