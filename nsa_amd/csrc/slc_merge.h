@@ -122,6 +122,20 @@ __device__ __forceinline__ void merge_two(const MergeArgs& m, long tg, int h, in
     const int4 q4 = *reinterpret_cast<const int4*>(m.slotmap + base + 4 * i);
     ps[4 * i] = q4.x; ps[4 * i + 1] = q4.y; ps[4 * i + 2] = q4.z; ps[4 * i + 3] = q4.w;
   }
+  // The compressed branch's rows and the three gate logits are requested here, after the slot map and before
+  // the wait for it: read where they are used (after the partials are summed) they would cost one more memory
+  // round trip per call.  The loads are unconditional so that the compiler can count them and wait for the slot
+  // map alone; an absent operand reads the slot map instead and the value is ignored.
+  const T* gs = reinterpret_cast<const T*>(m.g_slc);
+  const T* gw = reinterpret_cast<const T*>(m.g_swa);
+  const T* gcm = reinterpret_cast<const T*>(m.g_cmp);
+  const T* ocm = reinterpret_cast<const T*>(m.o_cmp);
+  const T* dummy = reinterpret_cast<const T*>(m.slotmap);
+  const vec8_t<T> ca = load8(ocm ? ocm + row * DV + pc_a * 8 : dummy);
+  const vec8_t<T> cb = load8(ocm ? ocm + row * DV + pc_b * 8 : dummy);
+  const T gs_raw = *(gs ? gs + row * m.gate_stride : dummy);
+  const T gw_raw = *(gw ? gw + row * m.gate_stride : dummy);
+  const T gc_raw = *(gcm ? gcm + row * m.gate_stride : dummy);
   // All of the slot map before the first partial is requested: the partial loads below are conditional, so the
   // in-order memory counter could otherwise only be waited down to zero when a later part of the map is needed,
   // which would split the loads into batches.
@@ -173,12 +187,8 @@ __device__ __forceinline__ void merge_two(const MergeArgs& m, long tg, int h, in
   }
   if (m.lse_slc_out != nullptr && pc_a == 0)
     m.lse_slc_out[row] = den > 0.f ? fmaf(M, m.scale, __logf(den)) : __builtin_huge_valf();
-  const T* gs = reinterpret_cast<const T*>(m.g_slc);
-  const T* gw = reinterpret_cast<const T*>(m.g_swa);
-  const T* gcm = reinterpret_cast<const T*>(m.g_cmp);
-  const T* ocm = reinterpret_cast<const T*>(m.o_cmp);
-  const float w_slc = (gs ? gate_of((float)gs[row * m.gate_stride], m.gate_act) : 1.f) * inv;
-  const float w_swa = gw ? gate_of((float)gw[row * m.gate_stride], m.gate_act) : 1.f;
+  const float w_slc = (gs ? gate_of((float)gs_raw, m.gate_act) : 1.f) * inv;
+  const float w_swa = gw ? gate_of((float)gw_raw, m.gate_act) : 1.f;
   float out_a[8], out_b[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
@@ -188,8 +198,7 @@ __device__ __forceinline__ void merge_two(const MergeArgs& m, long tg, int h, in
     out_b[e] += w_swa * (float)swa_b[e];
   }
   if (ocm) {
-    const float w = gcm ? gate_of((float)gcm[row * m.gate_stride], m.gate_act) : 1.f;
-    const vec8_t<T> ca = load8(ocm + row * DV + pc_a * 8), cb = load8(ocm + row * DV + pc_b * 8);
+    const float w = gcm ? gate_of((float)gc_raw, m.gate_act) : 1.f;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       out_a[e] += w * (float)ca[e];
