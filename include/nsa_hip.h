@@ -271,8 +271,12 @@ int nsa_slc_swa_bwd(const void* q, const void* k, const void* v, const void* o_s
  * ctx_lens int32[batch]: tokens in each cache including the current one; q [batch][hq][dk] is the
  * query of that token; gates [batch][hq][3] (selected, sliding, compressed) or NULL (all ones);
  * out [batch][hq][dv]; indices (optional) int32 [batch][hkv][top_n] receives the selected blocks.
- * nc_cap <= nsa_decode_max_compressed(). */
+ * nc_cap <= nsa_decode_max_compressed() (the kernel keeps a sequence's compressed scores in the registers of
+ * one workgroup; longer caches, up to nsa_decode_split_max_compressed() rows, go through
+ * nsa_decode_step_split) and a pooling geometry with at most nc_cap / 4 + 4 <= 640 bins per sequence
+ * (pool_stride >= 4); anything else returns NSA_ERR_UNSUPPORTED. */
 int nsa_decode_max_compressed(void);
+int nsa_decode_split_max_compressed(void);
 int nsa_decode_step(const void* q, const void* k_cache, const void* v_cache_t, const void* ck_cache,
                     const void* cv_cache_t, const int32_t* ctx_lens, const void* gates, void* out, int32_t* indices,
                     int batch, int hq, int hkv, int dk, int dv, int ctx_cap, int nc_cap, int block, int stride,
@@ -300,7 +304,9 @@ int nsa_decode_append_paged(const void* k_new, const void* v_new, void* k_pool, 
 /* The same step for small batches: the work of every (sequence, kv head) pair is spread over `splits`
  * workgroups (three launches: compressed slices, selection + window / selected chunks, merge), because one
  * workgroup per pair leaves most of the chip idle below ~128 pairs.  block_table NULL = contiguous caches
- * (ctx_cap used), else the paged pool (max_pages used).  Pooling 5 / 4 / 0 only.  The workspace holds
+ * (ctx_cap used), else the paged pool (max_pages used).  Pooling 5 / 4 / 0 only.  The compressed rows are cut
+ * into max(splits, ceil(nc_cap / 384)) <= 32 slices, so caches of up to nsa_decode_split_max_compressed() rows
+ * (contexts of ~196k tokens at stride 16) are served whatever the batch.  The workspace holds
  * partial results only; calls that share it must not overlap.  No counterpart in the reference. */
 int64_t nsa_decode_split_workspace_bytes(int batch, int hkv, int dv, int nc_cap, int splits);
 int nsa_decode_step_split(const void* q, const void* k_cache, const void* v_cache_t, const int32_t* block_table,

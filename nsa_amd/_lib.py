@@ -45,6 +45,7 @@ SIGNATURES = {
     "nsa_slc_swa_bwd_workspace_bytes": (_L, [_I] * 9),
     "nsa_slc_swa_bwd": (_I, [_P] * 16 + [_I] * 9 + [_F, _I, _I, _P, _P, _P, _P, _P, _L, _P]),
     "nsa_decode_max_compressed": (_I, []),
+    "nsa_decode_split_max_compressed": (_I, []),
     "nsa_decode_step": (_I, [_P] * 9 + [_I] * 15 + [_F, _I, _I, _P]),
     "nsa_qkv_rope": (_I, [_P] * 8 + [_I, _L] + [_I] * 14 + [_P]),
     "nsa_decode_append": (_I, [_P] * 7 + [_I] * 9 + [_P]),

@@ -431,6 +431,7 @@ int nsa_decode_append_paged(const void* k_new, const void* v_new, void* k_pool, 
 }
 
 int nsa_decode_max_compressed(void) { return nsa::decode_max_nc(); }
+int nsa_decode_split_max_compressed(void) { return nsa::decode_split_max_nc(); }
 
 static int decode_common(const char* what, const void* q, const void* k_cache, const void* v_cache_t,
                          const int32_t* block_table, int max_pages, const void* ck_cache, const void* cv_cache_t,
@@ -447,8 +448,11 @@ static int decode_common(const char* what, const void* q, const void* k_cache, c
   if (int rc = check_heads(what, hq, hkv, dk, dv)) return rc;
   if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "%s: scale must be positive", what);
   if (ctx_cap % 64 != 0 || nc_cap % 64 != 0) return fail(NSA_ERR_INVALID, "%s: cache capacities must be multiples of 64", what);
-  if (nc_cap > nsa::decode_max_nc())
-    return fail(NSA_ERR_UNSUPPORTED, "%s: at most %d compressed rows per sequence are built", what, nsa::decode_max_nc());
+  if (splits == 0 && nc_cap > nsa::decode_max_nc())
+    return fail(NSA_ERR_UNSUPPORTED, "%s: the one-workgroup step keeps at most %d compressed rows per sequence; "
+                "longer caches go through nsa_decode_step_split", what, nsa::decode_max_nc());
+  if (splits > 0 && nc_cap > nsa::decode_split_max_nc())
+    return fail(NSA_ERR_UNSUPPORTED, "%s: at most %d compressed rows per sequence are built", what, nsa::decode_split_max_nc());
   if (sel_block <= 0 || sel_block % 32 != 0) return fail(NSA_ERR_UNSUPPORTED, "%s: selection block must be a multiple of 32", what);
   if (pool_kernel <= 0 || pool_stride <= 0 || pool_pad < 0 || pool_pad >= pool_kernel || top_n <= 0)
     return fail(NSA_ERR_INVALID, "%s: bad pooling / top-n parameters", what);
@@ -468,6 +472,16 @@ static int decode_common(const char* what, const void* q, const void* k_cache, c
     const int rc = nsa::launch_decode_split(a, splits, workspace, stream);
     if (rc == -2) return fail(NSA_ERR_UNSUPPORTED, "%s: head dims or split count not built", what);
     return finish(rc, what);
+  }
+  {
+    // the one-workgroup kernel holds the pooled bins of a sequence in nc_cap / 4 + 4 floats of LDS and ten
+    // per lane in its top-n: pooling strides below 4 (selection blocks narrower than 4 compression strides)
+    // make more bins than that
+    const int span = nc_cap + 2 * pool_pad - pool_kernel;
+    const int ns_cap = span < 0 ? 0 : (span + pool_stride - 1) / pool_stride + 1;
+    if (ns_cap > nc_cap / 4 + 4 || ns_cap > 640)
+      return fail(NSA_ERR_UNSUPPORTED, "%s: up to %d pooled bins per sequence (pooling stride >= 4) are built, this "
+                  "geometry can make %d", what, nc_cap / 4 + 4 < 640 ? nc_cap / 4 + 4 : 640, ns_cap);
   }
   const int rc = nsa::launch_decode(a, stream);
   if (rc == -2) return fail(NSA_ERR_UNSUPPORTED, "%s: head dims not built (dk,dv in (64,64),(128,128),(192,128); fp32: no 192)", what);

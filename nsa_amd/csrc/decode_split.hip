@@ -224,7 +224,7 @@ decode_split_cmp_kernel(const DecodeArgs a, const SplitLayout L, float* __restri
 }
 
 // ---- B: selection, then window and selected chunks ---------------------------------------------------
-template <typename T, int DK, int DV, bool PAGED>
+template <typename T, int DK, int DV, bool PAGED, int PER>
 __global__ void __launch_bounds__(kSplitWaves * 64)
 decode_split_attend_kernel(const DecodeArgs a, const SplitLayout L, float* __restrict__ ws) {
   constexpr int NW = kSplitWaves, PLD = 17;
@@ -324,7 +324,7 @@ decode_split_attend_kernel(const DecodeArgs a, const SplitLayout L, float* __res
   if (my_win >= 0) issue_kv(f, w_first + 32 * my_win);
 
   // global log-sum-exp of the raw scores per head, and each slice's factor exp(M_s - lse).  One thread per
-  // (slice, statistic, head) fetches its value (sa <= 16: at most 512 of them) so that the 16 threads that
+  // (slice, statistic, head) fetches its value (sa <= 32: at most 1024 of them) so that the 16 threads that
   // combine them read LDS, not a chain of dependent global loads.
   float* st_l = part;                                          // [sa][32], free until the first put()
   for (int i = tid; i < L.sa * 32; i += NW * 64) st_l[i] = w_stat[i];
@@ -377,10 +377,9 @@ decode_split_attend_kernel(const DecodeArgs a, const SplitLayout L, float* __res
   }
   __syncthreads();
   if (wave == 0) {
-    constexpr int PER = (32 * kDecWaves * kDecMaxChunks / 4 + 63) / 64 + 1;
     __shared__ float cand_v[128];
     __shared__ int cand_i[128];
-    float v[PER];
+    float v[PER];                                              // the launcher picks PER with 64 * PER >= Ns
 #pragma unroll
     for (int k = 0; k < PER; ++k) {
       const int bb = lane + 64 * k;
@@ -429,12 +428,12 @@ decode_split_attend_kernel(const DecodeArgs a, const SplitLayout L, float* __res
 // grid (pair, DV / 16): thread = (head r, channel d).  The weights of all partial states go through LDS first
 // (one thread per state and head), and the weighted sums are unrolled over the most states there can be, so
 // that every load of a thread is in flight at once: the launch is pure latency otherwise.
-constexpr int kSplitMaxStates = 16;
+constexpr int kSplitMaxSplits = 16;      // workgroups per pair in kernel B (and the least number of slices in A)
+constexpr int kSplitMaxSlices = 32;      // slices of kernel A: up to 32 * 384 = 12288 compressed rows
 
-template <typename T, int DV>
+template <typename T, int DV, int MAXS>
 __global__ void __launch_bounds__(256)
 decode_split_merge_kernel(const DecodeArgs a, const SplitLayout L, const float* __restrict__ ws) {
-  constexpr int MAXS = kSplitMaxStates;
   __shared__ float sm[3][MAXS][16], sl[3][MAXS][16];           // branch 0 selected, 1 window, 2 compressed
   const int tid = threadIdx.x, r = tid & 15, dg = tid >> 4;
   const int bh = blockIdx.x, d = blockIdx.y * 16 + dg;
@@ -498,7 +497,9 @@ int set_smem(const void* fn, size_t bytes);
 template <typename T, int DK, int DV>
 static int launch_decode_split_t(const DecodeArgs& a, int splits, float* ws, hipStream_t st) {
   const SplitLayout L = split_layout(a, splits);
-  if (L.sa > 16 || L.sb > 16) return -2;
+  if (L.sa > kSplitMaxSlices || L.sb > kSplitMaxSplits) return -2;
+  const int ns_cap = (a.nc_cap + 3) / 4 + 1;                  // bound of the pooled bins (windows of 5 every 4)
+  const bool big = ns_cap > 64 * 10;                          // more bins than ten per lane: the wide top-n
   const int pairs = a.batch * a.hkv;
   const size_t base = ((size_t)kSplitWaves * DV * 17 + kSplitWaves * 32) * sizeof(float);
   const size_t smem_a = base + ((size_t)kSplitWaves * 16 + (size_t)L.nb * 16) * sizeof(float);
@@ -508,18 +509,29 @@ static int launch_decode_split_t(const DecodeArgs& a, int splits, float* ws, hip
     if (int rc = set_smem(reinterpret_cast<const void*>(fn), smem_a)) return rc;
     hipLaunchKernelGGL(fn, dim3(pairs, L.sa), dim3(kSplitWaves * 64), smem_a, st, a, L, ws);
   }
-  if (a.block_table != nullptr) {
-    auto fn = decode_split_attend_kernel<T, DK, DV, true>;
+  auto launch_b = [&](auto fn) -> int {
     if (int rc = set_smem(reinterpret_cast<const void*>(fn), smem_b)) return rc;
     hipLaunchKernelGGL(fn, dim3(pairs, L.sb), dim3(kSplitWaves * 64), smem_b, st, a, L, ws);
-  } else {
-    auto fn = decode_split_attend_kernel<T, DK, DV, false>;
-    if (int rc = set_smem(reinterpret_cast<const void*>(fn), smem_b)) return rc;
-    hipLaunchKernelGGL(fn, dim3(pairs, L.sb), dim3(kSplitWaves * 64), smem_b, st, a, L, ws);
-  }
-  hipLaunchKernelGGL((decode_split_merge_kernel<T, DV>), dim3(pairs, DV / 16), dim3(256), 0, st, a, L, ws);
+    return 0;
+  };
+  constexpr int PER_BIG = (kSplitMaxSlices * kSplitMaxSlice / 4 + 1 + 63) / 64;   // 3073 bins at most
+  static_assert(64 * 10 >= 32 * kDecWaves * kDecMaxChunks / 4 + 1, "ten bins per lane cover the short caches");
+  int rc;
+  if (a.block_table != nullptr)
+    rc = big ? launch_b(decode_split_attend_kernel<T, DK, DV, true, PER_BIG>)
+             : launch_b(decode_split_attend_kernel<T, DK, DV, true, 10>);
+  else
+    rc = big ? launch_b(decode_split_attend_kernel<T, DK, DV, false, PER_BIG>)
+             : launch_b(decode_split_attend_kernel<T, DK, DV, false, 10>);
+  if (rc) return rc;
+  if (L.sa > 16)
+    hipLaunchKernelGGL((decode_split_merge_kernel<T, DV, kSplitMaxSlices>), dim3(pairs, DV / 16), dim3(256), 0, st, a, L, ws);
+  else
+    hipLaunchKernelGGL((decode_split_merge_kernel<T, DV, 16>), dim3(pairs, DV / 16), dim3(256), 0, st, a, L, ws);
   return 0;
 }
+
+int decode_split_max_nc() { return kSplitMaxSlices * kSplitMaxSlice; }
 
 int launch_decode_split(const DecodeArgs& a, int splits, void* workspace, hipStream_t st) {
   float* ws = reinterpret_cast<float*>(workspace);

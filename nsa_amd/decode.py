@@ -34,12 +34,16 @@ class NSADecodeCache:
         self.ck = torch.zeros(batch, self.nc_cap, hkv, dk, **z)
         self.cvt = torch.zeros(batch, hkv, dv, self.nc_cap, **z)
         self.ctx_lens = torch.zeros(batch, dtype=torch.int32, device=device)
+        self._max_len = 0        # longest sequence, tracked on the host so that append() never waits for the GPU
 
     @torch.no_grad()
     def fill(self, k: torch.Tensor, v: torch.Tensor):
         """Loads a prefilled context: k [B,T,Hkv,Dk], v [B,T,Hkv,Dv] (same T for every sequence)."""
         from . import ops
         B, T = k.shape[:2]
+        if T > self.ctx_cap:
+            raise RuntimeError(f"{T} tokens do not fit the cache capacity of {self.ctx_cap}")
+        self._max_len = T
         self.k[:, :T] = k
         self.vt[:, :, :, :T] = v.permute(0, 2, 3, 1)
         nc = (T - self.block) // self.stride + 1 if T >= self.block else 0
@@ -54,7 +58,12 @@ class NSADecodeCache:
 
     @torch.no_grad()
     def append(self, k_new: torch.Tensor, v_new: torch.Tensor):
-        """k_new [B,Hkv,Dk], v_new [B,Hkv,Dv]: the next token of every sequence."""
+        """k_new [B,Hkv,Dk], v_new [B,Hkv,Dv]: the next token of every sequence.  Raises once the longest
+        sequence (as filled and appended through this object) has reached the capacity: the kernel would
+        drop the token and later steps would attend a stale last row."""
+        if self._max_len >= self.ctx_cap:
+            raise RuntimeError(f"a sequence would exceed the cache capacity of {self.ctx_cap} tokens")
+        self._max_len += 1
         pos = self.ctx_lens.clone()
         k_new, v_new = k_new.contiguous(), v_new.contiguous()      # keep the copies alive across the launch
         rc = _lib.load().nsa_decode_append(_ptr(k_new), _ptr(v_new), _ptr(self.k),
@@ -222,7 +231,9 @@ def nsa_decode_step(q: torch.Tensor, cache, gates: Optional[torch.Tensor] = None
     splits: how many workgroups share one (sequence, kv head) pair.  0 = one (the kernel the batch-64
     benchmark runs); None = chosen from the batch: up to 64 pairs a single workgroup per pair leaves
     most of the chip idle and its ~60 us critical path sets the step time, so the work is split 8 ways
-    (three launches, partial results in a workspace kept on the cache object)."""
+    (three launches, partial results in a workspace kept on the cache object).  Caches with more
+    compressed rows than one workgroup keeps in registers (contexts beyond ~36k tokens) always take the
+    split schedule, whose first launch cuts the compressed rows into slices of at most 384."""
     if not q.is_cuda:
         raise RuntimeError("NSA kernels run on the GPU only")
     B, hq, dk = q.shape
@@ -239,13 +250,20 @@ def nsa_decode_step(q: torch.Tensor, cache, gates: Optional[torch.Tensor] = None
     pool_p = cache.block // cache.stride - 2
     act = _lib.GATE_SIGMOID if gate_activation == "sigmoid" else _lib.GATE_IDENTITY
     paged = isinstance(cache, NSAPagedDecodeCache)
+    lib = _lib.load()
+    long_cache = cache.nc_cap > lib.nsa_decode_max_compressed()
     if splits is None:
         pairs = B * cache.hkv
         # measured at 32k context: 8 splits halve the step up to 32 pairs and still win at 64 (46 vs 64 us);
         # at 128 pairs one workgroup per pair is as fast and needs no workspace
         splits = 8 if pairs <= 64 and (pool_k, pool_s, pool_p) == (5, 4, 0) and selected_block_count <= 64 else 0
+        if long_cache and splits == 0:
+            splits = 1 if pairs > 64 else 8       # the compressed rows are sliced whatever `splits` says
+    elif splits == 0 and long_cache:
+        raise NotImplementedError(
+            "the one-workgroup decode step keeps at most %d compressed rows per sequence; this cache holds up "
+            "to %d (pass splits=None or a positive split count)" % (lib.nsa_decode_max_compressed(), cache.nc_cap))
     if splits:
-        lib = _lib.load()
         need = lib.nsa_decode_split_workspace_bytes(B, cache.hkv, cache.dv, cache.nc_cap, splits)
         ws = getattr(cache, "_split_ws", None)
         if ws is None or ws.numel() < need:
@@ -322,6 +340,8 @@ class NSADecodeGraph:
             self.cache.reserve_next()
         elif int(self.cache.ctx_cap) <= self._host_len():
             raise RuntimeError(f"a sequence would exceed the cache capacity of {self.cache.ctx_cap} tokens")
+        elif self.graph is not None:
+            self.cache._max_len += 1     # a replay appends without passing through cache.append()
         for buf, src in ((self.q, q), (self.k_new, k_new), (self.v_new, v_new), (self.gates, gates)):
             if buf is not None and src is not None and src is not buf:
                 buf.copy_(src)       # producers that write into the buffers themselves pass None (or the buffer)

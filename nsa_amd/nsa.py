@@ -45,7 +45,9 @@ class NSAAttention(nn.Module):
     ):
         super().__init__()
         if attention_dropout not in (0, 0.0, None):
-            raise NotImplementedError("attention dropout is not part of the forward kernels")
+            # the reference stores the value and never applies it (nsa/nsa.py:45, no use in forward)
+            import warnings
+            warnings.warn("NSAAttention: attention_dropout is stored but not applied, as in the reference")
         if compressor_mode not in ("conv", "mean") or gate_activation not in (None, "sigmoid"):
             raise ValueError("compressor_mode in {'conv','mean'}, gate_activation in {None,'sigmoid'}")
         self.causal = causal
@@ -82,7 +84,10 @@ class NSAAttention(nn.Module):
         """q [total,Hq,Dk], k [total,Hkv,Dk], v [total,Hkv,Dv], cu_seqlens int32 [B+1] -> [total,Hq,Dv].
 
         max_seqlen: longest sequence (int); 0/None means "all sequences have total/B tokens" as in
-        the reference.  gates [total,Hq,3] (selected, sliding, compressed) overrides the gating
+        the reference, which is checked against cu_seqlens (one small device read) and falls back to
+        the ragged path when the lengths differ.  softmax_scale follows the reference: None is
+        1/sqrt(Dk), anything else is used as a number (so True, which the reference's module test passes
+        positionally, means 1.0).  gates [total,Hq,3] (selected, sliding, compressed) overrides the gating
         Linear (pre-activation values).  stage_times: a list that receives (name, start_event,
         end_event) per kernel stage; return_indices also returns the int32 block ids [total,Hkv,S]."""
         causal = self.causal if causal is None else causal
@@ -91,9 +96,14 @@ class NSAAttention(nn.Module):
         total, hq, dk = q.shape
         hkv, dv = v.shape[1], v.shape[2]
         scale = self.softmax_scale
-        if scale is None or scale is True:
-            scale = 1.0 / math.sqrt(dk)
+        scale = 1.0 / math.sqrt(dk) if scale is None else float(scale)   # nsa/triton_attention.py:433-434
         uniform = not max_seqlen
+        if uniform and batch > 1:
+            # "uniform" is a promise about cu_seqlens; the kernels read the real offsets, so a ragged batch
+            # taken for a uniform one would size the compressed rows wrongly
+            lens = (cu[1:] - cu[:-1]).tolist()
+            if min(lens) != max(lens) or lens[0] * batch != total:
+                uniform, max_seqlen = False, max(lens)
         seq_len = total // batch if uniform else int(max_seqlen)
         params = [] if gates is not None else [self.gating.weight, self.gating.bias]
         if self.compressor.mode != "mean":

@@ -424,10 +424,12 @@ def nsa_forward_varlen(q, k, v, gates, cu_seqlens: Sequence[int], p: NSAParams, 
 
 
 def nsa_decode_step(q_last, k_cache, v_cache, gates_last, p: NSAParams, math_dtype=torch.float32,
-                    return_parts=False):
+                    return_parts=False, force_idx=None):
     """One new token per sequence.  q_last [Hq,Dk] is the query at position ctx-1, k_cache
     [ctx,Hkv,Dk] / v_cache [ctx,Hkv,Dv] already hold that token.  Defined as the last row of the
     prefill forward on the same cache (mean-pool compressor), computed here without the other rows.
+    force_idx [Hkv,S]: blocks to attend in the selected branch instead of the oracle's own picks
+    (which are still returned in parts["idx"]), so that outputs stay comparable when a tie flips a pick.
     """
     ctx = k_cache.shape[0]
     t = ctx - 1
@@ -445,6 +447,7 @@ def nsa_decode_step(q_last, k_cache, v_cache, gates_last, p: NSAParams, math_dty
         parts["pooled"] = pooled[0]
     else:
         idx = torch.full((Hkv, p.top_n), -1, dtype=torch.int64)
+    use_idx = idx if force_idx is None else force_idx
     n_vis = min(max((t - p.block) // p.stride + 1, 0), Nc) if t >= p.block else 0
     if n_vis > 0:
         s = torch.einsum("hgd,chd->hgc", q_last.to(math_dtype).reshape(Hkv, -1, Dk),
@@ -460,7 +463,7 @@ def nsa_decode_step(q_last, k_cache, v_cache, gates_last, p: NSAParams, math_dty
     o_swa = torch.zeros(Hkv, G, Dv, dtype=math_dtype)
     for h in range(Hkv):
         toks = []
-        for b in sorted(set(int(x) for x in idx[h] if x >= 0 and int(x) * p.sel_block <= t)):
+        for b in sorted(set(int(x) for x in use_idx[h] if x >= 0 and int(x) * p.sel_block <= t)):
             toks.extend(range(b * p.sel_block, min(b * p.sel_block + p.sel_block - 1, t) + 1))
         if toks:
             tk = torch.tensor(toks)

@@ -422,3 +422,59 @@ def test_layer_oracle_without_rope_is_the_reference_module_on_projected_inputs()
     q, k, v = (F.linear(x, w).view(T, -1, d) for w in (wq, wk, wv))
     o = O.nsa_forward_varlen(q, k, v, F.linear(q, gw, gb), [0, 60, T], p)
     assert torch.allclose(out, F.linear(o.reshape(T, -1), wo), atol=1e-5)
+
+
+def test_reference_signature_adapters_match_library_pipeline():
+    """oracle/torch_attention.py (the reference's attention_ref / get_indices / construct_local_mask
+    signatures, nsa/torch_attention.py:12,51,66) against library routines on the reference's batched
+    layout: masked SDPA for the output, softmax -> group sum -> avg_pool1d(ceil_mode) -> topk for
+    the indices, and the decode force_idx switch of the step oracle."""
+    from oracle import torch_attention as TA
+    B, T, Hq, Hkv, D, l, d, S = 2, 200, 8, 2, 32, 32, 16, 3
+    G = Hq // Hkv
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(B, T, Hq, D, generator=g, dtype=torch.float64)
+    Nc = O.compressed_len_conv(T, l, d)
+    ck = torch.randn(B, Nc, Hkv, D, generator=g, dtype=torch.float64)
+    cv = torch.randn(B, Nc, Hkv, D, generator=g, dtype=torch.float64)
+    ckr, cvr = ck.repeat_interleave(G, 2), cv.repeat_interleave(G, 2)          # the "(h g)" repeat of the module
+    out, idx = TA.attention_ref(q.float(), ckr.float(), cvr.float(), d, l, causal=True, pool_num_kv_head=Hkv,
+                                pool_kernel_size=5, pool_stride=4, pool_padding=0, select_block_count=S)
+    assert out.shape == (B, T, Hq, D) and idx.shape == (B, T, Hkv, S) and idx.dtype == torch.int64
+    hidden = TA.construct_local_mask(T, Nc, d, l)
+    assert hidden.shape == (T, Nc) and bool(hidden[l - 1].all()) and not bool(hidden[l, 0]) and bool(hidden[l, 1])
+    ref = F.scaled_dot_product_attention(q.transpose(1, 2), ckr.transpose(1, 2), cvr.transpose(1, 2),
+                                         attn_mask=~hidden[None, None]).transpose(1, 2)
+    ref = torch.where(hidden.all(-1)[None, :, None, None], torch.zeros_like(ref), ref)   # rows that see nothing
+    assert float((out.double() - ref).abs().max()) < 1e-5
+    p = torch.softmax(torch.einsum("bthd,bchd->bhtc", q, ckr), -1)
+    pooled = F.avg_pool1d(p.reshape(B, Hkv, G, T, Nc).sum(2).reshape(B * Hkv, T, Nc), 5, 4, 0, True)
+    lib_idx = torch.topk(pooled.reshape(B, Hkv, T, -1), S, dim=3).indices.transpose(1, 2)
+    assert torch.equal(idx.sort(-1).values, lib_idx.sort(-1).values)
+    assert torch.equal(TA.get_indices(p.float(), Hkv, 5, 4, 0, S).sort(-1).values, lib_idx.sort(-1).values)
+    # non-causal: every compressed row visible
+    out_nc, _ = TA.attention_ref(q.float(), ckr.float(), cvr.float(), d, l, causal=False)
+    ref_nc = F.scaled_dot_product_attention(q.transpose(1, 2), ckr.transpose(1, 2), cvr.transpose(1, 2)).transpose(1, 2)
+    assert float((out_nc.double() - ref_nc).abs().max()) < 1e-5
+    with pytest.raises(NotImplementedError):
+        TA.attention_ref(q, ckr, cvr, d, l, dropout_p=0.1)
+
+
+def test_decode_oracle_forced_picks():
+    """force_idx replaces the blocks of the selected branch only; the oracle's own picks still come back."""
+    ctx, Hq, Hkv, D = 700, 8, 2, 32
+    g = torch.Generator().manual_seed(6)
+    q = torch.randn(Hq, D, generator=g)
+    k = torch.randn(ctx, Hkv, D, generator=g)
+    v = torch.randn(ctx, Hkv, D, generator=g)
+    gates = torch.rand(Hq, 3, generator=g)
+    p = O.NSAParams(32, 16, 64, 3, 64)
+    a, pa = O.nsa_decode_step(q, k, v, gates, p, return_parts=True)
+    b, pb = O.nsa_decode_step(q, k, v, gates, p, return_parts=True, force_idx=pa["idx"])
+    assert torch.equal(a, b) and torch.equal(pa["idx"], pb["idx"])
+    other = torch.tensor([[0, 1, 2], [3, 4, 5]])
+    c, pc = O.nsa_decode_step(q, k, v, gates, p, return_parts=True, force_idx=other)
+    assert torch.equal(pc["idx"], pa["idx"]) and torch.equal(pc["o_cmp"], pa["o_cmp"]) and torch.equal(pc["o_swa"], pa["o_swa"])
+    blocks = torch.cat([torch.arange(0, 192), ])
+    s0 = (q.view(Hkv, -1, D)[0] @ k[blocks, 0].T) / math.sqrt(D)
+    assert torch.allclose(pc["o_slc"].view(Hkv, -1, D)[0], torch.softmax(s0, -1) @ v[blocks, 0], atol=1e-5)
