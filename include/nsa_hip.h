@@ -316,6 +316,24 @@ int nsa_decode_step_split(const void* q, const void* k_cache, const void* v_cach
                           int pool_stride, int pool_pad, int top_n, int window, float scale, int gate_act, int dtype,
                           int splits, void* workspace, int64_t workspace_bytes, nsa_stream_t stream);
 
+/* nsa_decode_step_split for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc): the same three launches and the same results, bit for bit,
+ * with the partial results in a fixed device array that is part of the library (nsa_decode_split_static_bytes()
+ * = 16 MiB, held on every GPU the library runs on until the process ends) instead of a caller workspace.  The
+ * call allocates and frees nothing; the first call on a device looks the array's address up.  Arguments as
+ * nsa_decode_step_split without workspace / workspace_bytes.  Returns NSA_ERR_RESOURCE when
+ * nsa_decode_split_workspace_bytes(batch, hkv, dv, nc_cap, splits) exceeds the array (about 70 (sequence, kv head)
+ * pairs at 32k context, D 128, 8 splits).  All calls on one GPU share the array and it keeps the last call's
+ * contents: calls that overlap in time on one GPU race, also across streams.  No counterpart in the reference,
+ * which has no decode path and leaves every allocation to PyTorch. */
+int64_t nsa_decode_split_static_bytes(void);
+int nsa_decode_step_split_static(const void* q, const void* k_cache, const void* v_cache_t, const int32_t* block_table,
+                                 int max_pages, const void* ck_cache, const void* cv_cache_t, const int32_t* ctx_lens,
+                                 const void* gates, void* out, int32_t* indices, int batch, int hq, int hkv, int dk,
+                                 int dv, int ctx_cap, int nc_cap, int block, int stride, int sel_block, int pool_kernel,
+                                 int pool_stride, int pool_pad, int top_n, int window, float scale, int gate_act,
+                                 int dtype, int splits, nsa_stream_t stream);
+
 /* Appends one token per sequence: k_new [batch][hkv][dk] -> row pos[b] of k_cache, v_new
  * [batch][hkv][dv] -> column pos[b] of v_cache_t, and, when pos[b]+1 completes a compression block,
  * the mean of the last `block` tokens as the next row / column of the compressed caches. */

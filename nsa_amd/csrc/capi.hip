@@ -439,7 +439,7 @@ static int decode_common(const char* what, const void* q, const void* k_cache, c
                          int hkv, int dk, int dv, int ctx_cap, int nc_cap, int block, int stride, int sel_block,
                          int pool_kernel, int pool_stride, int pool_pad, int top_n, int window, float scale,
                          int gate_act, int dtype, nsa_stream_t stream, int splits = 0, void* workspace = nullptr,
-                         int64_t workspace_bytes = 0) {
+                         int64_t workspace_bytes = 0, bool static_scratch = false) {
   if (!q || !k_cache || !v_cache_t || !ck_cache || !cv_cache_t || !ctx_lens || !out)
     return fail(NSA_ERR_INVALID, "%s: null pointer", what);
   if (batch <= 0 || ctx_cap <= 0 || nc_cap <= 0 || block <= 0 || stride <= 0 || window < 0)
@@ -467,6 +467,16 @@ static int decode_common(const char* what, const void* q, const void* k_cache, c
     if (pool_kernel != 5 || pool_stride != 4 || pool_pad != 0)
       return fail(NSA_ERR_UNSUPPORTED, "%s: the split step is built for pooling windows of 5 every 4 without padding", what);
     if (top_n > 64) return fail(NSA_ERR_UNSUPPORTED, "%s: at most 64 selected blocks", what);
+    if (static_scratch) {
+      const int rc = nsa::launch_decode_split_static(a, splits, stream);
+      if (rc == -1)
+        return fail(NSA_ERR_RESOURCE, "%s: the partial results of this call need %lld bytes, the library's fixed array "
+                    "holds %lld (fewer sequences, kv heads or splits per call)", what,
+                    (long long)nsa::decode_split_workspace_bytes(a, splits), (long long)nsa::decode_split_static_bytes());
+      if (rc == -2) return fail(NSA_ERR_UNSUPPORTED, "%s: head dims or split count not built", what);
+      if (rc == -4) return fail(NSA_ERR_LAUNCH, "%s: could not look up the library's scratch array on this device", what);
+      return finish(rc, what);
+    }
     if (!workspace || !aligned16(workspace) || workspace_bytes < nsa::decode_split_workspace_bytes(a, splits))
       return fail(NSA_ERR_INVALID, "%s: workspace missing, misaligned or smaller than nsa_decode_split_workspace_bytes", what);
     const int rc = nsa::launch_decode_split(a, splits, workspace, stream);
@@ -508,6 +518,22 @@ int nsa_decode_step_split(const void* q, const void* k_cache, const void* v_cach
                        block_table ? max_pages * 64 : ctx_cap, nc_cap, block, stride, sel_block, pool_kernel,
                        pool_stride, pool_pad, top_n, window, scale, gate_act, dtype, stream, splits, workspace,
                        workspace_bytes);
+}
+
+int64_t nsa_decode_split_static_bytes(void) { return nsa::decode_split_static_bytes(); }
+
+int nsa_decode_step_split_static(const void* q, const void* k_cache, const void* v_cache_t, const int32_t* block_table,
+                                 int max_pages, const void* ck_cache, const void* cv_cache_t, const int32_t* ctx_lens,
+                                 const void* gates, void* out, int32_t* indices, int batch, int hq, int hkv, int dk,
+                                 int dv, int ctx_cap, int nc_cap, int block, int stride, int sel_block, int pool_kernel,
+                                 int pool_stride, int pool_pad, int top_n, int window, float scale, int gate_act,
+                                 int dtype, int splits, nsa_stream_t stream) {
+  if (splits <= 0) return fail(NSA_ERR_INVALID, "decode_step_split_static: splits must be positive");
+  if (block_table && max_pages <= 0) return fail(NSA_ERR_INVALID, "decode_step_split_static: a block table needs max_pages");
+  return decode_common("decode_step_split_static", q, k_cache, v_cache_t, block_table, block_table ? max_pages : 0,
+                       ck_cache, cv_cache_t, ctx_lens, gates, out, indices, batch, hq, hkv, dk, dv,
+                       block_table ? max_pages * 64 : ctx_cap, nc_cap, block, stride, sel_block, pool_kernel,
+                       pool_stride, pool_pad, top_n, window, scale, gate_act, dtype, stream, splits, nullptr, 0, true);
 }
 
 int nsa_decode_step(const void* q, const void* k_cache, const void* v_cache_t, const void* ck_cache,

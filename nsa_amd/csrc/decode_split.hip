@@ -12,6 +12,8 @@
 //   C  merges the partial states of the three branches, gates, stores
 // Same arithmetic as the one-workgroup kernel up to the order of fp32 sums.  Pooling 5 / 4 / 0 only
 // (windows of 5 compressed rows every 4, the default geometry).
+#include <mutex>
+
 #include "decode_common.h"
 
 namespace nsa {
@@ -532,6 +534,38 @@ static int launch_decode_split_t(const DecodeArgs& a, int splits, float* ws, hip
 }
 
 int decode_split_max_nc() { return kSplitMaxSlices * kSplitMaxSlice; }
+
+// ---- the same step for callers that cannot allocate --------------------------------------------------
+// The partial results live in a fixed array of the library instead of a caller workspace.  Every GPU the
+// library runs on holds its own copy of the array at its own address; `scratch` itself is only the host-side
+// name of the symbol, so the device address is looked up once per device and that pointer is what the kernels
+// get.  All calls on one GPU share the array: calls that overlap in time race.
+constexpr long kStaticScratchBytes = 16L << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static void* g_scratch_ptr[kMaxDevices];           // device address of `scratch` on each GPU, null = not looked up yet
+static std::mutex g_scratch_mutex;
+
+long decode_split_static_bytes() { return kStaticScratchBytes; }
+
+// -1: the workspace of this call does not fit the array; -4: the symbol lookup failed
+int launch_decode_split_static(const DecodeArgs& a, int splits, hipStream_t st) {
+  if (decode_split_workspace_bytes(a, splits) > kStaticScratchBytes) return -1;
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return -4;
+  void* ptr;
+  {
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+      void* p = nullptr;
+      if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) return -4;
+      g_scratch_ptr[dev] = p;
+    }
+    ptr = g_scratch_ptr[dev];
+  }
+  return launch_decode_split(a, splits, ptr, st);
+}
 
 int launch_decode_split(const DecodeArgs& a, int splits, void* workspace, hipStream_t st) {
   float* ws = reinterpret_cast<float*>(workspace);

@@ -157,5 +157,8 @@ int decode_split_max_nc();
 // the same step spread over `splits` workgroups per (sequence, kv head), for small batches
 long decode_split_workspace_bytes(const DecodeArgs& a, int splits);
 int launch_decode_split(const DecodeArgs& a, int splits, void* workspace, hipStream_t st);
+// the same with the partial results in a fixed device array of the library (no workspace argument)
+long decode_split_static_bytes();
+int launch_decode_split_static(const DecodeArgs& a, int splits, hipStream_t st);
 
 }  // namespace nsa

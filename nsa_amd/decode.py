@@ -223,7 +223,8 @@ class NSAPagedDecodeCache:
 def nsa_decode_step(q: torch.Tensor, cache, gates: Optional[torch.Tensor] = None,
                     selection_block: int = 64, selected_block_count: int = 16, sliding_window: int = 512,
                     scale: Optional[float] = None, gate_activation: Optional[str] = None,
-                    return_indices: bool = False, splits: Optional[int] = None):
+                    return_indices: bool = False, splits: Optional[int] = None, out: Optional[torch.Tensor] = None,
+                    indices: Optional[torch.Tensor] = None, static_scratch: bool = False):
     """q [B,Hq,Dk]: queries of the newest cached token; cache: NSADecodeCache or NSAPagedDecodeCache.  gates [B,Hq,3] (selected, sliding,
     compressed; pre-activation if gate_activation == "sigmoid").  Returns out [B,Hq,Dv]
     (and int32 block indices [B,Hkv,S]).
@@ -233,16 +234,28 @@ def nsa_decode_step(q: torch.Tensor, cache, gates: Optional[torch.Tensor] = None
     most of the chip idle and its ~60 us critical path sets the step time, so the work is split 8 ways
     (three launches, partial results in a workspace kept on the cache object).  Caches with more
     compressed rows than one workgroup keeps in registers (contexts beyond ~36k tokens) always take the
-    split schedule, whose first launch cuts the compressed rows into slices of at most 384."""
+    split schedule, whose first launch cuts the compressed rows into slices of at most 384.
+
+    out [B,Hq,Dv] / indices int32 [B,Hkv,S]: result buffers of the caller (allocated here when None).
+    static_scratch: run the split schedule with its partial results in the library's own fixed device array
+    (nsa_decode_step_split_static): with `out` (and `indices`) given, the call then allocates nothing, for
+    callers that must not (graph capture, serving loops).  Calls that overlap on one GPU race on that array."""
     if not q.is_cuda:
         raise RuntimeError("NSA kernels run on the GPU only")
     B, hq, dk = q.shape
     q = q.contiguous()
     if scale is None:
         scale = 1.0 / math.sqrt(dk)
-    out = torch.empty(B, hq, cache.dv, dtype=q.dtype, device=q.device)
-    idx = torch.empty(B, cache.hkv, selected_block_count, dtype=torch.int32, device=q.device) \
-        if return_indices else None
+    if out is None:
+        out = torch.empty(B, hq, cache.dv, dtype=q.dtype, device=q.device)
+    elif out.shape != (B, hq, cache.dv) or out.dtype != q.dtype or not out.is_contiguous():
+        raise ValueError("out must be a contiguous [B,Hq,Dv] tensor of q's dtype")
+    idx = indices
+    if idx is None and return_indices:
+        idx = torch.empty(B, cache.hkv, selected_block_count, dtype=torch.int32, device=q.device)
+    elif idx is not None and (idx.shape != (B, cache.hkv, selected_block_count) or idx.dtype != torch.int32
+                              or not idx.is_contiguous()):
+        raise ValueError("indices must be a contiguous int32 [B,Hkv,S] tensor")
     if gates is not None:
         gates = gates.to(q.dtype).contiguous()
     pool_k = selection_block // cache.stride + 1
@@ -263,6 +276,17 @@ def nsa_decode_step(q: torch.Tensor, cache, gates: Optional[torch.Tensor] = None
         raise NotImplementedError(
             "the one-workgroup decode step keeps at most %d compressed rows per sequence; this cache holds up "
             "to %d (pass splits=None or a positive split count)" % (lib.nsa_decode_max_compressed(), cache.nc_cap))
+    if static_scratch:
+        splits = splits or 8
+        k_c, v_c = (cache.k_pool, cache.v_pool_t) if paged else (cache.k, cache.vt)
+        rc = lib.nsa_decode_step_split_static(
+            _ptr(q), _ptr(k_c), _ptr(v_c), _ptr(cache.block_table) if paged else None,
+            cache.max_pages if paged else 0, _ptr(cache.ck), _ptr(cache.cvt), _ptr(cache.ctx_lens), _ptr(gates),
+            _ptr(out), _ptr(idx), B, hq, cache.hkv, dk, cache.dv, cache.ctx_cap, cache.nc_cap, cache.block,
+            cache.stride, selection_block, pool_k, pool_s, pool_p, selected_block_count, sliding_window,
+            float(scale), act, _dtype_code(q), splits, _stream())
+        _lib.check(rc, "nsa_decode_step_split_static")
+        return (out, idx) if return_indices else out
     if splits:
         need = lib.nsa_decode_split_workspace_bytes(B, cache.hkv, cache.dv, cache.nc_cap, splits)
         ws = getattr(cache, "_split_ws", None)
