@@ -9,6 +9,11 @@
  *     with cu_seqlens[0] == 0 holds the row offsets; a batch of equal lengths is the special case
  *     cu_seqlens[b] = b*T
  *   - dtype: NSA_BF16 or NSA_F32 for every floating tensor of a call (accumulation is always fp32)
+ *   - GQA: hq / hkv query heads share one kv head.  Groups of 1..16 heads are built everywhere; the prefill
+ *     forward entry points (nsa_cmp_attn_*, nsa_block_select_fwd, nsa_swa_fwd, nsa_slc_*, nsa_swa_merge_fwd)
+ *     also take groups of 32, 48, 64, ... heads, which is what the reference's selected attention asks for
+ *     (HQ a multiple of 16 * H, nsa/selection_attn.py:800): they run as hq / (16 * hkv) sub-groups of 16 heads
+ *     that share the keys, values and block picks of their kv head.  Backward and decode: groups up to 16.
  *   - return value: 0 on success, negative on error (NSA_ERR_*); nsa_last_error_string() describes
  *     the last error of the calling thread.  No exception crosses this boundary.
  *   - "transposed" buffers hold one key-contiguous plane per head: element (h, d, col) lives at
@@ -83,7 +88,8 @@ int nsa_compress_bwd(const void* x, const void* w_lin, const void* d_out, void* 
  *   q [total, hq, dk]; ck rows at ck + (cu_cmp[b] + c)*ck_row_stride + h*ck_head_stride (dk elements);
  *   cvt transposed [hkv][dv][cvt_cols] over cu_cmp; o [total, hq, dv];
  *   indices [total, hkv, top_n] int32 or int64 (idx64), descending score, -1 where fewer bins exist;
- *   NULL skips the selection;  pooled (optional, float) [total, hkv, pooled_stride] receives the
+ *   NULL skips the selection;  pooled (optional, float) [total, hkv, sub, pooled_stride] with sub =
+ *   max(1, hq / (16 * hkv)) sub-groups (1 for GQA groups up to 16 heads) receives in its first sub-row the
  *   pooled block scores (bins past a sequence's last one up to max_ns are zeroed).  Pass it even when
  *   the scores are not wanted: with it (and a GQA group of 9..16 heads, pooling 5/4/0, max_ns <= 4096,
  *   top_n <= 64) the selection runs as two lean kernels that use it as their hand-over buffer, without
@@ -218,7 +224,8 @@ int nsa_swa_merge_fwd(const void* q, const void* k, const void* vt, const void* 
                       const void* workspace, int64_t workspace_bytes, nsa_stream_t stream);
 
 /* Bytes of the optional workspace of nsa_slc_combine_fwd; 0 when the shape has no block-major path
- * (bf16, selection blocks of 64 keys only). */
+ * (bf16, selection blocks of 64 keys only).  hkv: kv heads, times hq / (16 * hkv) when the GQA group has more
+ * than 16 heads (one set of partial results per sub-group of 16 query heads). */
 int64_t nsa_slc_workspace_bytes(int total, int batch, int hkv, int dk, int dv, int top_n, int block_size, int dtype);
 
 /* Backward of the compressed attention.  Replaces nsa/triton_attention.py:478-546

@@ -30,6 +30,8 @@ struct StreamParams {
   float scale;
   MergeArgs mg;      // MERGE kernels only: the selected-attention partials and the other branches
   float* lse_attn;   // optional: log-sum-exp (natural log) of the scaled visible scores, for the backward
+  int kv_rep;        // sub-groups of 16 query heads per kv head (1 unless the GQA group exceeds 16): hkv counts
+                     // sub-groups, and sub-group h reads the keys / values of kv head h / kv_rep
 };
 
 // MERGE (sliding window only): 0 = write the branch output; otherwise the epilogue merges the
@@ -54,6 +56,7 @@ stream_attn_kernel(const StreamParams a) {
   const SeqTile st = find_tile(a.cu_seq, a.batch, TQ, blockIdx.x);
   if (!st.valid) return;
   const int h = blockIdx.y;
+  const int hk = h / a.kv_rep;                 // kv head whose keys / values this (sub-)group reads
   const int t_last = min(st.t0 + TQ, st.len) - 1;
 
   // key space of this sequence
@@ -67,8 +70,8 @@ stream_attn_kernel(const StreamParams a) {
     nkeys = st.len;
     vtoff = transposed_offset(st.start, st.b);
   }
-  const T* kb = reinterpret_cast<const T*>(a.k) + (long)koff * a.k_row_stride + (long)h * a.k_head_stride;
-  const T* vtb = reinterpret_cast<const T*>(a.vt) + (long)h * DV * a.vt_cols + vtoff;
+  const T* kb = reinterpret_cast<const T*>(a.k) + (long)koff * a.k_row_stride + (long)hk * a.k_head_stride;
+  const T* vtb = reinterpret_cast<const T*>(a.vt) + (long)hk * DV * a.vt_cols + vtoff;
   const int W = a.window;
 
   auto last_visible = [&](int t) -> int {      // largest key index token t may attend
@@ -421,11 +424,12 @@ slc_combine_kernel(const SlcArgs a) {
   const SeqTile st = find_tile(a.cu_seq, a.batch, TQ, tile);
   if (!st.valid) return;
   const int S = a.top_n, BS = a.block_size;
+  const int hk = h / a.kv_rep, hkv_r = a.hkv / a.kv_rep;     // kv head of this (sub-)group, number of kv heads
   const T* qb = reinterpret_cast<const T*>(a.q);
-  const T* kb = reinterpret_cast<const T*>(a.k) + ((long)st.start * a.hkv + h) * DK + 8 * g;
-  const T* vtb = reinterpret_cast<const T*>(a.vt) + (long)h * DV * a.vt_cols + transposed_offset(st.start, st.b)
+  const T* kb = reinterpret_cast<const T*>(a.k) + ((long)st.start * hkv_r + hk) * DK + 8 * g;
+  const T* vtb = reinterpret_cast<const T*>(a.vt) + (long)hk * DV * a.vt_cols + transposed_offset(st.start, st.b)
                  + (long)n * a.vt_cols + 8 * g;
-  const long krow = (long)a.hkv * DK;
+  const long krow = (long)hkv_r * DK;
   const long vstep = 16L * a.vt_cols;
 
   RowGroup<T, DK, DV> grp[1];
@@ -443,7 +447,7 @@ slc_combine_kernel(const SlcArgs a) {
   for (int tk = 0; tk < tpg; ++tk) {
     const int tt = tfirst + tk;
     if (tt >= st.len) break;
-    const long irow = ((long)st.start + tt) * a.hkv + h;
+    const long irow = ((long)st.start + tt) * hkv_r + hk;
     int cnt = S;
     if (a.counts != nullptr) cnt = min(max(a.counts[irow], 0), S);
     long myidx = -1;
@@ -591,21 +595,21 @@ static int launch_stream_t(const StreamParams& a, int total, hipStream_t st) {
 template <typename T, int DK, int DV>
 static int launch_cmp_t(const CmpArgs& a, hipStream_t st) {
   StreamParams p{a.q, a.ck, a.cvt, a.o, a.lse, a.cu_seq, a.cu_cmp, a.batch, a.hq, a.hkv, a.ck_row_stride,
-                 a.ck_head_stride, a.cvt_cols, a.block, a.stride, 0, a.causal, a.scale, MergeArgs{}, a.lse_attn};
+                 a.ck_head_stride, a.cvt_cols, a.block, a.stride, 0, a.causal, a.scale, MergeArgs{}, a.lse_attn, a.kv_rep};
   return launch_stream_t<T, DK, DV, true>(p, a.total, st);
 }
 
 template <typename T, int DK, int DV>
 static int launch_swa_t(const SwaArgs& a, hipStream_t st) {
-  StreamParams p{a.q, a.k, a.vt, a.o, nullptr, a.cu_seq, a.cu_seq, a.batch, a.hq, a.hkv, (long)a.hkv * DK,
-                 (long)DK, a.vt_cols, 0, 0, a.window, 1, a.scale, MergeArgs{}, a.lse};
+  StreamParams p{a.q, a.k, a.vt, a.o, nullptr, a.cu_seq, a.cu_seq, a.batch, a.hq, a.hkv, (long)(a.hkv / a.kv_rep) * DK,
+                 (long)DK, a.vt_cols, 0, 0, a.window, 1, a.scale, MergeArgs{}, a.lse, a.kv_rep};
   return launch_stream_t<T, DK, DV, false>(p, a.total, st);
 }
 
 template <int DK, int DV>
 static int launch_swa_merge_t(const SwaArgs& a, const MergeArgs& m, hipStream_t st) {
-  StreamParams p{a.q, a.k, a.vt, nullptr, nullptr, a.cu_seq, a.cu_seq, a.batch, a.hq, a.hkv, (long)a.hkv * DK,
-                 (long)DK, a.vt_cols, 0, 0, a.window, 1, a.scale, m, a.lse};
+  StreamParams p{a.q, a.k, a.vt, nullptr, nullptr, a.cu_seq, a.cu_seq, a.batch, a.hq, a.hkv, (long)(a.hkv / a.kv_rep) * DK,
+                 (long)DK, a.vt_cols, 0, 0, a.window, 1, a.scale, m, a.lse, a.kv_rep};
   if (m.top_n == 16) return launch_stream_t<bf16_t, DK, DV, false, 16>(p, a.total, st);
   return launch_stream_t<bf16_t, DK, DV, false, 1>(p, a.total, st);
 }

@@ -29,9 +29,19 @@ int finish(int rc, const char* what) {
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-int check_heads(const char* what, int hq, int hkv, int dk, int dv) {
+// GQA groups of up to 16 heads are one MFMA tile column set.  The prefill forward also takes groups of 32, 48,
+// 64, ... heads (what the reference's selected attention asks for: HQ a multiple of 16 * H,
+// nsa/selection_attn.py:800): they run as hq / (16 * hkv) sub-groups of 16 heads that share the keys, values
+// and block picks of their kv head.  *kv_rep receives that count (1 for groups up to 16).
+int check_heads(const char* what, int hq, int hkv, int dk, int dv, int* kv_rep = nullptr) {
   if (hq <= 0 || hkv <= 0 || hq % hkv != 0) return fail(NSA_ERR_INVALID, "%s: hq must be a positive multiple of hkv", what);
-  if (hq / hkv > 16) return fail(NSA_ERR_UNSUPPORTED, "%s: GQA group size %d > 16 is not built", what, hq / hkv);
+  const int G = hq / hkv;
+  if (kv_rep) *kv_rep = 1;
+  if (G > 16) {
+    if (!kv_rep) return fail(NSA_ERR_UNSUPPORTED, "%s: GQA group size %d > 16 is not built for this call", what, G);
+    if (G % 16 != 0) return fail(NSA_ERR_UNSUPPORTED, "%s: GQA group size %d: groups beyond 16 heads must be multiples of 16", what, G);
+    *kv_rep = G / 16;
+  }
   if (dk % 32 != 0 || dv % 16 != 0) return fail(NSA_ERR_UNSUPPORTED, "%s: dk must be a multiple of 32 and dv of 16", what);
   return 0;
 }
@@ -107,7 +117,8 @@ static int cmp_common(const char* what, int stages, const void* q, const void* c
   if (attn && (!cvt || !o)) return fail(NSA_ERR_INVALID, "%s: null pointer", what);
   if (batch <= 0 || total <= 0 || block <= 0 || stride <= 0) return fail(NSA_ERR_INVALID, "%s: sizes must be positive", what);
   if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "%s: bad dtype", what);
-  if (int rc = check_heads(what, hq, hkv, dk, dv)) return rc;
+  int kv_rep = 1;
+  if (int rc = check_heads(what, hq, hkv, dk, dv, &kv_rep)) return rc;
   if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "%s: scale must be positive", what);
   if (ck_row_stride % 8 != 0 || ck_head_stride % 8 != 0 || (attn && cvt_cols % 64 != 0))
     return fail(NSA_ERR_INVALID, "%s: ck strides must be multiples of 8, cvt_cols of 64", what);
@@ -121,12 +132,15 @@ static int cmp_common(const char* what, int stages, const void* q, const void* c
   } else {
     max_ns = 0;
   }
-  nsa::CmpArgs a{q, ck, cvt, o, indices, pooled, lse, cu_seqlens, cu_cmp, batch, total, hq, hkv, dk, dv,
+  nsa::CmpArgs a{q, ck, cvt, o, indices, pooled, lse, cu_seqlens, cu_cmp, batch, total, hq, hkv * kv_rep, dk, dv,
                  (long)ck_row_stride, (long)ck_head_stride, cvt_cols, block, stride, pool_kernel, pool_stride,
-                 pool_pad, top_n, max_ns, pooled_stride, scale, idx64, dtype, causal, lse_attn};
+                 pool_pad, top_n, max_ns, pooled_stride, scale, idx64, dtype, causal, lse_attn, kv_rep};
   int rc = 0;
   if (attn) rc = nsa::launch_cmp_attn(a, stream);
   if (rc == 0 && select) rc = nsa::launch_select(a, stream);
+  if (rc == -6)
+    return fail(NSA_ERR_UNSUPPORTED, "%s: GQA groups beyond 16 heads are selected on the two-kernel schedule only "
+                "(pooled buffer given, pooling 5 / 4 / 0, max_ns <= 4096, top_n <= 64)", what);
   return finish(rc, what);
 }
 
@@ -246,11 +260,12 @@ int nsa_swa_fwd(const void* q, const void* k, const void* vt, void* o, float* ls
   if (!q || !k || !vt || !o || !cu_seqlens) return fail(NSA_ERR_INVALID, "swa: null pointer");
   if (batch <= 0 || total <= 0 || window <= 0) return fail(NSA_ERR_INVALID, "swa: sizes must be positive");
   if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "swa: bad dtype");
-  if (int rc = check_heads("swa", hq, hkv, dk, dv)) return rc;
+  int kv_rep = 1;
+  if (int rc = check_heads("swa", hq, hkv, dk, dv, &kv_rep)) return rc;
   if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "swa: scale must be positive");
   if (vt_cols % 64 != 0 || vt_cols < nsa_transposed_cols(total, batch)) return fail(NSA_ERR_INVALID, "swa: vt_cols too small or not a multiple of 64");
   if (!aligned16(q) || !aligned16(k) || !aligned16(vt) || !aligned16(o)) return fail(NSA_ERR_INVALID, "swa: pointers must be 16-byte aligned");
-  nsa::SwaArgs a{q, k, vt, o, cu_seqlens, batch, total, hq, hkv, dk, dv, vt_cols, window, scale, dtype, lse};
+  nsa::SwaArgs a{q, k, vt, o, cu_seqlens, batch, total, hq, hkv * kv_rep, dk, dv, vt_cols, window, scale, dtype, lse, kv_rep};
   return finish(nsa::launch_swa(a, stream), "swa");
 }
 
@@ -271,7 +286,8 @@ int nsa_slc_combine_fwd(const void* q, const void* k, const void* vt, const void
   if (!q || !k || !vt || !indices || !out || !cu_seqlens) return fail(NSA_ERR_INVALID, "slc_combine: null pointer");
   if (batch <= 0 || total <= 0) return fail(NSA_ERR_INVALID, "slc_combine: sizes must be positive");
   if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "slc_combine: bad dtype");
-  if (int rc = check_heads("slc_combine", hq, hkv, dk, dv)) return rc;
+  int kv_rep = 1;
+  if (int rc = check_heads("slc_combine", hq, hkv, dk, dv, &kv_rep)) return rc;
   if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "slc_combine: scale must be positive");
   if (top_n <= 0 || top_n > 64) return fail(NSA_ERR_UNSUPPORTED, "slc_combine: 1 <= top_n <= 64");
   if (block_size <= 0 || block_size % 8 != 0) return fail(NSA_ERR_UNSUPPORTED, "slc_combine: block_size must be a multiple of 8");
@@ -279,8 +295,8 @@ int nsa_slc_combine_fwd(const void* q, const void* k, const void* vt, const void
   if (gate_act != NSA_GATE_IDENTITY && gate_act != NSA_GATE_SIGMOID) return fail(NSA_ERR_INVALID, "slc_combine: bad gate activation");
   if (!aligned16(q) || !aligned16(k) || !aligned16(vt)) return fail(NSA_ERR_INVALID, "slc_combine: pointers must be 16-byte aligned");
   nsa::SlcArgs a{q, k, vt, indices, counts, g_slc, g_swa, g_cmp, (long)gate_stride, o_swa, o_cmp, out, cu_seqlens,
-                 batch, total, hq, hkv, dk, dv, vt_cols, top_n, block_size, scale, idx64, gate_act, dtype,
-                 workspace, (long)workspace_bytes, lse_slc};
+                 batch, total, hq, hkv * kv_rep, dk, dv, vt_cols, top_n, block_size, scale, idx64, gate_act, dtype,
+                 workspace, (long)workspace_bytes, lse_slc, kv_rep};
   if (workspace && !aligned16(workspace)) return fail(NSA_ERR_INVALID, "slc_combine: workspace must be 16-byte aligned");
   const int rc = nsa::launch_slc_combine(a, stream);
   if (rc == -5) return fail(NSA_ERR_UNSUPPORTED, "slc_combine: lse_slc needs the block-major schedule (bf16, 64-key blocks, a workspace)");
@@ -289,15 +305,16 @@ int nsa_slc_combine_fwd(const void* q, const void* k, const void* vt, const void
 
 static int slc_common_checks(const char* what, const void* q, const void* k, const void* vt, const int32_t* cu_seqlens,
                              int batch, int total, int hq, int hkv, int dk, int dv, int vt_cols, int top_n,
-                             int block_size, float scale, int dtype, const void* workspace, int64_t workspace_bytes) {
+                             int block_size, float scale, int dtype, const void* workspace, int64_t workspace_bytes,
+                             int* kv_rep) {
   if (!q || !k || !vt || !cu_seqlens || !workspace) return fail(NSA_ERR_INVALID, "%s: null pointer", what);
   if (batch <= 0 || total <= 0) return fail(NSA_ERR_INVALID, "%s: sizes must be positive", what);
   if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "%s: bad dtype", what);
-  if (int rc = check_heads(what, hq, hkv, dk, dv)) return rc;
+  if (int rc = check_heads(what, hq, hkv, dk, dv, kv_rep)) return rc;
   if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "%s: scale must be positive", what);
   if (vt_cols % 64 != 0 || vt_cols < nsa_transposed_cols(total, batch)) return fail(NSA_ERR_INVALID, "%s: vt_cols too small or not a multiple of 64", what);
   if (!aligned16(q) || !aligned16(k) || !aligned16(vt) || !aligned16(workspace)) return fail(NSA_ERR_INVALID, "%s: pointers must be 16-byte aligned", what);
-  const int64_t need = nsa_slc_workspace_bytes(total, batch, hkv, dk, dv, top_n, block_size, dtype);
+  const int64_t need = nsa_slc_workspace_bytes(total, batch, hkv * *kv_rep, dk, dv, top_n, block_size, dtype);
   if (need == 0) return fail(NSA_ERR_UNSUPPORTED, "%s: the block-major schedule needs bf16, 64-key blocks, top_n <= 64 and (dk,dv) in (64,64),(128,128),(192,128)", what);
   if (workspace_bytes < need) return fail(NSA_ERR_INVALID, "%s: workspace smaller than nsa_slc_workspace_bytes", what);
   return 0;
@@ -308,11 +325,12 @@ int nsa_slc_partials_fwd(const void* q, const void* k, const void* vt, const voi
                          int vt_cols, int top_n, int block_size, float scale, int idx64, int dtype, void* workspace,
                          int64_t workspace_bytes, nsa_stream_t stream) {
   if (!indices) return fail(NSA_ERR_INVALID, "slc_partials: null pointer");
+  int kv_rep = 1;
   if (int rc = slc_common_checks("slc_partials", q, k, vt, cu_seqlens, batch, total, hq, hkv, dk, dv, vt_cols, top_n,
-                                 block_size, scale, dtype, workspace, workspace_bytes)) return rc;
+                                 block_size, scale, dtype, workspace, workspace_bytes, &kv_rep)) return rc;
   nsa::SlcArgs a{q, k, vt, indices, counts, nullptr, nullptr, nullptr, 1, nullptr, nullptr, nullptr, cu_seqlens,
-                 batch, total, hq, hkv, dk, dv, vt_cols, top_n, block_size, scale, idx64, 0, dtype,
-                 workspace, (long)workspace_bytes, nullptr};
+                 batch, total, hq, hkv * kv_rep, dk, dv, vt_cols, top_n, block_size, scale, idx64, 0, dtype,
+                 workspace, (long)workspace_bytes, nullptr, kv_rep};
   return finish(nsa::launch_slc_partials(a, workspace, stream), "slc_partials");
 }
 
@@ -327,17 +345,18 @@ int nsa_swa_merge_fwd(const void* q, const void* k, const void* vt, const void* 
     return fail(NSA_ERR_INVALID, "swa_merge: pointers must be 16-byte aligned");
   if (window <= 0) return fail(NSA_ERR_INVALID, "swa_merge: window must be positive");
   if (gate_act != NSA_GATE_IDENTITY && gate_act != NSA_GATE_SIGMOID) return fail(NSA_ERR_INVALID, "swa_merge: bad gate activation");
+  int kv_rep = 1;
   if (int rc = slc_common_checks("swa_merge", q, k, vt, cu_seqlens, batch, total, hq, hkv, dk, dv, vt_cols, top_n,
-                                 block_size, scale, dtype, workspace, workspace_bytes)) return rc;
+                                 block_size, scale, dtype, workspace, workspace_bytes, &kv_rep)) return rc;
   if (!aligned16(out) || (o_cmp && !aligned16(o_cmp))) return fail(NSA_ERR_INVALID, "swa_merge: pointers must be 16-byte aligned");
   // the picks themselves are not needed here: the workspace's slot map says which have a partial
   nsa::SlcArgs sa{q, k, vt, nullptr, nullptr, g_slc, g_swa, g_cmp, (long)gate_stride, nullptr, o_cmp, out, cu_seqlens,
-                  batch, total, hq, hkv, dk, dv, vt_cols, top_n, block_size, scale, 0, gate_act, dtype,
-                  const_cast<void*>(workspace), (long)workspace_bytes, nullptr};
+                  batch, total, hq, hkv * kv_rep, dk, dv, vt_cols, top_n, block_size, scale, 0, gate_act, dtype,
+                  const_cast<void*>(workspace), (long)workspace_bytes, nullptr, kv_rep};
   nsa::MergeArgs m = nsa::slc_merge_args(sa, const_cast<void*>(workspace));
   m.o_slc_out = o_slc_out; m.o_swa_out = o_swa_out; m.lse_slc_out = lse_slc_out;
-  nsa::SwaArgs a{q, k, vt, nullptr, cu_seqlens, batch, total, hq, hkv, dk, dv, vt_cols, window, scale, dtype,
-                 lse_swa_out};
+  nsa::SwaArgs a{q, k, vt, nullptr, cu_seqlens, batch, total, hq, hkv * kv_rep, dk, dv, vt_cols, window, scale, dtype,
+                 lse_swa_out, kv_rep};
   return finish(nsa::launch_swa_merge(a, m, stream), "swa_merge");
 }
 

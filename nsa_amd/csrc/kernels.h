@@ -32,12 +32,16 @@ struct CmpArgs {
   int block, stride, pool_k, pool_s, pool_p, top_n, max_ns, pooled_stride;
   float scale; int idx64, dtype, causal;
   float* lse_attn;   // optional: natural-log log-sum-exp of the scaled visible scores (+inf: no key visible)
+  // GQA groups beyond 16 heads run as kv_rep = G / 16 sub-groups of 16: hkv then counts the sub-groups
+  // ("virtual" kv heads, hq / hkv == 16) and sub-group h reads the K / V rows of kv head h / kv_rep
+  int kv_rep = 1;
 };
 
 struct SwaArgs {
   const void* q; const void* k; const void* vt; void* o; const int32_t* cu_seq;
   int batch, total, hq, hkv, dk, dv, vt_cols, window; float scale; int dtype;
   float* lse;        // optional, as CmpArgs::lse_attn
+  int kv_rep = 1;    // as CmpArgs::kv_rep
 };
 
 struct SlcArgs {
@@ -48,6 +52,7 @@ struct SlcArgs {
   int idx64, gate_act, dtype;
   void* workspace; long workspace_bytes;
   float* lse;        // optional (block-major schedule only), as CmpArgs::lse_attn
+  int kv_rep = 1;    // as CmpArgs::kv_rep; indices and counts stay per real kv head
 };
 
 // Where the merge of the block-major partial results finds its inputs (all device pointers; the

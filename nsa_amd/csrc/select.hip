@@ -253,7 +253,8 @@ importance_stream_kernel(const CmpArgs a) {
   }
   Ns = min(Ns, a.max_ns);
   if (Ns == 0) return;
-  const T* ckb = reinterpret_cast<const T*>(a.ck) + (long)coff * a.ck_row_stride + (long)h * a.ck_head_stride;
+  // h counts sub-groups of 16 query heads; sub-group h scores against the compressed keys of kv head h / kv_rep
+  const T* ckb = reinterpret_cast<const T*>(a.ck) + (long)coff * a.ck_row_stride + (long)(h / a.kv_rep) * a.ck_head_stride;
 
   vec8_t<T> qf[NG][DK / 32];
   float lse_r[NG][4];        // lse * log2(e) of heads 4g+i of each token; +inf removes padded rows
@@ -401,13 +402,17 @@ importance_stream_kernel(const CmpArgs a) {
 // One wavefront per (token, kv head): window sums -> averages (ceil-mode pool, padding counted in
 // the divisor, written back over the sums, bins past the sequence's last one zeroed) and the top_n
 // bins in descending order, ties to the lower index, -1 where the sequence has fewer bins.
+// With kv_rep > 1 (GQA group of kv_rep * 16 heads) a.pooled holds one row of window sums per sub-group of 16
+// heads, kv_rep consecutive rows per kv head: they are added up here (the importance of a block is the sum over
+// all heads of the group), and the averages go to the first of them.
 template <int PER>
 __global__ void __launch_bounds__(256)
 topn_kernel(const CmpArgs a) {
   const int lane = threadIdx.x & 63;
-  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);       // token * hkv + head
-  if (row >= (long)a.total * a.hkv) return;
-  const int tg = (int)(row / a.hkv);
+  const int hkv_r = a.hkv / a.kv_rep;
+  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);       // token * (kv heads) + kv head
+  if (row >= (long)a.total * hkv_r) return;
+  const int tg = (int)(row / hkv_r);
   int sb = 0;
   {
     int hi = a.batch;
@@ -423,12 +428,19 @@ topn_kernel(const CmpArgs a) {
     if ((Ns - 1) * a.pool_s >= Nc + a.pool_p) --Ns;
   }
   Ns = min(Ns, a.max_ns);
-  float* prow = a.pooled + row * a.pooled_stride;
+  float* prow = a.pooled + row * a.kv_rep * a.pooled_stride;
   float v[PER];
 #pragma unroll
   for (int k = 0; k < PER; ++k) {
     const int b = lane + 64 * k;
     v[k] = b < Ns ? prow[b] : -1.f;
+  }
+  for (int r = 1; r < a.kv_rep; ++r) {
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      const int b = lane + 64 * k;
+      if (b < Ns) v[k] += prow[(long)r * a.pooled_stride + b];
+    }
   }
 #pragma unroll
   for (int k = 0; k < PER; ++k) {
@@ -495,7 +507,7 @@ static int launch_select_stream(const CmpArgs& a, hipStream_t st) {
   if (rc) return rc;
   const int tiles = a.total / TQ + a.batch;
   hipLaunchKernelGGL(fn, dim3(tiles, a.hkv), dim3(NW * 64), smem, st, a);
-  const int rows = (int)(((long)a.total * a.hkv + 3) / 4);
+  const int rows = (int)(((long)a.total * (a.hkv / a.kv_rep) + 3) / 4);
   if (a.max_ns <= 512) hipLaunchKernelGGL(topn_kernel<8>, dim3(rows), dim3(256), 0, st, a);
   else if (a.max_ns <= 1024) hipLaunchKernelGGL(topn_kernel<16>, dim3(rows), dim3(256), 0, st, a);
   else if (a.max_ns <= 2048) hipLaunchKernelGGL(topn_kernel<32>, dim3(rows), dim3(256), 0, st, a);
@@ -508,6 +520,7 @@ static int launch_select_t(const CmpArgs& a, hipStream_t st) {
   if (a.pooled != nullptr && a.max_ns <= 4096 && a.top_n <= 64 && group_pow2(a.hq / a.hkv) == 16 && a.pool_k == 5 &&
       a.pool_s == 4 && a.pool_p == 0)
     return launch_select_stream<T, DK>(a, st);
+  if (a.kv_rep > 1) return -6;      // groups beyond 16 heads exist on the two-kernel schedule only
   // four row groups per wavefront unless the per-token bins of such a tile outgrow the LDS
   constexpr int NGBIG = sizeof(T) == 2 ? 4 : 2;
   const int rc = launch_select_ng<T, DK, NGBIG>(a, st);

@@ -92,10 +92,11 @@ slc_bucket_kernel(const SlcArgs a, SlcWs ws) {
   const int h = (int)(th % a.hkv), tg = (int)(th / a.hkv);
   const int b = seq_of_token(a.cu_seq, a.batch, tg);
   const int t = tg - a.cu_seq[b];
+  const long th_r = (long)tg * (a.hkv / a.kv_rep) + h / a.kv_rep;      // picks and counts are per real kv head
   int cnt = a.top_n;
-  if (a.counts != nullptr) cnt = min(max(a.counts[th], 0), a.top_n);
-  const long idx = a.idx64 ? reinterpret_cast<const int64_t*>(a.indices)[id]
-                           : (long)reinterpret_cast<const int32_t*>(a.indices)[id];
+  if (a.counts != nullptr) cnt = min(max(a.counts[th_r], 0), a.top_n);
+  const long idx = a.idx64 ? reinterpret_cast<const int64_t*>(a.indices)[th_r * a.top_n + i]
+                           : (long)reinterpret_cast<const int32_t*>(a.indices)[th_r * a.top_n + i];
   const bool ok = i < cnt && idx >= 0 && idx <= t && idx * kBlk <= t;
   if (!ok) {
     if (FILL) ws.slotmap[id] = -1;
@@ -136,10 +137,11 @@ slc_bucket_lds_kernel(const SlcArgs a, SlcWs ws) {
     id = th * a.top_n + i;
     const int b = seq_of_token(a.cu_seq, a.batch, tg);
     const int t = tg - a.cu_seq[b];
+    const long th_r = (long)tg * (a.hkv / a.kv_rep) + h / a.kv_rep;    // picks and counts are per real kv head
     int cnt = a.top_n;
-    if (a.counts != nullptr) cnt = min(max(a.counts[th], 0), a.top_n);
-    const long idx = a.idx64 ? reinterpret_cast<const int64_t*>(a.indices)[id]
-                             : (long)reinterpret_cast<const int32_t*>(a.indices)[id];
+    if (a.counts != nullptr) cnt = min(max(a.counts[th_r], 0), a.top_n);
+    const long idx = a.idx64 ? reinterpret_cast<const int64_t*>(a.indices)[th_r * a.top_n + i]
+                             : (long)reinterpret_cast<const int32_t*>(a.indices)[th_r * a.top_n + i];
     const bool ok = i < cnt && idx >= 0 && idx <= t && idx * kBlk <= t;
     return ok ? ws.blkbase[b] + (int)idx : -1;
   };
@@ -232,15 +234,16 @@ slc_block_kernel(const SlcArgs a, const SlcWs ws) {
   // K block as A fragments: chunk c (32 keys) = tiles 2c, 2c+1 with permuted rows; V^T block per chunk
   vec8_t<T> kf[4][NK], vf[2][NV];
   {
-    const T* kb = reinterpret_cast<const T*>(a.k) + ((long)st.start * a.hkv + h) * DK + 8 * g;
-    const long krow = (long)a.hkv * DK;
+    const int hk = h / a.kv_rep, hkv_r = a.hkv / a.kv_rep;     // kv head of this (sub-)group, number of kv heads
+    const T* kb = reinterpret_cast<const T*>(a.k) + ((long)st.start * hkv_r + hk) * DK + 8 * g;
+    const long krow = (long)hkv_r * DK;
 #pragma unroll
     for (int tile = 0; tile < 4; ++tile) {
       const int row = min(st.t0 + 32 * (tile >> 1) + chunk_key_of_row(tile & 1, n), st.len - 1);
 #pragma unroll
       for (int kk = 0; kk < NK; ++kk) kf[tile][kk] = load8(kb + row * krow + 32 * kk);
     }
-    const T* vtb = reinterpret_cast<const T*>(a.vt) + (long)h * DV * a.vt_cols + transposed_offset(st.start, st.b) +
+    const T* vtb = reinterpret_cast<const T*>(a.vt) + (long)hk * DV * a.vt_cols + transposed_offset(st.start, st.b) +
                    (long)n * a.vt_cols + st.t0 + 8 * g;
 #pragma unroll
     for (int c = 0; c < 2; ++c)

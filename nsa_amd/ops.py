@@ -52,6 +52,14 @@ def pool_bins(nc: int, kernel: int, stride: int, pad: int) -> int:
     return ns
 
 
+def head_subgroups(hq: int, hkv: int) -> int:
+    """Sub-groups of 16 query heads per kv head: 1 for GQA groups up to 16; groups of 32, 48, 64, ... heads (the
+    reference's HQ % (16 * H) == 0, nsa/selection_attn.py:800) run as G / 16 sub-groups that share the keys,
+    values and block picks of their kv head."""
+    g = hq // hkv
+    return g // 16 if g > 16 and g % 16 == 0 else 1
+
+
 def transposed_cols(total_rows: int, batch: int) -> int:
     return _lib.load().nsa_transposed_cols(total_rows, batch)
 
@@ -127,8 +135,9 @@ def cmp_attn_select(q, ck, cvt, cu_seqlens, cu_cmp, batch, hkv, dv, ck_row_strid
     lse = torch.empty(total, hq, dtype=torch.float32, device=q.device)
     if select:
         idx = torch.empty(total, hkv, top_n, dtype=torch.int64 if idx64 else torch.int32, device=q.device)
-        # always given: with it the library runs its two-kernel schedule (window sums, then top-n)
-        pooled = torch.empty(total, hkv, max(max_ns, 1), dtype=torch.float32, device=q.device)
+        # always given: with it the library runs its two-kernel schedule (window sums, then top-n); one row per
+        # sub-group of 16 heads, the block scores end up in the first row of every kv head
+        pooled = torch.empty(total, hkv, head_subgroups(hq, hkv), max(max_ns, 1), dtype=torch.float32, device=q.device)
     lib = _lib.load()
     rc = lib.nsa_cmp_attn_select_fwd(
         _ptr(q), _ptr(ck), _ptr(cvt), _ptr(o), _ptr(idx), _ptr(pooled), _ptr(lse), _ptr(cu_seqlens), _ptr(cu_cmp),
@@ -137,7 +146,7 @@ def cmp_attn_select(q, ck, cvt, cu_seqlens, cu_cmp, batch, hkv, dv, ck_row_strid
         pool_stride, pool_pad, max(top_n, 1), max_ns, max(max_ns, 1), float(scale), int(bool(causal)),
         int(idx64), _dtype_code(q), _stream())
     _lib.check(rc, "nsa_cmp_attn_select_fwd")
-    return o, idx, (pooled if want_pooled else None)
+    return o, idx, (pooled[:, :, 0] if want_pooled else None)
 
 
 def cmp_attn(q, ck, cvt, cu_seqlens, cu_cmp, batch, hkv, dv, ck_row_stride, ck_head_stride, block, stride, scale,
@@ -167,14 +176,15 @@ def block_select(q, ck, lse, cu_seqlens, cu_cmp, batch, hkv, ck_row_stride, ck_h
     total, hq, dk = q.shape
     max_ns = pool_bins(max_nc, pool_kernel, pool_stride, pool_pad)
     idx = torch.empty(total, hkv, top_n, dtype=torch.int64 if idx64 else torch.int32, device=q.device)
-    # always given: with it the library runs its two-kernel schedule (window sums, then top-n)
-    pooled = torch.empty(total, hkv, max(max_ns, 1), dtype=torch.float32, device=q.device)
+    # always given: with it the library runs its two-kernel schedule (window sums, then top-n); one row per
+    # sub-group of 16 heads, the block scores end up in the first row of every kv head
+    pooled = torch.empty(total, hkv, head_subgroups(hq, hkv), max(max_ns, 1), dtype=torch.float32, device=q.device)
     rc = _lib.load().nsa_block_select_fwd(_ptr(q), _ptr(ck), _ptr(lse), _ptr(idx), _ptr(pooled), _ptr(cu_seqlens),
                                           _ptr(cu_cmp), batch, total, hq, hkv, dk, ck_row_stride, ck_head_stride,
                                           pool_kernel, pool_stride, pool_pad, top_n, max_ns, max(max_ns, 1),
                                           int(idx64), _dtype_code(q), _stream())
     _lib.check(rc, "nsa_block_select_fwd")
-    return idx, (pooled if want_pooled else None)
+    return idx, (pooled[:, :, 0] if want_pooled else None)
 
 
 def swa(q, k, vt, cu_seqlens, batch, window, scale, want_lse=False):
@@ -232,7 +242,8 @@ def slc_combine(q, k, vt, indices, counts, g_slc, g_swa, g_cmp, o_swa, o_cmp, cu
     lib = _lib.load()
     ws, ws_bytes = None, 0
     if block_major is not False:
-        need = lib.nsa_slc_workspace_bytes(total, batch, hkv, dk, dv, top_n, block_size, _dtype_code(q))
+        need = lib.nsa_slc_workspace_bytes(total, batch, hkv * head_subgroups(hq, hkv), dk, dv, top_n, block_size,
+                                           _dtype_code(q))
         if need > 0 and (block_major or need <= SLC_WORKSPACE_LIMIT):
             ws = torch.empty(need, dtype=torch.uint8, device=q.device)
             ws_bytes = need
@@ -250,7 +261,8 @@ def slc_combine(q, k, vt, indices, counts, g_slc, g_swa, g_cmp, o_swa, o_cmp, cu
 def slc_workspace(q, hkv, dv, top_n, block_size, batch):
     """Workspace tensor of the block-major selected attention, or None when the shape has none."""
     total, hq, dk = q.shape
-    need = _lib.load().nsa_slc_workspace_bytes(total, batch, hkv, dk, dv, top_n, block_size, _dtype_code(q))
+    need = _lib.load().nsa_slc_workspace_bytes(total, batch, hkv * head_subgroups(hq, hkv), dk, dv, top_n, block_size,
+                                               _dtype_code(q))
     if need <= 0 or need > SLC_WORKSPACE_LIMIT:
         return None
     return torch.empty(need, dtype=torch.uint8, device=q.device)

@@ -154,6 +154,15 @@ def test_cmp_select_block64_padded_pool():
     _cmp_case(torch.bfloat16, [1024, 333], 16, 1, 64, 64, 64, 16, 64, 4, seed=30)
 
 
+def test_cmp_select_groups_of_32_48_64_heads():
+    """GQA groups the reference's selected attention takes (HQ a multiple of 16 * H, nsa/selection_attn.py:800):
+    sub-groups of 16 heads share the compressed keys; the block scores are the sum over all heads of the group."""
+    _cmp_case(torch.bfloat16, [1500, 200], 64, 2, 128, 128, 32, 16, 64, 16, seed=43, scale_in=0.5)    # G=32
+    _cmp_case(torch.bfloat16, [1024], 48, 1, 64, 64, 32, 16, 64, 4, seed=44, scale_in=0.5)            # G=48
+    _cmp_case(torch.float32, [700], 64, 1, 64, 64, 32, 16, 64, 8, seed=45, scale_in=0.5)              # G=64, fp32
+    _cmp_case(torch.bfloat16, [2048], 64, 2, 192, 128, 32, 16, 64, 16, seed=46, scale_in=0.5)         # G=32, Dqk 192
+
+
 def test_cmp_select_odd_groups():
     _cmp_case(torch.float32, [500], 6, 2, 64, 64, 32, 16, 64, 2, seed=40)      # G=3 -> padded to 4
     _cmp_case(torch.float32, [500], 8, 1, 32, 32, 32, 16, 64, 2, seed=41)      # G=8
@@ -164,7 +173,8 @@ def test_cmp_select_odd_groups():
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("lens,Hq,Hkv,Dk,Dv,W", [([1024], 4, 1, 64, 64, 128), ([777, 40, 513], 32, 2, 128, 128, 512),
                                                  ([600], 16, 1, 192, 128, 100), ([130], 8, 2, 32, 32, 1),
-                                                 ([300], 6, 2, 64, 64, 1000)])
+                                                 ([300], 6, 2, 64, 64, 1000), ([500, 77], 64, 2, 128, 128, 128),
+                                                 ([300], 48, 1, 64, 64, 64)])
 def test_swa(dtype, lens, Hq, Hkv, Dk, Dv, W):
     ops = _ops()
     T = sum(lens)
@@ -199,7 +209,8 @@ def _random_indices(T, Hkv, S, bs, seed, poison=True):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("lens,Hq,Hkv,Dk,Dv,S,bs", [([256], 16, 1, 32, 32, 2, 32), ([512, 100], 32, 2, 128, 128, 8, 64),
                                                    ([384], 4, 1, 64, 64, 4, 64), ([200], 16, 1, 192, 128, 3, 64),
-                                                   ([160], 6, 2, 64, 64, 3, 16)])
+                                                   ([160], 6, 2, 64, 64, 3, 16), ([512, 100], 64, 2, 128, 128, 8, 64),
+                                                   ([300], 48, 1, 64, 64, 3, 32)])
 def test_slc_only(dtype, lens, Hq, Hkv, Dk, Dv, S, bs):
     ops = _ops()
     T = sum(lens)
@@ -230,7 +241,8 @@ def test_slc_only(dtype, lens, Hq, Hkv, Dk, Dv, S, bs):
 
 
 @pytest.mark.parametrize("lens,Hq,Hkv,Dk,Dv,S,W", [([512, 100], 32, 2, 128, 128, 8, 128), ([200], 16, 1, 192, 128, 3, 64),
-                                                  ([384], 4, 1, 64, 64, 4, 512), ([700, 330], 24, 2, 64, 64, 16, 256)])
+                                                  ([384], 4, 1, 64, 64, 4, 512), ([700, 330], 24, 2, 64, 64, 16, 256),
+                                                  ([700, 330], 64, 2, 128, 128, 16, 256), ([400], 48, 1, 192, 128, 4, 64)])
 def test_fused_partials_and_window_merge(lens, Hq, Hkv, Dk, Dv, S, W):
     """nsa_slc_partials_fwd + nsa_swa_merge_fwd against nsa_swa_fwd + nsa_slc_combine_fwd (token-major
     kernel) and against the oracle, with counts, invalid picks, gates and a compressed-branch input."""
@@ -268,7 +280,8 @@ def test_fused_partials_and_window_merge(lens, Hq, Hkv, Dk, Dv, S, W):
             err = max(err, max_abs(fused[s:e], ref))
         d = max_abs(fused, split)
         print("fused", lens, (Hq, Hkv, Dk, Dv, S, W), "counts", use_counts, "vs oracle", err, "vs split kernels", d)
-        assert err <= TOL[dtype] and d <= TOL[dtype]
+        # two kernels that each round once to bf16: where |out| > 4 they may differ by one unit in the last place
+        assert err <= TOL[dtype] and within(fused, split, dtype, large_values=True), (err, d)
         # the same launch can also leave what a backward pass keeps: the ungated branch outputs and their
         # log-sum-exps, equal to those of the stand-alone kernels
         out2, b_slc, b_swa, l_slc, l_swa = ops.swa_merge(qd, kd, vt, ws, S, g_slc, g_swa, g_cmp, o_cmp.to(DEV), cu,
@@ -321,14 +334,15 @@ def test_parallel_nsa_api_like_reference_test(dtype):
     assert max_abs(out_hf[0].transpose(0, 1), slc + swa) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("H", [2, 1])          # GQA groups of 16 and of 32 heads
 @pytest.mark.parametrize("dtype,bs,W", [(torch.bfloat16, 64, 128), (torch.bfloat16, 32, 48), (torch.float32, 32, 16)])
-def test_parallel_nsa_packed_cu_seqlens_and_tensor_counts(dtype, bs, W):
+def test_parallel_nsa_packed_cu_seqlens_and_tensor_counts(dtype, bs, W, H):
     """The public call in its varlen form (nsa/selection_attn.py:792-793: B == 1, packed [1,total,...]
     tensors, block ids local to each sequence) with a per-(token, head) count tensor (:431-434), random
     gates; every sequence against the per-token loop oracle."""
     import nsa_amd
     lens = [200, 64, 1, 333, 97]
-    T, H, HQ, D, S = sum(lens), 2, 32, 64, 3
+    T, HQ, D, S = sum(lens), 32, 64, 3
     q = randn(1, T, HQ, D, seed=90, scale=0.7, dtype=dtype)
     k = randn(1, T, H, D, seed=91, scale=0.7, dtype=dtype)
     v = randn(1, T, H, D, seed=92, dtype=dtype)
@@ -439,6 +453,14 @@ def test_module_cfg4_shape_reduced_dqk192():
 
 def test_module_varlen_ragged():
     _module_case(torch.bfloat16, [1100, 64, 1000, 33, 1536], 32, 2, 128, 128, 16, 512, seed=2, scale_in=0.5)
+
+
+def test_module_groups_of_32_and_64_heads():
+    """Hq 64 / Hkv 2 (what the reference's HQ % (16 * H) == 0 allows and a group limit of 16 refuses), ragged;
+    Hq 64 / Hkv 1 with the reference's learned compressor and raw gates."""
+    _module_case(torch.bfloat16, [1100, 64, 1000, 33, 1536], 64, 2, 128, 128, 16, 512, seed=7, scale_in=0.5)
+    _module_case(torch.bfloat16, [2048], 64, 1, 128, 128, 16, 512, seed=8, scale_in=0.7, mode="conv", act=None)
+    _module_case(torch.bfloat16, [1024], 96, 2, 192, 128, 8, 128, seed=9, scale_in=0.5)                # G=48, Dqk 192
 
 
 def test_module_reference_defaults_conv_raw_gates():

@@ -68,8 +68,20 @@ def test_argument_errors_do_not_launch(lib):
     assert rc == -1 and b"null" in lib.nsa_last_error_string()
     buf = ctypes.create_string_buffer(4096)
     p = ctypes.c_void_p((ctypes.addressof(buf) + 15) & ~15)
-    rc = lib.nsa_swa_fwd(p, p, p, p, None, p, 1, 64, 64, 2, 64, 64, 128, 16, 0.1, 0, None)
+    rc = lib.nsa_swa_fwd(p, p, p, p, None, p, 1, 64, 48, 2, 64, 64, 128, 16, 0.1, 0, None)      # GQA group of 24
     assert rc == -2 and b"group size" in lib.nsa_last_error_string()
+    rc = lib.nsa_decode_step(p, p, p, p, p, p, None, p, None, 1, 64, 2, 64, 64, 64, 64, 32, 16, 64, 5, 4, 0, 4, 16, 0.1,
+                             0, 0, None)                                                             # group of 32: prefill only
+    assert rc == -2 and b"group size" in lib.nsa_last_error_string()
+    rc = lib.nsa_decode_step(p, p, p, p, p, p, None, p, None, 1, 4, 1, 64, 64, 4096, 256, 32, 16, 32, 3, 2, 0, 4, 16,
+                             0.1, 0, 0, None)                                                        # 128 bins > 68
+    assert rc == -2 and b"pooled bins" in lib.nsa_last_error_string()
+    rc = lib.nsa_decode_step(p, p, p, p, p, p, None, p, None, 1, 4, 1, 64, 64, 65536, 4096, 32, 16, 64, 5, 4, 0, 4, 16,
+                             0.1, 0, 0, None)                                                        # one workgroup: 2304 rows
+    assert rc == -2 and b"nsa_decode_step_split" in lib.nsa_last_error_string()
+    rc = lib.nsa_decode_step_split_static(p, p, p, None, 0, p, p, p, None, p, None, 160, 64, 4, 128, 128, 32768, 2048, 32,
+                                          16, 64, 5, 4, 0, 16, 512, 0.1, 0, 0, 8, None)
+    assert rc == -3 and b"fixed array" in lib.nsa_last_error_string()
     rc = lib.nsa_swa_fwd(p, p, p, p, None, p, 1, 64, 4, 1, 48, 64, 128, 16, 0.1, 0, None)
     assert rc == -2
     rc = lib.nsa_swa_fwd(p, p, p, p, None, p, 1, 64, 4, 1, 64, 64, 128, 16, 0.1, 7, None)
