@@ -8,18 +8,22 @@
 // written to the other buffer afterwards, one barrier per chunk.  Every wavefront reads each K/V
 // fragment from LDS once and feeds it to NG MFMAs (register blocking over row groups).
 //
-// Softmax bookkeeping per row: one running maximum of the raw scores.  In the compressed branch it
-// runs over ALL compressed rows (the importance softmax is not causal) and serves both sums:
-//   li += exp(s - M)                         every row      -> lse = M + log(li)
+// Softmax bookkeeping of the compressed branch: two sums per row off one score tile,
+//   li += exp(s - M)                         every row      -> lse = M + log(li)   (importance softmax, not causal)
 //   l  += exp(scale*(s - M)), O += p V       visible rows   -> o = O / l
-// so each score tile costs one maximum reduction.  exp(scale*(s - M)) stays exact unless the
-// visible scores sit more than ~87/scale below the largest hidden one.
+// In the common pass M is fixed after the first 32 rows (no maximum, no rescale, no branch per chunk); a row
+// whose sums leave the safe range sends its workgroup through an exact second pass with a running maximum per
+// softmax (the attention one over the visible rows only), so neither a large hidden score nor a late large
+// score can cost a visible one its precision.
 //
 // The selected-block branch (one wavefront per row group, blocks read straight from global memory
 // in fragment layout) and the gated combine of the three branches live here as well.
+#include <type_traits>
+
 #include "slc_merge.h"
 
 namespace nsa {
+
 
 struct StreamParams {
   const void* q; const void* k; const void* vt; void* o; float* lse;
@@ -32,6 +36,8 @@ struct StreamParams {
   float* lse_attn;   // optional: log-sum-exp (natural log) of the scaled visible scores, for the backward
   int kv_rep;        // sub-groups of 16 query heads per kv head (1 unless the GQA group exceeds 16): hkv counts
                      // sub-groups, and sub-group h reads the keys / values of kv head h / kv_rep
+  int split_hidden;  // compressed branch: stop at cmp_visible_end(): the rows beyond carry no attention, they only feed
+                     // the importance log-sum-exp, which this caller did not ask for
 };
 
 // MERGE (sliding window only): 0 = write the branch output; otherwise the epilogue merges the
@@ -84,7 +90,8 @@ stream_attn_kernel(const StreamParams a) {
   RowMap rm[NG];
   int hi[NG], lo[NG];            // per lane: visible keys are lo..hi
   int g_hi_max[NG], g_hi_min[NG], g_lo_min[NG], g_lo_max[NG];   // wave uniform bounds over the group
-  float li[NG];
+  float li[NG];                  // compressed branch: this lane's share of the importance denominator ...
+  float mi[NG];                  // ... and its reference (the attention softmax keeps its own in grp[j].m)
 #pragma unroll
   for (int j = 0; j < NG; ++j) {
     const int gi = wave * NG + j;
@@ -92,6 +99,7 @@ stream_attn_kernel(const StreamParams a) {
     load_q(grp[j], reinterpret_cast<const T*>(a.q), (long)st.start, rm[j], st.len, a.hq, h, G, g);
     group_reset(grp[j]);
     li[j] = 0.f;
+    mi[j] = kNegInf;
     hi[j] = last_visible(rm[j].tok);
     lo[j] = CMP ? 0 : rm[j].tok - W + 1;
     const int tf = st.t0 + ((gi * 16) >> lgp);
@@ -102,13 +110,10 @@ stream_attn_kernel(const StreamParams a) {
     g_lo_max[j] = CMP ? 0 : tl - W + 1;
   }
   const float c_attn = a.scale * kLog2e;
-  // CMP runs two softmaxes off one reference (raw scores for the importance statistics, scaled ones
-  // for the attention): the slack, in raw score units, bounds the faster growing exponential
-  const float cmp_slack = kMaxSlackLog2 / fmaxf(kLog2e, c_attn);
-  const float cmp_probe = fast_exp2(cmp_slack * kLog2e);          // exp of the slack in raw-score units
   const int attn_end = last_visible(t_last);                      // last key any row of the tile attends
   const int c_begin = CMP ? 0 : (max(st.t0 - W + 1, 0) / CH) * CH;
-  const int c_end = CMP ? nkeys : t_last + 1;
+  const int c_end = CMP ? (a.split_hidden ? cmp_visible_end(st.t0, TQ, st.len, nkeys, a.block, a.stride, a.causal) : nkeys)
+                        : t_last + 1;
 
   // Per-thread element offsets of its staging pieces for chunk 0; a chunk adds one scalar.  Only the
   // last chunk of a sequence needs the row clamp.
@@ -176,150 +181,188 @@ stream_attn_kernel(const StreamParams a) {
   };
 
   wait_all_loads();
-  if (c_begin < c_end) {
-    const bool v0 = c_begin <= attn_end;
-    gload(c_begin, v0);
-    lstore(0, v0);
-  }
-  __syncthreads();
-  int buf = 0;
-  for (int c0 = c_begin; c0 < c_end; c0 += CH) {
-    const int cn = c0 + CH;
-    const bool has_next = cn < c_end;
-    const bool next_v = has_next && cn <= attn_end;
-    if (has_next) gload(cn, next_v);
+  // One pass over the key chunks.  FAST (compressed branch only): both softmaxes of a row run against one
+  // FIXED reference, the largest raw score of the first 32 compressed rows, so a chunk costs neither a
+  // maximum nor a branch; scores above the reference simply give exponentials above 1 (fp32 sums and bf16
+  // probabilities keep their relative precision at any magnitude).  What a fixed reference cannot rule out --
+  // a sum that overflows, or visible scores so far below the reference that their sum underflows -- is
+  // checked once per row after the pass, and a workgroup that finds such a row runs the pass again in the
+  // exact form (FAST = false): a running maximum per softmax, the importance one over all rows, the
+  // attention one over the visible rows only.
+  auto run_chunks = [&](auto fast_tag) {
+    constexpr bool FAST = decltype(fast_tag)::value;
+    if (c_begin < c_end) {
+      const bool v0 = c_begin <= attn_end;
+      gload(c_begin, v0);
+      lstore(0, v0);
+    }
+    __syncthreads();
+    int buf = 0;
+    for (int c0 = c_begin; c0 < c_end; c0 += CH) {
+      const int cn = c0 + CH;
+      const bool has_next = cn < c_end;
+      const bool next_v = has_next && cn <= attn_end;
+      if (has_next) gload(cn, next_v);
 
-    const T* bk = ldsK + buf * CH * KLD;
-    const T* bv = ldsV + buf * DV * VLD;
+      const T* bk = ldsK + buf * CH * KLD;
+      const T* bv = ldsV + buf * DV * VLD;
 #pragma unroll
-    for (int sub = 0; sub < CH / 32; ++sub) {
-      const int cb = c0 + 32 * sub;
-      if (cb >= c_end) break;
-      const bool first_sub = CMP && cb == c_begin;
-      bool act[NG];
-      bool any_act = false;
+      for (int sub = 0; sub < CH / 32; ++sub) {
+        const int cb = c0 + 32 * sub;
+        if (cb >= c_end) break;
+        bool act[NG];
+        bool any_act = false;
+#pragma unroll
+        for (int j = 0; j < NG; ++j) {
+          act[j] = cb <= g_hi_max[j] && (CMP || cb + 31 >= g_lo_min[j]);
+          any_act |= act[j];
+        }
+        if (!CMP && !any_act) continue;
+        f32x4_t s0[NG], s1[NG];
+        const T* ks = bk + 32 * sub * KLD + 8 * g;
+        scores32<T, DK, DV, NG>(ks + lds_key_of_row(0, n) * KLD, ks + lds_key_of_row(1, n) * KLD, grp, s0, s1);
+        const int swp = lds_key_swap(g);       // value i of this lane belongs to key cb + 8g + (i ^ swp)
+        vec8_t<T> pb[NG];
+        if constexpr (CMP) {
+          float s[NG][8];
+#pragma unroll
+          for (int j = 0; j < NG; ++j) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { s[j][i] = s0[j][i]; s[j][4 + i] = s1[j][i]; }
+          }
+          const int key0 = cb + 8 * g;
+          if (cb + 32 > nkeys) {                         // last chunk of the sequence only
+            asm volatile("" ::: "memory");
+#pragma unroll
+            for (int j = 0; j < NG; ++j)
+#pragma unroll
+              for (int i = 0; i < 8; ++i)
+                if (key0 + (i ^ swp) >= nkeys) s[j][i] = kNegInf;
+          }
+          if constexpr (FAST) {
+            if (cb == c_begin) {                         // the reference: largest score of the first 32 rows
+#pragma unroll
+              for (int j = 0; j < NG; ++j) {
+                float mx = s[j][0];
+#pragma unroll
+                for (int i = 1; i < 8; ++i) mx = fmaxf(mx, s[j][i]);
+                mi[j] = colgroup_max(mx);                // finite: key cb exists
+                grp[j].m = mi[j];
+              }
+            }
+#pragma unroll
+            for (int j = 0; j < NG; ++j) {
+              const float off_i = -mi[j] * kLog2e;
+              float ei[8];
+#pragma unroll
+              for (int i = 0; i < 8; ++i) ei[i] = fast_exp2(fmaf(s[j][i], kLog2e, off_i));
+              li[j] += sum8(ei);
+              if (act[j]) {
+                const float off_a = -mi[j] * c_attn;
+                const bool full = cb + 31 <= g_hi_min[j];
+                float p[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) p[i] = fast_exp2(fmaf(s[j][i], c_attn, off_a));
+                if (!full) {                             // the one or two chunks on the causal edge
+                  asm volatile("" ::: "memory");
+#pragma unroll
+                  for (int i = 0; i < 8; ++i)
+                    if (key0 + (i ^ swp) > hi[j]) p[i] = 0.f;
+                }
+                grp[j].l += sum8(p);
+                pb[j] = pack8<T>(p);
+              } else {
+                pb[j] = zero8<T>();
+              }
+            }
+          } else {
+#pragma unroll
+            for (int j = 0; j < NG; ++j) {
+              float mx = s[j][0];
+#pragma unroll
+              for (int i = 1; i < 8; ++i) mx = fmaxf(mx, s[j][i]);
+              mx = colgroup_max(mx);                     // finite: key cb exists
+              const float m_new = fmaxf(mi[j], mx);
+              const float off_i = -m_new * kLog2e;
+              float ei[8];
+#pragma unroll
+              for (int i = 0; i < 8; ++i) ei[i] = fast_exp2(fmaf(s[j][i], kLog2e, off_i));
+              li[j] = li[j] * fast_exp2((mi[j] - m_new) * kLog2e) + sum8(ei);     // exp2(-inf) = 0 on the first chunk
+              mi[j] = m_new;
+              if (act[j]) {
+                float sv[8], p[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) sv[i] = key0 + (i ^ swp) > hi[j] ? kNegInf : s[j][i];
+                softmax_update(grp[j], sv, c_attn, p);   // running maximum of the visible scores only
+                pb[j] = pack8<T>(p);
+              } else {
+                pb[j] = zero8<T>();
+              }
+            }
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < NG; ++j) {
+            float s[8], p[8];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { s[i] = s0[j][i]; s[4 + i] = s1[j][i]; }
+            const int key0 = cb + 8 * g;
+            const bool full = cb + 31 <= g_hi_min[j] && cb >= g_lo_max[j];
+            if (act[j]) {
+              if (!full) {                               // window edges
+                asm volatile("" ::: "memory");
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                  if (!(key0 + (i ^ swp) <= hi[j] && key0 + (i ^ swp) >= lo[j])) s[i] = kNegInf;
+              }
+              softmax_update(grp[j], s, c_attn, p);
+              pb[j] = pack8<T>(p);
+            } else {
+              pb[j] = zero8<T>();
+            }
+          }
+        }
+        // a group without visible keys in this chunk carries all-zero probabilities: one MFMA chain
+        // for all groups keeps the accumulators in place (no per-group control flow around them)
+        if (any_act) pv32_all<T, DK, DV, NG>(bv + n * VLD + 32 * sub + 8 * g, 16 * VLD, grp, pb);
+      }
+
+      if (has_next) lstore(buf ^ 1, next_v);
+      __syncthreads();
+      buf ^= 1;
+    }
+  };
+
+  float lt[NG], lit[NG];                       // denominators summed over the four lanes of a column
+  auto row_sums = [&]() {
+#pragma unroll
+    for (int j = 0; j < NG; ++j) {
+      lt[j] = colgroup_sum(grp[j].l);
+      lit[j] = CMP ? colgroup_sum(li[j]) : 0.f;
+    }
+  };
+  if constexpr (CMP) {
+    run_chunks(std::true_type{});
+    row_sums();
+    int bad = 0;
+#pragma unroll
+    for (int j = 0; j < NG; ++j) {
+      const bool sees = rm[j].valid && hi[j] >= 0 && c_begin < c_end;
+      bad |= !(lit[j] < 1e30f) || !(lt[j] < 1e30f) || (sees && !(lt[j] > 1e-30f));
+    }
+    if (__syncthreads_or(bad)) {               // rare: the whole workgroup repeats the pass in the exact form
 #pragma unroll
       for (int j = 0; j < NG; ++j) {
-        act[j] = cb <= g_hi_max[j] && (CMP || cb + 31 >= g_lo_min[j]);
-        any_act |= act[j];
+        group_reset(grp[j]);
+        li[j] = 0.f;
+        mi[j] = kNegInf;
       }
-      if (!CMP && !any_act) continue;
-      f32x4_t s0[NG], s1[NG];
-      const T* ks = bk + 32 * sub * KLD + 8 * g;
-      scores32<T, DK, DV, NG>(ks + lds_key_of_row(0, n) * KLD, ks + lds_key_of_row(1, n) * KLD, grp, s0, s1);
-      const int swp = lds_key_swap(g);       // value i of this lane belongs to key cb + 8g + (i ^ swp)
-      vec8_t<T> pb[NG];
-      if constexpr (CMP) {
-        // Scores of all groups first, so that the probe below is one branch per sub-chunk and the
-        // exponentials of the groups are independent straight-line work.
-        float s[NG][8], si[NG];
-#pragma unroll
-        for (int j = 0; j < NG; ++j) {
-#pragma unroll
-          for (int i = 0; i < 4; ++i) { s[j][i] = s0[j][i]; s[j][4 + i] = s1[j][i]; }
-        }
-        const int key0 = cb + 8 * g;
-        if (cb + 32 > nkeys) {                         // last chunk of the sequence only
-          asm volatile("" ::: "memory");
-#pragma unroll
-          for (int j = 0; j < NG; ++j)
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-              if (key0 + (i ^ swp) >= nkeys) s[j][i] = kNegInf;
-        }
-        // The raw-score exponentials are needed anyway (importance log-sum-exp), so they double as the
-        // overflow probe: a score more than the slack above the reference makes its exponential, and
-        // with it the lane's sum of 8, exceed 2^slack.  Only then (and on the very first chunk, while
-        // the reference is still -inf) is the maximum taken and the reference moved; the common case
-        // pays neither the 8-way maximum nor its reduction over the column's four lanes.
-        bool redo = first_sub;
-        if (!first_sub) {
-          bool over = false;
-#pragma unroll
-          for (int j = 0; j < NG; ++j) {
-            const float off_i = -grp[j].m * kLog2e;
-            float ei[8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) ei[i] = fast_exp2(fmaf(s[j][i], kLog2e, off_i));
-            si[j] = sum8(ei);
-            over |= si[j] > cmp_probe;
-          }
-          redo = __any(over);
-        }
-        if (redo) {
-#pragma unroll
-          for (int j = 0; j < NG; ++j) {
-            float mx = s[j][0];
-#pragma unroll
-            for (int i = 1; i < 8; ++i) mx = fmaxf(mx, s[j][i]);
-            mx = colgroup_max(mx);                     // finite: key cb exists
-            const float m_new = fmaxf(grp[j].m, mx);
-            const float d = grp[j].m - m_new;          // -inf on the first chunk, 0 when nothing moved
-            float beta = fast_exp2(d * kLog2e), alpha = fast_exp2(d * c_attn);
-            settle_factor(beta, alpha);
-            scale_inplace(li[j], beta);
-            scale_inplace(grp[j].l, alpha);
-#pragma unroll
-            for (int t = 0; t < DV / 16; ++t) scale_inplace(grp[j].o[t], alpha);
-            grp[j].m = m_new;
-            const float off_i = -m_new * kLog2e;
-            float ei[8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) ei[i] = fast_exp2(fmaf(s[j][i], kLog2e, off_i));
-            si[j] = sum8(ei);
-          }
-        }
-#pragma unroll
-        for (int j = 0; j < NG; ++j) {
-          li[j] += si[j];
-          if (act[j]) {
-            const float off_a = -grp[j].m * c_attn;
-            const bool full = cb + 31 <= g_hi_min[j];
-            float p[8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) p[i] = fast_exp2(fmaf(s[j][i], c_attn, off_a));
-            if (!full) {                               // the one or two chunks on the causal edge
-              asm volatile("" ::: "memory");
-#pragma unroll
-              for (int i = 0; i < 8; ++i)
-                if (key0 + (i ^ swp) > hi[j]) p[i] = 0.f;
-            }
-            grp[j].l += sum8(p);
-            pb[j] = pack8<T>(p);
-          } else {
-            pb[j] = zero8<T>();
-          }
-        }
-      } else {
-#pragma unroll
-        for (int j = 0; j < NG; ++j) {
-          float s[8], p[8];
-#pragma unroll
-          for (int i = 0; i < 4; ++i) { s[i] = s0[j][i]; s[4 + i] = s1[j][i]; }
-          const int key0 = cb + 8 * g;
-          const bool full = cb + 31 <= g_hi_min[j] && cb >= g_lo_max[j];
-          if (act[j]) {
-            if (!full) {                               // window edges
-              asm volatile("" ::: "memory");
-#pragma unroll
-              for (int i = 0; i < 8; ++i)
-                if (!(key0 + (i ^ swp) <= hi[j] && key0 + (i ^ swp) >= lo[j])) s[i] = kNegInf;
-            }
-            softmax_update(grp[j], s, c_attn, p);
-            pb[j] = pack8<T>(p);
-          } else {
-            pb[j] = zero8<T>();
-          }
-        }
-      }
-      // a group without visible keys in this chunk carries all-zero probabilities: one MFMA chain
-      // for all groups keeps the accumulators in place (no per-group control flow around them)
-      if (any_act) pv32_all<T, DK, DV, NG>(bv + n * VLD + 32 * sub + 8 * g, 16 * VLD, grp, pb);
+      run_chunks(std::false_type{});
+      row_sums();
     }
-
-    if (has_next) lstore(buf ^ 1, next_v);
-    __syncthreads();
-    buf ^= 1;
+  } else {
+    run_chunks(std::false_type{});
+    row_sums();
   }
 
   // Output rows leave through LDS (the K buffers are free after the loop's last barrier): the
@@ -331,8 +374,7 @@ stream_attn_kernel(const StreamParams a) {
   T* stage = ldsK + wave * 16 * OLD;
 #pragma unroll
   for (int j = 0; j < NG; ++j) {
-    const float lt = colgroup_sum(grp[j].l);
-    const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+    const float inv = lt[j] > 0.f ? 1.0f / lt[j] : 0.f;
     const long row = ((long)st.start + rm[j].tok) * a.hq + h * G + rm[j].gidx;
     store_rows<T, DV>(stage + n * OLD, grp[j].o, inv, g);
     constexpr int PIECES = DV / 8;
@@ -379,10 +421,9 @@ stream_attn_kernel(const StreamParams a) {
       }
     }
     if (a.lse_attn != nullptr && rm[j].valid && g == 0)
-      a.lse_attn[row] = lt > 0.f ? fmaf(grp[j].m, a.scale, __logf(lt)) : __builtin_huge_valf();
+      a.lse_attn[row] = lt[j] > 0.f ? fmaf(grp[j].m, a.scale, __logf(lt[j])) : __builtin_huge_valf();
     if (CMP && a.lse != nullptr) {
-      const float lit = colgroup_sum(li[j]);
-      if (rm[j].valid && g == 0) a.lse[row] = nkeys > 0 ? grp[j].m + __logf(lit) : 0.f;
+      if (rm[j].valid && g == 0) a.lse[row] = nkeys > 0 ? mi[j] + __logf(lit[j]) : 0.f;
     }
   }
 }
@@ -595,21 +636,24 @@ static int launch_stream_t(const StreamParams& a, int total, hipStream_t st) {
 template <typename T, int DK, int DV>
 static int launch_cmp_t(const CmpArgs& a, hipStream_t st) {
   StreamParams p{a.q, a.ck, a.cvt, a.o, a.lse, a.cu_seq, a.cu_cmp, a.batch, a.hq, a.hkv, a.ck_row_stride,
-                 a.ck_head_stride, a.cvt_cols, a.block, a.stride, 0, a.causal, a.scale, MergeArgs{}, a.lse_attn, a.kv_rep};
+                 a.ck_head_stride, a.cvt_cols, a.block, a.stride, 0, a.causal, a.scale, MergeArgs{}, a.lse_attn, a.kv_rep, 0};
+  // rows beyond the last one a tile's tokens may attend only feed the importance log-sum-exp: skipped when that
+  // is not asked for
+  if (a.causal && a.lse == nullptr) p.split_hidden = 1;
   return launch_stream_t<T, DK, DV, true>(p, a.total, st);
 }
 
 template <typename T, int DK, int DV>
 static int launch_swa_t(const SwaArgs& a, hipStream_t st) {
   StreamParams p{a.q, a.k, a.vt, a.o, nullptr, a.cu_seq, a.cu_seq, a.batch, a.hq, a.hkv, (long)(a.hkv / a.kv_rep) * DK,
-                 (long)DK, a.vt_cols, 0, 0, a.window, 1, a.scale, MergeArgs{}, a.lse, a.kv_rep};
+                 (long)DK, a.vt_cols, 0, 0, a.window, 1, a.scale, MergeArgs{}, a.lse, a.kv_rep, 0};
   return launch_stream_t<T, DK, DV, false>(p, a.total, st);
 }
 
 template <int DK, int DV>
 static int launch_swa_merge_t(const SwaArgs& a, const MergeArgs& m, hipStream_t st) {
   StreamParams p{a.q, a.k, a.vt, nullptr, nullptr, a.cu_seq, a.cu_seq, a.batch, a.hq, a.hkv, (long)(a.hkv / a.kv_rep) * DK,
-                 (long)DK, a.vt_cols, 0, 0, a.window, 1, a.scale, m, a.lse, a.kv_rep};
+                 (long)DK, a.vt_cols, 0, 0, a.window, 1, a.scale, m, a.lse, a.kv_rep, 0};
   if (m.top_n == 16) return launch_stream_t<bf16_t, DK, DV, false, 16>(p, a.total, st);
   return launch_stream_t<bf16_t, DK, DV, false, 1>(p, a.total, st);
 }

@@ -341,6 +341,16 @@ __device__ __forceinline__ void interleave_mfma_valu() {
   }
 }
 
+// Compressed rows a token tile needs when only the attention output is wanted: up to the last row its last token
+// may attend, rounded up to 64 and at least 64 (so that every row meets the first chunk, which sets its softmax
+// reference).  The rows beyond only feed the importance log-sum-exp.
+__device__ __forceinline__ int cmp_visible_end(int t0, int tq, int len, int nkeys, int block, int stride, int causal) {
+  if (!causal) return nkeys;
+  const int t_last = min(t0 + tq, len) - 1;
+  const int last = t_last >= block ? min((t_last - block) / stride, nkeys - 1) : -1;
+  return min(nkeys, max(64, ((last + 1 + 63) / 64) * 64));
+}
+
 __device__ __forceinline__ int ilog2(int x) { return 31 - __builtin_clz(x); }
 __device__ __forceinline__ int next_pow2(int x) {
   int p = 1;
