@@ -140,7 +140,11 @@ __host__ __device__ __forceinline__ int transposed_offset(int cu_b, int b) {
 }
 
 // Sequence / tile lookup for packed (varlen) inputs.  Tiles of `tq` tokens are numbered sequence
-// after sequence; a tile index past the last one yields valid = false.
+// after sequence; a tile index past the last one yields valid = false.  `tile` is the same for the
+// whole wavefront and all 64 lanes call together.  Small batches are scanned with scalar loads; from
+// 9 sequences on every lane takes one sequence of a run of 64, the run's tile counts are prefix-summed
+// across the wavefront, and the hit is broadcast: batch / 64 rounds of one coalesced load instead of
+// `batch` dependent scalar loads in every workgroup.
 struct SeqTile {
   int b, t0, start, len;
   bool valid;
@@ -149,17 +153,47 @@ __device__ __forceinline__ SeqTile find_tile(const int32_t* __restrict__ cu, int
   SeqTile r;
   r.valid = false;
   r.b = 0; r.t0 = 0; r.start = 0; r.len = 0;
-  int prev = cu[0];
-  for (int b = 0; b < batch; ++b) {
-    const int next = cu[b + 1];
-    const int len = next - prev;
+  if (batch <= 8) {
+    int prev = cu[0];
+    for (int b = 0; b < batch; ++b) {
+      const int next = cu[b + 1];
+      const int len = next - prev;
+      const int nt = (len + tq - 1) / tq;
+      if (tile < nt) {
+        r.b = b; r.t0 = tile * tq; r.start = prev; r.len = len; r.valid = true;
+        return r;
+      }
+      tile -= nt;
+      prev = next;
+    }
+    return r;
+  }
+  const int lane = __lane_id();
+  tile = __builtin_amdgcn_readfirstlane(tile);
+  int before = 0;                                    // tiles of the sequences before this run
+  for (int b0 = 0; b0 < batch; b0 += 64) {
+    const int b = b0 + lane;
+    const int s = b < batch ? cu[b] : 0;
+    const int len = b < batch ? cu[b + 1] - s : 0;
     const int nt = (len + tq - 1) / tq;
-    if (tile < nt) {
-      r.b = b; r.t0 = tile * tq; r.start = prev; r.len = len; r.valid = true;
+    int incl = nt;                                   // inclusive prefix sum over the run
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int up = __shfl_up(incl, d);
+      if (lane >= d) incl += up;
+    }
+    const int run = __builtin_amdgcn_readlane(incl, 63);
+    if (tile < before + run) {
+      const unsigned long long hit = __ballot(before + incl > tile);
+      const int w = __ffsll((long long)hit) - 1;     // first sequence whose tiles reach past `tile`
+      r.b = b0 + w;
+      r.start = __builtin_amdgcn_readlane(s, w);
+      r.len = __builtin_amdgcn_readlane(len, w);
+      r.t0 = (tile - before - __builtin_amdgcn_readlane(incl - nt, w)) * tq;
+      r.valid = true;
       return r;
     }
-    tile -= nt;
-    prev = next;
+    before += run;
   }
   return r;
 }

@@ -2,6 +2,7 @@
 with the CPU oracle on the same seeded inputs.  Bars: bf16 max-abs <= 2e-2, fp32 <= 1e-4, selected
 block sets identical except where the oracle's scores tie within 1e-3."""
 import math
+import random
 
 import pytest
 import torch
@@ -440,6 +441,8 @@ def _module_case(dtype, lens, Hq, Hkv, Dk, Dv, S, W, seed, scale_in, mode="mean"
                                           force_idx=idx[s:e], rows=rows)
         got = out[s:e] if rows is None else out[s:e][rows]
         err = max(err, max_abs(got, ref))
+        if not within(got, ref, dtype, large_values=(act is None)):
+            print("sequence", b, "of", e - s, "tokens: max-abs", max_abs(got, ref), "rows", rows)
         ok = ok and within(got, ref, dtype, large_values=(act is None))
         if parts["pooled"].shape[-1] > 0:
             r = O.compare_selection(idx[s:e] if rows is None else idx[s:e][rows], parts["idx_own"],
@@ -469,6 +472,17 @@ def test_module_cfg4_shape_reduced_dqk192():
 
 def test_module_varlen_ragged():
     _module_case(torch.bfloat16, [1100, 64, 1000, 33, 1536], 32, 2, 128, 128, 16, 512, seed=2, scale_in=0.5)
+
+
+def test_module_many_short_sequences():
+    """A serving-style batch: 150 ragged sequences (more than one 64-sequence run of the cooperative tile lookup),
+    some shorter than a compression block, one of a single token."""
+    rng = random.Random(11)
+    lens = [rng.randint(1, 200) for _ in range(150)]
+    lens[3], lens[70], lens[149] = 1, 31, 257
+    _module_case(torch.bfloat16, lens, 16, 1, 64, 64, 4, 64, seed=12, scale_in=0.5, rows_per_seq=6)
+    lens = [rng.randint(20, 400) for _ in range(20)]           # one partial run
+    _module_case(torch.bfloat16, lens, 32, 2, 128, 128, 8, 128, seed=13, scale_in=0.5, rows_per_seq=6)
 
 
 def test_module_groups_of_32_and_64_heads():

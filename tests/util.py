@@ -44,5 +44,5 @@ def sample_rows(T, n, seed, edges=(0, 1, 31, 32, 33, 63, 64, 65, 511, 512, 513))
     g = torch.Generator().manual_seed(seed)
     r = set(int(x) for x in torch.randint(0, T, (n,), generator=g))
     r.update(e for e in edges if e < T)
-    r.update((T - 1, T - 2, max(T - 65, 0)))
+    r.update((T - 1, max(T - 2, 0), max(T - 65, 0)))
     return torch.tensor(sorted(r))
