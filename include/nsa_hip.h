@@ -63,6 +63,15 @@ int nsa_compress_fwd(const void* x, const void* wt, const void* bias, void* out,
                      const int32_t* cu_seqlens, const int32_t* cu_out, int batch, int out_rows_bound,
                      int heads, int dim, int block, int stride, int dtype, nsa_stream_t stream);
 
+/* K and V of a layer in one call, as the reference's compress_kv(k, v, w_k, w_v, ...) takes them
+ * (nsa/compression_kv.py:269-289, KVCompressorVarlen.forward :291-312).  Same arguments as nsa_compress_fwd per
+ * tensor (k [total, heads, dk] -> ck, v [total, heads, dv] -> cv, both over cu_out); wk_t / wv_t both NULL = mean
+ * pooling, which then runs as ONE launch over both tensors; with weights it is the two GEMM launches. */
+int nsa_compress_kv_fwd(const void* k, const void* v, const void* wk_t, const void* wv_t, const void* bk,
+                        const void* bv, void* ck, void* cv, const int32_t* cu_seqlens, const int32_t* cu_out,
+                        int batch, int out_rows_bound, int heads, int dk, int dv, int block, int stride, int dtype,
+                        nsa_stream_t stream);
+
 /* Key-contiguous copy of a packed [rows, heads, dim] tensor (row_stride / head_stride in elements).
  * Layout preparation for the MFMA PV product; no counterpart in the reference. */
 int nsa_transpose_fwd(const void* x, void* out, const int32_t* cu, int batch, int heads, int dim,
@@ -93,7 +102,9 @@ int nsa_compress_bwd(const void* x, const void* w_lin, const void* d_out, void* 
  *   pooled block scores (bins past a sequence's last one up to max_ns are zeroed).  Pass it even when
  *   the scores are not wanted: with it (and a GQA group of 9..16 heads, pooling 5/4/0, max_ns <= 4096,
  *   top_n <= 64) the selection runs as two lean kernels that use it as their hand-over buffer, without
- *   it as one slower kernel that keeps the bins in LDS;
+ *   it as one slower kernel that keeps the bins in LDS;  keep_pooled == 0 says that the scores themselves are
+ *   not wanted: the buffer then only carries the window sums between the two kernels, its contents afterwards
+ *   are unspecified, and the second kernel saves writing the averages back;
  *   lse (float) [total, hq] receives the log-sum-exp of the raw scores q.ck over all compressed rows
  *   (the reference's M without its mask and scale); required when indices is given.
  *   Compressed row c of a sequence is visible to token t iff c*stride + block <= t (causal != 0;
@@ -104,7 +115,7 @@ int nsa_cmp_attn_select_fwd(const void* q, const void* ck, const void* cvt, void
                             int total, int hq, int hkv, int dk, int dv, int64_t ck_row_stride,
                             int64_t ck_head_stride, int cvt_cols, int block, int stride, int pool_kernel,
                             int pool_stride, int pool_pad, int top_n, int max_ns, int pooled_stride,
-                            float scale, int causal, int idx64, int dtype, nsa_stream_t stream);
+                            int keep_pooled, float scale, int causal, int idx64, int dtype, nsa_stream_t stream);
 
 /* The two halves of nsa_cmp_attn_select_fwd as separate launches: compressed attention (writes o
  * and lse) and block selection (reads lse).  Same arguments and meaning as above.
@@ -118,8 +129,8 @@ int nsa_cmp_attn_fwd(const void* q, const void* ck, const void* cvt, void* o, fl
 int nsa_block_select_fwd(const void* q, const void* ck, const float* lse, void* indices, float* pooled,
                          const int32_t* cu_seqlens, const int32_t* cu_cmp, int batch, int total, int hq, int hkv,
                          int dk, int64_t ck_row_stride, int64_t ck_head_stride, int pool_kernel, int pool_stride,
-                         int pool_pad, int top_n, int max_ns, int pooled_stride, int idx64, int dtype,
-                         nsa_stream_t stream);
+                         int pool_pad, int top_n, int max_ns, int pooled_stride, int keep_pooled, int idx64,
+                         int dtype, nsa_stream_t stream);
 
 /* Model integration: the glue between a layer's fused q/k/v(/gate) projection GEMM and the kernels
  * above.  The reference leaves this to its caller (nsa/nsa.py:83-135 receives q, k, v already split and

@@ -23,13 +23,14 @@ SIGNATURES = {
     "nsa_transposed_offset": (_I, [_I, _I]),
     "nsa_transposed_cols": (_I, [_I, _I]),
     "nsa_compress_fwd": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
+    "nsa_compress_kv_fwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
     "nsa_compress_bwd": (_I, [_P] * 8 + [_I] * 8 + [_P]),
     "nsa_transpose_fwd": (_I, [_P, _P, _P, _I, _I, _I, _L, _L, _I, _I, _P]),
     "nsa_cmp_attn_select_fwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _L, _I,
-                                     _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P]),
+                                     _I, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P]),
     "nsa_cmp_attn_fwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _L, _I, _I, _I, _F, _I, _I, _P]),
     "nsa_block_select_fwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _L, _L, _I, _I, _I, _I, _I, _I,
-                                  _I, _I, _P]),
+                                  _I, _I, _I, _P]),
     "nsa_gate_fwd": (_I, [_P, _P, _P, _P, _L, _I, _I, _P]),
     "nsa_gate_bwd": (_I, [_P] * 6 + [_L, _I, _I, _P]),
     "nsa_gate_combine_fwd": (_I, [_P] * 5 + [_L, _I, _I, _I, _P]),

@@ -49,8 +49,9 @@ def _compress_kv_nograd(k, v, w_k, w_v, cu, cu_out, out_rows, block_stride, bloc
     wv_t = w_v.detach().t().contiguous()
     kk = k if k.dtype in (torch.bfloat16, torch.float32) else k.to(torch.bfloat16)
     vv = v if v.dtype in (torch.bfloat16, torch.float32) else v.to(torch.bfloat16)
-    ck = ops.compress(kk, cu, cu_out, out_rows, block_size, block_stride, wk_t)
-    cv = ops.compress(vv, cu, cu_out, out_rows, block_size, block_stride, wv_t)
+    if kk.dtype != vv.dtype:
+        vv = vv.to(kk.dtype)
+    ck, cv = ops.compress_kv(kk, vv, cu, cu_out, out_rows, block_size, block_stride, wk_t, wv_t)
     return ck.to(torch.bfloat16), cv.to(torch.bfloat16), cu_out
 
 
@@ -128,13 +129,11 @@ class KVCompressor(nn.Module):
             ck = CompressFn.apply(k, wk, bk, cu, cu_out, rows, self.block_size, self.block_stride)
             cv = CompressFn.apply(v, wv, bv, cu, cu_out, rows, self.block_size, self.block_stride)
         elif self.mode == "mean":
-            ck = ops.compress(k, cu, cu_out, rows, self.block_size, self.block_stride)
-            cv = ops.compress(v, cu, cu_out, rows, self.block_size, self.block_stride)
+            ck, cv = ops.compress_kv(k, v, cu, cu_out, rows, self.block_size, self.block_stride)
         else:
-            ck = ops.compress(k, cu, cu_out, rows, self.block_size, self.block_stride,
-                              self._wt(self.compressor_k), self.compressor_k.bias)
-            cv = ops.compress(v, cu, cu_out, rows, self.block_size, self.block_stride,
-                              self._wt(self.compressor_v), self.compressor_v.bias)
+            ck, cv = ops.compress_kv(k, v, cu, cu_out, rows, self.block_size, self.block_stride,
+                                     self._wt(self.compressor_k), self._wt(self.compressor_v),
+                                     self.compressor_k.bias, self.compressor_v.bias)
         return ck, cv, cu_out, nc
 
     def forward(self, k, v, cu_seq_len, group=None):

@@ -75,6 +75,32 @@ int nsa_compress_fwd(const void* x, const void* wt, const void* bias, void* out,
   return finish(rc, "compress");
 }
 
+int nsa_compress_kv_fwd(const void* k, const void* v, const void* wk_t, const void* wv_t, const void* bk,
+                        const void* bv, void* ck, void* cv, const int32_t* cu_seqlens, const int32_t* cu_out,
+                        int batch, int out_rows_bound, int heads, int dk, int dv, int block, int stride, int dtype,
+                        nsa_stream_t stream) {
+  if (!k || !v || !ck || !cv) return fail(NSA_ERR_INVALID, "compress_kv: null pointer");
+  if ((wk_t == nullptr) != (wv_t == nullptr))
+    return fail(NSA_ERR_INVALID, "compress_kv: give both weights or neither");
+  if (wk_t) {                                   // learned compressor: one GEMM launch per tensor
+    const int rc = nsa_compress_fwd(k, wk_t, bk, ck, cu_seqlens, cu_out, batch, out_rows_bound, heads, dk, block,
+                                    stride, dtype, stream);
+    if (rc != NSA_OK) return rc;
+    return nsa_compress_fwd(v, wv_t, bv, cv, cu_seqlens, cu_out, batch, out_rows_bound, heads, dv, block, stride,
+                            dtype, stream);
+  }
+  if (!cu_seqlens || !cu_out) return fail(NSA_ERR_INVALID, "compress_kv: null pointer");
+  if (batch <= 0 || heads <= 0 || block <= 0 || stride <= 0 || out_rows_bound < 0)
+    return fail(NSA_ERR_INVALID, "compress_kv: sizes must be positive");
+  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "compress_kv: bad dtype");
+  if (dk % 8 != 0 || dv % 8 != 0) return fail(NSA_ERR_UNSUPPORTED, "compress_kv: dims must be multiples of 8");
+  if (!aligned16(k) || !aligned16(v) || !aligned16(ck) || !aligned16(cv))
+    return fail(NSA_ERR_INVALID, "compress_kv: pointers must be 16-byte aligned");
+  nsa::CompressArgs a{k, nullptr, nullptr, ck, cu_seqlens, cu_out, batch, out_rows_bound, heads, dk, block, stride, dtype};
+  a.x2 = v; a.out2 = cv; a.dim2 = dv;
+  return finish(nsa::launch_compress(a, stream), "compress_kv");
+}
+
 int nsa_compress_bwd(const void* x, const void* w_lin, const void* d_out, void* dx, float* dw, float* dbias,
                      const int32_t* cu_seqlens, const int32_t* cu_out, int batch, int total, int out_rows_bound,
                      int heads, int dim, int block, int stride, int dtype, nsa_stream_t stream) {
@@ -110,8 +136,8 @@ static int cmp_common(const char* what, int stages, const void* q, const void* c
                       void* indices, float* pooled, float* lse, float* lse_attn, const int32_t* cu_seqlens,
                       const int32_t* cu_cmp, int batch, int total, int hq, int hkv, int dk, int dv, int64_t ck_row_stride,
                       int64_t ck_head_stride, int cvt_cols, int block, int stride, int pool_kernel, int pool_stride,
-                      int pool_pad, int top_n, int max_ns, int pooled_stride, float scale, int causal, int idx64,
-                      int dtype, nsa_stream_t stream) {
+                      int pool_pad, int top_n, int max_ns, int pooled_stride, int keep_pooled, float scale, int causal,
+                      int idx64, int dtype, nsa_stream_t stream) {
   const bool attn = stages & 1, select = stages & 2;
   if (!q || !ck || !cu_seqlens || !cu_cmp) return fail(NSA_ERR_INVALID, "%s: null pointer", what);
   if (attn && (!cvt || !o)) return fail(NSA_ERR_INVALID, "%s: null pointer", what);
@@ -135,6 +161,7 @@ static int cmp_common(const char* what, int stages, const void* q, const void* c
   nsa::CmpArgs a{q, ck, cvt, o, indices, pooled, lse, cu_seqlens, cu_cmp, batch, total, hq, hkv * kv_rep, dk, dv,
                  (long)ck_row_stride, (long)ck_head_stride, cvt_cols, block, stride, pool_kernel, pool_stride,
                  pool_pad, top_n, max_ns, pooled_stride, scale, idx64, dtype, causal, lse_attn, kv_rep};
+  a.keep_pooled = keep_pooled != 0;
   int rc = 0;
   if (attn) rc = nsa::launch_cmp_attn(a, stream);
   if (rc == 0 && select) rc = nsa::launch_select(a, stream);
@@ -149,11 +176,11 @@ int nsa_cmp_attn_select_fwd(const void* q, const void* ck, const void* cvt, void
                             int total, int hq, int hkv, int dk, int dv, int64_t ck_row_stride,
                             int64_t ck_head_stride, int cvt_cols, int block, int stride, int pool_kernel,
                             int pool_stride, int pool_pad, int top_n, int max_ns, int pooled_stride,
-                            float scale, int causal, int idx64, int dtype, nsa_stream_t stream) {
+                            int keep_pooled, float scale, int causal, int idx64, int dtype, nsa_stream_t stream) {
   return cmp_common("cmp_attn_select", indices ? 3 : 1, q, ck, cvt, o, indices, pooled, lse, nullptr, cu_seqlens, cu_cmp,
                     batch, total, hq, hkv, dk, dv, ck_row_stride, ck_head_stride, cvt_cols, block, stride,
-                    pool_kernel, pool_stride, pool_pad, top_n, max_ns, pooled_stride, scale, causal, idx64, dtype,
-                    stream);
+                    pool_kernel, pool_stride, pool_pad, top_n, max_ns, pooled_stride, keep_pooled, scale, causal, idx64,
+                    dtype, stream);
 }
 
 int nsa_cmp_attn_fwd(const void* q, const void* ck, const void* cvt, void* o, float* lse, float* lse_attn,
@@ -161,18 +188,18 @@ int nsa_cmp_attn_fwd(const void* q, const void* ck, const void* cvt, void* o, fl
                      int dk, int dv, int64_t ck_row_stride, int64_t ck_head_stride, int cvt_cols, int block,
                      int stride, float scale, int causal, int dtype, nsa_stream_t stream) {
   return cmp_common("cmp_attn", 1, q, ck, cvt, o, nullptr, nullptr, lse, lse_attn, cu_seqlens, cu_cmp, batch, total, hq, hkv,
-                    dk, dv, ck_row_stride, ck_head_stride, cvt_cols, block, stride, 1, 1, 0, 1, 0, 0, scale, causal,
+                    dk, dv, ck_row_stride, ck_head_stride, cvt_cols, block, stride, 1, 1, 0, 1, 0, 0, 0, scale, causal,
                     0, dtype, stream);
 }
 
 int nsa_block_select_fwd(const void* q, const void* ck, const float* lse, void* indices, float* pooled,
                          const int32_t* cu_seqlens, const int32_t* cu_cmp, int batch, int total, int hq, int hkv,
                          int dk, int64_t ck_row_stride, int64_t ck_head_stride, int pool_kernel, int pool_stride,
-                         int pool_pad, int top_n, int max_ns, int pooled_stride, int idx64, int dtype,
-                         nsa_stream_t stream) {
+                         int pool_pad, int top_n, int max_ns, int pooled_stride, int keep_pooled, int idx64,
+                         int dtype, nsa_stream_t stream) {
   return cmp_common("block_select", 2, q, ck, nullptr, nullptr, indices, pooled, const_cast<float*>(lse), nullptr, cu_seqlens,
                     cu_cmp, batch, total, hq, hkv, dk, 16, ck_row_stride, ck_head_stride, 0, 1, 1, pool_kernel,
-                    pool_stride, pool_pad, top_n, max_ns, pooled_stride, 1.0f, 1, idx64, dtype, stream);
+                    pool_stride, pool_pad, top_n, max_ns, pooled_stride, keep_pooled, 1.0f, 1, idx64, dtype, stream);
 }
 
 int nsa_qkv_rope(void* packed, void* q, void* k, void* v, void* gates, const float* inv_freq,

@@ -9,6 +9,8 @@ struct CompressArgs {
   const void* x; const void* wt; const void* bias; void* out;
   const int32_t* cu_seq; const int32_t* cu_out;
   int batch, out_rows_bound, heads, dim, block, stride, dtype;
+  // mean pooling only: a second tensor over the same tokens (same heads, its own dim) for the same launch
+  const void* x2 = nullptr; void* out2 = nullptr; int dim2 = 0;
 };
 
 // Backward of the compression.  w_lin == nullptr: mean pooling (only dx).  w_lin is the weight in the
@@ -35,6 +37,9 @@ struct CmpArgs {
   // GQA groups beyond 16 heads run as kv_rep = G / 16 sub-groups of 16: hkv then counts the sub-groups
   // ("virtual" kv heads, hq / hkv == 16) and sub-group h reads the K / V rows of kv head h / kv_rep
   int kv_rep = 1;
+  // false: `pooled` only hands the window sums from the importance kernel to the top-n kernel; the averages are
+  // not written back (and the generic one-kernel selection does not write it at all)
+  bool keep_pooled = true;
 };
 
 struct SwaArgs {

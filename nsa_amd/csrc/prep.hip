@@ -24,32 +24,112 @@ __device__ __forceinline__ int upper_seq(const int32_t* __restrict__ cu, int bat
   return lo;
 }
 
+// One or two tensors over the same token axis (K and V of a layer) in one launch: blockIdx.y picks the tensor.
+#ifndef NSA_MEAN_U
+#define NSA_MEAN_U 32
+#endif
+struct MeanOperand {
+  const void* x;
+  void* out;
+  int dim;
+};
+
+// U rows of the window are requested before the first is added: the kernel is a pure stream whose time is the
+// memory latency times the number of dependent rounds, so a 32-row window is one round (bf16) or two (fp32).
 template <typename T>
 __global__ void __launch_bounds__(256)
-compress_mean_kernel(const T* __restrict__ x, T* __restrict__ out, const int32_t* __restrict__ cu_seq,
-                     const int32_t* __restrict__ cu_out, int batch, int heads, int dim, int block,
-                     int stride) {
-  const int ppr = heads * dim / 8;  // 8-element pieces per token row
+compress_mean_kernel(const MeanOperand s0, const MeanOperand s1, const int32_t* __restrict__ cu_seq,
+                     const int32_t* __restrict__ cu_out, int batch, int heads, int block, int stride) {
+  constexpr int U = NSA_MEAN_U / (int)(sizeof(T) / 2);
+  const MeanOperand s = blockIdx.y == 0 ? s0 : s1;
+  const int row_elems = heads * s.dim;
+  const int ppr = row_elems / 8;  // 8-element pieces per token row
   const long idx = (long)blockIdx.x * 256 + threadIdx.x;
   const int r = (int)(idx / ppr);
   const int piece = (int)(idx % ppr);
   if (r >= cu_out[batch]) return;
   const int b = upper_seq(cu_out, batch, r);
   const int n = r - cu_out[b];
-  const T* src = x + ((long)cu_seq[b] + (long)n * stride) * (heads * dim) + piece * 8;
+  const T* src = reinterpret_cast<const T*>(s.x) + ((long)cu_seq[b] + (long)n * stride) * row_elems + piece * 8;
   float acc[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) acc[i] = 0.f;
-#pragma unroll 4
-  for (int j = 0; j < block; ++j) {
-    const vec8_t<T> v = load8(src + (long)j * heads * dim);
+  for (int j0 = 0; j0 < block; j0 += U) {
+    vec8_t<T> v[U];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) acc[i] += (float)v[i];
+    for (int u = 0; u < U; ++u)
+      if (j0 + u < block) v[u] = load8(src + (long)(j0 + u) * row_elems);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (j0 + u < block) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] += (float)v[u][i];
+      }
   }
   const float inv = 1.0f / (float)block;
 #pragma unroll
   for (int i = 0; i < 8; ++i) acc[i] *= inv;
-  store8(out + (long)r * heads * dim + piece * 8, pack8<T>(acc));
+  store8(reinterpret_cast<T*>(s.out) + (long)r * row_elems + piece * 8, pack8<T>(acc));
+}
+
+// The same for windows of two strides (block == 2 * stride, stride <= 16: the usual 32 / 16), reading every token
+// row about once instead of twice.  A wavefront is 8 stride groups x 8 pieces (64 channels): lane (s, p) sums the
+// `stride` rows of group s -- the first half of output row r0 + s -- and takes the second half from lane (s + 1, p),
+// which has just summed exactly those rows as the first half of the next output row.  Lane group 7 only helps
+// (its output row belongs to the next wavefront); a lane whose neighbour is past the end or in another sequence
+// sums its second half itself.
+template <typename T>
+__global__ void __launch_bounds__(256)
+compress_mean_halves_kernel(const MeanOperand s0, const MeanOperand s1, const int32_t* __restrict__ cu_seq,
+                            const int32_t* __restrict__ cu_out, int batch, int heads, int stride) {
+  constexpr int U = 16;
+  const MeanOperand sp = blockIdx.y == 0 ? s0 : s1;
+  const int row_elems = heads * sp.dim;
+  const int cblocks = row_elems / 64;
+  const int lane = threadIdx.x & 63, s = lane >> 3, p = lane & 7;
+  const long item = (long)blockIdx.x * 4 + (threadIdx.x >> 6);       // (run of 7 output rows, 64-channel block)
+  const int total_out = cu_out[batch];
+  const long r0 = (item / cblocks) * 7;
+  if (r0 >= total_out) return;
+  const int col = (int)(item % cblocks) * 64 + p * 8;
+  const long r = r0 + s;
+  const bool valid = r < total_out;
+  int b = -1;
+  const T* src = reinterpret_cast<const T*>(sp.x);
+  if (valid) {
+    b = upper_seq(cu_out, batch, (int)r);
+    src += ((long)cu_seq[b] + (r - cu_out[b]) * stride) * row_elems + col;
+  }
+  auto half_sum = [&](const T* base, float (&acc)[8]) {
+    vec8_t<T> v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (u < stride) v[u] = load8(base + (long)u * row_elems);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (u < stride) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] += (float)v[u][i];
+      }
+  };
+  float g1[8], g2[8];
+  if (valid) half_sum(src, g1);
+  else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) g1[i] = 0.f;
+  }
+  const int b_next = __shfl_down(b, 8);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) g2[i] = __shfl_down(g1[i], 8);
+  if (!valid || s == 7) return;
+  if (b_next != b) half_sum(src + (long)stride * row_elems, g2);     // b_next is -1 past the end
+  const float inv = 0.5f / (float)stride;
+  float o[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) o[i] = (g1[i] + g2[i]) * inv;
+  store8(reinterpret_cast<T*>(sp.out) + r * row_elems + col, pack8<T>(o));
 }
 
 // One workgroup per (32 output rows, head).  The block's taps are dealt to the 4 wavefronts (split-K):
@@ -168,10 +248,20 @@ template <typename T>
 static int launch_compress_t(const CompressArgs& a, hipStream_t st) {
   if (a.out_rows_bound <= 0) return 0;
   if (a.wt == nullptr) {
-    const long threads = (long)a.out_rows_bound * (a.heads * a.dim / 8);
-    const int grid = (int)((threads + 255) / 256);
-    hipLaunchKernelGGL(compress_mean_kernel<T>, dim3(grid), dim3(256), 0, st, (const T*)a.x, (T*)a.out,
-                       a.cu_seq, a.cu_out, a.batch, a.heads, a.dim, a.block, a.stride);
+    const MeanOperand s0{a.x, a.out, a.dim};
+    const MeanOperand s1{a.x2 ? a.x2 : a.x, a.x2 ? a.out2 : a.out, a.x2 ? a.dim2 : a.dim};
+    const int dmax = a.x2 && a.dim2 > a.dim ? a.dim2 : a.dim;
+    if (a.block == 2 * a.stride && a.stride <= 16 && (a.heads * s0.dim) % 64 == 0 && (a.heads * s1.dim) % 64 == 0) {
+      const long items = ((long)a.out_rows_bound + 6) / 7 * (a.heads * dmax / 64);
+      const dim3 grid((unsigned)((items + 3) / 4), a.x2 ? 2 : 1);
+      hipLaunchKernelGGL(compress_mean_halves_kernel<T>, grid, dim3(256), 0, st, s0, s1, a.cu_seq, a.cu_out, a.batch,
+                         a.heads, a.stride);
+      return 0;
+    }
+    const long threads = (long)a.out_rows_bound * (a.heads * dmax / 8);
+    const dim3 grid((unsigned)((threads + 255) / 256), a.x2 ? 2 : 1);
+    hipLaunchKernelGGL(compress_mean_kernel<T>, grid, dim3(256), 0, st, s0, s1, a.cu_seq, a.cu_out, a.batch, a.heads,
+                       a.block, a.stride);
     return 0;
   }
   const dim3 grid((a.out_rows_bound + 31) / 32, a.heads);

@@ -449,8 +449,8 @@ topn_kernel(const CmpArgs a) {
       const int lo = b * a.pool_s - a.pool_p;
       const int div = min(lo + a.pool_k, Nc + a.pool_p) - lo;
       v[k] = v[k] / (float)div;
-      prow[b] = v[k];
-    } else if (b < a.max_ns) {
+      if (a.keep_pooled) prow[b] = v[k];
+    } else if (b < a.max_ns && a.keep_pooled) {
       prow[b] = 0.f;
     }
   }
@@ -521,11 +521,13 @@ static int launch_select_t(const CmpArgs& a, hipStream_t st) {
       a.pool_s == 4 && a.pool_p == 0)
     return launch_select_stream<T, DK>(a, st);
   if (a.kv_rep > 1) return -6;      // groups beyond 16 heads exist on the two-kernel schedule only
+  CmpArgs b = a;
+  if (!a.keep_pooled) b.pooled = nullptr;   // this kernel keeps its bins in LDS: nothing to hand over
   // four row groups per wavefront unless the per-token bins of such a tile outgrow the LDS
   constexpr int NGBIG = sizeof(T) == 2 ? 4 : 2;
-  const int rc = launch_select_ng<T, DK, NGBIG>(a, st);
+  const int rc = launch_select_ng<T, DK, NGBIG>(b, st);
   if (rc != -3) return rc;
-  return launch_select_ng<T, DK, 1>(a, st);
+  return launch_select_ng<T, DK, 1>(b, st);
 }
 
 int launch_select(const CmpArgs& a, hipStream_t st) {

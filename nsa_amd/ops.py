@@ -121,6 +121,36 @@ def compress(x: torch.Tensor, cu_seqlens: torch.Tensor, cu_out: torch.Tensor, ou
     return out
 
 
+def compress_kv(k: torch.Tensor, v: torch.Tensor, cu_seqlens: torch.Tensor, cu_out: torch.Tensor, out_rows: int,
+                block: int, stride: int, wk_t=None, wv_t=None, bk=None, bv=None):
+    """k [total, H, Dk], v [total, H, Dv] -> (ck [out_rows, H, Dk], cv [out_rows, H, Dv]).  Without weights
+    (mean over each window) both tensors go through one launch; w*_t are [D, block*D] as in compress()."""
+    _need_cuda(k, v, cu_seqlens, cu_out)
+    k, v = _dense(k), _dense(v)
+    total, H, Dk = k.shape
+    if v.shape[0] != total or v.shape[1] != H or v.dtype != k.dtype:
+        raise ValueError("k and v must share tokens, heads and dtype: %s vs %s" % (tuple(k.shape), tuple(v.shape)))
+    Dv = v.shape[2]
+    ck = torch.empty(out_rows, H, Dk, dtype=k.dtype, device=k.device)
+    cv = torch.empty(out_rows, H, Dv, dtype=v.dtype, device=v.device)
+    if (wk_t is None) != (wv_t is None):
+        raise ValueError("give both weights or neither")
+    if wk_t is not None:
+        wk_t, wv_t = _dense(wk_t.to(k.dtype)), _dense(wv_t.to(v.dtype))
+        if tuple(wk_t.shape) != (Dk, block * Dk) or tuple(wv_t.shape) != (Dv, block * Dv):
+            raise ValueError("weights must be [dim, block*dim], got %s and %s" % (tuple(wk_t.shape), tuple(wv_t.shape)))
+    bk = None if bk is None else _dense(bk.to(k.dtype))
+    bv = None if bv is None else _dense(bv.to(v.dtype))
+    if out_rows == 0:
+        return ck, cv
+    lib = _lib.load()
+    rc = lib.nsa_compress_kv_fwd(_ptr(k), _ptr(v), _ptr(wk_t), _ptr(wv_t), _ptr(bk), _ptr(bv), _ptr(ck), _ptr(cv),
+                                 _ptr(cu_seqlens), _ptr(cu_out), cu_seqlens.numel() - 1, out_rows, H, Dk, Dv, block,
+                                 stride, _dtype_code(k), _stream())
+    _lib.check(rc, "nsa_compress_kv_fwd")
+    return ck, cv
+
+
 def cmp_attn_select(q, ck, cvt, cu_seqlens, cu_cmp, batch, hkv, dv, ck_row_stride, ck_head_stride, block,
                     stride, pool_kernel, pool_stride, pool_pad, top_n, max_nc, scale, causal=True,
                     select=True, idx64=True, want_pooled=False):
@@ -143,8 +173,8 @@ def cmp_attn_select(q, ck, cvt, cu_seqlens, cu_cmp, batch, hkv, dv, ck_row_strid
         _ptr(q), _ptr(ck), _ptr(cvt), _ptr(o), _ptr(idx), _ptr(pooled), _ptr(lse), _ptr(cu_seqlens), _ptr(cu_cmp),
         batch,
         total, hq, hkv, dk, dv, ck_row_stride, ck_head_stride, cvt.shape[-1], block, stride, pool_kernel,
-        pool_stride, pool_pad, max(top_n, 1), max_ns, max(max_ns, 1), float(scale), int(bool(causal)),
-        int(idx64), _dtype_code(q), _stream())
+        pool_stride, pool_pad, max(top_n, 1), max_ns, max(max_ns, 1), int(bool(want_pooled)), float(scale),
+        int(bool(causal)), int(idx64), _dtype_code(q), _stream())
     _lib.check(rc, "nsa_cmp_attn_select_fwd")
     return o, idx, (pooled[:, :, 0] if want_pooled else None)
 
@@ -182,7 +212,7 @@ def block_select(q, ck, lse, cu_seqlens, cu_cmp, batch, hkv, ck_row_stride, ck_h
     rc = _lib.load().nsa_block_select_fwd(_ptr(q), _ptr(ck), _ptr(lse), _ptr(idx), _ptr(pooled), _ptr(cu_seqlens),
                                           _ptr(cu_cmp), batch, total, hq, hkv, dk, ck_row_stride, ck_head_stride,
                                           pool_kernel, pool_stride, pool_pad, top_n, max_ns, max(max_ns, 1),
-                                          int(idx64), _dtype_code(q), _stream())
+                                          int(bool(want_pooled)), int(idx64), _dtype_code(q), _stream())
     _lib.check(rc, "nsa_block_select_fwd")
     return idx, (pooled[:, :, 0] if want_pooled else None)
 

@@ -47,6 +47,42 @@ def test_compress_mean(dtype, lens, H, D, l, d):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("lens,H,Dk,Dv,l,d", [([1024], 1, 64, 64, 32, 16), ([300, 31, 64, 1000], 4, 192, 128, 32, 16),
+                                              ([200, 77], 2, 64, 128, 40, 8), ([31], 2, 32, 32, 32, 16),
+                                              ([300, 17, 16, 1000, 33], 4, 128, 64, 16, 8),
+                                              ([100, 45], 1, 32, 32, 32, 16)])
+def test_compress_kv_pair(dtype, lens, H, Dk, Dv, l, d):
+    """K and V through the paired entry point (one launch for mean pooling, head dims may differ, windows that
+    are not a multiple of the kernel's load round, a sequence with no compressed row) against the oracle, and
+    bit-identical to the one-tensor entry point."""
+    ops = _ops()
+    k = randn(sum(lens), H, Dk, seed=1, dtype=dtype)
+    v = randn(sum(lens), H, Dv, seed=2, dtype=dtype)
+    cu = _cu(lens)
+    cu_out = ops.compressed_offsets(cu, l, d, extra=1)
+    ncs = [O.compressed_len_conv(t, l, d) for t in lens]
+    ck, cv = ops.compress_kv(k.to(DEV), v.to(DEV), cu, cu_out, sum(ncs), l, d)
+    assert ck.shape == (sum(ncs), H, Dk) and cv.shape == (sum(ncs), H, Dv)
+    if sum(ncs) == 0:
+        return
+    for x, got in ((k, ck), (v, cv)):
+        ref = torch.cat([O.compress_meanpool(x[s:e], l, d, n) for s, e, n in
+                         zip(ragged_cu(lens)[:-1], ragged_cu(lens)[1:], ncs)])
+        assert max_abs(got, ref) <= (1e-6 if dtype == torch.float32 else 4e-3)
+        assert torch.equal(got, ops.compress(x.to(DEV), cu, cu_out, sum(ncs), l, d))
+    # learned compressor through the same entry point: the two GEMM launches
+    if Dk == Dv and l == 32:
+        wk = randn(l * Dk, Dk, seed=3, dtype=dtype, scale=0.05)
+        wv = randn(l * Dv, Dv, seed=4, dtype=dtype, scale=0.05)
+        ck2, cv2 = ops.compress_kv(k.to(DEV), v.to(DEV), cu, cu_out, sum(ncs), l, d, wk.t().contiguous().to(DEV),
+                                   wv.t().contiguous().to(DEV))
+        # (the GEMM adds its split-K partial sums in LDS in whatever order they arrive: equal up to rounding)
+        tol = 1e-5 if dtype == torch.float32 else 4e-3
+        assert max_abs(ck2, ops.compress(k.to(DEV), cu, cu_out, sum(ncs), l, d, wk.t().contiguous().to(DEV))) <= tol
+        assert max_abs(cv2, ops.compress(v.to(DEV), cu, cu_out, sum(ncs), l, d, wv.t().contiguous().to(DEV))) <= tol
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("lens,H,D,l,d,extra", [([256, 100], 2, 64, 32, 16, 1), ([1024] * 2, 2, 128, 64, 16, 0),
                                                 ([90], 1, 32, 8, 4, 1)])
 def test_compress_weighted(dtype, lens, H, D, l, d, extra):
