@@ -17,7 +17,9 @@ torch path) on a bounded sample of query rows of the same workload, on this host
 train_step (extra, not the headline metric): forward + backward of the same workload through the
 module's autograd path.  decode / decode_small_batch (extra): the decode step of benchmark config 5 at
 batch 64 and at batch 8.  layer (extra): the attention layer (projections, rotary embedding, NSA,
-output projection) around the same workload.
+output projection) around the same workload.  compress (extra): the mean-pooling and the learned compressor alone.
+roofline.traffic is read from the committed counter summary under profiles/ and only when the kernel sources
+still hash to the build it was measured on (roofline.traffic_source says which, or why not).
 """
 import argparse
 import json
@@ -40,8 +42,26 @@ WORKLOADS = {
     "prefill_cfg2": ([8192], 64, 4, 128, 128, 16, 512, 1),
 }
 BLOCK, STRIDE, SEL_BLOCK = 32, 16, 64
-# bytes per launch: (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0) KiB, factors from a 1 GiB device copy in the same run
-MEASURED_TRAFFIC = {("prefill_cfg4", "cmp_attn"): int((443594.0 * 2.0 + 532480.0) * 1024)}
+TRAFFIC_PROFILE = "profiles/prefill_cfg4_hbm_traffic.md"
+
+
+def measured_traffic(workload, kernel):
+    """HBM bytes per launch of `kernel` as the committed counter summary states them, and where they come from.
+    The summary carries a line `roofline.traffic: workload=<w> kernel=<k> bytes=<n> csrc_sha256=<digest>`; the
+    figure is only passed on when the kernel sources are still the ones it was measured on."""
+    import re
+    from nsa_amd.build import sources_digest
+    try:
+        text = open(os.path.join(ROOT, TRAFFIC_PROFILE)).read()
+    except OSError:
+        return None, "%s not found" % TRAFFIC_PROFILE
+    for m in re.finditer(r"roofline\.traffic:\s*workload=(\S+)\s+kernel=(\S+)\s+bytes=(\d+)\s+csrc_sha256=([0-9a-f]+)", text):
+        if m.group(1) == workload and m.group(2) == kernel:
+            now = sources_digest()
+            if m.group(4) != now:
+                return None, "%s was measured on other kernel sources (%s, this build %s)" % (TRAFFIC_PROFILE, m.group(4), now)
+            return int(m.group(3)), "%s (rocprofv3 FETCH_SIZE + WRITE_SIZE, kernel sources %s)" % (TRAFFIC_PROFILE, now)
+    return None, "%s has no figure for %s / %s" % (TRAFFIC_PROFILE, workload, kernel)
 
 
 def flops_model(lens, hq, hkv, dqk, dv, window, valid_blocks_total):
@@ -144,6 +164,45 @@ def decode_bench(steps, warmup):
             "achieved_GBps": nbytes / (us * 1e-6) / 1e9, "hbm_peak_GBps": PEAK_HBM_GBS,
             "hbm_frac": nbytes / (us * 1e-6) / 1e9 / PEAK_HBM_GBS,
             "workload": "decode_cfg5: batch 64 x 1 token, ctx 32768, Hq64/Hkv4, D128, top-16 x 64, window 512, bf16"}
+
+
+def compress_bench(k, v, cu, steps=20):
+    """The two compressors alone on the workload's K / V (extra): mean pooling is a pure HBM stream (algorithmic
+    bytes: K and V read once, the compressed rows written), the learned (Conv1d-equivalent) compressor a GEMM of
+    [rows x block*D] by [block*D x D] per head and tensor."""
+    import torch
+    from nsa_amd import ops
+    total, h, dk = k.shape
+    dv = v.shape[2]
+    batch = cu.numel() - 1
+    cu_out = ops.compressed_offsets(cu, BLOCK, STRIDE, extra=1)
+    rows = int(cu_out[-1].item())
+    gen = torch.Generator(device=k.device).manual_seed(11)
+    wk = (torch.randn(dk, BLOCK * dk, device=k.device, generator=gen) * 0.02).bfloat16()
+    wv = (torch.randn(dv, BLOCK * dv, device=k.device, generator=gen) * 0.02).bfloat16()
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        beg, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        beg.record()
+        for _ in range(steps):
+            fn()
+        end.record()
+        torch.cuda.synchronize()
+        return beg.elapsed_time(end) / steps * 1e3
+
+    us_mean = timed(lambda: ops.compress_kv(k, v, cu, cu_out, rows, BLOCK, STRIDE))
+    us_w = timed(lambda: ops.compress_kv(k, v, cu, cu_out, rows, BLOCK, STRIDE, wk, wv))
+    nbytes = (total + rows) * h * (dk + dv) * 2
+    flops = 2.0 * rows * h * BLOCK * (dk * dk + dv * dv)
+    return {"mean": {"us": us_mean, "algorithmic_bytes": nbytes, "achieved_GBps": nbytes / (us_mean * 1e-6) / 1e9,
+                     "hbm_frac": nbytes / (us_mean * 1e-6) / 1e9 / PEAK_HBM_GBS,
+                     "note": "back-to-back launches through the Python wrapper, host launch cost included"},
+            "learned": {"us": us_w, "flops": flops, "tflops": flops / (us_w * 1e-6) / 1e12,
+                        "mfma_peak_frac": flops / (us_w * 1e-6) / 1e12 / PEAK_BF16_TFLOPS},
+            "rows": rows, "batch": batch}
 
 
 def train_bench(m, q, k, v, gl, cu, max_len, total, f_eff, steps, warmup):
@@ -350,7 +409,7 @@ def main():
     dom_tflops = stage_tflops[dom]
     # HBM bytes per launch of that kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE (profiles/), only
     # recorded for the default workload
-    traffic = MEASURED_TRAFFIC.get((args.workload, dom))
+    traffic, traffic_source = measured_traffic(args.workload, dom)
     # The compressed-attention kernel also multiplies q with the compressed keys a token cannot see: the
     # importance softmax is normalised over all of them.  `executed` adds that uncredited part of QK^T.
     executed = None
@@ -372,9 +431,10 @@ def main():
         "stage_ms": stage_ms,
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": dom_tflops, "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": dom_tflops / PEAK_BF16_TFLOPS, "traffic": traffic,
-                     "executed": executed},
+                     "traffic_source": traffic_source, "executed": executed},
         "stage_effective_tflops": stage_tflops,
     }
+    res["compress"] = compress_bench(kd, vd, cu)
     if not args.no_backward:
         res["train_step"] = train_bench(m, qd, kd, vd, gd, cu, max_len, total, f_eff, max(2, min(args.steps, 5)), 2)
     if not args.no_layer and len(lens) == 1:

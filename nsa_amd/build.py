@@ -15,6 +15,19 @@ FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-Xclang", "-tar
          "-packed-fp32-ops", "-fno-honor-nans", "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option"]
 
 
+def sources_digest() -> str:
+    """First 12 hex digits of the SHA-256 over the kernel sources (file names and contents, sorted): names the
+    build a measurement was taken on."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(CSRC)):
+        if name.endswith((".hip", ".h")):
+            h.update(name.encode())
+            with open(os.path.join(CSRC, name), "rb") as f:
+                h.update(f.read())
+    return h.hexdigest()[:12]
+
+
 def _hipcc() -> str:
     for cand in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
         if cand and (os.path.isabs(cand) and os.path.exists(cand) or not os.path.isabs(cand)):
@@ -43,6 +56,10 @@ def build(verbose: bool = False, extra_flags=()) -> str:
         print("built", LIB)
     return LIB
 
+
+if __name__ == "__main__" and sys.argv[1:] == ["--digest"]:
+    print(sources_digest())
+    sys.exit(0)
 
 if __name__ == "__main__":
     build(verbose=True, extra_flags=sys.argv[1:])

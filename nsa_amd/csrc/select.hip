@@ -229,7 +229,7 @@ __device__ __forceinline__ float row_reduce_scatter4(float v0, float v1, float v
 // its quad to the next step, where it is completed with that step's first column.  Every bin is
 // written exactly once, 64 contiguous bytes per token and step, with no atomics.
 template <typename T, int DK, int NG, int NW>
-__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(4, 4)))
+__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NG <= 2 ? 4 : 2, NG <= 2 ? 4 : 2)))
 importance_stream_kernel(const CmpArgs a) {
   constexpr int CH = 64, KLD = DK + kLdsRowPad<T>, NT = NW * 64, TQ = NW * NG;
   constexpr int KPIECES = CH * DK / 8;
