@@ -8,7 +8,10 @@
  *   - tensors are packed ("varlen"): rows of all sequences back to back, `cu_seqlens` int32[batch+1]
  *     with cu_seqlens[0] == 0 holds the row offsets; a batch of equal lengths is the special case
  *     cu_seqlens[b] = b*T
- *   - dtype: NSA_BF16 or NSA_F32 for every floating tensor of a call (accumulation is always fp32)
+ *   - dtype: NSA_BF16 or NSA_F32 for every floating tensor of a call (accumulation is always fp32); the prefill
+ *     forward entry points (compress, transpose, gates, compressed / window / selected attention, block
+ *     selection, gated combine) also take NSA_F16, the dtype of the reference's own selection test
+ *     (tests/test_parallel_nsa.py:169); backward, decode and rotary entry points refuse it
  *   - GQA: hq / hkv query heads share one kv head.  Groups of 1..16 heads are built everywhere; the prefill
  *     forward entry points (nsa_cmp_attn_*, nsa_block_select_fwd, nsa_swa_fwd, nsa_slc_*, nsa_swa_merge_fwd)
  *     also take groups of 32, 48, 64, ... heads, which is what the reference's selected attention asks for
@@ -34,7 +37,7 @@ extern "C" {
 
 typedef struct ihipStream_t* nsa_stream_t; /* hipStream_t */
 
-enum { NSA_BF16 = 0, NSA_F32 = 1 };
+enum { NSA_BF16 = 0, NSA_F32 = 1, NSA_F16 = 2 };
 enum {
   NSA_OK = 0,
   NSA_ERR_INVALID = -1,     /* bad argument (null pointer, non-positive size, misalignment) */

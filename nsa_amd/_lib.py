@@ -11,7 +11,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libnsa_hip.so")
 
-NSA_BF16, NSA_F32 = 0, 1
+NSA_BF16, NSA_F32, NSA_F16 = 0, 1, 2
 GATE_IDENTITY, GATE_SIGMOID = 0, 1
 
 _P, _I, _L, _F = C.c_void_p, C.c_int, C.c_int64, C.c_float

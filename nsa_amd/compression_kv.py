@@ -35,8 +35,8 @@ def compress_kv(k, v, w_k, w_v, cu_seq_len, block_stride, block_size):
     cu_out = ops.compressed_offsets(cu, block_size, block_stride, extra=0)
     out_rows = int(cu_out[-1].item())      # the reference syncs here as well (cu_seq_len.tolist())
     if needs_grad(k, v, w_k, w_v):
-        kk = k if k.dtype in (torch.bfloat16, torch.float32) else k.to(torch.bfloat16)
-        vv = v if v.dtype in (torch.bfloat16, torch.float32) else v.to(torch.bfloat16)
+        kk = k if k.dtype in (torch.bfloat16, torch.float32, torch.float16) else k.to(torch.bfloat16)
+        vv = v if v.dtype in (torch.bfloat16, torch.float32, torch.float16) else v.to(torch.bfloat16)
         ck = CompressFn.apply(kk, w_k.to(kk.dtype), None, cu, cu_out, out_rows, block_size, block_stride)
         cv = CompressFn.apply(vv, w_v.to(vv.dtype), None, cu, cu_out, out_rows, block_size, block_stride)
         return ck.to(torch.bfloat16), cv.to(torch.bfloat16), cu_out
@@ -47,8 +47,8 @@ def compress_kv(k, v, w_k, w_v, cu_seq_len, block_stride, block_size):
 def _compress_kv_nograd(k, v, w_k, w_v, cu, cu_out, out_rows, block_stride, block_size):
     wk_t = w_k.detach().t().contiguous()
     wv_t = w_v.detach().t().contiguous()
-    kk = k if k.dtype in (torch.bfloat16, torch.float32) else k.to(torch.bfloat16)
-    vv = v if v.dtype in (torch.bfloat16, torch.float32) else v.to(torch.bfloat16)
+    kk = k if k.dtype in (torch.bfloat16, torch.float32, torch.float16) else k.to(torch.bfloat16)
+    vv = v if v.dtype in (torch.bfloat16, torch.float32, torch.float16) else v.to(torch.bfloat16)
     if kk.dtype != vv.dtype:
         vv = vv.to(kk.dtype)
     ck, cv = ops.compress_kv(kk, vv, cu, cu_out, out_rows, block_size, block_stride, wk_t, wv_t)

@@ -650,12 +650,12 @@ static int launch_swa_t(const SwaArgs& a, hipStream_t st) {
   return launch_stream_t<T, DK, DV, false>(p, a.total, st);
 }
 
-template <int DK, int DV>
+template <typename T, int DK, int DV>
 static int launch_swa_merge_t(const SwaArgs& a, const MergeArgs& m, hipStream_t st) {
   StreamParams p{a.q, a.k, a.vt, nullptr, nullptr, a.cu_seq, a.cu_seq, a.batch, a.hq, a.hkv, (long)(a.hkv / a.kv_rep) * DK,
                  (long)DK, a.vt_cols, 0, 0, a.window, 1, a.scale, m, a.lse, a.kv_rep, 0};
-  if (m.top_n == 16) return launch_stream_t<bf16_t, DK, DV, false, 16>(p, a.total, st);
-  return launch_stream_t<bf16_t, DK, DV, false, 1>(p, a.total, st);
+  if (m.top_n == 16) return launch_stream_t<T, DK, DV, false, 16>(p, a.total, st);
+  return launch_stream_t<T, DK, DV, false, 1>(p, a.total, st);
 }
 
 template <typename T, int DK, int DV>
@@ -679,6 +679,14 @@ static int launch_slc_t(const SlcArgs& a, hipStream_t st) {
         case 192128: return FN<bf16_t, 192, 128>(ARGS, ST);                           \
         default: return -2;                                                           \
       }                                                                               \
+    } else if ((ARGS).dtype == 2) {                                                   \
+      switch (key) {                                                                  \
+        case 32032: return FN<f16_t, 32, 32>(ARGS, ST);                               \
+        case 64064: return FN<f16_t, 64, 64>(ARGS, ST);                               \
+        case 128128: return FN<f16_t, 128, 128>(ARGS, ST);                            \
+        case 192128: return FN<f16_t, 192, 128>(ARGS, ST);                            \
+        default: return -2;                                                           \
+      }                                                                               \
     } else {                                                                          \
       switch (key) {                                                                  \
         case 32032: return FN<float, 32, 32>(ARGS, ST);                               \
@@ -693,11 +701,14 @@ static int launch_slc_t(const SlcArgs& a, hipStream_t st) {
 int launch_cmp_attn(const CmpArgs& a, hipStream_t st) { NSA_DISPATCH(launch_cmp_t, a, st); }
 int launch_swa(const SwaArgs& a, hipStream_t st) { NSA_DISPATCH(launch_swa_t, a, st); }
 int launch_swa_merge(const SwaArgs& a, const MergeArgs& m, hipStream_t st) {
-  if (a.dtype != 0) return -2;
-  switch (a.dk * 1000 + a.dv) {
-    case 64064: return launch_swa_merge_t<64, 64>(a, m, st);
-    case 128128: return launch_swa_merge_t<128, 128>(a, m, st);
-    case 192128: return launch_swa_merge_t<192, 128>(a, m, st);
+  if (a.dtype == 1) return -2;             // the partials are 16-bit
+  switch (a.dk * 1000 + a.dv + (a.dtype == 2 ? 1000000 : 0)) {
+    case 64064: return launch_swa_merge_t<bf16_t, 64, 64>(a, m, st);
+    case 128128: return launch_swa_merge_t<bf16_t, 128, 128>(a, m, st);
+    case 192128: return launch_swa_merge_t<bf16_t, 192, 128>(a, m, st);
+    case 1064064: return launch_swa_merge_t<f16_t, 64, 64>(a, m, st);
+    case 1128128: return launch_swa_merge_t<f16_t, 128, 128>(a, m, st);
+    case 1192128: return launch_swa_merge_t<f16_t, 192, 128>(a, m, st);
     default: return -2;
   }
 }

@@ -59,13 +59,16 @@ int nsa_transposed_cols(int total_rows, int batch) {
   return (need + 63) / 64 * 64;
 }
 
+// Forward prefill entry points take fp16 as well; backward, decode and rotary entry points are bf16 / fp32.
+static bool fwd_dtype_ok(int dtype) { return dtype == NSA_BF16 || dtype == NSA_F32 || dtype == NSA_F16; }
+
 int nsa_compress_fwd(const void* x, const void* wt, const void* bias, void* out, const int32_t* cu_seqlens,
                      const int32_t* cu_out, int batch, int out_rows_bound, int heads, int dim, int block,
                      int stride, int dtype, nsa_stream_t stream) {
   if (!x || !out || !cu_seqlens || !cu_out) return fail(NSA_ERR_INVALID, "compress: null pointer");
   if (batch <= 0 || heads <= 0 || block <= 0 || stride <= 0 || out_rows_bound < 0)
     return fail(NSA_ERR_INVALID, "compress: sizes must be positive");
-  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "compress: bad dtype");
+  if (!fwd_dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "compress: bad dtype");
   if (dim % 8 != 0) return fail(NSA_ERR_UNSUPPORTED, "compress: dim must be a multiple of 8");
   if (!aligned16(x) || !aligned16(out) || (wt && !aligned16(wt))) return fail(NSA_ERR_INVALID, "compress: pointers must be 16-byte aligned");
   if (wt && dim % 32 != 0) return fail(NSA_ERR_UNSUPPORTED, "compress: weighted path needs dim %% 32 == 0");
@@ -92,7 +95,7 @@ int nsa_compress_kv_fwd(const void* k, const void* v, const void* wk_t, const vo
   if (!cu_seqlens || !cu_out) return fail(NSA_ERR_INVALID, "compress_kv: null pointer");
   if (batch <= 0 || heads <= 0 || block <= 0 || stride <= 0 || out_rows_bound < 0)
     return fail(NSA_ERR_INVALID, "compress_kv: sizes must be positive");
-  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "compress_kv: bad dtype");
+  if (!fwd_dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "compress_kv: bad dtype");
   if (dk % 8 != 0 || dv % 8 != 0) return fail(NSA_ERR_UNSUPPORTED, "compress_kv: dims must be multiples of 8");
   if (!aligned16(k) || !aligned16(v) || !aligned16(ck) || !aligned16(cv))
     return fail(NSA_ERR_INVALID, "compress_kv: pointers must be 16-byte aligned");
@@ -127,7 +130,7 @@ int nsa_transpose_fwd(const void* x, void* out, const int32_t* cu, int batch, in
     return fail(NSA_ERR_INVALID, "transpose: dim must be a multiple of 8 and out_cols of 64");
   if (row_stride % 8 != 0 || head_stride % 8 != 0 || !aligned16(x) || !aligned16(out))
     return fail(NSA_ERR_INVALID, "transpose: strides must be multiples of 8 elements, pointers 16-byte aligned");
-  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "transpose: bad dtype");
+  if (!fwd_dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "transpose: bad dtype");
   nsa::TransposeArgs a{x, out, cu, batch, heads, dim, (long)row_stride, (long)head_stride, out_cols, dtype};
   return finish(nsa::launch_transpose(a, stream), "transpose");
 }
@@ -142,7 +145,7 @@ static int cmp_common(const char* what, int stages, const void* q, const void* c
   if (!q || !ck || !cu_seqlens || !cu_cmp) return fail(NSA_ERR_INVALID, "%s: null pointer", what);
   if (attn && (!cvt || !o)) return fail(NSA_ERR_INVALID, "%s: null pointer", what);
   if (batch <= 0 || total <= 0 || block <= 0 || stride <= 0) return fail(NSA_ERR_INVALID, "%s: sizes must be positive", what);
-  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "%s: bad dtype", what);
+  if (!fwd_dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "%s: bad dtype", what);
   int kv_rep = 1;
   if (int rc = check_heads(what, hq, hkv, dk, dv, &kv_rep)) return rc;
   if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "%s: scale must be positive", what);
@@ -235,7 +238,7 @@ int nsa_gate_fwd(const void* q, const void* weight, const void* bias, void* gate
                  nsa_stream_t stream) {
   if (!q || !weight || !gates) return fail(NSA_ERR_INVALID, "gate: null pointer");
   if (rows <= 0 || dim <= 0 || dim % 8 != 0) return fail(NSA_ERR_INVALID, "gate: rows must be positive and dim a positive multiple of 8");
-  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "gate: bad dtype");
+  if (!fwd_dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "gate: bad dtype");
   if (!aligned16(q) || !aligned16(weight)) return fail(NSA_ERR_INVALID, "gate: pointers must be 16-byte aligned");
   return finish(nsa::launch_gate(q, weight, bias, gates, (long)rows, dim, dtype, stream), "gate");
 }
@@ -254,7 +257,7 @@ int nsa_gate_bwd(const void* q, const void* weight, const void* d_gates, void* d
 static int gate_combine_common(const char* what, const nsa::GateCombineArgs& a, nsa_stream_t stream) {
   if (!a.gate_logits || !a.o_slc) return fail(NSA_ERR_INVALID, "%s: null pointer", what);
   if (a.rows <= 0 || a.dv <= 0 || a.dv % 8 != 0) return fail(NSA_ERR_INVALID, "%s: rows must be positive and dv a positive multiple of 8", what);
-  if (a.dtype != NSA_BF16 && a.dtype != NSA_F32) return fail(NSA_ERR_INVALID, "%s: bad dtype", what);
+  if (!fwd_dtype_ok(a.dtype)) return fail(NSA_ERR_INVALID, "%s: bad dtype", what);
   if (a.act != NSA_GATE_IDENTITY && a.act != NSA_GATE_SIGMOID) return fail(NSA_ERR_INVALID, "%s: bad gate activation", what);
   const void* ptrs[] = {a.o_slc, a.o_swa, a.o_cmp, a.out, a.d_out, a.d_slc, a.d_swa, a.d_cmp};
   for (const void* p : ptrs)
@@ -286,7 +289,7 @@ int nsa_swa_fwd(const void* q, const void* k, const void* vt, void* o, float* ls
                 nsa_stream_t stream) {
   if (!q || !k || !vt || !o || !cu_seqlens) return fail(NSA_ERR_INVALID, "swa: null pointer");
   if (batch <= 0 || total <= 0 || window <= 0) return fail(NSA_ERR_INVALID, "swa: sizes must be positive");
-  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "swa: bad dtype");
+  if (!fwd_dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "swa: bad dtype");
   int kv_rep = 1;
   if (int rc = check_heads("swa", hq, hkv, dk, dv, &kv_rep)) return rc;
   if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "swa: scale must be positive");
@@ -312,7 +315,7 @@ int nsa_slc_combine_fwd(const void* q, const void* k, const void* vt, const void
                         nsa_stream_t stream) {
   if (!q || !k || !vt || !indices || !out || !cu_seqlens) return fail(NSA_ERR_INVALID, "slc_combine: null pointer");
   if (batch <= 0 || total <= 0) return fail(NSA_ERR_INVALID, "slc_combine: sizes must be positive");
-  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "slc_combine: bad dtype");
+  if (!fwd_dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "slc_combine: bad dtype");
   int kv_rep = 1;
   if (int rc = check_heads("slc_combine", hq, hkv, dk, dv, &kv_rep)) return rc;
   if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "slc_combine: scale must be positive");
@@ -336,7 +339,7 @@ static int slc_common_checks(const char* what, const void* q, const void* k, con
                              int* kv_rep) {
   if (!q || !k || !vt || !cu_seqlens || !workspace) return fail(NSA_ERR_INVALID, "%s: null pointer", what);
   if (batch <= 0 || total <= 0) return fail(NSA_ERR_INVALID, "%s: sizes must be positive", what);
-  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "%s: bad dtype", what);
+  if (!fwd_dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "%s: bad dtype", what);
   if (int rc = check_heads(what, hq, hkv, dk, dv, kv_rep)) return rc;
   if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "%s: scale must be positive", what);
   if (vt_cols % 64 != 0 || vt_cols < nsa_transposed_cols(total, batch)) return fail(NSA_ERR_INVALID, "%s: vt_cols too small or not a multiple of 64", what);

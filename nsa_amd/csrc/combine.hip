@@ -176,6 +176,7 @@ static int gate_combine_t(const GateCombineArgs& a, hipStream_t st) {
 }
 
 int launch_gate_combine(const GateCombineArgs& a, hipStream_t st) {
+  if (a.dtype == 2) return gate_combine_t<f16_t>(a, st);
   return a.dtype == 0 ? gate_combine_t<bf16_t>(a, st) : gate_combine_t<float>(a, st);
 }
 

@@ -20,6 +20,8 @@ namespace nsa {
 
 typedef __bf16 bf16_t;
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16_t;
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef float f32x8_t __attribute__((ext_vector_type(8)));
 
@@ -29,11 +31,15 @@ constexpr float kNegInf = -__builtin_huge_valf();
 
 template <typename T> struct Vec8;
 template <> struct Vec8<bf16_t> { using type = bf16x8_t; };
+template <> struct Vec8<f16_t> { using type = f16x8_t; };
 template <> struct Vec8<float> { using type = f32x8_t; };
 template <typename T> using vec8_t = typename Vec8<T>::type;
 
 __device__ __forceinline__ f32x4_t mma16(bf16x8_t a, bf16x8_t b, f32x4_t c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4_t mma16(f16x8_t a, f16x8_t b, f32x4_t c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
 }
 __device__ __forceinline__ f32x4_t mma16(f32x8_t a, f32x8_t b, f32x4_t c) {
 #pragma unroll
@@ -45,6 +51,9 @@ __device__ __forceinline__ f32x4_t mma16(f32x8_t a, f32x8_t b, f32x4_t c) {
 __device__ __forceinline__ bf16x8_t load8(const bf16_t* p) {
   return *reinterpret_cast<const bf16x8_t*>(p);
 }
+__device__ __forceinline__ f16x8_t load8(const f16_t* p) {
+  return *reinterpret_cast<const f16x8_t*>(p);
+}
 __device__ __forceinline__ f32x8_t load8(const float* p) {
   const f32x4_t a = *reinterpret_cast<const f32x4_t*>(p);
   const f32x4_t b = *reinterpret_cast<const f32x4_t*>(p + 4);
@@ -55,6 +64,9 @@ __device__ __forceinline__ f32x8_t load8(const float* p) {
 }
 __device__ __forceinline__ void store8(bf16_t* p, bf16x8_t v) {
   *reinterpret_cast<bf16x8_t*>(p) = v;
+}
+__device__ __forceinline__ void store8(f16_t* p, f16x8_t v) {
+  *reinterpret_cast<f16x8_t*>(p) = v;
 }
 __device__ __forceinline__ void store8(float* p, f32x8_t v) {
   f32x4_t a, b;

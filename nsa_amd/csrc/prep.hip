@@ -281,6 +281,7 @@ static int launch_compress_t(const CompressArgs& a, hipStream_t st) {
 }
 
 int launch_compress(const CompressArgs& a, hipStream_t st) {
+  if (a.dtype == 2) return launch_compress_t<f16_t>(a, st);
   return a.dtype == 0 ? launch_compress_t<bf16_t>(a, st) : launch_compress_t<float>(a, st);
 }
 
@@ -329,6 +330,9 @@ int launch_gate(const void* x, const void* w, const void* bias, void* out, long 
   if (dtype == 0)
     hipLaunchKernelGGL(gate_kernel<bf16_t>, grid, dim3(256), 0, st, (const bf16_t*)x, (const bf16_t*)w,
                        (const bf16_t*)bias, (bf16_t*)out, rows, dim);
+  else if (dtype == 2)
+    hipLaunchKernelGGL(gate_kernel<f16_t>, grid, dim3(256), 0, st, (const f16_t*)x, (const f16_t*)w,
+                       (const f16_t*)bias, (f16_t*)out, rows, dim);
   else
     hipLaunchKernelGGL(gate_kernel<float>, grid, dim3(256), 0, st, (const float*)x, (const float*)w,
                        (const float*)bias, (float*)out, rows, dim);
@@ -336,6 +340,7 @@ int launch_gate(const void* x, const void* w, const void* bias, void* out, long 
 }
 
 int launch_transpose(const TransposeArgs& a, hipStream_t st) {
+  if (a.dtype == 2) return launch_transpose_t<f16_t>(a, st);
   return a.dtype == 0 ? launch_transpose_t<bf16_t>(a, st) : launch_transpose_t<float>(a, st);
 }
 

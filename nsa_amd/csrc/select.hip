@@ -540,6 +540,15 @@ int launch_select(const CmpArgs& a, hipStream_t st) {
       default: return -2;
     }
   }
+  if (a.dtype == 2) {
+    switch (a.dk) {
+      case 32: return launch_select_t<f16_t, 32>(a, st);
+      case 64: return launch_select_t<f16_t, 64>(a, st);
+      case 128: return launch_select_t<f16_t, 128>(a, st);
+      case 192: return launch_select_t<f16_t, 192>(a, st);
+      default: return -2;
+    }
+  }
   switch (a.dk) {
     case 32: return launch_select_t<float, 32>(a, st);
     case 64: return launch_select_t<float, 64>(a, st);

@@ -49,10 +49,10 @@ long slc_carve(const SlcArgs& a, void* base, SlcWs* ws, size_t elem, int part_wi
 
 static long carve(const SlcArgs& a, void* base, SlcWs* ws, size_t elem) { return slc_carve(a, base, ws, elem, a.dv); }
 
-long slc_workspace_bytes(const SlcArgs& a) { return carve(a, nullptr, nullptr, a.dtype == 0 ? 2 : 4); }
+long slc_workspace_bytes(const SlcArgs& a) { return carve(a, nullptr, nullptr, a.dtype == 1 ? 4 : 2); }
 
 bool slc_block_major_ok(const SlcArgs& a) {
-  return a.dtype == 0 && a.block_size == kBlk && a.top_n <= 64 && a.total < (1 << 26) &&
+  return a.dtype != 1 && a.block_size == kBlk && a.top_n <= 64 && a.total < (1 << 26) &&
          (a.dk == 64 || a.dk == 128 || a.dk == 192) && (a.dv == 64 || a.dv == 128);
 }
 
@@ -420,10 +420,13 @@ static int launch_merge_t(const SlcArgs& a, const SlcWs& ws, hipStream_t st) {
 int launch_slc_partials(const SlcArgs& a, void* workspace, hipStream_t st) {
   SlcWs ws;
   carve(a, workspace, &ws, 2);
-  switch (a.dk * 1000 + a.dv) {
+  switch (a.dk * 1000 + a.dv + (a.dtype == 2 ? 1000000 : 0)) {
     case 64064: return launch_partials_t<bf16_t, 64, 64>(a, ws, st);
     case 128128: return launch_partials_t<bf16_t, 128, 128>(a, ws, st);
     case 192128: return launch_partials_t<bf16_t, 192, 128>(a, ws, st);
+    case 1064064: return launch_partials_t<f16_t, 64, 64>(a, ws, st);
+    case 1128128: return launch_partials_t<f16_t, 128, 128>(a, ws, st);
+    case 1192128: return launch_partials_t<f16_t, 192, 128>(a, ws, st);
     default: return -2;
   }
 }
@@ -439,6 +442,7 @@ int launch_slc_block_major(const SlcArgs& a, void* workspace, hipStream_t st) {
   if (rc) return rc;
   SlcWs ws;
   carve(a, workspace, &ws, 2);
+  if (a.dtype == 2) return a.dv == 64 ? launch_merge_t<f16_t, 64>(a, ws, st) : launch_merge_t<f16_t, 128>(a, ws, st);
   return a.dv == 64 ? launch_merge_t<bf16_t, 64>(a, ws, st) : launch_merge_t<bf16_t, 128>(a, ws, st);
 }
 

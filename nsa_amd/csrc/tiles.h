@@ -73,6 +73,10 @@ __device__ __forceinline__ bf16x8_t load8_tr(const bf16_t* tile, int ld, int lan
   r[4] = b[0]; r[5] = b[1]; r[6] = b[2]; r[7] = b[3];
   return r;
 }
+// fp16: the same instruction (it moves 16-bit lanes whatever they hold)
+__device__ __forceinline__ f16x8_t load8_tr(const f16_t* tile, int ld, int lane) {
+  return __builtin_bit_cast(f16x8_t, load8_tr(reinterpret_cast<const bf16_t*>(tile), ld, lane));
+}
 __device__ __forceinline__ f32x8_t load8_tr(const float* tile, int ld, int lane) {
   const int m = lane & 15, g = lane >> 4;
   f32x8_t r;
@@ -102,6 +106,9 @@ __device__ __forceinline__ bf16x8_t load8_tr32(const bf16_t* tile, int ld, int l
   r[0] = a[0]; r[1] = a[1]; r[2] = a[2]; r[3] = a[3];
   r[4] = b[0]; r[5] = b[1]; r[6] = b[2]; r[7] = b[3];
   return r;
+}
+__device__ __forceinline__ f16x8_t load8_tr32(const f16_t* tile, int ld, int lane) {
+  return __builtin_bit_cast(f16x8_t, load8_tr32(reinterpret_cast<const bf16_t*>(tile), ld, lane));
 }
 __device__ __forceinline__ f32x8_t load8_tr32(const float* tile, int ld, int lane) {
   const int m = lane & 15, g = lane >> 4;
