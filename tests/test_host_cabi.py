@@ -91,6 +91,18 @@ def test_argument_errors_do_not_launch(lib):
     assert rc == -2 and b"block_size" in lib.nsa_last_error_string()
     rc = lib.nsa_compress_fwd(p, None, None, p, p, p, 1, 10, 2, 60, 32, 16, 0, None)
     assert rc == -2
+    # K and V in one call: both weights or neither, dims in pieces of 8, known dtypes (float16 = 2 is one of them
+    # in the forward, not in the backward)
+    rc = lib.nsa_compress_kv_fwd(p, p, p, None, None, None, p, p, p, p, 1, 10, 2, 64, 64, 32, 16, 0, None)
+    assert rc == -1 and b"both weights" in lib.nsa_last_error_string()
+    rc = lib.nsa_compress_kv_fwd(p, p, None, None, None, None, p, None, p, p, 1, 10, 2, 64, 64, 32, 16, 0, None)
+    assert rc == -1 and b"null" in lib.nsa_last_error_string()
+    rc = lib.nsa_compress_kv_fwd(p, p, None, None, None, None, p, p, p, p, 1, 10, 2, 64, 60, 32, 16, 0, None)
+    assert rc == -2
+    rc = lib.nsa_compress_kv_fwd(p, p, None, None, None, None, p, p, p, p, 1, 10, 2, 64, 64, 32, 16, 3, None)
+    assert rc == -1 and b"dtype" in lib.nsa_last_error_string()
+    rc = lib.nsa_compress_bwd(None, None, p, p, None, None, p, p, 1, 64, 3, 1, 64, 32, 16, 2, None)
+    assert rc == -1 and b"dtype" in lib.nsa_last_error_string()
 
 
 def test_python_wrappers_refuse_cpu_tensors_and_missing_library(monkeypatch):
