@@ -187,6 +187,17 @@ def test_backward_argument_errors_do_not_launch(lib):
     assert rc == -1 and b"null" in lib.nsa_last_error_string()
 
 
+def test_float16_is_refused_where_a_graph_would_be_built():
+    from nsa_amd.autograd import needs_grad
+    x = torch.zeros(2, 2, dtype=torch.float16, requires_grad=True)
+    with pytest.raises(NotImplementedError):
+        needs_grad(x)
+    with torch.no_grad():
+        assert not needs_grad(x)
+    assert not needs_grad(x.detach())
+    assert needs_grad(torch.zeros(2, dtype=torch.bfloat16, requires_grad=True))
+
+
 def test_training_path_is_taken_only_when_something_requires_grad():
     from nsa_amd.autograd import needs_grad
     a, b = torch.zeros(2), torch.zeros(2, requires_grad=True)
