@@ -650,6 +650,32 @@ def test_module_randomized_small_shapes():
         _module_case(dtype, lens, G * Hkv, Hkv, D, D, S, W, seed=300 + case, scale_in=0.6, mode=mode, act=act)
 
 
+def test_module_randomized_groups_beyond_16_and_float16():
+    """The same kind of sweep over what came later: GQA groups of 32 / 48 / 64 heads (sub-groups of 16), float16,
+    Dqk 192, batches of many short sequences."""
+    g = torch.Generator().manual_seed(4051)
+
+    def pick(options):
+        return options[int(torch.randint(0, len(options), (1,), generator=g))]
+
+    for case in range(16):
+        nseq = pick([1, 2, 3, 12, 40])
+        lens = [int(torch.randint(1, 500 if nseq < 10 else 120, (1,), generator=g)) for _ in range(nseq)]
+        if case % 5 == 0:
+            lens[0] = pick([1, 32, 33, 63, 64, 65, 129])
+        G = pick([16, 32, 48, 64]) if case % 2 == 0 else pick([4, 8, 16])
+        Hkv = pick([1, 2])
+        Dk, Dv = pick([(64, 64), (128, 128), (192, 128)])
+        S = pick([2, 5, 16])
+        W = pick([1, 64, 200, 512])
+        dtype = torch.float16 if case % 2 == 1 else pick([torch.bfloat16, torch.float16])
+        mode = "conv" if Dk == Dv and pick([0, 1, 1]) == 0 else "mean"
+        act = pick(["sigmoid", "sigmoid", None])
+        print("case", case, lens, G, Hkv, Dk, Dv, S, W, dtype, mode, act)
+        _module_case(dtype, lens, G * Hkv, Hkv, Dk, Dv, S, W, seed=700 + case, scale_in=0.6, mode=mode, act=act,
+                     rows_per_seq=None if sum(lens) <= 1500 else 24)
+
+
 def test_flash_attn_func_api():
     import nsa_amd
     from nsa_amd.compression_kv import KVCompressor
