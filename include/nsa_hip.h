@@ -8,10 +8,9 @@
  *   - tensors are packed ("varlen"): rows of all sequences back to back, `cu_seqlens` int32[batch+1]
  *     with cu_seqlens[0] == 0 holds the row offsets; a batch of equal lengths is the special case
  *     cu_seqlens[b] = b*T
- *   - dtype: NSA_BF16 or NSA_F32 for every floating tensor of a call (accumulation is always fp32); the prefill
- *     forward entry points (compress, transpose, gates, compressed / window / selected attention, block
- *     selection, gated combine) also take NSA_F16, the dtype of the reference's own selection test
- *     (tests/test_parallel_nsa.py:169); backward, decode and rotary entry points refuse it
+ *   - dtype: NSA_BF16, NSA_F16 or NSA_F32 for every floating tensor of a call (accumulation is always fp32).
+ *     NSA_F16 is the dtype of the reference's own selection test (tests/test_parallel_nsa.py:169); every entry
+ *     point takes it.  The 16-bit types share one set of shapes; fp32 lacks a few (stated per entry point)
  *   - GQA: hq / hkv query heads share one kv head.  Groups of 1..16 heads are built everywhere; the prefill
  *     forward entry points (nsa_cmp_attn_*, nsa_block_select_fwd, nsa_swa_fwd, nsa_slc_*, nsa_swa_merge_fwd)
  *     also take groups of 32, 48, 64, ... heads, which is what the reference's selected attention asks for
@@ -224,7 +223,7 @@ int nsa_slc_combine_fwd(const void* q, const void* k, const void* vt, const void
  *                          epilogue: o_slc_out / o_swa_out [total,hq,dv] (ungated branch outputs),
  *                          lse_slc_out / lse_swa_out (float [total,hq], as lse_slc above and lse of
  *                          nsa_swa_fwd).
- * bf16, 64-key selection blocks; other shapes return NSA_ERR_UNSUPPORTED (use nsa_swa_fwd +
+ * bf16 or fp16, 64-key selection blocks; other shapes return NSA_ERR_UNSUPPORTED (use nsa_swa_fwd +
  * nsa_slc_combine_fwd). */
 int nsa_slc_partials_fwd(const void* q, const void* k, const void* vt, const void* indices, const int32_t* counts,
                          const int32_t* cu_seqlens, int batch, int total, int hq, int hkv, int dk, int dv,
@@ -238,7 +237,7 @@ int nsa_swa_merge_fwd(const void* q, const void* k, const void* vt, const void* 
                       const void* workspace, int64_t workspace_bytes, nsa_stream_t stream);
 
 /* Bytes of the optional workspace of nsa_slc_combine_fwd; 0 when the shape has no block-major path
- * (bf16, selection blocks of 64 keys only).  hkv: kv heads, times hq / (16 * hkv) when the GQA group has more
+ * (bf16 or fp16, selection blocks of 64 keys only).  hkv: kv heads, times hq / (16 * hkv) when the GQA group has more
  * than 16 heads (one set of partial results per sub-group of 16 query heads). */
 int64_t nsa_slc_workspace_bytes(int total, int batch, int hkv, int dk, int dv, int top_n, int block_size, int dtype);
 

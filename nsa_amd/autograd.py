@@ -13,13 +13,8 @@ from . import ops
 
 
 def needs_grad(*tensors) -> bool:
-    """True when a call has to build an autograd graph.  The backward kernels take bfloat16 and float32 only:
-    float16 exists in the forward, so such a call is refused here, before any work, rather than in its backward."""
-    need = torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
-    if need and any(t is not None and t.dtype == torch.float16 for t in tensors):
-        raise NotImplementedError("float16 runs in the forward only (wrap the call in torch.no_grad()); "
-                                  "the backward kernels take bfloat16 and float32")
-    return need
+    """True when a call has to build an autograd graph."""
+    return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
 
 
 class CompressFn(torch.autograd.Function):

@@ -93,6 +93,13 @@ __device__ __forceinline__ void store4(bf16_t* p, const f32x4_t& v, float s) {
   for (int i = 0; i < 4; ++i) r[i] = (bf16_t)(v[i] * s);
   *reinterpret_cast<bf16x4v*>(p) = r;
 }
+__device__ __forceinline__ void store4(f16_t* p, const f32x4_t& v, float s) {
+  typedef _Float16 f16x4v __attribute__((ext_vector_type(4)));
+  f16x4v r;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) r[i] = (f16_t)(v[i] * s);
+  *reinterpret_cast<f16x4v*>(p) = r;
+}
 __device__ __forceinline__ void store4(float* p, const f32x4_t& v, float s) {
   f32x4_t r;
 #pragma unroll
@@ -761,7 +768,7 @@ long slc_swa_bwd_workspace_bytes(const SlcSwaBwdArgs& c) {
   take(off, (long)c.total * c.hq * 4);
   take(off, (long)c.total * c.hkv * c.dk * 4);
   take(off, (long)c.total * c.hkv * c.dv * 4);
-  if (c.top_n > 0) off += slc_carve(slc_args_of(c), nullptr, nullptr, c.dtype == 0 ? 2 : 4, c.dk);
+  if (c.top_n > 0) off += slc_carve(slc_args_of(c), nullptr, nullptr, c.dtype == 1 ? 4 : 2, c.dk);
   return off;
 }
 
@@ -834,6 +841,13 @@ static int launch_slc_swa_bwd_t(const SlcSwaBwdArgs& c, hipStream_t st) {
         case 64064: return FN<bf16_t, 64, 64>(ARGS, ST);                              \
         case 128128: return FN<bf16_t, 128, 128>(ARGS, ST);                           \
         case 192128: return FN<bf16_t, 192, 128>(ARGS, ST);                           \
+        default: return -2;                                                           \
+      }                                                                               \
+    } else if ((ARGS).dtype == 2) {                                                   \
+      switch (key) {                                                                  \
+        case 64064: return FN<f16_t, 64, 64>(ARGS, ST);                               \
+        case 128128: return FN<f16_t, 128, 128>(ARGS, ST);                            \
+        case 192128: return FN<f16_t, 192, 128>(ARGS, ST);                            \
         default: return -2;                                                           \
       }                                                                               \
     } else {                                                                          \

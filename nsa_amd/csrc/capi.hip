@@ -59,8 +59,7 @@ int nsa_transposed_cols(int total_rows, int batch) {
   return (need + 63) / 64 * 64;
 }
 
-// Forward prefill entry points take fp16 as well; backward, decode and rotary entry points are bf16 / fp32.
-static bool fwd_dtype_ok(int dtype) { return dtype == NSA_BF16 || dtype == NSA_F32 || dtype == NSA_F16; }
+static bool dtype_ok(int dtype) { return dtype == NSA_BF16 || dtype == NSA_F32 || dtype == NSA_F16; }
 
 int nsa_compress_fwd(const void* x, const void* wt, const void* bias, void* out, const int32_t* cu_seqlens,
                      const int32_t* cu_out, int batch, int out_rows_bound, int heads, int dim, int block,
@@ -68,7 +67,7 @@ int nsa_compress_fwd(const void* x, const void* wt, const void* bias, void* out,
   if (!x || !out || !cu_seqlens || !cu_out) return fail(NSA_ERR_INVALID, "compress: null pointer");
   if (batch <= 0 || heads <= 0 || block <= 0 || stride <= 0 || out_rows_bound < 0)
     return fail(NSA_ERR_INVALID, "compress: sizes must be positive");
-  if (!fwd_dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "compress: bad dtype");
+  if (!dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "compress: bad dtype");
   if (dim % 8 != 0) return fail(NSA_ERR_UNSUPPORTED, "compress: dim must be a multiple of 8");
   if (!aligned16(x) || !aligned16(out) || (wt && !aligned16(wt))) return fail(NSA_ERR_INVALID, "compress: pointers must be 16-byte aligned");
   if (wt && dim % 32 != 0) return fail(NSA_ERR_UNSUPPORTED, "compress: weighted path needs dim %% 32 == 0");
@@ -95,7 +94,7 @@ int nsa_compress_kv_fwd(const void* k, const void* v, const void* wk_t, const vo
   if (!cu_seqlens || !cu_out) return fail(NSA_ERR_INVALID, "compress_kv: null pointer");
   if (batch <= 0 || heads <= 0 || block <= 0 || stride <= 0 || out_rows_bound < 0)
     return fail(NSA_ERR_INVALID, "compress_kv: sizes must be positive");
-  if (!fwd_dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "compress_kv: bad dtype");
+  if (!dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "compress_kv: bad dtype");
   if (dk % 8 != 0 || dv % 8 != 0) return fail(NSA_ERR_UNSUPPORTED, "compress_kv: dims must be multiples of 8");
   if (!aligned16(k) || !aligned16(v) || !aligned16(ck) || !aligned16(cv))
     return fail(NSA_ERR_INVALID, "compress_kv: pointers must be 16-byte aligned");
@@ -112,7 +111,7 @@ int nsa_compress_bwd(const void* x, const void* w_lin, const void* d_out, void* 
   if (dw && !x) return fail(NSA_ERR_INVALID, "compress_bwd: the weight gradient needs x");
   if (batch <= 0 || total <= 0 || heads <= 0 || block <= 0 || stride <= 0 || out_rows_bound < 0)
     return fail(NSA_ERR_INVALID, "compress_bwd: sizes must be positive");
-  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "compress_bwd: bad dtype");
+  if (!dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "compress_bwd: bad dtype");
   if (dim % 8 != 0) return fail(NSA_ERR_UNSUPPORTED, "compress_bwd: dim must be a multiple of 8");
   if (!aligned16(d_out) || !aligned16(dx) || (x && !aligned16(x)) || (w_lin && !aligned16(w_lin)))
     return fail(NSA_ERR_INVALID, "compress_bwd: pointers must be 16-byte aligned");
@@ -130,7 +129,7 @@ int nsa_transpose_fwd(const void* x, void* out, const int32_t* cu, int batch, in
     return fail(NSA_ERR_INVALID, "transpose: dim must be a multiple of 8 and out_cols of 64");
   if (row_stride % 8 != 0 || head_stride % 8 != 0 || !aligned16(x) || !aligned16(out))
     return fail(NSA_ERR_INVALID, "transpose: strides must be multiples of 8 elements, pointers 16-byte aligned");
-  if (!fwd_dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "transpose: bad dtype");
+  if (!dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "transpose: bad dtype");
   nsa::TransposeArgs a{x, out, cu, batch, heads, dim, (long)row_stride, (long)head_stride, out_cols, dtype};
   return finish(nsa::launch_transpose(a, stream), "transpose");
 }
@@ -145,7 +144,7 @@ static int cmp_common(const char* what, int stages, const void* q, const void* c
   if (!q || !ck || !cu_seqlens || !cu_cmp) return fail(NSA_ERR_INVALID, "%s: null pointer", what);
   if (attn && (!cvt || !o)) return fail(NSA_ERR_INVALID, "%s: null pointer", what);
   if (batch <= 0 || total <= 0 || block <= 0 || stride <= 0) return fail(NSA_ERR_INVALID, "%s: sizes must be positive", what);
-  if (!fwd_dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "%s: bad dtype", what);
+  if (!dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "%s: bad dtype", what);
   int kv_rep = 1;
   if (int rc = check_heads(what, hq, hkv, dk, dv, &kv_rep)) return rc;
   if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "%s: scale must be positive", what);
@@ -210,7 +209,7 @@ int nsa_qkv_rope(void* packed, void* q, void* k, void* v, void* gates, const flo
                  int k_off, int v_off, int g_off, int hq, int hkv, int dk, int dv, int rope_off, int rope_dim,
                  int interleaved, int pack, int dtype, nsa_stream_t stream) {
   if (!packed || !q || !k || !v) return fail(NSA_ERR_INVALID, "qkv_rope: null pointer");
-  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "qkv_rope: bad dtype");
+  if (!dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "qkv_rope: bad dtype");
   if (total <= 0 || hq <= 0 || hkv <= 0 || dk <= 0 || dv <= 0 || dk % 8 != 0 || dv % 8 != 0)
     return fail(NSA_ERR_INVALID, "qkv_rope: sizes must be positive and head dims multiples of 8");
   if (ld % 8 != 0 || q_off % 8 != 0 || k_off % 8 != 0 || v_off % 8 != 0 || q_off < 0 || k_off < 0 || v_off < 0 ||
@@ -238,7 +237,7 @@ int nsa_gate_fwd(const void* q, const void* weight, const void* bias, void* gate
                  nsa_stream_t stream) {
   if (!q || !weight || !gates) return fail(NSA_ERR_INVALID, "gate: null pointer");
   if (rows <= 0 || dim <= 0 || dim % 8 != 0) return fail(NSA_ERR_INVALID, "gate: rows must be positive and dim a positive multiple of 8");
-  if (!fwd_dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "gate: bad dtype");
+  if (!dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "gate: bad dtype");
   if (!aligned16(q) || !aligned16(weight)) return fail(NSA_ERR_INVALID, "gate: pointers must be 16-byte aligned");
   return finish(nsa::launch_gate(q, weight, bias, gates, (long)rows, dim, dtype, stream), "gate");
 }
@@ -247,7 +246,7 @@ int nsa_gate_bwd(const void* q, const void* weight, const void* d_gates, void* d
                  int64_t rows, int dim, int dtype, nsa_stream_t stream) {
   if (!q || !weight || !d_gates || !dq || !dweight) return fail(NSA_ERR_INVALID, "gate_bwd: null pointer");
   if (rows <= 0 || dim <= 0 || dim % 8 != 0) return fail(NSA_ERR_INVALID, "gate_bwd: rows must be positive and dim a positive multiple of 8");
-  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "gate_bwd: bad dtype");
+  if (!dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "gate_bwd: bad dtype");
   if (!aligned16(q) || !aligned16(weight) || !aligned16(dq)) return fail(NSA_ERR_INVALID, "gate_bwd: pointers must be 16-byte aligned");
   const int rc = nsa::launch_gate_bwd(q, weight, d_gates, dq, dweight, dbias, (long)rows, dim, dtype, stream);
   if (rc == -2) return fail(NSA_ERR_UNSUPPORTED, "gate_bwd: built for dim 32/64/128/192/256");
@@ -257,7 +256,7 @@ int nsa_gate_bwd(const void* q, const void* weight, const void* d_gates, void* d
 static int gate_combine_common(const char* what, const nsa::GateCombineArgs& a, nsa_stream_t stream) {
   if (!a.gate_logits || !a.o_slc) return fail(NSA_ERR_INVALID, "%s: null pointer", what);
   if (a.rows <= 0 || a.dv <= 0 || a.dv % 8 != 0) return fail(NSA_ERR_INVALID, "%s: rows must be positive and dv a positive multiple of 8", what);
-  if (!fwd_dtype_ok(a.dtype)) return fail(NSA_ERR_INVALID, "%s: bad dtype", what);
+  if (!dtype_ok(a.dtype)) return fail(NSA_ERR_INVALID, "%s: bad dtype", what);
   if (a.act != NSA_GATE_IDENTITY && a.act != NSA_GATE_SIGMOID) return fail(NSA_ERR_INVALID, "%s: bad gate activation", what);
   const void* ptrs[] = {a.o_slc, a.o_swa, a.o_cmp, a.out, a.d_out, a.d_slc, a.d_swa, a.d_cmp};
   for (const void* p : ptrs)
@@ -289,7 +288,7 @@ int nsa_swa_fwd(const void* q, const void* k, const void* vt, void* o, float* ls
                 nsa_stream_t stream) {
   if (!q || !k || !vt || !o || !cu_seqlens) return fail(NSA_ERR_INVALID, "swa: null pointer");
   if (batch <= 0 || total <= 0 || window <= 0) return fail(NSA_ERR_INVALID, "swa: sizes must be positive");
-  if (!fwd_dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "swa: bad dtype");
+  if (!dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "swa: bad dtype");
   int kv_rep = 1;
   if (int rc = check_heads("swa", hq, hkv, dk, dv, &kv_rep)) return rc;
   if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "swa: scale must be positive");
@@ -315,7 +314,7 @@ int nsa_slc_combine_fwd(const void* q, const void* k, const void* vt, const void
                         nsa_stream_t stream) {
   if (!q || !k || !vt || !indices || !out || !cu_seqlens) return fail(NSA_ERR_INVALID, "slc_combine: null pointer");
   if (batch <= 0 || total <= 0) return fail(NSA_ERR_INVALID, "slc_combine: sizes must be positive");
-  if (!fwd_dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "slc_combine: bad dtype");
+  if (!dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "slc_combine: bad dtype");
   int kv_rep = 1;
   if (int rc = check_heads("slc_combine", hq, hkv, dk, dv, &kv_rep)) return rc;
   if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "slc_combine: scale must be positive");
@@ -329,7 +328,7 @@ int nsa_slc_combine_fwd(const void* q, const void* k, const void* vt, const void
                  workspace, (long)workspace_bytes, lse_slc, kv_rep};
   if (workspace && !aligned16(workspace)) return fail(NSA_ERR_INVALID, "slc_combine: workspace must be 16-byte aligned");
   const int rc = nsa::launch_slc_combine(a, stream);
-  if (rc == -5) return fail(NSA_ERR_UNSUPPORTED, "slc_combine: lse_slc needs the block-major schedule (bf16, 64-key blocks, a workspace)");
+  if (rc == -5) return fail(NSA_ERR_UNSUPPORTED, "slc_combine: lse_slc needs the block-major schedule (bf16 or fp16, 64-key blocks, a workspace)");
   return finish(rc, "slc_combine");
 }
 
@@ -339,13 +338,13 @@ static int slc_common_checks(const char* what, const void* q, const void* k, con
                              int* kv_rep) {
   if (!q || !k || !vt || !cu_seqlens || !workspace) return fail(NSA_ERR_INVALID, "%s: null pointer", what);
   if (batch <= 0 || total <= 0) return fail(NSA_ERR_INVALID, "%s: sizes must be positive", what);
-  if (!fwd_dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "%s: bad dtype", what);
+  if (!dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "%s: bad dtype", what);
   if (int rc = check_heads(what, hq, hkv, dk, dv, kv_rep)) return rc;
   if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "%s: scale must be positive", what);
   if (vt_cols % 64 != 0 || vt_cols < nsa_transposed_cols(total, batch)) return fail(NSA_ERR_INVALID, "%s: vt_cols too small or not a multiple of 64", what);
   if (!aligned16(q) || !aligned16(k) || !aligned16(vt) || !aligned16(workspace)) return fail(NSA_ERR_INVALID, "%s: pointers must be 16-byte aligned", what);
   const int64_t need = nsa_slc_workspace_bytes(total, batch, hkv * *kv_rep, dk, dv, top_n, block_size, dtype);
-  if (need == 0) return fail(NSA_ERR_UNSUPPORTED, "%s: the block-major schedule needs bf16, 64-key blocks, top_n <= 64 and (dk,dv) in (64,64),(128,128),(192,128)", what);
+  if (need == 0) return fail(NSA_ERR_UNSUPPORTED, "%s: the block-major schedule needs bf16 or fp16, 64-key blocks, top_n <= 64 and (dk,dv) in (64,64),(128,128),(192,128)", what);
   if (workspace_bytes < need) return fail(NSA_ERR_INVALID, "%s: workspace smaller than nsa_slc_workspace_bytes", what);
   return 0;
 }
@@ -406,7 +405,7 @@ int nsa_cmp_attn_bwd(const void* q, const void* ck, const void* cv, const void* 
   if (cmp_rows > 0 && (!ck || !cv || !dck || !dcv)) return fail(NSA_ERR_INVALID, "cmp_attn_bwd: null pointer");
   if (batch <= 0 || total <= 0 || cmp_rows < 0 || block <= 0 || stride <= 0)
     return fail(NSA_ERR_INVALID, "cmp_attn_bwd: sizes must be positive");
-  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "cmp_attn_bwd: bad dtype");
+  if (!dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "cmp_attn_bwd: bad dtype");
   if (int rc = check_heads("cmp_attn_bwd", hq, hkv, dk, dv)) return rc;
   if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "cmp_attn_bwd: scale must be positive");
   if (!aligned16(q) || !aligned16(ck) || !aligned16(cv) || (o && !aligned16(o)) || !aligned16(d_o) || !aligned16(dq) ||
@@ -446,7 +445,7 @@ int nsa_slc_swa_bwd(const void* q, const void* k, const void* v, const void* o_s
   if (slc && ((!o_slc && !delta_slc) || !lse_slc || !indices || top_n <= 0)) return fail(NSA_ERR_INVALID, "slc_swa_bwd: the selected branch needs o_slc, lse_slc, indices and top_n > 0");
   if (swa && ((!o_swa && !delta_swa) || !lse_swa || window <= 0)) return fail(NSA_ERR_INVALID, "slc_swa_bwd: the sliding branch needs o_swa, lse_swa and window > 0");
   if (batch <= 0 || total <= 0) return fail(NSA_ERR_INVALID, "slc_swa_bwd: sizes must be positive");
-  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "slc_swa_bwd: bad dtype");
+  if (!dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "slc_swa_bwd: bad dtype");
   if (int rc = check_heads("slc_swa_bwd", hq, hkv, dk, dv)) return rc;
   if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "slc_swa_bwd: scale must be positive");
   if (slc && (block_size != 64 || top_n > 64 || total >= (1 << 26)))
@@ -473,7 +472,7 @@ int nsa_decode_append_paged(const void* k_new, const void* v_new, void* k_pool, 
     return fail(NSA_ERR_INVALID, "decode_append_paged: null pointer");
   if (batch <= 0 || hkv <= 0 || dk <= 0 || dv <= 0 || max_pages <= 0 || nc_cap <= 0 || block <= 0 || stride <= 0)
     return fail(NSA_ERR_INVALID, "decode_append_paged: sizes must be positive");
-  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "decode_append_paged: bad dtype");
+  if (!dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "decode_append_paged: bad dtype");
   return finish(nsa::launch_decode_append_paged(k_new, v_new, k_pool, v_pool_t, block_table, max_pages, ck_cache,
                                                 cv_cache_t, pos, batch, hkv, dk, dv, nc_cap, block, stride, dtype,
                                                 stream), "decode_append_paged");
@@ -493,7 +492,7 @@ static int decode_common(const char* what, const void* q, const void* k_cache, c
     return fail(NSA_ERR_INVALID, "%s: null pointer", what);
   if (batch <= 0 || ctx_cap <= 0 || nc_cap <= 0 || block <= 0 || stride <= 0 || window < 0)
     return fail(NSA_ERR_INVALID, "%s: sizes must be positive", what);
-  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "%s: bad dtype", what);
+  if (!dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "%s: bad dtype", what);
   if (int rc = check_heads(what, hq, hkv, dk, dv)) return rc;
   if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "%s: scale must be positive", what);
   if (ctx_cap % 64 != 0 || nc_cap % 64 != 0) return fail(NSA_ERR_INVALID, "%s: cache capacities must be multiples of 64", what);
@@ -614,7 +613,7 @@ int nsa_decode_append(const void* k_new, const void* v_new, void* k_cache, void*
     return fail(NSA_ERR_INVALID, "decode_append: null pointer");
   if (batch <= 0 || hkv <= 0 || dk <= 0 || dv <= 0 || ctx_cap <= 0 || nc_cap <= 0 || block <= 0 || stride <= 0)
     return fail(NSA_ERR_INVALID, "decode_append: sizes must be positive");
-  if (dtype != NSA_BF16 && dtype != NSA_F32) return fail(NSA_ERR_INVALID, "decode_append: bad dtype");
+  if (!dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "decode_append: bad dtype");
   return finish(nsa::launch_decode_append(k_new, v_new, k_cache, v_cache_t, ck_cache, cv_cache_t, pos, batch, hkv, dk,
                                           dv, ctx_cap, nc_cap, block, stride, dtype, stream), "decode_append");
 }

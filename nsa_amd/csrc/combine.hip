@@ -202,6 +202,7 @@ static int gate_bwd_t(const void* q, const void* w, const void* d_gl, void* dq, 
 
 int launch_gate_bwd(const void* q, const void* w, const void* d_gl, void* dq, float* dw, float* db, long rows,
                     int dim, int dtype, hipStream_t st) {
+  if (dtype == 2) return gate_bwd_t<f16_t>(q, w, d_gl, dq, dw, db, rows, dim, st);
   return dtype == 0 ? gate_bwd_t<bf16_t>(q, w, d_gl, dq, dw, db, rows, dim, st)
                     : gate_bwd_t<float>(q, w, d_gl, dq, dw, db, rows, dim, st);
 }

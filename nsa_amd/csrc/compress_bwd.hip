@@ -248,6 +248,7 @@ static int launch_compress_bwd_t(const CompressBwdArgs& a, hipStream_t st) {
 }
 
 int launch_compress_bwd(const CompressBwdArgs& a, hipStream_t st) {
+  if (a.dtype == 2) return launch_compress_bwd_t<f16_t>(a, st);
   return a.dtype == 0 ? launch_compress_bwd_t<bf16_t>(a, st) : launch_compress_bwd_t<float>(a, st);
 }
 

@@ -457,6 +457,14 @@ int launch_decode(const DecodeArgs& a, hipStream_t st) {
       default: return -2;
     }
   }
+  if (a.dtype == 2) {
+    switch (key) {
+      case 64064: return launch_decode_t<f16_t, 64, 64>(a, st);
+      case 128128: return launch_decode_t<f16_t, 128, 128>(a, st);
+      case 192128: return launch_decode_t<f16_t, 192, 128>(a, st);
+      default: return -2;
+    }
+  }
   switch (key) {
     case 64064: return launch_decode_t<float, 64, 64>(a, st);
     case 128128: return launch_decode_t<float, 128, 128>(a, st);
@@ -471,6 +479,10 @@ int launch_decode_append(const void* k_new, const void* v_new, void* k_cache, vo
     hipLaunchKernelGGL(decode_append_kernel<bf16_t>, dim3(batch), dim3(256), 0, st, (const bf16_t*)k_new,
                        (const bf16_t*)v_new, (bf16_t*)k_cache, (bf16_t*)v_cache_t, (bf16_t*)ck_cache,
                        (bf16_t*)cv_cache_t, pos, hkv, dk, dv, ctx_cap, nc_cap, block, stride);
+  else if (dtype == 2)
+    hipLaunchKernelGGL(decode_append_kernel<f16_t>, dim3(batch), dim3(256), 0, st, (const f16_t*)k_new,
+                       (const f16_t*)v_new, (f16_t*)k_cache, (f16_t*)v_cache_t, (f16_t*)ck_cache,
+                       (f16_t*)cv_cache_t, pos, hkv, dk, dv, ctx_cap, nc_cap, block, stride);
   else
     hipLaunchKernelGGL(decode_append_kernel<float>, dim3(batch), dim3(256), 0, st, (const float*)k_new,
                        (const float*)v_new, (float*)k_cache, (float*)v_cache_t, (float*)ck_cache,
@@ -486,6 +498,10 @@ int launch_decode_append_paged(const void* k_new, const void* v_new, void* k_poo
     hipLaunchKernelGGL(decode_append_paged_kernel<bf16_t>, dim3(batch), dim3(256), 0, st, (const bf16_t*)k_new,
                        (const bf16_t*)v_new, (bf16_t*)k_pool, (bf16_t*)v_pool_t, block_table, max_pages,
                        (bf16_t*)ck_cache, (bf16_t*)cv_cache_t, pos, hkv, dk, dv, nc_cap, block, stride);
+  else if (dtype == 2)
+    hipLaunchKernelGGL(decode_append_paged_kernel<f16_t>, dim3(batch), dim3(256), 0, st, (const f16_t*)k_new,
+                       (const f16_t*)v_new, (f16_t*)k_pool, (f16_t*)v_pool_t, block_table, max_pages,
+                       (f16_t*)ck_cache, (f16_t*)cv_cache_t, pos, hkv, dk, dv, nc_cap, block, stride);
   else
     hipLaunchKernelGGL(decode_append_paged_kernel<float>, dim3(batch), dim3(256), 0, st, (const float*)k_new,
                        (const float*)v_new, (float*)k_pool, (float*)v_pool_t, block_table, max_pages,

@@ -578,6 +578,14 @@ int launch_decode_split(const DecodeArgs& a, int splits, void* workspace, hipStr
       default: return -2;
     }
   }
+  if (a.dtype == 2) {
+    switch (key) {
+      case 64064: return launch_decode_split_t<f16_t, 64, 64>(a, splits, ws, st);
+      case 128128: return launch_decode_split_t<f16_t, 128, 128>(a, splits, ws, st);
+      case 192128: return launch_decode_split_t<f16_t, 192, 128>(a, splits, ws, st);
+      default: return -2;
+    }
+  }
   switch (key) {
     case 64064: return launch_decode_split_t<float, 64, 64>(a, splits, ws, st);
     case 128128: return launch_decode_split_t<float, 128, 128>(a, splits, ws, st);

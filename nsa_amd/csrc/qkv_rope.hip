@@ -116,6 +116,7 @@ static int qkv_rope_t(const QkvRopeArgs& a, hipStream_t st) {
 }
 
 int launch_qkv_rope(const QkvRopeArgs& a, hipStream_t st) {
+  if (a.dtype == 2) return qkv_rope_t<f16_t>(a, st);
   return a.dtype == 0 ? qkv_rope_t<bf16_t>(a, st) : qkv_rope_t<float>(a, st);
 }
 

@@ -119,9 +119,9 @@ class NSAAttention(nn.Module):
         if q.shape[1] // k.shape[1] > 16:
             raise NotImplementedError("the NSA backward kernels are built for GQA groups of up to 16 heads; run "
                                       "inference under torch.no_grad()")
-        if q.dtype != torch.bfloat16 or self.selection_block_size != 64:
+        if q.dtype not in (torch.bfloat16, torch.float16) or self.selection_block_size != 64:
             raise NotImplementedError(
-                "the NSA backward kernels are built for bfloat16 and 64-key selection blocks; run inference under "
+                "the NSA backward kernels are built for bfloat16 / float16 and 64-key selection blocks; run inference under "
                 "torch.no_grad() (an input or a parameter of this call requires grad)")
         ck, cv, cu_cmp, nc = self.compressor.compress_packed(k, v, cu, seq_len=seq_len if uniform else None)
         max_nc = nc if nc is not None else conv_compressed_len(seq_len, self.compression_stride,

@@ -16,7 +16,7 @@ def _dtype_code(t: torch.Tensor) -> int:
         return _lib.NSA_BF16
     if t.dtype == torch.float32:
         return _lib.NSA_F32
-    if t.dtype == torch.float16:           # prefill forward only; the library refuses it elsewhere
+    if t.dtype == torch.float16:
         return _lib.NSA_F16
     raise TypeError("NSA kernels take bfloat16, float16 or float32 tensors, got %s" % t.dtype)
 

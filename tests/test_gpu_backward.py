@@ -1,7 +1,8 @@
 """GPU parity of the backward kernels: every gradient comes from the C ABI (nsa_cmp_attn_bwd,
 nsa_slc_swa_bwd, nsa_compress_bwd through the ctypes wrappers and the autograd functions built on them)
 and is compared with autograd through the CPU oracle's forward in float64 on the same seeded inputs.
-Bars: max-abs error <= tol * max(1, max|reference gradient|) with tol 2e-2 for bf16 and 1e-4 for fp32."""
+Bars: max-abs error <= tol * max(1, max|reference gradient|) with tol 2e-2 for bf16, 4e-3 for fp16 and 1e-4
+for fp32."""
 import math
 
 import pytest
@@ -12,7 +13,7 @@ from tests.util import make_qkv, ragged_cu, randn
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
-GTOL = {torch.bfloat16: 2e-2, torch.float32: 1e-4}
+GTOL = {torch.bfloat16: 2e-2, torch.float16: 4e-3, torch.float32: 1e-4}
 
 
 def _ops():
@@ -42,7 +43,7 @@ def _check(name, got, ref, dtype, floor=1.0):
 
 
 # ------------------------------------------------------------------------------ sliding window
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("lens,Hq,Hkv,Dk,Dv,W", [([300], 16, 1, 64, 64, 128), ([257, 40, 130], 32, 2, 128, 128, 100),
                                                  ([200], 16, 1, 192, 128, 64), ([130], 8, 2, 64, 64, 1),
                                                  ([150], 6, 2, 64, 64, 1000),
@@ -78,7 +79,7 @@ def test_swa_bwd(dtype, lens, Hq, Hkv, Dk, Dv, W):
 
 
 # ------------------------------------------------------------------------------ compressed attention
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("lens,Hq,Hkv,Dk,Dv,l,d,causal", [([600], 16, 1, 64, 64, 32, 16, True),
                                                           ([1300, 20, 333], 32, 2, 128, 128, 32, 16, True),
                                                           ([2500], 16, 1, 192, 128, 32, 16, True),
@@ -140,8 +141,9 @@ def _random_indices(T, Hkv, S, bs, seed):
 @pytest.mark.parametrize("lens,Hq,Hkv,Dk,Dv,S,W", [([384], 16, 1, 64, 64, 4, 0), ([512, 100], 32, 2, 128, 128, 8, 100),
                                                   ([330], 16, 1, 192, 128, 3, 64), ([700, 130], 24, 2, 64, 64, 16, 0),
                                                   ([200], 4, 1, 64, 64, 2, 32)])
-def test_slc_swa_bwd(lens, Hq, Hkv, Dk, Dv, S, W):
-    dtype, bs = torch.bfloat16, 64
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_slc_swa_bwd(lens, Hq, Hkv, Dk, Dv, S, W, dtype):
+    bs = 64
     ops = _ops()
     T = sum(lens)
     q, k, v, _ = make_qkv(T, Hq, Hkv, Dk, Dv, 170, dtype, 0.7)
@@ -181,7 +183,7 @@ def test_slc_swa_bwd(lens, Hq, Hkv, Dk, Dv, S, W):
 
 
 # ------------------------------------------------------------------------------ compression
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("S,W", [(16, 100), (4, 0), (0, 64)])
 def test_slc_swa_bwd_dq_add(dtype, S, W):
     """dq_add is summed into dq by the kernel that writes it: dk / dv unchanged, dq = plain result + dq_add (to
@@ -209,7 +211,7 @@ def test_slc_swa_bwd_dq_add(dtype, S, W):
             len(lens), bs, W, scale)
     dq0, dk0, dv0 = ops.slc_swa_bwd(*args)
     dq1, dk1, dv1 = ops.slc_swa_bwd(*args, dq_add=extra)
-    tol = 2.0 ** -7 if dtype == torch.bfloat16 else 1e-5
+    tol = {torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -10, torch.float32: 1e-5}[dtype]
     for a, b in ((dk0, dk1), (dv0, dv1)):      # fp32 atomics: the order of the sums differs from run to run
         assert float((a.double() - b.double()).abs().max()) <= tol * max(1.0, float(a.abs().max()))
     ref = dq0.double() + extra.double()
@@ -220,7 +222,7 @@ def test_slc_swa_bwd_dq_add(dtype, S, W):
         ops.slc_swa_bwd(*args, dq_add=extra[:, :, :32])
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("lens,H,D,l,d", [([300], 1, 64, 32, 16), ([300, 31, 64, 1000], 4, 128, 32, 16),
                                           ([200, 77], 2, 192, 64, 16), ([90], 2, 32, 8, 4)])
 def test_compress_mean_bwd(dtype, lens, H, D, l, d):
@@ -241,7 +243,7 @@ def test_compress_mean_bwd(dtype, lens, H, D, l, d):
         _check("dx", dx[s:e], rx, dtype)
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("lens,H,D,l,d,extra", [([256, 100], 2, 64, 32, 16, 1), ([1024] * 2, 2, 128, 64, 16, 0),
                                                 ([90, 7], 1, 32, 8, 4, 1), ([700], 4, 192, 32, 16, 1)])
 def test_compress_weighted_bwd(dtype, lens, H, D, l, d, extra):
@@ -278,11 +280,10 @@ def _leaf(t):
     return t.to(DEV).requires_grad_(True)
 
 
-def _module_backward_case(mode, lens, Hq, Hkv, Dk, Dv, act, S=4, W=64, seed=190):
+def _module_backward_case(mode, lens, Hq, Hkv, Dk, Dv, act, S=4, W=64, seed=190, dtype=torch.bfloat16):
     """NSAAttention end to end: gradients of every input and parameter against autograd through the
     oracle forward (float64, the module's own block picks forced so that score ties cannot differ)."""
     from nsa_amd.nsa import NSAAttention
-    dtype = torch.bfloat16
     T = sum(lens)
     p = O.NSAParams(block=32, stride=16, sel_block=64, top_n=S, window=W, scale=1.0 / math.sqrt(Dk))
     torch.manual_seed(5)
@@ -345,6 +346,15 @@ def test_module_backward(mode, lens, Hq, Hkv, Dk, Dv, act):
     _module_backward_case(mode, lens, Hq, Hkv, Dk, Dv, act)
 
 
+@pytest.mark.parametrize("mode,lens,Hq,Hkv,Dk,Dv,act", [("mean", [300, 200, 40], 32, 2, 128, 128, "sigmoid"),
+                                                        ("conv", [500], 16, 1, 64, 64, None),
+                                                        ("mean", [400], 16, 1, 192, 128, "sigmoid")])
+def test_module_backward_float16(mode, lens, Hq, Hkv, Dk, Dv, act):
+    """float16, the dtype of the reference's own selection test (tests/test_parallel_nsa.py:169), through
+    every backward kernel."""
+    _module_backward_case(mode, lens, Hq, Hkv, Dk, Dv, act, dtype=torch.float16)
+
+
 def test_module_backward_randomized_small_shapes():
     """Seeded sweep over ragged lengths (down to a single token and sequences without any compressed row),
     group sizes 1..16, top-n, window, both compressors and both gate conventions."""
@@ -384,11 +394,12 @@ def test_module_no_grad_path_unchanged():
     assert float((a.float() - b.detach().float()).abs().max()) <= 2e-2
 
 
-def test_parallel_nsa_and_flash_attn_backward():
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_parallel_nsa_and_flash_attn_backward(dtype):
     """The two functional entry points with the reference's tensor layouts ([B,T,H,D], head-repeated
     compressed keys): gradients of q, k, v and the gates."""
     import nsa_amd
-    dtype, B, T, Hq, Hkv, D, S, W, bs = torch.bfloat16, 2, 256, 32, 2, 64, 3, 32, 64
+    B, T, Hq, Hkv, D, S, W, bs = 2, 256, 32, 2, 64, 3, 32, 64
     scale = 1.0 / math.sqrt(D)
     q = randn(B, T, Hq, D, seed=200, scale=0.7, dtype=dtype)
     k = randn(B, T, Hkv, D, seed=201, scale=0.7, dtype=dtype)
@@ -460,7 +471,7 @@ def test_compress_kv_backward():
         _check("dw", w.grad, wr.grad, dtype)
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("T,Hq,D,Dv,act", [(300, 16, 64, 64, 1), (257, 6, 192, 128, 0), (64, 4, 128, 128, 1)])
 def test_gate_and_combine_kernels(dtype, T, Hq, D, Dv, act):
     """nsa_gate_combine_fwd / _bwd and nsa_gate_bwd against the same arithmetic in torch float64."""

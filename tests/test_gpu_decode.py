@@ -66,7 +66,7 @@ SCHEDULES = [None, 0]      # chosen from the batch (split for small batches) / o
 
 
 @pytest.mark.parametrize("splits", SCHEDULES)
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 def test_decode_small_ragged_contexts(dtype, splits):
     _check(dtype, [1024, 1000, 513, 64, 40, 33, 20, 1], 64, 4, 128, 128, 4, 128, seed=100, splits=splits)
 
@@ -78,8 +78,9 @@ def test_decode_gqa4_d64(dtype, splits):
 
 
 @pytest.mark.parametrize("splits", SCHEDULES)
-def test_decode_dqk192(splits):
-    _check(torch.bfloat16, [2048, 1536], 32, 2, 192, 128, 16, 512, seed=120, splits=splits)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_decode_dqk192(splits, dtype):
+    _check(dtype, [2048, 1536], 32, 2, 192, 128, 16, 512, seed=120, splits=splits)
 
 
 @pytest.mark.parametrize("splits", SCHEDULES)
@@ -98,6 +99,7 @@ def test_decode_cfg5_full_batch_default_dispatch():
 @pytest.mark.parametrize("dtype,Hq,Hkv,Dk,Dv,S,W", [
     (torch.bfloat16, 64, 4, 128, 128, 16, 512),
     (torch.bfloat16, 32, 2, 192, 128, 4, 128),
+    (torch.float16, 32, 2, 128, 128, 8, 100),
     (torch.float32, 8, 2, 64, 64, 4, 64),
 ])
 def test_paged_decode_against_oracle(dtype, Hq, Hkv, Dk, Dv, S, W, splits):

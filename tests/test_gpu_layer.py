@@ -29,7 +29,7 @@ def _layout(hq, hkv, dk, dv, lead=0, gap=8):
     return (q_off, k_off, v_off, g_off), ld
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("hq,hkv,dk,dv,off,rd,inter,explicit", [
     (64, 4, 192, 128, 128, 64, False, False),
     (8, 2, 64, 64, 0, 64, False, True),
@@ -63,7 +63,8 @@ def test_qkv_rope_split_matches_oracle(dtype, hq, hkv, dk, dv, off, rd, inter, e
         keep[off:off + rd] = False
         assert torch.equal(got[..., keep], src[..., keep])                       # content channels: a copy
         err = (got.double() - want.double()).abs()
-        bound = 1e-5 if dtype == torch.float32 else want.double().abs() * 2.0 ** -8 + 1e-6   # one rounding
+        ulp = 2.0 ** (-8 if dtype == torch.bfloat16 else -11)
+        bound = 1e-5 if dtype == torch.float32 else want.double().abs() * ulp + 1e-6        # one rounding
         assert bool((err <= bound).all()), float(err.max())
 
 

@@ -721,9 +721,6 @@ def test_error_paths():
         ops.swa(q, k, vt, cu, 1, 16, 0.1)
     with pytest.raises(TypeError):
         ops.swa(q.double(), k.double(), vt, cu, 1, 16, 0.1)
-    with pytest.raises(ValueError):                                   # float16 exists in the prefill forward only
-        ops.compress_bwd(torch.zeros(3, 1, 64, dtype=torch.float16, device=DEV), cu,
-                         torch.tensor([0, 3], dtype=torch.int32, device=DEV), 64, 32, 16)
     with pytest.raises(ValueError):
         ops.swa(q[:, :4].contiguous(), k, vt, cu, 1, 16, -1.0)
     with pytest.raises(RuntimeError):

@@ -91,8 +91,7 @@ def test_argument_errors_do_not_launch(lib):
     assert rc == -2 and b"block_size" in lib.nsa_last_error_string()
     rc = lib.nsa_compress_fwd(p, None, None, p, p, p, 1, 10, 2, 60, 32, 16, 0, None)
     assert rc == -2
-    # K and V in one call: both weights or neither, dims in pieces of 8, known dtypes (float16 = 2 is one of them
-    # in the forward, not in the backward)
+    # K and V in one call: both weights or neither, dims in pieces of 8, known dtypes (0, 1, 2)
     rc = lib.nsa_compress_kv_fwd(p, p, p, None, None, None, p, p, p, p, 1, 10, 2, 64, 64, 32, 16, 0, None)
     assert rc == -1 and b"both weights" in lib.nsa_last_error_string()
     rc = lib.nsa_compress_kv_fwd(p, p, None, None, None, None, p, None, p, p, 1, 10, 2, 64, 64, 32, 16, 0, None)
@@ -101,7 +100,7 @@ def test_argument_errors_do_not_launch(lib):
     assert rc == -2
     rc = lib.nsa_compress_kv_fwd(p, p, None, None, None, None, p, p, p, p, 1, 10, 2, 64, 64, 32, 16, 3, None)
     assert rc == -1 and b"dtype" in lib.nsa_last_error_string()
-    rc = lib.nsa_compress_bwd(None, None, p, p, None, None, p, p, 1, 64, 3, 1, 64, 32, 16, 2, None)
+    rc = lib.nsa_compress_bwd(None, None, p, p, None, None, p, p, 1, 64, 3, 1, 64, 32, 16, 3, None)
     assert rc == -1 and b"dtype" in lib.nsa_last_error_string()
 
 
@@ -187,15 +186,14 @@ def test_backward_argument_errors_do_not_launch(lib):
     assert rc == -1 and b"null" in lib.nsa_last_error_string()
 
 
-def test_float16_is_refused_where_a_graph_would_be_built():
+def test_needs_grad_follows_the_grad_mode():
     from nsa_amd.autograd import needs_grad
-    x = torch.zeros(2, 2, dtype=torch.float16, requires_grad=True)
-    with pytest.raises(NotImplementedError):
-        needs_grad(x)
-    with torch.no_grad():
-        assert not needs_grad(x)
-    assert not needs_grad(x.detach())
-    assert needs_grad(torch.zeros(2, dtype=torch.bfloat16, requires_grad=True))
+    for dtype in (torch.float16, torch.bfloat16, torch.float32):
+        x = torch.zeros(2, 2, dtype=dtype, requires_grad=True)
+        assert needs_grad(None, x)
+        with torch.no_grad():
+            assert not needs_grad(x)
+        assert not needs_grad(x.detach(), None)
 
 
 def test_training_path_is_taken_only_when_something_requires_grad():
