@@ -15,7 +15,9 @@
  *     forward entry points (nsa_cmp_attn_*, nsa_block_select_fwd, nsa_swa_fwd, nsa_slc_*, nsa_swa_merge_fwd)
  *     also take groups of 32, 48, 64, ... heads, which is what the reference's selected attention asks for
  *     (HQ a multiple of 16 * H, nsa/selection_attn.py:800): they run as hq / (16 * hkv) sub-groups of 16 heads
- *     that share the keys, values and block picks of their kv head.  Backward and decode: groups up to 16.
+ *     that share the keys, values and block picks of their kv head.  Backward and decode: groups up to 16 (a
+ *     caller runs the backward of a larger group as one call per sub-group of 16 heads and adds the key / value
+ *     gradients, as nsa_amd/ops.py does).
  *   - return value: 0 on success, negative on error (NSA_ERR_*); nsa_last_error_string() describes
  *     the last error of the calling thread.  No exception crosses this boundary.
  *   - "transposed" buffers hold one key-contiguous plane per head: element (h, d, col) lives at

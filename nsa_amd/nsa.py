@@ -116,9 +116,9 @@ class NSAAttention(nn.Module):
                                        return_indices)
 
     def _forward_train(self, q, k, v, cu, batch, scale, causal, seq_len, uniform, gates, return_indices):
-        if q.shape[1] // k.shape[1] > 16:
-            raise NotImplementedError("the NSA backward kernels are built for GQA groups of up to 16 heads; run "
-                                      "inference under torch.no_grad()")
+        if q.shape[1] // k.shape[1] > 16 and (q.shape[1] // k.shape[1]) % 16:
+            raise NotImplementedError("the NSA backward runs GQA groups of up to 16 heads and multiples of 16 "
+                                      "heads; run inference under torch.no_grad()")
         if q.dtype not in (torch.bfloat16, torch.float16) or self.selection_block_size != 64:
             raise NotImplementedError(
                 "the NSA backward kernels are built for bfloat16 / float16 and 64-key selection blocks; run inference under "

@@ -361,6 +361,14 @@ def gate_logits(q, weight, bias=None):
     return out
 
 
+def _subgroup(t, hkv, rep, r):
+    """Heads of sub-group r (16 of the rep * 16 query heads of every kv head) of a [total, Hq, ...] tensor, as a
+    contiguous [total, hkv * 16, ...] tensor."""
+    if t is None:
+        return None
+    return t.reshape(t.shape[0], hkv, rep, 16, *t.shape[2:])[:, :, r].reshape(t.shape[0], hkv * 16, *t.shape[2:]).contiguous()
+
+
 def cmp_attn_bwd(q, ck, cv, o, d_o, lse_attn, cu_seqlens, cu_cmp, batch, block, stride, scale, causal=True,
                  delta=None, rowscale=None):
     """Backward of the compressed attention.  q [total,Hq,Dk], ck [rows,Hkv,Dk], cv [rows,Hkv,Dv]
@@ -368,6 +376,23 @@ def cmp_attn_bwd(q, ck, cv, o, d_o, lse_attn, cu_seqlens, cu_cmp, batch, block, 
     delta (float32 [total,Hq]) = rowsum(o*d_o) if already known (o may then be None); rowscale (float32
     [total,Hq]) = a per-row gate applied to d_o inside the kernels.  Returns (dq, dck, dcv)."""
     _need_cuda(q, ck, cv, d_o, lse_attn, cu_seqlens, cu_cmp)
+    rep = head_subgroups(q.shape[1], cv.shape[1])
+    if rep > 1:
+        # groups of 32, 48, 64 ... heads: one call per sub-group of 16 heads (they share ck / cv, so the key
+        # gradients of the calls add up; summed in float32, rounded once)
+        hkv = cv.shape[1]
+        dq = torch.empty_like(q).view(q.shape[0], hkv, rep, 16, q.shape[2])
+        dck = torch.zeros(ck.shape, dtype=torch.float32, device=q.device)
+        dcv = torch.zeros(cv.shape, dtype=torch.float32, device=q.device)
+        for r in range(rep):
+            part = cmp_attn_bwd(_subgroup(q, hkv, rep, r), ck, cv, _subgroup(o, hkv, rep, r), _subgroup(d_o, hkv, rep, r),
+                                _subgroup(lse_attn, hkv, rep, r), cu_seqlens, cu_cmp, batch, block, stride, scale,
+                                causal=causal, delta=_subgroup(delta, hkv, rep, r),
+                                rowscale=_subgroup(rowscale, hkv, rep, r))
+            dq[:, :, r] = part[0].view(q.shape[0], hkv, 16, q.shape[2])
+            dck += part[1]
+            dcv += part[2]
+        return dq.view(q.shape), dck.to(ck.dtype), dcv.to(cv.dtype)
     q, ck, cv, d_o = (_dense(t) for t in (q, ck, cv, d_o))
     o = None if o is None else _dense(o)
     total, hq, dk = q.shape
@@ -393,6 +418,23 @@ def slc_swa_bwd(q, k, v, o_slc, d_o_slc, lse_slc, o_swa, d_o_swa, lse_swa, indic
     by the kernel that writes it (the compressed branch's dq).  Returns (dq, dk, dv), each the sum over
     the branches given."""
     _need_cuda(q, k, v, cu_seqlens)
+    rep = head_subgroups(q.shape[1], v.shape[1])
+    if rep > 1:
+        hkv = v.shape[1]
+        sub = lambda t, r: _subgroup(t, hkv, rep, r)     # noqa: E731
+        dq = torch.empty_like(q).view(q.shape[0], hkv, rep, 16, q.shape[2])
+        dk_sum = torch.zeros(k.shape, dtype=torch.float32, device=q.device)
+        dv_sum = torch.zeros(v.shape, dtype=torch.float32, device=q.device)
+        for r in range(rep):
+            part = slc_swa_bwd(sub(q, r), k, v, sub(o_slc, r), sub(d_o_slc, r), sub(lse_slc, r), sub(o_swa, r),
+                               sub(d_o_swa, r), sub(lse_swa, r), indices, counts, cu_seqlens, batch, block_size, window,
+                               scale, delta_slc=sub(delta_slc, r), delta_swa=sub(delta_swa, r),
+                               rowscale_slc=sub(rowscale_slc, r), rowscale_swa=sub(rowscale_swa, r),
+                               dq_add=sub(dq_add, r))
+            dq[:, :, r] = part[0].view(q.shape[0], hkv, 16, q.shape[2])
+            dk_sum += part[1]
+            dv_sum += part[2]
+        return dq.view(q.shape), dk_sum.to(k.dtype), dv_sum.to(v.dtype)
     q, k, v = _dense(q), _dense(k), _dense(v)
     total, hq, dk = q.shape
     hkv, dv = v.shape[1], v.shape[2]

@@ -56,7 +56,8 @@ def parallel_nsa(q: torch.Tensor,
     q [B,T,HQ,K], k [B,T,H,K], v [B,T,H,V], g_* [B,T,HQ], block_indices [B,T,H,S] (block numbers
     local to the sequence), block_counts None | int | [B,T,H]; head_first swaps dims 1 and 2.
     With cu_seqlens (B must be 1) the tensors are packed sequences.  GQA groups of 1..16 heads and of 32, 48,
-    64, ... heads run (the reference takes multiples of 16 only); the backward exists for groups up to 16.
+    64, ... heads run (the reference takes multiples of 16 only); the backward of a group beyond 16 heads runs as
+    one call per sub-group of 16 heads.
     A count tensor limits the picks of a (token, head) in the forward as well, which the reference's forward
     kernel does too (nsa/selection_attn.py:431-434)."""
     if scale is None:
@@ -81,8 +82,6 @@ def parallel_nsa(q: torch.Tensor,
     counts = None if block_counts is None else block_counts.reshape(B * T, H)
     idx = block_indices.reshape(B * T, H, -1)
     if needs_grad(q, k, v, g_slc, g_swa):
-        if HQ // H > 16:
-            raise NotImplementedError("the backward kernels are built for GQA groups of up to 16 heads")
         o_slc, o_swa = SlcSwaFn.apply(qp, kp, vp, idx, counts, cu, nb, block_size, window_size, float(scale))
         gs = g_slc.reshape(B * T, HQ).to(q.dtype)
         gw = g_swa.reshape(B * T, HQ).to(q.dtype) if o_swa is not None else torch.zeros_like(gs)

@@ -355,6 +355,15 @@ def test_module_backward_float16(mode, lens, Hq, Hkv, Dk, Dv, act):
     _module_backward_case(mode, lens, Hq, Hkv, Dk, Dv, act, dtype=torch.float16)
 
 
+@pytest.mark.parametrize("mode,lens,Hq,Hkv,Dk,Dv,act", [("mean", [300, 120], 32, 1, 64, 64, "sigmoid"),
+                                                        ("conv", [260], 96, 2, 128, 128, None),
+                                                        ("mean", [200], 64, 1, 192, 128, "sigmoid")])
+def test_module_backward_groups_of_32_48_64_heads(mode, lens, Hq, Hkv, Dk, Dv, act):
+    """What the reference's HQ % (16 * H) == 0 admits beyond 16 heads (nsa/selection_attn.py:800): the backward runs
+    one call per sub-group of 16 heads, the key / value gradients of the sub-groups add up."""
+    _module_backward_case(mode, lens, Hq, Hkv, Dk, Dv, act)
+
+
 def test_module_backward_randomized_small_shapes():
     """Seeded sweep over ragged lengths (down to a single token and sequences without any compressed row),
     group sizes 1..16, top-n, window, both compressors and both gate conventions."""
@@ -394,12 +403,12 @@ def test_module_no_grad_path_unchanged():
     assert float((a.float() - b.detach().float()).abs().max()) <= 2e-2
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_parallel_nsa_and_flash_attn_backward(dtype):
+@pytest.mark.parametrize("dtype,Hkv", [(torch.bfloat16, 2), (torch.float16, 2), (torch.bfloat16, 1)])
+def test_parallel_nsa_and_flash_attn_backward(dtype, Hkv):
     """The two functional entry points with the reference's tensor layouts ([B,T,H,D], head-repeated
-    compressed keys): gradients of q, k, v and the gates."""
+    compressed keys): gradients of q, k, v and the gates.  Hkv 1 = a GQA group of 32 heads."""
     import nsa_amd
-    B, T, Hq, Hkv, D, S, W, bs = 2, 256, 32, 2, 64, 3, 32, 64
+    B, T, Hq, D, S, W, bs = 2, 256, 32, 64, 3, 32, 64
     scale = 1.0 / math.sqrt(D)
     q = randn(B, T, Hq, D, seed=200, scale=0.7, dtype=dtype)
     k = randn(B, T, Hkv, D, seed=201, scale=0.7, dtype=dtype)
