@@ -225,7 +225,9 @@ int nsa_slc_combine_fwd(const void* q, const void* k, const void* vt, const void
  *                          epilogue: o_slc_out / o_swa_out [total,hq,dv] (ungated branch outputs),
  *                          lse_slc_out / lse_swa_out (float [total,hq], as lse_slc above and lse of
  *                          nsa_swa_fwd).
- * bf16 or fp16, 64-key selection blocks; other shapes return NSA_ERR_UNSUPPORTED (use nsa_swa_fwd +
+ * bf16 or fp16; selection blocks of 8, 16, 32 or a multiple of 64 keys, top_n * max(1, block_size / 64) <= 64 (the schedule works on 64-key
+ * blocks: a smaller selection block is a masked part of one, a larger one takes several slots per pick); other
+ * shapes return NSA_ERR_UNSUPPORTED (use nsa_swa_fwd +
  * nsa_slc_combine_fwd). */
 int nsa_slc_partials_fwd(const void* q, const void* k, const void* vt, const void* indices, const int32_t* counts,
                          const int32_t* cu_seqlens, int batch, int total, int hq, int hkv, int dk, int dv,
@@ -239,7 +241,7 @@ int nsa_swa_merge_fwd(const void* q, const void* k, const void* vt, const void* 
                       const void* workspace, int64_t workspace_bytes, nsa_stream_t stream);
 
 /* Bytes of the optional workspace of nsa_slc_combine_fwd; 0 when the shape has no block-major path
- * (bf16 or fp16, selection blocks of 64 keys only).  hkv: kv heads, times hq / (16 * hkv) when the GQA group has more
+ * (bf16 or fp16; selection blocks of 8, 16, 32 or a multiple of 64 keys, top_n * max(1, block_size / 64) <= 64).  hkv: kv heads, times hq / (16 * hkv) when the GQA group has more
  * than 16 heads (one set of partial results per sub-group of 16 query heads). */
 int64_t nsa_slc_workspace_bytes(int total, int batch, int hkv, int dk, int dv, int top_n, int block_size, int dtype);
 
@@ -267,7 +269,7 @@ int nsa_cmp_attn_bwd(const void* q, const void* ck, const void* cv, const void* 
  *   o_slc / d_o_slc / lse_slc: ungated output of the selected branch, its gradient, and lse_slc of
  *   nsa_slc_combine_fwd; o_swa / d_o_swa / lse_swa likewise for the window (lse of nsa_swa_fwd).
  *   A branch is skipped when its d_o is NULL.  indices / counts / idx64 / top_n / block_size as in
- *   nsa_slc_combine_fwd (64-key blocks only).  dq [total,hq,dk], dk_out [total,hkv,dk], dv_out
+ *   nsa_slc_combine_fwd (selection blocks of 8, 16, 32 or a multiple of 64 keys, top_n * max(1, block_size / 64) <= 64).  dq [total,hq,dk], dk_out [total,hkv,dk], dv_out
  *   [total,hkv,dv] receive the sums over the branches present and are fully overwritten.
  *   delta_* / rowscale_* (optional, float [total,hq]) as in nsa_cmp_attn_bwd, per branch.
  *   dq_add (optional, [total,hq,dk], must not overlap dq): added to dq in the kernel that writes it, e.g. the

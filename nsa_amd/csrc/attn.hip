@@ -703,9 +703,11 @@ int launch_swa(const SwaArgs& a, hipStream_t st) { NSA_DISPATCH(launch_swa_t, a,
 int launch_swa_merge(const SwaArgs& a, const MergeArgs& m, hipStream_t st) {
   if (a.dtype == 1) return -2;             // the partials are 16-bit
   switch (a.dk * 1000 + a.dv + (a.dtype == 2 ? 1000000 : 0)) {
+    case 32032: return launch_swa_merge_t<bf16_t, 32, 32>(a, m, st);
     case 64064: return launch_swa_merge_t<bf16_t, 64, 64>(a, m, st);
     case 128128: return launch_swa_merge_t<bf16_t, 128, 128>(a, m, st);
     case 192128: return launch_swa_merge_t<bf16_t, 192, 128>(a, m, st);
+    case 1032032: return launch_swa_merge_t<f16_t, 32, 32>(a, m, st);
     case 1064064: return launch_swa_merge_t<f16_t, 64, 64>(a, m, st);
     case 1128128: return launch_swa_merge_t<f16_t, 128, 128>(a, m, st);
     case 1192128: return launch_swa_merge_t<f16_t, 192, 128>(a, m, st);

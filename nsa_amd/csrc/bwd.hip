@@ -55,6 +55,8 @@ struct BwdArgs {
   void* dq;                       // query-stationary: [total][hq][dk]
   float* dk_acc; float* dv_acc;   // key-stationary: fp32 [key rows][hkv][.]
   SlcWs ws;                       // selected branch: bucketed pairs; ws.po = dq partials [pair][16][dk]
+  int slc_width;                  // selected branch: keys of a 64-key block one pair attends (the selection block
+                                  // size when that is below 64, where ws.sub holds the pair's first key)
   int tiles, items;               // key-stationary launch: key tiles, token items (compressed branch)
 };
 
@@ -195,6 +197,9 @@ bwd_kv_kernel(const BwdArgs a) {
   const T* dob = reinterpret_cast<const T*>(a.d_o);
 
   // tokens of chunk c: positions inside the sequence (pos*), validity of the second one
+  // selected branch, selection blocks below 64 keys: a pair sees keys [sub, sub + slc_width) of the block
+  const bool parts = MODE == kBwdSlc && a.slc_width < kBlk;
+  int subA = 0, subB = 0, nsubA = 0, nsubB = 0;
   auto chunk_tokens = [&](int c, int& posA, int& posB, bool& vB) {
     if (MODE == kBwdSlc) {
       posA = (int)(a.ws.list[first + 2 * c] >> 6) - seq_start;
@@ -294,8 +299,9 @@ bwd_kv_kernel(const BwdArgs a) {
   // selected mode: even lanes read the pair-list entry of a chunk's first token, odd lanes that of its second
   // (the first again when the chunk has one), as one load whose value is only split into the two positions
   // where they are used: a load from a wave-uniform address would be waited for where it is issued.
-  unsigned aftv = 0;
+  unsigned aftv = 0, afts = 0;
   auto list_entry = [&](int c) { return a.ws.list[first + min(2 * c + (lane & 1), count - 1)]; };
+  auto sub_entry = [&](int c) { return (unsigned)a.ws.sub[first + min(2 * c + (lane & 1), count - 1)]; };
   auto list_split = [&](unsigned v, int c, int& pA, int& pB, bool& vb) {
     pA = (int)(__builtin_amdgcn_readlane(v, 0) >> 6) - seq_start;
     pB = (int)(__builtin_amdgcn_readlane(v, 1) >> 6) - seq_start;
@@ -304,6 +310,13 @@ bwd_kv_kernel(const BwdArgs a) {
   chunk_tokens(0, posA, posB, vB);
   if (nchunks > 1) chunk_tokens(1, nxtA, nxtB, nxtV);
   if (MODE == kBwdSlc && nchunks > 2) aftv = list_entry(2);
+  if (parts) {
+    subA = a.ws.sub[first];
+    subB = a.ws.sub[first + min(1, count - 1)];
+    nsubA = a.ws.sub[first + min(2, count - 1)];
+    nsubB = a.ws.sub[first + min(3, count - 1)];
+    if (nchunks > 2) afts = sub_entry(2);
+  }
   gload(posA, posB);
   lstore(0);
   __syncthreads();
@@ -322,7 +335,10 @@ bwd_kv_kernel(const BwdArgs a) {
     const int tokpos = (g >> 1) ? posB : posA;
     bool vis = keyvalid && ((g >> 1) == 0 || vB);
     if (MODE == kBwdSwa) vis = vis && keypos <= tokpos && keypos > tokpos - a.window;
-    else if (MODE == kBwdSlc) vis = vis && keypos <= tokpos;
+    else if (MODE == kBwdSlc) {
+      vis = vis && keypos <= tokpos;
+      if (parts) vis = vis && (unsigned)(keypos - key0 - ((g >> 1) ? subB : subA)) < (unsigned)a.slc_width;
+    }
     else if (a.causal) vis = vis && keypos * a.stride + a.block <= tokpos;
 
     float s[8], dp[8], p[8], ds[8];
@@ -368,6 +384,11 @@ bwd_kv_kernel(const BwdArgs a) {
     int splA = 0, splB = 0;
     bool splV = false;
     if (MODE == kBwdSlc) list_split(aftv, c + 2, splA, splB, splV);
+    int splsA = 0, splsB = 0;
+    if (parts) {
+      splsA = (int)__builtin_amdgcn_readlane(afts, 0);
+      splsB = (int)__builtin_amdgcn_readlane(afts, 1);
+    }
     if (MODE == kBwdSlc) {
       // dQ^T[dk][row] = sum_key K[key][dk] dS[row][key]: this wavefront takes every NW-th 16-channel tile
       T* part = reinterpret_cast<T*>(a.ws.po);
@@ -392,6 +413,10 @@ bwd_kv_kernel(const BwdArgs a) {
     if (MODE == kBwdSlc) {
       nxtA = splA; nxtB = splB; nxtV = splV;
       if (c + 3 < nchunks) aftv = list_entry(c + 3);      // first touched an iteration from here
+      if (parts) {
+        subA = nsubA; subB = nsubB; nsubA = splsA; nsubB = splsB;
+        if (c + 3 < nchunks) afts = sub_entry(c + 3);
+      }
     } else if (c + 2 < nchunks) {
       chunk_tokens(c + 2, nxtA, nxtB, nxtV);
     }
@@ -759,7 +784,7 @@ static SlcArgs slc_args_of(const SlcSwaBwdArgs& c) {
   s.indices = c.indices; s.counts = c.counts; s.cu_seq = c.cu_seq; s.batch = c.batch; s.total = c.total;
   s.hq = c.hq; s.hkv = c.hkv; s.dk = c.dk; s.dv = c.dv; s.top_n = c.top_n; s.block_size = c.block_size;
   s.idx64 = c.idx64; s.dtype = c.dtype;
-  return s;
+  return slc_virtual(s);           // top_n counts 64-key slots from here on
 }
 
 long slc_swa_bwd_workspace_bytes(const SlcSwaBwdArgs& c) {
@@ -806,7 +831,7 @@ static int launch_slc_swa_bwd_t(const SlcSwaBwdArgs& c, hipStream_t st) {
     if (rc) return rc;
     if (c.delta_slc == nullptr) launch_delta<T>(c.o_slc, c.d_o_slc, delta_slc, (long)c.total * c.hq, DV, st);
     a.d_o = c.d_o_slc; a.lse = c.lse_slc; a.delta = c.delta_slc ? c.delta_slc : delta_slc;
-    a.rowscale = c.rowscale_slc; a.ws = ws;
+    a.rowscale = c.rowscale_slc; a.ws = ws; a.slc_width = min(c.block_size, kBlk);
     rc = launch_kv_t<T, DK, DV, kBwdSlc, 4>(a, c.total, st);
     if (rc) return rc;
   }
@@ -816,7 +841,7 @@ static int launch_slc_swa_bwd_t(const SlcSwaBwdArgs& c, hipStream_t st) {
     const int* slotmap = slc ? ws.slotmap : nullptr;
     const T* part = slc ? reinterpret_cast<const T*>(ws.po) : nullptr;
     const T* dq_in = swa ? reinterpret_cast<const T*>(c.dq) : nullptr;
-    const int top_n = slc ? c.top_n : 0;
+    const int top_n = slc ? slc_args_of(c).top_n : 0;      // slots per (token, head)
     if (top_n == 16)
       hipLaunchKernelGGL((slc_dq_merge_kernel<T, DK, 16>), grid, dim3(256), 0, st, slotmap, part, dq_in,
                          reinterpret_cast<const T*>(c.dq_add), reinterpret_cast<T*>(c.dq), (long)c.total, c.hq, c.hkv,
@@ -838,6 +863,7 @@ static int launch_slc_swa_bwd_t(const SlcSwaBwdArgs& c, hipStream_t st) {
     const int key = (ARGS).dk * 1000 + (ARGS).dv;                                     \
     if ((ARGS).dtype == 0) {                                                          \
       switch (key) {                                                                  \
+        case 32032: return FN<bf16_t, 32, 32>(ARGS, ST);                              \
         case 64064: return FN<bf16_t, 64, 64>(ARGS, ST);                              \
         case 128128: return FN<bf16_t, 128, 128>(ARGS, ST);                           \
         case 192128: return FN<bf16_t, 192, 128>(ARGS, ST);                           \
@@ -845,6 +871,7 @@ static int launch_slc_swa_bwd_t(const SlcSwaBwdArgs& c, hipStream_t st) {
       }                                                                               \
     } else if ((ARGS).dtype == 2) {                                                   \
       switch (key) {                                                                  \
+        case 32032: return FN<f16_t, 32, 32>(ARGS, ST);                               \
         case 64064: return FN<f16_t, 64, 64>(ARGS, ST);                               \
         case 128128: return FN<f16_t, 128, 128>(ARGS, ST);                            \
         case 192128: return FN<f16_t, 192, 128>(ARGS, ST);                            \
@@ -852,6 +879,7 @@ static int launch_slc_swa_bwd_t(const SlcSwaBwdArgs& c, hipStream_t st) {
       }                                                                               \
     } else {                                                                          \
       switch (key) {                                                                  \
+        case 32032: return FN<float, 32, 32>(ARGS, ST);                               \
         case 64064: return FN<float, 64, 64>(ARGS, ST);                               \
         case 128128: return FN<float, 128, 128>(ARGS, ST);                            \
         default: return -2;                                                           \

@@ -328,7 +328,7 @@ int nsa_slc_combine_fwd(const void* q, const void* k, const void* vt, const void
                  workspace, (long)workspace_bytes, lse_slc, kv_rep};
   if (workspace && !aligned16(workspace)) return fail(NSA_ERR_INVALID, "slc_combine: workspace must be 16-byte aligned");
   const int rc = nsa::launch_slc_combine(a, stream);
-  if (rc == -5) return fail(NSA_ERR_UNSUPPORTED, "slc_combine: lse_slc needs the block-major schedule (bf16 or fp16, 64-key blocks, a workspace)");
+  if (rc == -5) return fail(NSA_ERR_UNSUPPORTED, "slc_combine: lse_slc needs the block-major schedule (bf16 or fp16, selection blocks of 8, 16, 32 or a multiple of 64 keys, a workspace)");
   return finish(rc, "slc_combine");
 }
 
@@ -344,7 +344,7 @@ static int slc_common_checks(const char* what, const void* q, const void* k, con
   if (vt_cols % 64 != 0 || vt_cols < nsa_transposed_cols(total, batch)) return fail(NSA_ERR_INVALID, "%s: vt_cols too small or not a multiple of 64", what);
   if (!aligned16(q) || !aligned16(k) || !aligned16(vt) || !aligned16(workspace)) return fail(NSA_ERR_INVALID, "%s: pointers must be 16-byte aligned", what);
   const int64_t need = nsa_slc_workspace_bytes(total, batch, hkv * *kv_rep, dk, dv, top_n, block_size, dtype);
-  if (need == 0) return fail(NSA_ERR_UNSUPPORTED, "%s: the block-major schedule needs bf16 or fp16, 64-key blocks, top_n <= 64 and (dk,dv) in (64,64),(128,128),(192,128)", what);
+  if (need == 0) return fail(NSA_ERR_UNSUPPORTED, "%s: the block-major schedule needs bf16 or fp16, selection blocks of 8, 16, 32 or a multiple of 64 keys, top_n * max(1, block_size / 64) <= 64 and (dk,dv) in (64,64),(128,128),(192,128)", what);
   if (workspace_bytes < need) return fail(NSA_ERR_INVALID, "%s: workspace smaller than nsa_slc_workspace_bytes", what);
   return 0;
 }
@@ -416,7 +416,7 @@ int nsa_cmp_attn_bwd(const void* q, const void* ck, const void* cv, const void* 
   nsa::CmpBwdArgs a{q, ck, cv, o, d_o, lse, cu_seqlens, cu_cmp, batch, total, cmp_rows, hq, hkv, dk, dv, block, stride,
                     causal, scale, dtype, dq, dck, dcv, workspace, delta, rowscale};
   const int rc = nsa::launch_cmp_bwd(a, stream);
-  if (rc == -2) return fail(NSA_ERR_UNSUPPORTED, "cmp_attn_bwd: head dims not built (dk,dv in (64,64),(128,128),(192,128); fp32: no 192)");
+  if (rc == -2) return fail(NSA_ERR_UNSUPPORTED, "cmp_attn_bwd: head dims not built (dk,dv in (32,32),(64,64),(128,128),(192,128); fp32: no 192)");
   return finish(rc, "cmp_attn_bwd");
 }
 
@@ -448,8 +448,9 @@ int nsa_slc_swa_bwd(const void* q, const void* k, const void* v, const void* o_s
   if (!dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "slc_swa_bwd: bad dtype");
   if (int rc = check_heads("slc_swa_bwd", hq, hkv, dk, dv)) return rc;
   if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "slc_swa_bwd: scale must be positive");
-  if (slc && (block_size != 64 || top_n > 64 || total >= (1 << 26)))
-    return fail(NSA_ERR_UNSUPPORTED, "slc_swa_bwd: the selected branch is built for 64-key blocks, top_n <= 64");
+  if (slc && (!nsa::slc_block_size_ok(block_size) || (long)top_n * (block_size > 64 ? block_size / 64 : 1) > 64 ||
+              total >= (1 << 26)))
+    return fail(NSA_ERR_UNSUPPORTED, "slc_swa_bwd: the selected branch is built for selection blocks of 8, 16, 32 or a multiple of 64 keys and top_n * max(1, block_size / 64) <= 64");
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(dq) || !aligned16(dk_out) || !aligned16(dv_out) ||
       !aligned16(workspace) || (slc && ((o_slc && !aligned16(o_slc)) || !aligned16(d_o_slc))) ||
       (swa && ((o_swa && !aligned16(o_swa)) || !aligned16(d_o_swa))))
@@ -460,7 +461,7 @@ int nsa_slc_swa_bwd(const void* q, const void* k, const void* v, const void* o_s
                        total, hq, hkv, dk, dv, slc ? top_n : 0, block_size, swa ? window : 0, scale, idx64, dtype, dq,
                        dk_out, dv_out, workspace, delta_slc, delta_swa, rowscale_slc, rowscale_swa, dq_add};
   const int rc = nsa::launch_slc_swa_bwd(a, stream);
-  if (rc == -2) return fail(NSA_ERR_UNSUPPORTED, "slc_swa_bwd: head dims not built (dk,dv in (64,64),(128,128),(192,128); fp32: no 192)");
+  if (rc == -2) return fail(NSA_ERR_UNSUPPORTED, "slc_swa_bwd: head dims not built (dk,dv in (32,32),(64,64),(128,128),(192,128); fp32: no 192)");
   return finish(rc, "slc_swa_bwd");
 }
 

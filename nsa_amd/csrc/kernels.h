@@ -58,6 +58,10 @@ struct SlcArgs {
   void* workspace; long workspace_bytes;
   float* lse;        // optional (block-major schedule only), as CmpArgs::lse_attn
   int kv_rep = 1;    // as CmpArgs::kv_rep; indices and counts stay per real kv head
+  // Block-major schedule only (set by slc_virtual, 0 = not set): the schedule works on 64-key blocks.  A selection
+  // block of 128, 192, ... keys occupies pick_mult = block_size / 64 slots per pick and top_n counts slots; a
+  // selection block of 8, 16 or 32 keys is a masked part of the 64-key block that holds it (pick_mult = 1).
+  int pick_mult = 0;
 };
 
 // Where the merge of the block-major partial results finds its inputs (all device pointers; the
@@ -146,6 +150,7 @@ int launch_swa(const SwaArgs& a, hipStream_t st);
 int launch_slc_combine(const SlcArgs& a, hipStream_t st);
 long slc_workspace_bytes(const SlcArgs& a);
 bool slc_block_major_ok(const SlcArgs& a);
+bool slc_block_size_ok(int block_size);   // 8, 16, 32 or a multiple of 64 keys
 int launch_slc_block_major(const SlcArgs& a, void* workspace, hipStream_t st);
 int launch_slc_partials(const SlcArgs& a, void* workspace, hipStream_t st);
 MergeArgs slc_merge_args(const SlcArgs& a, void* workspace);

@@ -1,4 +1,5 @@
-// Block-major selected attention (bf16, selection blocks of 64 keys).
+// Block-major selected attention (16-bit types; 64-key blocks, and through them selection blocks of 8, 16, 32
+// keys — masked parts of a 64-key block — and of 128, 192, ... keys — several 64-key slots per pick).
 //
 // The token-major kernel gathers every selected K/V block again for every token: 40 KB per
 // (token, kv head, block), 43 GB per forward at T = 32k, and a CU cannot pull more than ~15 B/clk
@@ -19,6 +20,15 @@ namespace nsa {
 
 int set_smem(const void* fn, size_t bytes);
 
+SlcArgs slc_virtual(const SlcArgs& a) {
+  if (a.pick_mult != 0) return a;
+  SlcArgs v = a;
+  v.pick_mult = a.block_size > kBlk ? a.block_size / kBlk : 1;
+  v.top_n = a.top_n * v.pick_mult;
+  return v;
+}
+
+// a: as returned by slc_virtual
 long slc_carve(const SlcArgs& a, void* base, SlcWs* ws, size_t elem, int part_width) {
   const int nb = a.total / kBlk + a.batch;
   const long nkeys = (long)a.hkv * nb;
@@ -34,6 +44,7 @@ long slc_carve(const SlcArgs& a, void* base, SlcWs* ws, size_t elem, int part_wi
   const long o_nitems = take(4);
   const long o_list = take(pairs * 4);
   const long o_slot = take(pairs * 4);
+  const long o_sub = take(pairs);
   const long o_ml = take(pairs * 2 * 16 * 4);
   const long o_po = take(pairs * 16 * part_width * (long)elem);
   if (ws != nullptr) {
@@ -41,7 +52,7 @@ long slc_carve(const SlcArgs& a, void* base, SlcWs* ws, size_t elem, int part_wi
     ws->blkbase = (int*)(b + o_blkbase); ws->counts = (int*)(b + o_counts); ws->offsets = (int*)(b + o_offsets);
     ws->cursor = (int*)(b + o_cursor); ws->items = (int*)(b + o_items); ws->n_items = (int*)(b + o_nitems);
     ws->list = (uint32_t*)(b + o_list); ws->slotmap = (int*)(b + o_slot); ws->ml = (float*)(b + o_ml);
-    ws->po = b + o_po;
+    ws->po = b + o_po; ws->sub = (uint8_t*)(b + o_sub);
     ws->nb = nb; ws->pairs_cap = pairs; ws->items_cap = items_cap;
   }
   return off;
@@ -49,11 +60,34 @@ long slc_carve(const SlcArgs& a, void* base, SlcWs* ws, size_t elem, int part_wi
 
 static long carve(const SlcArgs& a, void* base, SlcWs* ws, size_t elem) { return slc_carve(a, base, ws, elem, a.dv); }
 
-long slc_workspace_bytes(const SlcArgs& a) { return carve(a, nullptr, nullptr, a.dtype == 1 ? 4 : 2); }
+long slc_workspace_bytes(const SlcArgs& a) { return carve(slc_virtual(a), nullptr, nullptr, a.dtype == 1 ? 4 : 2); }
+
+// selection blocks the 64-key schedule can express: 8, 16, 32 (parts of a block), 64, 128, 192, ... (whole blocks)
+bool slc_block_size_ok(int block_size) {
+  return block_size == 8 || block_size == 16 || block_size == 32 || (block_size > 0 && block_size % kBlk == 0);
+}
 
 bool slc_block_major_ok(const SlcArgs& a) {
-  return a.dtype != 1 && a.block_size == kBlk && a.top_n <= 64 && a.total < (1 << 26) &&
-         (a.dk == 64 || a.dk == 128 || a.dk == 192) && (a.dv == 64 || a.dv == 128);
+  return a.dtype != 1 && slc_block_size_ok(a.block_size) && slc_virtual(a).top_n <= 64 && a.total < (1 << 26) &&
+         ((a.dk == 32 && a.dv == 32) || (a.dk == 64 && a.dv == 64) || (a.dk == 128 && a.dv == 128) ||
+          (a.dk == 192 && a.dv == 128));
+}
+
+// Slot `i` of (token position t in its sequence, real kv head row th_r): the 64-key block it stands for (local to
+// the sequence) or -1 when the slot is unusable (beyond the count, a negative or future block), and the first
+// key of the selection block inside that 64-key block.
+__device__ __forceinline__ int slc_slot_block(const SlcArgs& a, long th_r, int i, int t, int& sub) {
+  const int real_n = a.top_n / a.pick_mult, pick = i / a.pick_mult;
+  int cnt = real_n;
+  if (a.counts != nullptr) cnt = min(max(a.counts[th_r], 0), real_n);
+  const long idx = a.idx64 ? reinterpret_cast<const int64_t*>(a.indices)[th_r * real_n + pick]
+                           : (long)reinterpret_cast<const int32_t*>(a.indices)[th_r * real_n + pick];
+  sub = 0;
+  if (pick >= cnt || idx < 0 || idx > t) return -1;
+  const long key0 = idx * a.block_size + (long)(i % a.pick_mult) * kBlk;   // first key of the slot
+  if (key0 > t) return -1;
+  sub = (int)(key0 % kBlk);
+  return (int)(key0 / kBlk);
 }
 
 // ---- bucket the pairs ---------------------------------------------------------------------------
@@ -93,21 +127,19 @@ slc_bucket_kernel(const SlcArgs a, SlcWs ws) {
   const int b = seq_of_token(a.cu_seq, a.batch, tg);
   const int t = tg - a.cu_seq[b];
   const long th_r = (long)tg * (a.hkv / a.kv_rep) + h / a.kv_rep;      // picks and counts are per real kv head
-  int cnt = a.top_n;
-  if (a.counts != nullptr) cnt = min(max(a.counts[th_r], 0), a.top_n);
-  const long idx = a.idx64 ? reinterpret_cast<const int64_t*>(a.indices)[th_r * a.top_n + i]
-                           : (long)reinterpret_cast<const int32_t*>(a.indices)[th_r * a.top_n + i];
-  const bool ok = i < cnt && idx >= 0 && idx <= t && idx * kBlk <= t;
-  if (!ok) {
+  int sub;
+  const int blk = slc_slot_block(a, th_r, i, t, sub);
+  if (blk < 0) {
     if (FILL) ws.slotmap[id] = -1;
     return;
   }
-  const int key = h * ws.nb + ws.blkbase[b] + (int)idx;
+  const int key = h * ws.nb + ws.blkbase[b] + blk;
   if (!FILL) {
     atomicAdd(&ws.counts[key], 1);
   } else {
     const int p = ws.offsets[key] + atomicAdd(&ws.cursor[key], 1);
     ws.list[p] = ((uint32_t)tg << 6) | (uint32_t)i;
+    ws.sub[p] = (uint8_t)sub;
     ws.slotmap[id] = p;
   }
 }
@@ -130,7 +162,7 @@ slc_bucket_lds_kernel(const SlcArgs a, SlcWs ws) {
   for (int i = threadIdx.x; i < ws.nb; i += 1024) hist[i] = 0;
   __syncthreads();
   const int entries = (t_end - t_begin) * a.top_n;
-  auto entry = [&](int e, long& id, int& tg, int& i) -> int {      // global block of the pair, or -1
+  auto entry = [&](int e, long& id, int& tg, int& i, int& sub) -> int {      // global block of the pair, or -1
     tg = t_begin + e / a.top_n;
     i = e % a.top_n;
     const long th = (long)tg * a.hkv + h;
@@ -138,16 +170,12 @@ slc_bucket_lds_kernel(const SlcArgs a, SlcWs ws) {
     const int b = seq_of_token(a.cu_seq, a.batch, tg);
     const int t = tg - a.cu_seq[b];
     const long th_r = (long)tg * (a.hkv / a.kv_rep) + h / a.kv_rep;    // picks and counts are per real kv head
-    int cnt = a.top_n;
-    if (a.counts != nullptr) cnt = min(max(a.counts[th_r], 0), a.top_n);
-    const long idx = a.idx64 ? reinterpret_cast<const int64_t*>(a.indices)[th_r * a.top_n + i]
-                             : (long)reinterpret_cast<const int32_t*>(a.indices)[th_r * a.top_n + i];
-    const bool ok = i < cnt && idx >= 0 && idx <= t && idx * kBlk <= t;
-    return ok ? ws.blkbase[b] + (int)idx : -1;
+    const int blk = slc_slot_block(a, th_r, i, t, sub);
+    return blk >= 0 ? ws.blkbase[b] + blk : -1;
   };
   for (int e = threadIdx.x; e < entries; e += 1024) {
-    long id; int tg, i;
-    const int gb = entry(e, id, tg, i);
+    long id; int tg, i, sub;
+    const int gb = entry(e, id, tg, i, sub);
     if (FILL) ws.slotmap[id] = gb >= 0 ? atomicAdd(&hist[gb], 1) : -1;     // rank inside this workgroup
     else if (gb >= 0) atomicAdd(&hist[gb], 1);
   }
@@ -163,11 +191,12 @@ slc_bucket_lds_kernel(const SlcArgs a, SlcWs ws) {
   if (!FILL) return;
   __syncthreads();
   for (int e = threadIdx.x; e < entries; e += 1024) {
-    long id; int tg, i;
-    const int gb = entry(e, id, tg, i);
+    long id; int tg, i, sub;
+    const int gb = entry(e, id, tg, i, sub);
     if (gb >= 0) {
       const int p = hist[gb] + ws.slotmap[id];
       ws.list[p] = ((uint32_t)tg << 6) | (uint32_t)i;
+      ws.sub[p] = (uint8_t)sub;
       ws.slotmap[id] = p;
     }
   }
@@ -212,7 +241,8 @@ slc_scan_kernel(SlcWs ws, int hkv) {
 
 // ---- one K/V block in registers, the queries that picked it streamed past ------------------------
 
-template <typename T, int DK, int DV>
+// SUB: selection blocks of fewer than 64 keys; a pair then attends keys [sub, sub + block_size) of its 64-key block.
+template <typename T, int DK, int DV, bool SUB>
 __global__ void __launch_bounds__(256)
 slc_block_kernel(const SlcArgs a, const SlcWs ws) {
   constexpr int NK = DK / 32, NV = DV / 16, OLD = DV + 8;
@@ -259,6 +289,8 @@ slc_block_kernel(const SlcArgs a, const SlcWs ws) {
   // load from a wave-uniform address inside the loop would be waited for where it is issued, and on this
   // hardware that wait (loads and stores share one in-order counter) also covers the stores of the pair before.
   const uint32_t ents = ws.list[first + min(lane, count - 1)];
+  int subs = 0;
+  if (SUB) subs = ws.sub[first + min(lane, count - 1)];
   uint32_t ent = __builtin_amdgcn_readlane(ents, 0);
   {
     const T* qp = qb + ((long)(ent >> 6) * a.hq + h * G + gc) * DK + 8 * g;
@@ -301,7 +333,15 @@ slc_block_kernel(const SlcArgs a, const SlcWs ws) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) { s[i] = acc[0][i]; s[4 + i] = acc[1][i]; s[8 + i] = acc[2][i]; s[12 + i] = acc[3][i]; }
     }
-    if (st.t0 + kBlk - 1 > t_loc) {                       // the block that contains the token itself
+    if (SUB) {                                            // part of a block: its keys up to the token
+      const int lo = __builtin_amdgcn_readlane(subs, j);
+      const int hi = min(lo + a.block_size, t_loc - st.t0 + 1);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int kb = 32 * (i >> 3) + 8 * g + (i & 7);
+        if (kb < lo || kb >= hi) s[i] = kNegInf;
+      }
+    } else if (st.t0 + kBlk - 1 > t_loc) {                // the block that contains the token itself
 #pragma unroll
       for (int i = 0; i < 16; ++i)
         if (st.t0 + 32 * (i >> 3) + 8 * g + (i & 7) > t_loc) s[i] = kNegInf;
@@ -309,7 +349,7 @@ slc_block_kernel(const SlcArgs a, const SlcWs ws) {
     float mx = s[0];
 #pragma unroll
     for (int i = 1; i < 16; ++i) mx = fmaxf(mx, s[i]);
-    mx = colgroup_max(mx);                                // finite: key t0 <= t_loc is visible
+    mx = colgroup_max(mx);                                // finite: the first key of the pick is visible
     float pr[16], sum = 0.f;
     const float off = -mx * c_attn;
 #pragma unroll
@@ -375,7 +415,8 @@ static MergeArgs merge_args_of(const SlcArgs& a, const SlcWs& ws) {
 }
 
 // bucket the (token, pick) pairs by (kv head, block): counts, offsets, pair list, slot map, work items
-int launch_slc_bucket(const SlcArgs& a, const SlcWs& ws, hipStream_t st) {
+int launch_slc_bucket(const SlcArgs& raw, const SlcWs& ws, hipStream_t st) {
+  const SlcArgs a = slc_virtual(raw);
   const long pairs = ws.pairs_cap;
   hipLaunchKernelGGL(slc_prep_kernel, dim3(1), dim3(256), 0, st, a.cu_seq, a.batch, ws, a.hkv);
   if (ws.nb <= kBucketMaxBins) {
@@ -403,7 +444,10 @@ template <typename T, int DK, int DV>
 static int launch_partials_t(const SlcArgs& a, const SlcWs& ws, hipStream_t st) {
   const int rc = launch_slc_bucket(a, ws, st);
   if (rc) return rc;
-  hipLaunchKernelGGL((slc_block_kernel<T, DK, DV>), dim3((ws.items_cap + 3) / 4), dim3(256), 0, st, a, ws);
+  if (a.block_size < kBlk)
+    hipLaunchKernelGGL((slc_block_kernel<T, DK, DV, true>), dim3((ws.items_cap + 3) / 4), dim3(256), 0, st, a, ws);
+  else
+    hipLaunchKernelGGL((slc_block_kernel<T, DK, DV, false>), dim3((ws.items_cap + 3) / 4), dim3(256), 0, st, a, ws);
   return 0;
 }
 
@@ -417,13 +461,16 @@ static int launch_merge_t(const SlcArgs& a, const SlcWs& ws, hipStream_t st) {
   return 0;
 }
 
-int launch_slc_partials(const SlcArgs& a, void* workspace, hipStream_t st) {
+int launch_slc_partials(const SlcArgs& raw, void* workspace, hipStream_t st) {
+  const SlcArgs a = slc_virtual(raw);
   SlcWs ws;
   carve(a, workspace, &ws, 2);
   switch (a.dk * 1000 + a.dv + (a.dtype == 2 ? 1000000 : 0)) {
+    case 32032: return launch_partials_t<bf16_t, 32, 32>(a, ws, st);
     case 64064: return launch_partials_t<bf16_t, 64, 64>(a, ws, st);
     case 128128: return launch_partials_t<bf16_t, 128, 128>(a, ws, st);
     case 192128: return launch_partials_t<bf16_t, 192, 128>(a, ws, st);
+    case 1032032: return launch_partials_t<f16_t, 32, 32>(a, ws, st);
     case 1064064: return launch_partials_t<f16_t, 64, 64>(a, ws, st);
     case 1128128: return launch_partials_t<f16_t, 128, 128>(a, ws, st);
     case 1192128: return launch_partials_t<f16_t, 192, 128>(a, ws, st);
@@ -431,19 +478,24 @@ int launch_slc_partials(const SlcArgs& a, void* workspace, hipStream_t st) {
   }
 }
 
-MergeArgs slc_merge_args(const SlcArgs& a, void* workspace) {
+MergeArgs slc_merge_args(const SlcArgs& raw, void* workspace) {
+  const SlcArgs a = slc_virtual(raw);
   SlcWs ws;
   carve(a, workspace, &ws, 2);
   return merge_args_of(a, ws);
 }
 
-int launch_slc_block_major(const SlcArgs& a, void* workspace, hipStream_t st) {
+int launch_slc_block_major(const SlcArgs& raw, void* workspace, hipStream_t st) {
+  const SlcArgs a = slc_virtual(raw);
   const int rc = launch_slc_partials(a, workspace, st);
   if (rc) return rc;
   SlcWs ws;
   carve(a, workspace, &ws, 2);
-  if (a.dtype == 2) return a.dv == 64 ? launch_merge_t<f16_t, 64>(a, ws, st) : launch_merge_t<f16_t, 128>(a, ws, st);
-  return a.dv == 64 ? launch_merge_t<bf16_t, 64>(a, ws, st) : launch_merge_t<bf16_t, 128>(a, ws, st);
+  if (a.dtype == 2)
+    return a.dv == 32 ? launch_merge_t<f16_t, 32>(a, ws, st)
+                      : a.dv == 64 ? launch_merge_t<f16_t, 64>(a, ws, st) : launch_merge_t<f16_t, 128>(a, ws, st);
+  return a.dv == 32 ? launch_merge_t<bf16_t, 32>(a, ws, st)
+                    : a.dv == 64 ? launch_merge_t<bf16_t, 64>(a, ws, st) : launch_merge_t<bf16_t, 128>(a, ws, st);
 }
 
 }  // namespace nsa

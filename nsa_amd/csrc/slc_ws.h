@@ -1,5 +1,7 @@
 // Workspace of the block-major selected attention: the (token, pick) pairs bucketed by
-// (kv head, 64-key block).  Shared by the forward and the backward kernels.
+// (kv head, 64-key block).  Shared by the forward and the backward kernels.  Selection blocks of other sizes
+// map onto 64-key blocks: a multiple of 64 keys takes several slots per pick, a divisor of 64 keys is a part
+// of one 64-key block, whose first key inside that block is kept per pair (sub).
 #pragma once
 #include "kernels.h"
 
@@ -11,12 +13,17 @@ constexpr int kBlk = 64;          // keys per selection block (4 MFMA tiles)
 struct SlcWs {
   int* blkbase; int* counts; int* offsets; int* cursor; int* items; int* n_items;
   uint32_t* list; int* slotmap; float* ml; void* po;
+  uint8_t* sub;    // per pair: first key of the selection block inside its 64-key block (0 unless block_size < 64)
   int nb;          // bound on the number of 64-key blocks over all sequences
-  long pairs_cap;  // total * hkv * top_n
+  long pairs_cap;  // total * hkv * slots per (token, head)
   int items_cap;
 };
 
 __host__ __device__ inline long slc_align_up(long x, long a) { return (x + a - 1) / a * a; }
+
+// The arguments as the block-major schedule sees them: top_n counts 64-key slots (see SlcArgs::pick_mult).
+// Idempotent.
+SlcArgs slc_virtual(const SlcArgs& a);
 
 // Lays the workspace out in `base` (ws == nullptr: only returns the size).  `part_width` is the row
 // width of the per-pair partial result (16 rows of part_width elements of `elem` bytes per pair).

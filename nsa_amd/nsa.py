@@ -119,9 +119,11 @@ class NSAAttention(nn.Module):
         if q.shape[1] // k.shape[1] > 16 and (q.shape[1] // k.shape[1]) % 16:
             raise NotImplementedError("the NSA backward runs GQA groups of up to 16 heads and multiples of 16 "
                                       "heads; run inference under torch.no_grad()")
-        if q.dtype not in (torch.bfloat16, torch.float16) or self.selection_block_size != 64:
+        bs = self.selection_block_size
+        if q.dtype not in (torch.bfloat16, torch.float16) or not (bs in (8, 16, 32) or bs % 64 == 0):
             raise NotImplementedError(
-                "the NSA backward kernels are built for bfloat16 / float16 and 64-key selection blocks; run inference under "
+                "the NSA backward kernels are built for bfloat16 / float16 and selection blocks of 8, 16, 32 or a "
+                "multiple of 64 keys; run inference under "
                 "torch.no_grad() (an input or a parameter of this call requires grad)")
         ck, cv, cu_cmp, nc = self.compressor.compress_packed(k, v, cu, seq_len=seq_len if uniform else None)
         max_nc = nc if nc is not None else conv_compressed_len(seq_len, self.compression_stride,

@@ -46,7 +46,7 @@ def _check(name, got, ref, dtype, floor=1.0):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("lens,Hq,Hkv,Dk,Dv,W", [([300], 16, 1, 64, 64, 128), ([257, 40, 130], 32, 2, 128, 128, 100),
                                                  ([200], 16, 1, 192, 128, 64), ([130], 8, 2, 64, 64, 1),
-                                                 ([150], 6, 2, 64, 64, 1000),
+                                                 ([150], 6, 2, 64, 64, 1000), ([190, 70], 16, 1, 32, 32, 50),
                                                  # 36 key tiles: several per XCD, windows that wrap around
                                                  ([1500, 700], 16, 2, 64, 64, 200)])
 def test_swa_bwd(dtype, lens, Hq, Hkv, Dk, Dv, W):
@@ -85,6 +85,7 @@ def test_swa_bwd(dtype, lens, Hq, Hkv, Dk, Dv, W):
                                                           ([2500], 16, 1, 192, 128, 32, 16, True),
                                                           ([260], 8, 2, 64, 64, 64, 16, True),
                                                           ([200], 4, 1, 64, 64, 32, 16, False),
+                                                          ([400, 90], 16, 2, 32, 32, 32, 16, True),
                                                           # 10 token items: more than one per XCD
                                                           ([5000], 16, 1, 64, 64, 32, 16, True)])
 def test_cmp_attn_bwd(dtype, lens, Hq, Hkv, Dk, Dv, l, d, causal):
@@ -143,7 +144,22 @@ def _random_indices(T, Hkv, S, bs, seed):
                                                   ([200], 4, 1, 64, 64, 2, 32)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_slc_swa_bwd(lens, Hq, Hkv, Dk, Dv, S, W, dtype):
-    bs = 64
+    _slc_swa_bwd_case(lens, Hq, Hkv, Dk, Dv, S, W, dtype, 64)
+
+
+@pytest.mark.parametrize("lens,Hq,Hkv,Dk,Dv,S,W,bs", [([300, 90], 16, 1, 64, 64, 5, 0, 32),
+                                                     ([260], 8, 2, 128, 128, 4, 40, 8),
+                                                     ([330], 16, 1, 192, 128, 6, 64, 16),
+                                                     ([700], 16, 1, 64, 64, 3, 100, 128),
+                                                     ([900, 100], 32, 2, 128, 128, 2, 0, 192),
+                                                     ([300], 16, 1, 32, 32, 3, 64, 32), ([300], 4, 2, 32, 32, 3, 0, 64)])
+def test_slc_swa_bwd_other_selection_block_sizes(lens, Hq, Hkv, Dk, Dv, S, W, bs):
+    """Selection blocks of 8, 16, 32 keys (the reference's own test uses 32, tests/test_parallel_nsa.py:169) run as
+    masked parts of a 64-key block, blocks of 128, 192 keys as several 64-key blocks per pick."""
+    _slc_swa_bwd_case(lens, Hq, Hkv, Dk, Dv, S, W, torch.bfloat16, bs)
+
+
+def _slc_swa_bwd_case(lens, Hq, Hkv, Dk, Dv, S, W, dtype, bs):
     ops = _ops()
     T = sum(lens)
     q, k, v, _ = make_qkv(T, Hq, Hkv, Dk, Dv, 170, dtype, 0.7)
@@ -280,14 +296,14 @@ def _leaf(t):
     return t.to(DEV).requires_grad_(True)
 
 
-def _module_backward_case(mode, lens, Hq, Hkv, Dk, Dv, act, S=4, W=64, seed=190, dtype=torch.bfloat16):
+def _module_backward_case(mode, lens, Hq, Hkv, Dk, Dv, act, S=4, W=64, seed=190, dtype=torch.bfloat16, sel_block=64):
     """NSAAttention end to end: gradients of every input and parameter against autograd through the
     oracle forward (float64, the module's own block picks forced so that score ties cannot differ)."""
     from nsa_amd.nsa import NSAAttention
     T = sum(lens)
-    p = O.NSAParams(block=32, stride=16, sel_block=64, top_n=S, window=W, scale=1.0 / math.sqrt(Dk))
+    p = O.NSAParams(block=32, stride=16, sel_block=sel_block, top_n=S, window=W, scale=1.0 / math.sqrt(Dk))
     torch.manual_seed(5)
-    mod = NSAAttention(Dk, causal=True, compression_stride=16, compression_block=32, selection_block=64,
+    mod = NSAAttention(Dk, causal=True, compression_stride=16, compression_block=32, selection_block=sel_block,
                        selected_block_count=S, sliding_window=W, device=DEV, dtype=dtype, compressor_mode=mode,
                        gate_activation=act)       # None: raw gates of either sign, as in the reference
     q, k, v, _ = make_qkv(T, Hq, Hkv, Dk, Dv, seed, dtype, 0.7)
@@ -362,6 +378,14 @@ def test_module_backward_groups_of_32_48_64_heads(mode, lens, Hq, Hkv, Dk, Dv, a
     """What the reference's HQ % (16 * H) == 0 admits beyond 16 heads (nsa/selection_attn.py:800): the backward runs
     one call per sub-group of 16 heads, the key / value gradients of the sub-groups add up."""
     _module_backward_case(mode, lens, Hq, Hkv, Dk, Dv, act)
+
+
+@pytest.mark.parametrize("lens,Hq,Hkv,D,sel_block,S", [([400, 130], 16, 1, 64, 32, 6), ([500], 32, 2, 128, 128, 3),
+                                                      ([300], 16, 1, 32, 32, 4)])
+def test_module_backward_other_selection_block_sizes(lens, Hq, Hkv, D, sel_block, S):
+    """Training through the module with selection blocks of 32 keys (what the reference's own selection test uses)
+    and of 128 keys, and with head dim 32."""
+    _module_backward_case("mean", lens, Hq, Hkv, D, D, "sigmoid", S=S, sel_block=sel_block)
 
 
 def test_module_backward_randomized_small_shapes():
@@ -452,6 +476,47 @@ def test_parallel_nsa_and_flash_attn_backward(dtype, Hkv):
     _check("dq", qd.grad, rq.grad, dtype)
     _check("dck", ckd.grad, rck.grad, dtype)
     _check("dcv", cvd.grad, rcv.grad, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_parallel_nsa_backward_in_the_shape_of_the_reference_test(dtype):
+    """The reference's own selection test (tests/test_parallel_nsa.py:168-236): B 2, T 64, H 1, HQ 16, D 32, S 2,
+    32-key selection blocks, window 128, float16, gates of ones that require grad, random counts, two rows with an
+    unusable first pick; forward and every gradient it compares (dq, dk, dv, dg_slc) plus dg_swa."""
+    import nsa_amd
+    B, T, H, HQ, D, S, bs, W = 2, 64, 1, 16, 32, 2, 32, 128
+    q = randn(B, T, HQ, D, seed=300, dtype=dtype)
+    k = randn(B, T, H, D, seed=301, dtype=dtype)
+    v = randn(B, T, H, D, seed=302, dtype=dtype)
+    g_slc, g_swa = torch.ones(B, T, HQ, dtype=dtype), torch.ones(B, T, HQ, dtype=dtype)
+    d_o = randn(B, T, HQ, D, seed=303, dtype=dtype)
+    gen = torch.Generator().manual_seed(304)
+    idx = torch.full((B, T, H, S), T, dtype=torch.long)
+    for b in range(B):
+        for t in range(T):
+            perm = torch.randperm(max(1, t // bs), generator=gen)[:S]
+            idx[b, t, 0, :len(perm)] = perm
+    idx = idx.sort(-1)[0]
+    idx[0, 0, 0, 0] = 4
+    idx[1, 63, 0, 0] = 7
+    counts = torch.randint(1, S + 1, (B, T, H), generator=gen)
+    leaves = [_leaf(t) for t in (q, k, v, g_slc, g_swa)]
+    o = nsa_amd.selection_attention(*leaves, idx.to(DEV), counts.to(DEV), bs, W)
+    o.backward(d_o.to(DEV))
+    scale = D ** -0.5
+    refs = [t.double().clone().requires_grad_(True) for t in (q, k, v, g_slc, g_swa)]
+    outs = []
+    for b in range(B):
+        o_slc = O.selected_attention(refs[0][b], refs[1][b], refs[2][b], idx[b], counts[b], bs, scale,
+                                     math_dtype=torch.float64)
+        o_swa = O.sliding_attention(refs[0][b], refs[1][b], refs[2][b], W, scale, math_dtype=torch.float64)
+        outs.append(O.gated_combine(refs[3][b], o_slc, refs[4][b], o_swa))
+    ref = torch.stack(outs)
+    ref.backward(d_o.double())
+    print("reference test shape", dtype)
+    _check("out", o.detach(), ref.detach(), dtype)
+    for name, a, r in zip(("dq", "dk", "dv", "dg_slc", "dg_swa"), leaves, refs):
+        _check(name, a.grad, r.grad, dtype)
 
 
 def test_compress_kv_backward():

@@ -263,7 +263,11 @@ def _random_indices(T, Hkv, S, bs, seed, poison=True):
 @pytest.mark.parametrize("lens,Hq,Hkv,Dk,Dv,S,bs", [([256], 16, 1, 32, 32, 2, 32), ([512, 100], 32, 2, 128, 128, 8, 64),
                                                    ([384], 4, 1, 64, 64, 4, 64), ([200], 16, 1, 192, 128, 3, 64),
                                                    ([160], 6, 2, 64, 64, 3, 16), ([512, 100], 64, 2, 128, 128, 8, 64),
-                                                   ([300], 48, 1, 64, 64, 3, 32)])
+                                                   ([300], 48, 1, 64, 64, 3, 32),
+                                                   # other selection block sizes on the 64-key schedule: parts of
+                                                   # a block (8, 16, 32 keys) and several blocks per pick (128, 192)
+                                                   ([300, 90], 16, 1, 64, 64, 5, 32), ([300], 8, 2, 128, 128, 4, 8),
+                                                   ([700], 16, 1, 64, 64, 3, 128), ([900, 100], 32, 2, 192, 128, 2, 192)])
 def test_slc_only(dtype, lens, Hq, Hkv, Dk, Dv, S, bs):
     ops = _ops()
     T = sum(lens)
@@ -275,7 +279,7 @@ def test_slc_only(dtype, lens, Hq, Hkv, Dk, Dv, S, bs):
     counts = torch.randint(0, S + 1, (T, Hkv), generator=g)
     vt = ops.transpose(v.to(DEV), cu, len(lens))
     scale = 1.0 / math.sqrt(Dk)
-    has_block_major = dtype != torch.float32 and bs == 64
+    has_block_major = dtype != torch.float32 and (bs in (8, 16, 32) or bs % 64 == 0) and Dk >= 64
     modes = ((False, torch.int64, False), (True, torch.int32, False)) + \
         (((False, torch.int32, True), (True, torch.int64, True)) if has_block_major else ())
     for use_counts, dt_idx, block_major in modes:

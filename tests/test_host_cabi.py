@@ -159,13 +159,18 @@ def test_backward_argument_errors_do_not_launch(lib):
     rc = lib.nsa_cmp_attn_bwd(p, p, p, p, p, p, None, None, p, p, 1, 64, 2, 16, 1, 64, 64, 32, 16, 0.1, 1, 0, p, p, p, p, 8, None)
     assert rc == -1 and b"workspace" in lib.nsa_last_error_string()
     assert lib.nsa_cmp_attn_bwd_workspace_bytes(64, 2, 16, 1, 64, 64) >= 64 * 16 * 4 + 2 * 2 * 64 * 4
-    # selected + sliding backward: a branch needs its saved tensors, the selected one 64-key blocks
+    # selected + sliding backward: a branch needs its saved tensors
     rc = lib.nsa_slc_swa_bwd(p, p, p, None, None, p, None, None, None, None, None, None, None, None, None, p, 1, 64, 16, 1, 64, 64, 4, 64, 0, 0.1, 1,
                              0, None, p, p, p, p, 1 << 30, None)
     assert rc == -1 and b"selected branch" in lib.nsa_last_error_string()
-    rc = lib.nsa_slc_swa_bwd(p, p, p, p, None, p, None, p, None, None, None, None, None, p, None, p, 1, 64, 16, 1, 64, 64, 4, 32, 0, 0.1, 1, 0, None, p, p,
-                             p, p, 1 << 30, None)
-    assert rc == -2 and b"64-key" in lib.nsa_last_error_string()
+    # selection blocks: 8, 16, 32 or a multiple of 64 keys, at most 64 slots of 64 keys per (token, head)
+    for block, top_n in ((48, 4), (24, 4), (128, 40)):
+        rc = lib.nsa_slc_swa_bwd(p, p, p, p, None, p, None, p, None, None, None, None, None, p, None, p, 1, 64, 16, 1, 64, 64, top_n, block, 0, 0.1, 1, 0,
+                                 None, p, p, p, p, 1 << 30, None)
+        assert rc == -2 and b"multiple of 64" in lib.nsa_last_error_string()
+    assert lib.nsa_slc_workspace_bytes(64, 1, 1, 64, 64, 4, 48, 0) == 0
+    assert lib.nsa_slc_workspace_bytes(64, 1, 1, 64, 64, 40, 128, 0) == 0
+    assert lib.nsa_slc_workspace_bytes(64, 1, 1, 64, 64, 4, 128, 0) > lib.nsa_slc_workspace_bytes(64, 1, 1, 64, 64, 4, 32, 0) > 0
     rc = lib.nsa_slc_swa_bwd(p, p, p, None, p, None, p, None, p, None, None, None, None, None, None, p, 1, 64, 16, 1, 64, 64, 0, 64, 0, 0.1, 1, 0, None, p, p,
                              p, p, 1 << 30, None)
     assert rc == -1 and b"sliding branch" in lib.nsa_last_error_string()
