@@ -240,6 +240,23 @@ int nsa_swa_merge_fwd(const void* q, const void* k, const void* vt, const void* 
                       void* o_slc_out, void* o_swa_out, float* lse_slc_out, float* lse_swa_out,
                       const void* workspace, int64_t workspace_bytes, nsa_stream_t stream);
 
+/* The same schedule as nsa_slc_partials_fwd + nsa_swa_merge_fwd in ONE call that walks the tokens in slabs, so
+ * that the partial results need only the workspace the caller has: every slab is bucketed, attended per block
+ * and merged in the window kernel's epilogue before the next one reuses the workspace (same stream order; the
+ * result is bit-identical to the two-call form).  The slab is the largest number of token tiles whose pair list
+ * and partial results fit workspace_bytes; nsa_slc_swa_fused_workspace_bytes gives the bytes for slabs of at
+ * least slab_tokens tokens (slab_tokens <= 0: all tokens at once = nsa_slc_workspace_bytes), 0 when the shape
+ * has no block-major schedule.  The slot map inside the workspace still covers every token (4 bytes per
+ * (token, kv head, pick)).  Arguments as in the two entry points above. */
+int64_t nsa_slc_swa_fused_workspace_bytes(int total, int batch, int hq, int hkv, int dk, int dv, int top_n,
+                                          int block_size, int dtype, int slab_tokens);
+int nsa_slc_swa_fused_fwd(const void* q, const void* k, const void* vt, const void* indices, const int32_t* counts,
+                          const void* g_slc, const void* g_swa, const void* g_cmp, int64_t gate_stride,
+                          const void* o_cmp, void* out, const int32_t* cu_seqlens, int batch, int total, int hq,
+                          int hkv, int dk, int dv, int vt_cols, int window, int top_n, int block_size, float scale,
+                          int idx64, int gate_act, int dtype, void* o_slc_out, void* o_swa_out, float* lse_slc_out,
+                          float* lse_swa_out, void* workspace, int64_t workspace_bytes, nsa_stream_t stream);
+
 /* Bytes of the optional workspace of nsa_slc_combine_fwd; 0 when the shape has no block-major path
  * (bf16 or fp16; selection blocks of 8, 16, 32 or a multiple of 64 keys, top_n * max(1, block_size / 64) <= 64).  hkv: kv heads, times hq / (16 * hkv) when the GQA group has more
  * than 16 heads (one set of partial results per sub-group of 16 query heads). */

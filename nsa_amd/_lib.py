@@ -41,6 +41,8 @@ SIGNATURES = {
     "nsa_slc_workspace_bytes": (_L, [_I, _I, _I, _I, _I, _I, _I, _I]),
     "nsa_slc_partials_fwd": (_I, [_P] * 6 + [_I] * 9 + [_F, _I, _I, _P, _L, _P]),
     "nsa_swa_merge_fwd": (_I, [_P] * 6 + [_L, _P, _P, _P] + [_I] * 10 + [_F, _I, _I, _P, _P, _P, _P, _P, _L, _P]),
+    "nsa_slc_swa_fused_workspace_bytes": (_L, [_I] * 10),
+    "nsa_slc_swa_fused_fwd": (_I, [_P] * 8 + [_L, _P, _P, _P] + [_I] * 10 + [_F, _I, _I, _I, _P, _P, _P, _P, _P, _L, _P]),
     "nsa_cmp_attn_bwd_workspace_bytes": (_L, [_I] * 6),
     "nsa_cmp_attn_bwd": (_I, [_P] * 10 + [_I] * 9 + [_F, _I, _I, _P, _P, _P, _P, _L, _P]),
     "nsa_slc_swa_bwd_workspace_bytes": (_L, [_I] * 9),

@@ -38,6 +38,7 @@ struct StreamParams {
                      // sub-groups, and sub-group h reads the keys / values of kv head h / kv_rep
   int split_hidden;  // compressed branch: stop at cmp_visible_end(): the rows beyond carry no attention, they only feed
                      // the importance log-sum-exp, which this caller did not ask for
+  int tile_base = 0; // first token tile of this launch (workgroup x takes tile tile_base + x)
 };
 
 // MERGE (sliding window only): 0 = write the branch output; otherwise the epilogue merges the
@@ -59,7 +60,7 @@ stream_attn_kernel(const StreamParams a) {
   const int n = lane & 15, g = lane >> 4;
   const int G = a.hq / a.hkv, Gp = next_pow2(G), lgp = ilog2(Gp);
   const int TQ = ROWS >> lgp;
-  const SeqTile st = find_tile(a.cu_seq, a.batch, TQ, blockIdx.x);
+  const SeqTile st = find_tile(a.cu_seq, a.batch, TQ, a.tile_base + blockIdx.x);
   if (!st.valid) return;
   const int h = blockIdx.y;
   const int hk = h / a.kv_rep;                 // kv head whose keys / values this (sub-)group reads
@@ -620,7 +621,7 @@ int group_pow2(int G) {
 }
 
 template <typename T, int DK, int DV, bool CMP, int MERGE = 0>
-static int launch_stream_t(const StreamParams& a, int total, hipStream_t st) {
+static int launch_stream_t(const StreamParams& a, int total, hipStream_t st, int tile_count = 0) {
   constexpr int NG = StreamTile<T, CMP>::NG, CH = StreamTile<T, CMP>::CH, NW = StreamTile<T, CMP>::NW;
   const int Gp = group_pow2(a.hq / a.hkv);
   const int TQ = NW * NG * 16 / Gp;
@@ -628,9 +629,16 @@ static int launch_stream_t(const StreamParams& a, int total, hipStream_t st) {
   auto fn = stream_attn_kernel<T, DK, DV, NG, CH, NW, CMP, MERGE>;
   const int rc = set_smem(reinterpret_cast<const void*>(fn), smem);
   if (rc) return rc;
-  const int tiles = total / TQ + a.batch;
+  const int tiles = tile_count > 0 ? tile_count : total / TQ + a.batch;
   hipLaunchKernelGGL(fn, dim3(tiles, a.hkv), dim3(NW * 64), smem, st, a);
   return 0;
+}
+
+// tokens per tile of the window kernel (what SlcArgs::tile_tokens / SwaArgs::tile_begin count in)
+int swa_tile_tokens(int hq, int hkv, int dtype) {
+  const int rows = dtype == 1 ? StreamTile<float, false>::NW * StreamTile<float, false>::NG * 16
+                              : StreamTile<bf16_t, false>::NW * StreamTile<bf16_t, false>::NG * 16;
+  return rows / group_pow2(hq / hkv);
 }
 
 template <typename T, int DK, int DV>
@@ -653,9 +661,9 @@ static int launch_swa_t(const SwaArgs& a, hipStream_t st) {
 template <typename T, int DK, int DV>
 static int launch_swa_merge_t(const SwaArgs& a, const MergeArgs& m, hipStream_t st) {
   StreamParams p{a.q, a.k, a.vt, nullptr, nullptr, a.cu_seq, a.cu_seq, a.batch, a.hq, a.hkv, (long)(a.hkv / a.kv_rep) * DK,
-                 (long)DK, a.vt_cols, 0, 0, a.window, 1, a.scale, m, a.lse, a.kv_rep, 0};
-  if (m.top_n == 16) return launch_stream_t<T, DK, DV, false, 16>(p, a.total, st);
-  return launch_stream_t<T, DK, DV, false, 1>(p, a.total, st);
+                 (long)DK, a.vt_cols, 0, 0, a.window, 1, a.scale, m, a.lse, a.kv_rep, 0, a.tile_begin};
+  if (m.top_n == 16) return launch_stream_t<T, DK, DV, false, 16>(p, a.total, st, a.tile_count);
+  return launch_stream_t<T, DK, DV, false, 1>(p, a.total, st, a.tile_count);
 }
 
 template <typename T, int DK, int DV>

@@ -389,6 +389,82 @@ int nsa_swa_merge_fwd(const void* q, const void* k, const void* vt, const void* 
   return finish(nsa::launch_swa_merge(a, m, stream), "swa_merge");
 }
 
+// Block-major selected attention + window attention + merge, one slab of token tiles at a time: the slab is as
+// large as the workspace allows, so the partial results need workspace_bytes, not nsa_slc_workspace_bytes.
+static nsa::SlcArgs fused_slab_args(int total, int batch, int hq, int hkv, int dk, int dv, int top_n, int block_size,
+                                    int dtype, int tiles) {
+  nsa::SlcArgs a{};
+  a.total = total; a.batch = batch; a.hq = hq; a.hkv = hkv; a.dk = dk; a.dv = dv; a.top_n = top_n;
+  a.block_size = block_size; a.dtype = dtype;
+  a.tile_tokens = nsa::swa_tile_tokens(hq, hkv, dtype);
+  a.tile_begin = 0; a.tile_count = tiles;
+  return a;
+}
+
+int64_t nsa_slc_swa_fused_workspace_bytes(int total, int batch, int hq, int hkv, int dk, int dv, int top_n,
+                                          int block_size, int dtype, int slab_tokens) {
+  if (total <= 0 || batch <= 0 || hq <= 0 || hkv <= 0 || top_n <= 0 || hq % hkv != 0) return 0;
+  int g = hq / hkv, kv_rep = 1;
+  if (g > 16) { if (g % 16) return 0; kv_rep = g / 16; }
+  nsa::SlcArgs a = fused_slab_args(total, batch, hq, hkv * kv_rep, dk, dv, top_n, block_size, dtype, 0);
+  if (!nsa::slc_block_major_ok(a)) return 0;
+  if (slab_tokens > 0 && slab_tokens < total) a.tile_count = (slab_tokens + a.tile_tokens - 1) / a.tile_tokens;
+  return nsa::slc_workspace_bytes(a);
+}
+
+int nsa_slc_swa_fused_fwd(const void* q, const void* k, const void* vt, const void* indices, const int32_t* counts,
+                          const void* g_slc, const void* g_swa, const void* g_cmp, int64_t gate_stride,
+                          const void* o_cmp, void* out, const int32_t* cu_seqlens, int batch, int total, int hq,
+                          int hkv, int dk, int dv, int vt_cols, int window, int top_n, int block_size, float scale,
+                          int idx64, int gate_act, int dtype, void* o_slc_out, void* o_swa_out, float* lse_slc_out,
+                          float* lse_swa_out, void* workspace, int64_t workspace_bytes, nsa_stream_t stream) {
+  const char* what = "slc_swa_fused";
+  if (!q || !k || !vt || !indices || !out || !cu_seqlens || !workspace) return fail(NSA_ERR_INVALID, "%s: null pointer", what);
+  if (batch <= 0 || total <= 0) return fail(NSA_ERR_INVALID, "%s: sizes must be positive", what);
+  if (!dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "%s: bad dtype", what);
+  int kv_rep = 1;
+  if (int rc = check_heads(what, hq, hkv, dk, dv, &kv_rep)) return rc;
+  if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "%s: scale must be positive", what);
+  if (window <= 0) return fail(NSA_ERR_INVALID, "%s: window must be positive", what);
+  if (top_n <= 0) return fail(NSA_ERR_INVALID, "%s: top_n must be positive", what);
+  if (gate_act != NSA_GATE_IDENTITY && gate_act != NSA_GATE_SIGMOID) return fail(NSA_ERR_INVALID, "%s: bad gate activation", what);
+  if (vt_cols % 64 != 0 || vt_cols < nsa_transposed_cols(total, batch)) return fail(NSA_ERR_INVALID, "%s: vt_cols too small or not a multiple of 64", what);
+  if (!aligned16(q) || !aligned16(k) || !aligned16(vt) || !aligned16(workspace) || !aligned16(out) ||
+      (o_cmp && !aligned16(o_cmp)) || (o_slc_out && !aligned16(o_slc_out)) || (o_swa_out && !aligned16(o_swa_out)))
+    return fail(NSA_ERR_INVALID, "%s: pointers must be 16-byte aligned", what);
+  const int hv = hkv * kv_rep;
+  nsa::SlcArgs probe = fused_slab_args(total, batch, hq, hv, dk, dv, top_n, block_size, dtype, 0);
+  if (!nsa::slc_block_major_ok(probe))
+    return fail(NSA_ERR_UNSUPPORTED, "%s: the block-major schedule needs bf16 or fp16, selection blocks of 8, 16, 32 or a multiple of 64 keys, top_n * max(1, block_size / 64) <= 64 and (dk,dv) in (32,32),(64,64),(128,128),(192,128)", what);
+  // the largest slab (in tiles) whose workspace fits
+  const int tile_tokens = probe.tile_tokens, total_tiles = total / tile_tokens + batch;
+  auto bytes_for = [&](int tiles) { probe.tile_count = tiles; return (int64_t)nsa::slc_workspace_bytes(probe); };
+  if (bytes_for(1) > workspace_bytes) return fail(NSA_ERR_INVALID, "%s: workspace smaller than nsa_slc_swa_fused_workspace_bytes for one tile of %d tokens", what, tile_tokens);
+  int lo = 1, hi = total_tiles;
+  while (lo < hi) {
+    const int mid = lo + (hi - lo + 1) / 2;
+    if (bytes_for(mid) <= workspace_bytes) lo = mid; else hi = mid - 1;
+  }
+  const int slab_tiles = lo;
+  for (int t0 = 0; t0 < total_tiles; t0 += slab_tiles) {
+    const int cnt = slab_tiles < total_tiles - t0 ? slab_tiles : total_tiles - t0;
+    nsa::SlcArgs sa{q, k, vt, indices, counts, g_slc, g_swa, g_cmp, (long)gate_stride, nullptr, o_cmp, out, cu_seqlens,
+                    batch, total, hq, hv, dk, dv, vt_cols, top_n, block_size, scale, idx64, gate_act, dtype,
+                    workspace, (long)workspace_bytes, nullptr, kv_rep};
+    sa.tile_tokens = tile_tokens; sa.tile_begin = t0; sa.tile_count = slab_tiles;   // capacity: always a full slab
+    int rc = nsa::launch_slc_partials(sa, workspace, stream);
+    if (rc) return finish(rc, what);
+    nsa::MergeArgs m = nsa::slc_merge_args(sa, workspace);
+    m.o_slc_out = o_slc_out; m.o_swa_out = o_swa_out; m.lse_slc_out = lse_slc_out;
+    nsa::SwaArgs wa{q, k, vt, nullptr, cu_seqlens, batch, total, hq, hv, dk, dv, vt_cols, window, scale, dtype,
+                    lse_swa_out, kv_rep};
+    wa.tile_begin = t0; wa.tile_count = cnt;
+    rc = nsa::launch_swa_merge(wa, m, stream);
+    if (rc) return finish(rc, what);
+  }
+  return finish(0, what);
+}
+
 int64_t nsa_cmp_attn_bwd_workspace_bytes(int total, int cmp_rows, int hq, int hkv, int dk, int dv) {
   if (total <= 0 || cmp_rows < 0 || hq <= 0 || hkv <= 0 || dk <= 0 || dv <= 0) return 0;
   nsa::CmpBwdArgs a{};

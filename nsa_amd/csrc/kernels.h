@@ -47,6 +47,7 @@ struct SwaArgs {
   int batch, total, hq, hkv, dk, dv, vt_cols, window; float scale; int dtype;
   float* lse;        // optional, as CmpArgs::lse_attn
   int kv_rep = 1;    // as CmpArgs::kv_rep
+  int tile_begin = 0, tile_count = 0;   // merge kernels: only these token tiles (tile_count 0 = all)
 };
 
 struct SlcArgs {
@@ -62,6 +63,10 @@ struct SlcArgs {
   // block of 128, 192, ... keys occupies pick_mult = block_size / 64 slots per pick and top_n counts slots; a
   // selection block of 8, 16 or 32 keys is a masked part of the 64-key block that holds it (pick_mult = 1).
   int pick_mult = 0;
+  // Block-major schedule, one slab of tokens at a time (tile_count 0 = all tokens): the tokens of the tiles
+  // tile_begin .. tile_begin + tile_count - 1 of tile_tokens tokens each, tiles numbered as find_tile numbers them
+  // (sequence by sequence).  Pair list and partial results are then sized for tile_count * tile_tokens tokens.
+  int tile_begin = 0, tile_count = 0, tile_tokens = 0;
 };
 
 // Where the merge of the block-major partial results finds its inputs (all device pointers; the
@@ -151,6 +156,7 @@ int launch_slc_combine(const SlcArgs& a, hipStream_t st);
 long slc_workspace_bytes(const SlcArgs& a);
 bool slc_block_major_ok(const SlcArgs& a);
 bool slc_block_size_ok(int block_size);   // 8, 16, 32 or a multiple of 64 keys
+int swa_tile_tokens(int hq, int hkv, int dtype);   // tokens per tile of the window kernel (hkv counts sub-groups)
 int launch_slc_block_major(const SlcArgs& a, void* workspace, hipStream_t st);
 int launch_slc_partials(const SlcArgs& a, void* workspace, hipStream_t st);
 MergeArgs slc_merge_args(const SlcArgs& a, void* workspace);

@@ -32,7 +32,10 @@ SlcArgs slc_virtual(const SlcArgs& a) {
 long slc_carve(const SlcArgs& a, void* base, SlcWs* ws, size_t elem, int part_width) {
   const int nb = a.total / kBlk + a.batch;
   const long nkeys = (long)a.hkv * nb;
-  const long pairs = (long)a.total * a.hkv * a.top_n;
+  const long slots = (long)a.total * a.hkv * a.top_n;                 // slot map: every token
+  long slab = a.total;                                               // pair list, partials: the tokens of one slab
+  if (a.tile_count > 0 && (long)a.tile_count * a.tile_tokens < slab) slab = (long)a.tile_count * a.tile_tokens;
+  const long pairs = slab * a.hkv * a.top_n;
   const int items_cap = (int)(pairs / kSeg + nkeys) + 1;
   long off = 0;
   auto take = [&](long bytes) { const long o = off; off = slc_align_up(off + bytes, 256); return o; };
@@ -43,7 +46,7 @@ long slc_carve(const SlcArgs& a, void* base, SlcWs* ws, size_t elem, int part_wi
   const long o_items = take((long)items_cap * 8);
   const long o_nitems = take(4);
   const long o_list = take(pairs * 4);
-  const long o_slot = take(pairs * 4);
+  const long o_slot = take(slots * 4);
   const long o_sub = take(pairs);
   const long o_ml = take(pairs * 2 * 16 * 4);
   const long o_po = take(pairs * 16 * part_width * (long)elem);
@@ -92,6 +95,18 @@ __device__ __forceinline__ int slc_slot_block(const SlcArgs& a, long th_r, int i
 
 // ---- bucket the pairs ---------------------------------------------------------------------------
 
+// Tokens [tb, te) of the slab (all tokens without one).  Every lane of the calling wavefronts takes part.
+__device__ __forceinline__ void slc_token_range(const SlcArgs& a, int& tb, int& te) {
+  tb = 0;
+  te = a.total;
+  if (a.tile_count > 0) {
+    const SeqTile s0 = find_tile(a.cu_seq, a.batch, a.tile_tokens, a.tile_begin);
+    tb = s0.valid ? s0.start + s0.t0 : a.total;
+    const SeqTile s1 = find_tile(a.cu_seq, a.batch, a.tile_tokens, a.tile_begin + a.tile_count);
+    te = s1.valid ? s1.start + s1.t0 : a.total;
+  }
+}
+
 __global__ void __launch_bounds__(256)
 slc_prep_kernel(const int32_t* __restrict__ cu, int batch, SlcWs ws, int hkv) {
   if (threadIdx.x == 0) {
@@ -119,8 +134,11 @@ __device__ __forceinline__ int seq_of_token(const int32_t* __restrict__ cu, int 
 template <bool FILL>
 __global__ void __launch_bounds__(256)
 slc_bucket_kernel(const SlcArgs a, SlcWs ws) {
-  const long id = (long)blockIdx.x * 256 + threadIdx.x;          // (token, head, pick)
-  if (id >= (long)a.total * a.hkv * a.top_n) return;
+  int tb, te;
+  slc_token_range(a, tb, te);
+  const long rel = (long)blockIdx.x * 256 + threadIdx.x;
+  if (rel >= (long)(te - tb) * a.hkv * a.top_n) return;
+  const long id = rel + (long)tb * a.hkv * a.top_n;              // (token, head, pick)
   const int i = (int)(id % a.top_n);
   const long th = id / a.top_n;
   const int h = (int)(th % a.hkv), tg = (int)(th / a.hkv);
@@ -157,8 +175,11 @@ __global__ void __launch_bounds__(1024)
 slc_bucket_lds_kernel(const SlcArgs a, SlcWs ws) {
   extern __shared__ int hist[];
   const int h = blockIdx.y;
-  const int t_begin = blockIdx.x * kBucketTok;
-  const int t_end = min(a.total, t_begin + kBucketTok);
+  int tb, te;
+  slc_token_range(a, tb, te);
+  const int t_begin = tb + blockIdx.x * kBucketTok;
+  if (t_begin >= te) return;
+  const int t_end = min(te, t_begin + kBucketTok);
   for (int i = threadIdx.x; i < ws.nb; i += 1024) hist[i] = 0;
   __syncthreads();
   const int entries = (t_end - t_begin) * a.top_n;
@@ -418,9 +439,10 @@ static MergeArgs merge_args_of(const SlcArgs& a, const SlcWs& ws) {
 int launch_slc_bucket(const SlcArgs& raw, const SlcWs& ws, hipStream_t st) {
   const SlcArgs a = slc_virtual(raw);
   const long pairs = ws.pairs_cap;
+  const long slab = pairs / ((long)a.hkv * a.top_n);               // tokens the slab can hold
   hipLaunchKernelGGL(slc_prep_kernel, dim3(1), dim3(256), 0, st, a.cu_seq, a.batch, ws, a.hkv);
   if (ws.nb <= kBucketMaxBins) {
-    const dim3 grid((a.total + kBucketTok - 1) / kBucketTok, a.hkv);
+    const dim3 grid((unsigned)((slab + kBucketTok - 1) / kBucketTok), a.hkv);
     const size_t smem = (size_t)ws.nb * sizeof(int);
     if (smem > 64 * 1024) {
       int rc = set_smem(reinterpret_cast<const void*>(slc_bucket_lds_kernel<false>), smem);

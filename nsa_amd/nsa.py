@@ -180,6 +180,13 @@ class NSAAttention(nn.Module):
                 q, k, vt, ws, idx.shape[-1], g_slc, g_swa, g_cmp, o_cmp, cu, batch, self.selection_block_size,
                 self.sliding_window, scale, gate_act=act))
         else:
+            out = None
+            if self.sliding_window > 0:
+                # the same schedule in token slabs when its one-slab workspace is beyond ops.SLC_WORKSPACE_LIMIT
+                out = stage("slc_swa_slabs", lambda: ops.slc_swa_fused(
+                    q, k, vt, idx, None, g_slc, g_swa, g_cmp, o_cmp, cu, batch, self.selection_block_size,
+                    self.sliding_window, scale, gate_act=act))
+        if ws is None and out is None:
             o_swa = stage("swa", lambda: ops.swa(q, k, vt, cu, batch, self.sliding_window, scale)) \
                 if self.sliding_window > 0 else None
             out = stage("slc_combine", lambda: ops.slc_combine(

@@ -4,6 +4,7 @@ from __future__ import annotations
 
 import ctypes as C
 import math
+import os
 from typing import Optional, Tuple
 
 import torch
@@ -248,7 +249,9 @@ def _gate_views(gates, q):
     return [None if g is None else g.to(q.dtype).contiguous() for g in gates], 1
 
 
-SLC_WORKSPACE_LIMIT = 48 << 30      # bytes; larger problems keep the token-major kernel
+# Bytes the block-major selected attention may take for its pair list and partial results in one piece (8.3 GiB at
+# 32768 tokens x 4 kv heads x 16 picks); beyond, the fused schedule walks the tokens in slabs of this size.
+SLC_WORKSPACE_LIMIT = int(os.environ.get("NSA_SLC_WORKSPACE_LIMIT", 16 << 30))
 
 
 def slc_combine(q, k, vt, indices, counts, g_slc, g_swa, g_cmp, o_swa, o_cmp, cu_seqlens, batch, block_size,
@@ -344,6 +347,47 @@ def swa_merge(q, k, vt, workspace, top_n, g_slc, g_swa, g_cmp, o_cmp, cu_seqlens
         gate_act, _dtype_code(q), _ptr(o_slc), _ptr(o_swa), _ptr(lse_slc), _ptr(lse_swa), _ptr(workspace),
         workspace.numel(), _stream())
     _lib.check(rc, "nsa_swa_merge_fwd")
+    return (out, o_slc, o_swa, lse_slc, lse_swa) if want_branches else out
+
+
+def slc_swa_fused(q, k, vt, indices, counts, g_slc, g_swa, g_cmp, o_cmp, cu_seqlens, batch, block_size, window, scale,
+                  gate_act=0, want_branches=False, workspace_limit=None):
+    """slc_partials + swa_merge as one call that walks the tokens in slabs sized to a workspace of at most
+    workspace_limit bytes (default SLC_WORKSPACE_LIMIT): what a context too long for the one-slab workspace
+    runs.  Returns as swa_merge; None when the shape has no block-major schedule."""
+    _need_cuda(q, k, vt, indices, cu_seqlens)
+    q, k = _dense(q), _dense(k)
+    total, hq, dk = q.shape
+    hkv, dv = vt.shape[0], vt.shape[1]
+    if indices.dtype not in (torch.int32, torch.int64):
+        raise TypeError("block indices must be int32 or int64")
+    indices = indices.contiguous()
+    top_n = indices.shape[-1]
+    if counts is not None:
+        counts = counts.to(torch.int32).contiguous()
+    lib = _lib.load()
+    limit = SLC_WORKSPACE_LIMIT if workspace_limit is None else int(workspace_limit)
+    geom = (total, batch, hq, hkv, dk, dv, top_n, block_size, _dtype_code(q))
+    need = lib.nsa_slc_swa_fused_workspace_bytes(*geom, 0)
+    if need <= 0:
+        return None
+    if need > limit:        # the entry point takes the largest slab these bytes hold; one tile is the least
+        need = max(limit, lib.nsa_slc_swa_fused_workspace_bytes(*geom, 1))
+    ws = torch.empty(need, dtype=torch.uint8, device=q.device)
+    (g_slc, g_swa, g_cmp), gs = _gate_views([g_slc, g_swa, g_cmp], q)
+    o_cmp = None if o_cmp is None else _dense(o_cmp)
+    out = torch.empty(total, hq, dv, dtype=q.dtype, device=q.device)
+    o_slc = o_swa = lse_slc = lse_swa = None
+    if want_branches:
+        o_slc, o_swa = torch.empty_like(out), torch.empty_like(out)
+        lse_slc = torch.empty(total, hq, dtype=torch.float32, device=q.device)
+        lse_swa = torch.empty_like(lse_slc)
+    rc = lib.nsa_slc_swa_fused_fwd(
+        _ptr(q), _ptr(k), _ptr(vt), _ptr(indices), _ptr(counts), _ptr(g_slc), _ptr(g_swa), _ptr(g_cmp), gs,
+        _ptr(o_cmp), _ptr(out), _ptr(cu_seqlens), batch, total, hq, hkv, dk, dv, vt.shape[-1], window, top_n,
+        block_size, float(scale), int(indices.dtype == torch.int64), gate_act, _dtype_code(q), _ptr(o_slc),
+        _ptr(o_swa), _ptr(lse_slc), _ptr(lse_swa), _ptr(ws), ws.numel(), _stream())
+    _lib.check(rc, "nsa_slc_swa_fused_fwd")
     return (out, o_slc, o_swa, lse_slc, lse_swa) if want_branches else out
 
 

@@ -106,6 +106,11 @@ def _parallel_nsa_nograd(qp, kp, vp, idx, counts, g_slc, g_swa, cu, nb, block_si
         o = ops.swa_merge(qp, kp, vt, ws, idx.shape[-1], g_slc.reshape(total, HQ), g_swa.reshape(total, HQ), None,
                           None, cu, nb, block_size, window_size, scale)
     else:
+        o = None
+        if window_size > 0:       # the same schedule in token slabs when the one-slab workspace is too large
+            o = ops.slc_swa_fused(qp, kp, vt, idx, counts, g_slc.reshape(total, HQ), g_swa.reshape(total, HQ), None,
+                                  None, cu, nb, block_size, window_size, scale)
+    if ws is None and o is None:
         o_swa = ops.swa(qp, kp, vt, cu, nb, window_size, scale) if window_size > 0 else None
         o = ops.slc_combine(qp, kp, vt, idx, counts, g_slc.reshape(total, HQ),
                             g_swa.reshape(total, HQ) if o_swa is not None else None, None, o_swa, None, cu, nb,

@@ -392,6 +392,45 @@ def test_parallel_nsa_api_like_reference_test(dtype):
     assert max_abs(out_hf[0].transpose(0, 1), slc + swa) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("lens,Hq,Hkv,Dk,Dv,S,W,bs", [([3000], 16, 1, 64, 64, 8, 100, 64),
+                                                     ([700, 1, 330, 64, 1500], 32, 2, 128, 128, 16, 256, 64),
+                                                     ([90] * 11 + [400, 33], 64, 2, 64, 64, 4, 64, 32),
+                                                     ([1200, 500], 16, 1, 192, 128, 3, 512, 128)])
+def test_token_slabs_equal_one_slab(lens, Hq, Hkv, Dk, Dv, S, W, bs):
+    """nsa_slc_swa_fused_fwd with a workspace for a fraction of the tokens (several slabs, slab edges inside
+    sequences, more than 8 sequences, a GQA group of 32 heads, 32- and 128-key selection blocks) against the
+    two-call schedule with the one-slab workspace: bit-identical outputs, branch outputs and log-sum-exps."""
+    ops = _ops()
+    from nsa_amd import _lib
+    dtype = torch.bfloat16
+    T = sum(lens)
+    q, k, v, gl = make_qkv(T, Hq, Hkv, Dk, Dv, 500, dtype, 0.7)
+    cu, cuh = _cu(lens), ragged_cu(lens)
+    idx = torch.cat([_random_indices(e - s, Hkv, S, bs, 501 + s, poison=e - s > 2) for s, e in zip(cuh[:-1], cuh[1:])])
+    g = torch.Generator().manual_seed(502)
+    counts = torch.randint(0, S + 1, (T, Hkv), generator=g).to(DEV)
+    qd, kd, idxd = q.to(DEV), k.to(DEV), idx.to(torch.int32).to(DEV)
+    vt = ops.transpose(v.to(DEV), cu, len(lens))
+    gates = [gl[..., i].contiguous().to(DEV) for i in range(3)]
+    o_cmp = randn(T, Hq, Dv, seed=503, dtype=dtype).to(DEV)
+    scale = 1.0 / math.sqrt(Dk)
+    ws = ops.slc_workspace(qd, Hkv, Dv, S, bs, len(lens))
+    ops.slc_partials(qd, kd, vt, idxd, counts, cu, len(lens), bs, scale, ws)
+    ref = ops.swa_merge(qd, kd, vt, ws, S, *gates, o_cmp, cu, len(lens), bs, W, scale, gate_act=1, want_branches=True)
+    lib = _lib.load()
+    geom = (T, len(lens), Hq, Hkv, Dk, Dv, S, bs, 0)
+    full = lib.nsa_slc_swa_fused_workspace_bytes(*geom, 0)
+    assert full == ws.numel()
+    for frac in (1, 3, 7):
+        limit = lib.nsa_slc_swa_fused_workspace_bytes(*geom, (T + frac - 1) // frac) if frac > 1 else full
+        assert frac == 1 or limit < full
+        got = ops.slc_swa_fused(qd, kd, vt, idxd, counts, *gates, o_cmp, cu, len(lens), bs, W, scale, gate_act=1,
+                                want_branches=True, workspace_limit=limit)
+        for name, a, b in zip(("out", "o_slc", "o_swa", "lse_slc", "lse_swa"), got, ref):
+            assert torch.equal(a, b), (name, frac)
+    print("slabs", lens, (Hq, Hkv, Dk, Dv, S, W, bs), "workspace", full, "->", limit)
+
+
 @pytest.mark.parametrize("H", [2, 1])          # GQA groups of 16 and of 32 heads
 @pytest.mark.parametrize("dtype,bs,W", [(torch.bfloat16, 64, 128), (torch.bfloat16, 32, 48), (torch.float32, 32, 16)])
 def test_parallel_nsa_packed_cu_seqlens_and_tensor_counts(dtype, bs, W, H):

@@ -89,6 +89,19 @@ def test_argument_errors_do_not_launch(lib):
     rc = lib.nsa_slc_combine_fwd(p, p, p, p, None, None, None, None, 1, None, None, p, None, p, 1, 64, 4, 1, 64, 64, 128,
                                  4, 60, 0.1, 1, 0, 0, None, 0, None)
     assert rc == -2 and b"block_size" in lib.nsa_last_error_string()
+    # the slab schedule: null pointers, a selection block the 64-key schedule cannot express, a workspace below one tile
+    fused = lambda ws, ws_bytes, block=64, q=p: lib.nsa_slc_swa_fused_fwd(      # noqa: E731
+        q, p, p, p, None, None, None, None, 1, None, p, p, 1, 4096, 16, 1, 64, 64, 4224, 128, 4, block, 0.1, 0, 0, 0, None,
+        None, None, None, ws, ws_bytes, None)
+    assert fused(p, 1 << 30, q=None) == -1 and b"null" in lib.nsa_last_error_string()
+    assert fused(None, 1 << 30) == -1
+    assert fused(p, 1 << 30, block=48) == -2 and b"multiple of 64" in lib.nsa_last_error_string()
+    assert fused(p, 1024) == -1 and b"one tile" in lib.nsa_last_error_string()
+    one_tile = lib.nsa_slc_swa_fused_workspace_bytes(4096, 1, 16, 1, 64, 64, 4, 64, 0, 1)
+    assert 0 < one_tile < lib.nsa_slc_swa_fused_workspace_bytes(4096, 1, 16, 1, 64, 64, 4, 64, 0, 1024) \
+        < lib.nsa_slc_swa_fused_workspace_bytes(4096, 1, 16, 1, 64, 64, 4, 64, 0, 0) \
+        == lib.nsa_slc_workspace_bytes(4096, 1, 1, 64, 64, 4, 64, 0)
+    assert lib.nsa_slc_swa_fused_workspace_bytes(4096, 1, 16, 1, 64, 64, 4, 64, 1, 0) == 0      # fp32: no block-major schedule
     rc = lib.nsa_compress_fwd(p, None, None, p, p, p, 1, 10, 2, 60, 32, 16, 0, None)
     assert rc == -2
     # K and V in one call: both weights or neither, dims in pieces of 8, known dtypes (0, 1, 2)
