@@ -157,7 +157,7 @@ slc_bucket_kernel(const SlcArgs a, SlcWs ws) {
   } else {
     const int p = ws.offsets[key] + atomicAdd(&ws.cursor[key], 1);
     ws.list[p] = ((uint32_t)tg << 6) | (uint32_t)i;
-    ws.sub[p] = (uint8_t)sub;
+    if (a.block_size < kBlk) ws.sub[p] = (uint8_t)sub;
     ws.slotmap[id] = p;
   }
 }
@@ -217,7 +217,7 @@ slc_bucket_lds_kernel(const SlcArgs a, SlcWs ws) {
     if (gb >= 0) {
       const int p = hist[gb] + ws.slotmap[id];
       ws.list[p] = ((uint32_t)tg << 6) | (uint32_t)i;
-      ws.sub[p] = (uint8_t)sub;
+      if (a.block_size < kBlk) ws.sub[p] = (uint8_t)sub;
       ws.slotmap[id] = p;
     }
   }

@@ -13,7 +13,8 @@ constexpr int kBlk = 64;          // keys per selection block (4 MFMA tiles)
 struct SlcWs {
   int* blkbase; int* counts; int* offsets; int* cursor; int* items; int* n_items;
   uint32_t* list; int* slotmap; float* ml; void* po;
-  uint8_t* sub;    // per pair: first key of the selection block inside its 64-key block (0 unless block_size < 64)
+  uint8_t* sub;    // per pair: first key of the selection block inside its 64-key block (written and read only when
+                   // block_size < 64)
   int nb;          // bound on the number of 64-key blocks over all sequences
   long pairs_cap;  // total * hkv * slots per (token, head)
   int items_cap;
