@@ -719,6 +719,34 @@ def test_module_randomized_groups_beyond_16_and_float16():
                      rows_per_seq=None if sum(lens) <= 1500 else 24)
 
 
+def test_module_randomized_selection_block_sizes_and_token_slabs(monkeypatch):
+    """The sweep once more over what came last: selection blocks of 32 and 128 keys on the 64-key schedule, head
+    dim 32, and (every second case) a workspace cap of 3 MB so that the selected branch runs in token slabs."""
+    from nsa_amd import ops
+    g = torch.Generator().manual_seed(5077)
+
+    def pick(options):
+        return options[int(torch.randint(0, len(options), (1,), generator=g))]
+
+    for case in range(14):
+        nseq = pick([1, 2, 3, 10])
+        lens = [int(torch.randint(1, 700 if nseq < 10 else 150, (1,), generator=g)) for _ in range(nseq)]
+        if case % 4 == 0:
+            lens[0] = pick([1, 31, 32, 33, 64, 127, 128, 129])
+        G = pick([4, 16, 16, 32])
+        Hkv = pick([1, 2])
+        Dk, Dv = pick([(32, 32), (64, 64), (128, 128), (192, 128)])
+        lsel = pick([32, 32, 128, 64]) if G <= 16 else 64      # groups beyond 16 heads: 64-key pooling geometry only
+        S = pick([2, 5, 16]) if lsel <= 64 else pick([2, 4])
+        W = pick([16, 64, 200, 512])
+        dtype = pick([torch.bfloat16, torch.float16])
+        act = pick(["sigmoid", "sigmoid", None])
+        monkeypatch.setattr(ops, "SLC_WORKSPACE_LIMIT", 3 << 20 if case % 2 else 16 << 30)
+        print("case", case, lens, G, Hkv, Dk, Dv, lsel, S, W, dtype, act, "slabs" if case % 2 else "one slab")
+        _module_case(dtype, lens, G * Hkv, Hkv, Dk, Dv, S, W, seed=900 + case, scale_in=0.6, act=act, lsel=lsel,
+                     rows_per_seq=None if sum(lens) <= 1500 else 24)
+
+
 def test_flash_attn_func_api():
     import nsa_amd
     from nsa_amd.compression_kv import KVCompressor
