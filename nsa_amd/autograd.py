@@ -92,7 +92,14 @@ class SlcSwaFn(torch.autograd.Function):
             ops.slc_partials(q, k, vt, idx, counts, cu, batch, block_size, scale, ws)
             _, o_slc, o_swa, lse_slc, lse_swa = ops.swa_merge(q, k, vt, ws, idx.shape[-1], None, None, None, None, cu,
                                                                batch, block_size, window, scale, want_branches=True)
-        else:
+        fused = None
+        if ws is None and idx is not None and window > 0:
+            # the same schedule in token slabs when its one-slab workspace is beyond ops.SLC_WORKSPACE_LIMIT
+            fused = ops.slc_swa_fused(q, k, vt, idx, counts, None, None, None, None, cu, batch, block_size, window, scale,
+                                      want_branches=True)
+        if fused is not None:
+            _, o_slc, o_swa, lse_slc, lse_swa = fused
+        elif ws is None:
             if idx is not None:
                 o_slc, lse_slc = ops.slc_combine(q, k, vt, idx, counts, None, None, None, None, None, cu, batch,
                                                  block_size, scale, block_major=True, want_lse=True)
@@ -175,7 +182,14 @@ class NSACoreFn(torch.autograd.Function):
             out, o_slc, o_swa, lse_slc, lse_swa = ops.swa_merge(
                 q, k, vt, ws, idx.shape[-1], g_slc, g_swa, g_cmp, o_cmp, cu, batch, sel_block, window, scale,
                 gate_act=gate_act, want_branches=True)
-        else:
+        fused = None
+        if ws is None and window > 0 and gl.dtype == q.dtype:
+            g_slc, g_swa, g_cmp = (gl[:, i].view(q.shape[0], q.shape[1]) for i in range(3))
+            fused = ops.slc_swa_fused(q, k, vt, idx, None, g_slc, g_swa, g_cmp, o_cmp, cu, batch, sel_block, window,
+                                      scale, gate_act=gate_act, want_branches=True)
+        if fused is not None:
+            out, o_slc, o_swa, lse_slc, lse_swa = fused
+        elif ws is None or gl.dtype != q.dtype:
             o_slc, lse_slc = ops.slc_combine(q, k, vt, idx, None, None, None, None, None, None, cu, batch, sel_block,
                                              scale, block_major=True, want_lse=True)
             o_swa = lse_swa = None

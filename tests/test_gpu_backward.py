@@ -388,6 +388,15 @@ def test_module_backward_other_selection_block_sizes(lens, Hq, Hkv, D, sel_block
     _module_backward_case("mean", lens, Hq, Hkv, D, D, "sigmoid", S=S, sel_block=sel_block)
 
 
+def test_training_forward_in_token_slabs(monkeypatch):
+    """With the one-slab workspace of the selected branch over ops.SLC_WORKSPACE_LIMIT the training forward runs the
+    slab schedule (module and functional form); outputs and gradients as before."""
+    from nsa_amd import ops
+    monkeypatch.setattr(ops, "SLC_WORKSPACE_LIMIT", 2 << 20)
+    _module_backward_case("mean", [700, 300, 90], 32, 2, 128, 128, "sigmoid", S=8, W=100)
+    test_parallel_nsa_and_flash_attn_backward(torch.bfloat16, 2)
+
+
 def test_module_backward_randomized_small_shapes():
     """Seeded sweep over ragged lengths (down to a single token and sequences without any compressed row),
     group sizes 1..16, top-n, window, both compressors and both gate conventions."""
