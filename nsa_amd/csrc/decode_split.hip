@@ -351,7 +351,7 @@ decode_split_attend_kernel(const DecodeArgs a, const SplitLayout L, float* __res
     f32x4_t x[4][4];
     int js[4], ss[4];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {                     // all loads of this round first
+    for (int u = 0; u < 4; ++u) {                     // all loads of this pass first
       const int idx = base + u * NW * 64 + tid;
       const int s = idx / L.nb, lb = idx % L.nb;
       const int j = s * (L.slice / 4) - 1 + lb;
