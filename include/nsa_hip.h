@@ -292,7 +292,13 @@ int nsa_cmp_attn_bwd(const void* q, const void* ck, const void* cv, const void* 
  *   dq_add (optional, [total,hq,dk], must not overlap dq): added to dq in the kernel that writes it, e.g. the
  *   dq of nsa_cmp_attn_bwd, so that the sum over all three branches needs no further pass.
  *   workspace: nsa_slc_swa_bwd_workspace_bytes (pass top_n = 0 there when the selected branch is
- *   skipped). */
+ *   skipped) runs the selected branch over all tokens at once.  A smaller workspace makes it walk the tokens in
+ *   slabs (pair list and dQ partials then cover one slab; dK / dV accumulate over the slabs, every dq row is
+ *   written by its slab): nsa_slc_swa_bwd_slab_workspace_bytes gives the bytes for slabs of at least slab_tokens
+ *   tokens (counted in tiles of 64; slab_tokens <= 0: all tokens), and the call takes the largest slab its
+ *   workspace_bytes hold; the least is one tile. */
+int64_t nsa_slc_swa_bwd_slab_workspace_bytes(int total, int batch, int hq, int hkv, int dk, int dv, int top_n,
+                                             int block_size, int dtype, int slab_tokens);
 int64_t nsa_slc_swa_bwd_workspace_bytes(int total, int batch, int hq, int hkv, int dk, int dv, int top_n,
                                         int block_size, int dtype);
 int nsa_slc_swa_bwd(const void* q, const void* k, const void* v, const void* o_slc, const void* o_swa,

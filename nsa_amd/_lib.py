@@ -46,6 +46,7 @@ SIGNATURES = {
     "nsa_cmp_attn_bwd_workspace_bytes": (_L, [_I] * 6),
     "nsa_cmp_attn_bwd": (_I, [_P] * 10 + [_I] * 9 + [_F, _I, _I, _P, _P, _P, _P, _L, _P]),
     "nsa_slc_swa_bwd_workspace_bytes": (_L, [_I] * 9),
+    "nsa_slc_swa_bwd_slab_workspace_bytes": (_L, [_I] * 10),
     "nsa_slc_swa_bwd": (_I, [_P] * 16 + [_I] * 9 + [_F, _I, _I, _P, _P, _P, _P, _P, _L, _P]),
     "nsa_decode_max_compressed": (_I, []),
     "nsa_decode_split_max_compressed": (_I, []),

@@ -635,15 +635,19 @@ bwd_cast_kernel(const float* __restrict__ src, T* __restrict__ dst, long n8) {
 // requested before any is summed; TOPN = 0: any top_n (0 included), one partial at a time.
 template <typename T, int DK, int TOPN>
 __global__ void __launch_bounds__(256)
-slc_dq_merge_kernel(const int* __restrict__ slotmap, const T* __restrict__ part, const T* __restrict__ dq_in,
-                    const T* __restrict__ dq_add, T* __restrict__ dq, long total, int hq, int hkv, int top_n) {
+slc_dq_merge_kernel(const SlcArgs s, const int* __restrict__ slotmap, const T* __restrict__ part,
+                    const T* __restrict__ dq_in, const T* __restrict__ dq_add, T* __restrict__ dq, int hq, int hkv,
+                    int top_n) {
   constexpr int PPR = DK / 8;
+  int tb, te;
+  slc_token_range(s, tb, te);                       // the tokens of this slab (all of them without slabs)
   const long id = (long)blockIdx.x * 256 + threadIdx.x;
-  if (id >= total * hq * PPR) return;
   const int pc = (int)(id % PPR);
-  const long row = id / PPR;
-  const int hq_i = (int)(row % hq);
-  const long tg = row / hq;
+  const long rel = id / PPR;                        // (token - tb) * hq + head
+  const int hq_i = (int)(rel % hq);
+  const long tg = tb + rel / hq;
+  if (tg >= te) return;
+  const long row = tg * hq + hq_i;
   const int G = hq / hkv;
   const int h = hq_i / G, n = hq_i % G;
   float acc[8];
@@ -787,14 +791,31 @@ static SlcArgs slc_args_of(const SlcSwaBwdArgs& c) {
   return slc_virtual(s);           // top_n counts 64-key slots from here on
 }
 
-long slc_swa_bwd_workspace_bytes(const SlcSwaBwdArgs& c) {
+constexpr int kBwdSlabTile = 64;     // tokens per tile in which the selected branch's token slabs are counted
+
+// selected branch in slabs of `tiles` tiles of kBwdSlabTile tokens (0: all tokens at once)
+static SlcArgs slab_args_of(const SlcSwaBwdArgs& c, int tile_begin, int tiles) {
+  SlcArgs s = slc_args_of(c);
+  s.tile_tokens = kBwdSlabTile; s.tile_begin = tile_begin; s.tile_count = tiles;
+  return s;
+}
+
+static long bwd_workspace_bytes(const SlcSwaBwdArgs& c, int tiles) {
   long off = 0;
   take(off, (long)c.total * c.hq * 4);
   take(off, (long)c.total * c.hq * 4);
   take(off, (long)c.total * c.hkv * c.dk * 4);
   take(off, (long)c.total * c.hkv * c.dv * 4);
-  if (c.top_n > 0) off += slc_carve(slc_args_of(c), nullptr, nullptr, c.dtype == 1 ? 4 : 2, c.dk);
+  if (c.top_n > 0) off += slc_carve(slab_args_of(c, 0, tiles), nullptr, nullptr, c.dtype == 1 ? 4 : 2, c.dk);
   return off;
+}
+
+long slc_swa_bwd_workspace_bytes(const SlcSwaBwdArgs& c) { return bwd_workspace_bytes(c, 0); }
+
+// slab_tokens <= 0 or >= total: all tokens at once
+long slc_swa_bwd_slab_workspace_bytes(const SlcSwaBwdArgs& c, int slab_tokens) {
+  const int tiles = slab_tokens > 0 && slab_tokens < c.total ? (slab_tokens + kBwdSlabTile - 1) / kBwdSlabTile : 0;
+  return bwd_workspace_bytes(c, tiles);
 }
 
 template <typename T, int DK, int DV>
@@ -823,33 +844,52 @@ static int launch_slc_swa_bwd_t(const SlcSwaBwdArgs& c, hipStream_t st) {
     if (rc == 0) rc = launch_kv_t<T, DK, DV, kBwdSwa, kKvWaves>(a, c.total, st);
     if (rc) return rc;
   }
-  SlcWs ws{};
+  auto dq_merge = [&](const SlcArgs& s, const SlcWs* ws, long slab_tokens) {   // dq = window dQ + partials + dq_add
+    const long threads = slab_tokens * c.hq * (DK / 8);
+    const dim3 grid((unsigned)((threads + 255) / 256));
+    const int* slotmap = ws ? ws->slotmap : nullptr;
+    const T* part = ws ? reinterpret_cast<const T*>(ws->po) : nullptr;
+    const T* dq_in = swa ? reinterpret_cast<const T*>(c.dq) : nullptr;
+    const int top_n = ws ? s.top_n : 0;                    // slots per (token, head)
+    if (top_n == 16)
+      hipLaunchKernelGGL((slc_dq_merge_kernel<T, DK, 16>), grid, dim3(256), 0, st, s, slotmap, part, dq_in,
+                         reinterpret_cast<const T*>(c.dq_add), reinterpret_cast<T*>(c.dq), c.hq, c.hkv, top_n);
+    else
+      hipLaunchKernelGGL((slc_dq_merge_kernel<T, DK, 0>), grid, dim3(256), 0, st, s, slotmap, part, dq_in,
+                         reinterpret_cast<const T*>(c.dq_add), reinterpret_cast<T*>(c.dq), c.hq, c.hkv, top_n);
+  };
   if (slc) {
-    const SlcArgs s = slc_args_of(c);
-    slc_carve(s, base + off, &ws, sizeof(T), DK);
-    rc = launch_slc_bucket(s, ws, st);
-    if (rc) return rc;
     if (c.delta_slc == nullptr) launch_delta<T>(c.o_slc, c.d_o_slc, delta_slc, (long)c.total * c.hq, DV, st);
     a.d_o = c.d_o_slc; a.lse = c.lse_slc; a.delta = c.delta_slc ? c.delta_slc : delta_slc;
-    a.rowscale = c.rowscale_slc; a.ws = ws; a.slc_width = min(c.block_size, kBlk);
-    rc = launch_kv_t<T, DK, DV, kBwdSlc, 4>(a, c.total, st);
-    if (rc) return rc;
-  }
-  if (slc || c.dq_add != nullptr) {          // dq = window dQ + partials of the selected branch + dq_add
-    const long threads = (long)c.total * c.hq * (DK / 8);
-    const dim3 grid((unsigned)((threads + 255) / 256));
-    const int* slotmap = slc ? ws.slotmap : nullptr;
-    const T* part = slc ? reinterpret_cast<const T*>(ws.po) : nullptr;
-    const T* dq_in = swa ? reinterpret_cast<const T*>(c.dq) : nullptr;
-    const int top_n = slc ? slc_args_of(c).top_n : 0;      // slots per (token, head)
-    if (top_n == 16)
-      hipLaunchKernelGGL((slc_dq_merge_kernel<T, DK, 16>), grid, dim3(256), 0, st, slotmap, part, dq_in,
-                         reinterpret_cast<const T*>(c.dq_add), reinterpret_cast<T*>(c.dq), (long)c.total, c.hq, c.hkv,
-                         top_n);
-    else
-      hipLaunchKernelGGL((slc_dq_merge_kernel<T, DK, 0>), grid, dim3(256), 0, st, slotmap, part, dq_in,
-                         reinterpret_cast<const T*>(c.dq_add), reinterpret_cast<T*>(c.dq), (long)c.total, c.hq, c.hkv,
-                         top_n);
+    a.rowscale = c.rowscale_slc; a.slc_width = min(c.block_size, kBlk);
+    // Token slabs: pair list and dQ partials are sized for one slab (the largest the workspace holds); every slab
+    // is bucketed, run through the block kernel (dK / dV accumulate over the slabs) and merged into dq before the
+    // next one reuses the memory.
+    const int total_tiles = c.total / kBwdSlabTile + c.batch;
+    int slab_tiles = total_tiles;
+    if (bwd_workspace_bytes(c, 0) > c.workspace_bytes) {
+      if (bwd_workspace_bytes(c, 1) > c.workspace_bytes) return -6;
+      int lo = 1, hi = total_tiles;
+      while (lo < hi) {
+        const int mid = lo + (hi - lo + 1) / 2;
+        if (bwd_workspace_bytes(c, mid) <= c.workspace_bytes) lo = mid; else hi = mid - 1;
+      }
+      slab_tiles = lo;
+    }
+    const bool whole = slab_tiles >= total_tiles;
+    for (int t0 = 0; t0 < total_tiles; t0 += slab_tiles) {
+      const SlcArgs s = slab_args_of(c, t0, whole ? 0 : slab_tiles);
+      SlcWs ws{};
+      slc_carve(s, base + off, &ws, sizeof(T), DK);
+      rc = launch_slc_bucket(s, ws, st);
+      if (rc) return rc;
+      a.ws = ws;
+      rc = launch_kv_t<T, DK, DV, kBwdSlc, 4>(a, c.total, st);
+      if (rc) return rc;
+      dq_merge(s, &ws, whole ? (long)c.total : std::min((long)slab_tiles * kBwdSlabTile, (long)c.total));
+    }
+  } else if (c.dq_add != nullptr) {
+    dq_merge(slab_args_of(c, 0, 0), nullptr, c.total);
   } else if (!swa) {
     fill_zero(reinterpret_cast<float*>(c.dq), (long)c.total * c.hq * DK * (long)sizeof(T) / 4, st);
   }

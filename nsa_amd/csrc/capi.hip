@@ -505,6 +505,15 @@ int64_t nsa_slc_swa_bwd_workspace_bytes(int total, int batch, int hq, int hkv, i
   return nsa::slc_swa_bwd_workspace_bytes(a);
 }
 
+int64_t nsa_slc_swa_bwd_slab_workspace_bytes(int total, int batch, int hq, int hkv, int dk, int dv, int top_n,
+                                             int block_size, int dtype, int slab_tokens) {
+  if (total <= 0 || batch <= 0 || hq <= 0 || hkv <= 0 || dk <= 0 || dv <= 0 || top_n < 0) return 0;
+  nsa::SlcSwaBwdArgs a{};
+  a.total = total; a.batch = batch; a.hq = hq; a.hkv = hkv; a.dk = dk; a.dv = dv; a.top_n = top_n;
+  a.block_size = block_size; a.dtype = dtype;
+  return nsa::slc_swa_bwd_slab_workspace_bytes(a, slab_tokens);
+}
+
 int nsa_slc_swa_bwd(const void* q, const void* k, const void* v, const void* o_slc, const void* o_swa,
                     const void* d_o_slc, const void* d_o_swa, const float* lse_slc, const float* lse_swa,
                     const float* delta_slc, const float* delta_swa, const float* rowscale_slc,
@@ -531,12 +540,14 @@ int nsa_slc_swa_bwd(const void* q, const void* k, const void* v, const void* o_s
       !aligned16(workspace) || (slc && ((o_slc && !aligned16(o_slc)) || !aligned16(d_o_slc))) ||
       (swa && ((o_swa && !aligned16(o_swa)) || !aligned16(d_o_swa))))
     return fail(NSA_ERR_INVALID, "slc_swa_bwd: pointers must be 16-byte aligned");
-  if (workspace_bytes < nsa_slc_swa_bwd_workspace_bytes(total, batch, hq, hkv, dk, dv, slc ? top_n : 0, block_size, dtype))
-    return fail(NSA_ERR_INVALID, "slc_swa_bwd: workspace smaller than nsa_slc_swa_bwd_workspace_bytes");
+  if (workspace_bytes < nsa_slc_swa_bwd_slab_workspace_bytes(total, batch, hq, hkv, dk, dv, slc ? top_n : 0, block_size, dtype, 1))
+    return fail(NSA_ERR_INVALID, "slc_swa_bwd: workspace smaller than nsa_slc_swa_bwd_slab_workspace_bytes for one slab of 64 tokens");
   nsa::SlcSwaBwdArgs a{q, k, v, o_slc, o_swa, d_o_slc, d_o_swa, lse_slc, lse_swa, indices, counts, cu_seqlens, batch,
                        total, hq, hkv, dk, dv, slc ? top_n : 0, block_size, swa ? window : 0, scale, idx64, dtype, dq,
-                       dk_out, dv_out, workspace, delta_slc, delta_swa, rowscale_slc, rowscale_swa, dq_add};
+                       dk_out, dv_out, workspace, (long)workspace_bytes, delta_slc, delta_swa, rowscale_slc, rowscale_swa,
+                       dq_add};
   const int rc = nsa::launch_slc_swa_bwd(a, stream);
+  if (rc == -6) return fail(NSA_ERR_INVALID, "slc_swa_bwd: workspace smaller than one slab of 64 tokens needs");
   if (rc == -2) return fail(NSA_ERR_UNSUPPORTED, "slc_swa_bwd: head dims not built (dk,dv in (32,32),(64,64),(128,128),(192,128); fp32: no 192)");
   return finish(rc, "slc_swa_bwd");
 }

@@ -103,6 +103,7 @@ struct SlcSwaBwdArgs {
   const void* indices; const int32_t* counts; const int32_t* cu_seq;
   int batch, total, hq, hkv, dk, dv, top_n, block_size, window; float scale; int idx64, dtype;
   void* dq; void* dk_out; void* dv_out; void* workspace;
+  long workspace_bytes;      // the selected branch runs in token slabs as large as these bytes allow
   const float* delta_slc; const float* delta_swa; const float* rowscale_slc; const float* rowscale_swa;   // as above
   const void* dq_add;        // optional [total][hq][dk]: added to dq (the compressed branch's dQ); not dq itself
 };
@@ -165,6 +166,7 @@ long cmp_bwd_workspace_bytes(const CmpBwdArgs& a);
 int launch_cmp_bwd(const CmpBwdArgs& a, hipStream_t st);
 long slc_swa_bwd_workspace_bytes(const SlcSwaBwdArgs& a);
 int launch_slc_swa_bwd(const SlcSwaBwdArgs& a, hipStream_t st);
+long slc_swa_bwd_slab_workspace_bytes(const SlcSwaBwdArgs& a, int slab_tokens);
 int launch_decode(const DecodeArgs& a, hipStream_t st);
 int launch_decode_append(const void* k_new, const void* v_new, void* k_cache, void* v_cache_t, void* ck_cache,
                          void* cv_cache_t, const int32_t* pos, int batch, int hkv, int dk, int dv, int ctx_cap,

@@ -95,18 +95,6 @@ __device__ __forceinline__ int slc_slot_block(const SlcArgs& a, long th_r, int i
 
 // ---- bucket the pairs ---------------------------------------------------------------------------
 
-// Tokens [tb, te) of the slab (all tokens without one).  Every lane of the calling wavefronts takes part.
-__device__ __forceinline__ void slc_token_range(const SlcArgs& a, int& tb, int& te) {
-  tb = 0;
-  te = a.total;
-  if (a.tile_count > 0) {
-    const SeqTile s0 = find_tile(a.cu_seq, a.batch, a.tile_tokens, a.tile_begin);
-    tb = s0.valid ? s0.start + s0.t0 : a.total;
-    const SeqTile s1 = find_tile(a.cu_seq, a.batch, a.tile_tokens, a.tile_begin + a.tile_count);
-    te = s1.valid ? s1.start + s1.t0 : a.total;
-  }
-}
-
 __global__ void __launch_bounds__(256)
 slc_prep_kernel(const int32_t* __restrict__ cu, int batch, SlcWs ws, int hkv) {
   if (threadIdx.x == 0) {

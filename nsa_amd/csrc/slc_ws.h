@@ -3,6 +3,7 @@
 // map onto 64-key blocks: a multiple of 64 keys takes several slots per pick, a divisor of 64 keys is a part
 // of one 64-key block, whose first key inside that block is kept per pair (sub).
 #pragma once
+#include "common.h"
 #include "kernels.h"
 
 namespace nsa {
@@ -29,6 +30,18 @@ SlcArgs slc_virtual(const SlcArgs& a);
 // Lays the workspace out in `base` (ws == nullptr: only returns the size).  `part_width` is the row
 // width of the per-pair partial result (16 rows of part_width elements of `elem` bytes per pair).
 long slc_carve(const SlcArgs& a, void* base, SlcWs* ws, size_t elem, int part_width);
+
+// Tokens [tb, te) of the slab (all tokens without one).  Every lane of the calling wavefronts takes part.
+__device__ __forceinline__ void slc_token_range(const SlcArgs& a, int& tb, int& te) {
+  tb = 0;
+  te = a.total;
+  if (a.tile_count > 0) {
+    const SeqTile s0 = find_tile(a.cu_seq, a.batch, a.tile_tokens, a.tile_begin);
+    tb = s0.valid ? s0.start + s0.t0 : a.total;
+    const SeqTile s1 = find_tile(a.cu_seq, a.batch, a.tile_tokens, a.tile_begin + a.tile_count);
+    te = s1.valid ? s1.start + s1.t0 : a.total;
+  }
+}
 
 // Fills counts / offsets / list / slotmap / items for a.indices (a.counts optional).
 int launch_slc_bucket(const SlcArgs& a, const SlcWs& ws, hipStream_t st);

@@ -499,7 +499,10 @@ def slc_swa_bwd(q, k, v, o_slc, d_o_slc, lse_slc, o_swa, d_o_swa, lse_swa, indic
             raise ValueError("dq_add must have the shape and dtype of q")
         dq_add = _dense(dq_add)
     lib = _lib.load()
-    need = lib.nsa_slc_swa_bwd_workspace_bytes(total, batch, hq, hkv, dk, dv, top_n, block_size, _dtype_code(q))
+    geom = (total, batch, hq, hkv, dk, dv, top_n, block_size, _dtype_code(q))
+    need = lib.nsa_slc_swa_bwd_workspace_bytes(*geom)
+    if need > SLC_WORKSPACE_LIMIT:      # token slabs: the call takes the largest slab these bytes hold
+        need = max(SLC_WORKSPACE_LIMIT, lib.nsa_slc_swa_bwd_slab_workspace_bytes(*geom, 1))
     ws = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
     rc = lib.nsa_slc_swa_bwd(
         _ptr(q), _ptr(k), _ptr(v), _ptr(o_slc if slc else None), _ptr(o_swa if swa_ else None),

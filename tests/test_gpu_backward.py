@@ -159,6 +159,29 @@ def test_slc_swa_bwd_other_selection_block_sizes(lens, Hq, Hkv, Dk, Dv, S, W, bs
     _slc_swa_bwd_case(lens, Hq, Hkv, Dk, Dv, S, W, torch.bfloat16, bs)
 
 
+@pytest.mark.parametrize("lens,Hq,Hkv,Dk,Dv,S,W,bs", [([1500, 700], 16, 2, 64, 64, 16, 200, 64),
+                                                     ([90] * 11 + [400, 33], 16, 1, 128, 128, 4, 0, 32),
+                                                     ([1000], 8, 1, 192, 128, 3, 64, 128)])
+def test_slc_swa_bwd_in_token_slabs(monkeypatch, lens, Hq, Hkv, Dk, Dv, S, W, bs):
+    """A workspace that holds a fraction of the (token, pick) pairs: the selected branch walks the tokens in slabs.
+    Gradients against the oracle as in the one-slab cases, and dq bit-identical to the one-slab run (dk / dv are
+    sums of fp32 atomics, equal to rounding)."""
+    from nsa_amd import _lib
+    ops = _ops()
+    T = sum(lens)
+    geom = (T, len(lens), Hq, Hkv, Dk, Dv, S, bs, 0)
+    lib = _lib.load()
+    full = lib.nsa_slc_swa_bwd_workspace_bytes(*geom)
+    small = lib.nsa_slc_swa_bwd_slab_workspace_bytes(*geom, (T + 4) // 5)
+    assert lib.nsa_slc_swa_bwd_slab_workspace_bytes(*geom, 1) < small < full
+    one = _slc_swa_bwd_case(lens, Hq, Hkv, Dk, Dv, S, W, torch.bfloat16, bs)
+    monkeypatch.setattr(ops, "SLC_WORKSPACE_LIMIT", small)
+    slabs = _slc_swa_bwd_case(lens, Hq, Hkv, Dk, Dv, S, W, torch.bfloat16, bs)
+    assert torch.equal(one[0], slabs[0])
+    for a, b in zip(one[1:], slabs[1:]):
+        assert float((a.double() - b.double()).abs().max()) <= 2.0 ** -7 * max(1.0, float(a.abs().max()))
+
+
 def _slc_swa_bwd_case(lens, Hq, Hkv, Dk, Dv, S, W, dtype, bs):
     ops = _ops()
     T = sum(lens)
@@ -196,6 +219,7 @@ def _slc_swa_bwd_case(lens, Hq, Hkv, Dk, Dv, S, W, dtype, bs):
             _check("dq", dq[s:e], rq, dtype)
             _check("dk", dk[s:e], rk, dtype)
             _check("dv", dv[s:e], rv, dtype)
+    return dq, dk, dv
 
 
 # ------------------------------------------------------------------------------ compression
