@@ -216,6 +216,30 @@ __device__ __forceinline__ float row_reduce_scatter4(float v0, float v1, float v
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
+// The same for two tokens whose heads share the 16 rows of a tile (rows 0-7 token A, rows 8-15 token B; v_t is the
+// per-lane sum of score tile t): ra / rb receive, in lane i, the head sum of column i of token A / B.
+__device__ __forceinline__ void row_reduce_scatter2x2(float v0, float v1, float v2, float v3, float& ra, float& rb) {
+  auto rs16 = [](float a, float b) {       // even row g: a summed over rows (g, g+1); odd row: b
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+  };
+  const float x = rs16(v0, v1), y = rs16(v2, v3);      // rows 0 / 1: tiles (0, 1) resp. (2, 3) of A; rows 2 / 3: of B
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(y), false, false);
+  ra = __uint_as_float(r[0]);
+  rb = __uint_as_float(r[1]);
+}
+
+// Four tokens of up to four heads each (lane row g = token g): a 4 x 4 transpose over the lane rows, r[t] gets,
+// in lane i, the head sum of column i of token t.
+__device__ __forceinline__ void row_transpose4(float v0, float v1, float v2, float v3, float (&r)[4]) {
+  const auto a = __builtin_amdgcn_permlane32_swap(__float_as_uint(v0), __float_as_uint(v2), false, false);
+  const auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v1), __float_as_uint(v3), false, false);
+  const auto c = __builtin_amdgcn_permlane16_swap(a[0], b[0], false, false);
+  const auto d = __builtin_amdgcn_permlane16_swap(a[1], b[1], false, false);
+  r[0] = __uint_as_float(c[0]); r[1] = __uint_as_float(c[1]);
+  r[2] = __uint_as_float(d[0]); r[3] = __uint_as_float(d[1]);
+}
+
 // Block importance for the common shape: GQA group of 9..16 heads (one token per row group) and
 // the default pooling (windows of 5 columns every 4, no padding).  Writes the raw window sums to
 // a.pooled; topn_kernel below turns them into averages and picks the blocks.
@@ -228,10 +252,12 @@ __device__ __forceinline__ float row_reduce_scatter4(float v0, float v1, float v
 // the next lane (wave_shl:1), so lanes 3, 7, .., 59 each store one finished bin and lane 63 carries
 // its quad to the next step, where it is completed with that step's first column.  Every bin is
 // written exactly once, 64 contiguous bytes per token and step, with no atomics.
-template <typename T, int DK, int NG, int NW>
+// TP tokens share the 16 rows of a tile: 1 for groups of 9..16 heads, 2 for 5..8 (rows 8t .. 8t+7 = token t),
+// 4 for up to 4 heads (rows 4t .. 4t+3); rows beyond the group's heads are padding (weight 0).
+template <typename T, int DK, int NG, int NW, int TP>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NG <= 2 ? 4 : 2, NG <= 2 ? 4 : 2)))
 importance_stream_kernel(const CmpArgs a) {
-  constexpr int CH = 64, KLD = DK + kLdsRowPad<T>, NT = NW * 64, TQ = NW * NG;
+  constexpr int CH = 64, KLD = DK + kLdsRowPad<T>, NT = NW * 64, TQ = NW * NG * TP, GP = 16 / TP;
   constexpr int KPIECES = CH * DK / 8;
   constexpr int KPT = (KPIECES + NT - 1) / NT;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -257,30 +283,41 @@ importance_stream_kernel(const CmpArgs a) {
   const T* ckb = reinterpret_cast<const T*>(a.ck) + (long)coff * a.ck_row_stride + (long)(h / a.kv_rep) * a.ck_head_stride;
 
   vec8_t<T> qf[NG][DK / 32];
-  float lse_r[NG][4];        // lse * log2(e) of heads 4g+i of each token; +inf removes padded rows
-  float* prow[NG];           // this token's row of window sums
-  int ns_tok[NG];            // Ns, or 0 for a token past the end of the sequence: nothing is stored
+  float lse_r[NG][4];        // lse * log2(e) of the heads in rows 4g+i; +inf removes padded rows
+  float* prow[NG][TP];       // a token's row of window sums
+  int ns_tok[NG][TP];        // Ns, or 0 for a token past the end of the sequence: nothing is stored
 #pragma unroll
   for (int j = 0; j < NG; ++j) {
-    const int tok = st.t0 + wave * NG + j;
-    const int tc = tok < st.len ? tok : st.len - 1;
-    const int gc = n < G ? n : G - 1;
-    const T* qp = reinterpret_cast<const T*>(a.q) + (((long)st.start + tc) * a.hq + h * G + gc) * DK + 8 * g;
+    const int tok0 = st.t0 + (wave * NG + j) * TP;         // first token of this row group
+    {
+      const int tok = tok0 + n / GP, hd = n % GP;          // row n of the tile
+      const int tc = tok < st.len ? tok : st.len - 1;
+      const int gc = hd < G ? hd : G - 1;
+      const T* qp = reinterpret_cast<const T*>(a.q) + (((long)st.start + tc) * a.hq + h * G + gc) * DK + 8 * g;
 #pragma unroll
-    for (int kk = 0; kk < DK / 32; ++kk) qf[j][kk] = load8(qp + 32 * kk);
+      for (int kk = 0; kk < DK / 32; ++kk) qf[j][kk] = load8(qp + 32 * kk);
+    }
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      lse_r[j][i] = (tok < st.len && 4 * g + i < G)
-                        ? a.lse[((long)st.start + tok) * a.hq + h * G + 4 * g + i] * kLog2e
-                        : __builtin_huge_valf();
-    prow[j] = a.pooled + (((long)st.start + tc) * a.hkv + h) * a.pooled_stride;
-    ns_tok[j] = tok < st.len ? Ns : 0;
+    for (int i = 0; i < 4; ++i) {
+      const int tok = tok0 + (4 * g + i) / GP, hd = (4 * g + i) % GP;
+      lse_r[j][i] = (tok < st.len && hd < G) ? a.lse[((long)st.start + tok) * a.hq + h * G + hd] * kLog2e
+                                             : __builtin_huge_valf();
+    }
+#pragma unroll
+    for (int t = 0; t < TP; ++t) {
+      const int tok = tok0 + t;
+      const int tc = tok < st.len ? tok : st.len - 1;
+      prow[j][t] = a.pooled + (((long)st.start + tc) * a.hkv + h) * a.pooled_stride;
+      ns_tok[j][t] = tok < st.len ? Ns : 0;
+    }
   }
   wait_all_loads();
 
-  float pend[NG];            // lane 63: the quad sum of the previous step's last bin
+  float pend[NG][TP];        // lane 63: the quad sum of the previous step's last bin
 #pragma unroll
-  for (int j = 0; j < NG; ++j) pend[j] = 0.f;
+  for (int j = 0; j < NG; ++j)
+#pragma unroll
+    for (int t = 0; t < TP; ++t) pend[j][t] = 0.f;
 
   vec8_t<T> kr[KPT];
   unsigned koff[KPT];
@@ -334,15 +371,21 @@ importance_stream_kernel(const CmpArgs a) {
     const int idx = carrier ? (c0 >> 2) - 1 : (c0 >> 2) + (lane >> 2);
 #pragma unroll
     for (int j = 0; j < NG; ++j) {
-      float r = row_reduce_scatter4(v[j][0], v[j][1], v[j][2], v[j][3]);   // lane i: column c0 + i
-      r = live ? r : 0.f;
-      const float t2 = r + dpp_f32<0xB1>(r);               // quad_perm [1,0,3,2]
-      const float quad = t2 + dpp_f32<0x4E>(t2);           // quad_perm [2,3,0,1]
-      const float nxt = dpp_f32<0x130>(r);                 // wave_shl:1 -> column c0 + i + 1 (0 in lane 63)
-      const float first = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(r), 0));
-      const float val = carrier ? pend[j] + first : quad + nxt;
-      if (writer && idx >= 0 && idx < ns_tok[j]) prow[j][idx] = val;
-      pend[j] = quad;
+      float rt[TP];                                          // lane i: column c0 + i of token t
+      if constexpr (TP == 1) rt[0] = row_reduce_scatter4(v[j][0], v[j][1], v[j][2], v[j][3]);
+      else if constexpr (TP == 2) row_reduce_scatter2x2(v[j][0], v[j][1], v[j][2], v[j][3], rt[0], rt[1]);
+      else row_transpose4(v[j][0], v[j][1], v[j][2], v[j][3], rt);
+#pragma unroll
+      for (int t = 0; t < TP; ++t) {
+        const float r = live ? rt[t] : 0.f;
+        const float t2 = r + dpp_f32<0xB1>(r);               // quad_perm [1,0,3,2]
+        const float quad = t2 + dpp_f32<0x4E>(t2);           // quad_perm [2,3,0,1]
+        const float nxt = dpp_f32<0x130>(r);                 // wave_shl:1 -> column c0 + i + 1 (0 in lane 63)
+        const float first = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(r), 0));
+        const float val = carrier ? pend[j][t] + first : quad + nxt;
+        if (writer && idx >= 0 && idx < ns_tok[j][t]) prow[j][t][idx] = val;
+        pend[j][t] = quad;
+      }
     }
   };
   // operation `op` of the exponentiation of tile `tp` held in sp: per group 4 x (fma, exp), 3 adds
@@ -395,7 +438,9 @@ importance_stream_kernel(const CmpArgs a) {
     const int b = (((Nc - 1) >> 6) << 4) + 15;             // last bin of the last step: no next column
 #pragma unroll
     for (int j = 0; j < NG; ++j)
-      if (b < ns_tok[j]) prow[j][b] = pend[j];
+#pragma unroll
+      for (int t = 0; t < TP; ++t)
+        if (b < ns_tok[j][t]) prow[j][t][b] = pend[j][t];
   }
 }
 
@@ -498,15 +543,24 @@ static int launch_select_ng(const CmpArgs& a, hipStream_t st) {
 #endif
 
 // Two kernels: window sums into a.pooled, then averages + top-n per (token, head).
-template <typename T, int DK>
-static int launch_select_stream(const CmpArgs& a, hipStream_t st) {
-  constexpr int NW = NSA_STREAM_NW, NG = sizeof(T) == 2 ? NSA_STREAM_NG : NSA_STREAM_NG / 2, TQ = NW * NG;
+template <typename T, int DK, int TP>
+static int launch_importance(const CmpArgs& a, hipStream_t st) {
+  constexpr int NW = NSA_STREAM_NW, NG = sizeof(T) == 2 ? NSA_STREAM_NG : NSA_STREAM_NG / 2, TQ = NW * NG * TP;
   const size_t smem = 2 * (size_t)64 * (DK + kLdsRowPad<T>) * sizeof(T);
-  auto fn = importance_stream_kernel<T, DK, NG, NW>;
+  auto fn = importance_stream_kernel<T, DK, NG, NW, TP>;
   const int rc = set_smem(reinterpret_cast<const void*>(fn), smem);
   if (rc) return rc;
   const int tiles = a.total / TQ + a.batch;
   hipLaunchKernelGGL(fn, dim3(tiles, a.hkv), dim3(NW * 64), smem, st, a);
+  return 0;
+}
+
+template <typename T, int DK>
+static int launch_select_stream(const CmpArgs& a, hipStream_t st) {
+  const int G = a.hq / a.hkv;      // 16 rows of a score tile = 1, 2 or 4 tokens
+  const int rc = G <= 4 ? launch_importance<T, DK, 4>(a, st)
+                        : G <= 8 ? launch_importance<T, DK, 2>(a, st) : launch_importance<T, DK, 1>(a, st);
+  if (rc) return rc;
   const int rows = (int)(((long)a.total * (a.hkv / a.kv_rep) + 3) / 4);
   if (a.max_ns <= 512) hipLaunchKernelGGL(topn_kernel<8>, dim3(rows), dim3(256), 0, st, a);
   else if (a.max_ns <= 1024) hipLaunchKernelGGL(topn_kernel<16>, dim3(rows), dim3(256), 0, st, a);
@@ -517,7 +571,8 @@ static int launch_select_stream(const CmpArgs& a, hipStream_t st) {
 
 template <typename T, int DK>
 static int launch_select_t(const CmpArgs& a, hipStream_t st) {
-  if (a.pooled != nullptr && a.max_ns <= 4096 && a.top_n <= 64 && group_pow2(a.hq / a.hkv) == 16 && a.pool_k == 5 &&
+  // (groups below 16 heads run with the missing heads as padded rows: their log-sum-exp is +inf, their weight 0)
+  if (a.pooled != nullptr && a.max_ns <= 4096 && a.top_n <= 64 && a.hq / a.hkv <= 16 && a.pool_k == 5 &&
       a.pool_s == 4 && a.pool_p == 0)
     return launch_select_stream<T, DK>(a, st);
   if (a.kv_rep > 1) return -6;      // groups beyond 16 heads exist on the two-kernel schedule only
