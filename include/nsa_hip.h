@@ -257,7 +257,9 @@ int nsa_slc_swa_fused_fwd(const void* q, const void* k, const void* vt, const vo
                           int idx64, int gate_act, int dtype, void* o_slc_out, void* o_swa_out, float* lse_slc_out,
                           float* lse_swa_out, void* workspace, int64_t workspace_bytes, nsa_stream_t stream);
 
-/* Bytes of the optional workspace of nsa_slc_combine_fwd; 0 when the shape has no block-major path
+/* Bytes of the optional workspace of nsa_slc_combine_fwd (an upper bound taken for GQA groups of 16 heads: the
+ * partial results of groups of at most 8 / 4 heads have 8 / 4 rows, nsa_slc_swa_fused_workspace_bytes(..., 0) gives
+ * the exact size, which the entry points accept); 0 when the shape has no block-major path
  * (bf16 or fp16; selection blocks of 8, 16, 32 or a multiple of 64 keys, top_n * max(1, block_size / 64) <= 64).  hkv: kv heads, times hq / (16 * hkv) when the GQA group has more
  * than 16 heads (one set of partial results per sub-group of 16 query heads). */
 int64_t nsa_slc_workspace_bytes(int total, int batch, int hkv, int dk, int dv, int top_n, int block_size, int dtype);

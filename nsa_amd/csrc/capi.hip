@@ -343,7 +343,8 @@ static int slc_common_checks(const char* what, const void* q, const void* k, con
   if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "%s: scale must be positive", what);
   if (vt_cols % 64 != 0 || vt_cols < nsa_transposed_cols(total, batch)) return fail(NSA_ERR_INVALID, "%s: vt_cols too small or not a multiple of 64", what);
   if (!aligned16(q) || !aligned16(k) || !aligned16(vt) || !aligned16(workspace)) return fail(NSA_ERR_INVALID, "%s: pointers must be 16-byte aligned", what);
-  const int64_t need = nsa_slc_workspace_bytes(total, batch, hkv * *kv_rep, dk, dv, top_n, block_size, dtype);
+  // with the query heads known the partial results have as many rows as the (padded) GQA group, not 16
+  const int64_t need = nsa_slc_swa_fused_workspace_bytes(total, batch, hq, hkv, dk, dv, top_n, block_size, dtype, 0);
   if (need == 0) return fail(NSA_ERR_UNSUPPORTED, "%s: the block-major schedule needs bf16 or fp16, selection blocks of 8, 16, 32 or a multiple of 64 keys, top_n * max(1, block_size / 64) <= 64 and (dk,dv) in (64,64),(128,128),(192,128)", what);
   if (workspace_bytes < need) return fail(NSA_ERR_INVALID, "%s: workspace smaller than nsa_slc_workspace_bytes", what);
   return 0;

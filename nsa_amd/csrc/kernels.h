@@ -73,6 +73,7 @@ struct SlcArgs {
 // first three live inside the selected-attention workspace).
 struct MergeArgs {
   const int* slotmap; const float* ml; const void* po;
+  int part_rows;     // rows of one partial result in po: 16, or 8 / 4 for GQA groups of at most 8 / 4 heads
   const void* g_slc; const void* g_swa; const void* g_cmp; long gate_stride;
   const void* o_cmp; void* out;
   int top_n, hq, hkv, gate_act; float scale;

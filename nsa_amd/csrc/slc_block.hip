@@ -29,7 +29,7 @@ SlcArgs slc_virtual(const SlcArgs& a) {
 }
 
 // a: as returned by slc_virtual
-long slc_carve(const SlcArgs& a, void* base, SlcWs* ws, size_t elem, int part_width) {
+long slc_carve(const SlcArgs& a, void* base, SlcWs* ws, size_t elem, int part_width, int part_rows) {
   const int nb = a.total / kBlk + a.batch;
   const long nkeys = (long)a.hkv * nb;
   const long slots = (long)a.total * a.hkv * a.top_n;                 // slot map: every token
@@ -49,7 +49,7 @@ long slc_carve(const SlcArgs& a, void* base, SlcWs* ws, size_t elem, int part_wi
   const long o_slot = take(slots * 4);
   const long o_sub = take(pairs);
   const long o_ml = take(pairs * 2 * 16 * 4);
-  const long o_po = take(pairs * 16 * part_width * (long)elem);
+  const long o_po = take(pairs * part_rows * part_width * (long)elem);
   if (ws != nullptr) {
     char* b = reinterpret_cast<char*>(base);
     ws->blkbase = (int*)(b + o_blkbase); ws->counts = (int*)(b + o_counts); ws->offsets = (int*)(b + o_offsets);
@@ -61,7 +61,9 @@ long slc_carve(const SlcArgs& a, void* base, SlcWs* ws, size_t elem, int part_wi
   return off;
 }
 
-static long carve(const SlcArgs& a, void* base, SlcWs* ws, size_t elem) { return slc_carve(a, base, ws, elem, a.dv); }
+static long carve(const SlcArgs& a, void* base, SlcWs* ws, size_t elem) {
+  return slc_carve(a, base, ws, elem, a.dv, slc_part_rows(a));
+}
 
 long slc_workspace_bytes(const SlcArgs& a) { return carve(slc_virtual(a), nullptr, nullptr, a.dtype == 1 ? 4 : 2); }
 
@@ -396,6 +398,162 @@ slc_block_kernel(const SlcArgs a, const SlcWs ws) {
   }
 }
 
+// The same for GQA groups of at most 8 (PP = 2) or 4 (PP = 4) heads: the 16 columns of a score tile hold PP pairs of
+// the segment (columns u * GP .. u * GP + GP - 1 = the heads of pair u of the step, GP = 16 / PP), so a step of the
+// same cost serves PP pairs, and a partial result has GP rows instead of 16.
+template <typename T, int DK, int DV, bool SUB, int PP>
+__global__ void __launch_bounds__(256)
+slc_block_packed_kernel(const SlcArgs a, const SlcWs ws) {
+  constexpr int NK = DK / 32, NV = DV / 16, OLD = DV + 8, GP = 16 / PP;
+  __shared__ __attribute__((aligned(16))) T stage[4][16 * OLD];    // per wavefront: one partial, head-major
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int n = lane & 15, g = lane >> 4;
+  const int item_id = blockIdx.x * 4 + wave;
+  if (item_id >= *ws.n_items) return;
+  const int key = ws.items[2 * item_id], seg = ws.items[2 * item_id + 1];
+  const int h = key / ws.nb, gb = key % ws.nb;
+  const SeqTile st = find_tile(a.cu_seq, a.batch, kBlk, gb);      // st.t0 = first key of the block
+  if (!st.valid) return;
+  const int G = a.hq / a.hkv;
+  const int first = ws.offsets[key] + seg * kSeg;
+  const int count = min(ws.counts[key] - seg * kSeg, kSeg);
+  const float c_attn = a.scale * kLog2e;
+
+  // K block as A fragments: chunk c (32 keys) = tiles 2c, 2c+1 with permuted rows; V^T block per chunk
+  vec8_t<T> kf[4][NK], vf[2][NV];
+  {
+    const int hk = h / a.kv_rep, hkv_r = a.hkv / a.kv_rep;     // kv head of this (sub-)group, number of kv heads
+    const T* kb = reinterpret_cast<const T*>(a.k) + ((long)st.start * hkv_r + hk) * DK + 8 * g;
+    const long krow = (long)hkv_r * DK;
+#pragma unroll
+    for (int tile = 0; tile < 4; ++tile) {
+      const int row = min(st.t0 + 32 * (tile >> 1) + chunk_key_of_row(tile & 1, n), st.len - 1);
+#pragma unroll
+      for (int kk = 0; kk < NK; ++kk) kf[tile][kk] = load8(kb + row * krow + 32 * kk);
+    }
+    const T* vtb = reinterpret_cast<const T*>(a.vt) + (long)hk * DV * a.vt_cols + transposed_offset(st.start, st.b) +
+                   (long)n * a.vt_cols + st.t0 + 8 * g;
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int t = 0; t < NV; ++t) vf[c][t] = load8(vtb + t * 16L * a.vt_cols + 32 * c);
+  }
+
+  const T* qb = reinterpret_cast<const T*>(a.q);
+  T* pob = reinterpret_cast<T*>(ws.po);
+  const int u = n / GP, hd = n % GP;                     // pair of the step and head of this column
+  const int gc = hd < G ? hd : G - 1;
+  vec8_t<T> qn[NK];
+  // The segment's pair-list entries (at most one per lane) in one load; entry j is taken out with readlane.  A
+  // load from a wave-uniform address inside the loop would be waited for where it is issued, and on this
+  // hardware that wait (loads and stores share one in-order counter) also covers the stores of the pair before.
+  const uint32_t ents = ws.list[first + min(lane, count - 1)];
+  int subs = 0;
+  if (SUB) subs = ws.sub[first + min(lane, count - 1)];
+  const int steps = (count + PP - 1) / PP;
+  // the pair of this lane's column in step j (past the end: the last pair again, computed and not stored)
+  auto entry_of = [&](int j) { return (uint32_t)__shfl((int)ents, min(j * PP + u, count - 1)); };
+  uint32_t ent = entry_of(0);
+  {
+    const T* qp = qb + ((long)(ent >> 6) * a.hq + h * G + gc) * DK + 8 * g;
+#pragma unroll
+    for (int kk = 0; kk < NK; ++kk) qn[kk] = load8(qp + 32 * kk);
+  }
+  // The K / V fragments are waited for here, once (an empty asm that takes each of them): left to the compiler,
+  // their waits sit inside the loop, where the fragments are first used, and, counting down to zero, would there
+  // also wait for the query just requested.
+#pragma unroll
+  for (int tile = 0; tile < 4; ++tile)
+#pragma unroll
+    for (int kk = 0; kk < NK; ++kk) asm volatile("" ::"v"(kf[tile][kk]));
+#pragma unroll
+  for (int c = 0; c < 2; ++c)
+#pragma unroll
+    for (int t = 0; t < NV; ++t) asm volatile("" ::"v"(vf[c][t]));
+  for (int j = 0; j < steps; ++j) {
+    vec8_t<T> qf[NK];
+#pragma unroll
+    for (int kk = 0; kk < NK; ++kk) qf[kk] = qn[kk];
+    const int tg = (int)(ent >> 6);
+    const int pf = first + j * PP;                        // first pair of the step
+    const bool stored = j * PP + u < count;
+    int lo = 0;
+    if (SUB) lo = __shfl(subs, min(j * PP + u, count - 1));
+    if (j + 1 < steps) {                                  // next queries in flight while these are multiplied
+      ent = entry_of(j + 1);
+      const T* qp = qb + ((long)(ent >> 6) * a.hq + h * G + gc) * DK + 8 * g;
+#pragma unroll
+      for (int kk = 0; kk < NK; ++kk) qn[kk] = load8(qp + 32 * kk);
+    }
+    const int t_loc = tg - st.start;                      // token position inside its sequence (per column)
+    float s[16];
+    {
+      f32x4_t acc[4];
+#pragma unroll
+      for (int tile = 0; tile < 4; ++tile) {
+        acc[tile] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < NK; ++kk) acc[tile] = mma16(kf[tile][kk], qf[kk], acc[tile]);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { s[i] = acc[0][i]; s[4 + i] = acc[1][i]; s[8 + i] = acc[2][i]; s[12 + i] = acc[3][i]; }
+    }
+    if (SUB) {                                            // part of a block: its keys up to the token
+      const int hi = min(lo + a.block_size, t_loc - st.t0 + 1);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int kb = 32 * (i >> 3) + 8 * g + (i & 7);
+        if (kb < lo || kb >= hi) s[i] = kNegInf;
+      }
+    } else {                                              // the block that contains the column's token: its keys up to it
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        if (st.t0 + 32 * (i >> 3) + 8 * g + (i & 7) > t_loc) s[i] = kNegInf;
+    }
+    float mx = s[0];
+#pragma unroll
+    for (int i = 1; i < 16; ++i) mx = fmaxf(mx, s[i]);
+    mx = colgroup_max(mx);                                // finite: the first key of the pick is visible
+    float pr[16], sum = 0.f;
+    const float off = -mx * c_attn;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) { pr[i] = fast_exp2(fmaf(s[i], c_attn, off)); sum += pr[i]; }
+    sum = colgroup_sum(sum);
+    float p0[8], p1[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { p0[i] = pr[i]; p1[i] = pr[8 + i]; }
+    const vec8_t<T> pb0 = pack8<T>(p0), pb1 = pack8<T>(p1);
+    const float inv = 1.0f / sum;
+    T* srow = &stage[wave][n * OLD + 4 * g];
+#pragma unroll
+    for (int t = 0; t < NV; ++t) {
+      f32x4_t o = {0.f, 0.f, 0.f, 0.f};
+      o = mma16(vf[0][t], pb0, o);
+      o = mma16(vf[1][t], pb1, o);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) srow[t * 16 + i] = (T)(o[i] * inv);
+    }
+    // head-major rows out of LDS: 16 lanes write one full row, a wavefront instruction 4 rows
+    {
+      // row n of the staged tile = head hd of pair pf + u: consecutive pairs, GP rows each, are consecutive rows
+      T* dst = pob + (long)pf * GP * DV;
+      const int rows = min(PP, count - j * PP) * GP;
+      constexpr int PIECES = DV / 8;                       // 16-byte pieces per row
+#pragma unroll
+      for (int k = 0; k < 16 * PIECES / 64; ++k) {
+        const int e = lane + 64 * k;
+        const int r = e / PIECES, pc = e % PIECES;
+        if (r < rows) store8(dst + r * DV + pc * 8, load8(&stage[wave][r * OLD + pc * 8]));
+      }
+    }
+    if (stored) {
+      ws.ml[((long)(pf + u) * 2 + 0) * 16 + hd] = mx;
+      ws.ml[((long)(pf + u) * 2 + 1) * 16 + hd] = sum;
+    }
+  }
+}
+
 // ---- merge the partials of every token, gate, add the other branches ---------------------------
 
 // One thread per (token, q head, 8 output channels).
@@ -419,7 +577,7 @@ slc_merge_kernel(const SlcArgs a, const MergeArgs m) {
 }
 
 static MergeArgs merge_args_of(const SlcArgs& a, const SlcWs& ws) {
-  return MergeArgs{ws.slotmap, ws.ml, ws.po, a.g_slc, a.g_swa, a.g_cmp, a.gate_stride, a.o_cmp, a.out,
+  return MergeArgs{ws.slotmap, ws.ml, ws.po, slc_part_rows(a), a.g_slc, a.g_swa, a.g_cmp, a.gate_stride, a.o_cmp, a.out,
                    a.top_n, a.hq, a.hkv, a.gate_act, a.scale, a.lse};
 }
 
@@ -454,10 +612,21 @@ template <typename T, int DK, int DV>
 static int launch_partials_t(const SlcArgs& a, const SlcWs& ws, hipStream_t st) {
   const int rc = launch_slc_bucket(a, ws, st);
   if (rc) return rc;
-  if (a.block_size < kBlk)
-    hipLaunchKernelGGL((slc_block_kernel<T, DK, DV, true>), dim3((ws.items_cap + 3) / 4), dim3(256), 0, st, a, ws);
-  else
-    hipLaunchKernelGGL((slc_block_kernel<T, DK, DV, false>), dim3((ws.items_cap + 3) / 4), dim3(256), 0, st, a, ws);
+  const dim3 grid((ws.items_cap + 3) / 4);
+  const bool sub = a.block_size < kBlk;
+  switch (slc_part_rows(a)) {
+    case 4:
+      if (sub) hipLaunchKernelGGL((slc_block_packed_kernel<T, DK, DV, true, 4>), grid, dim3(256), 0, st, a, ws);
+      else hipLaunchKernelGGL((slc_block_packed_kernel<T, DK, DV, false, 4>), grid, dim3(256), 0, st, a, ws);
+      break;
+    case 8:
+      if (sub) hipLaunchKernelGGL((slc_block_packed_kernel<T, DK, DV, true, 2>), grid, dim3(256), 0, st, a, ws);
+      else hipLaunchKernelGGL((slc_block_packed_kernel<T, DK, DV, false, 2>), grid, dim3(256), 0, st, a, ws);
+      break;
+    default:
+      if (sub) hipLaunchKernelGGL((slc_block_kernel<T, DK, DV, true>), grid, dim3(256), 0, st, a, ws);
+      else hipLaunchKernelGGL((slc_block_kernel<T, DK, DV, false>), grid, dim3(256), 0, st, a, ws);
+  }
   return 0;
 }
 

@@ -43,7 +43,7 @@ __device__ __forceinline__ vec8_t<T> merge_piece(const MergeArgs& m, long tg, in
         const long p = ps[i];
         mx[i] = m.ml[(p * 2) * 16 + n];
         l[i] = m.ml[(p * 2 + 1) * 16 + n];
-        o[i] = load8(pob + (p * 16 + n) * DV + pc * 8);
+        o[i] = load8(pob + (p * m.part_rows + n) * DV + pc * 8);
       }
     }
 #pragma unroll
@@ -63,7 +63,7 @@ __device__ __forceinline__ vec8_t<T> merge_piece(const MergeArgs& m, long tg, in
       if (p < 0) continue;
       const float mi = m.ml[(p * 2) * 16 + n];
       const float l = m.ml[(p * 2 + 1) * 16 + n];
-      const vec8_t<T> o = load8(pob + (p * 16 + n) * DV + pc * 8);
+      const vec8_t<T> o = load8(pob + (p * m.part_rows + n) * DV + pc * 8);
       const float m_new = fmaxf(M, mi);
       const float r_old = fast_exp2((M - m_new) * c_attn);        // 0 for the first partial
       const float w = fast_exp2((mi - m_new) * c_attn) * l;
@@ -150,8 +150,8 @@ __device__ __forceinline__ void merge_two(const MergeArgs& m, long tg, int h, in
       const long p = ps[i];
       mx[i] = m.ml[(p * 2) * 16 + n];
       l[i] = m.ml[(p * 2 + 1) * 16 + n];
-      oa[i] = load8(pob + (p * 16 + n) * DV + pc_a * 8);
-      ob[i] = load8(pob + (p * 16 + n) * DV + pc_b * 8);
+      oa[i] = load8(pob + (p * m.part_rows + n) * DV + pc_a * 8);
+      ob[i] = load8(pob + (p * m.part_rows + n) * DV + pc_b * 8);
     }
   }
   float M = kNegInf, den = 0.f, acc_a[8], acc_b[8];

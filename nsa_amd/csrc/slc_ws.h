@@ -29,7 +29,16 @@ SlcArgs slc_virtual(const SlcArgs& a);
 
 // Lays the workspace out in `base` (ws == nullptr: only returns the size).  `part_width` is the row
 // width of the per-pair partial result (16 rows of part_width elements of `elem` bytes per pair).
-long slc_carve(const SlcArgs& a, void* base, SlcWs* ws, size_t elem, int part_width);
+// part_rows: rows of a pair's partial result (16; the forward uses slc_part_rows).
+long slc_carve(const SlcArgs& a, void* base, SlcWs* ws, size_t elem, int part_width, int part_rows = 16);
+
+// Rows of a forward partial result: the heads of the GQA group padded to 4, 8 or 16 (16 when the query heads are
+// not known, as in a size query by kv heads alone).
+inline int slc_part_rows(const SlcArgs& a) {
+  if (a.hq <= 0 || a.hkv <= 0) return 16;
+  const int g = a.hq / a.hkv;
+  return g <= 4 ? 4 : g <= 8 ? 8 : 16;
+}
 
 // Tokens [tb, te) of the slab (all tokens without one).  Every lane of the calling wavefronts takes part.
 __device__ __forceinline__ void slc_token_range(const SlcArgs& a, int& tb, int& te) {

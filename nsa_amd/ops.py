@@ -296,8 +296,8 @@ def slc_combine(q, k, vt, indices, counts, g_slc, g_swa, g_cmp, o_swa, o_cmp, cu
 def slc_workspace(q, hkv, dv, top_n, block_size, batch):
     """Workspace tensor of the block-major selected attention, or None when the shape has none."""
     total, hq, dk = q.shape
-    need = _lib.load().nsa_slc_workspace_bytes(total, batch, hkv * head_subgroups(hq, hkv), dk, dv, top_n, block_size,
-                                               _dtype_code(q))
+    need = _lib.load().nsa_slc_swa_fused_workspace_bytes(total, batch, hq, hkv, dk, dv, top_n, block_size,
+                                                         _dtype_code(q), 0)
     if need <= 0 or need > SLC_WORKSPACE_LIMIT:
         return None
     return torch.empty(need, dtype=torch.uint8, device=q.device)

@@ -267,7 +267,10 @@ def _random_indices(T, Hkv, S, bs, seed, poison=True):
                                                    # other selection block sizes on the 64-key schedule: parts of
                                                    # a block (8, 16, 32 keys) and several blocks per pick (128, 192)
                                                    ([300, 90], 16, 1, 64, 64, 5, 32), ([300], 8, 2, 128, 128, 4, 8),
-                                                   ([700], 16, 1, 64, 64, 3, 128), ([900, 100], 32, 2, 192, 128, 2, 192)])
+                                                   ([700], 16, 1, 64, 64, 3, 128), ([900, 100], 32, 2, 192, 128, 2, 192),
+                                                   # groups of 8, 6 and 2 heads: 2 resp. 4 pairs share a score tile
+                                                   ([330, 77], 16, 2, 128, 128, 5, 64), ([300], 12, 2, 64, 64, 3, 32),
+                                                   ([500], 2, 1, 192, 128, 16, 64)])
 def test_slc_only(dtype, lens, Hq, Hkv, Dk, Dv, S, bs):
     ops = _ops()
     T = sum(lens)
@@ -299,7 +302,8 @@ def test_slc_only(dtype, lens, Hq, Hkv, Dk, Dv, S, bs):
 
 @pytest.mark.parametrize("lens,Hq,Hkv,Dk,Dv,S,W", [([512, 100], 32, 2, 128, 128, 8, 128), ([200], 16, 1, 192, 128, 3, 64),
                                                   ([384], 4, 1, 64, 64, 4, 512), ([700, 330], 24, 2, 64, 64, 16, 256),
-                                                  ([700, 330], 64, 2, 128, 128, 16, 256), ([400], 48, 1, 192, 128, 4, 64)])
+                                                  ([700, 330], 64, 2, 128, 128, 16, 256), ([400], 48, 1, 192, 128, 4, 64),
+                                                  ([700, 130], 16, 2, 128, 128, 16, 100), ([520], 3, 1, 64, 64, 7, 64)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_fused_partials_and_window_merge(lens, Hq, Hkv, Dk, Dv, S, W, dtype):
     """nsa_slc_partials_fwd + nsa_swa_merge_fwd against nsa_swa_fwd + nsa_slc_combine_fwd (token-major
