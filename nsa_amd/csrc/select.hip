@@ -272,10 +272,12 @@ importance_stream_kernel(const CmpArgs a) {
   const int h = blockIdx.y;
   const int coff = a.cu_cmp[st.b];
   const int Nc = a.cu_cmp[st.b + 1] - coff;
+  // pooling windows of ps + 1 columns every ps columns, no padding; ps = 2, 4 or 8 (selection blocks of 2, 4, 8 strides)
+  const int ps = a.pool_s, lps = ps == 2 ? 1 : ps == 4 ? 2 : 3;
   int Ns = 0;
-  if (Nc >= 5) {
-    Ns = (Nc - 5 + 3) / 4 + 1;
-    if ((Ns - 1) * 4 >= Nc) --Ns;
+  if (Nc >= ps + 1) {
+    Ns = (Nc - 2) / ps + 1;                     // ceil((Nc - (ps + 1)) / ps) + 1
+    if ((Ns - 1) * ps >= Nc) --Ns;
   }
   Ns = min(Ns, a.max_ns);
   if (Ns == 0) return;
@@ -355,7 +357,7 @@ importance_stream_kernel(const CmpArgs a) {
   gload(0);
   lstore(0);
   __syncthreads();
-  const bool writer = (lane & 3) == 3;
+  const bool writer = (lane & (ps - 1)) == ps - 1;       // last lane of a window's ps own columns
   const bool carrier = lane == 63;
   // Software pipeline inside every wavefront: while the matrix unit multiplies score tile i, the
   // vector ALU exponentiates tile i-1 (kept in `sp`), one or two operations after each MFMA.
@@ -368,7 +370,7 @@ importance_stream_kernel(const CmpArgs a) {
   for (int j = 0; j < NG; ++j) sp[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   auto pool_store = [&](int c0) {          // window sums of the step that started at column c0
     const bool live = c0 + lane < Nc;
-    const int idx = carrier ? (c0 >> 2) - 1 : (c0 >> 2) + (lane >> 2);
+    const int idx = carrier ? (c0 >> lps) - 1 : (c0 >> lps) + (lane >> lps);
 #pragma unroll
     for (int j = 0; j < NG; ++j) {
       float rt[TP];                                          // lane i: column c0 + i of token t
@@ -378,8 +380,9 @@ importance_stream_kernel(const CmpArgs a) {
 #pragma unroll
       for (int t = 0; t < TP; ++t) {
         const float r = live ? rt[t] : 0.f;
-        const float t2 = r + dpp_f32<0xB1>(r);               // quad_perm [1,0,3,2]
-        const float quad = t2 + dpp_f32<0x4E>(t2);           // quad_perm [2,3,0,1]
+        float quad = r + dpp_f32<0xB1>(r);                   // quad_perm [1,0,3,2]: pairs
+        if (ps >= 4) quad += dpp_f32<0x4E>(quad);            // quad_perm [2,3,0,1]: quads
+        if (ps == 8) quad += __shfl_xor(quad, 4);            // eight columns
         const float nxt = dpp_f32<0x130>(r);                 // wave_shl:1 -> column c0 + i + 1 (0 in lane 63)
         const float first = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(r), 0));
         const float val = carrier ? pend[j][t] + first : quad + nxt;
@@ -435,7 +438,7 @@ importance_stream_kernel(const CmpArgs a) {
   for (int op = 0; op < NOPS; ++op) exp_op(op, 3);
   pool_store(((Nc - 1) >> 6) << 6);
   if (carrier) {
-    const int b = (((Nc - 1) >> 6) << 4) + 15;             // last bin of the last step: no next column
+    const int b = ((((Nc - 1) >> 6) << 6) >> lps) + (64 >> lps) - 1;   // last bin of the last step: no next column
 #pragma unroll
     for (int j = 0; j < NG; ++j)
 #pragma unroll
@@ -572,8 +575,8 @@ static int launch_select_stream(const CmpArgs& a, hipStream_t st) {
 template <typename T, int DK>
 static int launch_select_t(const CmpArgs& a, hipStream_t st) {
   // (groups below 16 heads run with the missing heads as padded rows: their log-sum-exp is +inf, their weight 0)
-  if (a.pooled != nullptr && a.max_ns <= 4096 && a.top_n <= 64 && a.hq / a.hkv <= 16 && a.pool_k == 5 &&
-      a.pool_s == 4 && a.pool_p == 0)
+  if (a.pooled != nullptr && a.max_ns <= 4096 && a.top_n <= 64 && a.hq / a.hkv <= 16 &&
+      (a.pool_s == 2 || a.pool_s == 4 || a.pool_s == 8) && a.pool_k == a.pool_s + 1 && a.pool_p == 0)
     return launch_select_stream<T, DK>(a, st);
   if (a.kv_rep > 1) return -6;      // groups beyond 16 heads exist on the two-kernel schedule only
   CmpArgs b = a;
