@@ -43,8 +43,8 @@ struct StreamParams {
 
 // MERGE (sliding window only): 0 = write the branch output; otherwise the epilogue merges the
 // block-major selected-attention partials of its rows, applies the gates, adds the compressed
-// branch and writes the final output, so the window result never goes to memory (1 = any top_n,
-// 16 = top_n of exactly 16 with all partial loads in flight).
+// branch and writes the final output, so the window result never goes to memory (16 = top_n of exactly 16, all
+// partial loads in flight; 2 = any top_n, the picks in rounds of 16; 1 = one partial at a time, kept for reference).
 template <typename T, int DK, int DV, int NG, int CH, int NW, bool CMP, int MERGE = 0>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 stream_attn_kernel(const StreamParams a) {
@@ -380,7 +380,7 @@ stream_attn_kernel(const StreamParams a) {
     store_rows<T, DV>(stage + n * OLD, grp[j].o, inv, g);
     constexpr int PIECES = DV / 8;
     const int gi = wave * NG + j;
-    if constexpr (MERGE == 16) {
+    if constexpr (MERGE == 16 || MERGE == 2) {
       // a lane takes two pieces (pc, pc + PIECES / 2) of one row, so that 32 partial loads are in flight per lane
       constexpr int HALF = PIECES / 2;
 #pragma unroll
@@ -394,7 +394,7 @@ stream_attn_kernel(const StreamParams a) {
             const long orow = tg * a.hq + h * G + rr.gidx;
             const vec8_t<T> pa = load8(stage + r * OLD + pc * 8), pb = load8(stage + r * OLD + (pc + HALF) * 8);
             vec8_t<T> ra, rb;
-            merge_two<T, DV, 16>(a.mg, tg, h, rr.gidx, orow, pc, pc + HALF, pa, pb, ra, rb);
+            merge_two<T, DV, 16, MERGE == 16>(a.mg, tg, h, rr.gidx, orow, pc, pc + HALF, pa, pb, ra, rb);
             store8(reinterpret_cast<T*>(a.mg.out) + orow * DV + pc * 8, ra);
             store8(reinterpret_cast<T*>(a.mg.out) + orow * DV + (pc + HALF) * 8, rb);
           }
@@ -663,7 +663,7 @@ static int launch_swa_merge_t(const SwaArgs& a, const MergeArgs& m, hipStream_t 
   StreamParams p{a.q, a.k, a.vt, nullptr, nullptr, a.cu_seq, a.cu_seq, a.batch, a.hq, a.hkv, (long)(a.hkv / a.kv_rep) * DK,
                  (long)DK, a.vt_cols, 0, 0, a.window, 1, a.scale, m, a.lse, a.kv_rep, 0, a.tile_begin};
   if (m.top_n == 16) return launch_stream_t<T, DK, DV, false, 16>(p, a.total, st, a.tile_count);
-  return launch_stream_t<T, DK, DV, false, 1>(p, a.total, st, a.tile_count);
+  return launch_stream_t<T, DK, DV, false, 2>(p, a.total, st, a.tile_count);    // picks merged in rounds of 16
 }
 
 template <typename T, int DK, int DV>

@@ -632,7 +632,7 @@ bwd_cast_kernel(const float* __restrict__ src, T* __restrict__ dst, long n8) {
 
 // dq[token][head][8 channels] = (dq_in) + (dq_add) + sum over the token's usable picks of the pair partials.
 // TOPN > 0: top_n == TOPN, the slot map is read with vector loads and all partials of the piece are
-// requested before any is summed; TOPN = 0: any top_n (0 included), one partial at a time.
+// requested before any is summed; TOPN = 0: any top_n (0 included), in rounds of 16 slots.
 template <typename T, int DK, int TOPN>
 __global__ void __launch_bounds__(256)
 slc_dq_merge_kernel(const SlcArgs s, const int* __restrict__ slotmap, const T* __restrict__ part,
@@ -679,12 +679,24 @@ slc_dq_merge_kernel(const SlcArgs s, const int* __restrict__ slotmap, const T* _
 #pragma unroll
       for (int e = 0; e < 8; ++e) acc[e] += (float)x[i][e];
   } else {
-    for (int i = 0; i < top_n; ++i) {
-      const long p = slotmap[base + i];
-      if (p < 0) continue;
-      const vec8_t<T> x = load8(part + (p * 16 + n) * DK + pc * 8);
+    // any top_n: rounds of 16 slots, all partials of a round requested before the first is added
+    constexpr int R = 16;
+    for (int r0 = 0; r0 < top_n; r0 += R) {
+      int ps[R];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[e] += (float)x[e];
+      for (int i = 0; i < R; ++i) ps[i] = r0 + i < top_n ? slotmap[base + r0 + i] : -1;
+#pragma unroll
+      for (int i = 0; i < R; ++i) asm volatile("" ::"v"(ps[i]));
+      vec8_t<T> x[R];
+#pragma unroll
+      for (int i = 0; i < R; ++i) {
+        x[i] = zero8<T>();
+        if (ps[i] >= 0) x[i] = load8(part + ((long)ps[i] * 16 + n) * DK + pc * 8);
+      }
+#pragma unroll
+      for (int i = 0; i < R; ++i)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] += (float)x[i][e];
     }
   }
 #pragma unroll

@@ -557,7 +557,7 @@ slc_block_packed_kernel(const SlcArgs a, const SlcWs ws) {
 // ---- merge the partials of every token, gate, add the other branches ---------------------------
 
 // One thread per (token, q head, 8 output channels).
-template <typename T, int DV, int TOPN>
+template <typename T, int DV, int TOPN, bool EXACT>
 __global__ void __launch_bounds__(256)
 slc_merge_kernel(const SlcArgs a, const MergeArgs m) {
   constexpr int PPR = DV / 8;                                     // 8-channel pieces per output row
@@ -571,7 +571,7 @@ slc_merge_kernel(const SlcArgs a, const MergeArgs m) {
   const T* osw = reinterpret_cast<const T*>(a.o_swa);
   vec8_t<T> o_swa = zero8<T>();
   if (osw) o_swa = load8(osw + row * DV + pc * 8);
-  const vec8_t<T> r = merge_piece<T, DV, TOPN>(m, tg, hq_i / G, hq_i % G, row, pc, osw != nullptr, o_swa);
+  const vec8_t<T> r = merge_piece<T, DV, TOPN, EXACT>(m, tg, hq_i / G, hq_i % G, row, pc, osw != nullptr, o_swa);
   store8(reinterpret_cast<T*>(a.out) + row * DV + pc * 8, r);
   if (m.lse != nullptr && pc == 0) m.lse[row] = merge_lse(m, tg, hq_i / G, hq_i % G);
 }
@@ -635,8 +635,8 @@ static int launch_merge_t(const SlcArgs& a, const SlcWs& ws, hipStream_t st) {
   const long threads = (long)a.total * a.hq * (DV / 8);
   const dim3 mg((int)((threads + 255) / 256));
   const MergeArgs m = merge_args_of(a, ws);
-  if (a.top_n == 16) hipLaunchKernelGGL((slc_merge_kernel<T, DV, 16>), mg, dim3(256), 0, st, a, m);
-  else hipLaunchKernelGGL((slc_merge_kernel<T, DV, 0>), mg, dim3(256), 0, st, a, m);
+  if (a.top_n == 16) hipLaunchKernelGGL((slc_merge_kernel<T, DV, 16, true>), mg, dim3(256), 0, st, a, m);
+  else hipLaunchKernelGGL((slc_merge_kernel<T, DV, 16, false>), mg, dim3(256), 0, st, a, m);   // rounds of 16 picks
   return 0;
 }
 
