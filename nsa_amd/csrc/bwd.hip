@@ -454,9 +454,12 @@ bwd_kv_kernel(const BwdArgs a) {
 // ---- query-stationary: dQ of the compressed and sliding branches -----------------------------------
 
 // kQWaves / 4 wavefronts per SIMD.
-template <typename T, int DK, int DV, int MODE, int NW>
+// TP tokens share the 16 columns of a wavefront (GQA groups of at most 16 / TP heads: column n = head n % GP of
+// token n / GP, GP = 16 / TP); a column's key limits are then per lane.
+template <typename T, int DK, int DV, int MODE, int NW, int TP>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW / 4, NW / 4)))
 bwd_q_kernel(const BwdArgs a) {
+  constexpr int GP = 16 / TP;
   constexpr int KLD = DK + kLdsPad<T, true>, VLD = DV + kLdsPad<T, true>, NT = NW * 64;
   constexpr int KP = 32 * DK / 8, VP = 32 * DV / 8;
   constexpr int KPT = (KP + NT - 1) / NT, VPT = (VP + NT - 1) / NT;
@@ -470,12 +473,13 @@ bwd_q_kernel(const BwdArgs a) {
   const int G = a.hq / a.hkv;
   // compressed branch: the work of a tile grows with its position, so the last tiles start first
   const int tile_id = MODE == kBwdCmp ? (int)(gridDim.x - 1 - blockIdx.x) : (int)blockIdx.x;
-  const SeqTile st = find_tile(a.cu_seq, a.batch, NW, tile_id);
+  const SeqTile st = find_tile(a.cu_seq, a.batch, NW * TP, tile_id);
   if (!st.valid) return;
   const int h = blockIdx.y;
-  const int tok = st.t0 + wave;
+  const int hd = n % GP;                                   // head of this lane's column
+  const int tok = st.t0 + wave * TP + n / GP;              // its token
   const bool tokvalid = tok < st.len;
-  const int t_last = min(st.t0 + NW, st.len) - 1;
+  const int t_last = min(st.t0 + NW * TP, st.len) - 1;
 
   int koff, nkeys;
   if (MODE == kBwdCmp) { koff = a.cu_key[st.b]; nkeys = a.cu_key[st.b + 1] - koff; }
@@ -489,11 +493,15 @@ bwd_q_kernel(const BwdArgs a) {
   const int c_end = last_visible(t_last) + 1;
   const int my_hi = tokvalid ? last_visible(tok) : -1;
   const int my_lo = MODE == kBwdSwa ? tok - a.window + 1 : 0;
+  // wavefront-uniform limits over its TP tokens
+  const int w_tok0 = st.t0 + wave * TP;
+  const int w_hi = w_tok0 < st.len ? last_visible(min(w_tok0 + TP - 1, st.len - 1)) : -1;
+  const int w_lo = MODE == kBwdSwa ? w_tok0 - a.window + 1 : 0;
 
   vec8_t<T> qf[DK / 32], dof[DV / 32];
   float lse2, dl;
   {
-    const long row = ((long)st.start + min(tok, st.len - 1)) * a.hq + h * G + min(n, G - 1);
+    const long row = ((long)st.start + min(tok, st.len - 1)) * a.hq + h * G + min(hd, G - 1);
     const T* qp = reinterpret_cast<const T*>(a.q) + row * DK + 8 * g;
     const T* dp = reinterpret_cast<const T*>(a.d_o) + row * DV + 8 * g;
 #pragma unroll
@@ -562,7 +570,7 @@ bwd_q_kernel(const BwdArgs a) {
   for (int c0 = c_begin; c0 < c_end; c0 += 32) {
     const bool has_next = c0 + 32 < c_end;
     if (has_next) gload(c0 + 32);
-    if (c0 <= my_hi && c0 + 31 >= my_lo) {           // wavefront uniform: one token per wavefront
+    if (c0 <= w_hi && c0 + 31 >= w_lo) {             // wavefront uniform
       const T* ks = lds + buf * STAGE;
       const T* vs = ks + 32 * KLD;
       float s[8], dp[8], ds[8];
@@ -571,7 +579,7 @@ bwd_q_kernel(const BwdArgs a) {
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const int key = c0 + lane_row32(g, j);
-        const bool ok = key >= my_lo && key <= my_hi && n < G;
+        const bool ok = key >= my_lo && key <= my_hi && hd < G;
         const float e = fast_exp2(fmaf(s[j], c_attn, -lse2));
         ds[j] = ok ? e * (dp[j] - dl) : 0.f;
       }
@@ -584,8 +592,8 @@ bwd_q_kernel(const BwdArgs a) {
     buf ^= 1;
   }
 
-  if (tokvalid && n < G) {
-    T* dqp = reinterpret_cast<T*>(a.dq) + (((long)st.start + tok) * a.hq + h * G + n) * DK + 4 * g;
+  if (tokvalid && hd < G) {
+    T* dqp = reinterpret_cast<T*>(a.dq) + (((long)st.start + tok) * a.hq + h * G + hd) * DK + 4 * g;
 #pragma unroll
     for (int t = 0; t < DK / 16; ++t) store4(dqp + 16 * t, acc[t], a.scale);
   }
@@ -726,15 +734,22 @@ static int launch_kv_t(const BwdArgs& a, int key_rows, hipStream_t st) {
   return 0;
 }
 
-template <typename T, int DK, int DV, int MODE>
-static int launch_q_t(const BwdArgs& a, hipStream_t st) {
+template <typename T, int DK, int DV, int MODE, int TP>
+static int launch_q_impl(const BwdArgs& a, hipStream_t st) {
   constexpr int NW = kQWaves;
   const size_t smem = 2 * (size_t)(32 * (DK + kLdsPad<T, true>) + 32 * (DV + kLdsPad<T, true>)) * sizeof(T);
-  auto fn = bwd_q_kernel<T, DK, DV, MODE, NW>;
+  auto fn = bwd_q_kernel<T, DK, DV, MODE, NW, TP>;
   const int rc = set_smem(reinterpret_cast<const void*>(fn), smem);
   if (rc) return rc;
-  hipLaunchKernelGGL(fn, dim3(a.total / NW + a.batch, a.hkv), dim3(NW * 64), smem, st, a);
+  hipLaunchKernelGGL(fn, dim3(a.total / (NW * TP) + a.batch, a.hkv), dim3(NW * 64), smem, st, a);
   return 0;
+}
+
+template <typename T, int DK, int DV, int MODE>
+static int launch_q_t(const BwdArgs& a, hipStream_t st) {
+  const int G = a.hq / a.hkv;       // tokens per wavefront: 4 / 2 / 1 for groups of at most 4 / 8 / 16 heads
+  return G <= 4 ? launch_q_impl<T, DK, DV, MODE, 4>(a, st)
+                : G <= 8 ? launch_q_impl<T, DK, DV, MODE, 2>(a, st) : launch_q_impl<T, DK, DV, MODE, 1>(a, st);
 }
 
 static void fill_zero(float* p, long n, hipStream_t st) {        // n is a multiple of 4
