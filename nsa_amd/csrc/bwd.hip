@@ -113,10 +113,14 @@ __device__ __forceinline__ void store4(float* p, const f32x4_t& v, float s) {
 
 // Two wavefronts per SIMD: left alone the compiler takes 264 registers (one wavefront per SIMD); a budget of
 // 168 (three) spills the accumulators and more than doubles the run time.
-template <typename T, int DK, int DV, int MODE, int NW>
+// TP (window and compressed modes): tokens per 16 rows of a chunk for GQA groups of at most 16 / TP heads; row r of
+// a chunk is head r % GP of the chunk's token r / GP (GP = 16 / TP, TPC = 2 * TP tokens per chunk).
+template <typename T, int DK, int DV, int MODE, int NW, int TP = 1>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 bwd_kv_kernel(const BwdArgs a) {
   constexpr bool X32 = MODE != kBwdSlc;
+  constexpr int GP = 16 / TP, TPC = 2 * TP;
+  static_assert(MODE != kBwdSlc || TP == 1, "the selected branch keeps one pair per 16 rows");
   constexpr int QLD = DK + kLdsPad<T, X32>, OLD = DV + kLdsPad<T, X32>, NT = NW * 64, SLD = kBlk + 8;
   constexpr int QP = 32 * DK / 8, OP = 32 * DV / 8;                 // 16-byte pieces of one chunk
   constexpr int QPT = (QP + NT - 1) / NT, OPT = (OP + NT - 1) / NT;
@@ -162,13 +166,13 @@ bwd_kv_kernel(const BwdArgs a) {
     seq_start = st.start; key0 = st.t0; nkeys = st.len; key_base = st.start;
     t_begin = key0;
     t_end = min(key0 + NW * 16 + a.window - 1, st.len);
-    nchunks = (t_end - t_begin + 1) >> 1;
+    nchunks = (t_end - t_begin + TPC - 1) / TPC;
     // The key tiles resident on an XCD are 64 tokens apart, so in plain order tile i would stream a token 32
     // chunks after tile i + 1 did, long after it left the L2.  A full window spans `period` chunks and so holds
     // every chunk number modulo `period` once: each tile starts at its multiple of `period` and wraps around,
     // which makes the workgroups that run side by side stream the same tokens at the same time.
-    const int period = (NW * 16 + a.window) >> 1;
-    rot = (period - (t_begin >> 1) % period) % period;
+    const int period = (NW * 16 + a.window + TPC - 1) / TPC;
+    rot = (period - (t_begin / TPC) % period) % period;
     if (rot >= nchunks) rot = 0;
   } else {
     // The same idea for the compressed branch: all key tiles of one token item stream the same q / dO rows,
@@ -186,10 +190,10 @@ bwd_kv_kernel(const BwdArgs a) {
     seq_start = a.cu_seq[st.b];
     const int seq_len = a.cu_seq[st.b + 1] - seq_start;
     const int t_first = a.causal ? key0 * a.stride + a.block : 0;
-    t_begin = max(ti * kCmpSplit, t_first) & ~1;
+    t_begin = max(ti * kCmpSplit, t_first) & ~(TPC - 1);
     t_end = min((ti + 1) * kCmpSplit, seq_len);
     if (t_begin >= t_end) return;
-    nchunks = (t_end - t_begin + 1) >> 1;
+    nchunks = (t_end - t_begin + TPC - 1) / TPC;
   }
   if (nchunks <= 0) return;
 
@@ -207,7 +211,7 @@ bwd_kv_kernel(const BwdArgs a) {
       posB = vB ? (int)(a.ws.list[first + 2 * c + 1] >> 6) - seq_start : posA;
     } else {
       if (MODE == kBwdSwa) { c += rot; if (c >= nchunks) c -= nchunks; }
-      posA = t_begin + 2 * c;
+      posA = t_begin + TPC * c;
       vB = posA + 1 < t_end;
       posB = vB ? posA + 1 : posA;
     }
@@ -244,14 +248,20 @@ bwd_kv_kernel(const BwdArgs a) {
   float ors[OPT], sr = 0.f, srs = 1.f;       // the gates of the staged rows (1 without a.rowscale)
 #pragma unroll
   for (int i = 0; i < OPT; ++i) ors[i] = 1.f;
+  // token (position in the sequence, clamped to the last one of the work item) and head of row r of a chunk
+  auto row_tok = [&](int r, int posA, int posB) -> int {
+    if (MODE == kBwdSlc) return (r >> 4) ? posB : posA;
+    return min(posA + r / GP, t_end - 1);
+  };
+  auto row_head = [&](int r) -> int { return min(r % GP, G - 1); };
   auto gload = [&](int posA, int posB) {
 #pragma unroll
     for (int i = 0; i < QPT; ++i) {
       const int p = tid + i * NT;
       if (QP % NT == 0 || p < QP) {
         const int r = p / (DK / 8), pc = p % (DK / 8);
-        const long tg = seq_start + ((r >> 4) ? posB : posA);
-        qr[i] = load8(qb + (tg * a.hq + h * G + min(r & 15, G - 1)) * DK + pc * 8);
+        const long tg = seq_start + row_tok(r, posA, posB);
+        qr[i] = load8(qb + (tg * a.hq + h * G + row_head(r)) * DK + pc * 8);
       }
     }
 #pragma unroll
@@ -259,16 +269,16 @@ bwd_kv_kernel(const BwdArgs a) {
       const int p = tid + i * NT;
       if (OP % NT == 0 || p < OP) {
         const int r = p / (DV / 8), pc = p % (DV / 8);
-        const long tg = seq_start + ((r >> 4) ? posB : posA);
-        const long row = tg * a.hq + h * G + min(r & 15, G - 1);
+        const long tg = seq_start + row_tok(r, posA, posB);
+        const long row = tg * a.hq + h * G + row_head(r);
         orr[i] = load8(dob + row * DV + pc * 8);
         if (a.rowscale != nullptr) ors[i] = a.rowscale[row];       // used in lstore: nothing here waits for a load
       }
     }
     if (tid < 64) {
       const int r = tid & 31;
-      const long tg = seq_start + ((r >> 4) ? posB : posA);
-      const long row = tg * a.hq + h * G + min(r & 15, G - 1);
+      const long tg = seq_start + row_tok(r, posA, posB);
+      const long row = tg * a.hq + h * G + row_head(r);
       sr = tid < 32 ? a.lse[row] : a.delta[row];
       if (a.rowscale != nullptr) srs = a.rowscale[row];
     }
@@ -331,15 +341,24 @@ bwd_kv_kernel(const BwdArgs a) {
     const T* qs = lds + buf * STAGE;
     const T* os = qs + 32 * QLD;
     const float* ss = stat + buf * 64;
-    // the 8 rows of this lane (chunk_row(g, 0..7)) are heads of one token
-    const int tokpos = (g >> 1) ? posB : posA;
-    bool vis = keyvalid && ((g >> 1) == 0 || vB);
-    if (MODE == kBwdSwa) vis = vis && keypos <= tokpos && keypos > tokpos - a.window;
-    else if (MODE == kBwdSlc) {
-      vis = vis && keypos <= tokpos;
+    // the 8 rows of this lane: chunk_row(g, 0..3) are heads of one token, chunk_row(g, 4..7) of one token (the
+    // same one unless tokens share the 16 rows of a tile)
+    bool vis, vis_hi;
+    if (MODE == kBwdSlc) {
+      const int tokpos = (g >> 1) ? posB : posA;
+      vis = keyvalid && ((g >> 1) == 0 || vB) && keypos <= tokpos;
       if (parts) vis = vis && (unsigned)(keypos - key0 - ((g >> 1) ? subB : subA)) < (unsigned)a.slc_width;
+      vis_hi = vis;
+    } else {
+      auto sees = [&](int tokpos) -> bool {
+        bool v = keyvalid && tokpos < t_end;
+        if (MODE == kBwdSwa) v = v && keypos <= tokpos && keypos > tokpos - a.window;
+        else if (a.causal) v = v && keypos * a.stride + a.block <= tokpos;
+        return v;
+      };
+      vis = sees(posA + chunk_row<X32>(g, 0) / GP);
+      vis_hi = sees(posA + chunk_row<X32>(g, 4) / GP);
     }
-    else if (a.causal) vis = vis && keypos * a.stride + a.block <= tokpos;
 
     float s[8], dp[8], p[8], ds[8];
     if (MODE == kBwdSlc) {                    // K fragments from the block copy in LDS instead of 24 registers
@@ -360,7 +379,7 @@ bwd_kv_kernel(const BwdArgs a) {
     for (int j = 0; j < 8; ++j) {
       const float lse2 = j < 4 ? l0[j & 3] : l1[j & 3];
       const float dl = j < 4 ? e0[j & 3] : e1[j & 3];
-      const bool ok = vis && (chunk_row<X32>(g, j) & 15) < G;
+      const bool ok = (j < 4 ? vis : vis_hi) && chunk_row<X32>(g, j) % GP < G;
       const float e = fast_exp2(fmaf(s[j], c_attn, -lse2));
       p[j] = ok ? e : 0.f;
       ds[j] = ok ? e * (dp[j] - dl) : 0.f;
@@ -714,12 +733,12 @@ slc_dq_merge_kernel(const SlcArgs s, const int* __restrict__ slotmap, const T* _
 
 // ---- launchers ------------------------------------------------------------------------------------
 
-template <typename T, int DK, int DV, int MODE, int NW>
-static int launch_kv_t(const BwdArgs& a, int key_rows, hipStream_t st) {
+template <typename T, int DK, int DV, int MODE, int NW, int TP>
+static int launch_kv_impl(const BwdArgs& a, int key_rows, hipStream_t st) {
   constexpr int XP = kLdsPad<T, MODE != kBwdSlc>;
   size_t smem = 2 * (size_t)(32 * (DK + XP) + 32 * (DV + XP)) * sizeof(T) + 128 * sizeof(float);
   if (MODE == kBwdSlc) smem += ((size_t)kBlk * (DK + XP) + 32 * (kBlk + 8)) * sizeof(T);
-  auto fn = bwd_kv_kernel<T, DK, DV, MODE, NW>;
+  auto fn = bwd_kv_kernel<T, DK, DV, MODE, NW, TP>;
   const int rc = set_smem(reinterpret_cast<const void*>(fn), smem);
   if (rc) return rc;
   dim3 grid;
@@ -732,6 +751,16 @@ static int launch_kv_t(const BwdArgs& a, int key_rows, hipStream_t st) {
   else grid = dim3(kXcds * b.tiles * items_per_xcd * a.hkv);
   hipLaunchKernelGGL(fn, grid, dim3(NW * 64), smem, st, b);
   return 0;
+}
+
+template <typename T, int DK, int DV, int MODE, int NW>
+static int launch_kv_t(const BwdArgs& a, int key_rows, hipStream_t st) {
+  if constexpr (MODE != kBwdSlc) {    // 4 / 2 tokens per 16 rows for GQA groups of at most 4 / 8 heads
+    const int G = a.hq / a.hkv;
+    if (G <= 4) return launch_kv_impl<T, DK, DV, MODE, NW, 4>(a, key_rows, st);
+    if (G <= 8) return launch_kv_impl<T, DK, DV, MODE, NW, 2>(a, key_rows, st);
+  }
+  return launch_kv_impl<T, DK, DV, MODE, NW, 1>(a, key_rows, st);
 }
 
 template <typename T, int DK, int DV, int MODE, int TP>
