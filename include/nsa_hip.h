@@ -130,6 +130,16 @@ int nsa_cmp_attn_fwd(const void* q, const void* ck, const void* cvt, void* o, fl
                      const int32_t* cu_seqlens, const int32_t* cu_cmp, int batch, int total, int hq, int hkv,
                      int dk, int dv, int64_t ck_row_stride, int64_t ck_head_stride, int cvt_cols, int block,
                      int stride, float scale, int causal, int dtype, nsa_stream_t stream);
+
+/* nsa_cmp_attn_fwd that also evaluates the gating Linear of the module on q (nsa/nsa.py:61,117: gating(q) with
+ * weight [3,dk], bias [3] or NULL, both in q's dtype): the kernel multiplies the query fragments it holds anyway with
+ * the three weight rows, so the logits cost no pass over q.  gates [total,hq,3] (q's dtype) receives them (order:
+ * selected, sliding, compressed), as nsa_gate_fwd would. */
+int nsa_cmp_attn_gate_fwd(const void* q, const void* ck, const void* cvt, void* o, float* lse, float* lse_attn,
+                          const void* gate_weight, const void* gate_bias, void* gates, const int32_t* cu_seqlens,
+                          const int32_t* cu_cmp, int batch, int total, int hq, int hkv, int dk, int dv,
+                          int64_t ck_row_stride, int64_t ck_head_stride, int cvt_cols, int block, int stride,
+                          float scale, int causal, int dtype, nsa_stream_t stream);
 int nsa_block_select_fwd(const void* q, const void* ck, const float* lse, void* indices, float* pooled,
                          const int32_t* cu_seqlens, const int32_t* cu_cmp, int batch, int total, int hq, int hkv,
                          int dk, int64_t ck_row_stride, int64_t ck_head_stride, int pool_kernel, int pool_stride,

@@ -29,6 +29,7 @@ SIGNATURES = {
     "nsa_cmp_attn_select_fwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _L, _I,
                                      _I, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P]),
     "nsa_cmp_attn_fwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _L, _I, _I, _I, _F, _I, _I, _P]),
+    "nsa_cmp_attn_gate_fwd": (_I, [_P] * 11 + [_I, _I, _I, _I, _I, _I, _L, _L, _I, _I, _I, _F, _I, _I, _P]),
     "nsa_block_select_fwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _L, _L, _I, _I, _I, _I, _I, _I,
                                   _I, _I, _I, _P]),
     "nsa_gate_fwd": (_I, [_P, _P, _P, _P, _L, _I, _I, _P]),

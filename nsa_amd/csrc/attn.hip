@@ -39,6 +39,7 @@ struct StreamParams {
   int split_hidden;  // compressed branch: stop at cmp_visible_end(): the rows beyond carry no attention, they only feed
                      // the importance log-sum-exp, which this caller did not ask for
   int tile_base = 0; // first token tile of this launch (workgroup x takes tile tile_base + x)
+  const void* gate_w = nullptr; const void* gate_b = nullptr; void* gates = nullptr;   // as CmpArgs
 };
 
 // MERGE (sliding window only): 0 = write the branch output; otherwise the epilogue merges the
@@ -109,6 +110,30 @@ stream_attn_kernel(const StreamParams a) {
     g_hi_max[j] = last_visible(tl);          // below g_hi_min when the group lies past the sequence end
     g_lo_min[j] = CMP ? 0 : tf - W + 1;
     g_lo_max[j] = CMP ? 0 : tl - W + 1;
+  }
+  if constexpr (CMP) {
+    // The gating Linear on the query rows this wavefront holds: logits^T = W q^T as one more 16 x 16 tile per row
+    // group (W's three rows in rows 0..2 of the A operand), so lane group 0 ends with the three logits of column n.
+    if (a.gate_w != nullptr) {
+      const T* wp = reinterpret_cast<const T*>(a.gate_w) + (long)min(n, 2) * DK + 8 * g;
+      const T* bp = reinterpret_cast<const T*>(a.gate_b);
+      vec8_t<T> wf[DK / 32];
+#pragma unroll
+      for (int kk = 0; kk < DK / 32; ++kk) wf[kk] = n < 3 ? load8(wp + 32 * kk) : zero8<T>();
+      float bias[3] = {0.f, 0.f, 0.f};
+      if (bp != nullptr) { bias[0] = (float)bp[0]; bias[1] = (float)bp[1]; bias[2] = (float)bp[2]; }
+#pragma unroll
+      for (int j = 0; j < NG; ++j) {
+        f32x4_t gt = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < DK / 32; ++kk) gt = mma16(wf[kk], grp[j].q[kk], gt);
+        if (g == 0 && rm[j].valid) {
+          T* gp = reinterpret_cast<T*>(a.gates) + (((long)st.start + rm[j].tok) * a.hq + h * G + rm[j].gidx) * 3;
+#pragma unroll
+          for (int i = 0; i < 3; ++i) gp[i] = (T)(gt[i] + bias[i]);
+        }
+      }
+    }
   }
   const float c_attn = a.scale * kLog2e;
   const int attn_end = last_visible(t_last);                      // last key any row of the tile attends
@@ -645,6 +670,7 @@ template <typename T, int DK, int DV>
 static int launch_cmp_t(const CmpArgs& a, hipStream_t st) {
   StreamParams p{a.q, a.ck, a.cvt, a.o, a.lse, a.cu_seq, a.cu_cmp, a.batch, a.hq, a.hkv, a.ck_row_stride,
                  a.ck_head_stride, a.cvt_cols, a.block, a.stride, 0, a.causal, a.scale, MergeArgs{}, a.lse_attn, a.kv_rep, 0};
+  p.gate_w = a.gate_w; p.gate_b = a.gate_b; p.gates = a.gates;
   // rows beyond the last one a tile's tokens may attend only feed the importance log-sum-exp: skipped when that
   // is not asked for
   if (a.causal && a.lse == nullptr) p.split_hidden = 1;

@@ -139,8 +139,12 @@ static int cmp_common(const char* what, int stages, const void* q, const void* c
                       const int32_t* cu_cmp, int batch, int total, int hq, int hkv, int dk, int dv, int64_t ck_row_stride,
                       int64_t ck_head_stride, int cvt_cols, int block, int stride, int pool_kernel, int pool_stride,
                       int pool_pad, int top_n, int max_ns, int pooled_stride, int keep_pooled, float scale, int causal,
-                      int idx64, int dtype, nsa_stream_t stream) {
+                      int idx64, int dtype, nsa_stream_t stream, const void* gate_w = nullptr,
+                      const void* gate_b = nullptr, void* gates = nullptr) {
   const bool attn = stages & 1, select = stages & 2;
+  if ((gate_w != nullptr) != (gates != nullptr) || (gate_b && !gate_w))
+    return fail(NSA_ERR_INVALID, "%s: the gating Linear needs its weight and the gates buffer", what);
+  if (gate_w && !aligned16(gate_w)) return fail(NSA_ERR_INVALID, "%s: pointers must be 16-byte aligned", what);
   if (!q || !ck || !cu_seqlens || !cu_cmp) return fail(NSA_ERR_INVALID, "%s: null pointer", what);
   if (attn && (!cvt || !o)) return fail(NSA_ERR_INVALID, "%s: null pointer", what);
   if (batch <= 0 || total <= 0 || block <= 0 || stride <= 0) return fail(NSA_ERR_INVALID, "%s: sizes must be positive", what);
@@ -164,6 +168,7 @@ static int cmp_common(const char* what, int stages, const void* q, const void* c
                  (long)ck_row_stride, (long)ck_head_stride, cvt_cols, block, stride, pool_kernel, pool_stride,
                  pool_pad, top_n, max_ns, pooled_stride, scale, idx64, dtype, causal, lse_attn, kv_rep};
   a.keep_pooled = keep_pooled != 0;
+  a.gate_w = gate_w; a.gate_b = gate_b; a.gates = gates;
   int rc = 0;
   if (attn) rc = nsa::launch_cmp_attn(a, stream);
   if (rc == 0 && select) rc = nsa::launch_select(a, stream);
@@ -192,6 +197,17 @@ int nsa_cmp_attn_fwd(const void* q, const void* ck, const void* cvt, void* o, fl
   return cmp_common("cmp_attn", 1, q, ck, cvt, o, nullptr, nullptr, lse, lse_attn, cu_seqlens, cu_cmp, batch, total, hq, hkv,
                     dk, dv, ck_row_stride, ck_head_stride, cvt_cols, block, stride, 1, 1, 0, 1, 0, 0, 0, scale, causal,
                     0, dtype, stream);
+}
+
+int nsa_cmp_attn_gate_fwd(const void* q, const void* ck, const void* cvt, void* o, float* lse, float* lse_attn,
+                          const void* gate_weight, const void* gate_bias, void* gates, const int32_t* cu_seqlens,
+                          const int32_t* cu_cmp, int batch, int total, int hq, int hkv, int dk, int dv,
+                          int64_t ck_row_stride, int64_t ck_head_stride, int cvt_cols, int block, int stride,
+                          float scale, int causal, int dtype, nsa_stream_t stream) {
+  if (!gate_weight || !gates) return fail(NSA_ERR_INVALID, "cmp_attn_gate: null pointer");
+  return cmp_common("cmp_attn_gate", 1, q, ck, cvt, o, nullptr, nullptr, lse, lse_attn, cu_seqlens, cu_cmp, batch, total, hq,
+                    hkv, dk, dv, ck_row_stride, ck_head_stride, cvt_cols, block, stride, 1, 1, 0, 1, 0, 0, 0, scale,
+                    causal, 0, dtype, stream, gate_weight, gate_bias, gates);
 }
 
 int nsa_block_select_fwd(const void* q, const void* ck, const float* lse, void* indices, float* pooled,

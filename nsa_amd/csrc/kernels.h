@@ -40,6 +40,9 @@ struct CmpArgs {
   // false: `pooled` only hands the window sums from the importance kernel to the top-n kernel; the averages are
   // not written back (and the generic one-kernel selection does not write it at all)
   bool keep_pooled = true;
+  // optional: the gating Linear on q (weight [3][dk], bias [3] or null, in q's dtype) evaluated by the compressed-
+  // attention kernel on the query fragments it holds anyway; gates [total][hq][3] receives the logits
+  const void* gate_w = nullptr; const void* gate_b = nullptr; void* gates = nullptr;
 };
 
 struct SwaArgs {

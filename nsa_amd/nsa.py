@@ -159,14 +159,18 @@ class NSAAttention(nn.Module):
         max_nc = nc if nc is not None else conv_compressed_len(seq_len, self.compression_stride,
                                                                self.compression_block)
         cvt, vt = stage("transpose", lambda: (ops.transpose(cv, cu_cmp, batch), ops.transpose(v, cu, batch)))
-        o_cmp, lse = stage("cmp_attn", lambda: ops.cmp_attn(
-            q, ck, cvt, cu, cu_cmp, batch, hkv, dv, ck.stride(0), ck.stride(1), self.compression_block,
-            self.compression_stride, scale, causal=bool(causal)))
+        if gates is None:       # the gating Linear rides on the compressed-attention kernel's query fragments
+            o_cmp, lse, gates = stage("cmp_attn", lambda: ops.cmp_attn(
+                q, ck, cvt, cu, cu_cmp, batch, hkv, dv, ck.stride(0), ck.stride(1), self.compression_block,
+                self.compression_stride, scale, causal=bool(causal), gate_weight=self.gating.weight,
+                gate_bias=self.gating.bias))
+        else:
+            o_cmp, lse = stage("cmp_attn", lambda: ops.cmp_attn(
+                q, ck, cvt, cu, cu_cmp, batch, hkv, dv, ck.stride(0), ck.stride(1), self.compression_block,
+                self.compression_stride, scale, causal=bool(causal)))
         idx, _ = stage("block_select", lambda: ops.block_select(
             q, ck, lse, cu, cu_cmp, batch, hkv, ck.stride(0), ck.stride(1), self.pool_kernel_size,
             self.pool_stride, self.pool_padding, self.selected_block_count, max_nc, idx64=False))
-        if gates is None:
-            gates = stage("gates", lambda: ops.gate_logits(q, self.gating.weight, self.gating.bias))   # [total, Hq, 3]
         g = gates.reshape(total * hq, 3)
         g_slc, g_swa, g_cmp = (g[:, i].view(total, hq) for i in range(3))
         act = _lib.GATE_SIGMOID if self.gate_activation == "sigmoid" else _lib.GATE_IDENTITY

@@ -183,16 +183,29 @@ def cmp_attn_select(q, ck, cvt, cu_seqlens, cu_cmp, batch, hkv, dv, ck_row_strid
 
 
 def cmp_attn(q, ck, cvt, cu_seqlens, cu_cmp, batch, hkv, dv, ck_row_stride, ck_head_stride, block, stride, scale,
-             causal=True, want_lse_attn=False):
+             causal=True, want_lse_attn=False, gate_weight=None, gate_bias=None):
     """Compressed attention only.  Returns (o [total,Hq,dv], lse float32 [total,Hq]) where lse is the
     log-sum-exp of the raw scores over all compressed rows (what block_select reads); with
-    want_lse_attn a third tensor: the log-sum-exp of the scaled visible scores (what the backward reads)."""
+    want_lse_attn a third tensor: the log-sum-exp of the scaled visible scores (what the backward reads).
+    gate_weight [3,Dk] (+ gate_bias [3]): the same kernel also evaluates the gating Linear on q and the gate
+    logits [total,Hq,3] are returned as one more tensor."""
     _need_cuda(q, ck, cvt, cu_seqlens, cu_cmp)
     q = _dense(q)
     total, hq, dk = q.shape
     o = torch.empty(total, hq, dv, dtype=q.dtype, device=q.device)
     lse = torch.empty(total, hq, dtype=torch.float32, device=q.device)
     lse_attn = torch.empty(total, hq, dtype=torch.float32, device=q.device) if want_lse_attn else None
+    if gate_weight is not None:
+        _need_cuda(gate_weight)
+        w = _dense(gate_weight.to(q.dtype))
+        b = None if gate_bias is None else gate_bias.to(q.dtype).contiguous()
+        gates = torch.empty(total, hq, 3, dtype=q.dtype, device=q.device)
+        rc = _lib.load().nsa_cmp_attn_gate_fwd(
+            _ptr(q), _ptr(ck), _ptr(cvt), _ptr(o), _ptr(lse), _ptr(lse_attn), _ptr(w), _ptr(b), _ptr(gates),
+            _ptr(cu_seqlens), _ptr(cu_cmp), batch, total, hq, hkv, dk, dv, ck_row_stride, ck_head_stride,
+            cvt.shape[-1], block, stride, float(scale), int(bool(causal)), _dtype_code(q), _stream())
+        _lib.check(rc, "nsa_cmp_attn_gate_fwd")
+        return (o, lse, lse_attn, gates) if want_lse_attn else (o, lse, gates)
     rc = _lib.load().nsa_cmp_attn_fwd(_ptr(q), _ptr(ck), _ptr(cvt), _ptr(o), _ptr(lse), _ptr(lse_attn),
                                       _ptr(cu_seqlens), _ptr(cu_cmp), batch, total, hq, hkv, dk, dv, ck_row_stride,
                                       ck_head_stride, cvt.shape[-1], block, stride, float(scale), int(bool(causal)),

@@ -653,23 +653,39 @@ def test_gate_logits_match_linear(dtype, T, Hq, D):
 
 
 def test_module_own_gating_equals_explicit_gates():
-    """forward(gates=None) runs the gate kernel on the module's Linear; feeding those logits back in
-    through gates= must give the same output bit for bit."""
+    """forward(gates=None) evaluates the module's gating Linear inside the compressed-attention kernel
+    (nsa_cmp_attn_gate_fwd): those logits against the Linear in float64 (one rounding of the result may differ),
+    against the stand-alone gate kernel, and fed back in through gates= (same output bit for bit)."""
     from nsa_amd.nsa import NSAAttention
-    dtype, T, Hq, Hkv, D = torch.bfloat16, 640, 32, 2, 128
-    q, k, v, _ = make_qkv(T, Hq, Hkv, D, D, 173, dtype, 0.5)
-    torch.manual_seed(174)
-    m = NSAAttention(D, causal=True, selected_block_count=8, sliding_window=128, dtype=dtype, compressor_mode="mean",
-                     gate_activation="sigmoid").to(DEV)
-    cu = _cu([T])
-    with torch.no_grad():
-        a = m(q.to(DEV), k.to(DEV), v.to(DEV), cu, 0)
-    gl = _ops().gate_logits(q.to(DEV), m.gating.weight, m.gating.bias)
-    ref_gl = torch.nn.functional.linear(q.float(), m.gating.weight.detach().float().cpu(),
-                                        m.gating.bias.detach().float().cpu())
-    assert max_abs(gl.cpu(), ref_gl) <= 3e-2
-    b = m(q.to(DEV), k.to(DEV), v.to(DEV), cu, 0, gates=gl)
-    assert torch.equal(a, b)
+    from nsa_amd.compression_kv import conv_compressed_len
+    ops = _ops()
+    for dtype, lens, Hq, Hkv, Dk, Dv in ((torch.bfloat16, [640], 32, 2, 128, 128), (torch.float16, [300, 77], 12, 2, 192, 128),
+                                         (torch.float32, [200], 4, 1, 64, 64), (torch.bfloat16, [260], 64, 2, 64, 64)):
+        T = sum(lens)
+        q, k, v, _ = make_qkv(T, Hq, Hkv, Dk, Dv, 173, dtype, 0.5)
+        torch.manual_seed(174)
+        m = NSAAttention(Dk, causal=True, selected_block_count=8, sliding_window=128, dtype=dtype, compressor_mode="mean",
+                         gate_activation="sigmoid").to(DEV)
+        cu = _cu(lens)
+        qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+        with torch.no_grad():
+            a = m(qd, kd, vd, cu, max(lens))
+            ck, cv, cu_cmp, _ = m.compressor.compress_packed(kd, vd, cu, seq_len=None)
+            cvt = ops.transpose(cv, cu_cmp, len(lens))
+            o1, lse1 = ops.cmp_attn(qd, ck, cvt, cu, cu_cmp, len(lens), Hkv, Dv, ck.stride(0), ck.stride(1), 32, 16,
+                                    Dk ** -0.5)
+            o2, lse2, gl = ops.cmp_attn(qd, ck, cvt, cu, cu_cmp, len(lens), Hkv, Dv, ck.stride(0), ck.stride(1), 32, 16,
+                                        Dk ** -0.5, gate_weight=m.gating.weight, gate_bias=m.gating.bias)
+            assert torch.equal(o1, o2) and torch.equal(lse1, lse2)            # the attention itself is untouched
+            ref_gl = torch.nn.functional.linear(q.double(), m.gating.weight.detach().double().cpu(),
+                                                m.gating.bias.detach().double().cpu())
+            ulp = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11, torch.float32: 2.0 ** -20}[dtype]
+            err = (gl.double().cpu() - ref_gl).abs()
+            assert bool((err <= ref_gl.abs() * ulp + 1e-6).all()), float(err.max())
+            sep = ops.gate_logits(qd, m.gating.weight, m.gating.bias)
+            assert max_abs(gl, sep) <= (float(ref_gl.abs().max()) * 2 * ulp + 1e-6)
+            b = m(qd, kd, vd, cu, max(lens), gates=gl)
+        assert torch.equal(a, b)
 
 
 def test_module_randomized_small_shapes():
