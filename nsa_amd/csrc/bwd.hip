@@ -113,14 +113,13 @@ __device__ __forceinline__ void store4(float* p, const f32x4_t& v, float s) {
 
 // Two wavefronts per SIMD: left alone the compiler takes 264 registers (one wavefront per SIMD); a budget of
 // 168 (three) spills the accumulators and more than doubles the run time.
-// TP (window and compressed modes): tokens per 16 rows of a chunk for GQA groups of at most 16 / TP heads; row r of
-// a chunk is head r % GP of the chunk's token r / GP (GP = 16 / TP, TPC = 2 * TP tokens per chunk).
+// TP: tokens (selected mode: pairs of the block's list) per 16 rows of a chunk for GQA groups of at most 16 / TP
+// heads; row r of a chunk is head r % GP of the chunk's token or pair r / GP (GP = 16 / TP, TPC = 2 * TP per chunk).
 template <typename T, int DK, int DV, int MODE, int NW, int TP = 1>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 bwd_kv_kernel(const BwdArgs a) {
   constexpr bool X32 = MODE != kBwdSlc;
   constexpr int GP = 16 / TP, TPC = 2 * TP;
-  static_assert(MODE != kBwdSlc || TP == 1, "the selected branch keeps one pair per 16 rows");
   constexpr int QLD = DK + kLdsPad<T, X32>, OLD = DV + kLdsPad<T, X32>, NT = NW * 64, SLD = kBlk + 8;
   constexpr int QP = 32 * DK / 8, OP = 32 * DV / 8;                 // 16-byte pieces of one chunk
   constexpr int QPT = (QP + NT - 1) / NT, OPT = (OP + NT - 1) / NT;
@@ -151,7 +150,7 @@ bwd_kv_kernel(const BwdArgs a) {
     seq_start = st.start; key0 = st.t0; nkeys = st.len; key_base = st.start;
     first = a.ws.offsets[key] + seg * kSeg;
     count = min(a.ws.counts[key] - seg * kSeg, kSegGroup * kSeg);
-    nchunks = (count + 1) >> 1;
+    nchunks = (count + TPC - 1) / TPC;
   } else if (MODE == kBwdSwa) {
     // Workgroup w runs on XCD w % 8 (each XCD has its own L2).  Neighbouring key tiles stream almost the same
     // tokens (a 64-key tile and its 512-token window), so every XCD takes a contiguous run of key tiles: the
@@ -200,21 +199,15 @@ bwd_kv_kernel(const BwdArgs a) {
   const T* qb = reinterpret_cast<const T*>(a.q);
   const T* dob = reinterpret_cast<const T*>(a.d_o);
 
-  // tokens of chunk c: positions inside the sequence (pos*), validity of the second one
-  // selected branch, selection blocks below 64 keys: a pair sees keys [sub, sub + slc_width) of the block
+  // Tokens of chunk c, as positions inside the sequence.  Window and compressed modes: `pos`, the chunk's first
+  // token.  Selected branch: the chunk holds TPC pairs of the list, pair u in rows u * GP .. (its GQA group), and
+  // lane l carries the word of pair l % TPC: 64 x the position of its token (the last pair's again past the end
+  // of the list) + the first key it sees inside the block (selection blocks below 64 keys: a pair sees keys
+  // [sub, sub + slc_width) of the block).  pair_word hands a lane the word of any pair of the chunk.
   const bool parts = MODE == kBwdSlc && a.slc_width < kBlk;
-  int subA = 0, subB = 0, nsubA = 0, nsubB = 0;
-  auto chunk_tokens = [&](int c, int& posA, int& posB, bool& vB) {
-    if (MODE == kBwdSlc) {
-      posA = (int)(a.ws.list[first + 2 * c] >> 6) - seq_start;
-      vB = 2 * c + 1 < count;
-      posB = vB ? (int)(a.ws.list[first + 2 * c + 1] >> 6) - seq_start : posA;
-    } else {
-      if (MODE == kBwdSwa) { c += rot; if (c >= nchunks) c -= nchunks; }
-      posA = t_begin + TPC * c;
-      vB = posA + 1 < t_end;
-      posB = vB ? posA + 1 : posA;
-    }
+  auto chunk_first = [&](int c) -> int {
+    if (MODE == kBwdSwa) { c += rot; if (c >= nchunks) c -= nchunks; }
+    return t_begin + TPC * c;
   };
 
   // ---- stationary fragments: 16 keys of this wavefront
@@ -249,18 +242,19 @@ bwd_kv_kernel(const BwdArgs a) {
 #pragma unroll
   for (int i = 0; i < OPT; ++i) ors[i] = 1.f;
   // token (position in the sequence, clamped to the last one of the work item) and head of row r of a chunk
-  auto row_tok = [&](int r, int posA, int posB) -> int {
-    if (MODE == kBwdSlc) return (r >> 4) ? posB : posA;
-    return min(posA + r / GP, t_end - 1);
+  auto pair_word = [&](int words, int u) -> int { return __builtin_amdgcn_ds_bpermute(u << 2, words); };
+  auto row_tok = [&](int r, int pos, int words) -> int {
+    if (MODE == kBwdSlc) return pair_word(words, r / GP) >> 6;
+    return min(pos + r / GP, t_end - 1);
   };
   auto row_head = [&](int r) -> int { return min(r % GP, G - 1); };
-  auto gload = [&](int posA, int posB) {
+  auto gload = [&](int pos, int words) {
 #pragma unroll
     for (int i = 0; i < QPT; ++i) {
       const int p = tid + i * NT;
       if (QP % NT == 0 || p < QP) {
         const int r = p / (DK / 8), pc = p % (DK / 8);
-        const long tg = seq_start + row_tok(r, posA, posB);
+        const long tg = seq_start + row_tok(r, pos, words);
         qr[i] = load8(qb + (tg * a.hq + h * G + row_head(r)) * DK + pc * 8);
       }
     }
@@ -269,7 +263,7 @@ bwd_kv_kernel(const BwdArgs a) {
       const int p = tid + i * NT;
       if (OP % NT == 0 || p < OP) {
         const int r = p / (DV / 8), pc = p % (DV / 8);
-        const long tg = seq_start + row_tok(r, posA, posB);
+        const long tg = seq_start + row_tok(r, pos, words);
         const long row = tg * a.hq + h * G + row_head(r);
         orr[i] = load8(dob + row * DV + pc * 8);
         if (a.rowscale != nullptr) ors[i] = a.rowscale[row];       // used in lstore: nothing here waits for a load
@@ -277,7 +271,7 @@ bwd_kv_kernel(const BwdArgs a) {
     }
     if (tid < 64) {
       const int r = tid & 31;
-      const long tg = seq_start + row_tok(r, posA, posB);
+      const long tg = seq_start + row_tok(r, pos, words);
       const long row = tg * a.hq + h * G + row_head(r);
       sr = tid < 32 ? a.lse[row] : a.delta[row];
       if (a.rowscale != nullptr) srs = a.rowscale[row];
@@ -303,31 +297,27 @@ bwd_kv_kernel(const BwdArgs a) {
   };
 
   const float c_attn = a.scale * kLog2e;
-  // Token positions are carried in registers: pos = chunk c, nxt = chunk c + 1.
-  int posA, posB, nxtA = 0, nxtB = 0;
-  bool vB, nxtV = false;
-  // selected mode: even lanes read the pair-list entry of a chunk's first token, odd lanes that of its second
-  // (the first again when the chunk has one), as one load whose value is only split into the two positions
-  // where they are used: a load from a wave-uniform address would be waited for where it is issued.
+  // Token positions are carried in registers: pos / words = chunk c, nxt / nwords = chunk c + 1.
+  int pos = 0, nxt = 0, words = 0, nwords = 0;
+  // selected mode: lane l reads the pair-list entry of the chunk's pair l % TPC (the last entry of the list for
+  // pairs past its end) a chunk before its word is formed from it: the load is waited for where its value is
+  // first used, not where it is issued.
   unsigned aftv = 0, afts = 0;
-  auto list_entry = [&](int c) { return a.ws.list[first + min(2 * c + (lane & 1), count - 1)]; };
-  auto sub_entry = [&](int c) { return (unsigned)a.ws.sub[first + min(2 * c + (lane & 1), count - 1)]; };
-  auto list_split = [&](unsigned v, int c, int& pA, int& pB, bool& vb) {
-    pA = (int)(__builtin_amdgcn_readlane(v, 0) >> 6) - seq_start;
-    pB = (int)(__builtin_amdgcn_readlane(v, 1) >> 6) - seq_start;
-    vb = 2 * c + 1 < count;
-  };
-  chunk_tokens(0, posA, posB, vB);
-  if (nchunks > 1) chunk_tokens(1, nxtA, nxtB, nxtV);
-  if (MODE == kBwdSlc && nchunks > 2) aftv = list_entry(2);
-  if (parts) {
-    subA = a.ws.sub[first];
-    subB = a.ws.sub[first + min(1, count - 1)];
-    nsubA = a.ws.sub[first + min(2, count - 1)];
-    nsubB = a.ws.sub[first + min(3, count - 1)];
-    if (nchunks > 2) afts = sub_entry(2);
+  auto list_entry = [&](int c) { return a.ws.list[first + min(TPC * c + (lane & (TPC - 1)), count - 1)]; };
+  auto sub_entry = [&](int c) { return (unsigned)a.ws.sub[first + min(TPC * c + (lane & (TPC - 1)), count - 1)]; };
+  auto word_of = [&](unsigned v, unsigned sb) -> int { return (int)(((v >> 6) - (unsigned)seq_start) << 6 | sb); };
+  if (MODE == kBwdSlc) {
+    words = word_of(list_entry(0), parts ? sub_entry(0) : 0u);
+    if (nchunks > 1) nwords = word_of(list_entry(1), parts ? sub_entry(1) : 0u);
+    if (nchunks > 2) {
+      aftv = list_entry(2);
+      if (parts) afts = sub_entry(2);
+    }
+  } else {
+    pos = chunk_first(0);
+    if (nchunks > 1) nxt = chunk_first(1);
   }
-  gload(posA, posB);
+  gload(pos, words);
   lstore(0);
   __syncthreads();
   int buf = 0;
@@ -336,7 +326,7 @@ bwd_kv_kernel(const BwdArgs a) {
     // stores: with both unconditional the compiler knows that nothing is in flight at the top of the loop and
     // puts no wait there (one that would also cover the dQ partial stores just issued).
     const bool has_next = c + 1 < nchunks;
-    gload(has_next ? nxtA : posA, has_next ? nxtB : posB);
+    gload(has_next ? nxt : pos, has_next ? nwords : words);
 
     const T* qs = lds + buf * STAGE;
     const T* os = qs + 32 * QLD;
@@ -344,11 +334,16 @@ bwd_kv_kernel(const BwdArgs a) {
     // the 8 rows of this lane: chunk_row(g, 0..3) are heads of one token, chunk_row(g, 4..7) of one token (the
     // same one unless tokens share the 16 rows of a tile)
     bool vis, vis_hi;
+    const int left = count - TPC * c;         // selected branch: pairs from this chunk's first one to the end of the list
     if (MODE == kBwdSlc) {
-      const int tokpos = (g >> 1) ? posB : posA;
-      vis = keyvalid && ((g >> 1) == 0 || vB) && keypos <= tokpos;
-      if (parts) vis = vis && (unsigned)(keypos - key0 - ((g >> 1) ? subB : subA)) < (unsigned)a.slc_width;
-      vis_hi = vis;
+      auto sees = [&](int u) -> bool {        // pair u of the chunk
+        const int w = pair_word(words, u);
+        bool ok = keyvalid && u < left && keypos <= (w >> 6);
+        if (parts) ok = ok && (unsigned)(keypos - key0 - (w & 63)) < (unsigned)a.slc_width;
+        return ok;
+      };
+      vis = sees(chunk_row<X32>(g, 0) / GP);
+      vis_hi = GP >= 8 ? vis : sees(chunk_row<X32>(g, 4) / GP);
     } else {
       auto sees = [&](int tokpos) -> bool {
         bool v = keyvalid && tokpos < t_end;
@@ -356,8 +351,8 @@ bwd_kv_kernel(const BwdArgs a) {
         else if (a.causal) v = v && keypos * a.stride + a.block <= tokpos;
         return v;
       };
-      vis = sees(posA + chunk_row<X32>(g, 0) / GP);
-      vis_hi = sees(posA + chunk_row<X32>(g, 4) / GP);
+      vis = sees(pos + chunk_row<X32>(g, 0) / GP);
+      vis_hi = sees(pos + chunk_row<X32>(g, 4) / GP);
     }
 
     float s[8], dp[8], p[8], ds[8];
@@ -398,46 +393,40 @@ bwd_kv_kernel(const BwdArgs a) {
     // The next chunk goes to LDS before this chunk's dQ partials are stored: the counter that says "the gathers
     // have arrived" also counts stores, in order, so after the stores it would wait for their write round trip.
     lstore(buf ^ 1);
-    // aftv (chunk c + 2) was requested an iteration ago; it is split here, before the stores below, for the same
-    // reason
-    int splA = 0, splB = 0;
-    bool splV = false;
-    if (MODE == kBwdSlc) list_split(aftv, c + 2, splA, splB, splV);
-    int splsA = 0, splsB = 0;
-    if (parts) {
-      splsA = (int)__builtin_amdgcn_readlane(afts, 0);
-      splsB = (int)__builtin_amdgcn_readlane(afts, 1);
-    }
+    // aftv (chunk c + 2) was requested an iteration ago; its word is formed here, before the stores below, for the
+    // same reason
+    const int awords = MODE == kBwdSlc ? word_of(aftv, afts) : 0;
     if (MODE == kBwdSlc) {
       // dQ^T[dk][row] = sum_key K[key][dk] dS[row][key]: this wavefront takes every NW-th 16-channel tile
       T* part = reinterpret_cast<T*>(a.ws.po);
 #pragma unroll
       for (int t = wave; t < DK / 16; t += NW) {
 #pragma unroll
-        for (int r = 0; r < 2; ++r) {
-          if (r == 1 && !vB) break;
+        for (int r = 0; r < 2; ++r) {       // rows 16r .. 16r + 15 of the chunk: pairs r * TP .. r * TP + TP - 1
+          if (r * TP >= left) break;
           f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int step = 0; step < 2; ++step)
             acc = mma16(load8_tr(kblk + 32 * step * QLD + 16 * t, QLD, lane),
                         load8(dsl + (16 * r + n) * SLD + 32 * step + 8 * g), acc);
-          store4(part + ((long)(first + 2 * c + r) * 16 + n) * DK + 16 * t + 4 * g, acc, a.scale);
+          const int u = r * TP + n / GP;      // this lane's row: head n % GP of pair u
+          if (u < left && n % GP < G)
+            store4(part + ((long)(first + TPC * c + u) * 16 + n % GP) * DK + 16 * t + 4 * g, acc, a.scale);
         }
       }
     }
 
     __syncthreads();
     buf ^= 1;
-    posA = nxtA; posB = nxtB; vB = nxtV;
+    pos = nxt; words = nwords;
     if (MODE == kBwdSlc) {
-      nxtA = splA; nxtB = splB; nxtV = splV;
-      if (c + 3 < nchunks) aftv = list_entry(c + 3);      // first touched an iteration from here
-      if (parts) {
-        subA = nsubA; subB = nsubB; nsubA = splsA; nsubB = splsB;
-        if (c + 3 < nchunks) afts = sub_entry(c + 3);
+      nwords = awords;
+      if (c + 3 < nchunks) {                              // first touched an iteration from here
+        aftv = list_entry(c + 3);
+        if (parts) afts = sub_entry(c + 3);
       }
     } else if (c + 2 < nchunks) {
-      chunk_tokens(c + 2, nxtA, nxtB, nxtV);
+      nxt = chunk_first(c + 2);
     }
   }
 
@@ -755,11 +744,9 @@ static int launch_kv_impl(const BwdArgs& a, int key_rows, hipStream_t st) {
 
 template <typename T, int DK, int DV, int MODE, int NW>
 static int launch_kv_t(const BwdArgs& a, int key_rows, hipStream_t st) {
-  if constexpr (MODE != kBwdSlc) {    // 4 / 2 tokens per 16 rows for GQA groups of at most 4 / 8 heads
-    const int G = a.hq / a.hkv;
-    if (G <= 4) return launch_kv_impl<T, DK, DV, MODE, NW, 4>(a, key_rows, st);
-    if (G <= 8) return launch_kv_impl<T, DK, DV, MODE, NW, 2>(a, key_rows, st);
-  }
+  const int G = a.hq / a.hkv;         // 4 / 2 tokens (selected branch: pairs) per 16 rows for GQA groups of at most 4 / 8 heads
+  if (G <= 4) return launch_kv_impl<T, DK, DV, MODE, NW, 4>(a, key_rows, st);
+  if (G <= 8) return launch_kv_impl<T, DK, DV, MODE, NW, 2>(a, key_rows, st);
   return launch_kv_impl<T, DK, DV, MODE, NW, 1>(a, key_rows, st);
 }
 

@@ -141,7 +141,8 @@ def _random_indices(T, Hkv, S, bs, seed):
 
 @pytest.mark.parametrize("lens,Hq,Hkv,Dk,Dv,S,W", [([384], 16, 1, 64, 64, 4, 0), ([512, 100], 32, 2, 128, 128, 8, 100),
                                                   ([330], 16, 1, 192, 128, 3, 64), ([700, 130], 24, 2, 64, 64, 16, 0),
-                                                  ([200], 4, 1, 64, 64, 2, 32)])
+                                                  ([200], 4, 1, 64, 64, 2, 32), ([512, 100], 16, 2, 128, 128, 8, 100),
+                                                  ([700, 130], 12, 2, 64, 64, 16, 0), ([330], 3, 1, 192, 128, 3, 64)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_slc_swa_bwd(lens, Hq, Hkv, Dk, Dv, S, W, dtype):
     _slc_swa_bwd_case(lens, Hq, Hkv, Dk, Dv, S, W, dtype, 64)
@@ -152,7 +153,9 @@ def test_slc_swa_bwd(lens, Hq, Hkv, Dk, Dv, S, W, dtype):
                                                      ([330], 16, 1, 192, 128, 6, 64, 16),
                                                      ([700], 16, 1, 64, 64, 3, 100, 128),
                                                      ([900, 100], 32, 2, 128, 128, 2, 0, 192),
-                                                     ([300], 16, 1, 32, 32, 3, 64, 32), ([300], 4, 2, 32, 32, 3, 0, 64)])
+                                                     ([300], 16, 1, 32, 32, 3, 64, 32), ([300], 4, 2, 32, 32, 3, 0, 64),
+                                                     ([400, 90], 8, 1, 64, 64, 5, 0, 32),
+                                                     ([333], 12, 4, 128, 128, 6, 50, 16)])
 def test_slc_swa_bwd_other_selection_block_sizes(lens, Hq, Hkv, Dk, Dv, S, W, bs):
     """Selection blocks of 8, 16, 32 keys (the reference's own test uses 32, tests/test_parallel_nsa.py:169) run as
     masked parts of a 64-key block, blocks of 128, 192 keys as several 64-key blocks per pick."""
