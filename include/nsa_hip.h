@@ -366,7 +366,10 @@ int nsa_decode_append_paged(const void* k_new, const void* v_new, void* k_pool, 
  * (ctx_cap used), else the paged pool (max_pages used).  Pooling 5 / 4 / 0 only.  The compressed rows are cut
  * into max(splits, ceil(nc_cap / 384)) <= 32 slices, so caches of up to nsa_decode_split_max_compressed() rows
  * (contexts of ~196k tokens at stride 16) are served whatever the batch.  The workspace holds
- * partial results only; calls that share it must not overlap.  No counterpart in the reference. */
+ * partial results only; calls that share it must not overlap.  GQA groups of 32, 48 or 64 heads (what the
+ * reference's HQ % (16 * H) == 0 admits, nsa/selection_attn.py:800) run here and only here: every 16 heads of
+ * a group are a pair of their own on the kv head's caches, the importance is summed over the whole group before
+ * the top-n; size the workspace with hkv x (hq / hkv / 16) in place of hkv.  No counterpart in the reference. */
 int64_t nsa_decode_split_workspace_bytes(int batch, int hkv, int dv, int nc_cap, int splits);
 int nsa_decode_step_split(const void* q, const void* k_cache, const void* v_cache_t, const int32_t* block_table,
                           int max_pages, const void* ck_cache, const void* cv_cache_t, const int32_t* ctx_lens,

@@ -598,7 +598,12 @@ static int decode_common(const char* what, const void* q, const void* k_cache, c
   if (batch <= 0 || ctx_cap <= 0 || nc_cap <= 0 || block <= 0 || stride <= 0 || window < 0)
     return fail(NSA_ERR_INVALID, "%s: sizes must be positive", what);
   if (!dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "%s: bad dtype", what);
-  if (int rc = check_heads(what, hq, hkv, dk, dv)) return rc;
+  int kv_rep = 1;
+  if (int rc = check_heads(what, hq, hkv, dk, dv, &kv_rep)) return rc;
+  if (kv_rep > 1 && splits == 0)
+    return fail(NSA_ERR_UNSUPPORTED, "%s: the one-workgroup step is built for GQA groups of at most 16 heads; groups of "
+                "32, 48, 64 heads go through nsa_decode_step_split", what);
+  if (kv_rep > 4) return fail(NSA_ERR_UNSUPPORTED, "%s: GQA groups of at most 64 heads are built", what);
   if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "%s: scale must be positive", what);
   if (ctx_cap % 64 != 0 || nc_cap % 64 != 0) return fail(NSA_ERR_INVALID, "%s: cache capacities must be multiples of 64", what);
   if (splits == 0 && nc_cap > nsa::decode_max_nc())
@@ -615,6 +620,7 @@ static int decode_common(const char* what, const void* q, const void* k_cache, c
   nsa::DecodeArgs a{q, k_cache, v_cache_t, ck_cache, cv_cache_t, ctx_lens, gates, out, indices, batch, hq, hkv, dk, dv,
                     ctx_cap, nc_cap, block, stride, sel_block, pool_kernel, pool_stride, pool_pad, top_n, window, scale,
                     gate_act, dtype, block_table, max_pages};
+  a.kv_rep = kv_rep;
   if (splits > 0) {
     if (splits > 16) return fail(NSA_ERR_INVALID, "%s: at most 16 splits", what);
     if (pool_kernel != 5 || pool_stride != 4 || pool_pad != 0)

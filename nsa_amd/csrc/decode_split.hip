@@ -43,7 +43,7 @@ static SplitLayout split_layout(const DecodeArgs& a, int splits) {
 }
 
 long decode_split_workspace_bytes(const DecodeArgs& a, int splits) {
-  return split_layout(a, splits).total() * (long)a.batch * a.hkv * (long)sizeof(float);
+  return split_layout(a, splits).total() * (long)a.batch * a.hkv * max(a.kv_rep, 1) * (long)sizeof(float);
 }
 
 // ---- A: compressed rows of one slice ---------------------------------------------------------------
@@ -61,8 +61,9 @@ decode_split_cmp_kernel(const DecodeArgs a, const SplitLayout L, float* __restri
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 15, g = lane >> 4;
   const int bh = blockIdx.x, s = blockIdx.y;
-  const int b = bh / a.hkv, h = bh % a.hkv;
-  const int G = a.hq / a.hkv;
+  const int hs = a.hkv * a.kv_rep;                         // sub-groups of at most 16 query heads per sequence
+  const int b = bh / hs, h = bh % hs, hc = h / a.kv_rep;   // h: sub-group (query heads h * G ..), hc: its kv head
+  const int G = a.hq / hs;
   float* wsp = ws + (long)bh * L.total();
   float* w_stat = wsp + L.stat() + (long)s * 32;
   float* w_bins = wsp + L.bins() + (long)s * L.nb * 16;
@@ -80,8 +81,8 @@ decode_split_cmp_kernel(const DecodeArgs a, const SplitLayout L, float* __restri
   const int cmaxv = t >= a.block ? min((t - a.block) / a.stride, Nc - 1) : -1;   // last visible compressed row
   const float c_attn = a.scale * kLog2e;
   const long krow = (long)a.hkv * DK;
-  const T* ckseq = reinterpret_cast<const T*>(a.ck_cache) + ((long)b * a.nc_cap * a.hkv + h) * DK;
-  const T* cvt = reinterpret_cast<const T*>(a.cv_cache_t) + (((long)b * a.hkv + h) * DV + n) * a.nc_cap + 8 * g;
+  const T* ckseq = reinterpret_cast<const T*>(a.ck_cache) + ((long)b * a.nc_cap * a.hkv + hc) * DK;
+  const T* cvt = reinterpret_cast<const T*>(a.cv_cache_t) + (((long)b * a.hkv + hc) * DV + n) * a.nc_cap + 8 * g;
   const long cvstep = 16L * a.nc_cap;
 
   vec8_t<T> qf[DK / 32];
@@ -233,19 +234,21 @@ decode_split_attend_kernel(const DecodeArgs a, const SplitLayout L, float* __res
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   float* part = reinterpret_cast<float*>(smem_raw);            // [NW][DV][PLD]
   float* pstat = part + NW * DV * PLD;                         // [NW][2][16]
-  float* fac = pstat + NW * 2 * 16;                            // [sa][16]
-  float* pooled = fac + L.sa * 16;                             // [Ns]
+  float* fac = pstat + NW * 2 * 16;                            // [kv_rep][sa][16]
+  float* pooled = fac + a.kv_rep * L.sa * 16;                  // [Ns]
   int* sel = reinterpret_cast<int*>(pooled + ((a.nc_cap + 3) / 4 + 4));   // [top_n]
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 15, g = lane >> 4;
   const int bh = blockIdx.x, sb = blockIdx.y;
-  const int b = bh / a.hkv, h = bh % a.hkv;
-  const int G = a.hq / a.hkv;
+  const int hs = a.hkv * a.kv_rep;
+  const int b = bh / hs, h = bh % hs, hc = h / a.kv_rep;     // as in kernel A
+  const int G = a.hq / hs;
   float* wsp = ws + (long)bh * L.total();
-  const float* w_stat = wsp + L.stat();
-  const float* w_bins = wsp + L.bins();
+  // the selection sums the importance over every query head of the kv head: the statistics and window sums of
+  // all its sub-groups (consecutive pairs of the workspace) are read, so each of them takes the same blocks
+  const float* wsib = ws + (long)(bh - h % a.kv_rep) * L.total();
 
   const int cap = PAGED ? a.max_pages * 64 : a.ctx_cap;
   const int ctx = min(a.ctx_lens[b], cap);
@@ -260,10 +263,10 @@ decode_split_attend_kernel(const DecodeArgs a, const SplitLayout L, float* __res
   const float c_attn = a.scale * kLog2e;
 
   // ---- this workgroup's share of the 32-key chunks: item k goes to workgroup k % sb, wavefront (k / sb) % NW
-  const T* kseq = reinterpret_cast<const T*>(a.k_cache) + (PAGED ? (long)h * DK : ((long)b * a.ctx_cap * a.hkv + h) * DK);
+  const T* kseq = reinterpret_cast<const T*>(a.k_cache) + (PAGED ? (long)hc * DK : ((long)b * a.ctx_cap * a.hkv + hc) * DK);
   const long krow = (long)a.hkv * DK;
   const T* vt = reinterpret_cast<const T*>(a.v_cache_t) +
-                (PAGED ? ((long)h * DV + n) * 64 + 8 * g : (((long)b * a.hkv + h) * DV + n) * a.ctx_cap + 8 * g);
+                (PAGED ? ((long)hc * DV + n) * 64 + 8 * g : (((long)b * a.hkv + hc) * DV + n) * a.ctx_cap + 8 * g);
   const long vstep = PAGED ? 16L * 64 : 16L * a.ctx_cap;
   auto issue_kv = [&](ChunkFrags<T, DK, DV>& f, int cb) {
     if constexpr (PAGED) {
@@ -328,38 +331,44 @@ decode_split_attend_kernel(const DecodeArgs a, const SplitLayout L, float* __res
   // global log-sum-exp of the raw scores per head, and each slice's factor exp(M_s - lse).  One thread per
   // (slice, statistic, head) fetches its value (sa <= 32: at most 1024 of them) so that the 16 threads that
   // combine them read LDS, not a chain of dependent global loads.
-  float* st_l = part;                                          // [sa][32], free until the first put()
-  for (int i = tid; i < L.sa * 32; i += NW * 64) st_l[i] = w_stat[i];
+  float* st_l = part;                                          // [kv_rep][sa][32], free until the first put()
+  for (int i = tid; i < a.kv_rep * L.sa * 32; i += NW * 64)
+    st_l[i] = wsib[(long)(i / (L.sa * 32)) * L.total() + L.stat() + i % (L.sa * 32)];
   __syncthreads();
-  if (tid < 16) {
+  if (tid < 16 * a.kv_rep) {                                   // (sub-group, head)
+    const int hd = tid & 15;
+    const float* sj = st_l + (tid >> 4) * L.sa * 32;
+    float* fj = fac + (tid >> 4) * L.sa * 16;
     float M = kNegInf;
-    for (int s = 0; s < L.sa; ++s) M = fmaxf(M, st_l[s * 32 + tid]);
+    for (int s = 0; s < L.sa; ++s) M = fmaxf(M, sj[s * 32 + hd]);
     float Z = 0.f;
     for (int s = 0; s < L.sa; ++s) {
-      const float ms = st_l[s * 32 + tid];
-      if (ms != kNegInf) Z += st_l[s * 32 + 16 + tid] * fast_exp2((ms - M) * kLog2e);
+      const float ms = sj[s * 32 + hd];
+      if (ms != kNegInf) Z += sj[s * 32 + 16 + hd] * fast_exp2((ms - M) * kLog2e);
     }
-    const float lse2 = (Nc > 0 && tid < G) ? (M + __logf(Z)) * kLog2e : __builtin_huge_valf();   // padding heads drop out
+    const float lse2 = (Nc > 0 && hd < G) ? (M + __logf(Z)) * kLog2e : __builtin_huge_valf();   // padding heads drop out
     for (int s = 0; s < L.sa; ++s) {
-      const float ms = st_l[s * 32 + tid];
-      fac[s * 16 + tid] = ms == kNegInf ? 0.f : fast_exp2(fmaf(ms, kLog2e, -lse2));
+      const float ms = sj[s * 32 + hd];
+      fj[s * 16 + hd] = ms == kNegInf ? 0.f : fast_exp2(fmaf(ms, kLog2e, -lse2));
     }
   }
   for (int i = tid; i < Ns; i += NW * 64) pooled[i] = 0.f;
   __syncthreads();
-  for (int base = 0; base < L.sa * L.nb; base += 4 * NW * 64) {
+  const int per_sub = L.sa * L.nb;
+  for (int base = 0; base < a.kv_rep * per_sub; base += 4 * NW * 64) {
     f32x4_t x[4][4];
     int js[4], ss[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {                     // all loads of this pass first
       const int idx = base + u * NW * 64 + tid;
-      const int s = idx / L.nb, lb = idx % L.nb;
+      const int sub = idx / per_sub, rem = idx % per_sub;
+      const int s = rem / L.nb, lb = rem % L.nb;
       const int j = s * (L.slice / 4) - 1 + lb;
-      const bool ok = idx < L.sa * L.nb && j >= 0 && j < Ns && s * L.slice < Nc;
+      const bool ok = idx < a.kv_rep * per_sub && j >= 0 && j < Ns && s * L.slice < Nc;
       js[u] = ok ? j : -1;
-      ss[u] = s;
+      ss[u] = sub * L.sa + s;
       if (ok) {
-        const float* src = w_bins + ((long)s * L.nb + lb) * 16;
+        const float* src = wsib + (long)sub * L.total() + L.bins() + ((long)s * L.nb + lb) * 16;
 #pragma unroll
         for (int q4 = 0; q4 < 4; ++q4) x[u][q4] = *reinterpret_cast<const f32x4_t*>(src + 4 * q4);
       }
@@ -391,7 +400,7 @@ decode_split_attend_kernel(const DecodeArgs a, const SplitLayout L, float* __res
     wave_topn_shortlist<PER>(v, a.top_n, lane, cand_v, cand_i, [&](int rr, int val) {
       if (lane == 0) {
         sel[rr] = val;
-        if (a.indices != nullptr && sb == 0) a.indices[((long)b * a.hkv + h) * a.top_n + rr] = val;
+        if (a.indices != nullptr && sb == 0 && h % a.kv_rep == 0) a.indices[((long)b * a.hkv + hc) * a.top_n + rr] = val;
       }
     });
   }
@@ -439,8 +448,9 @@ decode_split_merge_kernel(const DecodeArgs a, const SplitLayout L, const float* 
   __shared__ float sm[3][MAXS][16], sl[3][MAXS][16];           // branch 0 selected, 1 window, 2 compressed
   const int tid = threadIdx.x, r = tid & 15, dg = tid >> 4;
   const int bh = blockIdx.x, d = blockIdx.y * 16 + dg;
-  const int b = bh / a.hkv, h = bh % a.hkv;
-  const int G = a.hq / a.hkv;
+  const int hs = a.hkv * a.kv_rep;
+  const int b = bh / hs, h = bh % hs;                       // h: sub-group, as in kernel A
+  const int G = a.hq / hs;
   const float* wsp = ws + (long)bh * L.total();
   const int cap = a.block_table != nullptr ? a.max_pages * 64 : a.ctx_cap;
   if (min(a.ctx_lens[b], cap) <= 0) return;
@@ -500,12 +510,13 @@ template <typename T, int DK, int DV>
 static int launch_decode_split_t(const DecodeArgs& a, int splits, float* ws, hipStream_t st) {
   const SplitLayout L = split_layout(a, splits);
   if (L.sa > kSplitMaxSlices || L.sb > kSplitMaxSplits) return -2;
+  if (a.kv_rep < 1 || (long)a.kv_rep * L.sa * 32 > (long)kSplitWaves * DV * 17 || 16 * a.kv_rep > kSplitWaves * 64) return -2;
   const int ns_cap = (a.nc_cap + 3) / 4 + 1;                  // bound of the pooled bins (windows of 5 every 4)
   const bool big = ns_cap > 64 * 10;                          // more bins than ten per lane: the wide top-n
-  const int pairs = a.batch * a.hkv;
+  const int pairs = a.batch * a.hkv * a.kv_rep;
   const size_t base = ((size_t)kSplitWaves * DV * 17 + kSplitWaves * 32) * sizeof(float);
   const size_t smem_a = base + ((size_t)kSplitWaves * 16 + (size_t)L.nb * 16) * sizeof(float);
-  const size_t smem_b = base + ((size_t)L.sa * 16 + (a.nc_cap + 3) / 4 + 4) * sizeof(float) + (size_t)a.top_n * sizeof(int) + 64;
+  const size_t smem_b = base + ((size_t)a.kv_rep * L.sa * 16 + (a.nc_cap + 3) / 4 + 4) * sizeof(float) + (size_t)a.top_n * sizeof(int) + 64;
   {
     auto fn = decode_split_cmp_kernel<T, DK, DV>;
     if (int rc = set_smem(reinterpret_cast<const void*>(fn), smem_a)) return rc;

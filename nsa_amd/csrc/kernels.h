@@ -132,6 +132,9 @@ struct DecodeArgs {
   // pool [page][hkv][dv][64]; page i of sequence b is block_table[b * max_pages + i]; ctx_cap is unused.
   // The compressed caches stay contiguous per sequence (1/16 of the K/V).
   const int32_t* block_table; int max_pages;
+  // GQA groups beyond 16 heads (split schedule only): sub-groups of 16 query heads per kv head; each runs as a
+  // pair of its own on the kv head's caches, and the selection sums the importance over all of them
+  int kv_rep = 1;
 };
 
 // Split of a projection GEMM's packed rows [q | k | v | gate logits] into the attention operands with

@@ -234,7 +234,8 @@ def nsa_decode_step(q: torch.Tensor, cache, gates: Optional[torch.Tensor] = None
     most of the chip idle and its ~60 us critical path sets the step time, so the work is split 8 ways
     (three launches, partial results in a workspace kept on the cache object).  Caches with more
     compressed rows than one workgroup keeps in registers (contexts beyond ~36k tokens) always take the
-    split schedule, whose first launch cuts the compressed rows into slices of at most 384.
+    split schedule, whose first launch cuts the compressed rows into slices of at most 384.  So do GQA groups of
+    32, 48 or 64 heads: every 16 heads run as a pair of their own, the picks come from the whole group.
 
     out [B,Hq,Dv] / indices int32 [B,Hkv,S]: result buffers of the caller (allocated here when None).
     static_scratch: run the split schedule with its partial results in the library's own fixed device array
@@ -265,13 +266,21 @@ def nsa_decode_step(q: torch.Tensor, cache, gates: Optional[torch.Tensor] = None
     paged = isinstance(cache, NSAPagedDecodeCache)
     lib = _lib.load()
     long_cache = cache.nc_cap > lib.nsa_decode_max_compressed()
+    group = hq // cache.hkv if hq % cache.hkv == 0 else 0
+    sub_groups = group // 16 if group > 16 and group % 16 == 0 else 1    # 16-head sub-groups per kv head
+    if sub_groups > 1:
+        # groups of 32, 48, 64 heads: the split schedule runs every 16 heads as a pair of their own
+        long_cache = True
     if splits is None:
-        pairs = B * cache.hkv
+        pairs = B * cache.hkv * sub_groups
         # measured at 32k context: 8 splits halve the step up to 32 pairs and still win at 64 (46 vs 64 us);
         # at 128 pairs one workgroup per pair is as fast and needs no workspace
         splits = 8 if pairs <= 64 and (pool_k, pool_s, pool_p) == (5, 4, 0) and selected_block_count <= 64 else 0
         if long_cache and splits == 0:
             splits = 1 if pairs > 64 else 8       # the compressed rows are sliced whatever `splits` says
+    elif splits == 0 and sub_groups > 1:
+        raise NotImplementedError("the one-workgroup decode step is built for GQA groups of at most 16 heads "
+                                  "(pass splits=None or a positive split count)")
     elif splits == 0 and long_cache:
         raise NotImplementedError(
             "the one-workgroup decode step keeps at most %d compressed rows per sequence; this cache holds up "
@@ -288,7 +297,7 @@ def nsa_decode_step(q: torch.Tensor, cache, gates: Optional[torch.Tensor] = None
         _lib.check(rc, "nsa_decode_step_split_static")
         return (out, idx) if return_indices else out
     if splits:
-        need = lib.nsa_decode_split_workspace_bytes(B, cache.hkv, cache.dv, cache.nc_cap, splits)
+        need = lib.nsa_decode_split_workspace_bytes(B, cache.hkv * sub_groups, cache.dv, cache.nc_cap, splits)
         ws = getattr(cache, "_split_ws", None)
         if ws is None or ws.numel() < need:
             ws = cache._split_ws = torch.empty(need, dtype=torch.uint8, device=q.device)

@@ -114,6 +114,33 @@ def test_paged_decode_cfg5_batch_one_workgroup():
            paged=True)
 
 
+@pytest.mark.parametrize("splits", [None, 1, 3])
+@pytest.mark.parametrize("dtype,Hq,Hkv,Dk,Dv,S,W,paged", [
+    (torch.bfloat16, 32, 1, 128, 128, 8, 128, False),
+    (torch.float16, 64, 2, 64, 64, 4, 100, False),
+    (torch.bfloat16, 96, 2, 192, 128, 16, 512, True),
+    (torch.bfloat16, 64, 1, 128, 128, 6, 64, True),
+    (torch.float32, 32, 1, 64, 64, 4, 0, False),
+])
+def test_decode_groups_of_32_48_64_heads(dtype, Hq, Hkv, Dk, Dv, S, W, paged, splits):
+    """GQA groups beyond 16 heads (the reference admits every multiple of 16, nsa/selection_attn.py:800): each 16
+    heads run as a pair of their own on the kv head's caches, the picks come from the importance of the whole
+    group (compare_selection checks them against the oracle's sum over all heads)."""
+    _check(dtype, [2048, 1000, 513, 65, 33, 1], Hq, Hkv, Dk, Dv, S, W, seed=140, splits=splits, paged=paged)
+
+
+def test_decode_big_group_long_context_and_refusal():
+    from nsa_amd.decode import NSADecodeCache, nsa_decode_step
+    _check(torch.bfloat16, [40000, 12345], 32, 1, 128, 128, 16, 512, seed=141)
+    cache = NSADecodeCache(1, 256, 1, 64, 64, device=DEV)
+    cache.fill(torch.zeros(1, 256, 1, 64, dtype=torch.bfloat16, device=DEV),
+               torch.zeros(1, 256, 1, 64, dtype=torch.bfloat16, device=DEV))
+    with pytest.raises(NotImplementedError):
+        nsa_decode_step(torch.zeros(1, 32, 64, dtype=torch.bfloat16, device=DEV), cache, splits=0)
+    with pytest.raises(RuntimeError):        # a group of 24 heads is neither <= 16 nor a multiple of 16
+        nsa_decode_step(torch.zeros(1, 24, 64, dtype=torch.bfloat16, device=DEV), cache)
+
+
 @pytest.mark.parametrize("ctx", [65536, 131072])
 def test_decode_long_context(ctx):
     """Caches beyond what one workgroup keeps in registers (2304 compressed rows) run on the sliced schedule."""

@@ -183,12 +183,13 @@ def test_layer_bf16_projections_match_unfused_oracle_and_equal_lengths_batch():
         assert err <= 2e-2 * max(1.0, float(want.float().abs().max()))
 
 
+@pytest.mark.parametrize("hq,hkv", [(16, 2), (64, 2)])
 @pytest.mark.parametrize("paged", [False, True])
-def test_layer_decode_continues_prefill(paged):
+def test_layer_decode_continues_prefill(paged, hq, hkv):
     """Prompt through the layer with a cache, then single-token calls: every decoded row equals the
-    corresponding row of one prefill over the whole sequence."""
+    corresponding row of one prefill over the whole sequence (also for a GQA group of 32 heads)."""
     from nsa_amd.decode import NSADecodeCache, NSAPagedDecodeCache
-    hidden, hq, hkv, dk, dv, rd = 256, 16, 2, 192, 128, 64
+    hidden, dk, dv, rd = 256, 192, 128, 64
     layer = _layer(torch.bfloat16, hidden, hq, hkv, dk, dv, rd, "mean", "sigmoid", 4, 64).to(DEV)
     B, T0, steps = 2, 250, 20
     x = randn(B, T0 + steps, hidden, seed=840, dtype=torch.bfloat16).to(DEV)
