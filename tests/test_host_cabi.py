@@ -71,7 +71,10 @@ def test_argument_errors_do_not_launch(lib):
     rc = lib.nsa_swa_fwd(p, p, p, p, None, p, 1, 64, 48, 2, 64, 64, 128, 16, 0.1, 0, None)      # GQA group of 24
     assert rc == -2 and b"group size" in lib.nsa_last_error_string()
     rc = lib.nsa_decode_step(p, p, p, p, p, p, None, p, None, 1, 64, 2, 64, 64, 64, 64, 32, 16, 64, 5, 4, 0, 4, 16, 0.1,
-                             0, 0, None)                                                             # group of 32: prefill only
+                             0, 0, None)                                        # group of 32: the split schedule only
+    assert rc == -2 and b"nsa_decode_step_split" in lib.nsa_last_error_string()
+    rc = lib.nsa_decode_step(p, p, p, p, p, p, None, p, None, 1, 48, 2, 64, 64, 64, 64, 32, 16, 64, 5, 4, 0, 4, 16, 0.1,
+                             0, 0, None)                                                             # group of 24
     assert rc == -2 and b"group size" in lib.nsa_last_error_string()
     rc = lib.nsa_decode_step(p, p, p, p, p, p, None, p, None, 1, 4, 1, 64, 64, 4096, 256, 32, 16, 32, 3, 2, 0, 4, 16,
                              0.1, 0, 0, None)                                                        # 128 bins > 68
