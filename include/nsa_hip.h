@@ -332,8 +332,9 @@ int nsa_slc_swa_bwd(const void* q, const void* k, const void* v, const void* o_s
  * out [batch][hq][dv]; indices (optional) int32 [batch][hkv][top_n] receives the selected blocks.
  * nc_cap <= nsa_decode_max_compressed() (the kernel keeps a sequence's compressed scores in the registers of
  * one workgroup; longer caches, up to nsa_decode_split_max_compressed() rows, go through
- * nsa_decode_step_split) and a pooling geometry with at most nc_cap / 4 + 4 <= 640 bins per sequence
- * (pool_stride >= 4); anything else returns NSA_ERR_UNSUPPORTED. */
+ * nsa_decode_step_split), a pooling geometry with at most nc_cap / 4 + 4 <= 640 bins per sequence
+ * (pool_stride >= 4) and a GQA group of at most 16 heads; anything else returns NSA_ERR_UNSUPPORTED and is served
+ * by nsa_decode_step_split. */
 int nsa_decode_max_compressed(void);
 int nsa_decode_split_max_compressed(void);
 int nsa_decode_step(const void* q, const void* k_cache, const void* v_cache_t, const void* ck_cache,
@@ -363,7 +364,9 @@ int nsa_decode_append_paged(const void* k_new, const void* v_new, void* k_pool, 
 /* The same step for small batches: the work of every (sequence, kv head) pair is spread over `splits`
  * workgroups (three launches: compressed slices, selection + window / selected chunks, merge), because one
  * workgroup per pair leaves most of the chip idle below ~128 pairs.  block_table NULL = contiguous caches
- * (ctx_cap used), else the paged pool (max_pages used).  Pooling 5 / 4 / 0 only.  The compressed rows are cut
+ * (ctx_cap used), else the paged pool (max_pages used).  Any pooling geometry with at most 3136 pooled bins per
+ * sequence (selection blocks of 32 keys at compression stride 16, which make more bins than the one-workgroup
+ * step holds, run here).  The compressed rows are cut
  * into max(splits, ceil(nc_cap / 384)) <= 32 slices, so caches of up to nsa_decode_split_max_compressed() rows
  * (contexts of ~196k tokens at stride 16) are served whatever the batch.  The workspace holds
  * partial results only; calls that share it must not overlap.  GQA groups of 32, 48 or 64 heads (what the
@@ -371,6 +374,10 @@ int nsa_decode_append_paged(const void* k_new, const void* v_new, void* k_pool, 
  * a group are a pair of their own on the kv head's caches, the importance is summed over the whole group before
  * the top-n; size the workspace with hkv x (hq / hkv / 16) in place of hkv.  No counterpart in the reference. */
 int64_t nsa_decode_split_workspace_bytes(int batch, int hkv, int dv, int nc_cap, int splits);
+/* The same size for any pooling geometry (the one above is for windows of 5 every 4, and an upper bound for
+ * windows of s + 1 every s >= 4). */
+int64_t nsa_decode_split_pooled_workspace_bytes(int batch, int hkv, int dv, int nc_cap, int splits, int pool_kernel,
+                                                int pool_stride, int pool_pad);
 int nsa_decode_step_split(const void* q, const void* k_cache, const void* v_cache_t, const int32_t* block_table,
                           int max_pages, const void* ck_cache, const void* cv_cache_t, const int32_t* ctx_lens,
                           const void* gates, void* out, int32_t* indices, int batch, int hq, int hkv, int dk, int dv,

@@ -56,6 +56,7 @@ SIGNATURES = {
     "nsa_decode_append": (_I, [_P] * 7 + [_I] * 9 + [_P]),
     "nsa_decode_step_paged": (_I, [_P] * 4 + [_I] + [_P] * 6 + [_I] * 14 + [_F, _I, _I, _P]),
     "nsa_decode_split_workspace_bytes": (_L, [_I] * 5),
+    "nsa_decode_split_pooled_workspace_bytes": (_L, [_I] * 8),
     "nsa_decode_step_split": (_I, [_P] * 4 + [_I] + [_P] * 6 + [_I] * 15 + [_F, _I, _I, _I, _P, _L, _P]),
     "nsa_decode_split_static_bytes": (_L, []),
     "nsa_decode_step_split_static": (_I, [_P] * 4 + [_I] + [_P] * 6 + [_I] * 15 + [_F, _I, _I, _I, _P]),

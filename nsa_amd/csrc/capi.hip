@@ -623,8 +623,6 @@ static int decode_common(const char* what, const void* q, const void* k_cache, c
   a.kv_rep = kv_rep;
   if (splits > 0) {
     if (splits > 16) return fail(NSA_ERR_INVALID, "%s: at most 16 splits", what);
-    if (pool_kernel != 5 || pool_stride != 4 || pool_pad != 0)
-      return fail(NSA_ERR_UNSUPPORTED, "%s: the split step is built for pooling windows of 5 every 4 without padding", what);
     if (top_n > 64) return fail(NSA_ERR_UNSUPPORTED, "%s: at most 64 selected blocks", what);
     if (static_scratch) {
       const int rc = nsa::launch_decode_split_static(a, splits, stream);
@@ -633,6 +631,7 @@ static int decode_common(const char* what, const void* q, const void* k_cache, c
                     "holds %lld (fewer sequences, kv heads or splits per call)", what,
                     (long long)nsa::decode_split_workspace_bytes(a, splits), (long long)nsa::decode_split_static_bytes());
       if (rc == -2) return fail(NSA_ERR_UNSUPPORTED, "%s: head dims or split count not built", what);
+      if (rc == -3) return fail(NSA_ERR_UNSUPPORTED, "%s: more pooled bins per sequence than the top-n holds (3136)", what);
       if (rc == -4) return fail(NSA_ERR_LAUNCH, "%s: could not look up the library's scratch array on this device", what);
       return finish(rc, what);
     }
@@ -640,6 +639,7 @@ static int decode_common(const char* what, const void* q, const void* k_cache, c
       return fail(NSA_ERR_INVALID, "%s: workspace missing, misaligned or smaller than nsa_decode_split_workspace_bytes", what);
     const int rc = nsa::launch_decode_split(a, splits, workspace, stream);
     if (rc == -2) return fail(NSA_ERR_UNSUPPORTED, "%s: head dims or split count not built", what);
+    if (rc == -3) return fail(NSA_ERR_UNSUPPORTED, "%s: more pooled bins per sequence than the top-n holds (3136)", what);
     return finish(rc, what);
   }
   {
@@ -657,11 +657,19 @@ static int decode_common(const char* what, const void* q, const void* k_cache, c
   return finish(rc, what);
 }
 
-int64_t nsa_decode_split_workspace_bytes(int batch, int hkv, int dv, int nc_cap, int splits) {
-  if (batch <= 0 || hkv <= 0 || dv <= 0 || nc_cap <= 0 || splits <= 0) return 0;
+int64_t nsa_decode_split_pooled_workspace_bytes(int batch, int hkv, int dv, int nc_cap, int splits, int pool_kernel,
+                                                int pool_stride, int pool_pad) {
+  if (batch <= 0 || hkv <= 0 || dv <= 0 || nc_cap <= 0 || splits <= 0 || pool_kernel <= 0 || pool_stride <= 0 ||
+      pool_pad < 0)
+    return 0;
   nsa::DecodeArgs a{};
   a.batch = batch; a.hkv = hkv; a.dv = dv; a.nc_cap = nc_cap;
+  a.pool_k = pool_kernel; a.pool_s = pool_stride; a.pool_p = pool_pad;
   return nsa::decode_split_workspace_bytes(a, splits);
+}
+
+int64_t nsa_decode_split_workspace_bytes(int batch, int hkv, int dv, int nc_cap, int splits) {
+  return nsa_decode_split_pooled_workspace_bytes(batch, hkv, dv, nc_cap, splits, 5, 4, 0);
 }
 
 int nsa_decode_step_split(const void* q, const void* k_cache, const void* v_cache_t, const int32_t* block_table,

@@ -10,8 +10,8 @@
 //      window sums, takes the top-n blocks (all SB workgroups get the same answer), then attends its share
 //      of the 32-key chunks of the window and of the selected blocks; partial states per branch
 //   C  merges the partial states of the three branches, gates, stores
-// Same arithmetic as the one-workgroup kernel up to the order of fp32 sums.  Pooling 5 / 4 / 0 only
-// (windows of 5 compressed rows every 4, the default geometry).
+// Same arithmetic as the one-workgroup kernel up to the order of fp32 sums.  Any pooling geometry; windows of 5
+// compressed rows every 4 (the default) add their rows to the bins three sums at a time, others row by row.
 #include <mutex>
 
 #include "decode_common.h"
@@ -25,6 +25,14 @@ constexpr int kSplitMaxSlice = 32 * kSplitWaves * kSplitMaxChunks;   // 384 rows
 // floats per (sequence, kv head) in the workspace
 struct SplitLayout {
   int sa, sb, slice, nb, dv;
+  int ns_cap;                          // bound of the pooled bins of a sequence
+  int pool_k, pool_s, pool_p;
+  // bin of a sequence that local bin 0 of the slice starting at row c_lo stands for: the first one a row of the
+  // slice can belong to (bin j pools rows j * s - p .. j * s - p + k - 1); may be -1 for the first slice
+  __host__ __device__ int first_bin(int c_lo) const {
+    const int x = c_lo + pool_p - pool_k + pool_s;
+    return x >= 0 ? x / pool_s : -((-x + pool_s - 1) / pool_s);
+  }
   __host__ __device__ long stat() const { return 0; }                                   // [sa][2][16]
   __host__ __device__ long bins() const { return (long)sa * 32; }                       // [sa][nb][16]
   __host__ __device__ long cmp() const { return bins() + (long)sa * nb * 16; }          // [sa][1 + dv][16]
@@ -37,7 +45,10 @@ static SplitLayout split_layout(const DecodeArgs& a, int splits) {
   l.sa = max(splits, (a.nc_cap + kSplitMaxSlice - 1) / kSplitMaxSlice);
   l.slice = ((a.nc_cap + l.sa - 1) / l.sa + 31) / 32 * 32;
   l.sb = splits;
-  l.nb = l.slice / 4 + 2;
+  l.pool_k = max(a.pool_k, 1); l.pool_s = max(a.pool_s, 1); l.pool_p = max(a.pool_p, 0);
+  l.nb = (l.slice + l.pool_k - 2) / l.pool_s + 2;            // bins that the rows of one slice can belong to
+  const int span = a.nc_cap + 2 * l.pool_p - l.pool_k;
+  l.ns_cap = span < 0 ? 0 : (span + l.pool_s - 1) / l.pool_s + 1;
   l.dv = a.dv;
   return l;
 }
@@ -162,9 +173,12 @@ decode_split_cmp_kernel(const DecodeArgs a, const SplitLayout L, float* __restri
   }
   if (tid < 16) { w_stat[tid] = M; w_stat[16 + tid] = Z; }          // head n = tid (wavefront 0, g = 0)
 
-  // pooled window sums per head, relative to the slice maximum: rows 4j .. 4j+4 make bin j; local bin
-  // index = j - (c_lo / 4 - 1), so that the bin a slice's first row completes is local bin 0
+  // pooled window sums per head, relative to the slice maximum; local bin index = j - L.first_bin(c_lo).
+  // Windows of 5 every 4: rows 4j .. 4j+4 make bin j, first_bin = c_lo / 4 - 1 (the bin that the slice's first
+  // row completes).
   const float Ml2 = M * kLog2e;
+  const bool fast_pool = L.pool_k == 5 && L.pool_s == 4 && L.pool_p == 0;
+  const int jf = L.first_bin(c_lo);
 #pragma unroll
   for (int i = 0; i < MAXC; ++i) {
     const int cb = c_lo + 32 * (wave + NW * i);
@@ -173,11 +187,24 @@ decode_split_cmp_kernel(const DecodeArgs a, const SplitLayout L, float* __restri
 #pragma unroll
       for (int e = 0; e < 8; ++e) v[e] = fast_exp2(fmaf(sc[i][e], kLog2e, -Ml2));     // 0 past c_hi
       const int c0 = cb + 8 * g;
-      if (c0 < c_hi) {
-        const int b0 = (c0 - c_lo) / 4 + 1;
-        atomicAdd(&binsL[(b0 - 1) * 16 + n], v[0]);
-        atomicAdd(&binsL[b0 * 16 + n], (v[0] + v[1]) + (v[2] + v[3]) + v[4]);
-        atomicAdd(&binsL[(b0 + 1) * 16 + n], (v[4] + v[5]) + (v[6] + v[7]));
+      if (fast_pool) {
+        if (c0 < c_hi) {
+          const int b0 = (c0 - c_lo) / 4 + 1;
+          atomicAdd(&binsL[(b0 - 1) * 16 + n], v[0]);
+          atomicAdd(&binsL[b0 * 16 + n], (v[0] + v[1]) + (v[2] + v[3]) + v[4]);
+          atomicAdd(&binsL[(b0 + 1) * 16 + n], (v[4] + v[5]) + (v[6] + v[7]));
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int c = c0 + e;
+          if (c < c_hi) {
+            const int num = c + L.pool_p - L.pool_k + 1;
+            const int b_lo = num <= 0 ? 0 : (num + L.pool_s - 1) / L.pool_s;
+            const int b_hi = min((c + L.pool_p) / L.pool_s, jf + L.nb - 1);
+            for (int bb = b_lo; bb <= b_hi; ++bb) atomicAdd(&binsL[(bb - jf) * 16 + n], v[e]);
+          }
+        }
       }
     }
   }
@@ -236,7 +263,7 @@ decode_split_attend_kernel(const DecodeArgs a, const SplitLayout L, float* __res
   float* pstat = part + NW * DV * PLD;                         // [NW][2][16]
   float* fac = pstat + NW * 2 * 16;                            // [kv_rep][sa][16]
   float* pooled = fac + a.kv_rep * L.sa * 16;                  // [Ns]
-  int* sel = reinterpret_cast<int*>(pooled + ((a.nc_cap + 3) / 4 + 4));   // [top_n]
+  int* sel = reinterpret_cast<int*>(pooled + L.ns_cap + 4);    // [top_n]
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -256,9 +283,9 @@ decode_split_attend_kernel(const DecodeArgs a, const SplitLayout L, float* __res
   const int t = ctx - 1;
   const int Nc = ctx >= a.block ? min((ctx - a.block) / a.stride + 1, a.nc_cap) : 0;
   int Ns = 0;
-  if (Nc >= 5) {
-    Ns = (Nc - 5 + 3) / 4 + 1;
-    if ((Ns - 1) * 4 >= Nc) --Ns;
+  if (Nc > 0 && Nc + 2 * L.pool_p >= L.pool_k) {
+    Ns = (Nc + 2 * L.pool_p - L.pool_k + L.pool_s - 1) / L.pool_s + 1;
+    if ((Ns - 1) * L.pool_s >= Nc + L.pool_p) --Ns;
   }
   const float c_attn = a.scale * kLog2e;
 
@@ -363,7 +390,7 @@ decode_split_attend_kernel(const DecodeArgs a, const SplitLayout L, float* __res
       const int idx = base + u * NW * 64 + tid;
       const int sub = idx / per_sub, rem = idx % per_sub;
       const int s = rem / L.nb, lb = rem % L.nb;
-      const int j = s * (L.slice / 4) - 1 + lb;
+      const int j = L.first_bin(s * L.slice) + lb;
       const bool ok = idx < a.kv_rep * per_sub && j >= 0 && j < Ns && s * L.slice < Nc;
       js[u] = ok ? j : -1;
       ss[u] = sub * L.sa + s;
@@ -395,7 +422,10 @@ decode_split_attend_kernel(const DecodeArgs a, const SplitLayout L, float* __res
     for (int k = 0; k < PER; ++k) {
       const int bb = lane + 64 * k;
       v[k] = -1.f;
-      if (bb < Ns) v[k] = pooled[bb] / (float)(min(4 * bb + 5, Nc) - 4 * bb);
+      if (bb < Ns) {
+        const int lo = bb * L.pool_s - L.pool_p;
+        v[k] = pooled[bb] / (float)(min(lo + L.pool_k, Nc + L.pool_p) - lo);
+      }
     }
     wave_topn_shortlist<PER>(v, a.top_n, lane, cand_v, cand_i, [&](int rr, int val) {
       if (lane == 0) {
@@ -511,12 +541,11 @@ static int launch_decode_split_t(const DecodeArgs& a, int splits, float* ws, hip
   const SplitLayout L = split_layout(a, splits);
   if (L.sa > kSplitMaxSlices || L.sb > kSplitMaxSplits) return -2;
   if (a.kv_rep < 1 || (long)a.kv_rep * L.sa * 32 > (long)kSplitWaves * DV * 17 || 16 * a.kv_rep > kSplitWaves * 64) return -2;
-  const int ns_cap = (a.nc_cap + 3) / 4 + 1;                  // bound of the pooled bins (windows of 5 every 4)
-  const bool big = ns_cap > 64 * 10;                          // more bins than ten per lane: the wide top-n
+  const bool big = L.ns_cap > 64 * 10;                        // more bins than ten per lane: the wide top-n
   const int pairs = a.batch * a.hkv * a.kv_rep;
   const size_t base = ((size_t)kSplitWaves * DV * 17 + kSplitWaves * 32) * sizeof(float);
   const size_t smem_a = base + ((size_t)kSplitWaves * 16 + (size_t)L.nb * 16) * sizeof(float);
-  const size_t smem_b = base + ((size_t)a.kv_rep * L.sa * 16 + (a.nc_cap + 3) / 4 + 4) * sizeof(float) + (size_t)a.top_n * sizeof(int) + 64;
+  const size_t smem_b = base + ((size_t)a.kv_rep * L.sa * 16 + L.ns_cap + 4) * sizeof(float) + (size_t)a.top_n * sizeof(int) + 64;
   {
     auto fn = decode_split_cmp_kernel<T, DK, DV>;
     if (int rc = set_smem(reinterpret_cast<const void*>(fn), smem_a)) return rc;
@@ -527,7 +556,8 @@ static int launch_decode_split_t(const DecodeArgs& a, int splits, float* ws, hip
     hipLaunchKernelGGL(fn, dim3(pairs, L.sb), dim3(kSplitWaves * 64), smem_b, st, a, L, ws);
     return 0;
   };
-  constexpr int PER_BIG = (kSplitMaxSlices * kSplitMaxSlice / 4 + 1 + 63) / 64;   // 3073 bins at most
+  constexpr int PER_BIG = (kSplitMaxSlices * kSplitMaxSlice / 4 + 1 + 63) / 64;   // 3073 bins (the longest cache, windows every 4)
+  if (L.ns_cap > 64 * PER_BIG) return -3;
   static_assert(64 * 10 >= 32 * kDecWaves * kDecMaxChunks / 4 + 1, "ten bins per lane cover the short caches");
   int rc;
   if (a.block_table != nullptr)

@@ -268,19 +268,28 @@ def nsa_decode_step(q: torch.Tensor, cache, gates: Optional[torch.Tensor] = None
     long_cache = cache.nc_cap > lib.nsa_decode_max_compressed()
     group = hq // cache.hkv if hq % cache.hkv == 0 else 0
     sub_groups = group // 16 if group > 16 and group % 16 == 0 else 1    # 16-head sub-groups per kv head
-    if sub_groups > 1:
+    # the one-workgroup kernel holds nc_cap / 4 + 4 pooled bins (640 at most): pooling strides below 4 (selection
+    # blocks of 32 keys at stride 16) make more and run on the split schedule, which holds 3136
+    span = cache.nc_cap + 2 * pool_p - pool_k
+    ns_cap = 0 if span < 0 else (span + pool_s - 1) // pool_s + 1
+    many_bins = ns_cap > min(cache.nc_cap // 4 + 4, 640)
+    if sub_groups > 1 or many_bins:
         # groups of 32, 48, 64 heads: the split schedule runs every 16 heads as a pair of their own
         long_cache = True
     if splits is None:
         pairs = B * cache.hkv * sub_groups
         # measured at 32k context: 8 splits halve the step up to 32 pairs and still win at 64 (46 vs 64 us);
         # at 128 pairs one workgroup per pair is as fast and needs no workspace
-        splits = 8 if pairs <= 64 and (pool_k, pool_s, pool_p) == (5, 4, 0) and selected_block_count <= 64 else 0
+        splits = 8 if pairs <= 64 and selected_block_count <= 64 else 0
         if long_cache and splits == 0:
             splits = 1 if pairs > 64 else 8       # the compressed rows are sliced whatever `splits` says
     elif splits == 0 and sub_groups > 1:
         raise NotImplementedError("the one-workgroup decode step is built for GQA groups of at most 16 heads "
                                   "(pass splits=None or a positive split count)")
+    elif splits == 0 and many_bins:
+        raise NotImplementedError("the one-workgroup decode step holds %d pooled bins per sequence, this geometry "
+                                  "makes up to %d (pass splits=None or a positive split count)"
+                                  % (min(cache.nc_cap // 4 + 4, 640), ns_cap))
     elif splits == 0 and long_cache:
         raise NotImplementedError(
             "the one-workgroup decode step keeps at most %d compressed rows per sequence; this cache holds up "
@@ -297,7 +306,8 @@ def nsa_decode_step(q: torch.Tensor, cache, gates: Optional[torch.Tensor] = None
         _lib.check(rc, "nsa_decode_step_split_static")
         return (out, idx) if return_indices else out
     if splits:
-        need = lib.nsa_decode_split_workspace_bytes(B, cache.hkv * sub_groups, cache.dv, cache.nc_cap, splits)
+        need = lib.nsa_decode_split_pooled_workspace_bytes(B, cache.hkv * sub_groups, cache.dv, cache.nc_cap, splits,
+                                                           pool_k, pool_s, pool_p)
         ws = getattr(cache, "_split_ws", None)
         if ws is None or ws.numel() < need:
             ws = cache._split_ws = torch.empty(need, dtype=torch.uint8, device=q.device)

@@ -209,8 +209,28 @@ def test_decode_one_workgroup_kernel_rejects_what_it_cannot_hold():
     small = NSADecodeCache(1, 4096, 1, 64, 64, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(NotImplementedError):
         nsa_decode_step(q, small, selection_block=32, splits=0)
-    with pytest.raises(NotImplementedError):
-        nsa_decode_step(q, small, selection_block=32)        # the split schedule is built for 5 / 4 / 0 only
+    nsa_decode_step(q, small, selection_block=32)            # the split schedule takes it (oracle cases below)
+
+
+@pytest.mark.parametrize("splits", [None, 1, 5])
+@pytest.mark.parametrize("dtype,Hq,Hkv,Dk,Dv,S,W,sel_block,paged", [
+    (torch.bfloat16, 16, 1, 128, 128, 8, 128, 32, False),
+    (torch.float16, 32, 2, 64, 64, 16, 100, 32, True),
+    (torch.bfloat16, 8, 2, 192, 128, 4, 64, 128, False),
+    (torch.bfloat16, 64, 2, 128, 128, 6, 0, 32, False),
+    (torch.float32, 4, 1, 64, 64, 3, 32, 96, True),
+])
+def test_decode_other_selection_block_sizes(dtype, Hq, Hkv, Dk, Dv, S, W, sel_block, paged, splits):
+    """Selection blocks of 32 keys (the reference's own selection test, tests/test_parallel_nsa.py:169; pooling
+    windows of 3 every 2, twice the bins of the default), 96 and 128 keys on the split schedule, whose first launch
+    adds the rows of such windows to the bins one by one."""
+    _check(dtype, [2048, 1000, 513, 100, 65, 33, 1], Hq, Hkv, Dk, Dv, S, W, seed=150, splits=splits, paged=paged,
+           sel_block=sel_block)
+
+
+def test_decode_selection_block_32_long_context():
+    _check(torch.bfloat16, [50000, 20001], 16, 1, 128, 128, 16, 512, seed=151, sel_block=32)
+    _check(torch.bfloat16, [3000] * 70, 16, 1, 64, 64, 4, 64, seed=152, sel_block=32, which=[0, 69])   # 70 pairs: splits = 1
 
 
 def test_cache_append_beyond_capacity_raises():

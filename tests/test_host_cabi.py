@@ -314,7 +314,13 @@ def test_split_decode_argument_errors_do_not_launch(lib):
 
     assert call(splits=0) == -1
     assert call(splits=17) == -1
-    assert call(pool=(3, 2, 0)) == -2 and b"pooling" in lib.nsa_last_error_string()
+    # other pooling geometries are served; their workspace is sized by the pooled variant (windows every 2 rows
+    # make twice the bins of the default, which the plain size function assumes)
+    pooled = lib.nsa_decode_split_pooled_workspace_bytes
+    assert pooled(2, 4, 128, 2048, 8, 5, 4, 0) == need
+    assert pooled(2, 4, 128, 2048, 8, 3, 2, 0) > need >= pooled(2, 4, 128, 2048, 8, 9, 8, 0)
+    assert pooled(2, 4, 128, 2048, 8, 0, 2, 0) == 0
+    assert call(pool=(3, 2, 0), ws_bytes=need) == -1 and b"workspace" in lib.nsa_last_error_string()
     assert call(ws=None) == -1
     assert call(ws_bytes=16) == -1 and b"workspace" in lib.nsa_last_error_string()
     assert call(top_n=65) == -2
