@@ -94,11 +94,11 @@ def test_qkv_rope_pack_is_the_transpose_of_split(inter):
     assert (again[:, ~covered] == 0).all()
 
 
-def _layer(dtype, hidden, hq, hkv, dk, dv, rd, mode, act, S, W, bias=False, inter=False, seed=0):
+def _layer(dtype, hidden, hq, hkv, dk, dv, rd, mode, act, S, W, bias=False, inter=False, seed=0, sel_block=64):
     from nsa_amd.layer import NSAAttentionLayer
     torch.manual_seed(seed)
     layer = NSAAttentionLayer(hidden, hq, hkv, qk_head_dim=dk, v_head_dim=dv, rope_dim=rd, rope_interleaved=inter,
-                              bias=bias, selected_block_count=S, sliding_window=W, compressor_mode=mode,
+                              bias=bias, selection_block=sel_block, selected_block_count=S, sliding_window=W, compressor_mode=mode,
                               gate_activation=act, dtype=dtype)
     with torch.no_grad():                      # livelier than the default init: gates of both signs
         layer.attn.gating.weight.normal_(0, 0.3)
@@ -183,14 +183,17 @@ def test_layer_bf16_projections_match_unfused_oracle_and_equal_lengths_batch():
         assert err <= 2e-2 * max(1.0, float(want.float().abs().max()))
 
 
-@pytest.mark.parametrize("hq,hkv", [(16, 2), (64, 2)])
+@pytest.mark.parametrize("hq,hkv,sel_block", [(16, 2, 64), (64, 2, 64), (16, 2, 32)])
 @pytest.mark.parametrize("paged", [False, True])
-def test_layer_decode_continues_prefill(paged, hq, hkv):
+def test_layer_decode_continues_prefill(paged, hq, hkv, sel_block):
     """Prompt through the layer with a cache, then single-token calls: every decoded row equals the
-    corresponding row of one prefill over the whole sequence (also for a GQA group of 32 heads)."""
+    corresponding row of one prefill over the whole sequence (also for a GQA group of 32 heads).  With selection
+    blocks of 32 keys the picks are a real choice (8 blocks, 4 picks), and a prefill row's picks depend on the
+    compressed rows after it (the importance softmax is normalised over all of them, per head, before the head
+    sum): there a decoded row is compared with the last row of a prefill over exactly the cached tokens."""
     from nsa_amd.decode import NSADecodeCache, NSAPagedDecodeCache
     hidden, dk, dv, rd = 256, 192, 128, 64
-    layer = _layer(torch.bfloat16, hidden, hq, hkv, dk, dv, rd, "mean", "sigmoid", 4, 64).to(DEV)
+    layer = _layer(torch.bfloat16, hidden, hq, hkv, dk, dv, rd, "mean", "sigmoid", 4, 64, sel_block=sel_block).to(DEV)
     B, T0, steps = 2, 250, 20
     x = randn(B, T0 + steps, hidden, seed=840, dtype=torch.bfloat16).to(DEV)
     with torch.no_grad():
@@ -200,12 +203,13 @@ def test_layer_decode_continues_prefill(paged, hq, hkv):
         else:
             cache = NSADecodeCache(B, 320, hkv, dk, dv, dtype=torch.bfloat16, device=DEV)
         first, _ = layer(x[:, :T0], past_key_value=cache, use_cache=True)
-        assert max_abs(first, full[:, :T0]) <= 2e-2
+        assert max_abs(first, full[:, :T0] if sel_block == 64 else layer(x[:, :T0])[0]) <= 2e-2
         worst = 0.0
         for s in range(steps):
             out, _ = layer(x[:, T0 + s:T0 + s + 1], past_key_value=cache, use_cache=True)
             assert out.shape == (B, 1, hidden)
-            worst = max(worst, max_abs(out[:, 0], full[:, T0 + s]))
+            row = full[:, T0 + s] if sel_block == 64 else layer(x[:, :T0 + s + 1])[0][:, -1]
+            worst = max(worst, max_abs(out[:, 0], row))
     print("layer decode vs prefill rows max_abs", worst)
     assert int(cache.ctx_lens[0]) == T0 + steps
     assert worst <= 3e-2
