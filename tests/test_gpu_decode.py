@@ -267,6 +267,29 @@ def test_decode_randomized_sweep():
                paged=case % 3 == 2)
 
 
+def test_decode_randomized_sweep_split_schedule_only_shapes():
+    """The same sweep over what only the split schedule serves: GQA groups of 32 and 48 heads, selection blocks
+    of 32, 96 and 128 keys (128 also runs on the one-workgroup kernel; here with explicit split counts)."""
+    g = torch.Generator().manual_seed(78)
+
+    def pick(options):
+        return options[int(torch.randint(0, len(options), (1,), generator=g))]
+
+    for case in range(16):
+        B = pick([1, 2, 3, 5])
+        ctxs = [int(torch.randint(1, 1500, (1,), generator=g)) for _ in range(B)]
+        if case % 4 == 0:
+            ctxs[0] = pick([1, 31, 32, 33, 47, 48, 63, 64, 65, 95, 96, 127, 128, 129])
+        G, Hkv = pick([2, 8, 16, 32, 48]), pick([1, 2])
+        sel_block = pick([32, 32, 96, 128]) if G <= 16 else pick([32, 64])
+        D = pick([64, 128])
+        S, W = pick([1, 3, 4, 16]), pick([0, 17, 64, 512])
+        dtype = pick([torch.bfloat16, torch.float16])
+        print("case", case, ctxs, G, Hkv, D, S, W, sel_block, dtype)
+        _check(dtype, ctxs, G * Hkv, Hkv, D, D, S, W, seed=500 + case, splits=[None, 1, 2, 7][case % 4],
+               paged=case % 3 == 1, sel_block=sel_block)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("splits", [1, 2, 3, 8, 16])
 def test_split_step_equals_one_workgroup_step(dtype, splits):
