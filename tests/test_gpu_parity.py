@@ -756,7 +756,7 @@ def test_module_randomized_selection_block_sizes_and_token_slabs(monkeypatch):
         G = pick([4, 16, 16, 32])
         Hkv = pick([1, 2])
         Dk, Dv = pick([(32, 32), (64, 64), (128, 128), (192, 128)])
-        lsel = pick([32, 32, 128, 64]) if G <= 16 else 64      # groups beyond 16 heads: 64-key pooling geometry only
+        lsel = pick([32, 32, 128, 64])
         S = pick([2, 5, 16]) if lsel <= 64 else pick([2, 4])
         W = pick([16, 64, 200, 512])
         dtype = pick([torch.bfloat16, torch.float16])
