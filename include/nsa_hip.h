@@ -104,8 +104,8 @@ int nsa_compress_bwd(const void* x, const void* w_lin, const void* d_out, void* 
  *   NULL skips the selection;  pooled (optional, float) [total, hkv, sub, pooled_stride] with sub =
  *   max(1, hq / (16 * hkv)) sub-groups (1 for GQA groups up to 16 heads) receives in its first sub-row the
  *   pooled block scores (bins past a sequence's last one up to max_ns are zeroed).  Pass it even when
- *   the scores are not wanted: with it (and a GQA group of 9..16 heads, pooling 5/4/0, max_ns <= 4096,
- *   top_n <= 64) the selection runs as two lean kernels that use it as their hand-over buffer, without
+ *   the scores are not wanted: with it (and pooling windows of s + 1 columns every s, s = 1, 2, 4 or 8, padding
+ *   below 64, max_ns <= 4096, top_n <= 64) the selection runs as two lean kernels that use it as their hand-over buffer, without
  *   it as one slower kernel that keeps the bins in LDS;  keep_pooled == 0 says that the scores themselves are
  *   not wanted: the buffer then only carries the window sums between the two kernels, its contents afterwards
  *   are unspecified, and the second kernel saves writing the averages back;

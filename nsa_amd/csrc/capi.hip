@@ -174,8 +174,8 @@ static int cmp_common(const char* what, int stages, const void* q, const void* c
   if (rc == 0 && select) rc = nsa::launch_select(a, stream);
   if (rc == -6)
     return fail(NSA_ERR_UNSUPPORTED, "%s: GQA groups beyond 16 heads are selected on the two-kernel schedule only "
-                "(pooled buffer given, pooling windows of s + 1 every s with s = 2, 4 or 8, i.e. selection blocks of 2, 4 or 8 "
-                "compression strides, max_ns <= 4096, top_n <= 64)", what);
+                "(pooled buffer given, pooling windows of s + 1 every s with s = 1, 2, 4 or 8, i.e. selection blocks of 1, 2, 4 "
+                "or 8 compression strides, max_ns <= 4096, top_n <= 64)", what);
   return finish(rc, what);
 }
 

@@ -272,12 +272,17 @@ importance_stream_kernel(const CmpArgs a) {
   const int h = blockIdx.y;
   const int coff = a.cu_cmp[st.b];
   const int Nc = a.cu_cmp[st.b + 1] - coff;
-  // pooling windows of ps + 1 columns every ps columns, no padding; ps = 2, 4 or 8 (selection blocks of 2, 4, 8 strides)
-  const int ps = a.pool_s, lps = ps == 2 ? 1 : ps == 4 ? 2 : 3;
+  // pooling windows of ps + 1 columns every ps columns; ps = 1, 2, 4 or 8 (selection blocks of 1, 2, 4, 8 strides).
+  // Padding of `pad` columns (compression blocks beyond two strides): column c sits at position c + pad of the
+  // padded row, the stream runs over positions 0 .. Nc + pad - 1 (lane i of a step = position x0 + i) and bin j
+  // pools positions j * ps .. j * ps + ps, so the bins stay aligned with the lanes whatever the padding.
+  const int ps = a.pool_s, lps = ps == 1 ? 0 : ps == 2 ? 1 : ps == 4 ? 2 : 3;
+  const int pad = a.pool_p;
+  const int Np = Nc + pad;                      // positions that hold a column
   int Ns = 0;
-  if (Nc >= ps + 1) {
-    Ns = (Nc - 2) / ps + 1;                     // ceil((Nc - (ps + 1)) / ps) + 1
-    if ((Ns - 1) * ps >= Nc) --Ns;
+  if (Nc > 0 && Nc + 2 * pad >= ps + 1) {
+    Ns = (Nc + 2 * pad - 2) / ps + 1;           // ceil((Nc + 2 pad - (ps + 1)) / ps) + 1
+    if ((Ns - 1) * ps >= Np) --Ns;
   }
   Ns = min(Ns, a.max_ns);
   if (Ns == 0) return;
@@ -328,18 +333,19 @@ importance_stream_kernel(const CmpArgs a) {
     const int p = tid + i * NT;
     koff[i] = (unsigned)((p / (DK / 8)) * (int)a.ck_row_stride + (p % (DK / 8)) * 8);
   }
-  auto gload = [&](int c0) {
-    if (c0 + CH <= Nc) {
+  auto gload = [&](int x0) {               // rows of the step at position x0: columns x0 - pad .. x0 - pad + CH - 1
+    const int c0 = x0 - pad;
+    if (c0 >= 0 && c0 + CH <= Nc) {
       const unsigned base = (unsigned)c0 * (unsigned)a.ck_row_stride;
 #pragma unroll
       for (int i = 0; i < KPT; ++i)
         if (KPIECES % NT == 0 || tid + i * NT < KPIECES) kr[i] = load8(ckb + (base + koff[i]));
-    } else {                                         // last step: clamp the row
+    } else {                                         // first step under padding, last step: clamp the row
 #pragma unroll
       for (int i = 0; i < KPT; ++i) {
         const int p = tid + i * NT;
         if (KPIECES % NT == 0 || p < KPIECES) {
-          const int sr = min(c0 + p / (DK / 8), Nc - 1);
+          const int sr = max(min(c0 + p / (DK / 8), Nc - 1), 0);
           kr[i] = load8(ckb + (long)sr * a.ck_row_stride + (p % (DK / 8)) * 8);
         }
       }
@@ -368,8 +374,8 @@ importance_stream_kernel(const CmpArgs a) {
   float v[NG][4], e[NG][4], ea[NG], eb[NG];
 #pragma unroll
   for (int j = 0; j < NG; ++j) sp[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  auto pool_store = [&](int c0) {          // window sums of the step that started at column c0
-    const bool live = c0 + lane < Nc;
+  auto pool_store = [&](int c0) {          // window sums of the step that started at position c0
+    const bool live = (unsigned)(c0 + lane - pad) < (unsigned)Nc;
     const int idx = carrier ? (c0 >> lps) - 1 : (c0 >> lps) + (lane >> lps);
 #pragma unroll
     for (int j = 0; j < NG; ++j) {
@@ -380,7 +386,8 @@ importance_stream_kernel(const CmpArgs a) {
 #pragma unroll
       for (int t = 0; t < TP; ++t) {
         const float r = live ? rt[t] : 0.f;
-        float quad = r + dpp_f32<0xB1>(r);                   // quad_perm [1,0,3,2]: pairs
+        float quad = r;
+        if (ps >= 2) quad += dpp_f32<0xB1>(r);               // quad_perm [1,0,3,2]: pairs
         if (ps >= 4) quad += dpp_f32<0x4E>(quad);            // quad_perm [2,3,0,1]: quads
         if (ps == 8) quad += __shfl_xor(quad, 4);            // eight columns
         const float nxt = dpp_f32<0x130>(r);                 // wave_shl:1 -> column c0 + i + 1 (0 in lane 63)
@@ -402,8 +409,8 @@ importance_stream_kernel(const CmpArgs a) {
     else { v[j][tp] = ea[j] + eb[j]; asm volatile("" : "+v"(v[j][tp])); }
   };
   int buf = 0;
-  for (int c0 = 0; c0 < Nc; c0 += CH) {
-    const bool has_next = c0 + CH < Nc;
+  for (int c0 = 0; c0 < Np; c0 += CH) {    // c0: position of the step's first lane
+    const bool has_next = c0 + CH < Np;
     if (has_next) gload(c0 + CH);
     const T* bk = ldsK + buf * CH * KLD;
 #pragma unroll
@@ -436,9 +443,9 @@ importance_stream_kernel(const CmpArgs a) {
   }
 #pragma unroll
   for (int op = 0; op < NOPS; ++op) exp_op(op, 3);
-  pool_store(((Nc - 1) >> 6) << 6);
+  pool_store(((Np - 1) >> 6) << 6);
   if (carrier) {
-    const int b = ((((Nc - 1) >> 6) << 6) >> lps) + (64 >> lps) - 1;   // last bin of the last step: no next column
+    const int b = ((((Np - 1) >> 6) << 6) >> lps) + (64 >> lps) - 1;   // last bin of the last step: no next column
 #pragma unroll
     for (int j = 0; j < NG; ++j)
 #pragma unroll
@@ -576,7 +583,8 @@ template <typename T, int DK>
 static int launch_select_t(const CmpArgs& a, hipStream_t st) {
   // (groups below 16 heads run with the missing heads as padded rows: their log-sum-exp is +inf, their weight 0)
   if (a.pooled != nullptr && a.max_ns <= 4096 && a.top_n <= 64 && a.hq / a.hkv <= 16 &&
-      (a.pool_s == 2 || a.pool_s == 4 || a.pool_s == 8) && a.pool_k == a.pool_s + 1 && a.pool_p == 0)
+      (a.pool_s == 1 || a.pool_s == 2 || a.pool_s == 4 || a.pool_s == 8) && a.pool_k == a.pool_s + 1 &&
+      a.pool_p >= 0 && a.pool_p < 64)
     return launch_select_stream<T, DK>(a, st);
   if (a.kv_rep > 1) return -6;      // groups beyond 16 heads exist on the two-kernel schedule only
   CmpArgs b = a;

@@ -467,8 +467,6 @@ def test_module_backward_randomized_block_sizes_and_groups():
         Hkv = pick([1, 2])
         D = pick([32, 64, 128]) if G <= 16 else pick([64, 128])
         sel_block = pick([16, 16, 32, 32, 128])       # (8 keys would be below the compression stride of 16)
-        if G > 16 and sel_block < 32:
-            sel_block = 32               # groups beyond 16 heads: selection blocks of 2, 4 or 8 compression strides
         S = pick([1, 2, 4, 7]) if sel_block >= 32 else pick([3, 8, 16])
         W = pick([1, 64, 100, 512])
         dtype = pick([torch.bfloat16, torch.float16])

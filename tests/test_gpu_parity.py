@@ -194,6 +194,23 @@ def test_cmp_select_block64_padded_pool():
     _cmp_case(torch.bfloat16, [1024, 333], 16, 1, 64, 64, 64, 16, 64, 4, seed=30)
 
 
+@pytest.mark.parametrize("dtype,lens,Hq,Hkv,Dk,Dv,l,d,lsel,S", [
+    (torch.bfloat16, [2100, 333, 70, 1], 64, 4, 128, 128, 64, 16, 64, 16),     # windows of 5 every 4, padding 2
+    (torch.float16, [1500, 65], 32, 2, 192, 128, 32, 8, 64, 8),                # 9 every 8, padding 2
+    (torch.bfloat16, [1024, 40], 16, 1, 64, 64, 32, 8, 32, 4),                 # 5 every 4, padding 2, stride 8
+    (torch.bfloat16, [1300, 257, 31], 16, 2, 128, 128, 32, 16, 16, 16),        # 2 every 1 (16-key selection blocks)
+    (torch.bfloat16, [900, 100], 8, 2, 64, 64, 32, 16, 16, 5),                 # 2 every 1, two tokens per tile
+    (torch.bfloat16, [700], 4, 1, 128, 128, 64, 16, 128, 3),                   # 9 every 8, padding 2, four tokens per tile
+    (torch.bfloat16, [1200, 90], 64, 2, 128, 128, 64, 16, 32, 6),              # a group of 32 heads, 3 every 2, padding 2
+    (torch.float32, [800, 130], 16, 1, 64, 64, 64, 16, 64, 4),
+])
+def test_cmp_select_other_pooling_geometries(dtype, lens, Hq, Hkv, Dk, Dv, l, d, lsel, S):
+    """Compression blocks beyond two strides pad the pooled row (pool_pad = block / stride - 2 columns on either
+    side, counted in the divisor); selection blocks of one stride pool windows of 2 columns every column.  Both run
+    on the two-kernel selection with the stream shifted by the padding."""
+    _cmp_case(dtype, lens, Hq, Hkv, Dk, Dv, l, d, lsel, S, seed=60, scale_in=0.5)
+
+
 def test_cmp_select_groups_of_32_48_64_heads():
     """GQA groups the reference's selected attention takes (HQ a multiple of 16 * H, nsa/selection_attn.py:800):
     sub-groups of 16 heads share the compressed keys; the block scores are the sum over all heads of the group."""
