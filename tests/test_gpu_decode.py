@@ -20,7 +20,8 @@ def _make(B, T, Hq, Hkv, Dk, Dv, seed, dtype, scale=0.5):
     return q, k, v, gl
 
 
-def _check(dtype, ctxs, Hq, Hkv, Dk, Dv, S, W, seed, which=None, splits=None, paged=False, sel_block=64):
+def _check(dtype, ctxs, Hq, Hkv, Dk, Dv, S, W, seed, which=None, splits=None, paged=False, sel_block=64, block=32,
+           stride=16):
     """One decode step through the C ABI against the CPU oracle on the same cache contents.
     splits: None = the schedule nsa_decode_step picks from the batch, 0 = the one-workgroup kernel
     (what the batch-64 benchmark times), > 0 = that many workgroups per pair.  paged: K/V in a shuffled
@@ -31,18 +32,19 @@ def _check(dtype, ctxs, Hq, Hkv, Dk, Dv, S, W, seed, which=None, splits=None, pa
     B, T = len(ctxs), max(ctxs)
     q, k, v, gl = _make(B, T, Hq, Hkv, Dk, Dv, seed, dtype)
     if paged:
-        cache = NSAPagedDecodeCache(B, sum((c + 63) // 64 for c in ctxs) + 2, T, Hkv, Dk, Dv, dtype=dtype, device=DEV)
+        cache = NSAPagedDecodeCache(B, sum((c + 63) // 64 for c in ctxs) + 2, T, Hkv, Dk, Dv, block=block, stride=stride,
+                                    dtype=dtype, device=DEV)
         random.Random(seed).shuffle(cache._free)
         for b, c in enumerate(ctxs):
             cache.fill(k[b, :c].to(DEV), v[b, :c].to(DEV), seq=b)
     else:
-        cache = NSADecodeCache(B, T, Hkv, Dk, Dv, dtype=dtype, device=DEV)
+        cache = NSADecodeCache(B, T, Hkv, Dk, Dv, block=block, stride=stride, dtype=dtype, device=DEV)
         cache.fill(k.to(DEV), v.to(DEV))
         cache.ctx_lens.copy_(torch.tensor(ctxs, dtype=torch.int32))
     out, idx = nsa_decode_step(q.to(DEV), cache, gl.to(DEV), sel_block, S, W, gate_activation="sigmoid",
                                return_indices=True, splits=splits)
     out, idx = out.cpu(), idx.cpu().long()
-    p = O.NSAParams(32, 16, sel_block, S, W)
+    p = O.NSAParams(block, stride, sel_block, S, W)
     gates = torch.sigmoid(gl.float()).to(dtype)
     worst, stats = 0.0, [0, 0, 0, 0]
     for b in (range(B) if which is None else which):
@@ -226,6 +228,23 @@ def test_decode_other_selection_block_sizes(dtype, Hq, Hkv, Dk, Dv, S, W, sel_bl
     adds the rows of such windows to the bins one by one."""
     _check(dtype, [2048, 1000, 513, 100, 65, 33, 1], Hq, Hkv, Dk, Dv, S, W, seed=150, splits=splits, paged=paged,
            sel_block=sel_block)
+
+
+@pytest.mark.parametrize("splits", [None, 0, 3])
+@pytest.mark.parametrize("dtype,Hq,Hkv,Dk,Dv,S,W,block,stride,sel_block,paged", [
+    (torch.bfloat16, 16, 1, 128, 128, 8, 128, 64, 16, 64, False),       # pooling windows of 5 every 4, padding 2
+    (torch.float16, 32, 2, 64, 64, 4, 100, 64, 16, 64, True),
+    (torch.bfloat16, 8, 2, 192, 128, 4, 64, 64, 16, 128, False),        # 9 every 8, padding 2
+    (torch.float32, 4, 1, 64, 64, 3, 32, 64, 32, 64, False),            # 3 every 2, stride 32
+])
+def test_decode_other_compression_geometries(dtype, Hq, Hkv, Dk, Dv, S, W, block, stride, sel_block, paged, splits):
+    """Compression blocks of 64 tokens (what the reference's own compression benchmark uses,
+    tests/benchmark_compression_kv_bwd.py:9) pad the pooled row by block / stride - 2 columns: both decode
+    schedules against the oracle."""
+    if splits == 0 and (sel_block // stride) < 4:
+        pytest.skip("the one-workgroup kernel holds pooling strides of 4 and more")
+    _check(dtype, [2048, 1000, 513, 100, 65, 33, 1], Hq, Hkv, Dk, Dv, S, W, seed=155, splits=splits, paged=paged,
+           sel_block=sel_block, block=block, stride=stride)
 
 
 def test_decode_selection_block_32_long_context():
