@@ -578,6 +578,15 @@ def test_module_fp16():
     _module_case(torch.float16, [1500], 64, 2, 128, 128, 16, 512, seed=23, scale_in=0.5)       # groups of 32 heads
 
 
+@pytest.mark.parametrize("l,d,lsel,S,mode", [(64, 16, 64, 16, "mean"), (64, 16, 64, 8, "conv"), (32, 8, 64, 8, "mean"),
+                                              (64, 32, 64, 6, "mean"), (32, 16, 16, 16, "mean")])
+def test_module_other_compression_geometries(l, d, lsel, S, mode):
+    """The whole forward with compression blocks of 64 tokens (the reference's compression benchmark,
+    tests/benchmark_compression_kv_bwd.py:9), a compression stride of 8 or 32, and selection blocks of one stride."""
+    _module_case(torch.bfloat16, [1300, 70, 1000, 33], 32, 2, 128, 128, S, 200, seed=24, scale_in=0.5, mode=mode, l=l,
+                 d=d, lsel=lsel)
+
+
 def test_module_varlen_ragged():
     _module_case(torch.bfloat16, [1100, 64, 1000, 33, 1536], 32, 2, 128, 128, 16, 512, seed=2, scale_in=0.5)
 
