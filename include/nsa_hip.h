@@ -332,8 +332,8 @@ int nsa_slc_swa_bwd(const void* q, const void* k, const void* v, const void* o_s
  * out [batch][hq][dv]; indices (optional) int32 [batch][hkv][top_n] receives the selected blocks.
  * nc_cap <= nsa_decode_max_compressed() (the kernel keeps a sequence's compressed scores in the registers of
  * one workgroup; longer caches, up to nsa_decode_split_max_compressed() rows, go through
- * nsa_decode_step_split), a pooling geometry with at most nc_cap / 4 + 4 <= 640 bins per sequence
- * (pool_stride >= 4) and a GQA group of at most 16 heads; anything else returns NSA_ERR_UNSUPPORTED and is served
+ * nsa_decode_step_split), a pooling geometry with at most nc_cap / 2 + 4 bins per sequence
+ * (pool_stride >= 2) and a GQA group of at most 16 heads; anything else returns NSA_ERR_UNSUPPORTED and is served
  * by nsa_decode_step_split. */
 int nsa_decode_max_compressed(void);
 int nsa_decode_split_max_compressed(void);

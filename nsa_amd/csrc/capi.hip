@@ -644,16 +644,16 @@ static int decode_common(const char* what, const void* q, const void* k_cache, c
     return finish(rc, what);
   }
   {
-    // the one-workgroup kernel holds the pooled bins of a sequence in nc_cap / 4 + 4 floats of LDS and ten
-    // per lane in its top-n: pooling strides below 4 (selection blocks narrower than 4 compression strides)
-    // make more bins than that
+    // the one-workgroup kernel holds the pooled bins of a sequence in LDS and in the registers of its top-n: up to
+    // nc_cap / 2 + 4 of them, i.e. pooling strides of 2 and more (selection blocks of two compression strides)
     const int span = nc_cap + 2 * pool_pad - pool_kernel;
     const int ns_cap = span < 0 ? 0 : (span + pool_stride - 1) / pool_stride + 1;
-    if (ns_cap > nc_cap / 4 + 4 || ns_cap > 640)
-      return fail(NSA_ERR_UNSUPPORTED, "%s: up to %d pooled bins per sequence (pooling stride >= 4) are built, this "
-                  "geometry can make %d", what, nc_cap / 4 + 4 < 640 ? nc_cap / 4 + 4 : 640, ns_cap);
+    if (ns_cap > nsa::decode_max_bins(nc_cap))
+      return fail(NSA_ERR_UNSUPPORTED, "%s: up to %d pooled bins per sequence (pooling stride >= 2) are built, this "
+                  "geometry can make %d; nsa_decode_step_split holds more", what, nsa::decode_max_bins(nc_cap), ns_cap);
   }
   const int rc = nsa::launch_decode(a, stream);
+  if (rc == -3) return fail(NSA_ERR_UNSUPPORTED, "%s: more pooled bins per sequence than the one-workgroup step holds", what);
   if (rc == -2) return fail(NSA_ERR_UNSUPPORTED, "%s: head dims not built (dk,dv in (64,64),(128,128),(192,128); fp32: no 192)", what);
   return finish(rc, what);
 }

@@ -28,7 +28,8 @@
 
 namespace nsa {
 
-template <typename T, int DK, int DV, bool PAGED>
+// WIDE: room for twice the pooled bins (pooling stride 2: selection blocks of two compression strides)
+template <typename T, int DK, int DV, bool PAGED, bool WIDE>
 __global__ void __launch_bounds__(kDecWaves * 64)
 decode_step_kernel(const DecodeArgs a) {
   constexpr int NW = kDecWaves, MAXC = kDecMaxChunks, PLD = 17;
@@ -37,7 +38,7 @@ decode_step_kernel(const DecodeArgs a) {
   float* pstat = part + NW * DV * PLD;                         // [NW][2][16]   (m, l) per wavefront
   float* pstat1 = pstat + NW * 2 * 16;                         // [NW][2][16]   score statistics of phase 1
   float* bins = pstat1 + NW * 2 * 16;                          // [Ns]
-  int* sel = reinterpret_cast<int*>(bins + ((a.nc_cap + 3) / 4 + 4));   // [top_n]
+  int* sel = reinterpret_cast<int*>(bins + decode_bins_cap(a.nc_cap, WIDE));   // [top_n]
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -216,6 +217,9 @@ decode_step_kernel(const DecodeArgs a) {
   // ---- phase 2a: importance bins from the registers (no memory traffic).  The head sum is a DPP
   // all-reduce over the 16 lanes of a row; lane n == 0 of every row then owns 8 consecutive columns.
   const bool fast_pool = a.pool_k == 5 && a.pool_s == 4 && a.pool_p == 0;
+  // windows of s + 1 columns every s, s = 1, 2, 4 or 8, any padding: see the runs below
+  const bool run_pool = a.pool_k == a.pool_s + 1 && (a.pool_s == 1 || a.pool_s == 2 || a.pool_s == 4 || a.pool_s == 8);
+  const int ls = a.pool_s == 1 ? 0 : a.pool_s == 2 ? 1 : a.pool_s == 4 ? 2 : 3;
 #pragma unroll
   for (int i = 0; i < MAXC; ++i) {
     const int cb = 32 * (wave + NW * i);
@@ -239,6 +243,29 @@ decode_step_kernel(const DecodeArgs a) {
           if (b0 >= 1 && b0 - 1 < Ns) atomicAdd(&bins[b0 - 1], v[0]);
           if (b0 < Ns) atomicAdd(&bins[b0], (v[0] + v[1]) + (v[2] + v[3]) + v[4]);
           if (b0 + 1 < Ns) atomicAdd(&bins[b0 + 1], (v[4] + v[5]) + (v[6] + v[7]));
+        } else if (run_pool) {
+          // bin j pools positions j * s .. j * s + s of the padded row (position = column + padding): the lane's 8
+          // consecutive columns are runs of equal bin, one atomic per run; a position that is a multiple of s is the
+          // first of its bin and also the last of the bin before
+          const int x0 = c0 + a.pool_p;
+          int cur = x0 >> ls;
+          float run = 0.f;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const int x = x0 + e;
+            if ((x & (a.pool_s - 1)) == 0) {
+              if (e == 0) {
+                if (cur >= 1 && cur - 1 < Ns) atomicAdd(&bins[cur - 1], v[0]);
+              } else {
+                if (cur < Ns) atomicAdd(&bins[cur], run + v[e]);
+                cur = x >> ls;
+              }
+              run = v[e];
+            } else {
+              run += v[e];
+            }
+          }
+          if (cur < Ns) atomicAdd(&bins[cur], run);
         } else {
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
@@ -257,7 +284,8 @@ decode_step_kernel(const DecodeArgs a) {
 
   // ---- phase 3 (wavefront 0 only): top-n blocks; each lane owns the bins b == lane (mod 64)
   if (wave == 0) {
-    constexpr int PER = (32 * kDecWaves * kDecMaxChunks / 4 + 63) / 64 + 1;
+    constexpr int PER = (32 * kDecWaves * kDecMaxChunks / (WIDE ? 2 : 4) + 63) / 64 + 1;
+    static_assert(64 * PER >= kDecBinsMax<WIDE>, "every bin needs a lane slot");
     __shared__ float cand_v[128];
     __shared__ int cand_i[128];
     float v[PER];
@@ -437,23 +465,28 @@ decode_append_paged_kernel(const T* __restrict__ k_new, const T* __restrict__ v_
 
 int set_smem(const void* fn, size_t bytes);
 
-template <typename T, int DK, int DV>
-static int launch_decode_t(const DecodeArgs& a, hipStream_t st) {
-  const size_t smem = ((size_t)kDecWaves * DV * 17 + kDecWaves * 64 + (a.nc_cap + 3) / 4 + 4) * sizeof(float) +
+template <typename T, int DK, int DV, bool PAGED, bool WIDE>
+static int launch_decode_v(const DecodeArgs& a, hipStream_t st) {
+  const size_t smem = ((size_t)kDecWaves * DV * 17 + kDecWaves * 64 + decode_bins_cap(a.nc_cap, WIDE)) * sizeof(float) +
                       (size_t)a.top_n * sizeof(int) + 64;
-  if (a.block_table != nullptr) {
-    auto fn = decode_step_kernel<T, DK, DV, true>;
-    const int rc = set_smem(reinterpret_cast<const void*>(fn), smem);
-    if (rc) return rc;
-    hipLaunchKernelGGL(fn, dim3(a.batch * a.hkv), dim3(kDecWaves * 64), smem, st, a);
-    return 0;
-  }
-  auto fn = decode_step_kernel<T, DK, DV, false>;
+  auto fn = decode_step_kernel<T, DK, DV, PAGED, WIDE>;
   const int rc = set_smem(reinterpret_cast<const void*>(fn), smem);
   if (rc) return rc;
   hipLaunchKernelGGL(fn, dim3(a.batch * a.hkv), dim3(kDecWaves * 64), smem, st, a);
   return 0;
 }
+
+template <typename T, int DK, int DV>
+static int launch_decode_t(const DecodeArgs& a, hipStream_t st) {
+  const int bins = decode_pooled_bins(a.nc_cap, a.pool_k, a.pool_s, a.pool_p);
+  if (bins > decode_bins_room(a.nc_cap, true)) return -3;
+  const bool wide = bins > decode_bins_room(a.nc_cap, false);
+  if (a.block_table != nullptr)
+    return wide ? launch_decode_v<T, DK, DV, true, true>(a, st) : launch_decode_v<T, DK, DV, true, false>(a, st);
+  return wide ? launch_decode_v<T, DK, DV, false, true>(a, st) : launch_decode_v<T, DK, DV, false, false>(a, st);
+}
+
+int decode_max_bins(int nc_cap) { return decode_bins_room(nc_cap, true); }
 
 int launch_decode(const DecodeArgs& a, hipStream_t st) {
   const int key = a.dk * 1000 + a.dv;

@@ -8,6 +8,23 @@ namespace nsa {
 constexpr int kDecWaves = 8;
 constexpr int kDecMaxChunks = 9;   // compressed 32-row chunks per wavefront kept in registers
 
+// Pooled bins of a sequence with nc compressed rows (windows of k every s, padding p, ceil mode).
+__host__ __device__ inline int decode_pooled_bins(int nc, int k, int s, int p) {
+  const int span = nc + 2 * p - k;
+  return span < 0 ? 0 : (span + s - 1) / s + 1;
+}
+// The one-workgroup step keeps the bins of its sequence in LDS (decode_bins_cap floats) and, for the top-n, in
+// the registers of one wavefront: a quarter of the compressed rows + 4 (pooling strides of 4 and more), or half of
+// them + 4 in the WIDE build (pooling stride 2).
+template <bool WIDE> constexpr int kDecBinsMax = 32 * kDecWaves * kDecMaxChunks / (WIDE ? 2 : 4) + 4;
+__host__ __device__ inline int decode_bins_cap(int nc_cap, bool wide) {
+  return wide ? (nc_cap + 1) / 2 + 4 : (nc_cap + 3) / 4 + 4;
+}
+__host__ __device__ inline int decode_bins_room(int nc_cap, bool wide) {
+  const int cap = decode_bins_cap(nc_cap, wide), most = wide ? kDecBinsMax<true> : kDecBinsMax<false>;
+  return cap < most ? cap : most;
+}
+
 template <typename T, int DK, int DV>
 struct DecState {              // online softmax state of one wavefront for one branch
   f32x4_t o[DV / 16];

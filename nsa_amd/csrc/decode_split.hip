@@ -178,6 +178,9 @@ decode_split_cmp_kernel(const DecodeArgs a, const SplitLayout L, float* __restri
   // row completes).
   const float Ml2 = M * kLog2e;
   const bool fast_pool = L.pool_k == 5 && L.pool_s == 4 && L.pool_p == 0;
+  // windows of s + 1 rows every s, s = 1, 2, 4 or 8, any padding: a lane's 8 rows are runs of equal bin
+  const bool run_pool = L.pool_k == L.pool_s + 1 && (L.pool_s == 1 || L.pool_s == 2 || L.pool_s == 4 || L.pool_s == 8);
+  const int ls = L.pool_s == 1 ? 0 : L.pool_s == 2 ? 1 : L.pool_s == 4 ? 2 : 3;
   const int jf = L.first_bin(c_lo);
 #pragma unroll
   for (int i = 0; i < MAXC; ++i) {
@@ -193,6 +196,31 @@ decode_split_cmp_kernel(const DecodeArgs a, const SplitLayout L, float* __restri
           atomicAdd(&binsL[(b0 - 1) * 16 + n], v[0]);
           atomicAdd(&binsL[b0 * 16 + n], (v[0] + v[1]) + (v[2] + v[3]) + v[4]);
           atomicAdd(&binsL[(b0 + 1) * 16 + n], (v[4] + v[5]) + (v[6] + v[7]));
+        }
+      } else if (run_pool) {
+        // bin j pools positions j * s .. j * s + s of the padded row (position = row + padding): one atomic per run
+        // of rows of equal bin; a position that is a multiple of s is the first of its bin and the last of the bin
+        // before.  Rows past c_hi carry 0; local bins stay within [0, L.nb).
+        if (c0 < c_hi) {
+          const int x0 = c0 + L.pool_p;
+          int cur = x0 >> ls;
+          float run = 0.f;
+          auto add = [&](int j, float val) {
+            const int lb = j - jf;
+            if (lb >= 0 && lb < L.nb) atomicAdd(&binsL[lb * 16 + n], val);
+          };
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const int x = x0 + e;
+            if ((x & (L.pool_s - 1)) == 0) {
+              if (e == 0) add(cur - 1, v[0]);
+              else { add(cur, run + v[e]); cur = x >> ls; }
+              run = v[e];
+            } else {
+              run += v[e];
+            }
+          }
+          add(cur, run);
         }
       } else {
 #pragma unroll

@@ -183,6 +183,7 @@ int launch_decode_append_paged(const void* k_new, const void* v_new, void* k_poo
                                const int32_t* pos, int batch, int hkv, int dk, int dv, int nc_cap, int block,
                                int stride, int dtype, hipStream_t st);
 int decode_max_nc();
+int decode_max_bins(int nc_cap);      // pooled bins per sequence that the one-workgroup step holds
 int decode_split_max_nc();
 // the same step spread over `splits` workgroups per (sequence, kv head), for small batches
 long decode_split_workspace_bytes(const DecodeArgs& a, int splits);

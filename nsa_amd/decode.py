@@ -268,11 +268,12 @@ def nsa_decode_step(q: torch.Tensor, cache, gates: Optional[torch.Tensor] = None
     long_cache = cache.nc_cap > lib.nsa_decode_max_compressed()
     group = hq // cache.hkv if hq % cache.hkv == 0 else 0
     sub_groups = group // 16 if group > 16 and group % 16 == 0 else 1    # 16-head sub-groups per kv head
-    # the one-workgroup kernel holds nc_cap / 4 + 4 pooled bins (640 at most): pooling strides below 4 (selection
-    # blocks of 32 keys at stride 16) make more and run on the split schedule, which holds 3136
+    # the one-workgroup kernel holds nc_cap / 2 + 4 pooled bins (pooling strides of 2 and more): selection blocks of
+    # one compression stride make more and run on the split schedule, which holds 3136
     span = cache.nc_cap + 2 * pool_p - pool_k
     ns_cap = 0 if span < 0 else (span + pool_s - 1) // pool_s + 1
-    many_bins = ns_cap > min(cache.nc_cap // 4 + 4, 640)
+    one_wg_bins = min((cache.nc_cap + 1) // 2 + 4, 1156)
+    many_bins = ns_cap > one_wg_bins
     if sub_groups > 1 or many_bins:
         # groups of 32, 48, 64 heads: the split schedule runs every 16 heads as a pair of their own
         long_cache = True
@@ -289,7 +290,7 @@ def nsa_decode_step(q: torch.Tensor, cache, gates: Optional[torch.Tensor] = None
     elif splits == 0 and many_bins:
         raise NotImplementedError("the one-workgroup decode step holds %d pooled bins per sequence, this geometry "
                                   "makes up to %d (pass splits=None or a positive split count)"
-                                  % (min(cache.nc_cap // 4 + 4, 640), ns_cap))
+                                  % (one_wg_bins, ns_cap))
     elif splits == 0 and long_cache:
         raise NotImplementedError(
             "the one-workgroup decode step keeps at most %d compressed rows per sequence; this cache holds up "

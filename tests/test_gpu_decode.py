@@ -202,19 +202,18 @@ def test_cache_append_matches_bulk_fill():
 
 def test_decode_one_workgroup_kernel_rejects_what_it_cannot_hold():
     """The register kernel refuses caches beyond its 2304 compressed rows and pooling geometries that make more
-    bins than its LDS row holds (a 32-token selection block at stride 16 = windows of 3 every 2)."""
+    bins than it holds (half the compressed rows: a 16-token selection block at stride 16 = windows of 2 every 1)."""
     from nsa_amd.decode import NSADecodeCache, nsa_decode_step
     cache = NSADecodeCache(1, 65536, 1, 64, 64, dtype=torch.bfloat16, device=DEV)
     q = torch.zeros(1, 4, 64, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(NotImplementedError):
         nsa_decode_step(q, cache, splits=0)
     small = NSADecodeCache(1, 4096, 1, 64, 64, dtype=torch.bfloat16, device=DEV)
-    with pytest.raises(NotImplementedError):
-        nsa_decode_step(q, small, selection_block=32, splits=0)
-    nsa_decode_step(q, small, selection_block=32)            # the split schedule takes it (oracle cases below)
+    nsa_decode_step(q, small, selection_block=32, splits=0)  # its wide build (oracle cases below)
+    nsa_decode_step(q, small, selection_block=32)            # the split schedule (oracle cases below)
 
 
-@pytest.mark.parametrize("splits", [None, 1, 5])
+@pytest.mark.parametrize("splits", [None, 0, 1, 5])
 @pytest.mark.parametrize("dtype,Hq,Hkv,Dk,Dv,S,W,sel_block,paged", [
     (torch.bfloat16, 16, 1, 128, 128, 8, 128, 32, False),
     (torch.float16, 32, 2, 64, 64, 16, 100, 32, True),
@@ -224,8 +223,11 @@ def test_decode_one_workgroup_kernel_rejects_what_it_cannot_hold():
 ])
 def test_decode_other_selection_block_sizes(dtype, Hq, Hkv, Dk, Dv, S, W, sel_block, paged, splits):
     """Selection blocks of 32 keys (the reference's own selection test, tests/test_parallel_nsa.py:169; pooling
-    windows of 3 every 2, twice the bins of the default), 96 and 128 keys on the split schedule, whose first launch
-    adds the rows of such windows to the bins one by one."""
+    windows of 3 every 2, twice the bins of the default: the wide build of the one-workgroup kernel), 96 and 128
+    keys, on both schedules (windows of s + 1 rows every s, s = 1, 2, 4, 8, go to the bins as runs of rows of equal
+    bin, others row by row)."""
+    if splits == 0 and Hq // Hkv > 16:
+        pytest.skip("the one-workgroup kernel takes groups of at most 16 heads")
     _check(dtype, [2048, 1000, 513, 100, 65, 33, 1], Hq, Hkv, Dk, Dv, S, W, seed=150, splits=splits, paged=paged,
            sel_block=sel_block)
 
@@ -241,15 +243,14 @@ def test_decode_other_compression_geometries(dtype, Hq, Hkv, Dk, Dv, S, W, block
     """Compression blocks of 64 tokens (what the reference's own compression benchmark uses,
     tests/benchmark_compression_kv_bwd.py:9) pad the pooled row by block / stride - 2 columns: both decode
     schedules against the oracle."""
-    if splits == 0 and (sel_block // stride) < 4:
-        pytest.skip("the one-workgroup kernel holds pooling strides of 4 and more")
     _check(dtype, [2048, 1000, 513, 100, 65, 33, 1], Hq, Hkv, Dk, Dv, S, W, seed=155, splits=splits, paged=paged,
            sel_block=sel_block, block=block, stride=stride)
 
 
 def test_decode_selection_block_32_long_context():
     _check(torch.bfloat16, [50000, 20001], 16, 1, 128, 128, 16, 512, seed=151, sel_block=32)
-    _check(torch.bfloat16, [3000] * 70, 16, 1, 64, 64, 4, 64, seed=152, sel_block=32, which=[0, 69])   # 70 pairs: splits = 1
+    _check(torch.bfloat16, [3000] * 70, 16, 1, 64, 64, 4, 64, seed=152, sel_block=32, which=[0, 69])   # 70 pairs: one workgroup each
+    _check(torch.bfloat16, [3000] * 70, 16, 1, 64, 64, 4, 64, seed=153, sel_block=32, which=[1, 68], splits=1)
 
 
 def test_cache_append_beyond_capacity_raises():

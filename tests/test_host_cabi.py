@@ -76,8 +76,8 @@ def test_argument_errors_do_not_launch(lib):
     rc = lib.nsa_decode_step(p, p, p, p, p, p, None, p, None, 1, 48, 2, 64, 64, 64, 64, 32, 16, 64, 5, 4, 0, 4, 16, 0.1,
                              0, 0, None)                                                             # group of 24
     assert rc == -2 and b"group size" in lib.nsa_last_error_string()
-    rc = lib.nsa_decode_step(p, p, p, p, p, p, None, p, None, 1, 4, 1, 64, 64, 4096, 256, 32, 16, 32, 3, 2, 0, 4, 16,
-                             0.1, 0, 0, None)                                                        # 128 bins > 68
+    rc = lib.nsa_decode_step(p, p, p, p, p, p, None, p, None, 1, 4, 1, 64, 64, 4096, 256, 32, 16, 32, 2, 1, 0, 4, 16,
+                             0.1, 0, 0, None)                                                        # 255 bins > 132
     assert rc == -2 and b"pooled bins" in lib.nsa_last_error_string()
     rc = lib.nsa_decode_step(p, p, p, p, p, p, None, p, None, 1, 4, 1, 64, 64, 65536, 4096, 32, 16, 64, 5, 4, 0, 4, 16,
                              0.1, 0, 0, None)                                                        # one workgroup: 2304 rows
