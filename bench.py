@@ -117,6 +117,31 @@ def cpu_baseline(q, k, v, gl, top_n, window, budget_s=20.0):
                        % (done_rows, spent, t_comp))
 
 
+def cpu_baseline_cfg1():
+    """Benchmark configuration 1 as it is defined: batch 1, 1024 tokens, Hq 4 / Hkv 1, head dim 64, fp32, q / k / v ~
+    N(0, 1) and gate logits ~ N(0, 1) from seed 0, compression 32 / 16 (mean), selection blocks of 64, top 4, window
+    128; the whole sequence through the CPU oracle on all host cores, one warm-up run and the median of three."""
+    import torch
+    from oracle import nsa_oracle as O
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    T, hq, hkv, d = 1024, 4, 1, 64
+    g = torch.Generator().manual_seed(0)
+    q, k, v = (torch.randn(T, h, d, generator=g) for h in (hq, hkv, hkv))
+    gates = torch.sigmoid(torch.randn(T, hq, 3, generator=g))
+    p = O.NSAParams(BLOCK, STRIDE, SEL_BLOCK, 4, 128)
+    times = []
+    for i in range(4):
+        t0 = time.perf_counter()
+        out = O.nsa_forward_single(q, k, v, gates, p)
+        times.append(time.perf_counter() - t0)
+    assert torch.isfinite(out).all()
+    med = sorted(times[1:])[1]
+    return dict(value=T / med, unit="tokens/s", cores=cores, kind="port", seconds_per_forward=med,
+                sample="CPU oracle, whole sequence of benchmark configuration 1 (1024 tokens, Hq4/Hkv1, D64, fp32), "
+                       "1 warm-up + 3 runs, median")
+
+
 def decode_bench(steps, warmup):
     """benchmark config 5: batch 64, one query token per sequence, 32768 cached tokens each (+ the
     compressed caches), Hq64/Hkv4, D128, top-16 blocks of 64, window 512, bf16."""
@@ -451,6 +476,7 @@ def main():
         res["decode_small_batch"] = decode_small
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(q, k, v, gl, top_n, window, args.cpu_budget)
+        res["cpu_baseline_cfg1"] = cpu_baseline_cfg1()
     print(json.dumps(res))
 
 

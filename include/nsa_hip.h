@@ -391,8 +391,10 @@ int nsa_decode_step_split(const void* q, const void* k_cache, const void* v_cach
  * = 16 MiB, held on every GPU the library runs on until the process ends) instead of a caller workspace.  The
  * call allocates and frees nothing; the first call on a device looks the array's address up.  Arguments as
  * nsa_decode_step_split without workspace / workspace_bytes.  Returns NSA_ERR_RESOURCE when
- * nsa_decode_split_workspace_bytes(batch, hkv, dv, nc_cap, splits) exceeds the array (about 70 (sequence, kv head)
- * pairs at 32k context, D 128, 8 splits).  All calls on one GPU share the array and it keeps the last call's
+ * nsa_decode_split_pooled_workspace_bytes(batch, hkv * sub_groups, dv, nc_cap, splits, pool_kernel, pool_stride,
+ * pool_pad) -- sub_groups = 16-head sub-groups of the GQA group, 1 up to 16 heads; the same figure as
+ * nsa_decode_split_workspace_bytes(batch, hkv, dv, nc_cap, splits) for the default pooling of 5 rows every 4 --
+ * exceeds the array (about 70 (sequence, kv head) pairs at 32k context, D 128, 8 splits).  All calls on one GPU share the array and it keeps the last call's
  * contents: calls that overlap in time on one GPU race, also across streams.  No counterpart in the reference,
  * which has no decode path and leaves every allocation to PyTorch. */
 int64_t nsa_decode_split_static_bytes(void);

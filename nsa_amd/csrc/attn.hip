@@ -94,6 +94,11 @@ stream_attn_kernel(const StreamParams a) {
   int g_hi_max[NG], g_hi_min[NG], g_lo_min[NG], g_lo_max[NG];   // wave uniform bounds over the group
   float li[NG];                  // compressed branch: this lane's share of the importance denominator ...
   float mi[NG];                  // ... and its reference (the attention softmax keeps its own in grp[j].m)
+  // float16 only: the largest 8-key sum of probabilities this lane has packed.  The sums are fp32, the packed
+  // probabilities are not: a float16 probability overflows at 65504 and loses its mantissa below 6e-5, ranges that
+  // the fp32 sums pass through unnoticed.
+  constexpr bool kNarrowP = std::is_same<T, f16_t>::value;
+  float pmax[NG];
 #pragma unroll
   for (int j = 0; j < NG; ++j) {
     const int gi = wave * NG + j;
@@ -102,6 +107,7 @@ stream_attn_kernel(const StreamParams a) {
     group_reset(grp[j]);
     li[j] = 0.f;
     mi[j] = kNegInf;
+    pmax[j] = 0.f;
     hi[j] = last_visible(rm[j].tok);
     lo[j] = CMP ? 0 : rm[j].tok - W + 1;
     const int tf = st.t0 + ((gi * 16) >> lgp);
@@ -295,7 +301,9 @@ stream_attn_kernel(const StreamParams a) {
                   for (int i = 0; i < 8; ++i)
                     if (key0 + (i ^ swp) > hi[j]) p[i] = 0.f;
                 }
-                grp[j].l += sum8(p);
+                const float p8 = sum8(p);
+                grp[j].l += p8;
+                if constexpr (kNarrowP) pmax[j] = fmaxf(pmax[j], p8);
                 pb[j] = pack8<T>(p);
               } else {
                 pb[j] = zero8<T>();
@@ -375,6 +383,13 @@ stream_attn_kernel(const StreamParams a) {
     for (int j = 0; j < NG; ++j) {
       const bool sees = rm[j].valid && hi[j] >= 0 && c_begin < c_end;
       bad |= !(lit[j] < 1e30f) || !(lt[j] < 1e30f) || (sees && !(lt[j] > 1e-30f));
+      if constexpr (kNarrowP) {
+        // every packed probability is at most its 8-key sum: below 3e4 none overflowed.  The largest 8-key sum of
+        // the row at or above 2^-7 puts the row's largest probability at or above 2^-10, a normal float16 with its
+        // whole mantissa; what lies 2^-14 and more below it is subnormal, as under a running maximum.
+        const float pm = colgroup_max(pmax[j]);
+        bad |= !(pm < 3e4f) || (sees && !(pm >= 0.0078125f));
+      }
     }
     if (__syncthreads_or(bad)) {               // rare: the whole workgroup repeats the pass in the exact form
 #pragma unroll

@@ -90,14 +90,17 @@ decode_step_kernel(const DecodeArgs a) {
   // merging of per-wavefront partial states (used as soon as a branch is complete), gate, accumulate
   // thread -> head r = tid % 16, channels 4*(tid/16) .. +3
   const int r = tid & 15, d0 = (tid >> 4) * 4;
-  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  // The output is (compressed + window) + selected whatever the order the phases ran in, so that an output row does
+  // not depend on the batch slot of its sequence: the first two share an accumulator (their sum does not depend on
+  // which came first), the selected branch keeps its own until the end.
+  float acc[2][4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
   const T* gp = reinterpret_cast<const T*>(a.gates);
   auto gate = [&](int which) -> float {
     if (gp == nullptr || r >= G) return 1.f;
     const float x = (float)gp[((long)b * a.hq + h * G + r) * 3 + which];
     return a.gate_act == 1 ? 1.0f / (1.0f + __expf(-x)) : x;
   };
-  auto merge = [&](const DecState<T, DK, DV>& st, float gate_w) {
+  auto merge = [&](const DecState<T, DK, DV>& st, float gate_w, float (&dst)[4]) {
     __syncthreads();
 #pragma unroll
     for (int tt = 0; tt < DV / 16; ++tt)
@@ -122,7 +125,7 @@ decode_step_kernel(const DecodeArgs a) {
     const float inv = den > 0.f ? gate_w / den : 0.f;
     if (d0 < DV) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) acc[i] += num[i] * inv;
+      for (int i = 0; i < 4; ++i) dst[i] += num[i] * inv;
     }
   };
 
@@ -144,12 +147,12 @@ decode_step_kernel(const DecodeArgs a) {
       chunk_attend<T, DK, DV>(swa, fb, qf, cb2, w_lo, t, c_attn, g);
       cb = cb3;
     }
-    merge(swa, gate(1));
+    merge(swa, gate(1), acc[1]);
   };
   // Where the window phase runs: 0 first, 1 between the compressed and the selected phase, 2 last.  The phases of
   // a step ramp up and drain one after the other, and with one workgroup per CU all CUs would do so at the same
   // moments; three orders spread the ramps of one third of the chip over the streaming of the rest (95.7 -> 91.4 us
-  // at batch 64 x 32768 tokens; two orders 93.3 us).  The branches are summed in the order they run.
+  // at batch 64 x 32768 tokens; two orders 93.3 us).  The branch results are kept apart and summed in one order.
   const int window_pos = (int)(blockIdx.x % 3);
   if (a.window > 0 && window_pos == 0) window_phase();
 
@@ -339,7 +342,7 @@ decode_step_kernel(const DecodeArgs a) {
     }
   }
   cmp.m = cmaxv >= 0 ? M : kNegInf;   // every wavefront used the common reference M
-  merge(cmp, gate(2));               // its barriers also publish the selected blocks
+  merge(cmp, gate(2), acc[1]);               // its barriers also publish the selected blocks
   if (a.window > 0 && window_pos == 1) window_phase();
 
   // ---- phase 4: selected blocks, 32-key chunks dealt round-robin, next chunk in flight
@@ -379,12 +382,12 @@ decode_step_kernel(const DecodeArgs a) {
       chunk_attend<T, DK, DV>(slc, fb, qf, cbb, k0b, k1b, c_attn, g);
     }
   }
-  merge(slc, gate(0));
+  merge(slc, gate(0), acc[0]);
   if (a.window > 0 && window_pos == 2) window_phase();
   if (r < G && d0 < DV) {
     T* op = reinterpret_cast<T*>(a.out) + ((long)b * a.hq + h * G + r) * DV + d0;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) op[i] = (T)acc[i];
+    for (int i = 0; i < 4; ++i) op[i] = (T)(acc[1][i] + acc[0][i]);
   }
 }
 

@@ -277,6 +277,9 @@ def nsa_decode_step(q: torch.Tensor, cache, gates: Optional[torch.Tensor] = None
     if sub_groups > 1 or many_bins:
         # groups of 32, 48, 64 heads: the split schedule runs every 16 heads as a pair of their own
         long_cache = True
+    if static_scratch and splits == 0:
+        raise ValueError("static_scratch runs the split schedule: pass splits=None or a positive split count "
+                         "(splits=0 asks for the one-workgroup step, which has no scratch buffer)")
     if splits is None:
         pairs = B * cache.hkv * sub_groups
         # measured at 32k context: 8 splits halve the step up to 32 pairs and still win at 64 (46 vs 64 us);
@@ -296,7 +299,7 @@ def nsa_decode_step(q: torch.Tensor, cache, gates: Optional[torch.Tensor] = None
             "the one-workgroup decode step keeps at most %d compressed rows per sequence; this cache holds up "
             "to %d (pass splits=None or a positive split count)" % (lib.nsa_decode_max_compressed(), cache.nc_cap))
     if static_scratch:
-        splits = splits or 8
+        splits = splits or 8          # None that resolved to the one-workgroup step: the split schedule all the same
         k_c, v_c = (cache.k_pool, cache.v_pool_t) if paged else (cache.k, cache.vt)
         rc = lib.nsa_decode_step_split_static(
             _ptr(q), _ptr(k_c), _ptr(v_c), _ptr(cache.block_table) if paged else None,

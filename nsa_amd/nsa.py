@@ -12,6 +12,29 @@ from .autograd import GateLinearFn, NSACoreFn, needs_grad
 from .compression_kv import KVCompressor, conv_compressed_len
 
 
+# What a `cu_seqlens` tensor was found to hold the last time its lengths were read on the host: keyed by the tensor
+# object (weak reference, so an address reused by a new tensor cannot hit) and its in-place version counter.
+_LENGTHS_SEEN: dict = {}
+
+
+def _sequence_lengths_once(cu_seqlens: torch.Tensor):
+    """(all lengths equal, longest length) of a cu_seqlens tensor.  The device-to-host read happens once per tensor
+    object and version; later calls with the same, unmodified tensor -- a serving loop, a benchmark -- cost nothing
+    and keep the forward free of host synchronisation."""
+    import weakref
+    key = id(cu_seqlens)
+    hit = _LENGTHS_SEEN.get(key)
+    if hit is not None and hit[0]() is cu_seqlens and hit[1] == cu_seqlens._version:
+        return hit[2]
+    lens = (cu_seqlens[1:] - cu_seqlens[:-1]).tolist()
+    res = (min(lens) == max(lens), int(max(lens)))
+    if len(_LENGTHS_SEEN) >= 16:
+        for k in [k for k, v in _LENGTHS_SEEN.items() if v[0]() is None] or list(_LENGTHS_SEEN)[:8]:
+            _LENGTHS_SEEN.pop(k, None)
+    _LENGTHS_SEEN[key] = (weakref.ref(cu_seqlens), cu_seqlens._version, res)
+    return res
+
+
 class NSAAttention(nn.Module):
     """Native Sparse Attention: compress -> compressed attention + block selection ->
     selected + sliding-window attention -> gated sum, all on hand-written gfx950 kernels.  Without
@@ -84,8 +107,10 @@ class NSAAttention(nn.Module):
         """q [total,Hq,Dk], k [total,Hkv,Dk], v [total,Hkv,Dv], cu_seqlens int32 [B+1] -> [total,Hq,Dv].
 
         max_seqlen: longest sequence (int); 0/None means "all sequences have total/B tokens" as in
-        the reference, which is checked against cu_seqlens (one small device read) and falls back to
-        the ragged path when the lengths differ.  softmax_scale follows the reference: None is
+        the reference, which is checked against cu_seqlens and falls back to the ragged path when the
+        lengths differ.  That check reads cu_seqlens on the host ONCE per tensor object (and in-place
+        version); pass max_seqlen, or call with the same cu_seqlens tensor again, and the forward has no
+        device-to-host synchronisation at all.  softmax_scale follows the reference: None is
         1/sqrt(Dk), anything else is used as a number (so True, which the reference's module test passes
         positionally, means 1.0).  gates [total,Hq,3] (selected, sliding, compressed) overrides the gating
         Linear (pre-activation values).  stage_times: a list that receives (name, start_event,
@@ -101,9 +126,9 @@ class NSAAttention(nn.Module):
         if uniform and batch > 1:
             # "uniform" is a promise about cu_seqlens; the kernels read the real offsets, so a ragged batch
             # taken for a uniform one would size the compressed rows wrongly
-            lens = (cu[1:] - cu[:-1]).tolist()
-            if min(lens) != max(lens) or lens[0] * batch != total:
-                uniform, max_seqlen = False, max(lens)
+            equal, longest = _sequence_lengths_once(cu_seqlens if cu_seqlens_k is None else cu_seqlens_k)
+            if not equal or longest * batch != total:
+                uniform, max_seqlen = False, longest
         seq_len = total // batch if uniform else int(max_seqlen)
         params = [] if gates is not None else [self.gating.weight, self.gating.bias]
         if self.compressor.mode != "mean":

@@ -219,12 +219,15 @@ def compressed_attention(q: torch.Tensor, ck: torch.Tensor, cv: torch.Tensor, bl
 # ----------------------------------------------------------------------------- selected / sliding
 
 def _masked_attention(qm, km, vm, allowed, scale):
-    """qm [t,Hkv,G,Dk], km [Tk,Hkv,Dk], vm [Tk,Hkv,Dv], allowed bool [t,Hkv,Tk] -> [t,Hkv,G,Dv]."""
+    """qm [t,Hkv,G,Dk], km [Tk,Hkv,Dk], vm [Tk,Hkv,Dv], allowed [t,Hkv,Tk] -> [t,Hkv,G,Dv].  `allowed` is a boolean
+    mask, or an integer count of how many times the key enters the softmax (0 = masked)."""
     s = torch.einsum("thgd,khd->thgk", qm, km) * scale
-    s = s.masked_fill(~allowed[:, :, None, :], float("-inf"))
+    s = s.masked_fill((allowed == 0)[:, :, None, :], float("-inf"))
     m = s.amax(-1, keepdim=True)
     m = torch.where(torch.isinf(m), torch.zeros_like(m), m)
     e = torch.exp(s - m)
+    if allowed.dtype != torch.bool:
+        e = e * allowed[:, :, None, :].to(e.dtype)
     z = e.sum(-1, keepdim=True)
     p = torch.where(z > 0, e / z.clamp_min(1e-300), torch.zeros_like(e))
     return torch.einsum("thgk,khv->thgv", p, vm)
@@ -237,6 +240,8 @@ def selected_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     """One sequence.  q [T,Hq,Dk], k [T,Hkv,Dk], v [T,Hkv,Dv], block_indices [T,Hkv,S] (block
     numbers local to the sequence).  Entry i of row t is used iff i < count, idx >= 0 and
     idx*block_size <= t; it contributes keys [idx*bs, min(idx*bs+bs-1, t)].  No usable entry -> 0.
+    A block id that occurs twice among a row's used entries enters the softmax twice, as in the reference's gather
+    (tests/test_parallel_nsa.py:133-146: k and v are gathered per entry, so a repeated block's keys are repeated).
     """
     T, Hq, Dk = q.shape
     _, Hkv, Dv = v.shape
@@ -257,12 +262,12 @@ def selected_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
         idx = block_indices[ids].to(torch.int64)                           # [n,Hkv,S]
         use = (torch.arange(S)[None, None, :] < counts[ids][:, :, None]) & (idx >= 0) \
             & (idx * block_size <= ids[:, None, None])
-        blk = torch.zeros(n, Hkv, nblk + 1, dtype=torch.bool)
+        blk = torch.zeros(n, Hkv, nblk + 1, dtype=torch.int64)             # times each block is used
         tgt = torch.where(use, idx, torch.full_like(idx, nblk)).clamp(max=nblk)
-        blk.scatter_(2, tgt, torch.ones_like(tgt, dtype=torch.bool))
+        blk.scatter_add_(2, tgt, torch.ones_like(tgt))
         blk = blk[..., :nblk]
         allowed = blk.repeat_interleave(block_size, dim=2)[..., :T]        # [n,Hkv,T]
-        allowed = allowed & (torch.arange(T)[None, None, :] <= ids[:, None, None])
+        allowed = allowed * (torch.arange(T)[None, None, :] <= ids[:, None, None])
         qm = q[ids].to(math_dtype).reshape(n, Hkv, G, Dk)
         out[pos] = _masked_attention(qm, km, vm, allowed, scale).reshape(n, Hq, Dv)
     return out
@@ -316,12 +321,10 @@ def selected_sliding_loop(q, k, v, block_indices, block_counts, block_size, wind
             cnt = S if block_counts is None else (
                 block_counts if isinstance(block_counts, int) else int(block_counts[t, h]))
             toks = []
-            seen = set()
             for i in range(min(cnt, S)):
                 b = int(block_indices[t, h, i])
-                if b < 0 or b * block_size > t or b in seen:
+                if b < 0 or b * block_size > t:
                     continue
-                seen.add(b)
                 toks.extend(range(b * block_size, min(b * block_size + block_size - 1, t) + 1))
             for g in range(G):
                 hq = h * G + g
@@ -463,7 +466,7 @@ def nsa_decode_step(q_last, k_cache, v_cache, gates_last, p: NSAParams, math_dty
     o_swa = torch.zeros(Hkv, G, Dv, dtype=math_dtype)
     for h in range(Hkv):
         toks = []
-        for b in sorted(set(int(x) for x in use_idx[h] if x >= 0 and int(x) * p.sel_block <= t)):
+        for b in (int(x) for x in use_idx[h] if x >= 0 and int(x) * p.sel_block <= t):    # a repeated id counts twice
             toks.extend(range(b * p.sel_block, min(b * p.sel_block + p.sel_block - 1, t) + 1))
         if toks:
             tk = torch.tensor(toks)

@@ -582,6 +582,34 @@ def test_parallel_nsa_backward_in_the_shape_of_the_reference_test(dtype):
         _check(name, a.grad, r.grad, dtype)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_parallel_nsa_backward_with_repeated_block_ids(dtype):
+    """A block listed twice by a row enters that row's softmax twice (tests/test_parallel_nsa.py:133-146): the
+    backward sees two (token, block) pairs with the same keys, and the gradients are those of the doubled weight."""
+    import nsa_amd
+    B, T, H, HQ, D, S, bs, W = 1, 256, 2, 16, 64, 4, 64, 32
+    q = randn(B, T, HQ, D, seed=310, dtype=dtype)
+    k = randn(B, T, H, D, seed=311, dtype=dtype)
+    v = randn(B, T, H, D, seed=312, dtype=dtype)
+    g_slc, g_swa = randn(B, T, HQ, seed=313, dtype=dtype), randn(B, T, HQ, seed=314, dtype=dtype)
+    d_o = randn(B, T, HQ, D, seed=315, dtype=dtype)
+    idx = _random_indices(T, H, S, bs, 316)[None].clone()
+    idx[..., 1] = idx[..., 0]
+    idx[:, T // 2:, 1, 3] = idx[:, T // 2:, 1, 0]
+    leaves = [_leaf(t) for t in (q, k, v, g_slc, g_swa)]
+    o = nsa_amd.selection_attention(*leaves, idx.to(DEV), None, bs, W)
+    o.backward(d_o.to(DEV))
+    scale = D ** -0.5
+    refs = [t.double().clone().requires_grad_(True) for t in (q, k, v, g_slc, g_swa)]
+    o_slc = O.selected_attention(refs[0][0], refs[1][0], refs[2][0], idx[0], None, bs, scale, math_dtype=torch.float64)
+    o_swa = O.sliding_attention(refs[0][0], refs[1][0], refs[2][0], W, scale, math_dtype=torch.float64)
+    ref = O.gated_combine(refs[3][0], o_slc, refs[4][0], o_swa)[None]
+    ref.backward(d_o.double())
+    _check("out", o.detach(), ref.detach(), dtype)
+    for name, a, r in zip(("dq", "dk", "dv", "dg_slc", "dg_swa"), leaves, refs):
+        _check(name, a.grad, r.grad, dtype)
+
+
 def test_compress_kv_backward():
     """compress_kv (functional, learned weights) and KVCompressorVarlen: gradients of k, v and the weights."""
     from nsa_amd.compression_kv import KVCompressorVarlen

@@ -64,6 +64,23 @@ def _check(dtype, ctxs, Hq, Hkv, Dk, Dv, S, W, seed, which=None, splits=None, pa
     assert stats[1] >= 0.99 * stats[0]
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_decode_one_workgroup_step_does_not_depend_on_the_batch_slot(dtype):
+    """The one-workgroup kernel runs its window phase at three different points of the step, by workgroup number;
+    the output is (compressed + window) + selected whatever that order, so the same sequence gives the same bits
+    in every batch slot."""
+    from nsa_amd.decode import NSADecodeCache, nsa_decode_step
+    B, T, Hq, Hkv, D, S, W = 7, 1500, 32, 2, 128, 8, 200
+    q, k, v, gl = _make(1, T, Hq, Hkv, D, D, 130, dtype)
+    q, k, v, gl = (x.expand(B, *x.shape[1:]).contiguous() for x in (q, k, v, gl))
+    cache = NSADecodeCache(B, T, Hkv, D, D, dtype=dtype, device=DEV)
+    cache.fill(k.to(DEV), v.to(DEV))
+    out, idx = nsa_decode_step(q.to(DEV), cache, gl.to(DEV), 64, S, W, gate_activation="sigmoid", return_indices=True,
+                               splits=0)
+    for b in range(1, B):         # 14 workgroups: every slot parity of (sequence, kv head) modulo 3 occurs
+        assert torch.equal(out[b], out[0]) and torch.equal(idx[b], idx[0])
+
+
 SCHEDULES = [None, 0]      # chosen from the batch (split for small batches) / one workgroup per pair
 
 

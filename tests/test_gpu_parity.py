@@ -122,7 +122,8 @@ def test_transpose_layout():
 
 
 # ------------------------------------------------------------------------------ compressed attention + selection
-def _cmp_case(dtype, lens, Hq, Hkv, Dk, Dv, l, d, lsel, S, seed, scale_in=1.0, late_key_scale=None, min_exact=0.99):
+def _cmp_case(dtype, lens, Hq, Hkv, Dk, Dv, l, d, lsel, S, seed, scale_in=1.0, late_key_scale=None, min_exact=0.99,
+              key_scale_range=None, softmax_scale=None):
     ops = _ops()
     p = O.NSAParams(l, d, lsel, S, 0)
     T = sum(lens)
@@ -130,13 +131,16 @@ def _cmp_case(dtype, lens, Hq, Hkv, Dk, Dv, l, d, lsel, S, seed, scale_in=1.0, l
     if late_key_scale is not None:          # keys of the later half of the packed tokens blown up
         k = k.clone()
         k[T // 2:] *= late_key_scale
+    if key_scale_range is not None:         # (first token, end token, factor)
+        k = k.clone()
+        k[key_scale_range[0]:key_scale_range[1]] *= key_scale_range[2]
     cu = _cu(lens)
     cu_cmp = ops.compressed_offsets(cu, l, d, extra=1)
     ncs = [O.compressed_len_conv(t, l, d) for t in lens]
     ck = ops.compress(k.to(DEV), cu, cu_cmp, sum(ncs), l, d)
     cv = ops.compress(v.to(DEV), cu, cu_cmp, sum(ncs), l, d)
     cvt = ops.transpose(cv, cu_cmp, len(lens))
-    scale = 1.0 / math.sqrt(Dk)
+    scale = 1.0 / math.sqrt(Dk) if softmax_scale is None else softmax_scale
     o, idx, pooled = ops.cmp_attn_select(q.to(DEV), ck, cvt, cu, cu_cmp, len(lens), Hkv, Dv, ck.stride(0),
                                          ck.stride(1), l, d, p.pool_kernel, p.pool_stride, p.pool_pad, S,
                                          max(ncs), scale, want_pooled=True)
@@ -220,7 +224,7 @@ def test_cmp_select_groups_of_32_48_64_heads():
     _cmp_case(torch.bfloat16, [2048], 64, 2, 192, 128, 32, 16, 64, 16, seed=46, scale_in=0.5)         # G=32, Dqk 192
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
 def test_cmp_select_scores_beyond_the_fixed_reference(dtype):
     """Inputs on which the kernel's common pass (one fixed softmax reference per row) must give way to its exact
     pass: raw scores spread over hundreds of units, so exponentials against an early reference overflow; and keys
@@ -231,6 +235,26 @@ def test_cmp_select_scores_beyond_the_fixed_reference(dtype):
     _cmp_case(dtype, [1024], 16, 1, 128, 128, 32, 16, 64, 16, seed=48, scale_in=1.0, late_key_scale=200.0, min_exact=0.0)
     _cmp_case(dtype, [2048], 64, 4, 192 if dtype == torch.bfloat16 else 128, 128, 32, 16, 64, 16, seed=49, scale_in=3.0,
               min_exact=0.0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_cmp_select_scores_between_the_float16_and_float32_ranges(dtype):
+    """Probabilities against the fixed reference that an fp32 sum holds easily and a float16 operand does not.  With
+    a softmax scale of 1 the attention logits are the raw scores, so the importance sum (fp32, overflows only 69 nats
+    above the reference) raises no alarm.  (a) Later keys 6.5 times larger: visible logits 15-40 nats above the largest
+    score of the first 32 compressed rows, probabilities of 1e7..1e17 -- infinite as float16.  (b) Keys of tokens
+    288..543 (compressed rows 17..32) 6 times larger: tokens below 288 see none of them, yet their reference is the
+    maximum over rows 0..31, so their visible probabilities are ~1e-9 -- zero as float16.  Both must come out as
+    under a running maximum (nsa/torch_attention.py:126-148)."""
+    a = _cmp_case(dtype, [1024, 200], 16, 1, 64, 64, 32, 16, 64, 4, seed=51, scale_in=1.0, softmax_scale=1.0,
+                  key_scale_range=(512, 1024, 6.5), min_exact=0.0)
+    b = _cmp_case(dtype, [1024], 32, 2, 64, 64, 32, 16, 64, 4, seed=52, scale_in=1.0, softmax_scale=1.0,
+                  key_scale_range=(288, 544, 6.0), min_exact=0.0)
+    # head dim 32: sqrt(32) = 5.7 raw units per nat, so a visible logit 11.1-12.2 nats above the reference overflows
+    # float16 (> 65504) while the raw-score exponential stays below the fp32 alarm
+    c = _cmp_case(dtype, [1024], 16, 1, 32, 32, 32, 16, 64, 4, seed=53, scale_in=1.0, key_scale_range=(512, 1024, 14.5),
+                  min_exact=0.0)
+    assert all(math.isfinite(w["o"]) for w in (a, b, c))
 
 
 def test_cmp_select_odd_groups():
@@ -481,6 +505,35 @@ def test_parallel_nsa_packed_cu_seqlens_and_tensor_counts(dtype, bs, W, H):
         slc, swa = O.selected_sliding_loop(q[0, s0:e0], k[0, s0:e0], v[0, s0:e0], idx[0, s0:e0], counts[0, s0:e0], bs, W)
         ref = g_slc[0, s0:e0, :, None].float() * slc + g_swa[0, s0:e0, :, None].float() * swa
         assert within(out[0, s0:e0], ref, dtype, large_values=True), max_abs(out[0, s0:e0], ref)
+
+
+@pytest.mark.parametrize("dtype,W", [(torch.bfloat16, 64), (torch.float16, 0), (torch.float32, 64), (torch.float32, 0)])
+def test_parallel_nsa_repeated_block_ids(dtype, W):
+    """block_indices that list a block twice (every row) or three times: the reference's naive loop gathers keys
+    and values per entry, so the block's keys enter the softmax once per occurrence
+    (tests/test_parallel_nsa.py:133-146).  16-bit inputs take the block-major schedule (one partial result per
+    (token, entry) pair), fp32 the token-major kernel."""
+    import nsa_amd
+    B, T, HQ, H, D, S, bs = 2, 320, 16, 2, 64, 6, 32
+    q = randn(B, T, HQ, D, seed=120, scale=0.7, dtype=dtype)
+    k = randn(B, T, H, D, seed=121, scale=0.7, dtype=dtype)
+    v = randn(B, T, H, D, seed=122, dtype=dtype)
+    g_slc = randn(B, T, HQ, seed=123, dtype=dtype)
+    g_swa = randn(B, T, HQ, seed=124, dtype=dtype)
+    idx = torch.stack([_random_indices(T, H, S, bs, 125 + b, poison=False) for b in range(B)])
+    idx[..., 1] = idx[..., 0]
+    idx[:, T // 2:, 0, 4] = idx[:, T // 2:, 0, 0]
+    out = nsa_amd.parallel_nsa(q.to(DEV), k.to(DEV), v.to(DEV), g_slc.to(DEV), g_swa.to(DEV), idx.to(DEV), None, bs,
+                               W).cpu()
+    once = idx.clone()
+    once[..., 1] = -1
+    differs = 0.0
+    for b in range(B):
+        slc, swa = O.selected_sliding_loop(q[b], k[b], v[b], idx[b], None, bs, W)
+        ref = g_slc[b, :, :, None].float() * slc + g_swa[b, :, :, None].float() * swa
+        assert within(out[b], ref, dtype, large_values=True), max_abs(out[b], ref)
+        differs = max(differs, max_abs(slc, O.selected_attention(q[b], k[b], v[b], once[b], None, bs)))
+    assert differs > 0.05          # counting the repeated block once would have been visible
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])

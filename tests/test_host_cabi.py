@@ -324,3 +324,24 @@ def test_split_decode_argument_errors_do_not_launch(lib):
     assert call(ws=None) == -1
     assert call(ws_bytes=16) == -1 and b"workspace" in lib.nsa_last_error_string()
     assert call(top_n=65) == -2
+
+
+def test_sequence_lengths_are_read_on_the_host_once_per_cu_seqlens_tensor(monkeypatch):
+    """NSAAttention.forward with max_seqlen 0 and a batch checks that the batch really is uniform.  The check reads
+    cu_seqlens once per tensor object and version; the second forward with the same tensor reads nothing."""
+    from nsa_amd import nsa as nsa_mod
+    cu = torch.tensor([0, 40, 80, 120], dtype=torch.int32)
+    reads = []
+    real = torch.Tensor.tolist
+    monkeypatch.setattr(torch.Tensor, "tolist", lambda self: (reads.append(1), real(self))[1])
+    assert nsa_mod._sequence_lengths_once(cu) == (True, 40)
+    assert nsa_mod._sequence_lengths_once(cu) == (True, 40)
+    assert len(reads) == 1
+    cu[2] = 90                                        # in-place change: version counter moves, lengths are re-read
+    assert nsa_mod._sequence_lengths_once(cu) == (False, 50)
+    assert len(reads) == 2
+    other = torch.tensor([0, 40, 80, 120], dtype=torch.int32)
+    assert nsa_mod._sequence_lengths_once(other) == (True, 40) and len(reads) == 3
+    for _ in range(40):                               # the table stays small
+        nsa_mod._sequence_lengths_once(torch.tensor([0, 3, 7]))
+    assert len(nsa_mod._LENGTHS_SEEN) <= 16

@@ -214,6 +214,57 @@ def test_token_loop_is_itself_sdpa_on_a_dense_case():
     torch.testing.assert_close(swa, ref, rtol=1e-9, atol=1e-10)
 
 
+def _gather_softmax(q, k, v, idx, bs, scale):
+    """Brute force in the shape of the reference's naive loop (tests/test_parallel_nsa.py:118-146): every entry of a
+    row's index list is expanded to its bs token positions, keys and values are GATHERED at those positions (so a
+    block listed twice is gathered twice), positions < 0 or > t are masked, one softmax over the S*bs gathered keys."""
+    T, Hq, D = q.shape
+    Hkv = k.shape[1]
+    G = Hq // Hkv
+    out = torch.zeros(T, Hq, v.shape[-1], dtype=D64)
+    pos = (idx[..., None] * bs + torch.arange(bs)).reshape(T, Hkv, -1)          # [T,Hkv,S*bs]
+    for t in range(T):
+        for h in range(Hq):
+            pt = pos[t, h // G]
+            kk, vv = k[pt.clamp(0, T - 1), h // G].double(), v[pt.clamp(0, T - 1), h // G].double()
+            sc = (kk @ q[t, h].double() * scale).masked_fill((pt < 0) | (pt > t), float("-inf"))
+            if torch.isinf(sc).all():
+                continue
+            out[t, h] = torch.softmax(sc, 0) @ vv
+    return out
+
+
+def test_repeated_block_ids_enter_the_softmax_once_per_occurrence():
+    T, Hq, Hkv, D, S, bs = 96, 4, 2, 16, 4, 16
+    q, k, v = _rand(T, Hq, D, seed=60), _rand(T, Hkv, D, seed=61), _rand(T, Hkv, D, seed=62)
+    g = torch.Generator().manual_seed(63)
+    idx = torch.randint(0, T // bs, (T, Hkv, S), generator=g)
+    idx[:, :, 1] = idx[:, :, 0]                       # every row lists its first block twice ...
+    idx[T // 2:, 0, 3] = idx[T // 2:, 0, 0]           # ... and half of the rows of head 0 three times
+    idx[5, :, 2] = -1
+    scale = 1.0 / math.sqrt(D)
+    ref = _gather_softmax(q, k, v, idx, bs, scale)
+    got = O.selected_attention(q, k, v, idx, None, bs, scale, D64, row_chunk=40)
+    torch.testing.assert_close(got, ref, rtol=1e-9, atol=1e-10)
+    loop, _ = O.selected_sliding_loop(q, k, v, idx, None, bs, 0)
+    torch.testing.assert_close(loop, ref, rtol=1e-9, atol=1e-10)
+    # and it differs from listing the block once (so the check above can fail)
+    once = idx.clone()
+    once[:, :, 1] = -1
+    once[T // 2:, 0, 3] = -1
+    assert (O.selected_attention(q, k, v, once, None, bs, scale, D64) - ref).abs().max() > 1e-3
+    # closed form: EVERY usable block listed twice is the same softmax as listing each once
+    both = torch.arange(T // bs).repeat(2).expand(T, Hkv, -1).contiguous()
+    torch.testing.assert_close(O.selected_attention(q, k, v, both, None, bs, scale, D64), _sdpa_causal(q, k, v),
+                               rtol=1e-9, atol=1e-10)
+    # decode step: a repeated pick in force_idx counts twice as well (last row of the prefill with the same list)
+    p = O.NSAParams(8, 4, bs, S, 0)
+    gates = torch.ones(Hq, 3, dtype=D64)
+    _, parts = O.nsa_decode_step(q[-1].double(), k.double(), v.double(), gates, p, D64, return_parts=True,
+                                 force_idx=idx[-1])
+    torch.testing.assert_close(parts["o_slc"], ref[-1], rtol=1e-9, atol=1e-10)
+
+
 # ---------------------------------------------------------------- combine / full forward
 def test_gated_combine_closed_form():
     a, b, c = _rand(5, 3, 4, seed=23), _rand(5, 3, 4, seed=24), _rand(5, 3, 4, seed=25)

@@ -41,11 +41,18 @@ def _case(lib, dtype, ctxs, Hq, Hkv, D, S, W, splits, seed):
     ref, ref_idx = torch.empty(B, Hq, D, dtype=dtype, device=DEV), torch.empty(B, Hkv, S, dtype=torch.int32, device=DEV)
     out, idx = torch.full_like(ref, float("nan")), torch.full_like(ref_idx, -7)
     assert _call(lib, False, q, cache, gl, ref, ref_idx, S, W, splits, ws) == 0
+    # one call beforehand: the first call on a device looks the array's address up and sets kernel attributes
+    warm, warm_idx = torch.empty_like(ref), torch.empty_like(ref_idx)
+    assert _call(lib, True, q, cache, gl, warm, warm_idx, S, W, splits) == 0, lib.nsa_last_error_string()
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
+    # free device memory as the driver counts it: an allocation inside the library (which PyTorch's own counters
+    # would not see) lowers it.  Nothing else allocates in between: no tensor is created, the stream exists.
+    free_before = torch.cuda.mem_get_info()[0]
+    torch_before = torch.cuda.memory_allocated()
     assert _call(lib, True, q, cache, gl, out, idx, S, W, splits) == 0, lib.nsa_last_error_string()
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] == free_before
+    assert torch.cuda.memory_allocated() == torch_before
     assert torch.equal(idx, ref_idx)
     assert torch.equal(out, ref) and torch.isfinite(out.float()).all()
     return cache, q, gl
@@ -68,6 +75,8 @@ def test_static_scratch_step_equals_workspace_step_twice_then_smaller():
     assert r.data_ptr() == out.data_ptr() and ri.data_ptr() == idx.data_ptr()
     ref, ref_idx = nsa_decode_step(q, cache, gl, 64, 4, 128, gate_activation="sigmoid", return_indices=True, splits=3)
     assert torch.equal(out, ref) and torch.equal(idx, ref_idx)
+    with pytest.raises(ValueError):          # splits=0 names the one-workgroup step, which has no scratch buffer
+        nsa_decode_step(q, cache, gl, 64, 4, 128, gate_activation="sigmoid", splits=0, static_scratch=True)
 
 
 def test_static_scratch_step_refuses_what_does_not_fit():
