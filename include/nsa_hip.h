@@ -146,6 +146,28 @@ int nsa_block_select_fwd(const void* q, const void* ck, const float* lse, void* 
                          int pool_pad, int top_n, int max_ns, int pooled_stride, int keep_pooled, int idx64,
                          int dtype, nsa_stream_t stream);
 
+/* Compressed attention AND block selection as the reference's one call computes them (_attention.forward,
+ * nsa/triton_attention.py:419-476: one q.ck product whose scores feed the attention, the softmax over all rows, the
+ * pooling and the top-k).  Arguments as nsa_cmp_attn_select_fwd, plus lse_attn as in nsa_cmp_attn_fwd and the gating
+ * Linear (gate_weight / gate_bias / gates, all NULL = none) as in nsa_cmp_attn_gate_fwd.
+ *   max_nc: the most compressed rows of any sequence of the batch (max_ns is the pooled-bin count that goes with it).
+ *   single_pass: -1 = run as ONE kernel when the shape qualifies (nsa_cmp_select_single_pass: GQA groups of 9..16
+ *   heads, 16-bit inputs, head dims (64,64), (128,128), (192,128), pooling windows of 5 rows every 4 without padding,
+ *   max_nc <= 2048, top_n <= 64), else as nsa_cmp_attn(_gate)_fwd followed by nsa_block_select_fwd; 0 = always the
+ *   latter; 1 = the one kernel or NSA_ERR_UNSUPPORTED.  The one kernel multiplies q with the compressed keys once,
+ *   keeps no score buffer and no pooled hand-over buffer: the window sums stay in registers per head until the
+ *   head's normaliser is known.  lse and pooled may be NULL then (pooled given and keep_pooled != 0: the averages are
+ *   written); on the other schedule lse is required and pooled selects the two-kernel selection as above. */
+int nsa_cmp_select_single_pass(int hq, int hkv, int dk, int dv, int pool_kernel, int pool_stride, int pool_pad,
+                               int top_n, int max_nc, int dtype);
+int nsa_cmp_select_fwd(const void* q, const void* ck, const void* cvt, void* o, void* indices, float* pooled, float* lse,
+                       float* lse_attn, const void* gate_weight, const void* gate_bias, void* gates,
+                       const int32_t* cu_seqlens, const int32_t* cu_cmp, int batch, int total, int hq, int hkv, int dk,
+                       int dv, int64_t ck_row_stride, int64_t ck_head_stride, int cvt_cols, int block, int stride,
+                       int pool_kernel, int pool_stride, int pool_pad, int top_n, int max_nc, int max_ns,
+                       int pooled_stride, int keep_pooled, float scale, int causal, int idx64, int dtype,
+                       int single_pass, nsa_stream_t stream);
+
 /* Model integration: the glue between a layer's fused q/k/v(/gate) projection GEMM and the kernels
  * above.  The reference leaves this to its caller (nsa/nsa.py:83-135 receives q, k, v already split and
  * rotated) and computes the gate logits with a separate Linear (nsa/nsa.py:61,117); here the gating

@@ -10,7 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT_DIR = os.path.join(HERE, "lib")
 LIB = os.path.join(OUT_DIR, "libnsa_hip.so")
-SOURCES = ["prep.hip", "attn.hip", "select.hip", "slc_block.hip", "bwd.hip", "compress_bwd.hip", "combine.hip", "qkv_rope.hip", "decode.hip", "decode_split.hip", "capi.hip"]
+SOURCES = ["prep.hip", "attn.hip", "cmp_select.hip", "select.hip", "slc_block.hip", "bwd.hip", "compress_bwd.hip", "combine.hip", "qkv_rope.hip", "decode.hip", "decode_split.hip", "capi.hip"]
 FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
          "-packed-fp32-ops", "-fno-honor-nans", "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option"]
 

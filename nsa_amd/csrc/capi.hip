@@ -140,7 +140,10 @@ static int cmp_common(const char* what, int stages, const void* q, const void* c
                       int64_t ck_head_stride, int cvt_cols, int block, int stride, int pool_kernel, int pool_stride,
                       int pool_pad, int top_n, int max_ns, int pooled_stride, int keep_pooled, float scale, int causal,
                       int idx64, int dtype, nsa_stream_t stream, const void* gate_w = nullptr,
-                      const void* gate_b = nullptr, void* gates = nullptr) {
+                      const void* gate_b = nullptr, void* gates = nullptr, int single_pass_max_nc = -1,
+                      int single_pass = 0) {
+  // single_pass_max_nc >= 0 (stages 3 only): the most compressed rows of any sequence, with which the call may run
+  // as ONE kernel (single_pass -1 = when the shape qualifies, 1 = or fail, 0 = never)
   const bool attn = stages & 1, select = stages & 2;
   if ((gate_w != nullptr) != (gates != nullptr) || (gate_b && !gate_w))
     return fail(NSA_ERR_INVALID, "%s: the gating Linear needs its weight and the gates buffer", what);
@@ -157,7 +160,7 @@ static int cmp_common(const char* what, int stages, const void* q, const void* c
   if (!aligned16(q) || !aligned16(ck) || (attn && (!aligned16(cvt) || !aligned16(o))))
     return fail(NSA_ERR_INVALID, "%s: pointers must be 16-byte aligned", what);
   if (select) {
-    if (!indices || !lse) return fail(NSA_ERR_INVALID, "%s: the selection needs indices and the lse buffer", what);
+    if (!indices || (!lse && single_pass != 1)) return fail(NSA_ERR_INVALID, "%s: the selection needs indices and the lse buffer", what);
     if (pool_kernel <= 0 || pool_stride <= 0 || pool_pad < 0 || pool_pad >= pool_kernel || top_n <= 0 || max_ns < 0)
       return fail(NSA_ERR_INVALID, "%s: bad pooling / top-n parameters", what);
     if (pooled && pooled_stride < max_ns) return fail(NSA_ERR_INVALID, "%s: pooled_stride < max_ns", what);
@@ -170,6 +173,13 @@ static int cmp_common(const char* what, int stages, const void* q, const void* c
   a.keep_pooled = keep_pooled != 0;
   a.gate_w = gate_w; a.gate_b = gate_b; a.gates = gates;
   int rc = 0;
+  if (attn && select && single_pass != 0 && single_pass_max_nc >= 0) {
+    if (nsa::cmp_select_single_pass_ok(a, single_pass_max_nc)) return finish(nsa::launch_cmp_select(a, stream), what);
+    if (single_pass == 1)
+      return fail(NSA_ERR_UNSUPPORTED, "%s: the single-pass kernel takes GQA groups of 9..16 heads, 16-bit inputs, head dims "
+                  "(64,64) (128,128) (192,128), pooling windows of 5 rows every 4 without padding, at most 2048 compressed "
+                  "rows per sequence and top_n <= 64", what);
+  }
   if (attn) rc = nsa::launch_cmp_attn(a, stream);
   if (rc == 0 && select) rc = nsa::launch_select(a, stream);
   if (rc == -6)
@@ -189,6 +199,33 @@ int nsa_cmp_attn_select_fwd(const void* q, const void* ck, const void* cvt, void
                     batch, total, hq, hkv, dk, dv, ck_row_stride, ck_head_stride, cvt_cols, block, stride,
                     pool_kernel, pool_stride, pool_pad, top_n, max_ns, pooled_stride, keep_pooled, scale, causal, idx64,
                     dtype, stream);
+}
+
+int nsa_cmp_select_single_pass(int hq, int hkv, int dk, int dv, int pool_kernel, int pool_stride, int pool_pad,
+                               int top_n, int max_nc, int dtype) {
+  if (hq <= 0 || hkv <= 0 || hq % hkv != 0) return 0;
+  nsa::CmpArgs a{};
+  a.hq = hq; a.hkv = hkv; a.dk = dk; a.dv = dv; a.pool_k = pool_kernel; a.pool_s = pool_stride; a.pool_p = pool_pad;
+  a.top_n = top_n; a.dtype = dtype; a.kv_rep = hq / hkv > 16 ? 2 : 1;
+  a.max_ns = max_nc >= 5 ? (max_nc - 2) / 4 + 1 : 0;
+  static int dummy;
+  a.indices = &dummy; a.cvt = &dummy; a.o = &dummy;         // the shape test only asks whether they are given
+  return nsa::cmp_select_single_pass_ok(a, max_nc) ? 1 : 0;
+}
+
+int nsa_cmp_select_fwd(const void* q, const void* ck, const void* cvt, void* o, void* indices, float* pooled, float* lse,
+                       float* lse_attn, const void* gate_weight, const void* gate_bias, void* gates,
+                       const int32_t* cu_seqlens, const int32_t* cu_cmp, int batch, int total, int hq, int hkv, int dk,
+                       int dv, int64_t ck_row_stride, int64_t ck_head_stride, int cvt_cols, int block, int stride,
+                       int pool_kernel, int pool_stride, int pool_pad, int top_n, int max_nc, int max_ns,
+                       int pooled_stride, int keep_pooled, float scale, int causal, int idx64, int dtype,
+                       int single_pass, nsa_stream_t stream) {
+  if (!indices) return fail(NSA_ERR_INVALID, "cmp_select: null pointer");
+  if (max_nc < 0 || single_pass < -1 || single_pass > 1) return fail(NSA_ERR_INVALID, "cmp_select: bad max_nc / single_pass");
+  return cmp_common("cmp_select", 3, q, ck, cvt, o, indices, pooled, lse, lse_attn, cu_seqlens, cu_cmp, batch, total, hq,
+                    hkv, dk, dv, ck_row_stride, ck_head_stride, cvt_cols, block, stride, pool_kernel, pool_stride,
+                    pool_pad, top_n, max_ns, pooled_stride, keep_pooled, scale, causal, idx64, dtype, stream, gate_weight,
+                    gate_bias, gates, max_nc, single_pass);
 }
 
 int nsa_cmp_attn_fwd(const void* q, const void* ck, const void* cvt, void* o, float* lse, float* lse_attn,

@@ -125,7 +125,11 @@ decode_step_kernel(const DecodeArgs a) {
     const float inv = den > 0.f ? gate_w / den : 0.f;
     if (d0 < DV) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) dst[i] += num[i] * inv;
+      for (int i = 0; i < 4; ++i) {
+        float pr = num[i] * inv;
+        asm volatile("" : "+v"(pr));       // keeps the product out of a fused multiply-add: only a + b == b + a
+        dst[i] += pr;
+      }
     }
   };
 

@@ -159,6 +159,10 @@ int launch_gate_bwd(const void* q, const void* w, const void* d_gl, void* dq, fl
                     int dim, int dtype, hipStream_t st);
 int launch_cmp_attn(const CmpArgs& a, hipStream_t st);
 int launch_select(const CmpArgs& a, hipStream_t st);
+// compressed attention + importance + top-n in one pass over the compressed keys (cmp_select.hip): whether the
+// shape qualifies (max_nc = most compressed rows of any sequence), and the launch
+bool cmp_select_single_pass_ok(const CmpArgs& a, int max_nc);
+int launch_cmp_select(const CmpArgs& a, hipStream_t st);
 int launch_swa(const SwaArgs& a, hipStream_t st);
 int launch_slc_combine(const SlcArgs& a, hipStream_t st);
 long slc_workspace_bytes(const SlcArgs& a);

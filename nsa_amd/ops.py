@@ -182,6 +182,53 @@ def cmp_attn_select(q, ck, cvt, cu_seqlens, cu_cmp, batch, hkv, dv, ck_row_strid
     return o, idx, (pooled[:, :, 0] if want_pooled else None)
 
 
+def cmp_select_single_pass(q, hkv, dv, pool_kernel, pool_stride, pool_pad, top_n, max_nc) -> bool:
+    """Whether cmp_select runs this shape as one kernel (one pass over the compressed keys)."""
+    return bool(_lib.load().nsa_cmp_select_single_pass(q.shape[1], hkv, q.shape[2], dv, pool_kernel, pool_stride,
+                                                       pool_pad, top_n, max_nc, _dtype_code(q)))
+
+
+def cmp_select(q, ck, cvt, cu_seqlens, cu_cmp, batch, hkv, dv, ck_row_stride, ck_head_stride, block, stride,
+               pool_kernel, pool_stride, pool_pad, top_n, max_nc, scale, causal=True, idx64=False,
+               want_pooled=False, want_lse_attn=False, gate_weight=None, gate_bias=None, single_pass=None):
+    """Compressed attention and block selection in one library call, as the reference's `_attention.forward`
+    (nsa/triton_attention.py:419-476).  Returns a dict: o [total,Hq,dv], indices [total,hkv,top_n], and on request
+    pooled [total,hkv,Ns], lse_attn [total,Hq] (what the backward reads), gates [total,Hq,3] (the gating Linear on q
+    when gate_weight [3,Dk] is given).
+    single_pass: None = one kernel when the shape qualifies (cmp_select_single_pass), otherwise compressed
+    attention, window sums and top-n as three launches; False = always the latter; True = the one kernel or an error."""
+    _need_cuda(q, ck, cvt, cu_seqlens, cu_cmp)
+    q = _dense(q)
+    total, hq, dk = q.shape
+    lib = _lib.load()
+    max_ns = pool_bins(max_nc, pool_kernel, pool_stride, pool_pad)
+    fused = single_pass is not False and cmp_select_single_pass(q, hkv, dv, pool_kernel, pool_stride, pool_pad,
+                                                                max(top_n, 1), max_nc)
+    o = torch.empty(total, hq, dv, dtype=q.dtype, device=q.device)
+    idx = torch.empty(total, hkv, top_n, dtype=torch.int64 if idx64 else torch.int32, device=q.device)
+    lse_attn = torch.empty(total, hq, dtype=torch.float32, device=q.device) if want_lse_attn else None
+    # the one kernel needs neither the importance log-sum-exp nor a hand-over buffer for the window sums
+    lse = None if fused else torch.empty(total, hq, dtype=torch.float32, device=q.device)
+    pooled = None
+    if want_pooled or not fused:
+        pooled = torch.empty(total, hkv, head_subgroups(hq, hkv), max(max_ns, 1), dtype=torch.float32, device=q.device)
+    w = b = gates = None
+    if gate_weight is not None:
+        _need_cuda(gate_weight)
+        w = _dense(gate_weight.to(q.dtype))
+        b = None if gate_bias is None else gate_bias.to(q.dtype).contiguous()
+        gates = torch.empty(total, hq, 3, dtype=q.dtype, device=q.device)
+    mode = -1 if single_pass is None else int(bool(single_pass))
+    rc = lib.nsa_cmp_select_fwd(
+        _ptr(q), _ptr(ck), _ptr(cvt), _ptr(o), _ptr(idx), _ptr(pooled), _ptr(lse), _ptr(lse_attn), _ptr(w), _ptr(b),
+        _ptr(gates), _ptr(cu_seqlens), _ptr(cu_cmp), batch, total, hq, hkv, dk, dv, ck_row_stride, ck_head_stride,
+        cvt.shape[-1], block, stride, pool_kernel, pool_stride, pool_pad, max(top_n, 1), max_nc, max_ns, max(max_ns, 1),
+        int(bool(want_pooled)), float(scale), int(bool(causal)), int(idx64), _dtype_code(q), mode, _stream())
+    _lib.check(rc, "nsa_cmp_select_fwd")
+    return dict(o=o, indices=idx, pooled=pooled[:, :, 0] if want_pooled else None, lse_attn=lse_attn, gates=gates,
+                single_pass=fused)
+
+
 def cmp_attn(q, ck, cvt, cu_seqlens, cu_cmp, batch, hkv, dv, ck_row_stride, ck_head_stride, block, stride, scale,
              causal=True, want_lse_attn=False, gate_weight=None, gate_bias=None):
     """Compressed attention only.  Returns (o [total,Hq,dv], lse float32 [total,Hq]) where lse is the
