@@ -160,7 +160,7 @@ static int cmp_common(const char* what, int stages, const void* q, const void* c
   if (!aligned16(q) || !aligned16(ck) || (attn && (!aligned16(cvt) || !aligned16(o))))
     return fail(NSA_ERR_INVALID, "%s: pointers must be 16-byte aligned", what);
   if (select) {
-    if (!indices || (!lse && single_pass != 1)) return fail(NSA_ERR_INVALID, "%s: the selection needs indices and the lse buffer", what);
+    if (!indices) return fail(NSA_ERR_INVALID, "%s: the selection needs indices and the lse buffer", what);
     if (pool_kernel <= 0 || pool_stride <= 0 || pool_pad < 0 || pool_pad >= pool_kernel || top_n <= 0 || max_ns < 0)
       return fail(NSA_ERR_INVALID, "%s: bad pooling / top-n parameters", what);
     if (pooled && pooled_stride < max_ns) return fail(NSA_ERR_INVALID, "%s: pooled_stride < max_ns", what);
@@ -180,6 +180,7 @@ static int cmp_common(const char* what, int stages, const void* q, const void* c
                   "(64,64) (128,128) (192,128), pooling windows of 5 rows every 4 without padding, at most 2048 compressed "
                   "rows per sequence and top_n <= 64", what);
   }
+  if (select && !lse) return fail(NSA_ERR_INVALID, "%s: the selection needs indices and the lse buffer", what);
   if (attn) rc = nsa::launch_cmp_attn(a, stream);
   if (rc == 0 && select) rc = nsa::launch_select(a, stream);
   if (rc == -6)
