@@ -434,10 +434,12 @@ def main():
     # stages are one kernel each, so the single dominant kernel is the longest of cmp_attn / swa.
     # With the fused schedule the selected branch is "slc_blocks" (bucket + per-block partials) and the
     # window branch "swa_combine" (window attention + merge of the partials + gated sum).
-    stage_flops = {"cmp_attn": fl["cmp"], "swa": fl["swa"], "slc_combine": fl["slc"],
+    # "cmp_select" is the one-pass kernel that does the work of cmp_attn + block_select (attention over the visible
+    # compressed rows, importance over all of them, top-n); it is credited with the attention flops only.
+    stage_flops = {"cmp_attn": fl["cmp"], "cmp_select": fl["cmp"], "swa": fl["swa"], "slc_combine": fl["slc"],
                    "swa_combine": fl["swa"], "slc_blocks": fl["slc"]}
     stage_tflops = {n: stage_flops[n] / (stage_ms[n] * 1e-3) / 1e12 for n in stage_flops if n in stage_ms}
-    dom = max(("cmp_attn", "swa", "swa_combine"), key=lambda n: stage_ms.get(n, 0.0))
+    dom = max(("cmp_attn", "cmp_select", "swa", "swa_combine"), key=lambda n: stage_ms.get(n, 0.0))
     dom_tflops = stage_tflops[dom]
     # HBM bytes per launch of that kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE (profiles/), only
     # recorded for the default workload
@@ -445,10 +447,24 @@ def main():
     # The compressed-attention kernel also multiplies q with the compressed keys a token cannot see: the
     # importance softmax is normalised over all of them.  `executed` adds that uncredited part of QK^T.
     executed = None
-    if dom == "cmp_attn":
-        qk_all = sum(2.0 * hq * dqk * x * max((x - BLOCK) // STRIDE + 1, 0) for x in lens)
-        qk_seen = fl["cmp"] * dqk / (dqk + dv)
+    qk_all = sum(2.0 * hq * dqk * x * max((x - BLOCK) // STRIDE + 1, 0) for x in lens)
+    qk_seen = fl["cmp"] * dqk / (dqk + dv)
+    if dom in ("cmp_attn", "cmp_select"):
         executed = (fl["cmp"] + max(qk_all - qk_seen, 0.0)) / (stage_ms[dom] * 1e-3) / 1e12
+    # flops the whole step executes on the matrix unit: the credited ones plus the non-causal part of QK^T, once
+    # in the one-pass kernel, twice (compressed attention, then the importance kernel) on the three-launch schedule
+    qk_passes = 1 if "cmp_select" in stage_ms else 2
+    executed_step = f_eff + max(qk_all - qk_seen, 0.0) + (qk_passes - 1) * qk_all
+    # The two HBM-bound stages of the step against 8 TB/s: bytes per launch from the committed counter summary
+    # (same source-digest rule as roofline.traffic), divided by the stage time measured here
+    roofline_hbm = {}
+    for stage_name, kernel in (("slc_blocks", "slc_blocks"), ("swa_combine", "swa_combine")):
+        if stage_name in stage_ms:
+            nbytes, src = measured_traffic(args.workload, kernel)
+            gbs = None if nbytes is None else nbytes / (stage_ms[stage_name] * 1e-3) / 1e9
+            roofline_hbm[stage_name] = {"bound": "hbm", "traffic": nbytes, "traffic_source": src, "achieved": gbs,
+                                        "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                        "frac": None if gbs is None else gbs / PEAK_HBM_GBS}
 
     res = {
         "metric": "nsa_prefill_fwd_tokens_per_s", "value": total / (ms * 1e-3), "unit": "tokens/s",
@@ -465,6 +481,9 @@ def main():
                      "unit": "TFLOP/s", "frac": dom_tflops / PEAK_BF16_TFLOPS, "traffic": traffic,
                      "traffic_source": traffic_source, "executed": executed},
         "stage_effective_tflops": stage_tflops,
+        "roofline_hbm": roofline_hbm,
+        "executed_tflops_whole_step": executed_step / (ms * 1e-3) / 1e12,
+        "executed_mfma_peak_frac_whole_step": executed_step / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
     }
     res["compress"] = compress_bench(kd, vd, cu)
     if not args.no_backward:

@@ -157,10 +157,25 @@ int nsa_block_select_fwd(const void* q, const void* ck, const float* lse, void* 
  *   latter; 1 = the one kernel or NSA_ERR_UNSUPPORTED.  The one kernel multiplies q with the compressed keys once,
  *   keeps no score buffer and no pooled hand-over buffer: the window sums stay in registers per head until the
  *   head's normaliser is known.  lse and pooled may be NULL then (pooled given and keep_pooled != 0: the averages are
- *   written); on the other schedule lse is required and pooled selects the two-kernel selection as above. */
+ *   written); on the other schedule lse is required and pooled selects the two-kernel selection as above.
+ *   frag / frag_chunks: the fragment-major copy of nsa_cmp_pack_fwd, which the one kernel reads instead of ck and cvt
+ *   (cvt may be NULL when single_pass == 1); NULL = the one kernel is not available. */
 int nsa_cmp_select_single_pass(int hq, int hkv, int dk, int dv, int pool_kernel, int pool_stride, int pool_pad,
                                int top_n, int max_nc, int dtype);
-int nsa_cmp_select_fwd(const void* q, const void* ck, const void* cvt, void* o, void* indices, float* pooled, float* lse,
+/* What the one kernel streams instead of ck / cvt: both in "fragment order", every 64-row chunk of a sequence stored
+ * exactly as the matrix instructions consume it (1 KB per operand fragment), so that the kernel's global -> LDS copy
+ * is a straight run of bytes done by the load unit and its LDS reads are free of bank conflicts.
+ *   ck rows as above; cv [rows][hkv][dv] ROW-major (cv_row_stride / cv_head_stride in elements), not its transpose;
+ *   frag: hkv * frag_chunks * 64 * (dk + dv) elements, frag_chunks >= nsa_cmp_pack_chunks(rows_bound, batch)
+ *   (rows_bound >= all compressed rows of the batch; chunk c of sequence b sits at slot cu_cmp[b] / 64 + b + c).
+ * 16-bit types, head dims (64,64), (128,128), (192,128).  No counterpart in the reference (Triton loads its tiles
+ * from the row-major tensors). */
+int nsa_cmp_pack_chunks(int total_rows, int batch);
+int nsa_cmp_pack_fwd(const void* ck, const void* cv, void* frag, const int32_t* cu_cmp, int batch, int rows_bound, int hkv,
+                     int dk, int dv, int64_t ck_row_stride, int64_t ck_head_stride, int64_t cv_row_stride,
+                     int64_t cv_head_stride, int frag_chunks, int dtype, nsa_stream_t stream);
+int nsa_cmp_select_fwd(const void* q, const void* ck, const void* cvt, const void* frag, int frag_chunks, void* o,
+                       void* indices, float* pooled, float* lse,
                        float* lse_attn, const void* gate_weight, const void* gate_bias, void* gates,
                        const int32_t* cu_seqlens, const int32_t* cu_cmp, int batch, int total, int hq, int hkv, int dk,
                        int dv, int64_t ck_row_stride, int64_t ck_head_stride, int cvt_cols, int block, int stride,

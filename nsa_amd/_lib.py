@@ -31,7 +31,9 @@ SIGNATURES = {
     "nsa_cmp_attn_fwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _L, _I, _I, _I, _F, _I, _I, _P]),
     "nsa_cmp_attn_gate_fwd": (_I, [_P] * 11 + [_I, _I, _I, _I, _I, _I, _L, _L, _I, _I, _I, _F, _I, _I, _P]),
     "nsa_cmp_select_single_pass": (_I, [_I] * 10),
-    "nsa_cmp_select_fwd": (_I, [_P] * 13 + [_I] * 6 + [_L, _L] + [_I] * 11 + [_F] + [_I] * 4 + [_P]),
+    "nsa_cmp_pack_chunks": (_I, [_I, _I]),
+    "nsa_cmp_pack_fwd": (_I, [_P] * 4 + [_I] * 5 + [_L] * 4 + [_I, _I, _P]),
+    "nsa_cmp_select_fwd": (_I, [_P] * 4 + [_I] + [_P] * 10 + [_I] * 6 + [_L, _L] + [_I] * 11 + [_F] + [_I] * 4 + [_P]),
     "nsa_block_select_fwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _L, _L, _I, _I, _I, _I, _I, _I,
                                   _I, _I, _I, _P]),
     "nsa_gate_fwd": (_I, [_P, _P, _P, _P, _L, _I, _I, _P]),

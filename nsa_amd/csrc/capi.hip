@@ -141,7 +141,7 @@ static int cmp_common(const char* what, int stages, const void* q, const void* c
                       int pool_pad, int top_n, int max_ns, int pooled_stride, int keep_pooled, float scale, int causal,
                       int idx64, int dtype, nsa_stream_t stream, const void* gate_w = nullptr,
                       const void* gate_b = nullptr, void* gates = nullptr, int single_pass_max_nc = -1,
-                      int single_pass = 0) {
+                      int single_pass = 0, const void* frag = nullptr, int frag_chunks = 0) {
   // single_pass_max_nc >= 0 (stages 3 only): the most compressed rows of any sequence, with which the call may run
   // as ONE kernel (single_pass -1 = when the shape qualifies, 1 = or fail, 0 = never)
   const bool attn = stages & 1, select = stages & 2;
@@ -149,7 +149,7 @@ static int cmp_common(const char* what, int stages, const void* q, const void* c
     return fail(NSA_ERR_INVALID, "%s: the gating Linear needs its weight and the gates buffer", what);
   if (gate_w && !aligned16(gate_w)) return fail(NSA_ERR_INVALID, "%s: pointers must be 16-byte aligned", what);
   if (!q || !ck || !cu_seqlens || !cu_cmp) return fail(NSA_ERR_INVALID, "%s: null pointer", what);
-  if (attn && (!cvt || !o)) return fail(NSA_ERR_INVALID, "%s: null pointer", what);
+  if (attn && ((!cvt && !frag) || !o)) return fail(NSA_ERR_INVALID, "%s: null pointer", what);
   if (batch <= 0 || total <= 0 || block <= 0 || stride <= 0) return fail(NSA_ERR_INVALID, "%s: sizes must be positive", what);
   if (!dtype_ok(dtype)) return fail(NSA_ERR_INVALID, "%s: bad dtype", what);
   int kv_rep = 1;
@@ -157,7 +157,7 @@ static int cmp_common(const char* what, int stages, const void* q, const void* c
   if (!(scale > 0.f)) return fail(NSA_ERR_INVALID, "%s: scale must be positive", what);
   if (ck_row_stride % 8 != 0 || ck_head_stride % 8 != 0 || (attn && cvt_cols % 64 != 0))
     return fail(NSA_ERR_INVALID, "%s: ck strides must be multiples of 8, cvt_cols of 64", what);
-  if (!aligned16(q) || !aligned16(ck) || (attn && (!aligned16(cvt) || !aligned16(o))))
+  if (!aligned16(q) || !aligned16(ck) || (attn && ((cvt && !aligned16(cvt)) || !aligned16(o))))
     return fail(NSA_ERR_INVALID, "%s: pointers must be 16-byte aligned", what);
   if (select) {
     if (!indices) return fail(NSA_ERR_INVALID, "%s: the selection needs indices and the lse buffer", what);
@@ -172,14 +172,18 @@ static int cmp_common(const char* what, int stages, const void* q, const void* c
                  pool_pad, top_n, max_ns, pooled_stride, scale, idx64, dtype, causal, lse_attn, kv_rep};
   a.keep_pooled = keep_pooled != 0;
   a.gate_w = gate_w; a.gate_b = gate_b; a.gates = gates;
+  a.frag = frag; a.frag_chunks = frag_chunks;
   int rc = 0;
+  if (frag && (!aligned16(frag) || frag_chunks < nsa::cmp_frag_chunks(0, batch)))
+    return fail(NSA_ERR_INVALID, "%s: bad fragment-major copy (alignment / chunk slots)", what);
   if (attn && select && single_pass != 0 && single_pass_max_nc >= 0) {
     if (nsa::cmp_select_single_pass_ok(a, single_pass_max_nc)) return finish(nsa::launch_cmp_select(a, stream), what);
     if (single_pass == 1)
       return fail(NSA_ERR_UNSUPPORTED, "%s: the single-pass kernel takes GQA groups of 9..16 heads, 16-bit inputs, head dims "
                   "(64,64) (128,128) (192,128), pooling windows of 5 rows every 4 without padding, at most 2048 compressed "
-                  "rows per sequence and top_n <= 64", what);
+                  "rows per sequence, top_n <= 64, and needs the fragment-major copy of nsa_cmp_pack_fwd", what);
   }
+  if (attn && !cvt) return fail(NSA_ERR_INVALID, "%s: null pointer", what);
   if (select && !lse) return fail(NSA_ERR_INVALID, "%s: the selection needs indices and the lse buffer", what);
   if (attn) rc = nsa::launch_cmp_attn(a, stream);
   if (rc == 0 && select) rc = nsa::launch_select(a, stream);
@@ -210,11 +214,33 @@ int nsa_cmp_select_single_pass(int hq, int hkv, int dk, int dv, int pool_kernel,
   a.top_n = top_n; a.dtype = dtype; a.kv_rep = hq / hkv > 16 ? 2 : 1;
   a.max_ns = max_nc >= 5 ? (max_nc - 2) / 4 + 1 : 0;
   static int dummy;
-  a.indices = &dummy; a.cvt = &dummy; a.o = &dummy;         // the shape test only asks whether they are given
+  a.indices = &dummy; a.frag = &dummy; a.o = &dummy;        // the shape test only asks whether they are given
   return nsa::cmp_select_single_pass_ok(a, max_nc) ? 1 : 0;
 }
 
-int nsa_cmp_select_fwd(const void* q, const void* ck, const void* cvt, void* o, void* indices, float* pooled, float* lse,
+int nsa_cmp_pack_chunks(int total_rows, int batch) { return nsa::cmp_frag_chunks(total_rows, batch); }
+
+int nsa_cmp_pack_fwd(const void* ck, const void* cv, void* frag, const int32_t* cu_cmp, int batch, int rows_bound, int hkv,
+                     int dk, int dv, int64_t ck_row_stride, int64_t ck_head_stride, int64_t cv_row_stride,
+                     int64_t cv_head_stride, int frag_chunks, int dtype, nsa_stream_t stream) {
+  if (!ck || !cv || !frag || !cu_cmp) return fail(NSA_ERR_INVALID, "cmp_pack: null pointer");
+  if (batch <= 0 || rows_bound < 0 || hkv <= 0) return fail(NSA_ERR_INVALID, "cmp_pack: sizes must be positive");
+  if (dtype != NSA_BF16 && dtype != NSA_F16) return fail(NSA_ERR_UNSUPPORTED, "cmp_pack: 16-bit types only");
+  if (ck_row_stride % 8 || ck_head_stride % 8 || cv_row_stride % 8 || cv_head_stride % 8 || !aligned16(ck) ||
+      !aligned16(cv) || !aligned16(frag))
+    return fail(NSA_ERR_INVALID, "cmp_pack: strides must be multiples of 8 elements, pointers 16-byte aligned");
+  if (frag_chunks < nsa::cmp_frag_chunks(rows_bound, batch))
+    return fail(NSA_ERR_INVALID, "cmp_pack: frag_chunks smaller than nsa_cmp_pack_chunks(rows_bound, batch)");
+  nsa::CmpArgs a{};
+  a.ck = ck; a.cvt = cv; a.frag = frag; a.frag_chunks = frag_chunks; a.cu_cmp = cu_cmp; a.batch = batch; a.hkv = hkv;
+  a.dk = dk; a.dv = dv; a.ck_row_stride = (long)ck_row_stride; a.ck_head_stride = (long)ck_head_stride; a.dtype = dtype;
+  const int rc = nsa::launch_frag_pack(a, (long)cv_row_stride, (long)cv_head_stride, rows_bound, stream);
+  if (rc == -2) return fail(NSA_ERR_UNSUPPORTED, "cmp_pack: head dims (64,64), (128,128), (192,128)");
+  return finish(rc, "cmp_pack");
+}
+
+int nsa_cmp_select_fwd(const void* q, const void* ck, const void* cvt, const void* frag, int frag_chunks, void* o,
+                       void* indices, float* pooled, float* lse,
                        float* lse_attn, const void* gate_weight, const void* gate_bias, void* gates,
                        const int32_t* cu_seqlens, const int32_t* cu_cmp, int batch, int total, int hq, int hkv, int dk,
                        int dv, int64_t ck_row_stride, int64_t ck_head_stride, int cvt_cols, int block, int stride,
@@ -226,7 +252,7 @@ int nsa_cmp_select_fwd(const void* q, const void* ck, const void* cvt, void* o, 
   return cmp_common("cmp_select", 3, q, ck, cvt, o, indices, pooled, lse, lse_attn, cu_seqlens, cu_cmp, batch, total, hq,
                     hkv, dk, dv, ck_row_stride, ck_head_stride, cvt_cols, block, stride, pool_kernel, pool_stride,
                     pool_pad, top_n, max_ns, pooled_stride, keep_pooled, scale, causal, idx64, dtype, stream, gate_weight,
-                    gate_bias, gates, max_nc, single_pass);
+                    gate_bias, gates, max_nc, single_pass, frag, frag_chunks);
 }
 
 int nsa_cmp_attn_fwd(const void* q, const void* ck, const void* cvt, void* o, float* lse, float* lse_attn,

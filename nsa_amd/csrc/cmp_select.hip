@@ -23,7 +23,9 @@
 // lower quad and sits one lane row further (or, for g = 3, in the next step) for the upper one.  Step i therefore
 // writes slot 2i (window 8i + 2g) and slot 2i + 1 (window 8i + 2g + 1; in lane row 3 the window 8i - 1 of the step
 // before, completed by this step's first row).  The last step's upper quad of lane row 3 has no next row and
-// stays in `pend`, a 129th value per lane.
+// stays in `pend`, a 129th value per lane.  Slots 0 .. 95 (rows 0 .. 1535) are registers; the slots of the last 512
+// rows go to a lane-private column of LDS (8 KB per wavefront): 128 more registers would not leave room for the
+// query fragments and the output accumulators of a 192-wide head at two wavefronts per SIMD.
 #include <type_traits>
 
 #include "tiles.h"
@@ -34,7 +36,76 @@ typedef float f32x32_t __attribute__((ext_vector_type(32)));
 
 int set_smem(const void* fn, size_t bytes);
 
-constexpr int kFusedMaxRows = 2048;      // compressed rows per sequence the bins have room for
+// ------------------------------------------------------------------------------------------------
+// Fragment-major copy of the compressed keys and values.
+//
+// The pass streams every 64-row chunk of a sequence's compressed K and V through LDS once per token tile.  With the
+// chunk stored in memory exactly as the matrix instructions consume it -- one 1 KB block per operand fragment, lane
+// l's 16 bytes at byte 16 l -- the global -> LDS copy is a straight run of bytes (done by the load unit itself,
+// global_load_lds, no staging registers and no LDS store instructions) and every fragment read is 64 consecutive
+// 16-byte pieces: no padding, no bank conflicts, whatever the row -> lane map.
+//   chunk = [ K part: step s (32 rows) | tile t (0/1) | depth block kk | lane | 8 elements ]
+//           [ V part: step s           | channel tile tv (16 channels)  | lane | 8 elements ]
+//   K fragment (s, t, kk), lane (m, g):  K[32 s + chunk_key_of_row(t, m)][32 kk + 8 g .. + 7]
+//   V fragment (s, tv),    lane (m, g):  V[32 s + 8 g .. + 7][16 tv + m]   (8 rows of one channel)
+// Chunk c of sequence b of kv head h sits at chunk slot cu_cmp[b] / 64 + b + c of that head (slots of different
+// sequences never overlap; at most total_rows / 64 + batch + 1 slots).  Rows past the sequence's last one are zero.
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+typedef __attribute__((address_space(1))) const void* global_void_ptr;
+
+// 16 bytes per lane from global memory straight into LDS: lane i's piece lands at lds + 16 i bytes (lds is the same
+// for the whole wavefront).  Counts as a vector-memory load of the wavefront until the data is in LDS.
+template <typename T>
+__device__ __forceinline__ void global_to_lds16(const T* src, T* lds) {
+  __builtin_amdgcn_global_load_lds((global_void_ptr)src, (lds_void_ptr)lds, 16, 0, 0);
+}
+
+__host__ __device__ __forceinline__ int frag_chunk_slot(int cu_b, int b) { return (cu_b >> 6) + b; }
+
+template <typename T, int DK, int DV>
+__global__ void __launch_bounds__(256)
+frag_pack_kernel(const T* __restrict__ ck, const T* __restrict__ cv, T* __restrict__ frag, const int32_t* cu_cmp,
+                 int batch, long ck_row_stride, long ck_head_stride, long cv_row_stride, long cv_head_stride,
+                 int frag_chunks) {
+  constexpr int KLD = DK + 8, VLD = DV + 2, NKK = DK / 32, NV = DV / 16, CHUNK = 64 * (DK + DV);
+  __shared__ __attribute__((aligned(16))) T sk[64 * KLD];
+  __shared__ T sv[64 * VLD];
+  const SeqTile st = find_tile(cu_cmp, batch, 64, blockIdx.x);
+  if (!st.valid) return;
+  const int h = blockIdx.y, tid = threadIdx.x;
+  const T* kb = ck + (long)(st.start + st.t0) * ck_row_stride + (long)h * ck_head_stride;
+  const T* vb = cv + (long)(st.start + st.t0) * cv_row_stride + (long)h * cv_head_stride;
+  const int rows = min(64, st.len - st.t0);
+  for (int p = tid; p < 64 * (DK / 8); p += 256) {
+    const int r = p / (DK / 8), pc = p % (DK / 8);
+    store8(sk + r * KLD + pc * 8, r < rows ? load8(kb + (long)r * ck_row_stride + pc * 8) : zero8<T>());
+  }
+  for (int p = tid; p < 64 * (DV / 8); p += 256) {
+    const int r = p / (DV / 8), pc = p % (DV / 8);
+    const vec8_t<T> x = r < rows ? load8(vb + (long)r * cv_row_stride + pc * 8) : zero8<T>();
+#pragma unroll
+    for (int e = 0; e < 8; ++e) sv[r * VLD + pc * 8 + e] = x[e];
+  }
+  __syncthreads();
+  T* out = frag + ((long)h * frag_chunks + frag_chunk_slot(st.start, st.b) + (st.t0 >> 6)) * CHUNK;
+  for (int p = tid; p < 64 * (DK / 8); p += 256) {
+    const int l = p & 63, f = p >> 6;                 // fragment f = (s * 2 + t) * NKK + kk
+    const int kk = f % NKK, t = (f / NKK) & 1, sstep = f / (2 * NKK);
+    const int m = l & 15, g = l >> 4;
+    store8(out + p * 8, load8(sk + (32 * sstep + chunk_key_of_row(t, m)) * KLD + 32 * kk + 8 * g));
+  }
+  for (int p = tid; p < 64 * (DV / 8); p += 256) {
+    const int l = p & 63, f = p >> 6;                 // fragment f = s * NV + tv
+    const int tv = f % NV, sstep = f / NV;
+    const int m = l & 15, g = l >> 4;
+    vec8_t<T> x;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = sv[(32 * sstep + 8 * g + e) * VLD + 16 * tv + m];
+    store8(out + 64 * DK + p * 8, x);
+  }
+}
+
+constexpr int kFusedMaxRows = 2048;      // compressed rows per sequence the window sums have room for
 
 // Top-n over the PER candidates every lane holds (score v[k] >= 0 with window number ix[k]; -1 = no candidate),
 // descending, ties to the lower window number; emit(r, window or -1).  The shortlist of tiles.h with explicit
@@ -128,14 +199,13 @@ __device__ __forceinline__ void scatter_level(const float (&in)[2 * N], float (&
 template <typename T, int DK, int DV>
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 cmp_select_kernel(const CmpArgs a) {
-  constexpr int NW = 8, CH = 64, NT = NW * 64, TQ = NW;
-  constexpr int KLD = DK + kLdsRowPad<T>, VLD = CH + kLdsRowPad<T>;
-  constexpr int KPIECES = CH * DK / 8, VPIECES = DV * CH / 8;
-  constexpr int KPT = (KPIECES + NT - 1) / NT, VPT = (VPIECES + NT - 1) / NT;
+  constexpr int NW = 8, TQ = NW, NKK = DK / 32, NV = DV / 16;
+  constexpr int KPART = 64 * DK, CHUNK = 64 * (DK + DV);          // elements of a chunk's K part / of a chunk
+  constexpr int NKB = KPART / 512, NVB = 64 * DV / 512;           // 1 KB blocks of the two parts
   constexpr bool kNarrowP = std::is_same<T, f16_t>::value;      // packed probabilities narrower than the fp32 sums
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  T* ldsK = reinterpret_cast<T*>(smem_raw);          // [2][CH][KLD]
-  T* ldsV = ldsK + 2 * CH * KLD;                     // [2][DV][VLD]
+  T* ldsC = reinterpret_cast<T*>(smem_raw);                        // [2][CHUNK]: chunks in fragment order
+  float* ldsB = reinterpret_cast<float*>(ldsC + 2 * CHUNK);        // [NW][32 slots][64 lanes]
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -148,9 +218,7 @@ cmp_select_kernel(const CmpArgs a) {
   const bool tok_ok = tok < st.len;
   const int koff = a.cu_cmp[st.b];
   const int nkeys = min(a.cu_cmp[st.b + 1] - koff, kFusedMaxRows);
-  const int vtoff = transposed_offset(koff, st.b);
-  const T* kb = reinterpret_cast<const T*>(a.ck) + (long)koff * a.ck_row_stride + (long)h * a.ck_head_stride;
-  const T* vtb = reinterpret_cast<const T*>(a.cvt) + (long)h * DV * a.cvt_cols + vtoff;
+  const T* fragb = reinterpret_cast<const T*>(a.frag) + ((long)h * a.frag_chunks + frag_chunk_slot(koff, st.b)) * CHUNK;
 
   auto last_visible = [&](int t) -> int {            // largest compressed row token t may attend
     if (!a.causal) return nkeys - 1;
@@ -179,7 +247,7 @@ cmp_select_kernel(const CmpArgs a) {
     const T* bp = reinterpret_cast<const T*>(a.gate_b);
     f32x4_t gt = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int kk = 0; kk < DK / 32; ++kk) gt = mma16(n < 3 ? load8(wp + 32 * kk) : zero8<T>(), grp[0].q[kk], gt);
+    for (int kk = 0; kk < NKK; ++kk) gt = mma16(n < 3 ? load8(wp + 32 * kk) : zero8<T>(), grp[0].q[kk], gt);
     if (g == 0 && rm.valid) {
       T* gp = reinterpret_cast<T*>(a.gates) + (((long)st.start + rm.tok) * a.hq + h * G + rm.gidx) * 3;
 #pragma unroll
@@ -188,77 +256,34 @@ cmp_select_kernel(const CmpArgs a) {
   }
   const float c_attn = a.scale * kLog2e;
 
-  // staging: every thread moves KPT + VPT 16-byte pieces of a 64-row chunk
-  vec8_t<T> kr[KPT], vr[VPT];
-  unsigned kpo[KPT], vpo[VPT];
+  // staging: the load unit copies the chunk, 1 KB per wavefront instruction; wavefront w takes blocks w, w + 8, ..
+  auto stage_chunk = [&](int c0, int buf, bool with_v) {
+    const T* src = fragb + (long)(c0 >> 6) * CHUNK + lane * 8;
+    T* dst = ldsC + buf * CHUNK;
 #pragma unroll
-  for (int i = 0; i < KPT; ++i) {
-    const int p = tid + i * NT;
-    kpo[i] = (unsigned)((p / (DK / 8)) * (int)a.ck_row_stride + (p % (DK / 8)) * 8);
-  }
-#pragma unroll
-  for (int i = 0; i < VPT; ++i) {
-    const int p = tid + i * NT;
-    vpo[i] = (unsigned)((p / (CH / 8)) * a.cvt_cols + (p % (CH / 8)) * 8);
-  }
-  auto gload = [&](int c0, bool with_v) {
-    if (c0 + CH <= nkeys) {
-      const unsigned base = (unsigned)c0 * (unsigned)a.ck_row_stride;
-#pragma unroll
-      for (int i = 0; i < KPT; ++i)
-        if (KPIECES % NT == 0 || tid + i * NT < KPIECES) kr[i] = load8(kb + (base + kpo[i]));
-    } else {                                         // last chunk of the sequence: clamp the row
-#pragma unroll
-      for (int i = 0; i < KPT; ++i) {
-        const int p = tid + i * NT;
-        if (KPIECES % NT == 0 || p < KPIECES) {
-          const int sr = min(c0 + p / (DK / 8), nkeys - 1);
-          kr[i] = load8(kb + (long)sr * a.ck_row_stride + (p % (DK / 8)) * 8);
-        }
-      }
-    }
+    for (int i = 0; i < (NKB + NW - 1) / NW; ++i)
+      if (NKB % NW == 0 || wave + i * NW < NKB) global_to_lds16(src + (wave + i * NW) * 512, dst + (wave + i * NW) * 512);
     if (with_v) {
 #pragma unroll
-      for (int i = 0; i < VPT; ++i)
-        if (VPIECES % NT == 0 || tid + i * NT < VPIECES) vr[i] = load8(vtb + ((unsigned)c0 + vpo[i]));
+      for (int i = 0; i < (NVB + NW - 1) / NW; ++i)
+        if (NVB % NW == 0 || wave + i * NW < NVB)
+          global_to_lds16(src + KPART + (wave + i * NW) * 512, dst + KPART + (wave + i * NW) * 512);
     }
   };
-  auto lstore = [&](int buf, bool with_v) {
-    T* dk = ldsK + buf * CH * KLD;
-#pragma unroll
-    for (int i = 0; i < KPT; ++i) {
-      const int p = tid + i * NT;
-      if (KPIECES % NT == 0 || p < KPIECES) store8(dk + (p / (DK / 8)) * KLD + (p % (DK / 8)) * 8, kr[i]);
-    }
-    if (with_v) {
-      T* dv = ldsV + buf * DV * VLD;
-#pragma unroll
-      for (int i = 0; i < VPT; ++i) {
-        const int p = tid + i * NT;
-        if (VPIECES % NT == 0 || p < VPIECES) {
-          // rows 16..31 of every 32-row step: the two 4-row halves trade places (see lds_key_of_row)
-          const int pc = p % (CH / 8);
-          vec8_t<T> x = vr[i];
-          if (pc & 2) {
-            vec8_t<T> y;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) y[e] = x[e ^ 4];
-            x = y;
-          }
-          store8(dv + (p / (CH / 8)) * VLD + pc * 8, x);
-        }
-      }
-    }
+  auto staged = [&]() {                       // this wavefront's blocks have landed; then everybody's
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
   };
 
-  const bool swapped = (g >> 1) != 0;        // value i of this lane is row 8g + (i ^ 4) of the step instead of 8g + i
-  const int swp = lds_key_swap(g);
   const bool last_row = g == 3;
   const int next_lane = ((lane + 16) & 63) << 2;
 
-  f32x32_t bq0, bq1, bq2, bq3;               // the window sums of this lane's head: slot s = bq<s / 32>[s % 32]
+  f32x32_t bq0, bq1, bq2;                    // the window sums of this lane's head: slot s < 96 = bq<s / 32>[s % 32]
 #pragma unroll
-  for (int i = 0; i < 32; ++i) { bq0[i] = 0.f; bq1[i] = 0.f; bq2[i] = 0.f; bq3[i] = 0.f; }
+  for (int i = 0; i < 32; ++i) { bq0[i] = 0.f; bq1[i] = 0.f; bq2[i] = 0.f; }
+  float* binl = ldsB + (wave * 32) * 64 + lane;      // slot 96 + j = binl[64 j]
+#pragma unroll
+  for (int i = 0; i < 32; ++i) binl[64 * i] = 0.f;
   float li = 0.f;                            // this lane's share of the importance denominator
   float pend = 0.f;                          // lane row 3: the upper quad of the step before
   float pmax = 0.f;                          // float16: the largest 8-row sum of packed probabilities
@@ -267,20 +292,28 @@ cmp_select_kernel(const CmpArgs a) {
 
   wait_all_loads();
 
-  // One 32-row step.  derive: the first step sets the references.
-  auto step32 = [&](f32x32_t& bins, int slot, int cb, const T* bk, const T* bv, bool derive) {
-    f32x4_t s0[1], s1[1];
-    const T* ks = bk + 8 * g;
-    scores32<T, DK, DV, 1>(ks + lds_key_of_row(0, n) * KLD, ks + lds_key_of_row(1, n) * KLD, grp, s0, s1);
-    float s[8];
+  // raw scores of one 32-row step: value i of lane (n, g) = row 8g + i of the step, head n
+  auto scores = [&](const T* kf, float (&s)[8]) {
+    f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int i = 0; i < 4; ++i) { s[i] = s0[0][i]; s[4 + i] = s1[0][i]; }
+    for (int kk = 0; kk < NKK; ++kk) {
+      s0 = mma16(load8(kf + kk * 512), grp[0].q[kk], s0);
+      s1 = mma16(load8(kf + (NKK + kk) * 512), grp[0].q[kk], s1);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { s[i] = s0[i]; s[4 + i] = s1[i]; }
+  };
+
+  // One 32-row step.  derive: the first step sets the references.  kf / vf: the step's fragments (this lane's piece)
+  auto step32 = [&](auto put, int slot, int cb, const T* kf, const T* vf, bool derive) {
+    float s[8];
+    scores(kf, s);
     const int key0 = cb + 8 * g;
     if (cb + 32 > nkeys) {                           // last step of the sequence only
       asm volatile("" ::: "memory");
 #pragma unroll
       for (int i = 0; i < 8; ++i)
-        if (key0 + (i ^ swp) >= nkeys) s[i] = kNegInf;
+        if (key0 + i >= nkeys) s[i] = kNegInf;
     }
     if (derive && cb == 0) {                         // the reference: largest score of the first 32 rows
       float mx = s[0];
@@ -293,14 +326,11 @@ cmp_select_kernel(const CmpArgs a) {
     float e[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) e[i] = fast_exp2(fmaf(s[i], kLog2e, off_i));
-    const float qlo = (e[0] + e[1]) + (e[2] + e[3]), qhi = (e[4] + e[5]) + (e[6] + e[7]);
-    li += qlo + qhi;
-    const float first = swapped ? e[4] : e[0];       // row 8g: completes the upper window of the lane row before
-    const float fifth = swapped ? e[0] : e[4];       // row 8g + 4: completes this lane's lower window
-    const float qa = swapped ? qhi : qlo, qb = swapped ? qlo : qhi;
-    const float nxt = __int_as_float(__builtin_amdgcn_ds_bpermute(next_lane, __float_as_int(first)));
-    bins[slot] = qa + fifth;
-    bins[slot + 1] = (last_row ? pend : qb) + nxt;
+    const float qa = (e[0] + e[1]) + (e[2] + e[3]), qb = (e[4] + e[5]) + (e[6] + e[7]);
+    li += qa + qb;
+    // e[0] (row 8g) completes the upper window of the lane row before, e[4] this lane's lower window
+    const float nxt = __int_as_float(__builtin_amdgcn_ds_bpermute(next_lane, __float_as_int(e[0])));
+    put(slot, qa + e[4], (last_row ? pend : qb) + nxt);
     pend = qb;
     if (cb <= hi) {                                  // the token attends rows of this step
       float p[8];
@@ -310,47 +340,41 @@ cmp_select_kernel(const CmpArgs a) {
         asm volatile("" ::: "memory");
 #pragma unroll
         for (int i = 0; i < 8; ++i)
-          if (key0 + (i ^ swp) > hi) p[i] = 0.f;
+          if (key0 + i > hi) p[i] = 0.f;
       }
       const float p8 = sum8(p);
       grp[0].l += p8;
       if constexpr (kNarrowP) pmax = fmaxf(pmax, p8);
-      vec8_t<T> pb[1];
-      pb[0] = pack8<T>(p);
-      pv32_all<T, DK, DV, 1>(bv + n * VLD + 8 * g, 16 * VLD, grp, pb);
+      const vec8_t<T> pb = pack8<T>(p);
+#pragma unroll
+      for (int t = 0; t < NV; ++t) grp[0].o[t] = mma16(load8(vf + t * 512), pb, grp[0].o[t]);
     }
   };
 
   auto run_pass = [&](bool derive) {
-    if (c_end > 0) {
-      gload(0, 0 <= attn_end);
-      lstore(0, 0 <= attn_end);
-    }
-    __syncthreads();
+    if (c_end > 0) stage_chunk(0, 0, 0 <= attn_end);
+    staged();
     int buf = 0;
     // 512 rows = 16 steps = 32 slots per section: inside a section the slots of one register block are written
     // in place with a scalar index
-    auto section = [&](f32x32_t& bins, int c_first) {
+    auto section = [&](auto put, int c_first) {
       const int c_stop = min(c_first + 512, c_end);
-      for (int c0 = c_first; c0 < c_stop; c0 += CH) {
-        const int cn = c0 + CH;
-        const bool has_next = cn < c_end;
-        const bool next_v = has_next && cn <= attn_end;
-        if (has_next) gload(cn, next_v);
-        const T* bk = ldsK + buf * CH * KLD;
-        const T* bv = ldsV + buf * DV * VLD;
+      for (int c0 = c_first; c0 < c_stop; c0 += 64) {
+        const int cn = c0 + 64;
+        if (cn < c_end) stage_chunk(cn, buf ^ 1, cn <= attn_end);
+        const T* kf = ldsC + buf * CHUNK + lane * 8;
+        const T* vf = kf + KPART;
         const int slot = (c0 - c_first) >> 4;
-        step32(bins, slot, c0, bk, bv, derive);
-        if (c0 + 32 < c_end) step32(bins, slot + 2, c0 + 32, bk + 32 * KLD, bv + 32, derive);
-        if (has_next) lstore(buf ^ 1, next_v);
-        __syncthreads();
+        step32(put, slot, c0, kf, vf, derive);
+        if (c0 + 32 < c_end) step32(put, slot + 2, c0 + 32, kf + 2 * NKK * 512, vf + NV * 512, derive);
+        staged();
         buf ^= 1;
       }
     };
-    section(bq0, 0);
-    section(bq1, 512);
-    section(bq2, 1024);
-    section(bq3, 1536);
+    section([&](int s, float x0, float x1) { bq0[s] = x0; bq0[s + 1] = x1; }, 0);
+    section([&](int s, float x0, float x1) { bq1[s] = x0; bq1[s + 1] = x1; }, 512);
+    section([&](int s, float x0, float x1) { bq2[s] = x0; bq2[s + 1] = x1; }, 1024);
+    section([&](int s, float x0, float x1) { binl[64 * s] = x0; binl[64 * s + 64] = x1; }, 1536);
   };
 
   run_pass(true);
@@ -368,33 +392,26 @@ cmp_select_kernel(const CmpArgs a) {
       // Rare: exact maxima first (scores only: the importance one over all rows, the attention one over the
       // visible rows), then the same pass with those as references -- no exponential exceeds 1.
       float mx_all = kNegInf, mx_vis = kNegInf;
-      if (c_end > 0) {
-        gload(0, false);
-        lstore(0, false);
-      }
-      __syncthreads();
+      if (c_end > 0) stage_chunk(0, 0, false);
+      staged();
       int buf = 0;
-      for (int c0 = 0; c0 < c_end; c0 += CH) {
-        const bool has_next = c0 + CH < c_end;
-        if (has_next) gload(c0 + CH, false);
-        const T* bk = ldsK + buf * CH * KLD;
+      for (int c0 = 0; c0 < c_end; c0 += 64) {
+        if (c0 + 64 < c_end) stage_chunk(c0 + 64, buf ^ 1, false);
+        const T* kf = ldsC + buf * CHUNK + lane * 8;
 #pragma unroll
         for (int sub = 0; sub < 2; ++sub) {
           const int cb = c0 + 32 * sub;
           if (cb >= c_end) break;
-          f32x4_t s0[1], s1[1];
-          const T* ks = bk + 32 * sub * KLD + 8 * g;
-          scores32<T, DK, DV, 1>(ks + lds_key_of_row(0, n) * KLD, ks + lds_key_of_row(1, n) * KLD, grp, s0, s1);
+          float s[8];
+          scores(kf + sub * 2 * NKK * 512, s);
 #pragma unroll
           for (int i = 0; i < 8; ++i) {
-            const float sv = i < 4 ? s0[0][i] : s1[0][i - 4];
-            const int key = cb + 8 * g + (i ^ swp);
-            if (key < nkeys) mx_all = fmaxf(mx_all, sv);
-            if (key <= hi) mx_vis = fmaxf(mx_vis, sv);
+            const int key = cb + 8 * g + i;
+            if (key < nkeys) mx_all = fmaxf(mx_all, s[i]);
+            if (key <= hi) mx_vis = fmaxf(mx_vis, s[i]);
           }
         }
-        if (has_next) lstore(buf ^ 1, false);
-        __syncthreads();
+        staged();
         buf ^= 1;
       }
       m_i = colgroup_max(mx_all);
@@ -412,12 +429,12 @@ cmp_select_kernel(const CmpArgs a) {
     }
   }
 
-  // ---- attention output: rows leave through LDS (the K buffers are free after the pass's last barrier)
+  // ---- attention output: rows leave through LDS (the chunk buffers are free after the pass's last barrier)
   constexpr int OLD = DV + 8, PIECES = DV / 8;
-  static_assert(NW * 16 * OLD * sizeof(T) + NW * 1024 <= (2 * CH * KLD + 2 * DV * VLD) * sizeof(T),
-                "output staging and the top-n shortlists must fit the K/V buffers");
+  static_assert(NW * 16 * OLD * sizeof(T) + NW * 1024 <= 2 * CHUNK * sizeof(T),
+                "output staging and the top-n shortlists must fit the chunk buffers");
   {
-    T* stage = ldsK + wave * 16 * OLD;
+    T* stage = ldsC + wave * 16 * OLD;
     const float inv = lt > 0.f ? 1.0f / lt : 0.f;
     store_rows<T, DV>(stage + n * OLD, grp[0].o, inv, g);
     T* ob = reinterpret_cast<T*>(a.o);
@@ -448,7 +465,7 @@ cmp_select_kernel(const CmpArgs a) {
     float x[128];
 #pragma unroll
     for (int i = 0; i < 32; ++i) {
-      x[i] = bq0[i] * w; x[32 + i] = bq1[i] * w; x[64 + i] = bq2[i] * w; x[96 + i] = bq3[i] * w;
+      x[i] = bq0[i] * w; x[32 + i] = bq1[i] * w; x[64 + i] = bq2[i] * w; x[96 + i] = binl[64 * i] * w;
     }
     // Partners: lane ^ 15 (row_mirror), ^ 7 (row_half_mirror), ^ 2, ^ 1 (quad permutations); each level is keyed on
     // a lane bit that its own partner flips and the later partners keep.  Lane n ends with the slots 16 k + c(n),
@@ -495,7 +512,7 @@ cmp_select_kernel(const CmpArgs a) {
   }
   int picked = -1;
   auto emit = [&](int r, int val) { picked = lane == r ? val : picked; };
-  float* cand_v = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(ldsK) + NW * 16 * OLD * sizeof(T)) + wave * 256;
+  float* cand_v = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(ldsC) + NW * 16 * OLD * sizeof(T)) + wave * 256;
   int* cand_i = reinterpret_cast<int*>(cand_v + 128);
   wave_topn_indexed<9>(v, ix, a.top_n, lane, cand_v, cand_i, emit);
   if (lane < a.top_n) {
@@ -511,14 +528,16 @@ bool cmp_select_single_pass_ok(const CmpArgs& a, int max_nc) {
   const int G = a.hq / a.hkv;
   return a.kv_rep == 1 && G >= 9 && G <= 16 && (a.dtype == 0 || a.dtype == 2) && a.pool_k == 5 && a.pool_s == 4 &&
          a.pool_p == 0 && max_nc <= kFusedMaxRows && a.max_ns <= 512 && a.top_n <= 64 && a.indices != nullptr &&
-         a.cvt != nullptr && a.o != nullptr &&
+         a.frag != nullptr && a.o != nullptr &&
          ((a.dk == 64 && a.dv == 64) || (a.dk == 128 && a.dv == 128) || (a.dk == 192 && a.dv == 128));
 }
 
+// chunk slots per kv head of the fragment-major copy for `total_rows` compressed rows in `batch` sequences
+int cmp_frag_chunks(int total_rows, int batch) { return total_rows / 64 + batch + 1; }
+
 template <typename T, int DK, int DV>
 static int launch_cmp_select_t(const CmpArgs& a, hipStream_t st) {
-  constexpr int CH = 64;
-  const size_t smem = 2 * ((size_t)CH * (DK + kLdsRowPad<T>) + (size_t)DV * (CH + kLdsRowPad<T>)) * sizeof(T);
+  const size_t smem = 2 * (size_t)64 * (DK + DV) * sizeof(T) + 8 * 32 * 64 * sizeof(float);
   auto fn = cmp_select_kernel<T, DK, DV>;
   const int rc = set_smem(reinterpret_cast<const void*>(fn), smem);
   if (rc) return rc;
@@ -527,25 +546,44 @@ static int launch_cmp_select_t(const CmpArgs& a, hipStream_t st) {
   return 0;
 }
 
-int launch_cmp_select(const CmpArgs& a, hipStream_t st) {
-  const int key = a.dk * 1000 + a.dv;
-  if (a.dtype == 0) {
-    switch (key) {
-      case 64064: return launch_cmp_select_t<bf16_t, 64, 64>(a, st);
-      case 128128: return launch_cmp_select_t<bf16_t, 128, 128>(a, st);
-      case 192128: return launch_cmp_select_t<bf16_t, 192, 128>(a, st);
-      default: return -2;
-    }
-  }
-  if (a.dtype == 2) {
-    switch (key) {
-      case 64064: return launch_cmp_select_t<f16_t, 64, 64>(a, st);
-      case 128128: return launch_cmp_select_t<f16_t, 128, 128>(a, st);
-      case 192128: return launch_cmp_select_t<f16_t, 192, 128>(a, st);
-      default: return -2;
-    }
-  }
-  return -2;
+template <typename T, int DK, int DV>
+static int launch_frag_pack_t(const CmpArgs& a, long cv_row_stride, long cv_head_stride, int rows_bound, hipStream_t st) {
+  const int tiles = rows_bound / 64 + a.batch;
+  hipLaunchKernelGGL((frag_pack_kernel<T, DK, DV>), dim3(tiles, a.hkv), dim3(256), 0, st,
+                     reinterpret_cast<const T*>(a.ck), reinterpret_cast<const T*>(a.cvt),
+                     reinterpret_cast<T*>(const_cast<void*>(a.frag)), a.cu_cmp, a.batch, a.ck_row_stride,
+                     a.ck_head_stride, cv_row_stride, cv_head_stride, a.frag_chunks);
+  return 0;
+}
+
+#define NSA_FUSED_DISPATCH(FN, ...)                                                   \
+  do {                                                                                \
+    const int key = a.dk * 1000 + a.dv;                                               \
+    if (a.dtype == 0) {                                                               \
+      switch (key) {                                                                  \
+        case 64064: return FN<bf16_t, 64, 64>(__VA_ARGS__);                           \
+        case 128128: return FN<bf16_t, 128, 128>(__VA_ARGS__);                        \
+        case 192128: return FN<bf16_t, 192, 128>(__VA_ARGS__);                        \
+        default: return -2;                                                           \
+      }                                                                               \
+    }                                                                                 \
+    if (a.dtype == 2) {                                                               \
+      switch (key) {                                                                  \
+        case 64064: return FN<f16_t, 64, 64>(__VA_ARGS__);                            \
+        case 128128: return FN<f16_t, 128, 128>(__VA_ARGS__);                         \
+        case 192128: return FN<f16_t, 192, 128>(__VA_ARGS__);                         \
+        default: return -2;                                                           \
+      }                                                                               \
+    }                                                                                 \
+    return -2;                                                                        \
+  } while (0)
+
+int launch_cmp_select(const CmpArgs& a, hipStream_t st) { NSA_FUSED_DISPATCH(launch_cmp_select_t, a, st); }
+
+// a.ck / a.cvt: the row-major compressed keys / VALUES (cv, not its transpose: rows at cv_row_stride, heads at
+// cv_head_stride), a.frag: the destination, a.frag_chunks: its chunk slots per head
+int launch_frag_pack(const CmpArgs& a, long cv_row_stride, long cv_head_stride, int rows_bound, hipStream_t st) {
+  NSA_FUSED_DISPATCH(launch_frag_pack_t, a, cv_row_stride, cv_head_stride, rows_bound, st);
 }
 
 }  // namespace nsa

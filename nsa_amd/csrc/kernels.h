@@ -43,6 +43,8 @@ struct CmpArgs {
   // optional: the gating Linear on q (weight [3][dk], bias [3] or null, in q's dtype) evaluated by the compressed-
   // attention kernel on the query fragments it holds anyway; gates [total][hq][3] receives the logits
   const void* gate_w = nullptr; const void* gate_b = nullptr; void* gates = nullptr;
+  // one-pass kernel only: the compressed keys and values in fragment order (cmp_select.hip) and its chunk slots per head
+  const void* frag = nullptr; int frag_chunks = 0;
 };
 
 struct SwaArgs {
@@ -163,6 +165,8 @@ int launch_select(const CmpArgs& a, hipStream_t st);
 // shape qualifies (max_nc = most compressed rows of any sequence), and the launch
 bool cmp_select_single_pass_ok(const CmpArgs& a, int max_nc);
 int launch_cmp_select(const CmpArgs& a, hipStream_t st);
+int cmp_frag_chunks(int total_rows, int batch);
+int launch_frag_pack(const CmpArgs& a, long cv_row_stride, long cv_head_stride, int rows_bound, hipStream_t st);
 int launch_swa(const SwaArgs& a, hipStream_t st);
 int launch_slc_combine(const SlcArgs& a, hipStream_t st);
 long slc_workspace_bytes(const SlcArgs& a);

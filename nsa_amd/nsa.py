@@ -48,6 +48,14 @@ class NSAAttention(nn.Module):
       v_head_dim       value head size when it differs from head_dim (e.g. 192 / 128)
     Unlike the reference, ragged `cu_seqlens` are honoured (each sequence is attended on its own)."""
 
+    # Fewest compressed rows (of the longest sequence) from which the one-pass kernel is taken when the shape
+    # qualifies.  0 = always: the kernel's fixed cost per token (scaling and adding the per-head window sums, the
+    # top-n) makes it a few per cent slower than the three launches on short sequences (T 8192: 0.37 against
+    # 0.35 ms; T 32768: 3.8 against 4.3 ms), but one schedule for every length keeps a packed batch bit-identical to
+    # its sequences run one by one (the two schedules add the window sums in different orders, so two nearly equal
+    # block scores may come out in the other order).
+    SINGLE_PASS_MIN_ROWS = 0
+
     def __init__(
         self,
         head_dim: int,
@@ -183,19 +191,37 @@ class NSAAttention(nn.Module):
             k, v, cu, seq_len=seq_len if uniform else None))
         max_nc = nc if nc is not None else conv_compressed_len(seq_len, self.compression_stride,
                                                                self.compression_block)
-        cvt, vt = stage("transpose", lambda: (ops.transpose(cv, cu_cmp, batch), ops.transpose(v, cu, batch)))
-        if gates is None:       # the gating Linear rides on the compressed-attention kernel's query fragments
-            o_cmp, lse, gates = stage("cmp_attn", lambda: ops.cmp_attn(
-                q, ck, cvt, cu, cu_cmp, batch, hkv, dv, ck.stride(0), ck.stride(1), self.compression_block,
-                self.compression_stride, scale, causal=bool(causal), gate_weight=self.gating.weight,
-                gate_bias=self.gating.bias))
+        one_pass = max_nc >= self.SINGLE_PASS_MIN_ROWS and ops.cmp_select_single_pass(
+            q, hkv, dv, self.pool_kernel_size, self.pool_stride, self.pool_padding, self.selected_block_count, max_nc)
+        if one_pass:    # the one-pass kernel streams ck / cv in fragment order; nobody reads the transposed cv
+            frag, vt = stage("transpose", lambda: (ops.cmp_pack(ck, cv, cu_cmp, batch), ops.transpose(v, cu, batch)))
         else:
-            o_cmp, lse = stage("cmp_attn", lambda: ops.cmp_attn(
-                q, ck, cvt, cu, cu_cmp, batch, hkv, dv, ck.stride(0), ck.stride(1), self.compression_block,
-                self.compression_stride, scale, causal=bool(causal)))
-        idx, _ = stage("block_select", lambda: ops.block_select(
-            q, ck, lse, cu, cu_cmp, batch, hkv, ck.stride(0), ck.stride(1), self.pool_kernel_size,
-            self.pool_stride, self.pool_padding, self.selected_block_count, max_nc, idx64=False))
+            cvt, vt = stage("transpose", lambda: (ops.transpose(cv, cu_cmp, batch), ops.transpose(v, cu, batch)))
+        own_gates = gates is None   # the gating Linear rides on the compressed-attention kernel's query fragments
+        if one_pass:
+            # one kernel, one pass over the compressed keys: attention, importance and top-n together
+            r = stage("cmp_select", lambda: ops.cmp_select(
+                q, ck, None, cu, cu_cmp, batch, hkv, dv, ck.stride(0), ck.stride(1), self.compression_block,
+                self.compression_stride, self.pool_kernel_size, self.pool_stride, self.pool_padding,
+                self.selected_block_count, max_nc, scale, causal=bool(causal),
+                gate_weight=self.gating.weight if own_gates else None,
+                gate_bias=self.gating.bias if own_gates else None, single_pass=True, frag=frag))
+            o_cmp, idx = r["o"], r["indices"]
+            if own_gates:
+                gates = r["gates"]
+        else:
+            if own_gates:
+                o_cmp, lse, gates = stage("cmp_attn", lambda: ops.cmp_attn(
+                    q, ck, cvt, cu, cu_cmp, batch, hkv, dv, ck.stride(0), ck.stride(1), self.compression_block,
+                    self.compression_stride, scale, causal=bool(causal), gate_weight=self.gating.weight,
+                    gate_bias=self.gating.bias))
+            else:
+                o_cmp, lse = stage("cmp_attn", lambda: ops.cmp_attn(
+                    q, ck, cvt, cu, cu_cmp, batch, hkv, dv, ck.stride(0), ck.stride(1), self.compression_block,
+                    self.compression_stride, scale, causal=bool(causal)))
+            idx, _ = stage("block_select", lambda: ops.block_select(
+                q, ck, lse, cu, cu_cmp, batch, hkv, ck.stride(0), ck.stride(1), self.pool_kernel_size,
+                self.pool_stride, self.pool_padding, self.selected_block_count, max_nc, idx64=False))
         g = gates.reshape(total * hq, 3)
         g_slc, g_swa, g_cmp = (g[:, i].view(total, hq) for i in range(3))
         act = _lib.GATE_SIGMOID if self.gate_activation == "sigmoid" else _lib.GATE_IDENTITY

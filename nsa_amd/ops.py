@@ -188,22 +188,44 @@ def cmp_select_single_pass(q, hkv, dv, pool_kernel, pool_stride, pool_pad, top_n
                                                        pool_pad, top_n, max_nc, _dtype_code(q)))
 
 
+def cmp_pack(ck, cv, cu_cmp, batch):
+    """ck [rows,H,Dk], cv [rows,H,Dv] (row-major, last dim contiguous) -> their fragment-major copy, which the
+    one-pass kernel of cmp_select streams: a flat tensor of H * chunks * 64 * (Dk + Dv) elements and `chunks`."""
+    _need_cuda(ck, cv, cu_cmp)
+    rows, h, dk = ck.shape
+    dv = cv.shape[2]
+    if ck.stride(2) != 1 or ck.data_ptr() % 16:
+        ck = _dense(ck)
+    if cv.stride(2) != 1 or cv.data_ptr() % 16:
+        cv = _dense(cv)
+    lib = _lib.load()
+    chunks = lib.nsa_cmp_pack_chunks(rows, batch)
+    frag = torch.empty(h * chunks * 64 * (dk + dv), dtype=ck.dtype, device=ck.device)
+    rc = lib.nsa_cmp_pack_fwd(_ptr(ck), _ptr(cv), _ptr(frag), _ptr(cu_cmp), batch, rows, h, dk, dv, ck.stride(0),
+                              ck.stride(1), cv.stride(0), cv.stride(1), chunks, _dtype_code(ck), _stream())
+    _lib.check(rc, "nsa_cmp_pack_fwd")
+    return frag, chunks
+
+
 def cmp_select(q, ck, cvt, cu_seqlens, cu_cmp, batch, hkv, dv, ck_row_stride, ck_head_stride, block, stride,
                pool_kernel, pool_stride, pool_pad, top_n, max_nc, scale, causal=True, idx64=False,
-               want_pooled=False, want_lse_attn=False, gate_weight=None, gate_bias=None, single_pass=None):
+               want_pooled=False, want_lse_attn=False, gate_weight=None, gate_bias=None, single_pass=None,
+               frag=None):
     """Compressed attention and block selection in one library call, as the reference's `_attention.forward`
     (nsa/triton_attention.py:419-476).  Returns a dict: o [total,Hq,dv], indices [total,hkv,top_n], and on request
     pooled [total,hkv,Ns], lse_attn [total,Hq] (what the backward reads), gates [total,Hq,3] (the gating Linear on q
     when gate_weight [3,Dk] is given).
-    single_pass: None = one kernel when the shape qualifies (cmp_select_single_pass), otherwise compressed
-    attention, window sums and top-n as three launches; False = always the latter; True = the one kernel or an error."""
-    _need_cuda(q, ck, cvt, cu_seqlens, cu_cmp)
+    single_pass: None = one kernel when the shape qualifies (cmp_select_single_pass) and `frag` is given, otherwise
+    compressed attention, window sums and top-n as three launches; False = always the latter; True = the one kernel
+    or an error.  frag: (tensor, chunks) from cmp_pack; cvt may be None when only the one kernel is to run."""
+    _need_cuda(q, ck, cu_seqlens, cu_cmp)
     q = _dense(q)
     total, hq, dk = q.shape
     lib = _lib.load()
     max_ns = pool_bins(max_nc, pool_kernel, pool_stride, pool_pad)
-    fused = single_pass is not False and cmp_select_single_pass(q, hkv, dv, pool_kernel, pool_stride, pool_pad,
-                                                                max(top_n, 1), max_nc)
+    fused = single_pass is not False and frag is not None and cmp_select_single_pass(
+        q, hkv, dv, pool_kernel, pool_stride, pool_pad, max(top_n, 1), max_nc)
+    frag_t, frag_chunks = frag if frag is not None else (None, 0)
     o = torch.empty(total, hq, dv, dtype=q.dtype, device=q.device)
     idx = torch.empty(total, hkv, top_n, dtype=torch.int64 if idx64 else torch.int32, device=q.device)
     lse_attn = torch.empty(total, hq, dtype=torch.float32, device=q.device) if want_lse_attn else None
@@ -220,9 +242,10 @@ def cmp_select(q, ck, cvt, cu_seqlens, cu_cmp, batch, hkv, dv, ck_row_stride, ck
         gates = torch.empty(total, hq, 3, dtype=q.dtype, device=q.device)
     mode = -1 if single_pass is None else int(bool(single_pass))
     rc = lib.nsa_cmp_select_fwd(
-        _ptr(q), _ptr(ck), _ptr(cvt), _ptr(o), _ptr(idx), _ptr(pooled), _ptr(lse), _ptr(lse_attn), _ptr(w), _ptr(b),
+        _ptr(q), _ptr(ck), _ptr(cvt), _ptr(frag_t), frag_chunks, _ptr(o), _ptr(idx), _ptr(pooled), _ptr(lse),
+        _ptr(lse_attn), _ptr(w), _ptr(b),
         _ptr(gates), _ptr(cu_seqlens), _ptr(cu_cmp), batch, total, hq, hkv, dk, dv, ck_row_stride, ck_head_stride,
-        cvt.shape[-1], block, stride, pool_kernel, pool_stride, pool_pad, max(top_n, 1), max_nc, max_ns, max(max_ns, 1),
+        cvt.shape[-1] if cvt is not None else 0, block, stride, pool_kernel, pool_stride, pool_pad, max(top_n, 1), max_nc, max_ns, max(max_ns, 1),
         int(bool(want_pooled)), float(scale), int(bool(causal)), int(idx64), _dtype_code(q), mode, _stream())
     _lib.check(rc, "nsa_cmp_select_fwd")
     return dict(o=o, indices=idx, pooled=pooled[:, :, 0] if want_pooled else None, lse_attn=lse_attn, gates=gates,

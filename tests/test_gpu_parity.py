@@ -151,7 +151,8 @@ def _cmp_case(dtype, lens, Hq, Hkv, Dk, Dv, l, d, lsel, S, seed, scale_in=1.0, l
     # compressed keys, window sums kept per head in registers), everything else as the three launches above
     r = ops.cmp_select(q.to(DEV), ck, cvt, cu, cu_cmp, len(lens), Hkv, Dv, ck.stride(0), ck.stride(1), l, d,
                        p.pool_kernel, p.pool_stride, p.pool_pad, S, max(ncs), scale, idx64=True, want_pooled=True,
-                       want_lse_attn=True)
+                       want_lse_attn=True, frag=ops.cmp_pack(ck, cv, cu_cmp, len(lens)) if dtype != torch.float32 and
+                       (Dk, Dv) in ((64, 64), (128, 128), (192, 128)) else None)
     torch.cuda.synchronize()
     if r["single_pass"]:
         w2 = _cmp_check(dtype, lens, ncs, q, ck, cv, r["o"].cpu(), r["indices"].cpu(), r["pooled"].cpu(), p, l, d, S,

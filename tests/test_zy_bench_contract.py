@@ -35,3 +35,13 @@ def test_bench_json_line():
     assert rf["achieved"] > 0 and abs(rf["frac"] - rf["achieved"] / rf["peak"]) < 1e-9
     cb = d["cpu_baseline"]
     assert cb["kind"] in ("port", "reference") and cb["value"] > 0 and cb["cores"] >= 1 and cb["sample"]
+    # the contracted CPU figure (whole sequence of benchmark configuration 1) next to the sampled one
+    c1 = d["cpu_baseline_cfg1"]
+    assert c1["kind"] == "port" and c1["value"] > 0 and c1["cores"] >= 1 and "configuration 1" in c1["sample"]
+    # the HBM-bound stages and the executed (not only credited) matrix rate of the whole step
+    assert d["executed_tflops_whole_step"] >= d["effective_tflops"]
+    for name, r in d["roofline_hbm"].items():
+        assert r["bound"] == "hbm" and r["unit"] == "GB/s" and r["peak"] == 8000.0 and r["traffic_source"]
+        assert (r["traffic"] is None) == (r["achieved"] is None)
+        if r["achieved"] is not None:
+            assert 0 < r["frac"] <= 1.0
