@@ -27,6 +27,7 @@
 // rows go to a lane-private column of LDS (8 KB per wavefront): 128 more registers would not leave room for the
 // query fragments and the output accumulators of a 192-wide head at two wavefronts per SIMD.
 #include <type_traits>
+#include <utility>
 
 #include "tiles.h"
 
@@ -35,6 +36,18 @@ namespace nsa {
 typedef float f32x32_t __attribute__((ext_vector_type(32)));
 
 int set_smem(const void* fn, size_t bytes);
+
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>), in order
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+// keeps a value (and the instruction that made it) at this point of the program
+__device__ __forceinline__ void pin(float& x) { asm volatile("" : "+v"(x)); }
 
 // ------------------------------------------------------------------------------------------------
 // Fragment-major copy of the compressed keys and values.
@@ -50,14 +63,20 @@ int set_smem(const void* fn, size_t bytes);
 //   V fragment (s, tv),    lane (m, g):  V[32 s + 8 g .. + 7][16 tv + m]   (8 rows of one channel)
 // Chunk c of sequence b of kv head h sits at chunk slot cu_cmp[b] / 64 + b + c of that head (slots of different
 // sequences never overlap; at most total_rows / 64 + batch + 1 slots).  Rows past the sequence's last one are zero.
-typedef __attribute__((address_space(3))) void* lds_void_ptr;
-typedef __attribute__((address_space(1))) const void* global_void_ptr;
-
 // 16 bytes per lane from global memory straight into LDS: lane i's piece lands at lds + 16 i bytes (lds is the same
 // for the whole wavefront).  Counts as a vector-memory load of the wavefront until the data is in LDS.
+// Written as assembly on purpose: the compiler books the built-in form as an access that may touch both memories,
+// and from then on answers every wait for an LDS read with "wait for all of them" -- which undoes a ring of
+// fragment reads in flight.  The callers wait for these loads themselves (s_waitcnt vmcnt(0) before the barrier
+// that publishes the chunk).  m0 is not named as clobbered: the compiler reserves it and sets it anew before every
+// use of its own (register indexing), never across a statement.
+__device__ __forceinline__ unsigned lds_address(const void* p) {
+  return (unsigned)(uintptr_t)((__attribute__((address_space(3))) const char*)p);
+}
 template <typename T>
 __device__ __forceinline__ void global_to_lds16(const T* src, T* lds) {
-  __builtin_amdgcn_global_load_lds((global_void_ptr)src, (lds_void_ptr)lds, 16, 0, 0);
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+               :: "v"(src), "s"(lds_address(lds)) : "memory");
 }
 
 __host__ __device__ __forceinline__ int frag_chunk_slot(int cu_b, int b) { return (cu_b >> 6) + b; }
@@ -257,7 +276,7 @@ cmp_select_kernel(const CmpArgs a) {
   const float c_attn = a.scale * kLog2e;
 
   // staging: the load unit copies the chunk, 1 KB per wavefront instruction; wavefront w takes blocks w, w + 8, ..
-  auto stage_chunk = [&](int c0, int buf, bool with_v) {
+  auto stage_chunk = [&](int c0, int buf, bool with_v) __attribute__((always_inline)) {
     const T* src = fragb + (long)(c0 >> 6) * CHUNK + lane * 8;
     T* dst = ldsC + buf * CHUNK;
 #pragma unroll
@@ -293,7 +312,7 @@ cmp_select_kernel(const CmpArgs a) {
   wait_all_loads();
 
   // raw scores of one 32-row step: value i of lane (n, g) = row 8g + i of the step, head n
-  auto scores = [&](const T* kf, float (&s)[8]) {
+  auto scores = [&](const T* kf, float (&s)[8]) __attribute__((always_inline)) {
     f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int kk = 0; kk < NKK; ++kk) {
@@ -304,72 +323,214 @@ cmp_select_kernel(const CmpArgs a) {
     for (int i = 0; i < 4; ++i) { s[i] = s0[i]; s[4 + i] = s1[i]; }
   };
 
-  // One 32-row step.  derive: the first step sets the references.  kf / vf: the step's fragments (this lane's piece)
-  auto step32 = [&](auto put, int slot, int cb, const T* kf, const T* vf, bool derive) {
-    float s[8];
-    scores(kf, s);
-    const int key0 = cb + 8 * g;
-    if (cb + 32 > nkeys) {                           // last step of the sequence only
-      asm volatile("" ::: "memory");
-#pragma unroll
-      for (int i = 0; i < 8; ++i)
-        if (key0 + i >= nkeys) s[i] = kNegInf;
-    }
-    if (derive && cb == 0) {                         // the reference: largest score of the first 32 rows
-      float mx = s[0];
-#pragma unroll
-      for (int i = 1; i < 8; ++i) mx = fmaxf(mx, s[i]);
-      m_i = m_a = colgroup_max(mx);                  // finite: row 0 exists
-      off_i = -m_i * kLog2e;
-      off_a = -m_a * c_attn;
-    }
-    float e[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) e[i] = fast_exp2(fmaf(s[i], kLog2e, off_i));
-    const float qa = (e[0] + e[1]) + (e[2] + e[3]), qb = (e[4] + e[5]) + (e[6] + e[7]);
-    li += qa + qb;
-    // e[0] (row 8g) completes the upper window of the lane row before, e[4] this lane's lower window
-    const float nxt = __int_as_float(__builtin_amdgcn_ds_bpermute(next_lane, __float_as_int(e[0])));
-    put(slot, qa + e[4], (last_row ? pend : qb) + nxt);
-    pend = qb;
-    if (cb <= hi) {                                  // the token attends rows of this step
-      float p[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) p[i] = fast_exp2(fmaf(s[i], c_attn, off_a));
-      if (cb + 31 > hi) {                            // the step on the causal edge
-        asm volatile("" ::: "memory");
-#pragma unroll
-        for (int i = 0; i < 8; ++i)
-          if (key0 + i > hi) p[i] = 0.f;
-      }
-      const float p8 = sum8(p);
-      grp[0].l += p8;
-      if constexpr (kNarrowP) pmax = fmaxf(pmax, p8);
-      const vec8_t<T> pb = pack8<T>(p);
-#pragma unroll
-      for (int t = 0; t < NV; ++t) grp[0].o[t] = mma16(load8(vf + t * 512), pb, grp[0].o[t]);
+  // ---- a chunk = two steps a, b; the common chunks are software-pipelined by hand
+  // A wavefront that runs "scores, softmax, P V" one after the other leaves the matrix unit idle during its vector
+  // work, and its SIMD partner, released by the same barrier, is in the same phase.  A chunk whose two steps are
+  // both fully visible (or both hidden) therefore runs as one fixed schedule of matrix instructions with the
+  // vector work of OTHER steps dealt out between them:
+  //   visible:  QK(a) | B(prev b)    QK(b) | A(a)    PV(a) | A(b)    PV(b) | B(a)
+  //   hidden:   QK(a) | B(prev b)    QK(b) | B(a)
+  // A(x) = attention probabilities of step x (8 exponentials, their sum, the packed operand of PV(x)), B(x) = the
+  // importance side (8 exponentials, the step's two window sums).  B of a chunk's second step is carried into the
+  // next chunk.  Fragments come from LDS through a ring of 4 register sets, requested 3 matrix instructions ahead.
+  // The visible schedule takes any chunk: the first one (its step a sets the references), the one on the causal edge
+  // and a tail chunk switch its masks on.  Either schedule ends with the same four values -- the window sums of the
+  // carried step and of step a -- and the register block of the section is written at ONE place behind the two
+  // bodies: two bodies that each wrote it would meet in a merge that costs a copy of the 32-register block.
+  constexpr int NQ = 2 * NKK;                      // matrix instructions of one step's scores
+  float cs[8];                                     // carried: scores of the previous chunk's second step ...
+  int cslot = -1;                                  // ... and its slot (-1: nothing carried)
+  bool creal = false;                              // ... and whether that step has rows at all
+  float bt[4], bnxt;                               // B's temporaries
+  float e_[8];
+  // real = false: a stand-in for a carried step that does not exist (scores -inf: every exponential 0); its zeros go
+  // to slots that the chunk's own first step overwrites right after, and it must leave `pend` alone
+  auto opB = [&](auto I, const float (&s)[8], float& w0, float& w1, bool real) __attribute__((always_inline)) {   // 17 operations
+    constexpr int i = decltype(I)::value;
+    if constexpr (i == 0) { e_[0] = fast_exp2(fmaf(s[0], kLog2e, off_i)); pin(e_[0]); }
+    else if constexpr (i == 1) { bnxt = __int_as_float(__builtin_amdgcn_ds_bpermute(next_lane, __float_as_int(e_[0]))); }
+    else if constexpr (i < 9) { e_[i - 1] = fast_exp2(fmaf(s[i - 1], kLog2e, off_i)); pin(e_[i - 1]); }
+    else if constexpr (i < 13) { bt[i - 9] = e_[2 * (i - 9)] + e_[2 * (i - 9) + 1]; pin(bt[i - 9]); }
+    else if constexpr (i == 13) { bt[0] += bt[1]; pin(bt[0]); }                       // lower quad
+    else if constexpr (i == 14) { bt[2] += bt[3]; pin(bt[2]); }                       // upper quad
+    else if constexpr (i == 15) { li += bt[0] + bt[2]; pin(li); }
+    else {
+      // e_[0] (row 8g) completes the upper window of the lane row before, e_[4] this lane's lower window
+      w0 = bt[0] + e_[4];
+      w1 = (last_row ? pend : bt[2]) + bnxt;
+      pend = real ? bt[2] : pend;
     }
   };
+  auto stepB = [&](const float (&s)[8], float& w0, float& w1, bool real) __attribute__((always_inline)) {
+    static_for<17>([&](auto O) { opB(O, s, w0, w1, real); });
+  };
+  float pt[4], p_[8];
+  // cb: first row of the step; edge: some of its rows are past the last one the token attends (their probability is 0)
+  auto opA = [&](auto I, const float (&s)[8], vec8_t<T>& pb, int cb, bool edge) __attribute__((always_inline)) {   // 17 operations
+    constexpr int i = decltype(I)::value;
+    if constexpr (i < 8) { p_[i] = fast_exp2(fmaf(s[i], c_attn, off_a)); pin(p_[i]); }
+    else if constexpr (i == 8) {
+      if (edge) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+          if (cb + 8 * g + k > hi) p_[k] = 0.f;
+      }
+    }
+    else if constexpr (i < 13) { pt[i - 9] = p_[2 * (i - 9)] + p_[2 * (i - 9) + 1]; pin(pt[i - 9]); }
+    else if constexpr (i == 13) { pt[0] += pt[1]; pin(pt[0]); }
+    else if constexpr (i == 14) { pt[2] += pt[3]; pin(pt[2]); }
+    else if constexpr (i == 15) {
+      const float p8 = pt[0] + pt[2];
+      grp[0].l += p8;
+      if constexpr (kNarrowP) pmax = fmaxf(pmax, p8);
+    } else { pb = pack8<T>(p_); }
+  };
+  // element offset of the fragment that matrix instruction J of a chunk reads (from this lane's piece of the chunk)
+  auto frag_off = [](int J) constexpr -> int {
+    if (J < 2 * NQ) { const int st = J / NQ, j = J % NQ; return (st * NQ + (j & 1) * NKK + (j >> 1)) * 512; }
+    return KPART + (J - 2 * NQ) * 512;             // PV(a): channel tiles 0 .. NV-1, PV(b): NV .. 2 NV-1
+  };
+  // VIS = true: the token attends rows of the chunk (any chunk may take this body: rows past the sequence end or past
+  // the token's last visible row are masked where the flags say so); false: a whole chunk the token does not attend.
+  // Out: the window sums of the carried step (wc) and of step a (wa); the scores of step b replace the carried ones.
+  auto chunk_piped = [&](auto vis_tag, const T* cf, int c0, bool carried, bool derive, float (&wc)[2], float (&wa)[2]) __attribute__((always_inline)) {
+    constexpr bool VIS = decltype(vis_tag)::value;
+    constexpr int NM = VIS ? 2 * NQ + 2 * NV : 2 * NQ, PF = 3;
+    const bool tail_a = VIS && c0 + 32 > nkeys, tail_b = VIS && c0 + 64 > nkeys;      // rows past the sequence end
+    const bool edge_a = c0 + 31 > hi, edge_b = c0 + 63 > hi;                          // rows past the causal limit
+    vec8_t<T> ring[4];
+    f32x4_t a0 = {0.f, 0.f, 0.f, 0.f}, a1 = a0, b0 = a0, b1 = a0;
+    float sa[8], sb[8];
+    vec8_t<T> pa, pbb;
+    static_for<PF>([&](auto J) { ring[J] = load8(cf + frag_off(J)); });
+    static_for<NM>([&](auto Jc) {
+      constexpr int J = decltype(Jc)::value;
+      if constexpr (J + PF < NM) ring[(J + PF) & 3] = load8(cf + frag_off(J + PF));
+      // the matrix instruction
+      if constexpr (J < NQ) {
+        if constexpr ((J & 1) == 0) a0 = mma16(ring[J & 3], grp[0].q[J >> 1], a0);
+        else a1 = mma16(ring[J & 3], grp[0].q[J >> 1], a1);
+      } else if constexpr (J < 2 * NQ) {
+        if constexpr ((J & 1) == 0) b0 = mma16(ring[J & 3], grp[0].q[(J - NQ) >> 1], b0);
+        else b1 = mma16(ring[J & 3], grp[0].q[(J - NQ) >> 1], b1);
+      } else if constexpr (J < 2 * NQ + NV) {
+        grp[0].o[J - 2 * NQ] = mma16(ring[J & 3], pa, grp[0].o[J - 2 * NQ]);
+      } else {
+        grp[0].o[J - 2 * NQ - NV] = mma16(ring[J & 3], pbb, grp[0].o[J - 2 * NQ - NV]);
+      }
+      // the scores of a step leave the accumulators right after its last matrix instruction
+      if constexpr (J == NQ - 1) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { sa[i] = a0[i]; sa[4 + i] = a1[i]; }
+        if constexpr (VIS) {
+          if (tail_a) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+              if (c0 + 8 * g + i >= nkeys) sa[i] = kNegInf;
+          }
+          if (derive && c0 == 0) {                   // the reference: largest score of the first 32 rows
+            float mx = sa[0];
+#pragma unroll
+            for (int i = 1; i < 8; ++i) mx = fmaxf(mx, sa[i]);
+            m_i = m_a = colgroup_max(mx);            // finite: row 0 exists
+            off_i = -m_i * kLog2e;
+            off_a = -m_a * c_attn;
+          }
+        }
+      }
+      if constexpr (J == 2 * NQ - 1) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { sb[i] = b0[i]; sb[4 + i] = b1[i]; }
+        if constexpr (VIS) {
+          if (tail_b) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+              if (c0 + 32 + 8 * g + i >= nkeys) sb[i] = kNegInf;
+          }
+        }
+      }
+      // this slot's share of the vector work
+      if constexpr (J < NQ) {                                    // B(carried step)
+        static_for<17>([&](auto O) {
+          constexpr int o = decltype(O)::value;
+          if constexpr (o >= J * 17 / NQ && o < (J + 1) * 17 / NQ) opB(O, cs, wc[0], wc[1], carried);
+        });
+      } else if constexpr (J < 2 * NQ) {                         // A(a) resp. B(a)
+        constexpr int K = J - NQ;
+        if constexpr (VIS) static_for<17>([&](auto O) {
+          constexpr int o = decltype(O)::value;
+          if constexpr (o >= K * 17 / NQ && o < (K + 1) * 17 / NQ) opA(O, sa, pa, c0, edge_a);
+        });
+        else static_for<17>([&](auto O) {
+          constexpr int o = decltype(O)::value;
+          if constexpr (o >= K * 17 / NQ && o < (K + 1) * 17 / NQ) opB(O, sa, wa[0], wa[1], true);
+        });
+      } else if constexpr (J < 2 * NQ + NV) {                    // A(b)
+        constexpr int K = J - 2 * NQ;
+        static_for<17>([&](auto O) {
+          constexpr int o = decltype(O)::value;
+          if constexpr (o >= K * 17 / NV && o < (K + 1) * 17 / NV) opA(O, sb, pbb, c0 + 32, edge_b);
+        });
+      } else {                                                   // B(a)
+        constexpr int K = J - 2 * NQ - NV;
+        static_for<17>([&](auto O) {
+          constexpr int o = decltype(O)::value;
+          if constexpr (o >= K * 17 / NV && o < (K + 1) * 17 / NV) opB(O, sa, wa[0], wa[1], true);
+        });
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
+#pragma unroll
+    for (int i = 0; i < 8; ++i) cs[i] = sb[i];
+  };
 
-  auto run_pass = [&](bool derive) {
-    if (c_end > 0) stage_chunk(0, 0, 0 <= attn_end);
+  auto run_pass = [&](bool derive) __attribute__((always_inline)) {
+    if (c_end > 0) stage_chunk(0, 0, true);        // the first chunk always runs the visible schedule
     staged();
     int buf = 0;
+    cslot = -1;
     // 512 rows = 16 steps = 32 slots per section: inside a section the slots of one register block are written
     // in place with a scalar index
-    auto section = [&](auto put, int c_first) {
+    auto section = [&](auto put, int c_first) __attribute__((always_inline)) {
       const int c_stop = min(c_first + 512, c_end);
       for (int c0 = c_first; c0 < c_stop; c0 += 64) {
         const int cn = c0 + 64;
-        if (cn < c_end) stage_chunk(cn, buf ^ 1, cn <= attn_end);
+        // values only where a wavefront runs the visible schedule: chunks some token attends, and a tail chunk
+        if (cn < c_end) stage_chunk(cn, buf ^ 1, cn <= attn_end || cn + 64 > nkeys);
         const T* kf = ldsC + buf * CHUNK + lane * 8;
-        const T* vf = kf + KPART;
         const int slot = (c0 - c_first) >> 4;
-        step32(put, slot, c0, kf, vf, derive);
-        if (c0 + 32 < c_end) step32(put, slot + 2, c0 + 32, kf + 2 * NKK * 512, vf + NV * 512, derive);
+        // nothing carried (first chunk of a section, or after a chunk of one step): a stand-in that writes zeros
+        // to this chunk's first two slots, which the chunk's step a overwrites below
+        const int slot_c = cslot >= 0 ? cslot : slot;
+        const bool carried = cslot >= 0 && creal;
+        if (cslot < 0) {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) cs[i] = kNegInf;
+        }
+        float wc[2], wa[2];
+        if (c0 > hi && c0 > 0 && cn <= nkeys) chunk_piped(std::false_type{}, kf, c0, carried, derive, wc, wa);
+        else chunk_piped(std::true_type{}, kf, c0, carried, derive, wc, wa);
+        // step b is carried; in a chunk of one step it is rows past the end (scores -inf, sums 0) and only its
+        // zeros are written -- `pend` must keep the last real step's quad
+        cslot = slot + 2;
+        creal = c0 + 32 < c_end;
+        put(slot_c, wc[0], wc[1]);
+        put(slot, wa[0], wa[1]);
         staged();
         buf ^= 1;
       }
+      // The step carried out of the section's last chunk belongs to this section's slots.  Nothing carried (the
+      // sequence ends before this section): zeros into slot 0 of a section that no window uses.
+      const bool carried = cslot >= 0 && creal;
+      const int slot_c = cslot >= 0 ? cslot : 0;
+      if (cslot < 0) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) cs[i] = kNegInf;
+      }
+      float wc[2];
+      stepB(cs, wc[0], wc[1], carried);
+      put(slot_c, wc[0], wc[1]);
+      cslot = -1;
     };
     section([&](int s, float x0, float x1) { bq0[s] = x0; bq0[s + 1] = x1; }, 0);
     section([&](int s, float x0, float x1) { bq1[s] = x0; bq1[s + 1] = x1; }, 512);
