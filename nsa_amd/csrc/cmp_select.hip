@@ -338,6 +338,7 @@ cmp_select_kernel(const CmpArgs a) {
   // carried step and of step a -- and the register block of the section is written at ONE place behind the two
   // bodies: two bodies that each wrote it would meet in a merge that costs a copy of the 32-register block.
   constexpr int NQ = 2 * NKK;                      // matrix instructions of one step's scores
+  constexpr int kOpsA = 25, kOpsB = 25;            // vector operations of A(x) / B(x)
   float cs[8];                                     // carried: scores of the previous chunk's second step ...
   int cslot = -1;                                  // ... and its slot (-1: nothing carried)
   bool creal = false;                              // ... and whether that step has rows at all
@@ -345,15 +346,16 @@ cmp_select_kernel(const CmpArgs a) {
   float e_[8];
   // real = false: a stand-in for a carried step that does not exist (scores -inf: every exponential 0); its zeros go
   // to slots that the chunk's own first step overwrites right after, and it must leave `pend` alone
-  auto opB = [&](auto I, const float (&s)[8], float& w0, float& w1, bool real) __attribute__((always_inline)) {   // 17 operations
+  auto opB = [&](auto I, const float (&s)[8], float& w0, float& w1, bool real) __attribute__((always_inline)) {   // kOpsB operations
     constexpr int i = decltype(I)::value;
-    if constexpr (i == 0) { e_[0] = fast_exp2(fmaf(s[0], kLog2e, off_i)); pin(e_[0]); }
-    else if constexpr (i == 1) { bnxt = __int_as_float(__builtin_amdgcn_ds_bpermute(next_lane, __float_as_int(e_[0]))); }
-    else if constexpr (i < 9) { e_[i - 1] = fast_exp2(fmaf(s[i - 1], kLog2e, off_i)); pin(e_[i - 1]); }
-    else if constexpr (i < 13) { bt[i - 9] = e_[2 * (i - 9)] + e_[2 * (i - 9) + 1]; pin(bt[i - 9]); }
-    else if constexpr (i == 13) { bt[0] += bt[1]; pin(bt[0]); }                       // lower quad
-    else if constexpr (i == 14) { bt[2] += bt[3]; pin(bt[2]); }                       // upper quad
-    else if constexpr (i == 15) { li += bt[0] + bt[2]; pin(li); }
+    // the multiply-adds first, the exponentials after them: neighbours in the instruction stream are independent
+    if constexpr (i < 8) { e_[i] = fmaf(s[i], kLog2e, off_i); pin(e_[i]); }
+    else if constexpr (i < 16) { e_[i - 8] = fast_exp2(e_[i - 8]); pin(e_[i - 8]); }
+    else if constexpr (i == 16) { bnxt = __int_as_float(__builtin_amdgcn_ds_bpermute(next_lane, __float_as_int(e_[0]))); }
+    else if constexpr (i < 21) { bt[i - 17] = e_[2 * (i - 17)] + e_[2 * (i - 17) + 1]; pin(bt[i - 17]); }
+    else if constexpr (i == 21) { bt[0] += bt[1]; pin(bt[0]); }                       // lower quad
+    else if constexpr (i == 22) { bt[2] += bt[3]; pin(bt[2]); }                       // upper quad
+    else if constexpr (i == 23) { li += bt[0] + bt[2]; pin(li); }
     else {
       // e_[0] (row 8g) completes the upper window of the lane row before, e_[4] this lane's lower window
       w0 = bt[0] + e_[4];
@@ -362,24 +364,25 @@ cmp_select_kernel(const CmpArgs a) {
     }
   };
   auto stepB = [&](const float (&s)[8], float& w0, float& w1, bool real) __attribute__((always_inline)) {
-    static_for<17>([&](auto O) { opB(O, s, w0, w1, real); });
+    static_for<kOpsB>([&](auto O) { opB(O, s, w0, w1, real); });
   };
   float pt[4], p_[8];
   // cb: first row of the step; edge: some of its rows are past the last one the token attends (their probability is 0)
-  auto opA = [&](auto I, const float (&s)[8], vec8_t<T>& pb, int cb, bool edge) __attribute__((always_inline)) {   // 17 operations
+  auto opA = [&](auto I, const float (&s)[8], vec8_t<T>& pb, int cb, bool edge) __attribute__((always_inline)) {   // kOpsA operations
     constexpr int i = decltype(I)::value;
-    if constexpr (i < 8) { p_[i] = fast_exp2(fmaf(s[i], c_attn, off_a)); pin(p_[i]); }
-    else if constexpr (i == 8) {
+    if constexpr (i < 8) { p_[i] = fmaf(s[i], c_attn, off_a); pin(p_[i]); }
+    else if constexpr (i < 16) { p_[i - 8] = fast_exp2(p_[i - 8]); pin(p_[i - 8]); }
+    else if constexpr (i == 16) {
       if (edge) {
 #pragma unroll
         for (int k = 0; k < 8; ++k)
           if (cb + 8 * g + k > hi) p_[k] = 0.f;
       }
     }
-    else if constexpr (i < 13) { pt[i - 9] = p_[2 * (i - 9)] + p_[2 * (i - 9) + 1]; pin(pt[i - 9]); }
-    else if constexpr (i == 13) { pt[0] += pt[1]; pin(pt[0]); }
-    else if constexpr (i == 14) { pt[2] += pt[3]; pin(pt[2]); }
-    else if constexpr (i == 15) {
+    else if constexpr (i < 21) { pt[i - 17] = p_[2 * (i - 17)] + p_[2 * (i - 17) + 1]; pin(pt[i - 17]); }
+    else if constexpr (i == 21) { pt[0] += pt[1]; pin(pt[0]); }
+    else if constexpr (i == 22) { pt[2] += pt[3]; pin(pt[2]); }
+    else if constexpr (i == 23) {
       const float p8 = pt[0] + pt[2];
       grp[0].l += p8;
       if constexpr (kNarrowP) pmax = fmaxf(pmax, p8);
@@ -451,31 +454,31 @@ cmp_select_kernel(const CmpArgs a) {
       }
       // this slot's share of the vector work
       if constexpr (J < NQ) {                                    // B(carried step)
-        static_for<17>([&](auto O) {
+        static_for<kOpsB>([&](auto O) {
           constexpr int o = decltype(O)::value;
-          if constexpr (o >= J * 17 / NQ && o < (J + 1) * 17 / NQ) opB(O, cs, wc[0], wc[1], carried);
+          if constexpr (o >= J * kOpsB / NQ && o < (J + 1) * kOpsB / NQ) opB(O, cs, wc[0], wc[1], carried);
         });
       } else if constexpr (J < 2 * NQ) {                         // A(a) resp. B(a)
         constexpr int K = J - NQ;
-        if constexpr (VIS) static_for<17>([&](auto O) {
+        if constexpr (VIS) static_for<kOpsA>([&](auto O) {
           constexpr int o = decltype(O)::value;
-          if constexpr (o >= K * 17 / NQ && o < (K + 1) * 17 / NQ) opA(O, sa, pa, c0, edge_a);
+          if constexpr (o >= K * kOpsA / NQ && o < (K + 1) * kOpsA / NQ) opA(O, sa, pa, c0, edge_a);
         });
-        else static_for<17>([&](auto O) {
+        else static_for<kOpsB>([&](auto O) {
           constexpr int o = decltype(O)::value;
-          if constexpr (o >= K * 17 / NQ && o < (K + 1) * 17 / NQ) opB(O, sa, wa[0], wa[1], true);
+          if constexpr (o >= K * kOpsB / NQ && o < (K + 1) * kOpsB / NQ) opB(O, sa, wa[0], wa[1], true);
         });
       } else if constexpr (J < 2 * NQ + NV) {                    // A(b)
         constexpr int K = J - 2 * NQ;
-        static_for<17>([&](auto O) {
+        static_for<kOpsA>([&](auto O) {
           constexpr int o = decltype(O)::value;
-          if constexpr (o >= K * 17 / NV && o < (K + 1) * 17 / NV) opA(O, sb, pbb, c0 + 32, edge_b);
+          if constexpr (o >= K * kOpsA / NV && o < (K + 1) * kOpsA / NV) opA(O, sb, pbb, c0 + 32, edge_b);
         });
       } else {                                                   // B(a)
         constexpr int K = J - 2 * NQ - NV;
-        static_for<17>([&](auto O) {
+        static_for<kOpsB>([&](auto O) {
           constexpr int o = decltype(O)::value;
-          if constexpr (o >= K * 17 / NV && o < (K + 1) * 17 / NV) opB(O, sa, wa[0], wa[1], true);
+          if constexpr (o >= K * kOpsB / NV && o < (K + 1) * kOpsB / NV) opB(O, sa, wa[0], wa[1], true);
         });
       }
       __builtin_amdgcn_sched_barrier(0);
