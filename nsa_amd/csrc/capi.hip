@@ -84,7 +84,15 @@ int nsa_compress_kv_fwd(const void* k, const void* v, const void* wk_t, const vo
   if (!k || !v || !ck || !cv) return fail(NSA_ERR_INVALID, "compress_kv: null pointer");
   if ((wk_t == nullptr) != (wv_t == nullptr))
     return fail(NSA_ERR_INVALID, "compress_kv: give both weights or neither");
-  if (wk_t) {                                   // learned compressor: one GEMM launch per tensor
+  if (wk_t && dtype != NSA_F32 && cu_seqlens && cu_out && batch > 0 && heads > 0 && block > 0 && stride > 0 &&
+      out_rows_bound >= 0 && aligned16(k) && aligned16(v) && aligned16(ck) && aligned16(cv) && aligned16(wk_t) &&
+      aligned16(wv_t)) {                        // learned compressor, 16-bit: both GEMMs in one launch
+    nsa::CompressArgs a{k, wk_t, bk, ck, cu_seqlens, cu_out, batch, out_rows_bound, heads, dk, block, stride, dtype};
+    a.x2 = v; a.out2 = cv; a.dim2 = dv; a.wt2 = wv_t; a.bias2 = bv;
+    const int rc = nsa::launch_compress(a, stream);
+    if (rc != -7) return finish(rc, "compress_kv");
+  }
+  if (wk_t) {                                   // otherwise one GEMM launch per tensor
     const int rc = nsa_compress_fwd(k, wk_t, bk, ck, cu_seqlens, cu_out, batch, out_rows_bound, heads, dk, block,
                                     stride, dtype, stream);
     if (rc != NSA_OK) return rc;

@@ -124,6 +124,9 @@ frag_pack_kernel(const T* __restrict__ ck, const T* __restrict__ cv, T* __restri
   }
 }
 
+#ifndef NSA_FUSED_GS
+#define NSA_FUSED_GS 2
+#endif
 constexpr int kFusedMaxRows = 2048;      // compressed rows per sequence the window sums have room for
 
 // Top-n over the PER candidates every lane holds (score v[k] >= 0 with window number ix[k]; -1 = no candidate),
@@ -332,7 +335,7 @@ cmp_select_kernel(const CmpArgs a) {
   //   hidden:   QK(a) | B(prev b)    QK(b) | B(a)
   // A(x) = attention probabilities of step x (8 exponentials, their sum, the packed operand of PV(x)), B(x) = the
   // importance side (8 exponentials, the step's two window sums).  B of a chunk's second step is carried into the
-  // next chunk.  Fragments come from LDS through a ring of 4 register sets, requested 3 matrix instructions ahead.
+  // next chunk.  Fragments come from LDS through a ring of 4 register sets, requested in pairs two matrix instructions ahead.
   // The visible schedule takes any chunk: the first one (its step a sets the references), the one on the causal edge
   // and a tail chunk switch its masks on.  Either schedule ends with the same four values -- the window sums of the
   // carried step and of step a -- and the register block of the section is written at ONE place behind the two
@@ -398,28 +401,34 @@ cmp_select_kernel(const CmpArgs a) {
   // Out: the window sums of the carried step (wc) and of step a (wa); the scores of step b replace the carried ones.
   auto chunk_piped = [&](auto vis_tag, const T* cf, int c0, bool carried, bool derive, float (&wc)[2], float (&wa)[2]) __attribute__((always_inline)) {
     constexpr bool VIS = decltype(vis_tag)::value;
-    constexpr int NM = VIS ? 2 * NQ + 2 * NV : 2 * NQ, PF = 3;
+    constexpr int NM = VIS ? 2 * NQ + 2 * NV : 2 * NQ, GS = NSA_FUSED_GS;
     const bool tail_a = VIS && c0 + 32 > nkeys, tail_b = VIS && c0 + 64 > nkeys;      // rows past the sequence end
     const bool edge_a = c0 + 31 > hi, edge_b = c0 + 63 > hi;                          // rows past the causal limit
-    vec8_t<T> ring[4];
+    vec8_t<T> ring[2 * GS];
     f32x4_t a0 = {0.f, 0.f, 0.f, 0.f}, a1 = a0, b0 = a0, b1 = a0;
     float sa[8], sb[8];
     vec8_t<T> pa, pbb;
-    static_for<PF>([&](auto J) { ring[J] = load8(cf + frag_off(J)); });
+    // fragments are requested GS at a time, GS matrix instructions ahead: one wait per group
+    static_for<GS>([&](auto J) { ring[J] = load8(cf + frag_off(J)); });
     static_for<NM>([&](auto Jc) {
       constexpr int J = decltype(Jc)::value;
-      if constexpr (J + PF < NM) ring[(J + PF) & 3] = load8(cf + frag_off(J + PF));
+      if constexpr (J % GS == 0) {
+        static_for<GS>([&](auto Kc) {
+          constexpr int F = J + GS + decltype(Kc)::value;
+          if constexpr (F < NM) ring[F % (2 * GS)] = load8(cf + frag_off(F));
+        });
+      }
       // the matrix instruction
       if constexpr (J < NQ) {
-        if constexpr ((J & 1) == 0) a0 = mma16(ring[J & 3], grp[0].q[J >> 1], a0);
-        else a1 = mma16(ring[J & 3], grp[0].q[J >> 1], a1);
+        if constexpr ((J & 1) == 0) a0 = mma16(ring[J % (2 * GS)], grp[0].q[J >> 1], a0);
+        else a1 = mma16(ring[J % (2 * GS)], grp[0].q[J >> 1], a1);
       } else if constexpr (J < 2 * NQ) {
-        if constexpr ((J & 1) == 0) b0 = mma16(ring[J & 3], grp[0].q[(J - NQ) >> 1], b0);
-        else b1 = mma16(ring[J & 3], grp[0].q[(J - NQ) >> 1], b1);
+        if constexpr ((J & 1) == 0) b0 = mma16(ring[J % (2 * GS)], grp[0].q[(J - NQ) >> 1], b0);
+        else b1 = mma16(ring[J % (2 * GS)], grp[0].q[(J - NQ) >> 1], b1);
       } else if constexpr (J < 2 * NQ + NV) {
-        grp[0].o[J - 2 * NQ] = mma16(ring[J & 3], pa, grp[0].o[J - 2 * NQ]);
+        grp[0].o[J - 2 * NQ] = mma16(ring[J % (2 * GS)], pa, grp[0].o[J - 2 * NQ]);
       } else {
-        grp[0].o[J - 2 * NQ - NV] = mma16(ring[J & 3], pbb, grp[0].o[J - 2 * NQ - NV]);
+        grp[0].o[J - 2 * NQ - NV] = mma16(ring[J % (2 * GS)], pbb, grp[0].o[J - 2 * NQ - NV]);
       }
       // the scores of a step leave the accumulators right after its last matrix instruction
       if constexpr (J == NQ - 1) {
@@ -481,7 +490,7 @@ cmp_select_kernel(const CmpArgs a) {
           if constexpr (o >= K * kOpsB / NV && o < (K + 1) * kOpsB / NV) opB(O, sa, wa[0], wa[1], true);
         });
       }
-      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (J % GS == GS - 1) __builtin_amdgcn_sched_barrier(0);
     });
 #pragma unroll
     for (int i = 0; i < 8; ++i) cs[i] = sb[i];
@@ -622,6 +631,11 @@ cmp_select_kernel(const CmpArgs a) {
 
   // ---- block importance: scale by the head's normaliser, add the heads, average, pick
   const long orow = ((long)st.start + tok) * a.hkv + h;
+  // 1 / rows of window `bin`: 5, fewer for the windows that reach past the sequence's last row
+  auto window_rcp = [&](int bin) -> float {
+    const int len = min(4 * bin + 5, nkeys) - 4 * bin;
+    return len >= 5 ? 0.2f : len == 4 ? 0.25f : len == 3 ? (1.0f / 3.0f) : len == 2 ? 0.5f : 1.0f;
+  };
   float v[9];
   int ix[9];
   {
@@ -650,8 +664,7 @@ cmp_select_kernel(const CmpArgs a) {
         ok = i >= 1 && i < steps;
       }
       ok = ok && bin < Ns;
-      const int lo = 4 * bin;
-      v[k] = ok ? r8[k] / (float)(min(lo + 5, nkeys) - lo) : -1.f;
+      v[k] = ok ? r8[k] * window_rcp(bin) : -1.f;
       ix[k] = ok ? bin : 0x7fffffff;
     }
     // the 129th value: the last step's upper window of lane row 3 (no next row), owned by lane (n = 0, g = 3)
@@ -661,9 +674,9 @@ cmp_select_kernel(const CmpArgs a) {
     tail += dpp_f32<0x141>(tail);
     tail += dpp_f32<0x140>(tail);
     {
-      const int bin = 8 * steps - 1, lo = 4 * bin;
+      const int bin = 8 * steps - 1;
       const bool ok = last_row && n == 0 && steps > 0 && bin < Ns;
-      v[8] = ok ? tail / (float)(min(lo + 5, nkeys) - lo) : -1.f;
+      v[8] = ok ? tail * window_rcp(bin) : -1.f;
       ix[8] = ok ? bin : 0x7fffffff;
     }
   }

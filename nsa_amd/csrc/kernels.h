@@ -9,8 +9,10 @@ struct CompressArgs {
   const void* x; const void* wt; const void* bias; void* out;
   const int32_t* cu_seq; const int32_t* cu_out;
   int batch, out_rows_bound, heads, dim, block, stride, dtype;
-  // mean pooling only: a second tensor over the same tokens (same heads, its own dim) for the same launch
+  // a second tensor over the same tokens (same heads, its own dim) for the same launch: mean pooling, or the
+  // learned compressor with the second tensor's weight and bias
   const void* x2 = nullptr; void* out2 = nullptr; int dim2 = 0;
+  const void* wt2 = nullptr; const void* bias2 = nullptr;
 };
 
 // Backward of the compression.  w_lin == nullptr: mean pooling (only dx).  w_lin is the weight in the

@@ -201,6 +201,124 @@ compress_weighted_kernel(const T* __restrict__ x, const T* __restrict__ wt, cons
   }
 }
 
+// The learned compressor as a tiled GEMM (16-bit types): out[row][:] = sum_j x[token(row) + j][:] W_j + bias, i.e.
+// [rows x block*DIM] x [block*DIM x DIM] per head with rows that overlap in memory (row r of sequence b starts at
+// token cu_seq[b] + r*stride).  One workgroup owns 64 output rows of one head and ALL DIM output channels; the
+// reduction runs in steps of 32 (one 32-channel slice of one tap): the step's x tile [64 x 32] and weight tile
+// [DIM x 32] are staged in LDS in fragment order (1 KB per operand fragment, so the reads are conflict-free),
+// double buffered, one barrier per step.  The four wavefronts split the output channels; each weight fragment read
+// from LDS feeds four matrix instructions (the four 16-row groups), each x fragment DIM / 64.  Against one
+// workgroup per 32 rows that streams the weight from L2 fragment by fragment, every weight byte fetched now meets
+// twice the rows, comes in whole cache lines, and K and V go in ONE launch (blockIdx.z picks the tensor).
+template <typename T, int DIM>
+__device__ __forceinline__ void compress_gemm_body(const T* __restrict__ x, const T* __restrict__ wt,
+                                                   const T* __restrict__ bias, T* __restrict__ out,
+                                                   const int32_t* __restrict__ cu_seq,
+                                                   const int32_t* __restrict__ cu_out, int batch, int heads, int block,
+                                                   int stride, unsigned char* smem) {
+  constexpr int TM = 64, NCT = DIM / 64, WP = DIM * 4 / 256;      // col tiles per wavefront, weight pieces per thread
+  static_assert(DIM % 64 == 0, "the output channels are dealt to four wavefronts in 16-channel tiles");
+  T* xs = reinterpret_cast<T*>(smem);                  // [2][4 row groups][64 lanes][8]
+  T* ws = xs + 2 * 4 * 512;                            // [2][DIM / 16 col tiles][64 lanes][8]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int total_out = cu_out[batch];
+  const int m0 = blockIdx.x * TM, h = blockIdx.y;
+  if (m0 >= total_out) return;
+  const int K = block * DIM;
+  // staging: thread t moves x piece t (row group t / 64, lane t % 64) and weight pieces t, t + 256, ...
+  const T* xsrc;
+  {
+    const int rc = min(m0 + (tid >> 6) * 16 + (lane & 15), total_out - 1);
+    const int b = upper_seq(cu_out, batch, rc);
+    xsrc = x + (((long)cu_seq[b] + (long)(rc - cu_out[b]) * stride) * heads + h) * DIM + 8 * (lane >> 4);
+  }
+  const T* wsrc[WP];
+#pragma unroll
+  for (int i = 0; i < WP; ++i) {
+    const int q = tid + i * 256;
+    wsrc[i] = wt + (long)((q >> 6) * 16 + (lane & 15)) * K + 8 * (lane >> 4);
+  }
+  f32x4_t acc[4][NCT];
+#pragma unroll
+  for (int rg = 0; rg < 4; ++rg)
+#pragma unroll
+    for (int ct = 0; ct < NCT; ++ct) acc[rg][ct] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const int steps = block * (DIM / 32);
+  vec8_t<T> xr, wr[WP];
+  auto gload = [&](int s) {
+    const int j = s / (DIM / 32), kk = s % (DIM / 32);
+    xr = load8(xsrc + (long)j * heads * DIM + 32 * kk);
+#pragma unroll
+    for (int i = 0; i < WP; ++i) wr[i] = load8(wsrc[i] + 32 * s);
+  };
+  auto lstore = [&](int buf) {
+    store8(xs + buf * 4 * 512 + tid * 8, xr);
+#pragma unroll
+    for (int i = 0; i < WP; ++i) store8(ws + buf * (DIM / 16) * 512 + (tid + i * 256) * 8, wr[i]);
+  };
+  gload(0);
+  lstore(0);
+  __syncthreads();
+  int buf = 0;
+  for (int s = 0; s < steps; ++s) {
+    if (s + 1 < steps) gload(s + 1);
+    const T* xb = xs + buf * 4 * 512 + lane * 8;
+    const T* wb = ws + buf * (DIM / 16) * 512 + wave * NCT * 512 + lane * 8;
+    vec8_t<T> xf[4];
+#pragma unroll
+    for (int rg = 0; rg < 4; ++rg) xf[rg] = load8(xb + rg * 512);
+#pragma unroll
+    for (int ct = 0; ct < NCT; ++ct) {
+      const vec8_t<T> wa = load8(wb + ct * 512);
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) acc[rg][ct] = mma16(wa, xf[rg], acc[rg][ct]);     // out^T tile: rows = channels
+    }
+    if (s + 1 < steps) lstore(buf ^ 1);
+    __syncthreads();
+    buf ^= 1;
+  }
+  // epilogue through LDS: lane (n, g) holds channels 4g .. 4g+3 of row n; whole rows leave in 16-byte pieces
+  constexpr int LD = DIM + 4;
+  float* tile = reinterpret_cast<float*>(smem);        // [64][LD]  (the staging buffers are free: last barrier passed)
+  const int n = lane & 15, g = lane >> 4;
+#pragma unroll
+  for (int rg = 0; rg < 4; ++rg)
+#pragma unroll
+    for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) tile[(rg * 16 + n) * LD + (wave * NCT + ct) * 16 + 4 * g + i] = acc[rg][ct][i];
+  __syncthreads();
+  for (int p = tid; p < TM * (DIM / 8); p += 256) {
+    const int r = p / (DIM / 8), pc = p % (DIM / 8);
+    if (m0 + r >= total_out) continue;
+    float v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      v[e] = tile[r * LD + pc * 8 + e];
+      if (bias != nullptr) v[e] += (float)bias[pc * 8 + e];
+    }
+    store8(out + ((long)(m0 + r) * heads + h) * DIM + pc * 8, pack8<T>(v));
+  }
+}
+
+struct GemmOperand { const void* x; const void* wt; const void* bias; void* out; };
+
+template <typename T, int D0, int D1>
+__global__ void __launch_bounds__(256)
+compress_gemm_kernel(const GemmOperand s0, const GemmOperand s1, const int32_t* __restrict__ cu_seq,
+                     const int32_t* __restrict__ cu_out, int batch, int heads, int block, int stride) {
+  constexpr int DMAX = D0 > D1 ? D0 : D1;
+  constexpr int STAGE = 2 * (4 + DMAX / 16) * 512 * (int)sizeof(T), EPI = 64 * (DMAX + 4) * 4;
+  __shared__ __attribute__((aligned(16))) unsigned char smem[STAGE > EPI ? STAGE : EPI];
+  if (blockIdx.z == 0)
+    compress_gemm_body<T, D0>((const T*)s0.x, (const T*)s0.wt, (const T*)s0.bias, (T*)s0.out, cu_seq, cu_out, batch, heads,
+                              block, stride, smem);
+  else
+    compress_gemm_body<T, D1>((const T*)s1.x, (const T*)s1.wt, (const T*)s1.bias, (T*)s1.out, cu_seq, cu_out, batch, heads,
+                              block, stride, smem);
+}
+
 // out[(h*dim + d) * out_cols + col], col = transposed_offset(cu[b], b) + row; every other column is 0.
 template <typename T>
 __global__ void __launch_bounds__(256)
@@ -263,6 +381,21 @@ static int launch_compress_t(const CompressArgs& a, hipStream_t st) {
     hipLaunchKernelGGL(compress_mean_kernel<T>, grid, dim3(256), 0, st, s0, s1, a.cu_seq, a.cu_out, a.batch, a.heads,
                        a.block, a.stride);
     return 0;
+  }
+  if constexpr (sizeof(T) == 2) {
+    // the tiled GEMM for head dims that split over four wavefronts; K and V of a layer in one launch
+    const int d0 = a.dim, d1 = a.x2 ? a.dim2 : a.dim;
+    const GemmOperand s0{a.x, a.wt, a.bias, a.out}, s1{a.x2, a.wt2, a.bias2, a.out2};
+    const dim3 ggrid((a.out_rows_bound + 63) / 64, a.heads, a.x2 ? 2 : 1);
+#define NSA_GEMM(DA, DB)                                                                                     \
+    if (d0 == DA && d1 == DB) {                                                                              \
+      hipLaunchKernelGGL((compress_gemm_kernel<T, DA, DB>), ggrid, dim3(256), 0, st, s0, s1, a.cu_seq, a.cu_out, \
+                         a.batch, a.heads, a.block, a.stride);                                               \
+      return 0;                                                                                              \
+    }
+    NSA_GEMM(64, 64) NSA_GEMM(128, 128) NSA_GEMM(192, 192) NSA_GEMM(192, 128)
+#undef NSA_GEMM
+    if (a.x2) return -7;      // no paired instance for these head dims: the caller launches the tensors one by one
   }
   const dim3 grid((a.out_rows_bound + 31) / 32, a.heads);
 #define NSA_WEIGHTED(D)                                                                              \
