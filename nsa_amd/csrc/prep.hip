@@ -14,6 +14,8 @@
 
 namespace nsa {
 
+int set_smem(const void* fn, size_t bytes);
+
 __device__ __forceinline__ int upper_seq(const int32_t* __restrict__ cu, int batch, int r) {
   // largest b in [0,batch) with cu[b] <= r   (cu non-decreasing, cu[0] <= r assumed)
   int lo = 0, hi = batch;  // invariant: cu[lo] <= r, answer in [lo, hi)
@@ -204,83 +206,104 @@ compress_weighted_kernel(const T* __restrict__ x, const T* __restrict__ wt, cons
 // The learned compressor as a tiled GEMM (16-bit types): out[row][:] = sum_j x[token(row) + j][:] W_j + bias, i.e.
 // [rows x block*DIM] x [block*DIM x DIM] per head with rows that overlap in memory (row r of sequence b starts at
 // token cu_seq[b] + r*stride).  One workgroup owns 64 output rows of one head and ALL DIM output channels; the
-// reduction runs in steps of 32 (one 32-channel slice of one tap): the step's x tile [64 x 32] and weight tile
-// [DIM x 32] are staged in LDS in fragment order (1 KB per operand fragment, so the reads are conflict-free),
-// double buffered, one barrier per step.  The four wavefronts split the output channels; each weight fragment read
-// from LDS feeds four matrix instructions (the four 16-row groups), each x fragment DIM / 64.  Against one
-// workgroup per 32 rows that streams the weight from L2 fragment by fragment, every weight byte fetched now meets
-// twice the rows, comes in whole cache lines, and K and V go in ONE launch (blockIdx.z picks the tensor).
+// reduction runs in steps of 64 (one 64-channel slice of one tap, two matrix-instruction depths).  A step's operands
+// -- 2 x 4 x fragments and 2 x DIM / 16 weight fragments of 1 KB -- go from global memory straight into LDS
+// (global_load_lds: every lane names the 16 bytes of its place in the fragment, so the tile arrives in fragment
+// order and the reads are conflict-free) through a ring of kGemmRing step buffers, kGemmRing - 1 steps ahead: the
+// GEMM is small (one workgroup per CU), so nothing but the loads in flight hides the memory latency.  One barrier
+// per step.  The four wavefronts split the output channels; each weight fragment read from LDS feeds four matrix
+// instructions (the four 16-row groups), each x fragment DIM / 64.  K and V of a layer go in ONE launch
+// (blockIdx.z picks the tensor).  What bounds it: a CU takes in about 16 bytes per clock from L2 however the loads
+// are issued, and a 64-row tile needs block * DIM * 2 * (64 + DIM) bytes for 2 * 64 * DIM * block * DIM flops.
+constexpr int kGemmRing = 4;
+
+__device__ __forceinline__ void gemm_wait_loads(int n) {      // at most n vector-memory loads of this wavefront outstanding
+  switch (n) {
+#define NSA_WAIT_CASE(N) case N: asm volatile("s_waitcnt vmcnt(" #N ")" ::: "memory"); break;
+    NSA_WAIT_CASE(4) NSA_WAIT_CASE(8) NSA_WAIT_CASE(12) NSA_WAIT_CASE(16) NSA_WAIT_CASE(20) NSA_WAIT_CASE(24)
+    NSA_WAIT_CASE(2) NSA_WAIT_CASE(6) NSA_WAIT_CASE(10) NSA_WAIT_CASE(14) NSA_WAIT_CASE(18)
+    NSA_WAIT_CASE(3) NSA_WAIT_CASE(9) NSA_WAIT_CASE(15)
+#undef NSA_WAIT_CASE
+    default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+  }
+}
+
+template <typename T>
+__device__ __forceinline__ void gemm_global_to_lds16(const T* src, const T* lds) {
+  const unsigned dst = (unsigned)(uintptr_t)((__attribute__((address_space(3))) const char*)lds);
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(src), "s"(dst) : "memory");
+}
+
 template <typename T, int DIM>
 __device__ __forceinline__ void compress_gemm_body(const T* __restrict__ x, const T* __restrict__ wt,
                                                    const T* __restrict__ bias, T* __restrict__ out,
                                                    const int32_t* __restrict__ cu_seq,
                                                    const int32_t* __restrict__ cu_out, int batch, int heads, int block,
                                                    int stride, unsigned char* smem) {
-  constexpr int TM = 64, NCT = DIM / 64, WP = DIM * 4 / 256;      // col tiles per wavefront, weight pieces per thread
+  constexpr int TM = 64, NCT = DIM / 64;               // 16-channel tiles per wavefront
+  constexpr int SLOT = 2 * (4 + DIM / 16) * 512;       // elements of one 64-deep step's operands in LDS
+  constexpr int LPS = 2 * (1 + NCT);                   // loads per step and wavefront
   static_assert(DIM % 64 == 0, "the output channels are dealt to four wavefronts in 16-channel tiles");
-  T* xs = reinterpret_cast<T*>(smem);                  // [2][4 row groups][64 lanes][8]
-  T* ws = xs + 2 * 4 * 512;                            // [2][DIM / 16 col tiles][64 lanes][8]
+  T* ring = reinterpret_cast<T*>(smem);                // [kGemmRing][2 halves][x fragments 0..3 | weight fragments]
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int total_out = cu_out[batch];
   const int m0 = blockIdx.x * TM, h = blockIdx.y;
   if (m0 >= total_out) return;
   const int K = block * DIM;
-  // staging: thread t moves x piece t (row group t / 64, lane t % 64) and weight pieces t, t + 256, ...
+  // wavefront w brings x fragment w (rows m0 + 16 w ..) and the weight fragments of its own channel tiles; the two
+  // 32-deep halves of a step are requested back to back: together a lane group reads whole 128-byte lines
   const T* xsrc;
   {
-    const int rc = min(m0 + (tid >> 6) * 16 + (lane & 15), total_out - 1);
+    const int rc = min(m0 + wave * 16 + (lane & 15), total_out - 1);
     const int b = upper_seq(cu_out, batch, rc);
     xsrc = x + (((long)cu_seq[b] + (long)(rc - cu_out[b]) * stride) * heads + h) * DIM + 8 * (lane >> 4);
   }
-  const T* wsrc[WP];
-#pragma unroll
-  for (int i = 0; i < WP; ++i) {
-    const int q = tid + i * 256;
-    wsrc[i] = wt + (long)((q >> 6) * 16 + (lane & 15)) * K + 8 * (lane >> 4);
-  }
+  const T* wsrc = wt + (long)(wave * NCT * 16 + (lane & 15)) * K + 8 * (lane >> 4);
   f32x4_t acc[4][NCT];
 #pragma unroll
   for (int rg = 0; rg < 4; ++rg)
 #pragma unroll
     for (int ct = 0; ct < NCT; ++ct) acc[rg][ct] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  const int steps = block * (DIM / 32);
-  vec8_t<T> xr, wr[WP];
-  auto gload = [&](int s) {
-    const int j = s / (DIM / 32), kk = s % (DIM / 32);
-    xr = load8(xsrc + (long)j * heads * DIM + 32 * kk);
+  const int steps = block * (DIM / 64);
+  auto issue = [&](int s) {
+    const int j = s / (DIM / 64), kk = s % (DIM / 64);
+    T* slot = ring + (s % kGemmRing) * SLOT;
 #pragma unroll
-    for (int i = 0; i < WP; ++i) wr[i] = load8(wsrc[i] + 32 * s);
-  };
-  auto lstore = [&](int buf) {
-    store8(xs + buf * 4 * 512 + tid * 8, xr);
+    for (int hf = 0; hf < 2; ++hf)
+      gemm_global_to_lds16(xsrc + (long)j * heads * DIM + 64 * kk + 32 * hf, slot + hf * (SLOT / 2) + wave * 512);
 #pragma unroll
-    for (int i = 0; i < WP; ++i) store8(ws + buf * (DIM / 16) * 512 + (tid + i * 256) * 8, wr[i]);
+    for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf)
+        gemm_global_to_lds16(wsrc + (long)ct * 16 * K + 64 * s + 32 * hf,
+                             slot + hf * (SLOT / 2) + (4 + wave * NCT + ct) * 512);
   };
-  gload(0);
-  lstore(0);
-  __syncthreads();
-  int buf = 0;
+  for (int s = 0; s < kGemmRing - 1 && s < steps; ++s) issue(s);
   for (int s = 0; s < steps; ++s) {
-    if (s + 1 < steps) gload(s + 1);
-    const T* xb = xs + buf * 4 * 512 + lane * 8;
-    const T* wb = ws + buf * (DIM / 16) * 512 + wave * NCT * 512 + lane * 8;
-    vec8_t<T> xf[4];
+    // steps s + 1 .. min(s + kGemmRing - 2, steps - 1) may still be in flight; step s must have landed
+    gemm_wait_loads(LPS * (min(s + kGemmRing - 2, steps - 1) - s));
+    __syncthreads();                                   // everybody's part of step s is in; step s - 1 is consumed
+    if (s + kGemmRing - 1 < steps) issue(s + kGemmRing - 1);
 #pragma unroll
-    for (int rg = 0; rg < 4; ++rg) xf[rg] = load8(xb + rg * 512);
+    for (int hf = 0; hf < 2; ++hf) {
+      const T* xb = ring + (s % kGemmRing) * SLOT + hf * (SLOT / 2) + lane * 8;
+      const T* wb = xb + (4 + wave * NCT) * 512;
+      vec8_t<T> xf[4];
 #pragma unroll
-    for (int ct = 0; ct < NCT; ++ct) {
-      const vec8_t<T> wa = load8(wb + ct * 512);
+      for (int rg = 0; rg < 4; ++rg) xf[rg] = load8(xb + rg * 512);
 #pragma unroll
-      for (int rg = 0; rg < 4; ++rg) acc[rg][ct] = mma16(wa, xf[rg], acc[rg][ct]);     // out^T tile: rows = channels
+      for (int ct = 0; ct < NCT; ++ct) {
+        const vec8_t<T> wa = load8(wb + ct * 512);
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) acc[rg][ct] = mma16(wa, xf[rg], acc[rg][ct]);   // out^T tile: rows = channels
+      }
     }
-    if (s + 1 < steps) lstore(buf ^ 1);
-    __syncthreads();
-    buf ^= 1;
   }
+  __syncthreads();
   // epilogue through LDS: lane (n, g) holds channels 4g .. 4g+3 of row n; whole rows leave in 16-byte pieces
   constexpr int LD = DIM + 4;
-  float* tile = reinterpret_cast<float*>(smem);        // [64][LD]  (the staging buffers are free: last barrier passed)
+  float* tile = reinterpret_cast<float*>(smem);        // [64][LD]  (the ring is free: last barrier passed)
   const int n = lane & 15, g = lane >> 4;
 #pragma unroll
   for (int rg = 0; rg < 4; ++rg)
@@ -304,13 +327,16 @@ __device__ __forceinline__ void compress_gemm_body(const T* __restrict__ x, cons
 
 struct GemmOperand { const void* x; const void* wt; const void* bias; void* out; };
 
+template <typename T> constexpr size_t compress_gemm_smem(int dmax) {
+  const size_t ring = (size_t)kGemmRing * 2 * (4 + dmax / 16) * 512 * sizeof(T), epi = (size_t)64 * (dmax + 4) * 4;
+  return ring > epi ? ring : epi;
+}
+
 template <typename T, int D0, int D1>
 __global__ void __launch_bounds__(256)
 compress_gemm_kernel(const GemmOperand s0, const GemmOperand s1, const int32_t* __restrict__ cu_seq,
                      const int32_t* __restrict__ cu_out, int batch, int heads, int block, int stride) {
-  constexpr int DMAX = D0 > D1 ? D0 : D1;
-  constexpr int STAGE = 2 * (4 + DMAX / 16) * 512 * (int)sizeof(T), EPI = 64 * (DMAX + 4) * 4;
-  __shared__ __attribute__((aligned(16))) unsigned char smem[STAGE > EPI ? STAGE : EPI];
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];      // compress_gemm_smem<T>(max(D0, D1))
   if (blockIdx.z == 0)
     compress_gemm_body<T, D0>((const T*)s0.x, (const T*)s0.wt, (const T*)s0.bias, (T*)s0.out, cu_seq, cu_out, batch, heads,
                               block, stride, smem);
@@ -389,8 +415,11 @@ static int launch_compress_t(const CompressArgs& a, hipStream_t st) {
     const dim3 ggrid((a.out_rows_bound + 63) / 64, a.heads, a.x2 ? 2 : 1);
 #define NSA_GEMM(DA, DB)                                                                                     \
     if (d0 == DA && d1 == DB) {                                                                              \
-      hipLaunchKernelGGL((compress_gemm_kernel<T, DA, DB>), ggrid, dim3(256), 0, st, s0, s1, a.cu_seq, a.cu_out, \
-                         a.batch, a.heads, a.block, a.stride);                                               \
+      const size_t smem = compress_gemm_smem<T>(DA > DB ? DA : DB);                                          \
+      auto fn = compress_gemm_kernel<T, DA, DB>;                                                             \
+      if (const int rc = set_smem(reinterpret_cast<const void*>(fn), smem)) return rc;                       \
+      hipLaunchKernelGGL(fn, ggrid, dim3(256), smem, st, s0, s1, a.cu_seq, a.cu_out, a.batch, a.heads, a.block, \
+                         a.stride);                                                                          \
       return 0;                                                                                              \
     }
     NSA_GEMM(64, 64) NSA_GEMM(128, 128) NSA_GEMM(192, 192) NSA_GEMM(192, 128)
