@@ -345,3 +345,35 @@ def test_sequence_lengths_are_read_on_the_host_once_per_cu_seqlens_tensor(monkey
     for _ in range(40):                               # the table stays small
         nsa_mod._sequence_lengths_once(torch.tensor([0, 3, 7]))
     assert len(nsa_mod._LENGTHS_SEEN) <= 16
+
+
+def test_single_pass_eligibility_and_pack_errors_on_the_host(lib):
+    # which shapes the one-kernel compressed attention + selection takes: answered without a GPU
+    base = dict(hq=64, hkv=4, dk=192, dv=128, pk=5, ps=4, pp=0, top_n=16, max_nc=2047, dtype=0)
+
+    def ok(**kw):
+        return lib.nsa_cmp_select_single_pass(*{**base, **kw}.values())
+
+    assert ok() == 1 and ok(dtype=2) == 1 and ok(dk=128) == 1 and ok(dk=64, dv=64) == 1 and ok(hq=36) == 1
+    assert ok(max_nc=2048) == 1 and ok(max_nc=2049) == 0                       # 2048 compressed rows per sequence
+    assert ok(dtype=1) == 0                                                    # fp32 stays on the three launches
+    assert ok(hq=32) == 0 and ok(hq=128) == 0 and ok(hq=0) == 0 and ok(hq=65) == 0   # groups of 9..16 heads
+    assert ok(dk=192, dv=192) == 0 and ok(dk=32, dv=32) == 0
+    assert ok(pk=3, ps=2) == 0 and ok(pp=1) == 0 and ok(top_n=65) == 0
+    # chunk slots of the fragment-major copy: room for every sequence's partial last chunk
+    for rows, batch in [(0, 1), (63, 1), (64, 1), (2047, 1), (5000, 7)]:
+        assert lib.nsa_cmp_pack_chunks(rows, batch) >= (rows + 63) // 64 + batch - (1 if rows else 0)
+    buf = ctypes.create_string_buffer(4096)
+    p = ctypes.c_void_p((ctypes.addressof(buf) + 15) & ~15)
+    pack = lambda ck=p, chunks=40, dtype=0, stride=768, dk=192: lib.nsa_cmp_pack_fwd(      # noqa: E731
+        ck, p, p, p, 1, 2047, 4, dk, 128, stride, dk, 512, 128, chunks, dtype, None)
+    assert pack(ck=None) == -1 and b"null" in lib.nsa_last_error_string()
+    assert pack(dtype=1) == -2 and b"16-bit" in lib.nsa_last_error_string()
+    assert pack(stride=772) == -1 and b"multiples of 8" in lib.nsa_last_error_string()
+    assert pack(chunks=8) == -1 and b"nsa_cmp_pack_chunks" in lib.nsa_last_error_string()
+    # the selection entry point: indices are not optional, single_pass is -1 / 0 / 1
+    sel = lambda indices=p, single_pass=-1: lib.nsa_cmp_select_fwd(      # noqa: E731
+        p, p, p, p, 40, p, indices, None, p, None, None, None, None, p, p, 1, 4096, 64, 4, 192, 128, 768, 192, 4160, 32,
+        16, 5, 4, 0, 16, 255, 64, 0, 0, 0.1, 1, 0, 0, single_pass, None)
+    assert sel(indices=None) == -1 and b"null" in lib.nsa_last_error_string()
+    assert sel(single_pass=2) == -1 and b"single_pass" in lib.nsa_last_error_string()
