@@ -377,3 +377,49 @@ def test_single_pass_eligibility_and_pack_errors_on_the_host(lib):
         16, 5, 4, 0, 16, 255, 64, 0, 0, 0.1, 1, 0, 0, single_pass, None)
     assert sel(indices=None) == -1 and b"null" in lib.nsa_last_error_string()
     assert sel(single_pass=2) == -1 and b"single_pass" in lib.nsa_last_error_string()
+
+
+def test_module_inference_takes_the_single_pass_kernel_exactly_when_the_library_says_so(monkeypatch):
+    """The module's no-grad forward asks the library whether the shape runs as one kernel and stages the matching
+    operands: the fragment-major copy for the single pass, the transposed compressed values otherwise."""
+    from nsa_amd import nsa as nsa_mod, ops
+    calls = []
+
+    def fake(name, ret):
+        def f(*a, **kw):
+            calls.append((name, kw))
+            return ret(*a, **kw) if callable(ret) else ret
+        return f
+
+    def run(hq, dtype, T=640):
+        del calls[:]
+        hkv, d = 4, 128
+        m = nsa_mod.NSAAttention(d, causal=True, device="cpu", dtype=dtype, compressor_mode="mean")
+        q = torch.zeros(T, hq, d, dtype=dtype)
+        k = torch.zeros(T, hkv, d, dtype=dtype)
+        nc = (T - 32) // 16 + 1
+        o = torch.zeros(T, hq, d, dtype=dtype)
+        idx = torch.zeros(T, hkv, 16, dtype=torch.int32)
+        gates = torch.zeros(T, hq, 3, dtype=dtype)
+        monkeypatch.setattr(m.compressor, "compress_packed", fake("compress", (k[:nc], k[:nc], torch.tensor([0, nc]), nc)))
+        monkeypatch.setattr(ops, "cmp_pack", fake("cmp_pack", ("frag", 1)))
+        monkeypatch.setattr(ops, "transpose", fake("transpose", "t"))
+        monkeypatch.setattr(ops, "cmp_select", fake("cmp_select", dict(o=o, indices=idx, gates=gates)))
+        monkeypatch.setattr(ops, "cmp_attn", fake("cmp_attn", (o, "lse", gates)))
+        monkeypatch.setattr(ops, "block_select", fake("block_select", (idx, None)))
+        monkeypatch.setattr(ops, "slc_workspace", fake("slc_workspace", "ws"))
+        monkeypatch.setattr(ops, "slc_partials", fake("slc_partials", None))
+        monkeypatch.setattr(ops, "swa_merge", fake("swa_merge", o))
+        with torch.no_grad():
+            out = m._forward_infer(q, k, k, torch.tensor([0, T], dtype=torch.int32), 1, 0.1, True, T, True, None, None,
+                                   False)
+        assert out is o
+        return [c[0] for c in calls]
+
+    one = run(64, torch.bfloat16)                                  # group of 16, 16-bit: the single pass
+    assert one == ["compress", "cmp_pack", "transpose", "cmp_select", "slc_workspace", "slc_partials", "swa_merge"]
+    assert calls[3][1]["single_pass"] is True and calls[3][1]["frag"] == ("frag", 1)
+    three = run(32, torch.bfloat16)                                # group of 8: compressed attention, then selection
+    assert three == ["compress", "transpose", "transpose", "cmp_attn", "block_select", "slc_workspace", "slc_partials",
+                     "swa_merge"]
+    assert run(64, torch.float32)[3] == "cmp_attn"                 # fp32: three launches
