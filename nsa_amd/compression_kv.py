@@ -91,9 +91,16 @@ class KVCompressor(nn.Module):
         self.compressor_v = nn.Conv1d(v_head_dim, v_head_dim, block_size, block_stride, **factory_kwargs)
 
     def _wt(self, conv: nn.Conv1d) -> torch.Tensor:
-        # [o, i, j] -> [o, j*D + i]
+        """[o, i, j] -> [o, j*D + i], the layout the kernels read.  The no-grad path asks for it on every forward, so
+        the copy is kept until the parameter changes (another tensor, another storage, or an in-place update)."""
         w = conv.weight.detach()
-        return w.permute(0, 2, 1).reshape(w.shape[0], -1).contiguous()
+        key = (id(conv.weight), w.data_ptr(), conv.weight._version, w.dtype, w.device)
+        cache = self.__dict__.setdefault("_wt_cache", {})
+        hit = cache.get(id(conv))
+        if hit is None or hit[0] != key:
+            hit = (key, w.permute(0, 2, 1).reshape(w.shape[0], -1).contiguous())
+            cache[id(conv)] = hit
+        return hit[1]
 
     @staticmethod
     def _w_lin(conv: nn.Conv1d) -> torch.Tensor:

@@ -423,3 +423,21 @@ def test_module_inference_takes_the_single_pass_kernel_exactly_when_the_library_
     assert three == ["compress", "transpose", "transpose", "cmp_attn", "block_select", "slc_workspace", "slc_partials",
                      "swa_merge"]
     assert run(64, torch.float32)[3] == "cmp_attn"                 # fp32: three launches
+
+
+def test_conv_compressor_keeps_its_kernel_layout_weight_until_the_parameter_changes():
+    from nsa_amd.compression_kv import KVCompressor
+    c = KVCompressor(16, 32, 8, device="cpu", dtype=torch.float32)
+    w0 = c._wt(c.compressor_k)
+    assert w0.shape == (8, 32 * 8)
+    assert torch.equal(w0, c.compressor_k.weight.detach().permute(0, 2, 1).reshape(8, -1))
+    assert c._wt(c.compressor_k) is w0 and c._wt(c.compressor_v) is not w0       # per convolution
+    with torch.no_grad():
+        c.compressor_k.weight.mul_(2.0)                                          # an optimizer step
+    w1 = c._wt(c.compressor_k)
+    assert w1 is not w0 and torch.equal(w1, 2.0 * w0)
+    c.load_state_dict({k: torch.ones_like(v) for k, v in c.state_dict().items()})   # copy_ bumps the version too
+    assert torch.equal(c._wt(c.compressor_k), torch.ones(8, 32 * 8))
+    c.compressor_k.weight = torch.nn.Parameter(torch.zeros(8, 8, 32))            # a new parameter object
+    assert torch.equal(c._wt(c.compressor_k), torch.zeros(8, 32 * 8))
+    assert "_wt_cache" not in c.state_dict()
